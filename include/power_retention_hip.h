@@ -1,0 +1,113 @@
+/*
+ * C ABI of libpower_retention_hip.so: the gfx950 (MI355X) kernels behind the four operators of
+ * symmetric power retention and their backward passes.
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer, 16-byte aligned, to a dense row-major tensor of the stated
+ *     shape; nothing is allocated, freed or synchronised inside the library; outputs and workspaces are
+ *     provided by the caller; inputs are never written.
+ *   - dtype: PR_BF16 / PR_F16 for Q, K, V, states and outputs (PR_F32 additionally for pr_discumsum_*);
+ *     gates, row statistics and key sums are always fp32.
+ *   - stream: a hipStream_t (NULL = default stream); calls only enqueue work.
+ *   - return value: 0 on success, PR_ERR_* (< 0) for arguments the kernels do not support (nothing
+ *     is launched), or a positive hipError_t from the launch.  pr_last_error() describes the last
+ *     failure on the calling thread.
+ *   - head dim d (= value dim) in {32, 64, 128}; deg = 2 for everything that touches the state;
+ *     r = query heads per kv head.
+ *
+ * Each entry point names the reference interface it replaces (paths relative to the reference tree).
+ */
+#ifndef POWER_RETENTION_HIP_H
+#define POWER_RETENTION_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum { PR_BF16 = 0, PR_F16 = 1, PR_F32 = 2 };
+enum {
+  PR_OK = 0,
+  PR_ERR_DTYPE = -1,     /* unsupported dtype */
+  PR_ERR_HEAD_DIM = -2,  /* unsupported head dim */
+  PR_ERR_ARG = -3,       /* null / misaligned pointer, non-positive size, inconsistent sizes */
+  PR_ERR_DEG = -4        /* unsupported degree */
+};
+
+int pr_abi_version(void);
+const char* pr_last_error(void);
+
+/* Size D of the expanded state for head dim d: 256 * T(T+1)/2, T = d/16; -1 if d is not a multiple of 16.
+ * Replaces retention/_utils.py:18-19 compute_expanded_dim. */
+int pr_expanded_dim(int d, int deg);
+
+/* attention(Q, K, V, log_G_accum, deg, scale, norm) -- retention/_attention/reference.py:10-69,
+ * Triton twin retention/_attention/triton.py:606-721 (_attn_fwd).
+ *   Q [B,tq,h*r,d], K,V [B,tk,h,d], G [B,tk,h] fp32 accumulated log gate or NULL
+ *   -> O [B,tq,h*r,d]; l, rowmax [B,tq,h*r] fp32 (either may be NULL when norm != 0).
+ *   norm != 0 writes o/l to O, otherwise the unnormalised o. Queries are aligned to the end of the keys. */
+int pr_attention_fwd(const void* Q, const void* K, const void* V, const float* G, void* O, float* l, float* rowmax,
+                     int B, int tq, int tk, int h, int r, int d, float scale, int deg, int norm, int dtype,
+                     void* stream);
+
+/* Backward of the above w.r.t. (o, l) of the norm == 0 form -- retention/_attention/triton.py:228-603,723-810.
+ *   rowmax as returned by the forward; dO [B,tq,h*r,d]; dl [B,tq,h*r] fp32 or NULL (zero)
+ *   -> dQ [B,tq,h*r,d], dK, dV [B,tk,h,d]; when G != NULL also dGq [B,tq,h*r] (sum_j dz_ij) and
+ *   dGk [B,tk,h] (-sum_i dz_ij), whose sum over the aligned positions is d log_G_accum. */
+int pr_attention_bwd(const void* Q, const void* K, const void* V, const float* G, const float* rowmax,
+                     const void* dO, const float* dl, void* dQ, void* dK, void* dV, float* dGq, float* dGk, int B,
+                     int tq, int tk, int h, int r, int d, float scale, int deg, int dtype, void* stream);
+
+/* update_state(K, V, deg) -- retention/_update_state/reference.py:33-52,86-94,
+ * Triton twin retention/_update_state/triton.py:61-133,280-320.
+ *   K, V [BN,c,h,d] (BN = b*n chunks) -> S [BN,h,D,d], s [BN,h,D] fp32. */
+int pr_update_state_fwd(const void* K, const void* V, void* S, float* s, int BN, int c, int h, int d, int deg,
+                        int dtype, void* stream);
+
+/* Backward -- retention/_update_state/reference.py:55-83, Triton twin retention/_update_state/triton.py:148-260.
+ *   dS [BN,h,D,d], ds [BN,h,D] fp32 -> dK, dV [BN,c,h,d]. */
+int pr_update_state_bwd(const void* K, const void* V, const void* dS, const float* ds, void* dK, void* dV, int BN,
+                        int c, int h, int d, int deg, int dtype, void* stream);
+
+/* discumsum(X, log_G) -- retention/_discumsum/reference.py:3-15, Triton twin retention/_discumsum/triton.py:34-94.
+ *   X [B,n,H,F], log_G [B,n,H] fp32 -> Y [B,n_out,H,F], Y[0]=0, Y[k+1]=Y[k]*exp(log_G[k])+X[k];
+ *   n_out = n+1 (the operator) or n (the last entry, which the composed path discards, is not produced).
+ *   F must be a multiple of 16 bytes / sizeof(dtype). */
+int pr_discumsum_fwd(const void* X, const float* log_G, void* Y, int B, int n, int n_out, int H, int64_t F,
+                     int dtype, void* stream);
+
+/* Backward -- autograd of retention/_discumsum/reference.py:3-15 (Triton twin retention/_discumsum/triton.py:111-204).
+ *   dY, Y [B,n_out,H,F] -> dX [B,n,H,F], dlog_G [B,n,H] fp32 (deterministic two-pass reduction).
+ *   workspace: pr_discumsum_bwd_workspace() bytes of device memory. */
+size_t pr_discumsum_bwd_workspace(int B, int n, int H, int64_t F, int dtype);
+int pr_discumsum_bwd(const void* dY, const void* Y, const float* log_G, void* dX, float* dlog_G, void* workspace,
+                     int B, int n, int n_out, int H, int64_t F, int dtype, void* stream);
+
+/* query_state(Q, S, s, Y_attn, l_attn, rowmax, deg, scale, zero_initial_state) --
+ * retention/_query_state/reference.py:36-96,166-191, Triton twin retention/_query_state/triton.py:54-169,478-544.
+ *   Q [BN,c,h*r,d] (already gated), S [BN,h,D,d], s [BN,h,D] fp32,
+ *   Y_attn [BN,c,h*r,d] / l_attn, rowmax [BN,c,h*r] fp32, all three NULL when there is no attention part
+ *   -> O [BN,c,h*r,d] and den [BN,c,h*r] fp32, the normaliser in the scaled units the backward expects.
+ *   scale_p = scale^deg; n = chunks per batch entry; zero_initial_state != 0 declares S, s of chunk 0 of every
+ *   batch entry to be zero (they are then not read). */
+int pr_query_state_fwd(const void* Q, const void* S, const float* s, const void* Y_attn, const float* l_attn,
+                       const float* rowmax, void* O, float* den, int BN, int n, int c, int h, int r, int d,
+                       float scale_p, int deg, int zero_initial_state, int dtype, void* stream);
+
+/* Backward -- formulas of retention/_query_state/triton.py:546-553 (kernels :184-448).
+ *   O, den from the forward; dO [BN,c,h*r,d]
+ *   -> dQ [BN,c,h*r,d], dS [BN,h,D,d], ds [BN,h,D] fp32, and, when rowmax != NULL,
+ *      dY_attn [BN,c,h*r,d], dl_attn [BN,c,h*r] fp32.
+ *   workspace: pr_query_state_bwd_workspace() bytes (scaled dO and two fp32 row vectors). */
+size_t pr_query_state_bwd_workspace(int BN, int c, int h, int r, int d, int dtype);
+int pr_query_state_bwd(const void* Q, const void* S, const float* s, const float* rowmax, const void* O,
+                       const float* den, const void* dO, void* dQ, void* dS, float* ds, void* dY_attn,
+                       float* dl_attn, void* workspace, int BN, int n, int c, int h, int r, int d, float scale_p,
+                       int deg, int zero_initial_state, int dtype, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* POWER_RETENTION_HIP_H */

@@ -1,0 +1,53 @@
+"""Builds libpower_retention_hip.so for gfx950 from the .hip sources in this directory.
+
+    python retention_integration_amd/csrc/build.py [--jobs N]
+
+The library is written next to the package (retention_integration_amd/libpower_retention_hip.so).
+"""
+import argparse
+import concurrent.futures as cf
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+OUT = os.path.join(os.path.dirname(HERE), "libpower_retention_hip.so")
+SOURCES = ["capi", "discumsum", "sympow_tn", "sympow_nn", "sympow_grad", "attention_fwd", "attention_bwd", "elementwise"]
+FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Xclang", "-target-feature", "-Xclang",
+         "-packed-fp32-ops", "-Wno-unused-command-line-argument"]
+
+
+def hipcc():
+    for cand in (os.environ.get("HIPCC"), "/opt/rocm/bin/hipcc", "hipcc"):
+        if cand and (os.path.sep not in cand or os.path.exists(cand)):
+            return cand
+    raise RuntimeError("hipcc not found")
+
+
+def compile_one(name):
+    obj = os.path.join(HERE, "build", name + ".o")
+    cmd = [hipcc(), *FLAGS, "-c", os.path.join(HERE, name + ".hip"), "-o", obj]
+    p = subprocess.run(cmd, capture_output=True, text=True)
+    err = "\n".join(l for l in p.stderr.splitlines() if "not a recognized feature" not in l)
+    if p.returncode != 0:
+        raise RuntimeError(f"hipcc failed for {name}.hip:\n{err}")
+    return obj
+
+
+def build(jobs=8, verbose=True):
+    os.makedirs(os.path.join(HERE, "build"), exist_ok=True)
+    with cf.ThreadPoolExecutor(max_workers=jobs) as ex:
+        objs = list(ex.map(compile_one, SOURCES))
+    cmd = [hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", OUT, *objs]
+    p = subprocess.run(cmd, capture_output=True, text=True)
+    if p.returncode != 0:
+        raise RuntimeError("link failed:\n" + p.stderr)
+    if verbose:
+        print("built", OUT)
+    return OUT
+
+
+if __name__ == "__main__":
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--jobs", type=int, default=min(8, os.cpu_count() or 1))
+    build(ap.parse_args().jobs)

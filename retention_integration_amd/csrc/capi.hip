@@ -1,0 +1,167 @@
+// extern "C" surface of libpower_retention_hip.so: argument checks and dispatch only.
+#include "../../include/power_retention_hip.h"
+
+#include <cstdarg>
+#include <cstdio>
+
+#include "common.h"
+#include "kernels.h"
+
+
+namespace {
+thread_local char g_err[256] = "";
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+bool bad_ptr(const void* p) { return p == nullptr || (reinterpret_cast<uintptr_t>(p) & 15u) != 0; }
+bool bad_opt(const void* p) { return p != nullptr && (reinterpret_cast<uintptr_t>(p) & 15u) != 0; }
+int finish(int rc, const char* what) {
+  if (rc == 0) return 0;
+  if (rc == -1) return fail(PR_ERR_DTYPE, "%s: unsupported dtype", what);
+  if (rc == -2) return fail(PR_ERR_HEAD_DIM, "%s: head dim must be 32, 64 or 128", what);
+  return fail(rc, "%s: launch failed: %s", what, hipGetErrorString((hipError_t)rc));
+}
+int check_common(const char* what, int d, int deg, int dtype, bool state) {
+  if (state && deg != 2) return fail(PR_ERR_DEG, "%s: only deg=2 has a state layout (got %d)", what, deg);
+  if (!state && (deg <= 0 || deg % 2 != 0)) return fail(PR_ERR_DEG, "%s: deg must be a positive even integer (got %d)", what, deg);
+  if (dtype != PR_BF16 && dtype != PR_F16) return fail(PR_ERR_DTYPE, "%s: dtype must be bf16 or fp16", what);
+  if (d != 32 && d != 64 && d != 128) return fail(PR_ERR_HEAD_DIM, "%s: head dim must be 32, 64 or 128 (got %d)", what, d);
+  return 0;
+}
+size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
+}  // namespace
+
+extern "C" {
+
+int pr_abi_version(void) { return 1; }
+const char* pr_last_error(void) { return g_err; }
+
+int pr_expanded_dim(int d, int deg) {
+  if (deg != 2 || d <= 0 || d % 16 != 0) return -1;
+  return pr::expanded_dim(d);
+}
+
+int pr_attention_fwd(const void* Q, const void* K, const void* V, const float* G, void* O, float* l, float* rowmax,
+                     int B, int tq, int tk, int h, int r, int d, float scale, int deg, int norm, int dtype,
+                     void* stream) {
+  if (int rc = check_common("attention_fwd", d, deg, dtype, false)) return rc;
+  if (bad_ptr(Q) || bad_ptr(K) || bad_ptr(V) || bad_ptr(O) || bad_opt(G) || bad_opt(l) || bad_opt(rowmax))
+    return fail(PR_ERR_ARG, "attention_fwd: null or misaligned pointer");
+  if (!norm && (!l || !rowmax)) return fail(PR_ERR_ARG, "attention_fwd: l and rowmax are required when norm == 0");
+  if (B <= 0 || tq <= 0 || tk <= 0 || h <= 0 || r <= 0 || tq > tk)
+    return fail(PR_ERR_ARG, "attention_fwd: need B,tq,tk,h,r > 0 and tq <= tk (got %d %d %d %d %d)", B, tq, tk, h, r);
+  pr::AttnFwdArgs a{Q, K, V, G, O, l, rowmax, tq, tk, h, r, scale, (float)deg, norm};
+  return finish(pr::attention_fwd(a, B, d, dtype, (hipStream_t)stream), "attention_fwd");
+}
+
+int pr_attention_bwd(const void* Q, const void* K, const void* V, const float* G, const float* rowmax,
+                     const void* dO, const float* dl, void* dQ, void* dK, void* dV, float* dGq, float* dGk, int B,
+                     int tq, int tk, int h, int r, int d, float scale, int deg, int dtype, void* stream) {
+  if (int rc = check_common("attention_bwd", d, deg, dtype, false)) return rc;
+  if (bad_ptr(Q) || bad_ptr(K) || bad_ptr(V) || bad_ptr(rowmax) || bad_ptr(dO) || bad_ptr(dQ) || bad_ptr(dK) ||
+      bad_ptr(dV) || bad_opt(G) || bad_opt(dl) || bad_opt(dGq) || bad_opt(dGk))
+    return fail(PR_ERR_ARG, "attention_bwd: null or misaligned pointer");
+  if (G && (!dGq || !dGk)) return fail(PR_ERR_ARG, "attention_bwd: dGq and dGk are required when G is given");
+  if (B <= 0 || tq <= 0 || tk <= 0 || h <= 0 || r <= 0 || tq > tk)
+    return fail(PR_ERR_ARG, "attention_bwd: need B,tq,tk,h,r > 0 and tq <= tk");
+  pr::AttnBwdArgs a{Q, K, V, G, rowmax, dO, dl, dQ, dK, dV, G ? dGq : nullptr, G ? dGk : nullptr,
+                    tq, tk, h, r, scale, (float)deg};
+  return finish(pr::attention_bwd(a, B, d, dtype, (hipStream_t)stream), "attention_bwd");
+}
+
+int pr_update_state_fwd(const void* K, const void* V, void* S, float* s, int BN, int c, int h, int d, int deg,
+                        int dtype, void* stream) {
+  if (int rc = check_common("update_state_fwd", d, deg, dtype, true)) return rc;
+  if (bad_ptr(K) || bad_ptr(V) || bad_ptr(S) || bad_ptr(s)) return fail(PR_ERR_ARG, "update_state_fwd: null or misaligned pointer");
+  if (BN <= 0 || c <= 0 || h <= 0) return fail(PR_ERR_ARG, "update_state_fwd: need BN,c,h > 0");
+  return finish(pr::sympow_tn(K, V, nullptr, S, s, BN, c, h, 1, d, 1, dtype, (hipStream_t)stream), "update_state_fwd");
+}
+
+int pr_update_state_bwd(const void* K, const void* V, const void* dS, const float* ds, void* dK, void* dV, int BN,
+                        int c, int h, int d, int deg, int dtype, void* stream) {
+  if (int rc = check_common("update_state_bwd", d, deg, dtype, true)) return rc;
+  if (bad_ptr(K) || bad_ptr(V) || bad_ptr(dS) || bad_ptr(ds) || bad_ptr(dK) || bad_ptr(dV))
+    return fail(PR_ERR_ARG, "update_state_bwd: null or misaligned pointer");
+  if (BN <= 0 || c <= 0 || h <= 0) return fail(PR_ERR_ARG, "update_state_bwd: need BN,c,h > 0");
+  pr::NNArgs nn{K, dS, nullptr, dV, nullptr, nullptr, nullptr, nullptr, 1.f, c, h, 1, 1, 0};
+  if (int rc = finish(pr::sympow_nn(nn, BN, d, 1, 0, dtype, (hipStream_t)stream), "update_state_bwd(dV)")) return rc;
+  pr::GradArgs g{K, V, nullptr, dS, ds, dK, c, h, 1, 1, 0};
+  return finish(pr::sympow_grad(g, BN, d, 1, dtype, (hipStream_t)stream), "update_state_bwd(dK)");
+}
+
+int pr_discumsum_fwd(const void* X, const float* log_G, void* Y, int B, int n, int n_out, int H, int64_t F,
+                     int dtype, void* stream) {
+  if (dtype != PR_BF16 && dtype != PR_F16 && dtype != PR_F32) return fail(PR_ERR_DTYPE, "discumsum_fwd: unsupported dtype");
+  if (bad_ptr(X) || bad_ptr(Y) || log_G == nullptr) return fail(PR_ERR_ARG, "discumsum_fwd: null or misaligned pointer");
+  const int vec = dtype == PR_F32 ? 4 : 8;
+  if (B <= 0 || n <= 0 || H <= 0 || F <= 0 || F % vec != 0 || (n_out != n && n_out != n + 1))
+    return fail(PR_ERR_ARG, "discumsum_fwd: need B,n,H > 0, F a multiple of %d, n_out in {n, n+1}", vec);
+  return finish(pr::discumsum_fwd(X, log_G, Y, B, n, n_out, H, (long)F, dtype, (hipStream_t)stream), "discumsum_fwd");
+}
+
+size_t pr_discumsum_bwd_workspace(int B, int n, int H, int64_t F, int dtype) {
+  return (size_t)pr::discumsum_bwd_workspace_floats(B, n, H, (long)F, dtype) * sizeof(float);
+}
+
+int pr_discumsum_bwd(const void* dY, const void* Y, const float* log_G, void* dX, float* dlog_G, void* workspace,
+                     int B, int n, int n_out, int H, int64_t F, int dtype, void* stream) {
+  if (dtype != PR_BF16 && dtype != PR_F16 && dtype != PR_F32) return fail(PR_ERR_DTYPE, "discumsum_bwd: unsupported dtype");
+  if (bad_ptr(dY) || bad_ptr(Y) || log_G == nullptr || bad_ptr(dX) || dlog_G == nullptr || bad_ptr(workspace))
+    return fail(PR_ERR_ARG, "discumsum_bwd: null or misaligned pointer");
+  const int vec = dtype == PR_F32 ? 4 : 8;
+  if (B <= 0 || n <= 0 || H <= 0 || F <= 0 || F % vec != 0 || (n_out != n && n_out != n + 1))
+    return fail(PR_ERR_ARG, "discumsum_bwd: need B,n,H > 0, F a multiple of %d, n_out in {n, n+1}", vec);
+  return finish(pr::discumsum_bwd(dY, Y, log_G, dX, dlog_G, (float*)workspace, B, n, n_out, H, (long)F, dtype,
+                                  (hipStream_t)stream), "discumsum_bwd");
+}
+
+int pr_query_state_fwd(const void* Q, const void* S, const float* s, const void* Y_attn, const float* l_attn,
+                       const float* rowmax, void* O, float* den, int BN, int n, int c, int h, int r, int d,
+                       float scale_p, int deg, int zero_initial_state, int dtype, void* stream) {
+  if (int rc = check_common("query_state_fwd", d, deg, dtype, true)) return rc;
+  if (bad_ptr(Q) || bad_ptr(S) || bad_ptr(s) || bad_ptr(O) || bad_ptr(den) || bad_opt(Y_attn) || bad_opt(l_attn) ||
+      bad_opt(rowmax))
+    return fail(PR_ERR_ARG, "query_state_fwd: null or misaligned pointer");
+  if ((Y_attn != nullptr) != (l_attn != nullptr) || (Y_attn != nullptr) != (rowmax != nullptr))
+    return fail(PR_ERR_ARG, "query_state_fwd: Y_attn, l_attn and rowmax must be given together");
+  if (BN <= 0 || n <= 0 || c <= 0 || h <= 0 || r <= 0 || BN % n != 0)
+    return fail(PR_ERR_ARG, "query_state_fwd: need BN,n,c,h,r > 0 and BN a multiple of n");
+  pr::NNArgs a{Q, S, s, O, den, Y_attn, l_attn, rowmax, scale_p, c, h, r, n, zero_initial_state ? 1 : 0};
+  return finish(pr::sympow_nn(a, BN, d, 0, 1, dtype, (hipStream_t)stream), "query_state_fwd");
+}
+
+size_t pr_query_state_bwd_workspace(int BN, int c, int h, int r, int d, int dtype) {
+  (void)dtype;
+  const size_t rows = (size_t)BN * c * h * r;
+  return align256(rows * d * 2) + align256(rows * sizeof(float));
+}
+
+int pr_query_state_bwd(const void* Q, const void* S, const float* s, const float* rowmax, const void* O,
+                       const float* den, const void* dO, void* dQ, void* dS, float* ds, void* dY_attn,
+                       float* dl_attn, void* workspace, int BN, int n, int c, int h, int r, int d, float scale_p,
+                       int deg, int zero_initial_state, int dtype, void* stream) {
+  if (int rc = check_common("query_state_bwd", d, deg, dtype, true)) return rc;
+  if (bad_ptr(Q) || bad_ptr(S) || bad_ptr(s) || bad_ptr(O) || bad_ptr(den) || bad_ptr(dO) || bad_ptr(dQ) ||
+      bad_ptr(dS) || bad_ptr(ds) || bad_ptr(workspace) || bad_opt(rowmax) || bad_opt(dY_attn) || bad_opt(dl_attn))
+    return fail(PR_ERR_ARG, "query_state_bwd: null or misaligned pointer");
+  if (rowmax && (!dY_attn || !dl_attn)) return fail(PR_ERR_ARG, "query_state_bwd: dY_attn and dl_attn are required when rowmax is given");
+  if (BN <= 0 || n <= 0 || c <= 0 || h <= 0 || r <= 0 || BN % n != 0)
+    return fail(PR_ERR_ARG, "query_state_bwd: need BN,n,c,h,r > 0 and BN a multiple of n");
+  const size_t rows = (size_t)BN * c * h * r;
+  void* dOs = workspace;
+  float* cvec = (float*)((char*)workspace + align256(rows * d * 2));
+  hipStream_t st = (hipStream_t)stream;
+  if (int rc = finish(pr::qs_bwd_prep(O, dO, den, rowmax, dOs, cvec, rowmax ? dY_attn : nullptr,
+                                      rowmax ? dl_attn : nullptr, (long)rows, d, scale_p, dtype, st),
+                      "query_state_bwd(prep)"))
+    return rc;
+  if (int rc = finish(pr::sympow_tn(Q, dOs, cvec, dS, ds, BN, c, h, r, d, 0, dtype, st), "query_state_bwd(dS)")) return rc;
+  pr::GradArgs g{Q, dOs, cvec, S, s, dQ, c, h, r, n, zero_initial_state ? 1 : 0};
+  return finish(pr::sympow_grad(g, BN, d, 0, dtype, st), "query_state_bwd(dQ)");
+}
+
+}  // extern "C"

@@ -1,0 +1,173 @@
+// Gated exclusive scan over the chunk axis (HBM-bound).
+//
+//   Y[0] = 0,  Y[k+1] = Y[k] * exp(log_G[k]) + X[k]
+//
+// X: [B, n, H, F], log_G: [B, n, H] fp32, Y: [B, n_out, H, F] with n_out = n + 1 (the reference
+// operator, retention/_discumsum/reference.py:3-15) or n (the composed path keeps only the first
+// n entries, retention/power_retention_maker.py:167-170).  Every thread owns 16 bytes of the
+// feature axis and walks the chunks in order with an fp32 running state; loads for the next
+// chunks are issued ahead of the dependent multiply-add so the walk is bandwidth bound.
+#include "common.h"
+#include "kernels.h"
+
+namespace pr {
+
+template <typename T> struct Pack16 { enum { N = 16 / sizeof(T) }; typedef __attribute__((ext_vector_type(16 / sizeof(T)))) T type; };
+
+template <typename T, int AHEAD>
+__global__ __launch_bounds__(256) void discumsum_fwd_kernel(const T* __restrict__ X, const float* __restrict__ logG,
+                                                            T* __restrict__ Y, int n, int n_out, int H, long F) {
+  constexpr int N = Pack16<T>::N;
+  typedef typename Pack16<T>::type vec;
+  const long per_bh = F / N;
+  const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  const int bh = blockIdx.y;
+  if (idx >= per_bh) return;
+  const int b = bh / H, hh = bh % H;
+  const vec* x = (const vec*)(X + ((long)b * n * H + hh) * F) + idx;
+  vec* y = (vec*)(Y + ((long)b * n_out * H + hh) * F) + idx;
+  const long xs = (long)H * F / N;  // stride between chunks, in vectors
+  const float* lg = logG + (long)b * n * H + hh;
+
+  float st[N];
+#pragma unroll
+  for (int i = 0; i < N; i++) st[i] = 0.f;
+  vec zero;
+#pragma unroll
+  for (int i = 0; i < N; i++) zero[i] = (T)0.f;
+  y[0] = zero;
+
+  const int steps = n_out - 1;  // chunks that are consumed
+  vec buf[AHEAD];
+#pragma unroll
+  for (int a = 0; a < AHEAD; a++)
+    if (a < steps) buf[a] = x[(long)a * xs];
+  for (int k0 = 0; k0 < steps; k0 += AHEAD) {
+#pragma unroll
+    for (int a = 0; a < AHEAD; a++) {
+      const int k = k0 + a;
+      if (k < steps) {
+        const vec cur = buf[a];
+        if (k + AHEAD < steps) buf[a] = x[(long)(k + AHEAD) * xs];
+        const float g = (k == 0) ? 0.f : __expf(lg[(long)k * H]);
+        vec o;
+#pragma unroll
+        for (int i = 0; i < N; i++) {
+          st[i] = st[i] * g + to_f32(cur[i]);
+          o[i] = (T)st[i];
+        }
+        y[(long)(k + 1) * xs] = o;
+      }
+    }
+  }
+}
+
+// Reverse scan: r_k = dY[k+1] + exp(log_G[k+1]) * r_{k+1};  dX[k] = r_k;
+// dlog_G[k] = exp(log_G[k]) * sum_F Y[k] * r_k, written as one partial per wave (summed by
+// discumsum_reduce_kernel in a fixed order, so the result is deterministic).
+template <typename T>
+__global__ __launch_bounds__(256) void discumsum_bwd_kernel(const T* __restrict__ dY, const T* __restrict__ Y,
+                                                            const float* __restrict__ logG, T* __restrict__ dX,
+                                                            float* __restrict__ partial, int n, int n_out, int H,
+                                                            long F, int waves_per_bh) {
+  constexpr int N = Pack16<T>::N;
+  typedef typename Pack16<T>::type vec;
+  const long per_bh = F / N;
+  const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  const int bh = blockIdx.y;
+  const bool live = idx < per_bh;
+  const int b = bh / H, hh = bh % H;
+  const long safe = live ? idx : 0;
+  const vec* dy = (const vec*)(dY + ((long)b * n_out * H + hh) * F) + safe;
+  const vec* y = (const vec*)(Y + ((long)b * n_out * H + hh) * F) + safe;
+  vec* dx = (vec*)(dX + ((long)b * n * H + hh) * F) + safe;
+  const long xs = (long)H * F / N;
+  const float* lg = logG + (long)b * n * H + hh;
+  const int wave = (blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+  float* part = partial + ((long)bh * waves_per_bh + wave) * n;
+
+  float r[N];
+#pragma unroll
+  for (int i = 0; i < N; i++) r[i] = 0.f;
+  float g_next = 0.f;  // exp(log_G[k+1]); r_n = 0 so its value at k = n-1 is irrelevant
+  for (int k = n - 1; k >= 0; k--) {
+    vec d, yk;
+    const bool has = (k + 1 < n_out);
+    if (has) d = dy[(long)(k + 1) * xs];
+    yk = y[(long)k * xs];
+    const float gk = __expf(lg[(long)k * H]);
+    float dot = 0.f;
+    vec o;
+#pragma unroll
+    for (int i = 0; i < N; i++) {
+      r[i] = r[i] * g_next + (has ? to_f32(d[i]) : 0.f);
+      o[i] = (T)r[i];
+      dot += to_f32(yk[i]) * r[i];
+    }
+    if (live) dx[(long)k * xs] = o;
+    dot = wave_sum(live ? dot : 0.f);
+    if (lane_id() == 0) part[k] = dot * gk;
+    g_next = gk;
+  }
+}
+
+__global__ void discumsum_reduce_kernel(const float* __restrict__ partial, float* __restrict__ dlogG, int n, int H,
+                                        int waves_per_bh, int BH) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;  // over BH * n
+  if (i >= BH * n) return;
+  const int bh = i / n, k = i % n;
+  const int b = bh / H, hh = bh % H;
+  float s = 0.f;
+  for (int w = 0; w < waves_per_bh; w++) s += partial[((long)bh * waves_per_bh + w) * n + k];
+  dlogG[((long)b * n + k) * H + hh] = s;
+}
+
+template <typename T>
+static int launch_fwd(const void* X, const float* logG, void* Y, int B, int n, int n_out, int H, long F, hipStream_t st) {
+  constexpr int N = Pack16<T>::N;
+  const long per_bh = F / N;
+  dim3 grid((unsigned)((per_bh + 255) / 256), (unsigned)(B * H));
+  hipLaunchKernelGGL((discumsum_fwd_kernel<T, 4>), grid, dim3(256), 0, st, (const T*)X, logG, (T*)Y, n, n_out, H, F);
+  return (int)hipGetLastError();
+}
+template <typename T>
+static int launch_bwd(const void* dY, const void* Y, const float* logG, void* dX, float* dlogG, float* partial, int B,
+                      int n, int n_out, int H, long F, hipStream_t st) {
+  constexpr int N = Pack16<T>::N;
+  const long per_bh = F / N;
+  const unsigned blocks = (unsigned)((per_bh + 255) / 256);
+  const int waves = blocks * 4;
+  dim3 grid(blocks, (unsigned)(B * H));
+  hipLaunchKernelGGL((discumsum_bwd_kernel<T>), grid, dim3(256), 0, st, (const T*)dY, (const T*)Y, logG, (T*)dX, partial,
+                     n, n_out, H, F, waves);
+  const int tot = B * H * n;
+  hipLaunchKernelGGL(discumsum_reduce_kernel, dim3((tot + 255) / 256), dim3(256), 0, st, partial, dlogG, n, H, waves,
+                     B * H);
+  return (int)hipGetLastError();
+}
+
+int discumsum_fwd(const void* X, const float* logG, void* Y, int B, int n, int n_out, int H, long F, int dtype,
+                  hipStream_t st) {
+  switch (dtype) {
+    case DT_BF16: return launch_fwd<bf16_t>(X, logG, Y, B, n, n_out, H, F, st);
+    case DT_F16: return launch_fwd<f16_t>(X, logG, Y, B, n, n_out, H, F, st);
+    case DT_F32: return launch_fwd<float>(X, logG, Y, B, n, n_out, H, F, st);
+  }
+  return -1;
+}
+long discumsum_bwd_workspace_floats(int B, int n, int H, long F, int dtype) {
+  const int N = dtype == DT_F32 ? 4 : 8;
+  const long blocks = (F / N + 255) / 256;
+  return (long)B * H * blocks * 4 * n;
+}
+int discumsum_bwd(const void* dY, const void* Y, const float* logG, void* dX, float* dlogG, float* partial, int B, int n,
+                  int n_out, int H, long F, int dtype, hipStream_t st) {
+  switch (dtype) {
+    case DT_BF16: return launch_bwd<bf16_t>(dY, Y, logG, dX, dlogG, partial, B, n, n_out, H, F, st);
+    case DT_F16: return launch_bwd<f16_t>(dY, Y, logG, dX, dlogG, partial, B, n, n_out, H, F, st);
+    case DT_F32: return launch_bwd<float>(dY, Y, logG, dX, dlogG, partial, B, n, n_out, H, F, st);
+  }
+  return -1;
+}
+
+}  // namespace pr

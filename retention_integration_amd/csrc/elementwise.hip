@@ -1,0 +1,76 @@
+// Row-wise preparation for the query_state backward (formulas: retention/_query_state/triton.py:546-553):
+//   delta = sum_e O*dO,  beta = max(rowmax, log sqrt(D)),  f = 1/den,
+//   w_attn = exp(rowmax - beta),  w_qs = scale^p * exp(-beta)       (w_attn = 0, w_qs = 1 without attention part)
+//   dOs = w_qs f dO,  cvec = -w_qs f delta,  dY_attn = w_attn f dO,  dl_attn = -w_attn f delta.
+#include "common.h"
+#include "kernels.h"
+
+namespace pr {
+
+template <typename T, int DH>
+__global__ __launch_bounds__(256) void qs_bwd_prep_kernel(const T* __restrict__ O, const T* __restrict__ dO,
+                                                          const float* __restrict__ den,
+                                                          const float* __restrict__ rowmax, T* __restrict__ dOs,
+                                                          float* __restrict__ cvec, T* __restrict__ dYa,
+                                                          float* __restrict__ dla, long rows, float scale_p) {
+  typedef typename VecOf<T>::v8 v8;
+  constexpr int LPR = DH / 8;  // lanes per row
+  const long gid = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  const long row = gid / LPR;
+  const int col = (int)(gid % LPR) * 8;
+  const bool live = row < rows;
+  const long r = live ? row : 0;
+  float o[8], g[8];
+  unpack8(*(const v8*)(O + r * DH + col), o);
+  unpack8(*(const v8*)(dO + r * DH + col), g);
+  float delta = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; i++) delta += o[i] * g[i];
+#pragma unroll
+  for (int m = 1; m < LPR; m <<= 1) delta += __shfl_xor(delta, m);
+  const float f = 1.f / den[r];
+  float wa = 0.f, wq = 1.f;
+  if (rowmax) {
+    constexpr int D = 128 * (DH / 16) * (DH / 16 + 1);
+    const float m = rowmax[r], beta = fmaxf(m, 0.5f * __logf((float)D));
+    wa = __expf(m - beta);
+    wq = scale_p * __expf(-beta);
+  }
+  if (!live) return;
+  float a[8], b[8];
+#pragma unroll
+  for (int i = 0; i < 8; i++) {
+    a[i] = g[i] * (wq * f);
+    b[i] = g[i] * (wa * f);
+  }
+  *(v8*)(dOs + r * DH + col) = pack8<T>(a);
+  if (dYa) *(v8*)(dYa + r * DH + col) = pack8<T>(b);
+  if (col == 0) {
+    cvec[r] = -wq * f * delta;
+    if (dla) dla[r] = -wa * f * delta;
+  }
+}
+
+template <typename T>
+static int prep_launch(const void* O, const void* dO, const float* den, const float* rowmax, void* dOs, float* cvec,
+                       void* dYa, float* dla, long rows, int d, float scale_p, hipStream_t st) {
+  const long threads = rows * (d / 8);
+  dim3 grid((unsigned)((threads + 255) / 256));
+#define PR_PREP(DD)                                                                                                    \
+  case DD:                                                                                                             \
+    hipLaunchKernelGGL((qs_bwd_prep_kernel<T, DD>), grid, dim3(256), 0, st, (const T*)O, (const T*)dO, den, rowmax,    \
+                       (T*)dOs, cvec, (T*)dYa, dla, rows, scale_p);                                                    \
+    break;
+  switch (d) { PR_PREP(32) PR_PREP(64) PR_PREP(128) default: return -2; }
+#undef PR_PREP
+  return (int)hipGetLastError();
+}
+
+int qs_bwd_prep(const void* O, const void* dO, const float* den, const float* rowmax, void* dOs, float* cvec,
+                void* dY_attn, float* dl_attn, long rows, int d, float scale_p, int dtype, hipStream_t st) {
+  if (dtype == DT_BF16) return prep_launch<bf16_t>(O, dO, den, rowmax, dOs, cvec, dY_attn, dl_attn, rows, d, scale_p, st);
+  if (dtype == DT_F16) return prep_launch<f16_t>(O, dO, den, rowmax, dOs, cvec, dY_attn, dl_attn, rows, d, scale_p, st);
+  return -1;
+}
+
+}  // namespace pr

@@ -1,0 +1,84 @@
+// Host-side entry points of the kernel translation units and their argument blocks.
+#pragma once
+#include <hip/hip_runtime.h>
+
+namespace pr {
+
+// discumsum.hip
+int discumsum_fwd(const void* X, const float* logG, void* Y, int B, int n, int n_out, int H, long F, int dtype,
+                  hipStream_t st);
+int discumsum_bwd(const void* dY, const void* Y, const float* logG, void* dX, float* dlogG, float* partial, int B,
+                  int n, int n_out, int H, long F, int dtype, hipStream_t st);
+long discumsum_bwd_workspace_floats(int B, int n, int H, long F, int dtype);
+
+// sympow_tn.hip: A [BN,c,h*r,d], Bm [BN,c,h*r,d], w [BN,c,h*r] or null -> S [BN,h,D,d], s [BN,h,D]
+int sympow_tn(const void* A, const void* Bm, const float* w, void* S, float* s, int BN, int c, int h, int r, int d,
+              int use_mult, int dtype, hipStream_t st);
+
+// sympow_nn.hip
+enum { NN_EPI_PLAIN = 0, NN_EPI_MERGE = 1 };
+struct NNArgs {
+  const void* X;        // [BN, c, h*r, d]
+  const void* B;        // [BN, h, D, d]
+  const float* sB;      // [BN, h, D] or null
+  void* out;            // [BN, c, h*r, d]
+  float* den;           // [BN, c, h*r]   (merge only)
+  const void* Y_attn;   // [BN, c, h*r, d] or null
+  const float* l_attn;  // [BN, c, h*r]
+  const float* rowmax;  // [BN, c, h*r]
+  float scale_p;        // scale^deg
+  int c, h, r, n;       // n: chunks per batch entry
+  int skip_first;       // chunk 0 of every batch entry has a zero state
+};
+int sympow_nn(const NNArgs& a, int BN, int d, int mult, int epi, int dtype, hipStream_t st);
+
+// sympow_grad.hip
+struct GradArgs {
+  const void* X;      // [BN, c, h*r, d]
+  const void* G;      // [BN, c, h*r, d]
+  const float* cvec;  // [BN, c, h*r] or null (= 1)
+  const void* B;      // [BN, h, D, d]
+  const float* sB;    // [BN, h, D]
+  void* dX;           // [BN, c, h*r, d]
+  int c, h, r, n;
+  int skip_first;     // chunk 0 of every batch entry has a zero state: dX = 0 there
+};
+int sympow_grad(const GradArgs& a, int BN, int d, int mult, int dtype, hipStream_t st);
+
+// attention_fwd.hip / attention_bwd.hip
+struct AttnFwdArgs {
+  const void* Q;    // [B, tq, h*r, d]
+  const void* K;    // [B, tk, h, d]
+  const void* V;    // [B, tk, h, d]
+  const float* G;   // [B, tk, h] accumulated log gate, or null
+  void* O;          // [B, tq, h*r, d]
+  float* l;         // [B, tq, h*r]
+  float* rowmax;    // [B, tq, h*r]
+  int tq, tk, h, r;
+  float scale, deg;
+  int norm;
+};
+int attention_fwd(const AttnFwdArgs& a, int B, int d, int dtype, hipStream_t st);
+struct AttnBwdArgs {
+  const void* Q;        // [B, tq, h*r, d]
+  const void* K;        // [B, tk, h, d]
+  const void* V;        // [B, tk, h, d]
+  const float* G;       // [B, tk, h] or null
+  const float* rowmax;  // [B, tq, h*r]
+  const void* dO;       // [B, tq, h*r, d]
+  const float* dl;      // [B, tq, h*r] or null
+  void* dQ;             // [B, tq, h*r, d]
+  void* dK;             // [B, tk, h, d]
+  void* dV;             // [B, tk, h, d]
+  float* dGq;           // [B, tq, h*r]   (only when G)
+  float* dGk;           // [B, tk, h]     (only when G; already negated)
+  int tq, tk, h, r;
+  float scale, deg;
+};
+int attention_bwd(const AttnBwdArgs& a, int B, int d, int dtype, hipStream_t st);
+
+// elementwise.hip
+int qs_bwd_prep(const void* O, const void* dO, const float* den, const float* rowmax, void* dOs, float* cvec,
+                void* dY_attn, float* dl_attn, long rows, int d, float scale_p, int dtype, hipStream_t st);
+
+}  // namespace pr

@@ -1,0 +1,184 @@
+"""GPU parity of the four HIP operators (through the C ABI) against the CPU oracle.
+
+The oracle runs in fp32 on the same 16-bit-rounded inputs; the bar is the one the benchmark contract
+states: relative L2 error <= 1e-2 on outputs and <= 2e-2 on gradients.
+"""
+import math
+
+import pytest
+import torch
+
+import oracle
+
+pytestmark = pytest.mark.gpu
+
+OUT_TOL, GRAD_TOL = 1e-2, 2e-2
+DEV = "cuda"
+
+
+def rel_l2(got, want):
+    got, want = got.detach().float().cpu(), want.detach().float().cpu()
+    return ((got - want).norm() / want.norm().clamp_min(1e-30)).item()
+
+
+def check(name, got, want, tol):
+    assert got.shape == want.shape, f"{name}: shape {tuple(got.shape)} vs {tuple(want.shape)}"
+    assert torch.isfinite(got.float()).all(), f"{name}: non-finite values"
+    err = rel_l2(got, want)
+    print(f"  {name}: rel-L2 {err:.3e}", flush=True)
+    assert err <= tol, f"{name}: rel-L2 {err:.3e} > {tol}"
+
+
+def rnd(*shape, dtype, scale=1.0, seed=None):
+    g = torch.Generator().manual_seed(seed if seed is not None else hash(shape) % 2 ** 31)
+    return (torch.randn(*shape, generator=g) * scale).to(dtype)
+
+
+def gates(*shape, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    return torch.nn.functional.logsigmoid(torch.randn(*shape, generator=g))
+
+
+def dev(x, grad=False):
+    if x is None:
+        return None
+    y = x.to(DEV)
+    return y.requires_grad_(True) if grad else y
+
+
+def gold(x, grad=False):
+    if x is None:
+        return None
+    y = x.float().clone() if x.is_floating_point() else x.clone()
+    return y.requires_grad_(True) if grad else y
+
+
+@pytest.fixture(scope="module")
+def pra():
+    import retention_integration_amd as pra
+    return pra
+
+
+# ---------------------------------------------------------------- discumsum
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("keep_last", [True, False])
+def test_discumsum(pra, dtype, keep_last):
+    b, n, h, D, e = 2, 5, 3, 256, 16
+    X, lg, dY = rnd(b, n, h, D, e, dtype=dtype, seed=1), gates(b, n, h, seed=2), None
+    Xg, lgg = dev(X, True), dev(lg, True)
+    Y = pra.discumsum(Xg, lgg, keep_last=keep_last)
+    Xo, lgo = gold(X, True), gold(lg, True)
+    Yo = oracle.discumsum(Xo, lgo)
+    if not keep_last:
+        Yo = Yo[:, :n]
+    check("Y", Y, Yo, OUT_TOL if dtype != torch.float32 else 1e-5)
+    dY = rnd(*Yo.shape, dtype=dtype, seed=3)
+    Y.backward(dev(dY))
+    Yo.backward(gold(dY))
+    check("dX", Xg.grad, Xo.grad, GRAD_TOL if dtype != torch.float32 else 1e-5)
+    check("dlog_G", lgg.grad, lgo.grad, GRAD_TOL if dtype != torch.float32 else 1e-4)
+
+
+def test_discumsum_1d_features(pra):
+    X, lg = rnd(1, 4, 2, 768, dtype=torch.float32, seed=4), gates(1, 4, 2, seed=5)
+    check("Y", pra.discumsum(dev(X), dev(lg)), oracle.discumsum(X, lg), 1e-5)
+
+
+# ---------------------------------------------------------------- update_state
+@pytest.mark.parametrize("dtype,d,c", [(torch.bfloat16, 64, 128), (torch.bfloat16, 32, 48), (torch.float16, 128, 64),
+                                       (torch.float16, 64, 32), (torch.bfloat16, 128, 32)])
+def test_update_state(pra, dtype, d, c):
+    b, n, h = 1, 2, 2
+    K, V = rnd(b, n, c, h, d, dtype=dtype, scale=d ** -0.25, seed=10), rnd(b, n, c, h, d, dtype=dtype, seed=11)
+    Kg, Vg = dev(K, True), dev(V, True)
+    S, s = pra.update_state(Kg, Vg, 2)
+    Ko, Vo = gold(K, True), gold(V, True)
+    So, so = oracle.update_state(Ko, Vo, 2)
+    check("S", S, So, OUT_TOL)
+    check("s", s, so, OUT_TOL)
+    dS, ds = rnd(*So.shape, dtype=dtype, seed=12), rnd(*so.shape, dtype=torch.float32, seed=13)
+    torch.autograd.backward([S, s], [dev(dS), dev(ds)])
+    torch.autograd.backward([So, so], [gold(dS), gold(ds)])
+    check("dK", Kg.grad, Ko.grad, GRAD_TOL)
+    check("dV", Vg.grad, Vo.grad, GRAD_TOL)
+
+
+def test_update_state_inference_form(pra):
+    K, V = rnd(2, 40, 2, 64, dtype=torch.bfloat16, scale=0.35, seed=14), rnd(2, 40, 2, 64, dtype=torch.bfloat16, seed=15)
+    S, s = pra.update_state(dev(K), dev(V), 2)
+    So, so = oracle.update_state(gold(K), gold(V), 2)
+    assert S.shape == (2, 2, 2560, 64) and s.shape == (2, 2, 2560)
+    check("S", S, So, OUT_TOL)
+    check("s", s, so, OUT_TOL)
+
+
+# ---------------------------------------------------------------- query_state
+@pytest.mark.parametrize("dtype,d,c,r,zis,attn", [
+    (torch.bfloat16, 64, 128, 1, True, True), (torch.bfloat16, 32, 40, 2, False, True),
+    (torch.float16, 128, 64, 1, True, True), (torch.bfloat16, 64, 256, 1, False, False),
+    (torch.bfloat16, 64, 16, 4, False, True)])
+def test_query_state(pra, dtype, d, c, r, zis, attn):
+    b, n, h = 1, 2, 2
+    D = oracle.expanded_dim(d)
+    Q = rnd(b, n, c, h * r, d, dtype=dtype, seed=20)
+    # a state that real keys produced, so the normaliser phi(Q).s = sum_j (q.k_j)^2 stays positive
+    Ks = rnd(b, n, 48, h, d, dtype=torch.float32, scale=d ** -0.25, seed=21)
+    Vs = rnd(b, n, 48, h, d, dtype=torch.float32, seed=22)
+    S, s = oracle.update_state(Ks, Vs, 2)
+    S = S.to(dtype)
+    assert S.shape == (b, n, h, D, d)
+    if zis:
+        S[:, 0] = 0
+        s[:, 0] = 0
+    Ya = rnd(b, n, c, h * r, d, dtype=dtype, seed=23) if attn else None
+    la = (rnd(b, n, c, h * r, dtype=torch.float32, seed=24).abs() + c) if attn else None
+    rm = (rnd(b, n, c, h * r, dtype=torch.float32, seed=25).abs() * 3 + 1.0) if attn else None
+    scale = 1.0 / math.sqrt(d)
+    g_in = [dev(Q, True), dev(S, True), dev(s, True), dev(Ya, attn), dev(la, attn)]
+    o_in = [gold(Q, True), gold(S, True), gold(s, True), gold(Ya, attn), gold(la, attn)]
+    O = pra.query_state(*g_in, dev(rm), 2, scale, zis)
+    Oo = oracle.query_state(*o_in, gold(rm), 2, scale, zis)
+    check("O", O, Oo, OUT_TOL)
+    dO = rnd(*Oo.shape, dtype=dtype, seed=26)
+    O.backward(dev(dO))
+    Oo.backward(gold(dO))
+    names = ["dQ", "dS", "ds", "dY_attn", "dl_attn"]
+    for nm, a, b_ in zip(names, g_in, o_in):
+        if a is None:
+            continue
+        ga, gb = a.grad, b_.grad
+        if zis and nm in ("dS", "ds"):  # chunk 0 state is declared zero: its gradient is not meaningful
+            ga, gb = ga[:, 1:], gb[:, 1:]
+        check(nm, ga, gb, GRAD_TOL)
+
+
+# ---------------------------------------------------------------- attention
+@pytest.mark.parametrize("dtype,d,tq,tk,r,gated,norm", [
+    (torch.bfloat16, 64, 128, 128, 1, True, False), (torch.bfloat16, 64, 200, 200, 1, False, True),
+    (torch.float16, 128, 96, 96, 1, True, False), (torch.bfloat16, 32, 1, 130, 2, True, False),
+    (torch.bfloat16, 64, 70, 150, 2, True, True), (torch.bfloat16, 64, 384, 384, 1, True, False)])
+def test_attention(pra, dtype, d, tq, tk, r, gated, norm):
+    b, h = 2, 2
+    Q, K, V = (rnd(b, tq, h * r, d, dtype=dtype, seed=30), rnd(b, tk, h, d, dtype=dtype, seed=31),
+               rnd(b, tk, h, d, dtype=dtype, seed=32))
+    A = gates(b, tk, h, seed=33).cumsum(1) if gated else None
+    scale = 1.0 / math.sqrt(d)
+    g_in = [dev(Q, True), dev(K, True), dev(V, True), dev(A, gated)]
+    o_in = [gold(Q, True), gold(K, True), gold(V, True), gold(A, gated)]
+    out = pra.attention(*g_in, 2, scale=scale, norm=norm)
+    ref = oracle.attention(*o_in, 2, scale=scale, norm=norm)
+    if norm:
+        check("Y", out, ref, OUT_TOL)
+        dY = rnd(*ref.shape, dtype=dtype, seed=34)
+        out.backward(dev(dY))
+        ref.backward(gold(dY))
+    else:
+        check("rowmax", out[2], ref[2], 1e-3)
+        check("l", out[1], ref[1], OUT_TOL)
+        check("o", out[0], ref[0], OUT_TOL)
+        dO, dl = rnd(*ref[0].shape, dtype=dtype, seed=35), rnd(*ref[1].shape, dtype=torch.float32, seed=36)
+        torch.autograd.backward([out[0], out[1]], [dev(dO), dev(dl)])
+        torch.autograd.backward([ref[0], ref[1]], [gold(dO), gold(dl)])
+    for nm, a, b_ in zip(["dQ", "dK", "dV", "dG"], g_in, o_in):
+        if a is not None:
+            check(nm, a.grad, b_.grad, GRAD_TOL)
