@@ -1,0 +1,186 @@
+"""GPU parity of the composed functions against the CPU oracle, the golden vectors written from the
+reference, and size-independent invariants at larger shapes (ref test strategy:
+perf/tests/chunk_consistency_tests.py:21-45, perf/tests/inference_tests.py:38-51, perf/tests/gqa_tests.py:72-129).
+"""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+
+pytestmark = pytest.mark.gpu
+
+OUT_TOL, GRAD_TOL = 1e-2, 2e-2
+DEV = "cuda"
+G = os.path.join(os.path.dirname(__file__), "golden")
+
+
+def rel_l2(got, want):
+    got, want = got.detach().float().cpu(), want.detach().float().cpu()
+    return ((got - want).norm() / want.norm().clamp_min(1e-30)).item()
+
+
+def check(name, got, want, tol):
+    assert got.shape == want.shape, f"{name}: shape {tuple(got.shape)} vs {tuple(want.shape)}"
+    assert torch.isfinite(got.float()).all(), f"{name}: non-finite values"
+    err = rel_l2(got, want)
+    print(f"  {name}: rel-L2 {err:.3e}", flush=True)
+    assert err <= tol, f"{name}: rel-L2 {err:.3e} > {tol}"
+
+
+def make_inputs(b, t, h, r, d, dtype, gated, seed=0, std=1.0):
+    g = torch.Generator().manual_seed(seed)
+    Q = (torch.randn(b, t, h * r, d, generator=g) * std).to(dtype)
+    K = (torch.randn(b, t, h, d, generator=g) * std).to(dtype)
+    V = (torch.randn(b, t, h, d, generator=g) * std).to(dtype)
+    lg = torch.nn.functional.logsigmoid(torch.randn(b, t, h, generator=g)) if gated else None
+    return Q, K, V, lg
+
+
+@pytest.fixture(scope="module")
+def pra():
+    import retention_integration_amd as pra
+    return pra
+
+
+def run_both(pra, Q, K, V, lg, chunk, dO=None, **kw):
+    gi = [x.to(DEV).requires_grad_(True) if x is not None else None for x in (Q, K, V, lg)]
+    oi = [x.float().clone().requires_grad_(True) if x is not None else None for x in (Q, K, V, lg)]
+    Y = pra.power_retention(*gi, deg=2, chunk_size=chunk, **kw)
+    Yo = oracle.power_retention(*oi, deg=2, chunk_size=chunk, **kw)
+    check("Y", Y, Yo, OUT_TOL)
+    if dO is not None:
+        Y.backward(dO.to(DEV))
+        Yo.backward(dO.float())
+        for nm, a, b_ in zip(["dQ", "dK", "dV", "dlog_G"], gi, oi):
+            if a is not None:
+                check(nm, a.grad, b_.grad, GRAD_TOL)
+    return Y
+
+
+@pytest.mark.parametrize("dtype,b,t,h,r,d,chunk,gated", [
+    (torch.bfloat16, 2, 1024, 8, 1, 64, 128, True),     # BASELINE config 1 shape (there in fp32 on the CPU)
+    (torch.bfloat16, 1, 512, 2, 2, 64, 128, True),      # GQA
+    (torch.bfloat16, 1, 300, 2, 1, 32, 64, True),       # padding (300 -> 320), d = 32
+    (torch.float16, 1, 512, 2, 1, 128, 128, False),     # config 5 flavour: fp16, d = 128, ungated
+    (torch.bfloat16, 1, 2048, 1, 1, 64, 1024, True),    # headline chunk size
+    (torch.bfloat16, 1, 96, 2, 1, 64, None, True),      # quadratic path
+])
+def test_power_retention_fwd_bwd(pra, dtype, b, t, h, r, d, chunk, gated):
+    std = 0.5 if dtype == torch.float16 else 1.0
+    Q, K, V, lg = make_inputs(b, t, h, r, d, dtype, gated, seed=t + d, std=std)
+    g = torch.Generator().manual_seed(7)
+    dO = torch.randn(b, t, h * r, d, generator=g).to(dtype)
+    run_both(pra, Q, K, V, lg, chunk, dO)
+
+
+def test_fp32_inputs_are_rejected_loudly(pra):
+    Q, K, V, lg = make_inputs(1, 256, 1, 1, 64, torch.float32, True)
+    with pytest.raises((AssertionError, TypeError, RuntimeError)):
+        pra.power_retention(*(x.to(DEV) for x in (Q, K, V, lg)), deg=2, chunk_size=128)
+
+
+def test_chunked_equals_quadratic_on_gpu(pra):
+    Q, K, V, lg = (x.to(DEV) for x in make_inputs(1, 1024, 4, 1, 64, torch.bfloat16, True, seed=3))
+    a = pra.power_retention(Q, K, V, lg, deg=2, chunk_size=128)
+    b_ = pra.power_retention(Q, K, V, lg, deg=2, chunk_size=None)
+    c_ = pra.power_retention(Q, K, V, lg, deg=2, chunk_size=256)
+    check("chunk128 vs quadratic", a, b_, OUT_TOL)
+    check("chunk256 vs quadratic", c_, b_, OUT_TOL)
+
+
+def test_gqa_equals_repeated_heads_on_gpu(pra):
+    Q, K, V, lg = (x.to(DEV) for x in make_inputs(1, 512, 2, 4, 64, torch.bfloat16, True, seed=4))
+    a = pra.power_retention(Q, K, V, lg, deg=2, chunk_size=128)
+    b_ = pra.power_retention(Q, K.repeat_interleave(4, 2), V.repeat_interleave(4, 2), lg.repeat_interleave(4, 2),
+                             deg=2, chunk_size=128)
+    check("gqa vs mha", a, b_, 2e-3)
+
+
+def load(name):
+    z = np.load(os.path.join(G, name))
+    return {k: torch.from_numpy(z[k]) if z[k].ndim else float(z[k]) for k in z.files}
+
+
+def test_golden_power_retention(pra):
+    v = load("power_retention_d32.npz")
+    bf = lambda x: x.to(torch.bfloat16).to(DEV)  # noqa: E731
+    Y = pra.power_retention(bf(v["Q"]), bf(v["K"]), bf(v["V"]), v["log_G"].to(DEV), deg=2, chunk_size=16)
+    check("Y vs reference (chunked)", Y, v["Y_chunked"], 1.5e-2)  # golden ran on unrounded fp32 inputs
+    Yq = pra.power_retention(bf(v["Q"]), bf(v["K"]), bf(v["V"]), v["log_G"].to(DEV), deg=2, chunk_size=None)
+    check("Y vs reference (quadratic)", Yq, v["Y_quadratic"], 1.5e-2)
+
+
+def test_golden_update_state_layout(pra):
+    v = load("update_state_d32.npz")
+    S, s = pra.update_state(v["K"].to(torch.bfloat16).to(DEV), v["V"].to(torch.bfloat16).to(DEV), 2)
+    check("S vs reference", S, v["S"], 1.5e-2)
+    check("s vs reference", s, v["N"], 1.5e-2)
+
+
+def test_golden_inference(pra):
+    v = load("inference_d32.npz")
+    bf = lambda x: x.to(torch.bfloat16).to(DEV)  # noqa: E731
+    Y0, st, sk = pra.power_retention_inference(bf(v["Q0"]), bf(v["K0"]), bf(v["V0"]), v["log_G0"].to(DEV), None, None,
+                                               deg=2, switch_over_seq_len=16)
+    check("Y0", Y0, v["Y0"], 1.5e-2)
+    check("state0", st, v["state0"], 1.5e-2)
+    check("sum_of_keys0", sk, v["sum_of_keys0"], 1.5e-2)
+    Y1, st1, sk1 = pra.power_retention_inference(bf(v["Q1"]), bf(v["K1"]), bf(v["V1"]), v["log_G1"].to(DEV),
+                                                 bf(v["state0"]), v["sum_of_keys0"].to(DEV), deg=2,
+                                                 switch_over_seq_len=3)
+    check("Y1", Y1, v["Y1"], 1.5e-2)
+    check("state1", st1, v["state1"], 1.5e-2)
+    check("sum_of_keys1", sk1, v["sum_of_keys1"], 1.5e-2)
+
+
+@pytest.mark.parametrize("gated", [True, False])
+def test_inference_prefill_then_decode_matches_oracle(pra, gated):
+    b, h, r, d, t0, steps = 2, 2, 2, 64, 256, 4
+    Q, K, V, lg = make_inputs(b, t0 + steps, h, r, d, torch.bfloat16, gated, seed=11)
+    sl = lambda x, a, e: None if x is None else x[:, a:e]  # noqa: E731
+    dv = lambda x: None if x is None else x.to(DEV)  # noqa: E731
+    f32 = lambda x: None if x is None else x.float()  # noqa: E731
+    Y, st, sk = pra.power_retention_inference(dv(Q[:, :t0]), dv(K[:, :t0]), dv(V[:, :t0]), dv(sl(lg, 0, t0)), None, None,
+                                              deg=2, switch_over_seq_len=t0)
+    Yo, sto, sko = oracle.power_retention_inference(f32(Q[:, :t0]), f32(K[:, :t0]), f32(V[:, :t0]), sl(lg, 0, t0), None,
+                                                    None, deg=2, switch_over_seq_len=t0)
+    check("prefill Y", Y, Yo, OUT_TOL)
+    check("prefill state", st, sto, OUT_TOL)
+    check("prefill sum_of_keys", sk, sko, OUT_TOL)
+    for i in range(t0, t0 + steps):  # recurrent decode: query the state, then fold the new token in
+        a = (dv(Q[:, i:i + 1]), dv(K[:, i:i + 1]), dv(V[:, i:i + 1]), dv(sl(lg, i, i + 1)))
+        o = (f32(Q[:, i:i + 1]), f32(K[:, i:i + 1]), f32(V[:, i:i + 1]), sl(lg, i, i + 1))
+        Y, st, sk = pra.power_retention_inference(*a, st, sk, deg=2, switch_over_seq_len=1)
+        Yo, sto, sko = oracle.power_retention_inference(*o, sto, sko, deg=2, switch_over_seq_len=1)
+        check(f"decode {i} Y", Y, Yo, OUT_TOL)
+    check("final state", st, sto, OUT_TOL)
+    check("final sum_of_keys", sk, sko, OUT_TOL)
+
+
+def test_inference_state_parity_on_gpu(pra):
+    Q, K, V, _ = make_inputs(1, 129, 2, 2, 64, torch.bfloat16, False, seed=12)
+    q = Q[:, -1:].to(DEV)
+    Y, st, sk = pra.power_retention_inference(q, K.to(DEV), V.to(DEV), None, None, None, deg=2, switch_over_seq_len=129)
+    Y2, st2, sk2 = pra.power_retention_inference(q, None, None, None, st, sk, deg=2, switch_over_seq_len=129)
+    check("Y from state vs Y from cache", Y2, Y, OUT_TOL)
+    assert st2 is st and sk2 is sk
+
+
+def test_large_shape_invariants(pra):
+    """Headline shape: finite output, normalised rows (V = 1 -> Y = 1), linearity in V."""
+    b, t, h, d, c = 1, 65536, 8, 64, 1024
+    Q, K, V, lg = (x.to(DEV) for x in make_inputs(b, t, h, 1, d, torch.bfloat16, True, seed=5))
+    Y = pra.power_retention(Q, K, V, lg, deg=2, chunk_size=c)
+    assert Y.shape == (b, t, h, d) and torch.isfinite(Y.float()).all()
+    ones = pra.power_retention(Q, K, torch.ones_like(V), lg, deg=2, chunk_size=c)
+    err = (ones.float() - 1).abs()
+    print(f"  V=1 -> max |Y-1| = {err.max().item():.3e}, rms = {err.pow(2).mean().sqrt().item():.3e}", flush=True)
+    assert err.pow(2).mean().sqrt().item() < 1e-2 and err.max().item() < 1e-1  # bf16 state: a few ulp at worst
+    Y2 = pra.power_retention(Q, K, 2 * V, lg, deg=2, chunk_size=c)
+    check("linearity in V", Y2, 2 * Y.float(), 1e-2)
+    # the first chunk sees no state: it must equal quadratic attention on that chunk alone
+    Yq = pra.power_retention(Q[:, :c], K[:, :c], V[:, :c], lg[:, :c], deg=2, chunk_size=None)
+    check("chunk 0 vs quadratic", Y[:, :c], Yq, 1e-2)
