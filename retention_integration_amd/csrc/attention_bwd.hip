@@ -4,11 +4,16 @@
 //
 //   P = exp(z - m),  dP = dO V^T + dl,  dz = P * dP,  dV = P^T dO,
 //   dGq_i = sum_j dz_ij,  dGk_j = -sum_i dz_ij,
-//   dsr = dz * deg * scale * sign(s) / (|s| + 1e-7),  dQ = dsr K,  dK = dsr^T Q.
+//   d(q.k) = dz * deg * sign(s) / (|q.k| + 1e-7/scale),  dQ = d(q.k) K,  dK = d(q.k)^T Q.
 //
 // Two kernels, each recomputing P: one owns query rows and walks the keys (dQ, dGq), the other owns keys
 // and walks the query rows (dK, dV, dGk).  Products are oriented so that every accumulator layout is
 // already the operand layout of the next contraction (see attention_fwd.hip).
+//
+// No logarithm or division per pair: with a = |q.k| + eps/scale,
+//   P = a^deg * E,  E = scale^deg * exp(G_q - m - G_k),  d(q.k)/deg = sign(s) * a^(deg-1) * E * dP,
+// and away from the diagonal E factors into a per-row and a per-key exponential around a reference
+// gate R (the gate at the last key of the key tile, so both exponents are <= 0 for decaying gates).
 #include "common.h"
 #include "kernels.h"
 
@@ -16,19 +21,40 @@ namespace pr {
 
 constexpr int AB_BN = 64;   // keys per step in the dQ kernel
 constexpr int AB_BM = 32;   // query rows per step in the dK/dV kernel
-constexpr float AB_LOG_EPS = 1e-7f;
+constexpr float AB_LOG_EPS = 1e-7f, AB_EXP_CLAMP = 80.f;
+
+// a^(deg-2) for even deg
+template <bool DEG2> __device__ __forceinline__ float pow_m2(float a, int half_deg) {
+  if (DEG2) return 1.f;
+  const float a2 = a * a;
+  float p = 1.f;
+  for (int k = 1; k < half_deg; k++) p *= a2;
+  return p;
+}
+
+// One pair: s = raw q.k, E as above, dpl = dP (incl. dl).  Returns P, dz and d(q.k)/deg.
+template <bool DEG2>
+__device__ __forceinline__ void pair_grad(float s, float E, float dpl, float eps_s, int half_deg, float& p, float& dz,
+                                          float& dsr) {
+  const float as = fabsf(s) + eps_s;
+  const float t1 = pow_m2<DEG2>(as, half_deg) * as * E;   // a^(deg-1) E
+  p = t1 * as;
+  dz = p * dpl;
+  dsr = copysignf(t1, s) * dpl;
+}
 
 // ------------------------------------------------------------------ dQ, dGq
-template <typename T, int DH, int MT>
-__global__ __launch_bounds__(256) void attention_bwd_dq_kernel(AttnBwdArgs a) {
+template <typename T, int DH, int MT, bool DEG2>
+__global__ __launch_bounds__(256, 2) void attention_bwd_dq_kernel(AttnBwdArgs a) {
   typedef typename VecOf<T>::v8 v8;
   typedef typename VecOf<T>::v4 v4;
   constexpr int LD = DH + 8, KS = DH / 32, NT = DH / 16, KT = AB_BN / 16, ROWS = 64 * MT;
   constexpr int CH = AB_BN * DH / 8, PT = (CH + 255) / 256;
+  constexpr int GS = 2 * AB_BN + 4;
   extern __shared__ __attribute__((aligned(16))) char smem[];
   T* Kt = (T*)smem;
   T* Vt = Kt + 2 * AB_BN * LD;
-  float* gk = (float*)(Vt + 2 * AB_BN * LD);
+  float* gk = (float*)(Vt + 2 * AB_BN * LD);   // [2][GS]: raw gate [BN], exp(R - gate) [BN], R
 
   const int tid = threadIdx.x, l = tid & 63, g = l >> 4, wave = tid >> 6, tcol = l & 15;
   const int b = blockIdx.y / a.h, hh = blockIdx.y % a.h;
@@ -40,12 +66,15 @@ __global__ __launch_bounds__(256) void attention_bwd_dq_kernel(AttnBwdArgs a) {
   const T* Vg = (const T*)a.V + (long)b * a.tk * a.h * DH + hh * DH;
   const float* Gg = a.G ? a.G + (long)b * a.tk * a.h + hh : nullptr;
   const long kstride = (long)a.h * DH;
+  const int half_deg = (int)a.deg / 2;
+  const float eps_s = AB_LOG_EPS / a.scale;
+  const float scale_p = __powf(a.scale, a.deg);
 
   v8 Qf[MT][KS], dOf[MT][KS];
   int ti[MT];
   long qoff[MT];
   bool live[MT];
-  float Gq[MT], mrow[MT], dlr[MT], dgq[MT];
+  float base[MT], dlr[MT], dgq[MT];   // base = G_q - m
 #pragma unroll
   for (int mi = 0; mi < MT; mi++) {
     const int row = row0 + wave * 16 * MT + 16 * mi + tcol;
@@ -65,8 +94,7 @@ __global__ __launch_bounds__(256) void attention_bwd_dq_kernel(AttnBwdArgs a) {
       dOf[mi][ks] = __builtin_bit_cast(v8, z2);
     }
     const long so = (long)b * a.tq * hq + qoff[mi];
-    Gq[mi] = Gg ? Gg[(long)ti[mi] * a.h] : 0.f;
-    mrow[mi] = a.rowmax[so];
+    base[mi] = (Gg ? Gg[(long)ti[mi] * a.h] : 0.f) - a.rowmax[so];
     dlr[mi] = a.dl ? a.dl[so] : 0.f;
     dgq[mi] = 0.f;
   }
@@ -82,7 +110,7 @@ __global__ __launch_bounds__(256) void attention_bwd_dq_kernel(AttnBwdArgs a) {
   const int ntiles = (kmax + AB_BN - 1) / AB_BN;
 
   u32x4 rk[PT], rv[PT];
-  float rg = 0.f;
+  float rg = 0.f, rR = 0.f;
   auto fetch = [&](int j0) {
 #pragma unroll
     for (int i = 0; i < PT; i++) {
@@ -95,7 +123,10 @@ __global__ __launch_bounds__(256) void attention_bwd_dq_kernel(AttnBwdArgs a) {
         rv[i] = *(const u32x4*)(Vg + key * kstride + col);
       }
     }
-    if (tid < AB_BN) rg = (Gg && j0 + tid < a.tk) ? Gg[(long)(j0 + tid) * a.h] : 0.f;
+    if (tid < AB_BN && Gg) {
+      rg = Gg[(long)min(j0 + tid, a.tk - 1) * a.h];
+      rR = Gg[(long)min(j0 + AB_BN - 1, a.tk - 1) * a.h];
+    }
   };
   auto stash = [&](int stage) {
 #pragma unroll
@@ -107,10 +138,13 @@ __global__ __launch_bounds__(256) void attention_bwd_dq_kernel(AttnBwdArgs a) {
         *(u32x4*)(Vt + o) = rv[i];
       }
     }
-    if (tid < AB_BN) gk[stage * AB_BN + tid] = rg;
+    if (tid < AB_BN) {
+      gk[stage * GS + tid] = rg;
+      gk[stage * GS + AB_BN + tid] = __expf(fminf(rR - rg, AB_EXP_CLAMP));
+      if (tid == 0) gk[stage * GS + 2 * AB_BN] = rR;
+    }
   };
 
-  const float cds = a.deg * a.scale;
   fetch(0);
   for (int it = 0; it < ntiles; it++) {
     const int j0 = it * AB_BN, stage = it & 1;
@@ -119,8 +153,12 @@ __global__ __launch_bounds__(256) void attention_bwd_dq_kernel(AttnBwdArgs a) {
     if (it + 1 < ntiles) fetch(j0 + AB_BN);
     const T* kt_ = Kt + stage * AB_BN * LD;
     const T* vt_ = Vt + stage * AB_BN * LD;
-    const float* gk_ = gk + stage * AB_BN;
-    const bool need_mask = (j0 + AB_BN - 1 > first_ti) || (j0 + AB_BN > a.tk);
+    const float* gk_ = gk + stage * GS;
+    const bool diag = (j0 + AB_BN - 1 > first_ti) || (j0 + AB_BN > a.tk);
+    const float R = gk_[2 * AB_BN];
+    float eu[MT];
+#pragma unroll
+    for (int mi = 0; mi < MT; mi++) eu[mi] = scale_p * (diag ? 1.f : __expf(fminf(base[mi] - R, AB_EXP_CLAMP)));
 
     v8 dsf[MT][KT / 2];
 #pragma unroll
@@ -135,7 +173,7 @@ __global__ __launch_bounds__(256) void attention_bwd_dq_kernel(AttnBwdArgs a) {
           kf[ks] = lds_frag<T>(kt_, LD, 16 * kt, 32 * ks);
           vf[ks] = lds_frag<T>(vt_, LD, 16 * kt, 32 * ks);
         }
-        const f32x4 gkv = *(const f32x4*)(gk_ + 16 * kt + 4 * g);
+        const f32x4 gkv = *(const f32x4*)(gk_ + (diag ? 0 : AB_BN) + 16 * kt + 4 * g);
 #pragma unroll
         for (int mi = 0; mi < MT; mi++) {
           f32x4 s = {0, 0, 0, 0}, dp = {0, 0, 0, 0};
@@ -146,16 +184,18 @@ __global__ __launch_bounds__(256) void attention_bwd_dq_kernel(AttnBwdArgs a) {
           }
 #pragma unroll
           for (int v = 0; v < 4; v++) {
-            const float ss = s[v] * a.scale;
-            const float as = fabsf(ss) + AB_LOG_EPS;
-            float p = __expf(a.deg * __logf(as) + (Gq[mi] - gkv[v]) - mrow[mi]);
-            if (need_mask) {
+            float E;
+            if (diag) {
               const int key = j0 + 16 * kt + 4 * g + v;
-              if (key > ti[mi] || key >= a.tk) p = 0.f;
+              E = eu[mi] * __expf(fminf(base[mi] - gkv[v], AB_EXP_CLAMP));
+              if (key > ti[mi] || key >= a.tk) E = 0.f;
+            } else {
+              E = eu[mi] * gkv[v];
             }
-            const float dz = p * (dp[v] + dlr[mi]);
+            float p, dz, dsr;
+            pair_grad<DEG2>(s[v], E, dp[v] + dlr[mi], eps_s, half_deg, p, dz, dsr);
             dgq[mi] += dz;
-            d8[mi][4 * half + v] = dz * cds * (ss < 0.f ? -1.f : 1.f) / as;
+            d8[mi][4 * half + v] = dsr;
           }
         }
       }
@@ -185,7 +225,7 @@ __global__ __launch_bounds__(256) void attention_bwd_dq_kernel(AttnBwdArgs a) {
     for (int nt = 0; nt < NT; nt++) {
       float o4[4];
 #pragma unroll
-      for (int v = 0; v < 4; v++) o4[v] = acc[mi][nt][v];
+      for (int v = 0; v < 4; v++) o4[v] = acc[mi][nt][v] * a.deg;
       *(v4*)(dQg + qoff[mi] * DH + 16 * nt + 4 * g) = pack4<T>(o4);
     }
     if (g == 0 && a.dGq) a.dGq[(long)b * a.tq * hq + qoff[mi]] = tot;
@@ -193,8 +233,8 @@ __global__ __launch_bounds__(256) void attention_bwd_dq_kernel(AttnBwdArgs a) {
 }
 
 // ------------------------------------------------------------------ dK, dV, dGk
-template <typename T, int DH, int MK>
-__global__ __launch_bounds__(256) void attention_bwd_dkv_kernel(AttnBwdArgs a) {
+template <typename T, int DH, int MK, bool DEG2>
+__global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a) {
   typedef typename VecOf<T>::v8 v8;
   typedef typename VecOf<T>::v4 v4;
   constexpr int LD = DH + 8, KS = DH / 32, NT = DH / 16, QT = AB_BM / 16, KEYS = 64 * MK;
@@ -202,7 +242,7 @@ __global__ __launch_bounds__(256) void attention_bwd_dkv_kernel(AttnBwdArgs a) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   T* Qt = (T*)smem;                       // [2][BM][LD]
   T* dOt = Qt + 2 * AB_BM * LD;           // [2][BM][LD]
-  float* rowv = (float*)(dOt + 2 * AB_BM * LD);  // [2][3][BM]: G_q - m, dl, time index
+  float* rowv = (float*)(dOt + 2 * AB_BM * LD);  // [2][4][BM]: G_q - m, dl, time index, scale^deg exp(G_q - m - R)
 
   const int tid = threadIdx.x, l = tid & 63, g = l >> 4, wave = tid >> 6, kcol = l & 15;
   const int b = blockIdx.y / a.h, hh = blockIdx.y % a.h;
@@ -214,11 +254,16 @@ __global__ __launch_bounds__(256) void attention_bwd_dkv_kernel(AttnBwdArgs a) {
   const T* Vg = (const T*)a.V + (long)b * a.tk * a.h * DH + hh * DH;
   const float* Gg = a.G ? a.G + (long)b * a.tk * a.h + hh : nullptr;
   const long kstride = (long)a.h * DH;
+  const int half_deg = (int)a.deg / 2;
+  const float eps_s = AB_LOG_EPS / a.scale;
+  const float scale_p = __powf(a.scale, a.deg);
+  const int last_key = min(key0 + KEYS, a.tk) - 1;
+  const float R = Gg ? Gg[(long)last_key * a.h] : 0.f;   // reference gate of this key block
 
   v8 Kf[MK][KS], Vf[MK][KS];
   int key[MK];
   bool live[MK];
-  float Gk[MK], dgk[MK];
+  float Gk[MK], ev[MK], dgk[MK];
 #pragma unroll
   for (int kj = 0; kj < MK; kj++) {
     key[kj] = key0 + wave * 16 * MK + 16 * kj + kcol;
@@ -234,6 +279,7 @@ __global__ __launch_bounds__(256) void attention_bwd_dkv_kernel(AttnBwdArgs a) {
       Vf[kj][ks] = __builtin_bit_cast(v8, z2);
     }
     Gk[kj] = (Gg && live[kj]) ? Gg[(long)key[kj] * a.h] : 0.f;
+    ev[kj] = __expf(fminf(R - Gk[kj], AB_EXP_CLAMP));
     dgk[kj] = 0.f;
   }
   f32x4 accK[MK][NT], accV[MK][NT];
@@ -247,7 +293,6 @@ __global__ __launch_bounds__(256) void attention_bwd_dkv_kernel(AttnBwdArgs a) {
 
   // folded rows that can see any key of this workgroup: time index >= key0
   const int row_begin = max(0, (key0 - shift) * a.r) / AB_BM * AB_BM;
-  const int last_key = min(key0 + KEYS, a.tk) - 1;
   const int nsteps = (rows - row_begin + AB_BM - 1) / AB_BM;
 
   u32x4 rq[PT], rdo[PT];
@@ -289,14 +334,14 @@ __global__ __launch_bounds__(256) void attention_bwd_dkv_kernel(AttnBwdArgs a) {
       }
     }
     if (tid < AB_BM) {
-      float* rv = rowv + stage * 3 * AB_BM;
+      float* rv = rowv + stage * 4 * AB_BM;
       rv[tid] = r0;
       rv[AB_BM + tid] = r1;
       rv[2 * AB_BM + tid] = r2;
+      rv[3 * AB_BM + tid] = scale_p * __expf(fminf(r0 - R, AB_EXP_CLAMP));
     }
   };
 
-  const float cds = a.deg * a.scale;
   if (nsteps > 0) fetch(row_begin);
   for (int it = 0; it < nsteps; it++) {
     const int rbase = row_begin + it * AB_BM, stage = it & 1;
@@ -305,9 +350,9 @@ __global__ __launch_bounds__(256) void attention_bwd_dkv_kernel(AttnBwdArgs a) {
     if (it + 1 < nsteps) fetch(rbase + AB_BM);
     const T* qt_ = Qt + stage * AB_BM * LD;
     const T* dot_ = dOt + stage * AB_BM * LD;
-    const float* rv = rowv + stage * 3 * AB_BM;
-    // masking is needed unless every row of the step sees every key of the workgroup and is real
-    const bool need_mask = (rbase / a.r + shift < last_key) || (rbase + AB_BM > rows) || (key0 + KEYS > a.tk);
+    const float* rv = rowv + stage * 4 * AB_BM;
+    // exact per-pair path unless every row of the step is real and sees every (real) key of the workgroup
+    const bool diag = (rbase / a.r + shift < last_key) || (rbase + AB_BM > rows) || (key0 + KEYS > a.tk);
 
     v8 pf[MK], dsf[MK];
     {
@@ -320,7 +365,7 @@ __global__ __launch_bounds__(256) void attention_bwd_dkv_kernel(AttnBwdArgs a) {
           qf[ks] = lds_frag<T>(qt_, LD, 16 * qt, 32 * ks);
           dof[ks] = lds_frag<T>(dot_, LD, 16 * qt, 32 * ks);
         }
-        const f32x4 gm = *(const f32x4*)(rv + 16 * qt + 4 * g);
+        const f32x4 gm = *(const f32x4*)(rv + (diag ? 0 : 3 * AB_BM) + 16 * qt + 4 * g);
         const f32x4 dlv = *(const f32x4*)(rv + AB_BM + 16 * qt + 4 * g);
         const f32x4 tiv = *(const f32x4*)(rv + 2 * AB_BM + 16 * qt + 4 * g);
 #pragma unroll
@@ -333,16 +378,18 @@ __global__ __launch_bounds__(256) void attention_bwd_dkv_kernel(AttnBwdArgs a) {
           }
 #pragma unroll
           for (int v = 0; v < 4; v++) {
-            const float ss = s[v] * a.scale;
-            const float as = fabsf(ss) + AB_LOG_EPS;
-            float p = __expf(a.deg * __logf(as) + (gm[v] - Gk[kj]));
-            if (need_mask) {
-              if ((float)key[kj] > tiv[v] || !live[kj]) p = 0.f;
+            float E;
+            if (diag) {
+              E = scale_p * __expf(fminf(gm[v] - Gk[kj], AB_EXP_CLAMP));
+              if ((float)key[kj] > tiv[v] || !live[kj]) E = 0.f;
+            } else {
+              E = gm[v] * ev[kj];
             }
-            const float dz = p * (dp[v] + dlv[v]);
+            float p, dz, dsr;
+            pair_grad<DEG2>(s[v], E, dp[v] + dlv[v], eps_s, half_deg, p, dz, dsr);
             dgk[kj] -= dz;
             p8[kj][4 * qt + v] = p;
-            d8[kj][4 * qt + v] = dz * cds * (ss < 0.f ? -1.f : 1.f) / as;
+            d8[kj][4 * qt + v] = dsr;
           }
         }
       }
@@ -380,7 +427,7 @@ __global__ __launch_bounds__(256) void attention_bwd_dkv_kernel(AttnBwdArgs a) {
       float k4[4], v4f[4];
 #pragma unroll
       for (int v = 0; v < 4; v++) {
-        k4[v] = accK[kj][nt][v];
+        k4[v] = accK[kj][nt][v] * a.deg;
         v4f[v] = accV[kj][nt][v];
       }
       *(v4*)(dKg + key[kj] * kstride + 16 * nt + 4 * g) = pack4<T>(k4);
@@ -390,21 +437,21 @@ __global__ __launch_bounds__(256) void attention_bwd_dkv_kernel(AttnBwdArgs a) {
   }
 }
 
-template <typename T, int DH> static int attn_bwd_launch(const AttnBwdArgs& a, int B, hipStream_t st) {
+template <typename T, int DH, bool DEG2> static int attn_bwd_launch(const AttnBwdArgs& a, int B, hipStream_t st) {
   {
     constexpr int MT = DH <= 64 ? 2 : 1;
-    constexpr size_t smem = 2 * 2 * AB_BN * (DH + 8) * sizeof(T) + 2 * AB_BN * sizeof(float);
+    constexpr size_t smem = 2 * 2 * AB_BN * (DH + 8) * sizeof(T) + 2 * (2 * AB_BN + 4) * sizeof(float);
     const int rows = a.tq * a.r;
     dim3 grid((rows + 64 * MT - 1) / (64 * MT), (unsigned)(B * a.h));
-    auto kern = attention_bwd_dq_kernel<T, DH, MT>;
+    auto kern = attention_bwd_dq_kernel<T, DH, MT, DEG2>;
     allow_big_lds((const void*)kern, smem);
     hipLaunchKernelGGL(kern, grid, dim3(256), smem, st, a);
   }
   {
     constexpr int MK = DH <= 64 ? 2 : 1;
-    constexpr size_t smem = 2 * 2 * AB_BM * (DH + 8) * sizeof(T) + 2 * 3 * AB_BM * sizeof(float);
+    constexpr size_t smem = 2 * 2 * AB_BM * (DH + 8) * sizeof(T) + 2 * 4 * AB_BM * sizeof(float);
     dim3 grid((a.tk + 64 * MK - 1) / (64 * MK), (unsigned)(B * a.h));
-    auto kern = attention_bwd_dkv_kernel<T, DH, MK>;
+    auto kern = attention_bwd_dkv_kernel<T, DH, MK, DEG2>;
     allow_big_lds((const void*)kern, smem);
     hipLaunchKernelGGL(kern, grid, dim3(256), smem, st, a);
   }
@@ -414,9 +461,9 @@ template <typename T, int DH> static int attn_bwd_launch(const AttnBwdArgs& a, i
 int attention_bwd(const AttnBwdArgs& a, int B, int d, int dtype, hipStream_t st) {
 #define PR_AB(T)                                                                                                       \
   switch (d) {                                                                                                         \
-    case 32: return attn_bwd_launch<T, 32>(a, B, st);                                                                  \
-    case 64: return attn_bwd_launch<T, 64>(a, B, st);                                                                  \
-    case 128: return attn_bwd_launch<T, 128>(a, B, st);                                                                \
+    case 32: return a.deg == 2.f ? attn_bwd_launch<T, 32, true>(a, B, st) : attn_bwd_launch<T, 32, false>(a, B, st);   \
+    case 64: return a.deg == 2.f ? attn_bwd_launch<T, 64, true>(a, B, st) : attn_bwd_launch<T, 64, false>(a, B, st);   \
+    case 128: return a.deg == 2.f ? attn_bwd_launch<T, 128, true>(a, B, st) : attn_bwd_launch<T, 128, false>(a, B, st);\
     default: return -2;                                                                                                \
   }
   if (dtype == DT_BF16) { PR_AB(bf16_t) }

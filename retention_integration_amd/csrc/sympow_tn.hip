@@ -163,7 +163,7 @@ __device__ __forceinline__ void tn_body(const T* __restrict__ A, const T* __rest
 }
 
 template <typename T, int DK, int DV, int XPW, bool HAS_W>
-__global__ __launch_bounds__(256) void sympow_tn_kernel(const T* __restrict__ A, const T* __restrict__ Bm,
+__global__ __launch_bounds__(256, 2) void sympow_tn_kernel(const T* __restrict__ A, const T* __restrict__ Bm,
                                                         const float* __restrict__ w, T* __restrict__ S,
                                                         float* __restrict__ s, int c, int hA, int r, int h,
                                                         int use_mult) {

@@ -153,11 +153,13 @@ def test_query_state(pra, dtype, d, c, r, zis, attn):
 
 
 # ---------------------------------------------------------------- attention
-@pytest.mark.parametrize("dtype,d,tq,tk,r,gated,norm", [
-    (torch.bfloat16, 64, 128, 128, 1, True, False), (torch.bfloat16, 64, 200, 200, 1, False, True),
-    (torch.float16, 128, 96, 96, 1, True, False), (torch.bfloat16, 32, 1, 130, 2, True, False),
-    (torch.bfloat16, 64, 70, 150, 2, True, True), (torch.bfloat16, 64, 384, 384, 1, True, False)])
-def test_attention(pra, dtype, d, tq, tk, r, gated, norm):
+@pytest.mark.parametrize("dtype,d,tq,tk,r,gated,norm,deg", [
+    (torch.bfloat16, 64, 128, 128, 1, True, False, 2), (torch.bfloat16, 64, 200, 200, 1, False, True, 2),
+    (torch.float16, 128, 96, 96, 1, True, False, 2), (torch.bfloat16, 32, 1, 130, 2, True, False, 2),
+    (torch.bfloat16, 64, 70, 150, 2, True, True, 2), (torch.bfloat16, 64, 384, 384, 1, True, False, 2),
+    (torch.bfloat16, 64, 1024, 1024, 1, True, False, 2), (torch.bfloat16, 64, 160, 160, 1, True, False, 4),
+    (torch.bfloat16, 32, 128, 128, 2, False, True, 4)])
+def test_attention(pra, dtype, d, tq, tk, r, gated, norm, deg):
     b, h = 2, 2
     Q, K, V = (rnd(b, tq, h * r, d, dtype=dtype, seed=30), rnd(b, tk, h, d, dtype=dtype, seed=31),
                rnd(b, tk, h, d, dtype=dtype, seed=32))
@@ -165,8 +167,8 @@ def test_attention(pra, dtype, d, tq, tk, r, gated, norm):
     scale = 1.0 / math.sqrt(d)
     g_in = [dev(Q, True), dev(K, True), dev(V, True), dev(A, gated)]
     o_in = [gold(Q, True), gold(K, True), gold(V, True), gold(A, gated)]
-    out = pra.attention(*g_in, 2, scale=scale, norm=norm)
-    ref = oracle.attention(*o_in, 2, scale=scale, norm=norm)
+    out = pra.attention(*g_in, deg, scale=scale, norm=norm)
+    ref = oracle.attention(*o_in, deg, scale=scale, norm=norm)
     if norm:
         check("Y", out, ref, OUT_TOL)
         dY = rnd(*ref.shape, dtype=dtype, seed=34)
