@@ -107,6 +107,24 @@ int pr_query_state_bwd(const void* Q, const void* S, const float* s, const float
                        float* dl_attn, void* workspace, int BN, int n, int c, int h, int r, int d, float scale_p,
                        int deg, int zero_initial_state, int dtype, void* stream);
 
+/* Gate arithmetic of the chunked algorithm, forward -- retention/power_retention_maker.py:146-153,163-164,183-186.
+ *   log_G [BN,c,h] fp32 (BN = b*n chunks of length c <= 8192), K [BN,c,h,d], Q [BN,c,h*r,d]
+ *   -> A [BN,c,h] = cumsum over the chunk, lcs [BN,h] = A[c-1],
+ *      Kd = K * exp((A[c-1] - A)/deg), Qg = Q * exp(A/deg). */
+int pr_chunk_prep_fwd(const float* log_G, const void* K, const void* Q, float* A, float* lcs, void* Kd, void* Qg, int BN,
+                      int c, int h, int r, int d, int deg, int dtype, void* stream);
+
+/* Backward of the same glue plus the final gradient sums (autograd of retention/power_retention_maker.py:143-193).
+ *   A as above or NULL for the ungated path (then dG_attn, dlcs_*, dlog_G are ignored);
+ *   dKd, dQg: gradients w.r.t. Kd, Qg; dK_attn, dQ_attn, dV_attn: from the attention backward; dV_state: from the
+ *   update_state backward; dG_attn [BN,c,h]: gradient w.r.t. A from the attention backward; dlcs_a, dlcs_b [BN,h]:
+ *   gradients w.r.t. lcs from the two scans
+ *   -> dK, dQ, dV (may alias dK_attn, dQ_attn, dV_attn), dlog_G [BN,c,h]. */
+int pr_chunk_glue_bwd(const float* A, const void* Kd, const void* dKd, const void* Qg, const void* dQg,
+                      const void* dK_attn, const void* dQ_attn, const void* dV_attn, const void* dV_state,
+                      const float* dG_attn, const float* dlcs_a, const float* dlcs_b, void* dK, void* dQ, void* dV,
+                      float* dlog_G, int BN, int c, int h, int r, int d, int deg, int dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

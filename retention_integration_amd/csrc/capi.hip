@@ -23,6 +23,7 @@ int finish(int rc, const char* what) {
   if (rc == 0) return 0;
   if (rc == -1) return fail(PR_ERR_DTYPE, "%s: unsupported dtype", what);
   if (rc == -2) return fail(PR_ERR_HEAD_DIM, "%s: head dim must be 32, 64 or 128", what);
+  if (rc == -5) return fail(PR_ERR_ARG, "%s: chunk longer than 8192 is not supported", what);
   return fail(rc, "%s: launch failed: %s", what, hipGetErrorString((hipError_t)rc));
 }
 int check_common(const char* what, int d, int deg, int dtype, bool state) {
@@ -162,6 +163,33 @@ int pr_query_state_bwd(const void* Q, const void* S, const float* s, const float
   if (int rc = finish(pr::sympow_tn(Q, dOs, cvec, dS, ds, BN, c, h, r, d, 0, dtype, st), "query_state_bwd(dS)")) return rc;
   pr::GradArgs g{Q, dOs, cvec, S, s, dQ, c, h, r, n, zero_initial_state ? 1 : 0};
   return finish(pr::sympow_grad(g, BN, d, 0, dtype, st), "query_state_bwd(dQ)");
+}
+
+
+int pr_chunk_prep_fwd(const float* log_G, const void* K, const void* Q, float* A, float* lcs, void* Kd, void* Qg, int BN,
+                      int c, int h, int r, int d, int deg, int dtype, void* stream) {
+  if (int rc = check_common("chunk_prep_fwd", d, deg, dtype, false)) return rc;
+  if (log_G == nullptr || bad_ptr(K) || bad_ptr(Q) || A == nullptr || lcs == nullptr || bad_ptr(Kd) || bad_ptr(Qg))
+    return fail(PR_ERR_ARG, "chunk_prep_fwd: null or misaligned pointer");
+  if (BN <= 0 || c <= 0 || h <= 0 || r <= 0) return fail(PR_ERR_ARG, "chunk_prep_fwd: need BN,c,h,r > 0");
+  return finish(pr::chunk_prep_fwd(log_G, K, Q, A, lcs, Kd, Qg, BN, c, h, r, d, deg, dtype, (hipStream_t)stream),
+                "chunk_prep_fwd");
+}
+
+int pr_chunk_glue_bwd(const float* A, const void* Kd, const void* dKd, const void* Qg, const void* dQg,
+                      const void* dK_attn, const void* dQ_attn, const void* dV_attn, const void* dV_state,
+                      const float* dG_attn, const float* dlcs_a, const float* dlcs_b, void* dK, void* dQ, void* dV,
+                      float* dlog_G, int BN, int c, int h, int r, int d, int deg, int dtype, void* stream) {
+  if (int rc = check_common("chunk_glue_bwd", d, deg, dtype, false)) return rc;
+  if (bad_ptr(Kd) || bad_ptr(dKd) || bad_ptr(Qg) || bad_ptr(dQg) || bad_ptr(dK_attn) || bad_ptr(dQ_attn) ||
+      bad_ptr(dV_attn) || bad_ptr(dV_state) || bad_ptr(dK) || bad_ptr(dQ) || bad_ptr(dV))
+    return fail(PR_ERR_ARG, "chunk_glue_bwd: null or misaligned pointer");
+  if (A && (!dG_attn || !dlcs_a || !dlcs_b || !dlog_G))
+    return fail(PR_ERR_ARG, "chunk_glue_bwd: gated call needs dG_attn, dlcs_a, dlcs_b and dlog_G");
+  if (BN <= 0 || c <= 0 || h <= 0 || r <= 0) return fail(PR_ERR_ARG, "chunk_glue_bwd: need BN,c,h,r > 0");
+  return finish(pr::chunk_glue_bwd(A, Kd, dKd, Qg, dQg, dK_attn, dQ_attn, dV_attn, dV_state, dG_attn, dlcs_a, dlcs_b,
+                                   dK, dQ, dV, dlog_G, BN, c, h, r, d, deg, dtype, (hipStream_t)stream),
+                "chunk_glue_bwd");
 }
 
 }  // extern "C"

@@ -106,12 +106,108 @@ __device__ __forceinline__ typename VecOf<T>::v8 lds_frag(const T* tile, int ld,
   return *(const typename VecOf<T>::v8*)(tile + (n0 + (l & 15)) * ld + k0 + 8 * (l >> 4));
 }
 
+// ---- swizzled LDS tiles filled by asynchronous global->LDS copies ---------------------------
+// A tile is [rows][CPR chunks of 16 bytes] with no padding; chunk c of row r is stored at chunk
+// slot c ^ swz(r), which spreads the 16 rows an operand load touches over all banks.  The copy
+// instruction (global_load_lds_dwordx4) writes lane i's 16 bytes at wave_base + 16*i, so a wave
+// fills 64 consecutive chunk slots and every lane fetches the global chunk that belongs in its slot.
+// Completion is tracked by vmcnt only: the consumer waits with wait_vmcnt<N>() and then barriers.
+// swz is a bijection of the rows that share a bank phase, bit-rotated so that the four consecutive rows a
+// transposing read touches land in different pairs of chunk slots as well.
+template <int CPR> __device__ __forceinline__ int swz(int row) {
+  static_assert(CPR == 4 || CPR == 8 || CPR == 16, "rows of 64, 128 or 256 bytes");
+  if (CPR == 8) {
+    const int k = (row >> 1) & 7;
+    return ((k & 1) << 2) | (k >> 1);
+  } else if (CPR == 16) {
+    const int k = row & 15;
+    return ((k & 3) << 2) | (k >> 2);
+  }
+  return (row >> 2) & 3;
+}
+
+template <int N> __device__ __forceinline__ void wait_vmcnt() {
+  static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+  __builtin_amdgcn_s_waitcnt((N & 0xF) | ((N >> 4) << 14) | (0x7 << 4) | (0xF << 8));
+}
+
+__device__ __forceinline__ void async_copy16(const void* gsrc, void* lds_wave_base) {
+  __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)gsrc,
+                                   (__attribute__((address_space(3))) void*)lds_wave_base, 16, 0, 0);
+}
+__device__ __forceinline__ void async_copy4(const void* gsrc, void* lds_wave_base) {
+  __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)gsrc,
+                                   (__attribute__((address_space(3))) void*)lds_wave_base, 4, 0, 0);
+}
+
+// Issue the copies of a tile of R rows (R*CPR a multiple of 256) by a 256-thread workgroup: every thread
+// issues exactly R*CPR/256 copies.  row_ptr(row) returns the global address of the row's first byte and
+// must be valid for every row (clamp out-of-range rows; zero them afterwards with zero_tile_rows).
+template <int CPR, int R, typename F> __device__ __forceinline__ void async_load_tile(char* tile, F row_ptr) {
+  static_assert((R * CPR) % 256 == 0, "tile must be a whole number of workgroup-wide copies");
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+#pragma unroll
+  for (int ii = 0; ii < R * CPR / 256; ii++) {
+    const int inst = ii * 4 + wave;
+    const int pos = inst * 64 + lane, row = pos / CPR, c = (pos % CPR) ^ swz<CPR>(row);
+    async_copy16(row_ptr(row) + 16 * c, tile + inst * 1024);
+  }
+}
+// Zero rows [first_bad, R) of a tile (same slot ownership as async_load_tile; call after the wait, before the barrier).
+template <int CPR, int R> __device__ __forceinline__ void zero_tile_rows(char* tile, int first_bad) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+#pragma unroll
+  for (int ii = 0; ii < R * CPR / 256; ii++) {
+    const int pos = (ii * 4 + wave) * 64 + lane;
+    if (pos / CPR >= first_bad) *(u32x4*)(tile + pos * 16) = (u32x4){0, 0, 0, 0};
+  }
+}
+
+// Operand loads from a swizzled tile of T (same conventions as lds_frag / lds_frag_tr / lds_frag_tr4).
+template <typename T, int CPR>
+__device__ __forceinline__ typename VecOf<T>::v8 sw_frag(const char* tile, int n0, int k0) {
+  const int l = lane_id(), row = n0 + (l & 15), c = (k0 + 8 * (l >> 4)) / 8;
+  return *(const typename VecOf<T>::v8*)(tile + row * (CPR * 16) + ((c ^ swz<CPR>(row)) * 16));
+}
+template <typename T, int CPR>
+__device__ __forceinline__ typename VecOf<T>::v4 sw_frag_tr4(const char* tile, int krow, int n0) {
+  const int l = lane_id(), s = l & 15, row = krow + (s >> 2), col = n0 + 4 * (s & 3);
+  const char* p = tile + row * (CPR * 16) + (((col / 8) ^ swz<CPR>(row)) * 16) + (col % 8) * 2;
+  typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+  s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)p);
+  return __builtin_bit_cast(typename VecOf<T>::v4, v);
+}
+template <typename T, int CPR>
+__device__ __forceinline__ typename VecOf<T>::v8 sw_frag_tr(const char* tile, int k0, int n0) {
+  const int g = lane_id() >> 4;
+  typename VecOf<T>::v4 lo = sw_frag_tr4<T, CPR>(tile, k0 + 8 * g, n0);
+  typename VecOf<T>::v4 hi = sw_frag_tr4<T, CPR>(tile, k0 + 8 * g + 4, n0);
+  return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+}
+
 // Broadcast lane N of every 16-lane row to the whole row (folds into the consuming VALU op).
 template <int N> __device__ __forceinline__ float row_bcast(float x) {
-  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x150 + N, 0xf, 0xf, true));
+  return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, x), 0x150 + N, 0xf, 0xf, true));
 }
 template <int N> __device__ __forceinline__ uint32_t row_bcast_u32(uint32_t x) {
   return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x150 + N, 0xf, 0xf, true);
+}
+
+// bcast_lane_N_of_row(src) * row in ONE VALU op.  The compiler only folds the row broadcast into the multiply
+// for some operand orders, so the instruction is spelled out.  It is opaque to the hazard recogniser: src must
+// have been written at least two wait states earlier -- callers put dpp_fence() between producing src and the
+// first use.
+template <int N> __device__ __forceinline__ float mul_row_bcast(float src, float row) {
+  float r;
+  asm("v_mul_f32_dpp %0, %1, %2 row_newbcast:%3 row_mask:0xf bank_mask:0xf bound_ctrl:1"
+      : "=v"(r)
+      : "v"(src), "v"(row), "n"(N));
+  return r;
+}
+__device__ __forceinline__ void dpp_fence() {
+  __builtin_amdgcn_sched_barrier(0);
+  asm volatile("s_nop 1");
+  __builtin_amdgcn_sched_barrier(0);
 }
 
 // Sum over the four 16-lane rows of a wave (lanes l, l+16, l+32, l+48); every lane gets the total.

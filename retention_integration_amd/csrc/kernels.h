@@ -81,4 +81,12 @@ int attention_bwd(const AttnBwdArgs& a, int B, int d, int dtype, hipStream_t st)
 int qs_bwd_prep(const void* O, const void* dO, const float* den, const float* rowmax, void* dOs, float* cvec,
                 void* dY_attn, float* dl_attn, long rows, int d, float scale_p, int dtype, hipStream_t st);
 
+// chunk_glue.hip (return -5: chunk longer than the LDS-resident gate vector allows)
+int chunk_prep_fwd(const float* logG, const void* K, const void* Q, float* A, float* lcs, void* Kd, void* Qg, int BN,
+                   int c, int h, int r, int d, int deg, int dtype, hipStream_t st);
+int chunk_glue_bwd(const float* A, const void* Kd, const void* dKd, const void* Qg, const void* dQg,
+                   const void* dK_attn, const void* dQ_attn, const void* dV_attn, const void* dV_state,
+                   const float* dG_attn, const float* dlcs_a, const float* dlcs_b, void* dK, void* dQ, void* dV,
+                   float* dlogG, int BN, int c, int h, int r, int d, int deg, int dtype, hipStream_t st);
+
 }  // namespace pr

@@ -9,24 +9,25 @@
 //                                                              (ref: retention/_query_state/triton.py:546-553)
 //
 // One workgroup = 4 waves; a wave owns XPW of the 16 "x" columns of one 16x16 feature block
-// (y, xb) and all DV value columns, and contracts over the rows in steps of 32.  The phi tile is
+// (y, xb) and all DV value columns, and contracts over the rows 32 at a time.  The phi tile is
 // never stored: the A-operand of each matrix-core op is produced in registers as the product of a
 // row-broadcast (DPP) of column x with the 16 columns 16*y..16*y+15, both read transposed from one
 // row-major LDS tile.  s uses the identity s[(x, j)] = (A^T diag(w) A)[x, j], one extra matrix-core op
-// per step.
+// per step.  Row tiles of A and B arrive through a 3-deep ring of asynchronous global->LDS copies.
 #include "common.h"
 #include "kernels.h"
 
 namespace pr {
 
-constexpr int TN_KT = 32;  // rows contracted per step
+constexpr int TN_KT = 64;   // rows per pipeline stage (two contraction steps of 32)
+constexpr int TN_NST = 3;   // stages in the ring
 
 template <typename T, int X> struct PhiTile;
 template <int X> struct PhiTile<bf16_t, X> {
   static __device__ __forceinline__ bf16x8 make(const bf16x8&, const bf16x8&, const float* rowf, const float* srcf) {
     float p[8];
 #pragma unroll
-    for (int r = 0; r < 8; r++) p[r] = row_bcast<X>(srcf[r]) * rowf[r];
+    for (int r = 0; r < 8; r++) p[r] = mul_row_bcast<X>(srcf[r], rowf[r]);
     return pack8<bf16_t>(p);
   }
 };
@@ -44,60 +45,26 @@ __device__ __forceinline__ void tn_body(const T* __restrict__ A, const T* __rest
                                         T* __restrict__ S, float* __restrict__ s, int c, int hA, int r, int hh,
                                         int bn, int h, int y, int xb, bool active, bool use_mult, char* smem) {
   typedef typename VecOf<T>::v8 v8;
-  constexpr int LDA = DK + 8, LDB = DV + 8, NT = DV / 16;
-  constexpr int A_CH = TN_KT * DK / 8, B_CH = TN_KT * DV / 8;  // 16-byte chunks per tile
-  constexpr int A_PT = (A_CH + 255) / 256, B_PT = (B_CH + 255) / 256;
-  T* At = (T*)smem;                                   // [2][KT][LDA]
-  T* Bt = At + 2 * TN_KT * LDA;                       // [2][KT][LDB]
-  float* wt = (float*)(Bt + 2 * TN_KT * LDB);         // [2][KT]
+  constexpr int NT = DV / 16, CA = DK / 8, CB = DV / 8;            // 16-byte chunks per row
+  constexpr int A_BYTES = TN_KT * DK * 2, B_BYTES = TN_KT * DV * 2, W_BYTES = TN_KT * 4;
+  constexpr int STAGE = A_BYTES + B_BYTES + W_BYTES;
+  constexpr int LOADS = (TN_KT * CA + TN_KT * CB) / 256;           // copies per thread per stage (w rides on wave 0)
   const int tid = threadIdx.x, l = tid & 63, g = l >> 4;
   const int rows = c * r;
-  const long a_base = (long)bn * c * hA * DK, b_base = (long)bn * c * hA * DV, w_base = (long)bn * c * hA;
-
-  u32x4 ra[A_PT], rb[B_PT];
-  float rw = 0.f;
-  auto fetch = [&](int step) {
-#pragma unroll
-    for (int i = 0; i < A_PT; i++) {
-      const int ch = tid + 256 * i;
-      const int row = step * TN_KT + ch / (DK / 8), col = (ch % (DK / 8)) * 8;
-      ra[i] = (u32x4){0, 0, 0, 0};
-      if (ch < A_CH && row < rows) {
-        const int t = row / r, rr = row - t * r;
-        ra[i] = *(const u32x4*)(A + a_base + ((long)t * hA + hh * r + rr) * DK + col);
-      }
-    }
-#pragma unroll
-    for (int i = 0; i < B_PT; i++) {
-      const int ch = tid + 256 * i;
-      const int row = step * TN_KT + ch / (DV / 8), col = (ch % (DV / 8)) * 8;
-      rb[i] = (u32x4){0, 0, 0, 0};
-      if (ch < B_CH && row < rows) {
-        const int t = row / r, rr = row - t * r;
-        rb[i] = *(const u32x4*)(Bm + b_base + ((long)t * hA + hh * r + rr) * DV + col);
-      }
-    }
-    if (HAS_W && tid < TN_KT) {
-      const int row = step * TN_KT + tid;
-      rw = 0.f;
-      if (row < rows) {
-        const int t = row / r, rr = row - t * r;
-        rw = w[w_base + (long)t * hA + hh * r + rr];
-      }
-    }
+  const char* a_base = (const char*)(A + (long)bn * c * hA * DK);
+  const char* b_base = (const char*)(Bm + (long)bn * c * hA * DV);
+  const float* w_base = w + (long)bn * c * hA;
+  auto row_index = [&](int row) -> long {   // element offset of a (clamped) folded row, per unit of the last dim
+    row = min(row, rows - 1);
+    const int t = row / r, rr = row - t * r;
+    return (long)t * hA + hh * r + rr;
   };
-  auto stash = [&](int stage) {
-#pragma unroll
-    for (int i = 0; i < A_PT; i++) {
-      const int ch = tid + 256 * i;
-      if (ch < A_CH) *(u32x4*)(At + stage * TN_KT * LDA + (ch / (DK / 8)) * LDA + (ch % (DK / 8)) * 8) = ra[i];
-    }
-#pragma unroll
-    for (int i = 0; i < B_PT; i++) {
-      const int ch = tid + 256 * i;
-      if (ch < B_CH) *(u32x4*)(Bt + stage * TN_KT * LDB + (ch / (DV / 8)) * LDB + (ch % (DV / 8)) * 8) = rb[i];
-    }
-    if (HAS_W && tid < TN_KT) wt[stage * TN_KT + tid] = rw;
+  auto issue = [&](int step) {
+    char* st = smem + (step % TN_NST) * STAGE;
+    const int r0 = step * TN_KT;
+    async_load_tile<CA, TN_KT>(st, [&](int row) { return a_base + row_index(r0 + row) * (DK * 2); });
+    async_load_tile<CB, TN_KT>(st + A_BYTES, [&](int row) { return b_base + row_index(r0 + row) * (DV * 2); });
+    if (HAS_W && tid < 64) async_copy4(w_base + row_index(r0 + tid), st + A_BYTES + B_BYTES);
   };
 
   f32x4 acc[XPW][NT];
@@ -108,37 +75,42 @@ __device__ __forceinline__ void tn_body(const T* __restrict__ A, const T* __rest
   f32x4 sacc = {0, 0, 0, 0};
 
   const int steps = (rows + TN_KT - 1) / TN_KT;
-  fetch(0);
+  issue(0);
+  if (steps > 1) issue(1);
   for (int step = 0; step < steps; step++) {
-    const int stage = step & 1;
-    stash(stage);
+    char* st = smem + (step % TN_NST) * STAGE;
+    if (step + 1 < steps) wait_vmcnt<LOADS>(); else wait_vmcnt<0>();
+    if ((step + 1) * TN_KT > rows) zero_tile_rows<CA, TN_KT>(st, rows - step * TN_KT);
     __syncthreads();
-    if (step + 1 < steps) fetch(step + 1);
+    if (step + 2 < steps) issue(step + 2);
     if (active) {
-      const T* at = At + stage * TN_KT * LDA;
-      const T* bt = Bt + stage * TN_KT * LDB;
-      v8 kfy = lds_frag_tr<T>(at, LDA, 0, 16 * y);
-      v8 kfx = (xb == y) ? kfy : lds_frag_tr<T>(at, LDA, 0, 16 * xb);
-      v8 vf[NT];
+      const float* wt = (const float*)(st + A_BYTES + B_BYTES);
+#pragma unroll 1
+      for (int ks = 0; ks < TN_KT / 32; ks++) {
+        v8 kfy = sw_frag_tr<T, CA>(st, 32 * ks, 16 * y);
+        v8 kfx = (xb == y) ? kfy : sw_frag_tr<T, CA>(st, 32 * ks, 16 * xb);
+        v8 vf[NT];
 #pragma unroll
-      for (int nt = 0; nt < NT; nt++) vf[nt] = lds_frag_tr<T>(bt, LDB, 0, 16 * nt);
-      float rowf[8], srcf[8];
-      unpack8(kfy, rowf);
-      unpack8(kfx, srcf);
-      if (HAS_W) {
-        float sc[8];
-        const float* wp = wt + stage * TN_KT + 8 * g;
+        for (int nt = 0; nt < NT; nt++) vf[nt] = sw_frag_tr<T, CB>(st + A_BYTES, 32 * ks, 16 * nt);
+        float rowf[8], srcf[8];
+        unpack8(kfy, rowf);
+        unpack8(kfx, srcf);
+        if (HAS_W) {
+          float sc[8];
+          const float* wp = wt + 32 * ks + 8 * g;
 #pragma unroll
-        for (int q = 0; q < 8; q++) sc[q] = srcf[q] * wp[q];
-        sacc = mfma16(kfy, pack8<T>(sc), sacc);
-      } else {
-        sacc = mfma16(kfy, kfx, sacc);
+          for (int q = 0; q < 8; q++) sc[q] = srcf[q] * wp[q];
+          sacc = mfma16(kfy, pack8<T>(sc), sacc);
+        } else {
+          sacc = mfma16(kfy, kfx, sacc);
+        }
+        dpp_fence();  // srcf is read through DPP below
+        static_for<XPW>([&](auto xi) {
+          v8 a = PhiTile<T, PART * XPW + xi.value>::make(kfy, kfx, rowf, srcf);
+#pragma unroll
+          for (int nt = 0; nt < NT; nt++) acc[xi.value][nt] = mfma16(a, vf[nt], acc[xi.value][nt]);
+        });
       }
-      static_for<XPW>([&](auto xi) {
-        v8 a = PhiTile<T, PART * XPW + xi.value>::make(kfy, kfx, rowf, srcf);
-#pragma unroll
-        for (int nt = 0; nt < NT; nt++) acc[xi.value][nt] = mfma16(a, vf[nt], acc[xi.value][nt]);
-      });
     }
   }
   if (!active) return;
@@ -164,10 +136,10 @@ __device__ __forceinline__ void tn_body(const T* __restrict__ A, const T* __rest
 
 template <typename T, int DK, int DV, int XPW, bool HAS_W>
 __global__ __launch_bounds__(256, 2) void sympow_tn_kernel(const T* __restrict__ A, const T* __restrict__ Bm,
-                                                        const float* __restrict__ w, T* __restrict__ S,
-                                                        float* __restrict__ s, int c, int hA, int r, int h,
-                                                        int use_mult) {
-  extern __shared__ __attribute__((aligned(16))) char smem[];
+                                                           const float* __restrict__ w, T* __restrict__ S,
+                                                           float* __restrict__ s, int c, int hA, int r, int h,
+                                                           int use_mult) {
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
   constexpr int PARTS = 16 / XPW;
   constexpr int NB = (DK / 16) * (DK / 16 + 1) / 2;
   const int task = blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -198,14 +170,17 @@ static int tn_launch(const void* A, const void* Bm, const float* w, void* S, flo
   constexpr int XPW = DV <= 64 ? 8 : 4;
   constexpr int NB = (DK / 16) * (DK / 16 + 1) / 2;
   constexpr int TASKS = NB * (16 / XPW);
-  constexpr size_t smem = 2 * TN_KT * ((DK + 8) + (DV + 8)) * sizeof(T) + 2 * TN_KT * sizeof(float);
+  constexpr size_t smem = TN_NST * (TN_KT * DK * 2 + TN_KT * DV * 2 + TN_KT * 4);
   dim3 grid((TASKS + 3) / 4, (unsigned)(BN * h));
-  if (w)
-    hipLaunchKernelGGL((sympow_tn_kernel<T, DK, DV, XPW, true>), grid, dim3(256), smem, st, (const T*)A, (const T*)Bm, w,
-                       (T*)S, s, c, h * r, r, h, use_mult);
-  else
-    hipLaunchKernelGGL((sympow_tn_kernel<T, DK, DV, XPW, false>), grid, dim3(256), smem, st, (const T*)A, (const T*)Bm,
-                       w, (T*)S, s, c, h * r, r, h, use_mult);
+  if (w) {
+    auto kern = sympow_tn_kernel<T, DK, DV, XPW, true>;
+    allow_big_lds((const void*)kern, smem);
+    hipLaunchKernelGGL(kern, grid, dim3(256), smem, st, (const T*)A, (const T*)Bm, w, (T*)S, s, c, h * r, r, h, use_mult);
+  } else {
+    auto kern = sympow_tn_kernel<T, DK, DV, XPW, false>;
+    allow_big_lds((const void*)kern, smem);
+    hipLaunchKernelGGL(kern, grid, dim3(256), smem, st, (const T*)A, (const T*)Bm, w, (T*)S, s, c, h * r, r, h, use_mult);
+  }
   return (int)hipGetLastError();
 }
 

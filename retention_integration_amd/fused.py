@@ -1,0 +1,121 @@
+"""The chunked power-retention path as ONE autograd node over the HIP library.
+
+Same arithmetic as composing the four operators through ``make_power_retention``
+(ref: retention/power_retention_maker.py:142-197), but the glue between the operators (chunk-local
+cumsum of the gates, key discounting, query gating, and their gradients) runs in two fused HIP kernels
+instead of a dozen elementwise launches, and only the first n entries of the scans are produced.
+"""
+from __future__ import annotations
+
+import torch
+
+from . import _lib
+from .ops import expanded_dim
+
+
+def _empty(shape, dtype, device):
+    return torch.empty(shape, dtype=dtype, device=device)
+
+
+class _ChunkedPowerRetention(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, Q, K, V, log_G, deg, scale, c):
+        lib = _lib.load()
+        st = _lib.stream()
+        b, t, hq, d = Q.shape
+        h = K.shape[2]
+        r = hq // h
+        n = t // c
+        BN = b * n
+        D = expanded_dim(d)
+        dev, dt = Q.device, Q.dtype
+        code = _lib.dtype_code(dt)
+        f32 = torch.float32
+        gated = log_G is not None
+        p = _lib.ptr
+
+        if gated:
+            A, lcs = _empty((BN, c, h), f32, dev), _empty((BN, h), f32, dev)
+            Kd, Qg = torch.empty_like(K), torch.empty_like(Q)
+            _lib.check(lib.pr_chunk_prep_fwd(p(log_G), p(K), p(Q), p(A), p(lcs), p(Kd), p(Qg), BN, c, h, r, d, deg, code,
+                                             st), "chunk_prep_fwd")
+        else:
+            A, Kd, Qg = None, K, Q
+            lcs = torch.zeros((BN, h), dtype=f32, device=dev)
+
+        S, s = _empty((BN, h, D, d), dt, dev), _empty((BN, h, D), f32, dev)
+        _lib.check(lib.pr_update_state_fwd(p(Kd), p(V), p(S), p(s), BN, c, h, d, 2, code, st), "update_state_fwd")
+        Sc, sc = torch.empty_like(S), torch.empty_like(s)
+        _lib.check(lib.pr_discumsum_fwd(p(S), p(lcs), p(Sc), b, n, n, h, D * d, code, st), "discumsum_fwd")
+        _lib.check(lib.pr_discumsum_fwd(p(s), p(lcs), p(sc), b, n, n, h, D, _lib.PR_F32, st), "discumsum_fwd")
+        del S, s
+
+        Ya = torch.empty_like(Q)
+        la, rm = _empty((BN, c, hq), f32, dev), _empty((BN, c, hq), f32, dev)
+        _lib.check(lib.pr_attention_fwd(p(Q), p(K), p(V), p(A), p(Ya), p(la), p(rm), BN, c, c, h, r, d, scale, deg, 0,
+                                        code, st), "attention_fwd")
+        O, den = torch.empty_like(Q), _empty((BN, c, hq), f32, dev)
+        _lib.check(lib.pr_query_state_fwd(p(Qg), p(Sc), p(sc), p(Ya), p(la), p(rm), p(O), p(den), BN, n, c, h, r, d,
+                                          scale ** deg, 2, 1, code, st), "query_state_fwd")
+        ctx.save_for_backward(Q, K, V, A, lcs, Kd if gated else None, Qg if gated else None, Sc, sc, rm, O, den)
+        ctx.meta = (deg, scale, c, gated)
+        return O
+
+    @staticmethod
+    def backward(ctx, dO):
+        Q, K, V, A, lcs, Kd, Qg, Sc, sc, rm, O, den = ctx.saved_tensors
+        deg, scale, c, gated = ctx.meta
+        if not gated:
+            Kd, Qg = K, Q
+        lib = _lib.load()
+        st = _lib.stream()
+        b, t, hq, d = Q.shape
+        h = K.shape[2]
+        r = hq // h
+        n = t // c
+        BN = b * n
+        D = expanded_dim(d)
+        dev, dt = Q.device, Q.dtype
+        code = _lib.dtype_code(dt)
+        f32, u8 = torch.float32, torch.uint8
+        p = _lib.ptr
+        dO = dO.contiguous()
+
+        dQg, dSc, dsc = torch.empty_like(Q), torch.empty_like(Sc), torch.empty_like(sc)
+        dYa, dla = torch.empty_like(Q), torch.empty_like(den)
+        ws = _empty((lib.pr_query_state_bwd_workspace(BN, c, h, r, d, code),), u8, dev)
+        _lib.check(lib.pr_query_state_bwd(p(Qg), p(Sc), p(sc), p(rm), p(O), p(den), p(dO), p(dQg), p(dSc), p(dsc),
+                                          p(dYa), p(dla), p(ws), BN, n, c, h, r, d, scale ** deg, 2, 1, code, st),
+                   "query_state_bwd")
+        dQa, dKa, dVa = torch.empty_like(Q), torch.empty_like(K), torch.empty_like(V)
+        dGq = _empty((BN, c, hq), f32, dev) if gated else None
+        dGk = _empty((BN, c, h), f32, dev) if gated else None
+        _lib.check(lib.pr_attention_bwd(p(Q), p(K), p(V), p(A), p(rm), p(dYa), p(dla), p(dQa), p(dKa), p(dVa), p(dGq),
+                                        p(dGk), BN, c, c, h, r, d, scale, deg, code, st), "attention_bwd")
+        if gated:
+            dGa = dGk.add_(dGq.view(BN, c, h, r).sum(-1)) if r > 1 else dGk.add_(dGq)
+        else:
+            dGa = None
+
+        dS, ds = torch.empty_like(Sc), torch.empty_like(sc)
+        dl1, dl2 = torch.empty_like(lcs), torch.empty_like(lcs)
+        ws = _empty((max(lib.pr_discumsum_bwd_workspace(b, n, h, D * d, code),
+                         lib.pr_discumsum_bwd_workspace(b, n, h, D, _lib.PR_F32)),), u8, dev)
+        _lib.check(lib.pr_discumsum_bwd(p(dSc), p(Sc), p(lcs), p(dS), p(dl1), p(ws), b, n, n, h, D * d, code, st),
+                   "discumsum_bwd")
+        _lib.check(lib.pr_discumsum_bwd(p(dsc), p(sc), p(lcs), p(ds), p(dl2), p(ws), b, n, n, h, D, _lib.PR_F32, st),
+                   "discumsum_bwd")
+        dKd, dVs = torch.empty_like(K), torch.empty_like(V)
+        _lib.check(lib.pr_update_state_bwd(p(Kd), p(V), p(dS), p(ds), p(dKd), p(dVs), BN, c, h, d, 2, code, st),
+                   "update_state_bwd")
+        dlg = _empty((b, t, h), f32, dev) if gated else None
+        # results are written in place over the attention gradients
+        _lib.check(lib.pr_chunk_glue_bwd(p(A), p(Kd), p(dKd), p(Qg), p(dQg), p(dKa), p(dQa), p(dVa), p(dVs), p(dGa),
+                                         p(dl1), p(dl2), p(dKa), p(dQa), p(dVa), p(dlg), BN, c, h, r, d, deg, code, st),
+                   "chunk_glue_bwd")
+        return dQa, dKa, dVa, dlg, None, None, None
+
+
+def chunked_power_retention(Q, K, V, log_G, deg, scale, chunk_size):
+    """Q [b,t,hq,d], K, V [b,t,h,d] contiguous, t a multiple of chunk_size, log_G [b,t,h] fp32 or None."""
+    return _ChunkedPowerRetention.apply(Q, K, V, log_G, int(deg), float(scale), int(chunk_size))

@@ -17,11 +17,13 @@ def _pad_time(x, pad, dims_after):
 
 
 def make_power_retention(update_state_impl, query_state_impl, discumsum_impl, attention_impl, *,
-                         scan_keeps_last=True):
+                         scan_keeps_last=True, chunked_impl=None):
     """Build ``power_retention`` from operator implementations.
 
     ``scan_keeps_last=False`` declares that ``discumsum_impl(X, log_G)`` already returns only the first n
-    entries of the scan (the composed path never reads the last one).
+    entries of the scan (the composed path never reads the last one).  ``chunked_impl(Q, K, V, log_G, deg,
+    scale, chunk_size)``, when given, replaces the composition of the four operators on the chunked branch
+    (same result; used for the fused single-node path).
     """
 
     def power_retention(Q, K, V, log_G=None, initial_state=None, return_final_state=False,
@@ -68,6 +70,10 @@ def make_power_retention(update_state_impl, query_state_impl, discumsum_impl, at
         if switch_over_seq_len is None or t <= switch_over_seq_len:  # quadratic form (:128-140)
             A = log_G.cumsum(1) if gated else None
             return attention_impl(Q, K, V, A, deg, scale=scale, norm=True)
+
+        if chunked_impl is not None:
+            return chunked_impl(Q.contiguous(), K.contiguous(), V.contiguous(),
+                                log_G.contiguous() if gated else None, deg, scale, c)
 
         Qc, Kc, Vc = Q.view(b, n, c, hq, d), K.view(b, n, c, h, d), V.view(b, n, c, h, d)
         if gated:

@@ -54,9 +54,20 @@ def run_both(pra, Q, K, V, lg, chunk, dO=None, **kw):
     if dO is not None:
         Y.backward(dO.to(DEV))
         Yo.backward(dO.float())
+        tol = {n: GRAD_TOL for n in ("dQ", "dK", "dV", "dlog_G")}
+        if chunk is None:
+            # Quadratic path on a short sequence: the first rows see one or two keys, their true gradient is a
+            # cancellation to ~0 and any 16-bit run leaves a residual there.  Use the reference's own bar for such
+            # cases (ref: perf/_checks.py:272-320): no worse than a small multiple of the 16-bit reference's error.
+            ri = [x.clone().requires_grad_(True) if x is not None else None for x in (Q, K, V, lg)]
+            Yr = oracle.power_retention(*ri, deg=2, chunk_size=chunk, **kw)
+            Yr.backward(dO)
+            for nm, r_, g_ in zip(tol, ri, oi):
+                if r_ is not None:
+                    tol[nm] = max(GRAD_TOL, 2.0 * rel_l2(r_.grad, g_.grad))
         for nm, a, b_ in zip(["dQ", "dK", "dV", "dlog_G"], gi, oi):
             if a is not None:
-                check(nm, a.grad, b_.grad, GRAD_TOL)
+                check(nm, a.grad, b_.grad, tol[nm])
     return Y
 
 
@@ -74,6 +85,22 @@ def test_power_retention_fwd_bwd(pra, dtype, b, t, h, r, d, chunk, gated):
     g = torch.Generator().manual_seed(7)
     dO = torch.randn(b, t, h * r, d, generator=g).to(dtype)
     run_both(pra, Q, K, V, lg, chunk, dO)
+
+
+@pytest.mark.parametrize("gated,r", [(True, 1), (True, 2), (False, 1)])
+def test_fused_node_equals_operator_composition(pra, gated, r):
+    """power_retention (one fused autograd node) vs the same function assembled from the four operators
+    through make_power_retention: same kernels, so agreement is at rounding level."""
+    Q, K, V, lg = make_inputs(2, 512, 2, r, 64, torch.bfloat16, gated, seed=21)
+    dO = torch.randn(2, 512, 2 * r, 64, generator=torch.Generator().manual_seed(3)).to(torch.bfloat16).to(DEV)
+    outs = []
+    for fn in (pra.power_retention, pra.power_retention_composed):
+        xs = [x.to(DEV).requires_grad_(True) if x is not None else None for x in (Q, K, V, lg)]
+        Y = fn(*xs, deg=2, chunk_size=128)
+        Y.backward(dO)
+        outs.append([Y] + [x.grad for x in xs if x is not None])
+    for nm, a, b_ in zip(["Y", "dQ", "dK", "dV", "dlog_G"], *outs):
+        check(f"fused vs composed {nm}", a, b_, 4e-3)
 
 
 def test_fp32_inputs_are_rejected_loudly(pra):
