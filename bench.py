@@ -81,7 +81,7 @@ def op_breakdown(pra, Q, K, V, lg, dO, cfg, iters=5):
     dOc = dO.view(b, n, c, h, d)
     res["query_state_bwd"] = event_time_ms(lambda: ops.query_state_bwd(Qc, Sc, sc, rm5, O, den, dOc, scale ** 2, True), iters)
     dOf = dO.view(b * n, c, h, d)
-    res["attention_bwd"] = event_time_ms(lambda: ops.attention_bwd(Qf, Kf, Vf, Af, rm, dOf, la, 2, scale), iters)
+    res["attention_bwd"] = event_time_ms(lambda: ops.attention_bwd(Qf, Kf, Vf, Af, rm, dOf, la, None, 2, scale), iters)
     res["discumsum_bwd(S)"] = event_time_ms(lambda: ops.discumsum_bwd(Sc, Sc, lcs), iters)
     res["update_state_bwd"] = event_time_ms(lambda: ops.update_state_bwd(Kc, Vc, S, s), iters)
     return {k: round(v, 4) for k, v in res.items()}

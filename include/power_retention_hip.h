@@ -53,12 +53,16 @@ int pr_attention_fwd(const void* Q, const void* K, const void* V, const float* G
                      void* stream);
 
 /* Backward of the above w.r.t. (o, l) of the norm == 0 form -- retention/_attention/triton.py:228-603,723-810.
- *   rowmax as returned by the forward; dO [B,tq,h*r,d]; dl [B,tq,h*r] fp32 or NULL (zero)
+ *   rowmax as returned by the forward; dO [B,tq,h*r,d]; dl [B,tq,h*r] fp32 or NULL (zero);
+ *   dO_scale [B,tq,h*r] fp32 or NULL: the gradient of o is dO * dO_scale[row], scaled in fp32 (the norm != 0
+ *   form passes dY with dO_scale = 1/l and dl = -sum(dY*Y)/l, which keeps the cancellation of rows that see
+ *   a single key exact)
  *   -> dQ [B,tq,h*r,d], dK, dV [B,tk,h,d]; when G != NULL also dGq [B,tq,h*r] (sum_j dz_ij) and
  *   dGk [B,tk,h] (-sum_i dz_ij), whose sum over the aligned positions is d log_G_accum. */
 int pr_attention_bwd(const void* Q, const void* K, const void* V, const float* G, const float* rowmax,
-                     const void* dO, const float* dl, void* dQ, void* dK, void* dV, float* dGq, float* dGk, int B,
-                     int tq, int tk, int h, int r, int d, float scale, int deg, int dtype, void* stream);
+                     const void* dO, const float* dl, const float* dO_scale, void* dQ, void* dK, void* dV,
+                     float* dGq, float* dGk, int B, int tq, int tk, int h, int r, int d, float scale, int deg,
+                     int dtype, void* stream);
 
 /* update_state(K, V, deg) -- retention/_update_state/reference.py:33-52,86-94,
  * Triton twin retention/_update_state/triton.py:61-133,280-320.

@@ -25,7 +25,7 @@ SIGNATURES = {
     "pr_last_error": (c_char_p, []),
     "pr_expanded_dim": (c_int, [_I, _I]),
     "pr_attention_fwd": (c_int, [_P] * 7 + [_I] * 6 + [_F, _I, _I, _I, _P]),
-    "pr_attention_bwd": (c_int, [_P] * 12 + [_I] * 6 + [_F, _I, _I, _P]),
+    "pr_attention_bwd": (c_int, [_P] * 13 + [_I] * 6 + [_F, _I, _I, _P]),
     "pr_update_state_fwd": (c_int, [_P] * 4 + [_I] * 6 + [_P]),
     "pr_update_state_bwd": (c_int, [_P] * 6 + [_I] * 6 + [_P]),
     "pr_discumsum_fwd": (c_int, [_P] * 3 + [_I] * 4 + [c_int64, _I, _P]),

@@ -74,7 +74,7 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dq_kernel(AttnBwdArgs a)
   int ti[MT];
   long qoff[MT];
   bool live[MT];
-  float base[MT], dlr[MT], dgq[MT];   // base = G_q - m
+  float base[MT], dlr[MT], dgq[MT], osc[MT];   // base = G_q - m
 #pragma unroll
   for (int mi = 0; mi < MT; mi++) {
     const int row = row0 + wave * 16 * MT + 16 * mi + tcol;
@@ -96,6 +96,7 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dq_kernel(AttnBwdArgs a)
     const long so = (long)b * a.tq * hq + qoff[mi];
     base[mi] = (Gg ? Gg[(long)ti[mi] * a.h] : 0.f) - a.rowmax[so];
     dlr[mi] = a.dl ? a.dl[so] : 0.f;
+    osc[mi] = a.dO_scale ? a.dO_scale[so] : 1.f;
     dgq[mi] = 0.f;
   }
   f32x4 acc[MT][NT];
@@ -193,7 +194,7 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dq_kernel(AttnBwdArgs a)
               E = eu[mi] * gkv[v];
             }
             float p, dz, dsr;
-            pair_grad<DEG2>(s[v], E, dp[v] + dlr[mi], eps_s, half_deg, p, dz, dsr);
+            pair_grad<DEG2>(s[v], E, dp[v] * osc[mi] + dlr[mi], eps_s, half_deg, p, dz, dsr);
             dgq[mi] += dz;
             d8[mi][4 * half + v] = dsr;
           }
@@ -242,7 +243,7 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
   extern __shared__ __attribute__((aligned(16))) char smem[];
   T* Qt = (T*)smem;                       // [2][BM][LD]
   T* dOt = Qt + 2 * AB_BM * LD;           // [2][BM][LD]
-  float* rowv = (float*)(dOt + 2 * AB_BM * LD);  // [2][4][BM]: G_q - m, dl, time index, scale^deg exp(G_q - m - R)
+  float* rowv = (float*)(dOt + 2 * AB_BM * LD);  // [2][5][BM]: G_q - m, dl, time index, scale^deg exp(G_q - m - R), dO scale
 
   const int tid = threadIdx.x, l = tid & 63, g = l >> 4, wave = tid >> 6, kcol = l & 15;
   const int b = blockIdx.y / a.h, hh = blockIdx.y % a.h;
@@ -296,7 +297,7 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
   const int nsteps = (rows - row_begin + AB_BM - 1) / AB_BM;
 
   u32x4 rq[PT], rdo[PT];
-  float r0 = 0.f, r1 = 0.f, r2 = 0.f;
+  float r0 = 0.f, r1 = 0.f, r2 = 0.f, r3 = 1.f;
   auto fetch = [&](int rbase) {
 #pragma unroll
     for (int i = 0; i < PT; i++) {
@@ -313,13 +314,14 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
     }
     if (tid < AB_BM) {
       const int row = rbase + tid;
-      r0 = 0.f; r1 = 0.f; r2 = -1.f;  // time index -1: sees no key
+      r0 = 0.f; r1 = 0.f; r2 = -1.f; r3 = 1.f;  // time index -1: sees no key
       if (row < rows) {
         const int t = row / a.r;
         const long so = (long)b * a.tq * hq + (long)t * hq + hh * a.r + (row - t * a.r);
         r0 = (Gg ? Gg[(long)(t + shift) * a.h] : 0.f) - a.rowmax[so];
         r1 = a.dl ? a.dl[so] : 0.f;
         r2 = (float)(t + shift);
+        r3 = a.dO_scale ? a.dO_scale[so] : 1.f;
       }
     }
   };
@@ -334,11 +336,12 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
       }
     }
     if (tid < AB_BM) {
-      float* rv = rowv + stage * 4 * AB_BM;
+      float* rv = rowv + stage * 5 * AB_BM;
       rv[tid] = r0;
       rv[AB_BM + tid] = r1;
       rv[2 * AB_BM + tid] = r2;
       rv[3 * AB_BM + tid] = scale_p * __expf(fminf(r0 - R, AB_EXP_CLAMP));
+      rv[4 * AB_BM + tid] = r3;
     }
   };
 
@@ -350,7 +353,7 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
     if (it + 1 < nsteps) fetch(rbase + AB_BM);
     const T* qt_ = Qt + stage * AB_BM * LD;
     const T* dot_ = dOt + stage * AB_BM * LD;
-    const float* rv = rowv + stage * 4 * AB_BM;
+    const float* rv = rowv + stage * 5 * AB_BM;
     // exact per-pair path unless every row of the step is real and sees every (real) key of the workgroup
     const bool diag = (rbase / a.r + shift < last_key) || (rbase + AB_BM > rows) || (key0 + KEYS > a.tk);
 
@@ -368,6 +371,7 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
         const f32x4 gm = *(const f32x4*)(rv + (diag ? 0 : 3 * AB_BM) + 16 * qt + 4 * g);
         const f32x4 dlv = *(const f32x4*)(rv + AB_BM + 16 * qt + 4 * g);
         const f32x4 tiv = *(const f32x4*)(rv + 2 * AB_BM + 16 * qt + 4 * g);
+        const f32x4 osv = *(const f32x4*)(rv + 4 * AB_BM + 16 * qt + 4 * g);
 #pragma unroll
         for (int kj = 0; kj < MK; kj++) {
           f32x4 s = {0, 0, 0, 0}, dp = {0, 0, 0, 0};
@@ -386,9 +390,9 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
               E = gm[v] * ev[kj];
             }
             float p, dz, dsr;
-            pair_grad<DEG2>(s[v], E, dp[v] + dlv[v], eps_s, half_deg, p, dz, dsr);
+            pair_grad<DEG2>(s[v], E, dp[v] * osv[v] + dlv[v], eps_s, half_deg, p, dz, dsr);
             dgk[kj] -= dz;
-            p8[kj][4 * qt + v] = p;
+            p8[kj][4 * qt + v] = p * osv[v];
             d8[kj][4 * qt + v] = dsr;
           }
         }
@@ -449,7 +453,7 @@ template <typename T, int DH, bool DEG2> static int attn_bwd_launch(const AttnBw
   }
   {
     constexpr int MK = DH <= 64 ? 2 : 1;
-    constexpr size_t smem = 2 * 2 * AB_BM * (DH + 8) * sizeof(T) + 2 * 4 * AB_BM * sizeof(float);
+    constexpr size_t smem = 2 * 2 * AB_BM * (DH + 8) * sizeof(T) + 2 * 5 * AB_BM * sizeof(float);
     dim3 grid((a.tk + 64 * MK - 1) / (64 * MK), (unsigned)(B * a.h));
     auto kern = attention_bwd_dkv_kernel<T, DH, MK, DEG2>;
     allow_big_lds((const void*)kern, smem);

@@ -171,9 +171,10 @@ __global__ __launch_bounds__(256) void attention_fwd_kernel(AttnFwdArgs a) {
           }
           p[kt][v] = w;
           mx[mi] = fmaxf(mx[mi], w);
-          lsum[mi] += w;
         }
       }
+      // the row sum is taken over the weights as the matrix cores will see them (rounded to 16 bit), so that
+      // o / l is an exact average (ref rounds p before summing: retention/_attention/reference.py:52-55)
 #pragma unroll
       for (int kp = 0; kp < KT / 2; kp++) {
         float q8[8];
@@ -183,6 +184,9 @@ __global__ __launch_bounds__(256) void attention_fwd_kernel(AttnFwdArgs a) {
           q8[4 + v] = p[2 * kp + 1][v];
         }
         pf[mi][kp] = pack8<T>(q8);
+        unpack8(pf[mi][kp], q8);
+#pragma unroll
+        for (int v = 0; v < 8; v++) lsum[mi] += q8[v];
       }
     }
     // O^T += V^T P^T, 32 keys per step: elements 0-3 are keys 4g.. of the first 16, 4-7 of the second 16

@@ -60,8 +60,9 @@ int pr_attention_fwd(const void* Q, const void* K, const void* V, const float* G
 }
 
 int pr_attention_bwd(const void* Q, const void* K, const void* V, const float* G, const float* rowmax,
-                     const void* dO, const float* dl, void* dQ, void* dK, void* dV, float* dGq, float* dGk, int B,
-                     int tq, int tk, int h, int r, int d, float scale, int deg, int dtype, void* stream) {
+                     const void* dO, const float* dl, const float* dO_scale, void* dQ, void* dK, void* dV,
+                     float* dGq, float* dGk, int B, int tq, int tk, int h, int r, int d, float scale, int deg,
+                     int dtype, void* stream) {
   if (int rc = check_common("attention_bwd", d, deg, dtype, false)) return rc;
   if (bad_ptr(Q) || bad_ptr(K) || bad_ptr(V) || bad_ptr(rowmax) || bad_ptr(dO) || bad_ptr(dQ) || bad_ptr(dK) ||
       bad_ptr(dV) || bad_opt(G) || bad_opt(dl) || bad_opt(dGq) || bad_opt(dGk))
@@ -69,7 +70,7 @@ int pr_attention_bwd(const void* Q, const void* K, const void* V, const float* G
   if (G && (!dGq || !dGk)) return fail(PR_ERR_ARG, "attention_bwd: dGq and dGk are required when G is given");
   if (B <= 0 || tq <= 0 || tk <= 0 || h <= 0 || r <= 0 || tq > tk)
     return fail(PR_ERR_ARG, "attention_bwd: need B,tq,tk,h,r > 0 and tq <= tk");
-  pr::AttnBwdArgs a{Q, K, V, G, rowmax, dO, dl, dQ, dK, dV, G ? dGq : nullptr, G ? dGk : nullptr,
+  pr::AttnBwdArgs a{Q, K, V, G, rowmax, dO, dl, dO_scale, dQ, dK, dV, G ? dGq : nullptr, G ? dGk : nullptr,
                     tq, tk, h, r, scale, (float)deg};
   return finish(pr::attention_bwd(a, B, d, dtype, (hipStream_t)stream), "attention_bwd");
 }

@@ -67,6 +67,7 @@ struct AttnBwdArgs {
   const float* rowmax;  // [B, tq, h*r]
   const void* dO;       // [B, tq, h*r, d]
   const float* dl;      // [B, tq, h*r] or null
+  const float* dO_scale;  // [B, tq, h*r] or null: dO is used as dO * dO_scale[row] (scaled in fp32)
   void* dQ;             // [B, tq, h*r, d]
   void* dK;             // [B, tk, h, d]
   void* dV;             // [B, tk, h, d]

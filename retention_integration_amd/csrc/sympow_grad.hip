@@ -10,42 +10,59 @@
 //   * update_state backward, dK: X = K, G = V, cvec = 1, B = dS, sB = ds, m = 2 below the block diagonal
 //                                                  (ref: retention/_update_state/reference.py:55-83)
 //
-// dphi is never stored.  A workgroup = 4 waves owns 64*MT rows (16*MT per wave).  For one x column X and
-// one 16-wide strip y the wave forms the 16x16 tile dphi^T[i, row] (i = feature within the strip) on the
-// matrix cores, B rows straight from LDS as the A operand and G^T from registers as the B operand,
-// then folds it twice on the VALU: into dX[row, 16y+i] (times X[row, X]) kept in registers, and into
-// dX[row, X] (dot with X[row, 16y+i] over i) reduced across the wave and parked in LDS.
+// dphi is never stored.  A workgroup = 4 waves owns 64*MT rows (16*MT per wave) and sweeps B in memory order,
+// 64 feature rows (four x columns of one 16-wide strip y) per pipeline stage, through a 3-deep ring of
+// asynchronous global->LDS copies.  For an x column X the wave forms the 16x16 tile dphi^T[i, row] on the matrix
+// cores (B rows from LDS as the A operand, G^T from registers as the B operand) and folds it twice:
+//   * into dX[row, 16y+i]: multiply by the per-row scalar X[row, X] and accumulate (VALU);
+//   * into dX[row, X]: multiply elementwise by X[row, 16y+i], round to 16 bit and sum over i on the matrix
+//     cores with a 0/1 selector operand that routes the sum of column X to accumulator row X % 16.
+// Both land in the same accumulator layout (coordinate on the accumulator rows, workgroup row on the lanes), so
+// the result never leaves registers.  The sB term is linear in X: dX_s = cvec * (X M) with the symmetric d x d
+// matrix M[a, b] = sum of m_f sB[f] over the stored features pairing a and b; it is one small product at the end.
+// Workgroups that share a state (the row blocks of one (chunk, head)) are placed on the same XCD so that the
+// state is fetched from HBM once and re-read from that XCD's L2.
 #include "common.h"
 #include "kernels.h"
 
 namespace pr {
 
-template <typename T, int DK, int DV, int MT, int XS, bool MULT>
-__global__ __launch_bounds__(256) void sympow_grad_kernel(GradArgs a) {
+constexpr int GR_FR = 64;    // feature rows per stage
+constexpr int GR_NST = 3;
+
+template <typename T> struct OnePair;   // two packed 1.0 values
+template <> struct OnePair<bf16_t> { static constexpr uint32_t v = 0x3F803F80u; static constexpr float down = 1.f, up = 1.f; };
+template <> struct OnePair<f16_t> { static constexpr uint32_t v = 0x3C003C00u; static constexpr float down = 1.f / 256.f, up = 256.f; };
+
+template <typename T, int DK, int DV, int MT, bool MULT>
+__global__ __launch_bounds__(256, 2) void sympow_grad_kernel(GradArgs a, int row_blocks, int npairs) {
   typedef typename VecOf<T>::v8 v8;
   typedef typename VecOf<T>::v4 v4;
-  constexpr int TT = DK / 16, KS = DV / 32, LDB = DV + 8, ROWS = 64 * MT;
-  constexpr int D = 128 * TT * (TT + 1);
-  constexpr int SROWS = 16 * XS;                     // B rows per strip per stage
-  constexpr int CH_PER_Y = SROWS * DV / 8;           // 16-byte chunks per strip
-  constexpr int MAX_PT = (TT * CH_PER_Y + 255) / 256;
-  constexpr int NSTAGE = TT * (16 / XS);
-  extern __shared__ __attribute__((aligned(16))) char smem[];
-  T* bt = (T*)smem;                                   // [2][TT][SROWS][LDB]
-  float* st = (float*)(bt + 2 * TT * SROWS * LDB);    // [2][TT][SROWS]
-  float* dxb = st + 2 * TT * SROWS;                   // [ROWS][DK + 1]
-  constexpr int LDD = DK + 1;
+  constexpr int TT = DK / 16, KS = DV / 32, KX = DK / 32, ROWS = 64 * MT, CB = DV / 8, CX = DK / 8;
+  constexpr int D = 128 * TT * (TT + 1), NSTEP = D / GR_FR;
+  constexpr int STAGE = GR_FR * DV * 2;
+  constexpr int LOADS = GR_FR * CB / 256;
+  constexpr int LDM = DK + 8;
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  char* ring = smem;                                         // [NST][STAGE]; reused for M at the end
+  char* xt = ring + GR_NST * STAGE;                          // [ROWS][DK] T, swizzled
+
+  // XCD-aware placement: consecutive workgroup ids go to different XCDs, so id % 8 picks the XCD
+  const int xcd = blockIdx.x % 8, slot = blockIdx.x / 8;
+  const int pair = (slot / row_blocks) * 8 + xcd;
+  if (pair >= npairs) return;
+  const int row0 = (slot % row_blocks) * ROWS;
+  const int bn = pair / a.h, hh = pair % a.h;
 
   const int tid = threadIdx.x, l = tid & 63, g = l >> 4, wave = tid >> 6, tcol = l & 15;
-  const int bn = blockIdx.y / a.h, hh = blockIdx.y % a.h;
   const int hA = a.h * a.r, rows = a.c * a.r;
-  const int row0 = blockIdx.x * ROWS;
   const T* Xg = (const T*)a.X + (long)bn * a.c * hA * DK;
   const T* Gg = (const T*)a.G + (long)bn * a.c * hA * DV;
-  const T* Bg = (const T*)a.B + ((long)bn * a.h + hh) * D * DV;
+  const char* Bg = (const char*)((const T*)a.B + ((long)bn * a.h + hh) * D * DV);
   const float* sBg = a.sB + ((long)bn * a.h + hh) * D;
   T* dXg = (T*)a.dX + (long)bn * a.c * hA * DK;
   auto row_off = [&](int row) -> long {
+    row = min(row, rows - 1);
     const int t = row / a.r, rr = row - t * a.r;
     return (long)t * hA + hh * a.r + rr;
   };
@@ -58,175 +75,180 @@ __global__ __launch_bounds__(256) void sympow_grad_kernel(GradArgs a) {
     return;
   }
 
+  auto issue = [&](int step) {
+    const char* src = Bg + (long)step * GR_FR * DV * 2;
+    async_load_tile<CB, GR_FR>(ring + (step % GR_NST) * STAGE, [&](int row) { return src + row * (DV * 2); });
+  };
+  // X rows of this workgroup (waited for together with stage 0), then the first two stages
+  async_load_tile<CX, ROWS>(xt, [&](int row) { return (const char*)(Xg + row_off(row0 + row) * DK); });
+  issue(0);
+  issue(1);
+
   // per-lane row data (row = this lane's column of the dphi^T tiles)
   v8 Gf[MT][KS];
-  float xr[MT][TT][4];
   float cv[MT];
-  long roff[MT];
-  bool rlive[MT];
+  int lrow[MT];
+  bool live[MT];
 #pragma unroll
   for (int mi = 0; mi < MT; mi++) {
-    const int row = row0 + wave * 16 * MT + 16 * mi + tcol;
-    rlive[mi] = row < rows;
-    roff[mi] = row_off(rlive[mi] ? row : 0);
+    lrow[mi] = wave * 16 * MT + 16 * mi + tcol;
+    live[mi] = row0 + lrow[mi] < rows;
+    const long ro = row_off(row0 + lrow[mi]);
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) {
-      u32x4 z = {0, 0, 0, 0};
-      if (rlive[mi]) z = *(const u32x4*)(Gg + roff[mi] * DV + 32 * ks + 8 * g);
+      u32x4 z = *(const u32x4*)(Gg + ro * DV + 32 * ks + 8 * g);
+      if (!live[mi]) z = (u32x4){0, 0, 0, 0};
       Gf[mi][ks] = __builtin_bit_cast(v8, z);
     }
-#pragma unroll
-    for (int y = 0; y < TT; y++) {
-      u32x2 z = {0, 0};
-      if (rlive[mi]) z = *(const u32x2*)(Xg + roff[mi] * DK + 16 * y + 4 * g);
-      v4 h4 = __builtin_bit_cast(v4, z);
-#pragma unroll
-      for (int v = 0; v < 4; v++) xr[mi][y][v] = (float)h4[v];
-    }
-    cv[mi] = rlive[mi] ? (a.cvec ? a.cvec[(long)bn * a.c * hA + roff[mi]] : 1.f) : 0.f;
+    cv[mi] = live[mi] ? (a.cvec ? a.cvec[(long)bn * a.c * hA + ro] : 1.f) : 0.f;
   }
-  f32x4 accA[MT][TT];
-#pragma unroll
-  for (int mi = 0; mi < MT; mi++)
-#pragma unroll
-    for (int y = 0; y < TT; y++) accA[mi][y] = (f32x4){0, 0, 0, 0};
-
-  // stage s covers x columns Xbase .. Xbase+XS-1 of block column xb, strips y = xb .. TT-1
-  u32x4 rb[MAX_PT];
-  float rs[(TT * SROWS + 255) / 256];
-  T xnext[MT][XS];  // X[row, Xbase + xx] of the stage being fetched
-  auto fetch = [&](int s) {
-    const int xb = s / (16 / XS), Xbase = 16 * xb + XS * (s % (16 / XS));
-    const int ny = TT - xb;
-#pragma unroll
-    for (int mi = 0; mi < MT; mi++)
-#pragma unroll
-      for (int xx = 0; xx < XS; xx++) xnext[mi][xx] = rlive[mi] ? Xg[roff[mi] * DK + Xbase + xx] : (T)0.f;
-#pragma unroll
-    for (int i = 0; i < MAX_PT; i++) {
-      const int ch = tid + 256 * i;
-      if (ch < ny * CH_PER_Y) {
-        const int yy = ch / CH_PER_Y, rem = ch % CH_PER_Y, y = xb + yy;
-        const int rl = rem / (DV / 8), col = (rem % (DV / 8)) * 8;
-        rb[i] = *(const u32x4*)(Bg + (long)(128 * y * (y + 1) + 16 * Xbase + rl) * DV + col);
-      }
-    }
-#pragma unroll
-    for (int i = 0; i < (TT * SROWS + 255) / 256; i++) {
-      const int j = tid + 256 * i;
-      if (j < ny * SROWS) {
-        const int yy = j / SROWS, y = xb + yy;
-        rs[i] = sBg[128 * y * (y + 1) + 16 * Xbase + j % SROWS];
-      }
-    }
+  auto x_ptr = [&](int mi, int col) -> const char* {   // address of X[lrow[mi], col] in the swizzled tile
+    return xt + lrow[mi] * (DK * 2) + (((col / 8) ^ swz<CX>(lrow[mi])) * 16) + (col % 8) * 2;
   };
-  auto stash = [&](int s, int stage) {
-    const int xb = s / (16 / XS);
-    const int ny = TT - xb;
-    T* b = bt + stage * TT * SROWS * LDB;
+
+  f32x4 acc[MT][TT];            // dX^T[16*blk + 4g + v, row]
+  f32x4 accA[MT], accB[MT];     // contributions of the current 16x16 feature block (y, xb)
+  float xr[MT][4];              // X[row, 16y + 4g + v]
 #pragma unroll
-    for (int i = 0; i < MAX_PT; i++) {
-      const int ch = tid + 256 * i;
-      if (ch < ny * CH_PER_Y) {
-        const int yy = ch / CH_PER_Y, rem = ch % CH_PER_Y;
-        *(u32x4*)(b + (yy * SROWS + rem / (DV / 8)) * LDB + (rem % (DV / 8)) * 8) = rb[i];
-      }
-    }
+  for (int mi = 0; mi < MT; mi++) {
 #pragma unroll
-    for (int i = 0; i < (TT * SROWS + 255) / 256; i++) {
-      const int j = tid + 256 * i;
-      if (j < ny * SROWS) st[stage * TT * SROWS + j] = rs[i];
+    for (int k = 0; k < TT; k++) acc[mi][k] = (f32x4){0, 0, 0, 0};
+    accA[mi] = (f32x4){0, 0, 0, 0};
+    accB[mi] = (f32x4){0, 0, 0, 0};
+  }
+  int y_cur = 0, xb_cur = 0;
+  auto commit_block = [&]() {
+    const float m = (MULT && xb_cur < y_cur) ? 2.f : 1.f;
+#pragma unroll
+    for (int mi = 0; mi < MT; mi++) {
+      static_for<TT>([&](auto k) {
+        if (k.value == y_cur) acc[mi][k.value] += accA[mi] * m;
+        if (k.value == xb_cur) acc[mi][k.value] += accB[mi] * m;
+      });
+      accA[mi] = (f32x4){0, 0, 0, 0};
+      accB[mi] = (f32x4){0, 0, 0, 0};
     }
   };
 
-  fetch(0);
-  for (int s = 0; s < NSTAGE; s++) {
-    const int stage = s & 1;
-    stash(s, stage);
-    float xcur[MT][XS];
-#pragma unroll
-    for (int mi = 0; mi < MT; mi++)
-#pragma unroll
-      for (int xx = 0; xx < XS; xx++) xcur[mi][xx] = (float)xnext[mi][xx];
+  for (int step = 0; step < NSTEP; step++) {
+    const char* st = ring + (step % GR_NST) * STAGE;
+    if (step + 1 < NSTEP) wait_vmcnt<LOADS>(); else wait_vmcnt<0>();
     __syncthreads();
-    if (s + 1 < NSTAGE) fetch(s + 1);
-    const int xb = s / (16 / XS), Xbase = 16 * xb + XS * (s % (16 / XS));
-    const T* b = bt + stage * TT * SROWS * LDB;
-    const float* sv = st + stage * TT * SROWS;
+    if (step + 2 < NSTEP) issue(step + 2);
+    const int f0 = step * GR_FR;
+    int y = 0;
+    while (128 * (y + 1) * (y + 2) <= f0) y++;
+    const int X0 = (f0 - 128 * y * (y + 1)) / 16, xb = X0 / 16;
+    if (step == 0 || y != y_cur || xb != xb_cur) {
+      if (step > 0) commit_block();
+      if (step == 0 || y != y_cur) {
 #pragma unroll
-    for (int xx = 0; xx < XS; xx++) {
-      const int X = Xbase + xx;
-      float xX[MT], pd[MT], po[MT];
+        for (int mi = 0; mi < MT; mi++) {
+          const v4 h4 = *(const v4*)x_ptr(mi, 16 * y + 4 * g);
 #pragma unroll
-      for (int mi = 0; mi < MT; mi++) {
-        xX[mi] = xcur[mi][xx];
-        pd[mi] = 0.f;
-        po[mi] = 0.f;
-      }
-#pragma unroll
-      for (int yy = 0; yy < TT; yy++) {
-        const int y = xb + yy;
-        if (y < TT) {
-          v8 af[KS];
-#pragma unroll
-          for (int ks = 0; ks < KS; ks++) af[ks] = lds_frag<T>(b + yy * SROWS * LDB, LDB, 16 * xx, 32 * ks);
-          const f32x4 s4 = *(const f32x4*)(sv + yy * SROWS + 16 * xx + 4 * g);
-          const bool off = MULT && (yy > 0);
-#pragma unroll
-          for (int mi = 0; mi < MT; mi++) {
-            f32x4 dphi = s4 * cv[mi];
-#pragma unroll
-            for (int ks = 0; ks < KS; ks++) dphi = mfma16(af[ks], Gf[mi][ks], dphi);
-            const float xs = off ? 2.f * xX[mi] : xX[mi];
-            // xr is indexed by the runtime strip y: select with a compile-time loop
-            float dot = 0.f;
-#pragma unroll
-            for (int yc = 0; yc < TT; yc++) {
-              if (yc == y) {
-                accA[mi][yc] += dphi * xs;
-#pragma unroll
-                for (int v = 0; v < 4; v++) dot += xr[mi][yc][v] * dphi[v];
-              }
-            }
-            if (off) po[mi] += dot; else pd[mi] += dot;
-          }
+          for (int v = 0; v < 4; v++) xr[mi][v] = (float)h4[v];
         }
       }
+      y_cur = y;
+      xb_cur = xb;
+    }
+#pragma unroll
+    for (int pr2 = 0; pr2 < GR_FR / 32; pr2++) {
+      const int X = X0 + 2 * pr2, m0 = X % 16;
+      v8 af0[KS], af1[KS];
+#pragma unroll
+      for (int ks = 0; ks < KS; ks++) {
+        af0[ks] = sw_frag<T, CB>(st, 32 * pr2, 32 * ks);
+        af1[ks] = sw_frag<T, CB>(st, 32 * pr2 + 16, 32 * ks);
+      }
+      // selector: accumulator row m0 sums the first 16 contraction slots (column X), row m0+1 the last 16
+      const uint32_t s_lo = (tcol == m0) ? OnePair<T>::v : 0u, s_hi = (tcol == m0 + 1) ? OnePair<T>::v : 0u;
+      const v8 sel = __builtin_bit_cast(v8, (u32x4){s_lo, s_lo, s_hi, s_hi});
 #pragma unroll
       for (int mi = 0; mi < MT; mi++) {
-        const float tot = sum_over_rows(pd[mi] + 2.f * po[mi]);
-        if (g == (X & 3)) dxb[(wave * 16 * MT + 16 * mi + tcol) * LDD + X] = tot;
+        f32x4 d0 = {0, 0, 0, 0}, d1 = {0, 0, 0, 0};
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) {
+          d0 = mfma16(af0[ks], Gf[mi][ks], d0);
+          d1 = mfma16(af1[ks], Gf[mi][ks], d1);
+        }
+        const float x0 = (float)*(const T*)x_ptr(mi, X), x1 = (float)*(const T*)x_ptr(mi, X + 1);
+        accA[mi] += d0 * x0 + d1 * x1;
+        float w8[8];
+#pragma unroll
+        for (int v = 0; v < 4; v++) {
+          w8[v] = xr[mi][v] * d0[v];
+          w8[4 + v] = xr[mi][v] * d1[v];
+        }
+        accB[mi] = mfma16(sel, pack8<T>(w8), accB[mi]);
       }
     }
   }
-  __syncthreads();
+  commit_block();
+
+  // sB term: dX_s^T[w, row] = cvec[row] * sum_a M[w, a] X[row, a], M in two 16-bit parts (high, low) built in the
+  // (now idle) ring memory.
+  T* Mt = (T*)ring;   // [DK][LDM]
+  for (int part = 0; part < 2; part++) {
+    __syncthreads();
+    for (int idx = tid; idx < DK * DK; idx += 256) {
+      const int w = idx / DK, aa = idx % DK, yw = w / 16, ya = aa / 16;
+      float val;
+      if (ya == yw) {
+        val = sBg[128 * yw * (yw + 1) + 16 * aa + (w - 16 * yw)] + sBg[128 * yw * (yw + 1) + 16 * w + (aa - 16 * yw)];
+      } else {
+        const int lo = ya < yw ? aa : w, hi = ya < yw ? w : aa, yh = hi / 16;
+        val = sBg[128 * yh * (yh + 1) + 16 * lo + (hi - 16 * yh)] * (MULT ? 2.f : 1.f);
+      }
+      val *= OnePair<T>::down;
+      const T hi16 = (T)val;
+      Mt[w * LDM + aa] = part == 0 ? hi16 : (T)(val - (float)hi16);
+    }
+    __syncthreads();
 #pragma unroll
-  for (int mi = 0; mi < MT; mi++)
+    for (int mi = 0; mi < MT; mi++) {
+      v8 xf[KX];
 #pragma unroll
-    for (int y = 0; y < TT; y++)
+      for (int ks = 0; ks < KX; ks++) xf[ks] = *(const v8*)x_ptr(mi, 32 * ks + 8 * g);
 #pragma unroll
-      for (int v = 0; v < 4; v++) dxb[(wave * 16 * MT + 16 * mi + tcol) * LDD + 16 * y + 4 * g + v] += accA[mi][y][v];
-  __syncthreads();
-  for (int i = tid; i < ROWS * DK / 8; i += 256) {
-    const int rl = i / (DK / 8), col = (i % (DK / 8)) * 8;
-    if (row0 + rl < rows) {
-      float f[8];
+      for (int wt = 0; wt < TT; wt++) {
+        f32x4 t = {0, 0, 0, 0};
 #pragma unroll
-      for (int j = 0; j < 8; j++) f[j] = dxb[rl * LDD + col + j];
-      *(v8*)(dXg + row_off(row0 + rl) * DK + col) = pack8<T>(f);
+        for (int ks = 0; ks < KX; ks++) t = mfma16(lds_frag<T>(Mt, LDM, 16 * wt, 32 * ks), xf[ks], t);
+        acc[mi][wt] += t * (cv[mi] * OnePair<T>::up);
+      }
+    }
+  }
+
+#pragma unroll
+  for (int mi = 0; mi < MT; mi++) {
+    if (!live[mi]) continue;
+    const long ro = row_off(row0 + lrow[mi]);
+#pragma unroll
+    for (int k = 0; k < TT; k++) {
+      float o4[4];
+#pragma unroll
+      for (int v = 0; v < 4; v++) o4[v] = acc[mi][k][v];
+      *(v4*)(dXg + ro * DK + 16 * k + 4 * g) = pack4<T>(o4);
     }
   }
 }
 
 template <typename T, int DK, int DV, bool MULT> static int grad_launch(const GradArgs& a, int BN, hipStream_t st) {
-  constexpr int MT = 2, XS = DK <= 64 ? 2 : 1, TT = DK / 16;
-  constexpr size_t smem = 2 * TT * 16 * XS * (DV + 8) * sizeof(T) + 2 * TT * 16 * XS * sizeof(float) +
-                          64 * MT * (DK + 1) * sizeof(float);
-  const int rows = a.c * a.r;
-  dim3 grid((rows + 64 * MT - 1) / (64 * MT), (unsigned)(BN * a.h));
-  auto kern = sympow_grad_kernel<T, DK, DV, MT, XS, MULT>;
-  allow_big_lds((const void*)kern, smem);
-  hipLaunchKernelGGL(kern, grid, dim3(256), smem, st, a);
+  const int rows = a.c * a.r, npairs = BN * a.h;
+  auto go = [&](auto mt) {
+    constexpr int MT = decltype(mt)::value;
+    constexpr size_t ring = GR_NST * GR_FR * DV * 2, mtile = (size_t)DK * (DK + 8) * 2;
+    constexpr size_t smem = (ring > mtile ? ring : mtile) + 64 * MT * DK * 2;
+    const int row_blocks = (rows + 64 * MT - 1) / (64 * MT);
+    dim3 grid((unsigned)(((npairs + 7) / 8) * 8 * row_blocks));
+    auto kern = sympow_grad_kernel<T, DK, DV, MT, MULT>;
+    allow_big_lds((const void*)kern, smem);
+    hipLaunchKernelGGL(kern, grid, dim3(256), smem, st, a, row_blocks, npairs);
+  };
+  if (DK <= 64 && rows >= 256) go(IC<4>{});
+  else if (DK <= 64 && rows > 64) go(IC<2>{});
+  else go(IC<1>{});
   return (int)hipGetLastError();
 }
 

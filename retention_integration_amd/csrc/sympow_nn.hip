@@ -8,18 +8,23 @@
 //   * update_state backward, dV (m = 2 below the block diagonal): X = K, B = dS
 //                                                (ref: retention/_update_state/reference.py:61)
 //
-// A workgroup = 4 waves owns 64*MT rows; each wave 16*MT rows and all DV columns.  B is streamed
-// through LDS in its memory order, 32 features (two x columns of one 16-wide y strip) per step, and
-// read with the transposing LDS load; the phi operand is built in registers from the wave's own rows
-// (one scalar x[X] times eight x[16y+..] values per lane).  sB rides along as two extra bf16/fp16
-// columns (high and low part of the fp32 value) of the B tile.
+// A workgroup = 4 waves owns 64*MT rows; each wave 16*MT rows and all DV columns.  B streams through a
+// 3-deep ring of asynchronous global->LDS copies in its memory order, 64 features (four x columns of one
+// 16-wide y strip) per stage, and is read with the transposing LDS load; the phi operand is built in
+// registers from the wave's own rows (one scalar x[X] times eight x[16y+..] values per lane).
+// aux is a quadratic form, aux[row] = x_row^T M x_row with M[a, b] = sB[f(a, b)] on the stored pairs, so it
+// costs one small d x d product per row tile instead of an extra column in every step.
+// Row blocks that share a state are placed on the same XCD (one HBM fetch, L2 re-reads).
 #include "common.h"
 #include "kernels.h"
 
 namespace pr {
 
-constexpr int NN_KF = 32;
+constexpr int NN_FR = 64;   // feature rows per stage
+constexpr int NN_NST = 3;
 
+// Stage order over (strip y, first x column X0, a multiple of 4).  With the key-side multiplier the tiles
+// below the block diagonal come first so that the accumulators can be doubled once.
 template <bool MULT> struct FeatIter {
   int y, X0, phase, T;
   __device__ void init(int T_) {
@@ -28,9 +33,9 @@ template <bool MULT> struct FeatIter {
   }
   __device__ bool done() const { return y >= T; }
   __device__ int f0() const { return 128 * y * (y + 1) + 16 * X0; }
-  // returns true when the step just consumed was the last one below the diagonal
+  // returns true when the stage just consumed was the last one below the diagonal
   __device__ bool next() {
-    X0 += 2;
+    X0 += 4;
     if (phase == 0) {
       if (X0 == 16 * y) { y++; X0 = 0; }
       if (y == T) { phase = 1; y = 0; X0 = 0; return true; }
@@ -50,7 +55,7 @@ template <> struct ScaleS<f16_t> { static constexpr float down = 1.f / 256.f, up
 template <typename T> struct PhiRow;
 template <> struct PhiRow<bf16_t> {
   float row[8];
-  __device__ __forceinline__ void load(const bf16_t* p) { unpack8(*(const bf16x8*)p, row); }
+  __device__ __forceinline__ void load(const char* p) { unpack8(*(const bf16x8*)p, row); }
   __device__ __forceinline__ bf16x8 make(bf16_t x) const {
     const float xs = (float)x;
     float p[8];
@@ -61,135 +66,163 @@ template <> struct PhiRow<bf16_t> {
 };
 template <> struct PhiRow<f16_t> {
   f16x8 row;
-  __device__ __forceinline__ void load(const f16_t* p) { row = *(const f16x8*)p; }
+  __device__ __forceinline__ void load(const char* p) { row = *(const f16x8*)p; }
   __device__ __forceinline__ f16x8 make(f16_t x) const { return row * x; }
 };
 
 template <typename T, int DK, int DV, int MT, bool MULT, int EPI>
-__global__ __launch_bounds__(256) void sympow_nn_kernel(NNArgs a) {
+__global__ __launch_bounds__(256, 2) void sympow_nn_kernel(NNArgs a, int row_blocks, int npairs) {
   typedef typename VecOf<T>::v8 v8;
-  constexpr int LDX = DK + 8, LDB = DV + 16 + 8, NT = DV / 16, TT = DK / 16;
+  typedef typename VecOf<T>::v4 v4;
+  constexpr int NT = DV / 16, TT = DK / 16, KX = DK / 32, CB = DV / 8, CX = DK / 8;
   constexpr int D = 128 * TT * (TT + 1);
-  constexpr int ROWS = 64 * MT;
-  constexpr int B_CH = NN_KF * DV / 8, B_PT = (B_CH + 255) / 256;
-  constexpr int X_CH = ROWS * DK / 8, X_PT = (X_CH + 255) / 256;
-  extern __shared__ __attribute__((aligned(16))) char smem[];
-  T* xt = (T*)smem;                 // [ROWS][LDX]
-  T* bt = xt + ROWS * LDX;          // [2][KF][LDB]
+  constexpr int ROWS = 64 * MT, STAGE = NN_FR * DV * 2, LOADS = NN_FR * CB / 256, LDM = DK + 8;
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  char* ring = smem;                          // [NST][STAGE]; reused for M and the aux exchange at the end
+  char* xt = ring + NN_NST * STAGE;           // [ROWS][DK] T, swizzled
 
-  const int tid = threadIdx.x, l = tid & 63, g = l >> 4, wave = tid >> 6;
-  const int bn = blockIdx.y / a.h, hh = blockIdx.y % a.h;
+  const int xcd = blockIdx.x % 8, slot = blockIdx.x / 8;
+  const int pair = (slot / row_blocks) * 8 + xcd;
+  if (pair >= npairs) return;
+  const int row0 = (slot % row_blocks) * ROWS;
+  const int bn = pair / a.h, hh = pair % a.h;
+
+  const int tid = threadIdx.x, l = tid & 63, g = l >> 4, wave = tid >> 6, tcol = l & 15;
   const int hA = a.h * a.r, rows = a.c * a.r;
-  const int row0 = blockIdx.x * ROWS;
-  const T* X = (const T*)a.X + (long)bn * a.c * hA * DK;
-  const T* Bg = (const T*)a.B + ((long)bn * a.h + hh) * D * DV;
+  const T* Xg = (const T*)a.X + (long)bn * a.c * hA * DK;
+  const char* Bg = (const char*)((const T*)a.B + ((long)bn * a.h + hh) * D * DV);
   const float* sBg = a.sB ? a.sB + ((long)bn * a.h + hh) * D : nullptr;
-  auto row_off = [&](int row) -> long {  // element offset of a folded row, per unit of the last dim
+  auto row_off = [&](int row) -> long {  // element offset of a (clamped) folded row, per unit of the last dim
+    row = min(row, rows - 1);
     const int t = row / a.r, rr = row - t * a.r;
     return (long)t * hA + hh * a.r + rr;
   };
-
-  // stage the X rows and clear the B tiles (the unused aux columns must stay zero)
-#pragma unroll
-  for (int i = 0; i < X_PT; i++) {
-    const int ch = tid + 256 * i;
-    if (ch < X_CH) {
-      const int rl = ch / (DK / 8), col = (ch % (DK / 8)) * 8;
-      u32x4 v = {0, 0, 0, 0};
-      if (row0 + rl < rows) v = *(const u32x4*)(X + row_off(row0 + rl) * DK + col);
-      *(u32x4*)(xt + rl * LDX + col) = v;
-    }
-  }
-  for (int i = tid; i < 2 * NN_KF * LDB / 2; i += 256) ((uint32_t*)bt)[i] = 0;
+  auto x_ptr = [&](int lrow, int col) -> const char* {
+    return xt + lrow * (DK * 2) + (((col / 8) ^ swz<CX>(lrow)) * 16) + (col % 8) * 2;
+  };
+  auto issue = [&](int f0, int ringpos) {
+    const char* src = Bg + (long)f0 * DV * 2;
+    async_load_tile<CB, NN_FR>(ring + ringpos * STAGE, [&](int row) { return src + row * (DV * 2); });
+  };
 
   const bool skip = (EPI == NN_EPI_MERGE) && a.skip_first && (bn % a.n == 0);
-  f32x4 acc[MT][NT + 1];
+  f32x4 acc[MT][NT];
 #pragma unroll
   for (int i = 0; i < MT; i++)
 #pragma unroll
-    for (int j = 0; j <= NT; j++) acc[i][j] = (f32x4){0, 0, 0, 0};
-
-  if (!skip) {
-    u32x4 rb[B_PT];
-    float rs = 0.f;
-    auto fetch = [&](int f0) {
+    for (int j = 0; j < NT; j++) acc[i][j] = (f32x4){0, 0, 0, 0};
+  float aux[MT];   // aux of the row this lane holds as an accumulator COLUMN (row0 + wave*16*MT + 16*mi + tcol)
 #pragma unroll
-      for (int i = 0; i < B_PT; i++) {
-        const int ch = tid + 256 * i;
-        if (ch < B_CH) rb[i] = *(const u32x4*)(Bg + (long)(f0 + ch / (DV / 8)) * DV + (ch % (DV / 8)) * 8);
-      }
-      if (sBg && tid < NN_KF) rs = sBg[f0 + tid];
-    };
-    auto stash = [&](int stage) {
-      T* b = bt + stage * NN_KF * LDB;
-#pragma unroll
-      for (int i = 0; i < B_PT; i++) {
-        const int ch = tid + 256 * i;
-        if (ch < B_CH) *(u32x4*)(b + (ch / (DV / 8)) * LDB + (ch % (DV / 8)) * 8) = rb[i];
-      }
-      if (sBg && tid < NN_KF) {
-        const float v = rs * ScaleS<T>::down;
-        const T hi = (T)v;
-        b[tid * LDB + DV] = hi;
-        b[tid * LDB + DV + 1] = (T)(v - (float)hi);
-      }
-    };
+  for (int mi = 0; mi < MT; mi++) aux[mi] = 0.f;
 
+  async_load_tile<CX, ROWS>(xt, [&](int row) { return (const char*)(Xg + row_off(row0 + row) * DK); });
+  if (skip) {
+    wait_vmcnt<0>();
+    __syncthreads();
+  } else {
     FeatIter<MULT> cur, nxt;
     cur.init(TT);
     nxt.init(TT);
-    fetch(nxt.f0());
-    nxt.next();
-    PhiRow<T> prow[MT];
-    int y_loaded = -1, stage = 0;
-    __syncthreads();  // X rows staged, B tiles cleared
-    while (!cur.done()) {
-      stash(stage);
-      __syncthreads();
-      if (!nxt.done()) fetch(nxt.f0());
+    int issued = 0;
+    for (; issued < 2 && !nxt.done(); issued++) {
+      issue(nxt.f0(), issued % NN_NST);
       nxt.next();
-      const T* b = bt + stage * NN_KF * LDB;
+    }
+    PhiRow<T> prow[MT];
+    int y_loaded = -1, step = 0;
+    while (!cur.done()) {
+      const char* st = ring + (step % NN_NST) * STAGE;
+      if (issued > step + 1) wait_vmcnt<LOADS>(); else wait_vmcnt<0>();
+      __syncthreads();
+      if (!nxt.done()) {
+        issue(nxt.f0(), issued % NN_NST);
+        nxt.next();
+        issued++;
+      }
       if (cur.y != y_loaded) {
         y_loaded = cur.y;
 #pragma unroll
-        for (int mi = 0; mi < MT; mi++)
-          prow[mi].load(xt + (wave * 16 * MT + 16 * mi + (l & 15)) * LDX + 16 * cur.y + 8 * (g & 1));
+        for (int mi = 0; mi < MT; mi++) prow[mi].load(x_ptr(wave * 16 * MT + 16 * mi + tcol, 16 * cur.y + 8 * (g & 1)));
       }
-      v8 vf[NT + 1];
 #pragma unroll
-      for (int nt = 0; nt <= NT; nt++) vf[nt] = lds_frag_tr<T>(b, LDB, 0, 16 * nt);
+      for (int ks = 0; ks < NN_FR / 32; ks++) {
+        v8 vf[NT];
 #pragma unroll
-      for (int mi = 0; mi < MT; mi++) {
-        const T xs = xt[(wave * 16 * MT + 16 * mi + (l & 15)) * LDX + cur.X0 + (g >> 1)];
-        const v8 af = prow[mi].make(xs);
+        for (int nt = 0; nt < NT; nt++) vf[nt] = sw_frag_tr<T, CB>(st, 32 * ks, 16 * nt);
 #pragma unroll
-        for (int nt = 0; nt <= NT; nt++) acc[mi][nt] = mfma16(af, vf[nt], acc[mi][nt]);
+        for (int mi = 0; mi < MT; mi++) {
+          const T xs = *(const T*)x_ptr(wave * 16 * MT + 16 * mi + tcol, cur.X0 + 2 * ks + (g >> 1));
+          const v8 af = prow[mi].make(xs);
+#pragma unroll
+          for (int nt = 0; nt < NT; nt++) acc[mi][nt] = mfma16(af, vf[nt], acc[mi][nt]);
+        }
       }
       if (cur.next()) {
 #pragma unroll
         for (int mi = 0; mi < MT; mi++)
 #pragma unroll
-          for (int nt = 0; nt <= NT; nt++) acc[mi][nt] *= 2.f;
+          for (int nt = 0; nt < NT; nt++) acc[mi][nt] *= 2.f;
       }
-      stage ^= 1;
+      step++;
+    }
+
+    if (EPI == NN_EPI_MERGE) {
+      // aux[row] = sum_{a,b} x[a] M[a,b] x[b]: U^T[b, row] = sum_a M[a,b] x[row,a] on the matrix cores (M in a high
+      // and a low 16-bit part), then a dot with x[row, b] down the accumulator rows.
+      T* Mt = (T*)ring;   // [DK (b)][LDM (a)]
+      for (int part = 0; part < 2; part++) {
+        __syncthreads();
+        for (int idx = tid; idx < DK * DK; idx += 256) {
+          const int b_ = idx / DK, aa = idx % DK, yb = b_ / 16;
+          float val = 0.f;
+          if (aa < 16 * (yb + 1)) val = sBg[128 * yb * (yb + 1) + 16 * aa + (b_ - 16 * yb)] * ScaleS<T>::down;
+          const T hi16 = (T)val;
+          Mt[b_ * LDM + aa] = part == 0 ? hi16 : (T)(val - (float)hi16);
+        }
+        __syncthreads();
+#pragma unroll
+        for (int mi = 0; mi < MT; mi++) {
+          const int lrow = wave * 16 * MT + 16 * mi + tcol;
+          v8 xf[KX];
+#pragma unroll
+          for (int ks = 0; ks < KX; ks++) xf[ks] = *(const v8*)x_ptr(lrow, 32 * ks + 8 * g);
+#pragma unroll
+          for (int wt = 0; wt < TT; wt++) {
+            f32x4 t = {0, 0, 0, 0};
+#pragma unroll
+            for (int ks = 0; ks < KX; ks++) t = mfma16(lds_frag<T>(Mt, LDM, 16 * wt, 32 * ks), xf[ks], t);
+            const v4 xb4 = *(const v4*)x_ptr(lrow, 16 * wt + 4 * g);
+#pragma unroll
+            for (int v = 0; v < 4; v++) aux[mi] += t[v] * (float)xb4[v];
+          }
+        }
+      }
     }
   }
 
   // epilogue: accumulator element v of lane l is row 4*(l/16)+v, column 16*nt + l%16
   T* out = (T*)a.out + (long)bn * a.c * hA * DV;
-  const float log_gamma = 0.5f * __logf((float)D);
+  if (EPI == NN_EPI_MERGE) {
+    // hand aux from the lane that holds the row as a column to the lanes that hold it as accumulator rows
+    float* ax = (float*)ring;
+    __syncthreads();
 #pragma unroll
-  for (int mi = 0; mi < MT; mi++) {
+    for (int mi = 0; mi < MT; mi++) {
+      const float tot = sum_over_rows(aux[mi]) * ScaleS<T>::up;
+      if (g == 0) ax[wave * 16 * MT + 16 * mi + tcol] = tot;
+    }
+    __syncthreads();
+    constexpr float log_gamma_2 = 0.f;
+    (void)log_gamma_2;
+    const float log_gamma = 0.5f * __logf((float)D);
 #pragma unroll
-    for (int v = 0; v < 4; v++) {
-      const int row = row0 + wave * 16 * MT + 16 * mi + 4 * g + v;
-      if (row >= rows) continue;
-      const long ro = row_off(row);
-      if (EPI == NN_EPI_PLAIN) {
+    for (int mi = 0; mi < MT; mi++) {
 #pragma unroll
-        for (int nt = 0; nt < NT; nt++) out[ro * DV + 16 * nt + (l & 15)] = (T)acc[mi][nt][v];
-      } else {
-        const float lqs = (row_bcast<0>(acc[mi][NT][v]) + row_bcast<1>(acc[mi][NT][v])) * ScaleS<T>::up;
+      for (int v = 0; v < 4; v++) {
+        const int lrow = wave * 16 * MT + 16 * mi + 4 * g + v, row = row0 + lrow;
+        if (row >= rows) continue;
+        const long ro = row_off(row);
+        const float lqs = ax[lrow];
         float wa = 0.f, wq = 1.f, la = 0.f;
         const T* ya = nullptr;
         if (a.Y_attn) {
@@ -205,27 +238,42 @@ __global__ __launch_bounds__(256) void sympow_nn_kernel(NNArgs a) {
         const float inv = 1.f / den;
 #pragma unroll
         for (int nt = 0; nt < NT; nt++) {
-          const int e = 16 * nt + (l & 15);
+          const int e = 16 * nt + tcol;
           float num = acc[mi][nt][v] * wq;
           if (ya) num += (float)ya[e] * wa;
           out[ro * DV + e] = (T)(num * inv);
         }
-        if ((l & 15) == 0) a.den[(long)bn * a.c * hA + ro] = den;
+        if (tcol == 0) a.den[(long)bn * a.c * hA + ro] = den;
       }
     }
+  } else {
+#pragma unroll
+    for (int mi = 0; mi < MT; mi++)
+#pragma unroll
+      for (int v = 0; v < 4; v++) {
+        const int row = row0 + wave * 16 * MT + 16 * mi + 4 * g + v;
+        if (row >= rows) continue;
+        const long ro = row_off(row);
+#pragma unroll
+        for (int nt = 0; nt < NT; nt++) out[ro * DV + 16 * nt + tcol] = (T)acc[mi][nt][v];
+      }
   }
 }
 
 template <typename T, int DK, int DV, bool MULT, int EPI> static int nn_launch(const NNArgs& a, int BN, hipStream_t st) {
-  const int rows = a.c * a.r;
+  const int rows = a.c * a.r, npairs = BN * a.h;
   auto go = [&](auto mt) {
     constexpr int MT = decltype(mt)::value;
-    constexpr size_t smem = (64 * MT * (DK + 8) + 2 * NN_KF * (DV + 24)) * sizeof(T);
-    dim3 grid((rows + 64 * MT - 1) / (64 * MT), (unsigned)(BN * a.h));
-    hipLaunchKernelGGL((sympow_nn_kernel<T, DK, DV, MT, MULT, EPI>), grid, dim3(256), smem, st, a);
+    constexpr size_t ring = NN_NST * NN_FR * DV * 2, mtile = (size_t)DK * (DK + 8) * 2;
+    constexpr size_t smem = (ring > mtile ? ring : mtile) + 64 * MT * DK * 2;
+    const int row_blocks = (rows + 64 * MT - 1) / (64 * MT);
+    dim3 grid((unsigned)(((npairs + 7) / 8) * 8 * row_blocks));
+    auto kern = sympow_nn_kernel<T, DK, DV, MT, MULT, EPI>;
+    allow_big_lds((const void*)kern, smem);
+    hipLaunchKernelGGL(kern, grid, dim3(256), smem, st, a, row_blocks, npairs);
   };
   if (DK <= 64 && rows >= 256) go(IC<4>{});
-  else if (rows >= 128) go(IC<2>{});
+  else if (rows > 64) go(IC<2>{});
   else go(IC<1>{});
   return (int)hipGetLastError();
 }

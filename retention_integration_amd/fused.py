@@ -90,8 +90,8 @@ class _ChunkedPowerRetention(torch.autograd.Function):
         dQa, dKa, dVa = torch.empty_like(Q), torch.empty_like(K), torch.empty_like(V)
         dGq = _empty((BN, c, hq), f32, dev) if gated else None
         dGk = _empty((BN, c, h), f32, dev) if gated else None
-        _lib.check(lib.pr_attention_bwd(p(Q), p(K), p(V), p(A), p(rm), p(dYa), p(dla), p(dQa), p(dKa), p(dVa), p(dGq),
-                                        p(dGk), BN, c, c, h, r, d, scale, deg, code, st), "attention_bwd")
+        _lib.check(lib.pr_attention_bwd(p(Q), p(K), p(V), p(A), p(rm), p(dYa), p(dla), None, p(dQa), p(dKa), p(dVa),
+                                        p(dGq), p(dGk), BN, c, c, h, r, d, scale, deg, code, st), "attention_bwd")
         if gated:
             dGa = dGk.add_(dGq.view(BN, c, h, r).sum(-1)) if r > 1 else dGk.add_(dGq)
         else:

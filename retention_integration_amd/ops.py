@@ -61,7 +61,8 @@ def _(Q, K, V, G, deg, scale, norm):
 
 @torch.library.custom_op("pr::attention_bwd", mutates_args=(), device_types="cuda")
 def attention_bwd(Q: Tensor, K: Tensor, V: Tensor, G: Optional[Tensor], rowmax: Tensor, dO: Tensor,
-                  dl: Optional[Tensor], deg: int, scale: float) -> Tuple[Tensor, Tensor, Tensor, Tensor]:
+                  dl: Optional[Tensor], dO_scale: Optional[Tensor], deg: int,
+                  scale: float) -> Tuple[Tensor, Tensor, Tensor, Tensor]:
     b, tq, hq, d = Q.shape
     _, tk, h, _ = K.shape
     r = hq // h
@@ -72,7 +73,8 @@ def attention_bwd(Q: Tensor, K: Tensor, V: Tensor, G: Optional[Tensor], rowmax: 
         dGk = torch.empty((b, tk, h), dtype=torch.float32, device=Q.device)
     lib = _lib.load()
     _lib.check(lib.pr_attention_bwd(_lib.ptr(Q), _lib.ptr(K), _lib.ptr(V), _lib.ptr(G), _lib.ptr(rowmax),
-                                    _lib.ptr(dO), _lib.ptr(dl), _lib.ptr(dQ), _lib.ptr(dK), _lib.ptr(dV),
+                                    _lib.ptr(dO), _lib.ptr(dl), _lib.ptr(dO_scale), _lib.ptr(dQ), _lib.ptr(dK),
+                                    _lib.ptr(dV),
                                     _lib.ptr(dGq), _lib.ptr(dGk), b, tq, tk, h, r, d, float(scale), int(deg),
                                     _lib.dtype_code(Q.dtype), _lib.stream()), "attention_bwd")
     if G is None:
@@ -84,7 +86,7 @@ def attention_bwd(Q: Tensor, K: Tensor, V: Tensor, G: Optional[Tensor], rowmax: 
 
 
 @attention_bwd.register_fake
-def _(Q, K, V, G, rowmax, dO, dl, deg, scale):
+def _(Q, K, V, G, rowmax, dO, dl, dO_scale, deg, scale):
     dG = Q.new_empty((0,), dtype=torch.float32) if G is None else torch.empty_like(G)
     return torch.empty_like(Q), torch.empty_like(K), torch.empty_like(V), dG
 
@@ -98,12 +100,12 @@ def _attention_setup(ctx, inputs, output):
 
 def _attention_backward(ctx, dO, dl, drowmax):
     Q, K, V, G, O, l, rowmax = ctx.saved_tensors
-    if ctx.norm:  # O = o / l: chain back to the unnormalised pair (o, l)
-        dlu = -(dO.float() * O.float()).sum(-1) / l
-        dOu = (dO.float() / l.unsqueeze(-1)).to(dO.dtype)
+    if ctx.norm:  # O = o / l: chain back to the unnormalised pair (o, l); the 1/l on dO is applied in the kernel
+        osc = 1.0 / l
+        dlu = -(dO.float() * O.float()).sum(-1) * osc
     else:
-        dOu, dlu = dO, dl
-    dQ, dK, dV, dG = attention_bwd(Q, K, V, G, rowmax, dOu.contiguous(), _cont(dlu), ctx.deg, ctx.scale)
+        dlu, osc = dl, None
+    dQ, dK, dV, dG = attention_bwd(Q, K, V, G, rowmax, dO.contiguous(), _cont(dlu), _cont(osc), ctx.deg, ctx.scale)
     return dQ, dK, dV, (dG if G is not None else None), None, None, None
 
 
