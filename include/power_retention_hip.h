@@ -119,15 +119,18 @@ int pr_chunk_prep_fwd(const float* log_G, const void* K, const void* Q, float* A
                       int c, int h, int r, int d, int deg, int dtype, void* stream);
 
 /* Backward of the same glue plus the final gradient sums (autograd of retention/power_retention_maker.py:143-193).
- *   A as above or NULL for the ungated path (then dG_attn, dlcs_*, dlog_G are ignored);
+ *   A, lcs as above, or A = NULL for the ungated path (then lcs, dG_attn, dlcs_*, dlog_G, workspace are ignored);
  *   dKd, dQg: gradients w.r.t. Kd, Qg; dK_attn, dQ_attn, dV_attn: from the attention backward; dV_state: from the
  *   update_state backward; dG_attn [BN,c,h]: gradient w.r.t. A from the attention backward; dlcs_a, dlcs_b [BN,h]:
  *   gradients w.r.t. lcs from the two scans
- *   -> dK, dQ, dV (may alias dK_attn, dQ_attn, dV_attn), dlog_G [BN,c,h]. */
-int pr_chunk_glue_bwd(const float* A, const void* Kd, const void* dKd, const void* Qg, const void* dQg,
-                      const void* dK_attn, const void* dQ_attn, const void* dV_attn, const void* dV_state,
-                      const float* dG_attn, const float* dlcs_a, const float* dlcs_b, void* dK, void* dQ, void* dV,
-                      float* dlog_G, int BN, int c, int h, int r, int d, int deg, int dtype, void* stream);
+ *   -> dK, dQ, dV (may alias dK_attn, dQ_attn, dV_attn), dlog_G [BN,c,h].
+ *   workspace: pr_chunk_glue_bwd_workspace() bytes. */
+size_t pr_chunk_glue_bwd_workspace(int BN, int c, int h);
+int pr_chunk_glue_bwd(const float* A, const float* lcs, const void* Kd, const void* dKd, const void* Qg,
+                      const void* dQg, const void* dK_attn, const void* dQ_attn, const void* dV_attn,
+                      const void* dV_state, const float* dG_attn, const float* dlcs_a, const float* dlcs_b, void* dK,
+                      void* dQ, void* dV, float* dlog_G, void* workspace, int BN, int c, int h, int r, int d, int deg,
+                      int dtype, void* stream);
 
 #ifdef __cplusplus
 }

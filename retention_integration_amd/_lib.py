@@ -35,7 +35,8 @@ SIGNATURES = {
     "pr_query_state_bwd_workspace": (c_size_t, [_I] * 6),
     "pr_query_state_bwd": (c_int, [_P] * 13 + [_I] * 6 + [_F, _I, _I, _I, _P]),
     "pr_chunk_prep_fwd": (c_int, [_P] * 7 + [_I] * 7 + [_P]),
-    "pr_chunk_glue_bwd": (c_int, [_P] * 16 + [_I] * 7 + [_P]),
+    "pr_chunk_glue_bwd_workspace": (c_size_t, [_I] * 3),
+    "pr_chunk_glue_bwd": (c_int, [_P] * 18 + [_I] * 7 + [_P]),
 }
 
 _lib = None

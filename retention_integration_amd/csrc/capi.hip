@@ -177,19 +177,25 @@ int pr_chunk_prep_fwd(const float* log_G, const void* K, const void* Q, float* A
                 "chunk_prep_fwd");
 }
 
-int pr_chunk_glue_bwd(const float* A, const void* Kd, const void* dKd, const void* Qg, const void* dQg,
-                      const void* dK_attn, const void* dQ_attn, const void* dV_attn, const void* dV_state,
-                      const float* dG_attn, const float* dlcs_a, const float* dlcs_b, void* dK, void* dQ, void* dV,
-                      float* dlog_G, int BN, int c, int h, int r, int d, int deg, int dtype, void* stream) {
+size_t pr_chunk_glue_bwd_workspace(int BN, int c, int h) {
+  return (size_t)pr::chunk_glue_bwd_workspace_floats(BN, c, h) * sizeof(float);
+}
+
+int pr_chunk_glue_bwd(const float* A, const float* lcs, const void* Kd, const void* dKd, const void* Qg,
+                      const void* dQg, const void* dK_attn, const void* dQ_attn, const void* dV_attn,
+                      const void* dV_state, const float* dG_attn, const float* dlcs_a, const float* dlcs_b, void* dK,
+                      void* dQ, void* dV, float* dlog_G, void* workspace, int BN, int c, int h, int r, int d, int deg,
+                      int dtype, void* stream) {
   if (int rc = check_common("chunk_glue_bwd", d, deg, dtype, false)) return rc;
   if (bad_ptr(Kd) || bad_ptr(dKd) || bad_ptr(Qg) || bad_ptr(dQg) || bad_ptr(dK_attn) || bad_ptr(dQ_attn) ||
       bad_ptr(dV_attn) || bad_ptr(dV_state) || bad_ptr(dK) || bad_ptr(dQ) || bad_ptr(dV))
     return fail(PR_ERR_ARG, "chunk_glue_bwd: null or misaligned pointer");
-  if (A && (!dG_attn || !dlcs_a || !dlcs_b || !dlog_G))
-    return fail(PR_ERR_ARG, "chunk_glue_bwd: gated call needs dG_attn, dlcs_a, dlcs_b and dlog_G");
+  if (A && (!lcs || !dG_attn || !dlcs_a || !dlcs_b || !dlog_G || !workspace))
+    return fail(PR_ERR_ARG, "chunk_glue_bwd: gated call needs lcs, dG_attn, dlcs_a, dlcs_b, dlog_G and workspace");
   if (BN <= 0 || c <= 0 || h <= 0 || r <= 0) return fail(PR_ERR_ARG, "chunk_glue_bwd: need BN,c,h,r > 0");
-  return finish(pr::chunk_glue_bwd(A, Kd, dKd, Qg, dQg, dK_attn, dQ_attn, dV_attn, dV_state, dG_attn, dlcs_a, dlcs_b,
-                                   dK, dQ, dV, dlog_G, BN, c, h, r, d, deg, dtype, (hipStream_t)stream),
+  return finish(pr::chunk_glue_bwd(A, lcs, Kd, dKd, Qg, dQg, dK_attn, dQ_attn, dV_attn, dV_state, dG_attn, dlcs_a,
+                                   dlcs_b, dK, dQ, dV, dlog_G, (float*)workspace, BN, c, h, r, d, deg, dtype,
+                                   (hipStream_t)stream),
                 "chunk_glue_bwd");
 }
 

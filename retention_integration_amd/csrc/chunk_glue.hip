@@ -1,4 +1,4 @@
-// Per-chunk gate arithmetic of the chunked algorithm, fused into two HBM-bound kernels
+// Per-chunk gate arithmetic of the chunked algorithm, as HBM-bound kernels
 // (ref: retention/power_retention_maker.py:143-186 and its autograd):
 //
 // forward  : A = cumsum_c(log_G),  lcs = A[c-1],  Kd = K * exp((A[c-1] - A)/deg),  Qg = Q * exp(A/deg)
@@ -6,7 +6,8 @@
 //            dA_t = dG_attn_t + (sum_d dQg.Qg - sum_d dKd.Kd)_t / deg,
 //            dA_{c-1} += (sum_{t,d} dKd.Kd)/deg + dlcs,   dlog_G = reverse-cumsum_c(dA)
 //
-// One workgroup per (chunk, kv head); the chunk's gate vector lives in LDS.
+// The scans over the chunk (one workgroup per (chunk, head), gate vector in LDS) are separate tiny kernels;
+// the row-wise parts are fully parallel over (chunk, position, head) with 16 bytes per lane.
 #include "common.h"
 #include "kernels.h"
 
@@ -38,50 +39,53 @@ __device__ inline void block_scan(float* a, float* tot, int c, bool reverse) {
   __syncthreads();
 }
 
-template <typename T, int DH>
-__global__ __launch_bounds__(256) void chunk_prep_fwd_kernel(const float* __restrict__ logG, const T* __restrict__ K,
-                                                             const T* __restrict__ Q, float* __restrict__ A,
-                                                             float* __restrict__ lcs, T* __restrict__ Kd,
-                                                             T* __restrict__ Qg, int c, int h, int r, float inv_deg) {
-  typedef typename VecOf<T>::v8 v8;
+// A[bn, :, hh] = cumsum(log_G[bn, :, hh]);  lcs[bn, hh] = A[bn, c-1, hh]
+__global__ __launch_bounds__(256) void gate_scan_fwd_kernel(const float* __restrict__ logG, float* __restrict__ A,
+                                                            float* __restrict__ lcs, int c, int h) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
-  float* a = (float*)smem;     // [c]
-  float* tot = a + c;          // [256]
-  const int tid = threadIdx.x, bn = blockIdx.x / h, hh = blockIdx.x % h, hq = h * r;
-  const float* lg = logG + (long)bn * c * h + hh;
-  for (int i = tid; i < c; i += 256) a[i] = lg[(long)i * h];
+  float* a = (float*)smem;
+  float* tot = a + c;
+  const int tid = threadIdx.x, bn = blockIdx.x / h, hh = blockIdx.x % h;
+  const long base = (long)bn * c * h + hh;
+  for (int i = tid; i < c; i += 256) a[i] = logG[base + (long)i * h];
   __syncthreads();
   block_scan(a, tot, c, false);
-  float* Ao = A + (long)bn * c * h + hh;
-  for (int i = tid; i < c; i += 256) Ao[(long)i * h] = a[i];
-  const float a_last = a[c - 1];
-  if (tid == 0) lcs[(long)bn * h + hh] = a_last;
+  for (int i = tid; i < c; i += 256) A[base + (long)i * h] = a[i];
+  if (tid == 0) lcs[(long)bn * h + hh] = a[c - 1];
+}
 
-  constexpr int LPR = DH / 8;          // threads per row
-  const int sub = tid % LPR, col = sub * 8;
-  for (int t = tid / LPR; t < c; t += 256 / LPR) {
-    const float w = __expf((a_last - a[t]) * inv_deg), u = __expf(a[t] * inv_deg);
-    {
-      const long o = (((long)bn * c + t) * h + hh) * DH + col;
-      float f[8];
-      unpack8(*(const v8*)(K + o), f);
+// one group of DH/8 lanes per (chunk, position, kv head)
+template <typename T, int DH>
+__global__ __launch_bounds__(256) void gate_apply_fwd_kernel(const float* __restrict__ A, const float* __restrict__ lcs,
+                                                             const T* __restrict__ K, const T* __restrict__ Q,
+                                                             T* __restrict__ Kd, T* __restrict__ Qg, long groups,
+                                                             int c, int h, int r, float inv_deg) {
+  typedef typename VecOf<T>::v8 v8;
+  constexpr int LPR = DH / 8;
+  const long gid = ((long)blockIdx.x * 256 + threadIdx.x) / LPR;
+  if (gid >= groups) return;
+  const int col = (threadIdx.x % LPR) * 8;
+  const int hh = (int)(gid % h);
+  const long bn = gid / ((long)c * h);
+  const float at = A[gid], al = lcs[bn * h + hh];
+  const float w = __expf((al - at) * inv_deg), u = __expf(at * inv_deg);
+  float f[8];
+  unpack8(*(const v8*)(K + gid * DH + col), f);
 #pragma unroll
-      for (int i = 0; i < 8; i++) f[i] *= w;
-      *(v8*)(Kd + o) = pack8<T>(f);
-    }
-    for (int rr = 0; rr < r; rr++) {
-      const long o = (((long)bn * c + t) * hq + hh * r + rr) * DH + col;
-      float f[8];
-      unpack8(*(const v8*)(Q + o), f);
+  for (int i = 0; i < 8; i++) f[i] *= w;
+  *(v8*)(Kd + gid * DH + col) = pack8<T>(f);
+  for (int rr = 0; rr < r; rr++) {
+    const long o = (gid * r + rr) * DH + col;
+    unpack8(*(const v8*)(Q + o), f);
 #pragma unroll
-      for (int i = 0; i < 8; i++) f[i] *= u;
-      *(v8*)(Qg + o) = pack8<T>(f);
-    }
+    for (int i = 0; i < 8; i++) f[i] *= u;
+    *(v8*)(Qg + o) = pack8<T>(f);
   }
 }
 
 struct GlueBwdArgs {
   const float* A;       // [BN, c, h] or null (ungated)
+  const float* lcs;     // [BN, h]
   const void* Kd;       // [BN, c, h, d]
   const void* dKd;      // [BN, c, h, d]
   const void* Qg;       // [BN, c, hq, d]
@@ -91,100 +95,115 @@ struct GlueBwdArgs {
   const void* dV_attn;  // [BN, c, h, d]
   const void* dV_state; // [BN, c, h, d]
   const float* dG_attn; // [BN, c, h]
-  const float* dlcs_a;  // [BN, h]
-  const float* dlcs_b;  // [BN, h]
   void* dK;
   void* dQ;
   void* dV;
-  float* dlogG;         // [BN, c, h]
+  float* dA;            // [BN, c, h]  (the dlog_G buffer; scanned in place afterwards)
+  float* dotk;          // [BN, c, h]  workspace: sum_d dKd.Kd per row
+  long groups;
   int c, h, r;
   float inv_deg;
 };
 
-template <typename T, int DH> __global__ __launch_bounds__(256) void chunk_glue_bwd_kernel(GlueBwdArgs g) {
+template <typename T, int DH> __global__ __launch_bounds__(256) void glue_rows_bwd_kernel(GlueBwdArgs g) {
   typedef typename VecOf<T>::v8 v8;
-  extern __shared__ __attribute__((aligned(16))) char smem[];
-  float* da = (float*)smem;       // [c]
-  float* tot = da + g.c;          // [256]
-  const int tid = threadIdx.x, c = g.c, h = g.h, r = g.r, hq = h * r;
-  const int bn = blockIdx.x / h, hh = blockIdx.x % h;
-  const bool gated = g.A != nullptr;
-  const float* Ai = gated ? g.A + (long)bn * c * h + hh : nullptr;
-  const float a_last = gated ? Ai[(long)(c - 1) * h] : 0.f;
-
   constexpr int LPR = DH / 8;
-  const int sub = tid % LPR, col = sub * 8;
-  float ksum = 0.f;   // this thread's share of sum_{t,d} dKd.Kd
-  for (int t = tid / LPR; t < c; t += 256 / LPR) {
-    const float at = gated ? Ai[(long)t * h] : 0.f;
-    const float w = gated ? __expf((a_last - at) * g.inv_deg) : 1.f, u = gated ? __expf(at * g.inv_deg) : 1.f;
-    float dotk = 0.f, dotq = 0.f;
-    {
-      const long o = (((long)bn * c + t) * h + hh) * DH + col;
-      float kd[8], dkd[8], dka[8], dva[8], dvs[8], ok[8], ov[8];
-      unpack8(*(const v8*)((const T*)g.Kd + o), kd);
-      unpack8(*(const v8*)((const T*)g.dKd + o), dkd);
-      unpack8(*(const v8*)((const T*)g.dK_attn + o), dka);
-      unpack8(*(const v8*)((const T*)g.dV_attn + o), dva);
-      unpack8(*(const v8*)((const T*)g.dV_state + o), dvs);
+  const long gid = ((long)blockIdx.x * 256 + threadIdx.x) / LPR;
+  const bool live = gid < g.groups;
+  const long gi = live ? gid : 0;
+  const int sub = threadIdx.x % LPR, col = sub * 8;
+  const int hh = (int)(gi % g.h);
+  const long bn = gi / ((long)g.c * g.h);
+  const bool gated = g.A != nullptr;
+  float w = 1.f, u = 1.f;
+  if (gated) {
+    const float at = g.A[gi], al = g.lcs[bn * g.h + hh];
+    w = __expf((al - at) * g.inv_deg);
+    u = __expf(at * g.inv_deg);
+  }
+  float dotk = 0.f, dotq = 0.f;
+  {
+    const long o = gi * DH + col;
+    float kd[8], dkd[8], dka[8], dva[8], dvs[8], ok[8], ov[8];
+    unpack8(*(const v8*)((const T*)g.Kd + o), kd);
+    unpack8(*(const v8*)((const T*)g.dKd + o), dkd);
+    unpack8(*(const v8*)((const T*)g.dK_attn + o), dka);
+    unpack8(*(const v8*)((const T*)g.dV_attn + o), dva);
+    unpack8(*(const v8*)((const T*)g.dV_state + o), dvs);
 #pragma unroll
-      for (int i = 0; i < 8; i++) {
-        dotk += kd[i] * dkd[i];
-        ok[i] = dka[i] + dkd[i] * w;
-        ov[i] = dva[i] + dvs[i];
-      }
+    for (int i = 0; i < 8; i++) {
+      dotk += kd[i] * dkd[i];
+      ok[i] = dka[i] + dkd[i] * w;
+      ov[i] = dva[i] + dvs[i];
+    }
+    if (live) {
       *(v8*)((T*)g.dK + o) = pack8<T>(ok);
       *(v8*)((T*)g.dV + o) = pack8<T>(ov);
     }
-    for (int rr = 0; rr < r; rr++) {
-      const long o = (((long)bn * c + t) * hq + hh * r + rr) * DH + col;
-      float qg[8], dqg[8], dqa[8], oq[8];
-      unpack8(*(const v8*)((const T*)g.Qg + o), qg);
-      unpack8(*(const v8*)((const T*)g.dQg + o), dqg);
-      unpack8(*(const v8*)((const T*)g.dQ_attn + o), dqa);
+  }
+  for (int rr = 0; rr < g.r; rr++) {
+    const long o = (gi * g.r + rr) * DH + col;
+    float qg[8], dqg[8], dqa[8], oq[8];
+    unpack8(*(const v8*)((const T*)g.Qg + o), qg);
+    unpack8(*(const v8*)((const T*)g.dQg + o), dqg);
+    unpack8(*(const v8*)((const T*)g.dQ_attn + o), dqa);
 #pragma unroll
-      for (int i = 0; i < 8; i++) {
-        dotq += qg[i] * dqg[i];
-        oq[i] = dqa[i] + dqg[i] * u;
-      }
-      *(v8*)((T*)g.dQ + o) = pack8<T>(oq);
+    for (int i = 0; i < 8; i++) {
+      dotq += qg[i] * dqg[i];
+      oq[i] = dqa[i] + dqg[i] * u;
     }
-    if (gated) {
+    if (live) *(v8*)((T*)g.dQ + o) = pack8<T>(oq);
+  }
+  if (gated) {
 #pragma unroll
-      for (int m = 1; m < LPR; m <<= 1) {
-        dotk += __shfl_xor(dotk, m);
-        dotq += __shfl_xor(dotq, m);
-      }
-      if (sub == 0) {
-        da[t] = g.dG_attn[((long)bn * c + t) * h + hh] + (dotq - dotk) * g.inv_deg;
-        ksum += dotk;
-      }
+    for (int m = 1; m < LPR; m <<= 1) {
+      dotk += __shfl_xor(dotk, m);
+      dotq += __shfl_xor(dotq, m);
+    }
+    if (live && sub == 0) {
+      g.dA[gi] = g.dG_attn[gi] + (dotq - dotk) * g.inv_deg;
+      g.dotk[gi] = dotk;
     }
   }
-  if (!gated) return;
-  // total of dKd.Kd over the chunk
-  tot[tid] = ksum;
+}
+
+// dA[c-1] += (sum_t dotk)/deg + dlcs_a + dlcs_b, then dlog_G = reverse cumsum of dA (in place)
+__global__ __launch_bounds__(256) void gate_scan_bwd_kernel(float* __restrict__ dA, const float* __restrict__ dotk,
+                                                            const float* __restrict__ dlcs_a,
+                                                            const float* __restrict__ dlcs_b, int c, int h,
+                                                            float inv_deg) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  float* a = (float*)smem;
+  float* tot = a + c;
+  const int tid = threadIdx.x, bn = blockIdx.x / h, hh = blockIdx.x % h;
+  const long base = (long)bn * c * h + hh;
+  float ks = 0.f;
+  for (int i = tid; i < c; i += 256) {
+    a[i] = dA[base + (long)i * h];
+    ks += dotk[base + (long)i * h];
+  }
+  tot[tid] = ks;
   __syncthreads();
   for (int off = 128; off > 0; off >>= 1) {
     if (tid < off) tot[tid] += tot[tid + off];
     __syncthreads();
   }
-  if (tid == 0) da[c - 1] += tot[0] * g.inv_deg + g.dlcs_a[(long)bn * h + hh] + g.dlcs_b[(long)bn * h + hh];
+  if (tid == 0) a[c - 1] += tot[0] * inv_deg + dlcs_a[(long)bn * h + hh] + dlcs_b[(long)bn * h + hh];
   __syncthreads();
-  block_scan(da, tot, c, true);
-  float* out = g.dlogG + (long)bn * c * h + hh;
-  for (int i = tid; i < c; i += 256) out[(long)i * h] = da[i];
+  block_scan(a, tot, c, true);
+  for (int i = tid; i < c; i += 256) dA[base + (long)i * h] = a[i];
 }
 
 template <typename T>
 static int prep_launch(const float* logG, const void* K, const void* Q, float* A, float* lcs, void* Kd, void* Qg, int BN,
                        int c, int h, int r, int d, int deg, hipStream_t st) {
   const size_t smem = (size_t)(c + 256) * sizeof(float);
-  dim3 grid((unsigned)(BN * h));
+  hipLaunchKernelGGL(gate_scan_fwd_kernel, dim3((unsigned)(BN * h)), dim3(256), smem, st, logG, A, lcs, c, h);
+  const long groups = (long)BN * c * h;
 #define PR_CP(DD)                                                                                                      \
   case DD:                                                                                                             \
-    hipLaunchKernelGGL((chunk_prep_fwd_kernel<T, DD>), grid, dim3(256), smem, st, logG, (const T*)K, (const T*)Q, A,   \
-                       lcs, (T*)Kd, (T*)Qg, c, h, r, 1.f / deg);                                                       \
+    hipLaunchKernelGGL((gate_apply_fwd_kernel<T, DD>), dim3((unsigned)((groups * (DD / 8) + 255) / 256)), dim3(256), 0, \
+                       st, A, lcs, (const T*)K, (const T*)Q, (T*)Kd, (T*)Qg, groups, c, h, r, 1.f / deg);              \
     break;
   switch (d) { PR_CP(32) PR_CP(64) PR_CP(128) default: return -2; }
 #undef PR_CP
@@ -199,25 +218,35 @@ int chunk_prep_fwd(const float* logG, const void* K, const void* Q, float* A, fl
   return -1;
 }
 
-int chunk_glue_bwd(const float* A, const void* Kd, const void* dKd, const void* Qg, const void* dQg,
+long chunk_glue_bwd_workspace_floats(int BN, int c, int h) { return (long)BN * c * h; }
+
+int chunk_glue_bwd(const float* A, const float* lcs, const void* Kd, const void* dKd, const void* Qg, const void* dQg,
                    const void* dK_attn, const void* dQ_attn, const void* dV_attn, const void* dV_state,
                    const float* dG_attn, const float* dlcs_a, const float* dlcs_b, void* dK, void* dQ, void* dV,
-                   float* dlogG, int BN, int c, int h, int r, int d, int deg, int dtype, hipStream_t st) {
+                   float* dlogG, float* workspace, int BN, int c, int h, int r, int d, int deg, int dtype,
+                   hipStream_t st) {
   if (c > GLUE_MAX_C) return -5;
-  GlueBwdArgs g{A, Kd, dKd, Qg, dQg, dK_attn, dQ_attn, dV_attn, dV_state, dG_attn, dlcs_a, dlcs_b,
-                dK, dQ, dV, dlogG, c, h, r, 1.f / deg};
-  const size_t smem = (size_t)(c + 256) * sizeof(float);
-  dim3 grid((unsigned)(BN * h));
+  const long groups = (long)BN * c * h;
+  GlueBwdArgs g{A, lcs, Kd, dKd, Qg, dQg, dK_attn, dQ_attn, dV_attn, dV_state, dG_attn,
+                dK, dQ, dV, dlogG, workspace, groups, c, h, r, 1.f / deg};
 #define PR_GB(T, DD)                                                                                                   \
-  case DD: hipLaunchKernelGGL((chunk_glue_bwd_kernel<T, DD>), grid, dim3(256), smem, st, g); break;
+  case DD:                                                                                                             \
+    hipLaunchKernelGGL((glue_rows_bwd_kernel<T, DD>), dim3((unsigned)((groups * (DD / 8) + 255) / 256)), dim3(256), 0,  \
+                       st, g);                                                                                         \
+    break;
 #define PR_GBT(T)                                                                                                      \
-  switch (d) { PR_GB(T, 32) PR_GB(T, 64) PR_GB(T, 128) default: return -2; }                                           \
-  return (int)hipGetLastError();
+  switch (d) { PR_GB(T, 32) PR_GB(T, 64) PR_GB(T, 128) default: return -2; }
   if (dtype == DT_BF16) { PR_GBT(bf16_t) }
-  if (dtype == DT_F16) { PR_GBT(f16_t) }
+  else if (dtype == DT_F16) { PR_GBT(f16_t) }
+  else return -1;
 #undef PR_GBT
 #undef PR_GB
-  return -1;
+  if (A) {
+    const size_t smem = (size_t)(c + 256) * sizeof(float);
+    hipLaunchKernelGGL(gate_scan_bwd_kernel, dim3((unsigned)(BN * h)), dim3(256), smem, st, dlogG, workspace, dlcs_a,
+                       dlcs_b, c, h, 1.f / deg);
+  }
+  return (int)hipGetLastError();
 }
 
 }  // namespace pr

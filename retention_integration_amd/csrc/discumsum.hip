@@ -14,6 +14,18 @@ namespace pr {
 
 template <typename T> struct Pack16 { enum { N = 16 / sizeof(T) }; typedef __attribute__((ext_vector_type(16 / sizeof(T)))) T type; };
 
+// Sum over the 64 lanes of a wave without LDS traffic inside a row: four rotate-adds (DPP) give every lane its
+// row total, two cross-row exchanges finish.
+__device__ __forceinline__ float wave_sum_dpp(float x) {
+#define PR_ROR(n) __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x120 + n, 0xf, 0xf, true))
+  x += PR_ROR(8);
+  x += PR_ROR(4);
+  x += PR_ROR(2);
+  x += PR_ROR(1);
+#undef PR_ROR
+  return sum_over_rows(x);
+}
+
 template <typename T, int AHEAD>
 __global__ __launch_bounds__(256) void discumsum_fwd_kernel(const T* __restrict__ X, const float* __restrict__ logG,
                                                             T* __restrict__ Y, int n, int n_out, int H, long F) {
@@ -65,7 +77,8 @@ __global__ __launch_bounds__(256) void discumsum_fwd_kernel(const T* __restrict_
 // Reverse scan: r_k = dY[k+1] + exp(log_G[k+1]) * r_{k+1};  dX[k] = r_k;
 // dlog_G[k] = exp(log_G[k]) * sum_F Y[k] * r_k, written as one partial per wave (summed by
 // discumsum_reduce_kernel in a fixed order, so the result is deterministic).
-template <typename T>
+// partial layout: [BH][n][waves_per_bh]
+template <typename T, int AHEAD>
 __global__ __launch_bounds__(256) void discumsum_bwd_kernel(const T* __restrict__ dY, const T* __restrict__ Y,
                                                             const float* __restrict__ logG, T* __restrict__ dX,
                                                             float* __restrict__ partial, int n, int n_out, int H,
@@ -84,42 +97,66 @@ __global__ __launch_bounds__(256) void discumsum_bwd_kernel(const T* __restrict_
   const long xs = (long)H * F / N;
   const float* lg = logG + (long)b * n * H + hh;
   const int wave = (blockIdx.x * blockDim.x + threadIdx.x) >> 6;
-  float* part = partial + ((long)bh * waves_per_bh + wave) * n;
+  float* part = partial + (long)bh * n * waves_per_bh + wave;
 
   float r[N];
 #pragma unroll
   for (int i = 0; i < N; i++) r[i] = 0.f;
-  float g_next = 0.f;  // exp(log_G[k+1]); r_n = 0 so its value at k = n-1 is irrelevant
-  for (int k = n - 1; k >= 0; k--) {
-    vec d, yk;
-    const bool has = (k + 1 < n_out);
-    if (has) d = dy[(long)(k + 1) * xs];
-    yk = y[(long)k * xs];
-    const float gk = __expf(lg[(long)k * H]);
-    float dot = 0.f;
-    vec o;
+  vec zero;
 #pragma unroll
-    for (int i = 0; i < N; i++) {
-      r[i] = r[i] * g_next + (has ? to_f32(d[i]) : 0.f);
-      o[i] = (T)r[i];
-      dot += to_f32(yk[i]) * r[i];
+  for (int i = 0; i < N; i++) zero[i] = (T)0.f;
+  // step j = 0 .. n-1 handles chunk k = n-1-j; dY[k+1] exists when k+1 < n_out
+  vec bd[AHEAD], by[AHEAD];
+#pragma unroll
+  for (int a = 0; a < AHEAD; a++) {
+    const int k = n - 1 - a;
+    if (k >= 0) {
+      bd[a] = (k + 1 < n_out) ? dy[(long)(k + 1) * xs] : zero;
+      by[a] = y[(long)k * xs];
     }
-    if (live) dx[(long)k * xs] = o;
-    dot = wave_sum(live ? dot : 0.f);
-    if (lane_id() == 0) part[k] = dot * gk;
-    g_next = gk;
+  }
+  float g_next = 0.f;  // exp(log_G[k+1]); r_n = 0 so its value at k = n-1 is irrelevant
+  for (int j0 = 0; j0 < n; j0 += AHEAD) {
+#pragma unroll
+    for (int a = 0; a < AHEAD; a++) {
+      const int k = n - 1 - (j0 + a);
+      if (k >= 0) {
+        const vec d = bd[a], yk = by[a];
+        const int kn = k - AHEAD;
+        if (kn >= 0) {
+          bd[a] = dy[(long)(kn + 1) * xs];   // kn + 1 <= n - AHEAD < n_out
+          by[a] = y[(long)kn * xs];
+        }
+        const float gk = __expf(lg[(long)k * H]);
+        float dot = 0.f;
+        vec o;
+#pragma unroll
+        for (int i = 0; i < N; i++) {
+          r[i] = r[i] * g_next + to_f32(d[i]);
+          o[i] = (T)r[i];
+          dot += to_f32(yk[i]) * r[i];
+        }
+        if (live) dx[(long)k * xs] = o;
+        dot = wave_sum_dpp(live ? dot : 0.f);
+        if (lane_id() == 0) part[(long)k * waves_per_bh] = dot * gk;
+        g_next = gk;
+      }
+    }
   }
 }
 
-__global__ void discumsum_reduce_kernel(const float* __restrict__ partial, float* __restrict__ dlogG, int n, int H,
-                                        int waves_per_bh, int BH) {
-  const int i = blockIdx.x * blockDim.x + threadIdx.x;  // over BH * n
-  if (i >= BH * n) return;
-  const int bh = i / n, k = i % n;
+// one wave per (bh, k): sums the waves_per_bh partials in a fixed order
+__global__ __launch_bounds__(256) void discumsum_reduce_kernel(const float* __restrict__ partial, float* __restrict__ dlogG,
+                                                               int n, int H, int waves_per_bh, int BH) {
+  const int w = (blockIdx.x * blockDim.x + threadIdx.x) >> 6;  // over BH * n
+  if (w >= BH * n) return;
+  const int bh = w / n, k = w % n;
   const int b = bh / H, hh = bh % H;
+  const float* p = partial + (long)w * waves_per_bh;
   float s = 0.f;
-  for (int w = 0; w < waves_per_bh; w++) s += partial[((long)bh * waves_per_bh + w) * n + k];
-  dlogG[((long)b * n + k) * H + hh] = s;
+  for (int i = lane_id(); i < waves_per_bh; i += 64) s += p[i];
+  s = wave_sum_dpp(s);
+  if (lane_id() == 0) dlogG[((long)b * n + k) * H + hh] = s;
 }
 
 template <typename T>
@@ -127,7 +164,11 @@ static int launch_fwd(const void* X, const float* logG, void* Y, int B, int n, i
   constexpr int N = Pack16<T>::N;
   const long per_bh = F / N;
   dim3 grid((unsigned)((per_bh + 255) / 256), (unsigned)(B * H));
-  hipLaunchKernelGGL((discumsum_fwd_kernel<T, 4>), grid, dim3(256), 0, st, (const T*)X, logG, (T*)Y, n, n_out, H, F);
+  // few threads in flight (small F): keep many chunks' loads outstanding per thread instead
+  if (per_bh * B * H < 256 * 1024)
+    hipLaunchKernelGGL((discumsum_fwd_kernel<T, 16>), grid, dim3(256), 0, st, (const T*)X, logG, (T*)Y, n, n_out, H, F);
+  else
+    hipLaunchKernelGGL((discumsum_fwd_kernel<T, 4>), grid, dim3(256), 0, st, (const T*)X, logG, (T*)Y, n, n_out, H, F);
   return (int)hipGetLastError();
 }
 template <typename T>
@@ -138,11 +179,15 @@ static int launch_bwd(const void* dY, const void* Y, const float* logG, void* dX
   const unsigned blocks = (unsigned)((per_bh + 255) / 256);
   const int waves = blocks * 4;
   dim3 grid(blocks, (unsigned)(B * H));
-  hipLaunchKernelGGL((discumsum_bwd_kernel<T>), grid, dim3(256), 0, st, (const T*)dY, (const T*)Y, logG, (T*)dX, partial,
-                     n, n_out, H, F, waves);
+  if (per_bh * B * H < 256 * 1024)
+    hipLaunchKernelGGL((discumsum_bwd_kernel<T, 8>), grid, dim3(256), 0, st, (const T*)dY, (const T*)Y, logG, (T*)dX,
+                       partial, n, n_out, H, F, waves);
+  else
+    hipLaunchKernelGGL((discumsum_bwd_kernel<T, 2>), grid, dim3(256), 0, st, (const T*)dY, (const T*)Y, logG, (T*)dX,
+                       partial, n, n_out, H, F, waves);
   const int tot = B * H * n;
-  hipLaunchKernelGGL(discumsum_reduce_kernel, dim3((tot + 255) / 256), dim3(256), 0, st, partial, dlogG, n, H, waves,
-                     B * H);
+  hipLaunchKernelGGL(discumsum_reduce_kernel, dim3((tot * 64 + 255) / 256), dim3(256), 0, st, partial, dlogG, n, H,
+                     waves, B * H);
   return (int)hipGetLastError();
 }
 

@@ -85,9 +85,11 @@ int qs_bwd_prep(const void* O, const void* dO, const float* den, const float* ro
 // chunk_glue.hip (return -5: chunk longer than the LDS-resident gate vector allows)
 int chunk_prep_fwd(const float* logG, const void* K, const void* Q, float* A, float* lcs, void* Kd, void* Qg, int BN,
                    int c, int h, int r, int d, int deg, int dtype, hipStream_t st);
-int chunk_glue_bwd(const float* A, const void* Kd, const void* dKd, const void* Qg, const void* dQg,
+long chunk_glue_bwd_workspace_floats(int BN, int c, int h);
+int chunk_glue_bwd(const float* A, const float* lcs, const void* Kd, const void* dKd, const void* Qg, const void* dQg,
                    const void* dK_attn, const void* dQ_attn, const void* dV_attn, const void* dV_state,
                    const float* dG_attn, const float* dlcs_a, const float* dlcs_b, void* dK, void* dQ, void* dV,
-                   float* dlogG, int BN, int c, int h, int r, int d, int deg, int dtype, hipStream_t st);
+                   float* dlogG, float* workspace, int BN, int c, int h, int r, int d, int deg, int dtype,
+                   hipStream_t st);
 
 }  // namespace pr

@@ -110,9 +110,10 @@ class _ChunkedPowerRetention(torch.autograd.Function):
                    "update_state_bwd")
         dlg = _empty((b, t, h), f32, dev) if gated else None
         # results are written in place over the attention gradients
-        _lib.check(lib.pr_chunk_glue_bwd(p(A), p(Kd), p(dKd), p(Qg), p(dQg), p(dKa), p(dQa), p(dVa), p(dVs), p(dGa),
-                                         p(dl1), p(dl2), p(dKa), p(dQa), p(dVa), p(dlg), BN, c, h, r, d, deg, code, st),
-                   "chunk_glue_bwd")
+        ws = _empty((lib.pr_chunk_glue_bwd_workspace(BN, c, h),), u8, dev) if gated else None
+        _lib.check(lib.pr_chunk_glue_bwd(p(A), p(lcs), p(Kd), p(dKd), p(Qg), p(dQg), p(dKa), p(dQa), p(dVa), p(dVs),
+                                         p(dGa), p(dl1), p(dl2), p(dKa), p(dQa), p(dVa), p(dlg), p(ws), BN, c, h, r, d,
+                                         deg, code, st), "chunk_glue_bwd")
         return dQa, dKa, dVa, dlg, None, None, None
 
 
