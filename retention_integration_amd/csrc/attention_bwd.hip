@@ -150,7 +150,7 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dq_kernel(AttnBwdArgs a)
   for (int it = 0; it < ntiles; it++) {
     const int j0 = it * AB_BN, stage = it & 1;
     stash(stage);
-    __syncthreads();
+    lds_barrier();
     if (it + 1 < ntiles) fetch(j0 + AB_BN);
     const T* kt_ = Kt + stage * AB_BN * LD;
     const T* vt_ = Vt + stage * AB_BN * LD;
@@ -349,7 +349,7 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
   for (int it = 0; it < nsteps; it++) {
     const int rbase = row_begin + it * AB_BM, stage = it & 1;
     stash(stage);
-    __syncthreads();
+    lds_barrier();
     if (it + 1 < nsteps) fetch(rbase + AB_BM);
     const T* qt_ = Qt + stage * AB_BM * LD;
     const T* dot_ = dOt + stage * AB_BM * LD;

@@ -5,24 +5,30 @@
 //   norm: returns o / l;  otherwise (o, l, m).
 //
 // Query rows of the r query heads that share a kv head are folded into one row axis of length tq*r.
-// A workgroup = 4 waves owns 64*MT folded rows of one (batch, kv head); keys stream through LDS 64 at
-// a time.  All products are formed transposed (S^T = K Q^T, O^T = V^T P^T) so that the accumulator
-// layout of S^T is directly the operand layout of the second contraction and no data moves between
-// lanes; row statistics live one row per lane column.
+// A workgroup = 4 waves owns 64*MT folded rows of one (batch, kv head); keys stream 64 at a time through a
+// 3-deep ring of asynchronous global->LDS copies.  All products are formed transposed (S^T = K Q^T,
+// O^T = V^T P^T) so that the accumulator layout of S^T is directly the operand layout of the second
+// contraction and no data moves between lanes; row statistics live one row per lane column.
 //
-// The weights are evaluated without logarithms: w = exp(z) = (|s| + 1e-7)^deg * exp(G_q - G_k) is
-// accumulated unnormalised (w <= (|s|+eps)^deg because gates only decay), its running maximum is
-// tracked, and the row is divided by max_j w at the end, which gives exactly exp(z - m) sums.  For
-// key tiles entirely in a row's past the gate factor is split as exp(G_q - R) * exp(R - G_k) with R
-// the gate at the tile's last key, so the exponentials are per row and per key, not per pair; only
-// the tiles that touch the diagonal evaluate exp(G_q - G_k) per pair.
+// The weights are evaluated without logarithms: w = exp(z) = (|s| + 1e-7)^deg * exp(G_q - G_k) is accumulated
+// unnormalised (w <= (|s|+eps)^deg because gates only decay), its running maximum is tracked, and the row is
+// divided by max_j w at the end, which gives exactly the exp(z - m) sums.  For key tiles entirely in a wave's
+// past the gate factor is split as exp(G_q - R) * exp(R - G_k) with R the gate at the tile's last key, so the
+// exponentials are per row and per key, not per pair; only the tile on the wave's diagonal evaluates
+// exp(G_q - G_k) per pair, and tiles entirely in the wave's future are skipped.  The row sums come from the
+// matrix cores as well (an all-ones operand against the rounded weights), so o / l is an exact average
+// (ref rounds p before summing: retention/_attention/reference.py:52-55).
 #include "common.h"
 #include "kernels.h"
 
 namespace pr {
 
-constexpr int AT_BN = 64;
+constexpr int AT_BN = 64, AT_NST = 3;
 constexpr float AT_LOG_EPS = 1e-7f, AT_SUM_EPS = 1e-6f, AT_EXP_CLAMP = 80.f;
+
+template <typename T> struct OnesBits;
+template <> struct OnesBits<bf16_t> { static constexpr uint32_t v = 0x3F803F80u; };
+template <> struct OnesBits<f16_t> { static constexpr uint32_t v = 0x3C003C00u; };
 
 template <bool DEG2> __device__ __forceinline__ float pow_even(float a, int half_deg) {  // a^(2*half_deg)
   const float a2 = a * a;
@@ -32,39 +38,59 @@ template <bool DEG2> __device__ __forceinline__ float pow_even(float a, int half
   return p;
 }
 
-template <typename T, int DH, int MT, bool DEG2>
-__global__ __launch_bounds__(256) void attention_fwd_kernel(AttnFwdArgs a) {
+template <typename T, int DH, int MT, bool DEG2, int OCC>
+__global__ __launch_bounds__(256, OCC) void attention_fwd_kernel(AttnFwdArgs a) {
   typedef typename VecOf<T>::v8 v8;
   typedef typename VecOf<T>::v4 v4;
-  constexpr int LD = DH + 8, KS = DH / 32, NT = DH / 16, KT = AT_BN / 16, ROWS = 64 * MT;
-  constexpr int CH = AT_BN * DH / 8, PT = (CH + 255) / 256;
-  extern __shared__ __attribute__((aligned(16))) char smem[];
-  T* Kt = (T*)smem;                           // [2][BN][LD]
-  T* Vt = Kt + 2 * AT_BN * LD;                // [2][BN][LD]
-  constexpr int GS = 2 * AT_BN + 4;
-  float* gk = (float*)(Vt + 2 * AT_BN * LD);  // [2][GS]: raw gate [BN], exp(R - gate) [BN], R
+  typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+  typedef __attribute__((address_space(3))) v8 lds_v8;
+  typedef __attribute__((address_space(3))) f32x4 lds_f32x4;
+  typedef __attribute__((address_space(3))) char lds_char;
+  constexpr int KS = DH / 32, NT = DH / 16, KT = AT_BN / 16, ROWS = 64 * MT, CPR = DH / 8, RB = CPR * 16;
+  constexpr int TILE = AT_BN * RB;                  // bytes of one K or V tile
+  constexpr int STAGE = 2 * TILE + 4 * AT_BN * 4;   // K, V, raw gates, two sets of key gate factors
+  constexpr int LOADS = 2 * AT_BN * CPR / 256;      // tile copies per thread per stage
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
 
-  const int tid = threadIdx.x, l = tid & 63, g = l >> 4, wave = tid >> 6, tcol = l & 15;
+  const int tid = threadIdx.x, l = tid & 63, g = l >> 4, tcol = l & 15;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform, so branches on it are scalar
   const int b = blockIdx.y / a.h, hh = blockIdx.y % a.h;
   const int hq = a.h * a.r, rows = a.tq * a.r, shift = a.tk - a.tq;
   const int row0 = blockIdx.x * ROWS;
   const T* Qg = (const T*)a.Q + (long)b * a.tq * hq * DH;
-  const T* Kg = (const T*)a.K + (long)b * a.tk * a.h * DH + hh * DH;
-  const T* Vg = (const T*)a.V + (long)b * a.tk * a.h * DH + hh * DH;
+  const char* Kg = (const char*)((const T*)a.K + (long)b * a.tk * a.h * DH + hh * DH);
+  const char* Vg = (const char*)((const T*)a.V + (long)b * a.tk * a.h * DH + hh * DH);
   const float* Gg = a.G ? a.G + (long)b * a.tk * a.h + hh : nullptr;
-  const long kstride = (long)a.h * DH;
+  const long kstride = (long)a.h * DH * 2;
   const int half_deg = (int)a.deg / 2;
   const float eps_s = AT_LOG_EPS / a.scale;          // |scale*x| + eps = scale * (|x| + eps/scale)
-  const float scale_p = __powf(a.scale, a.deg);
+  const float scale_p = __expf(a.deg * __logf(a.scale));
+
+  const int last_row = min(row0 + ROWS, rows) - 1;
+  const int kmax = min(a.tk, last_row / a.r + shift + 1);   // keys any row of the workgroup can see
+  const int ntiles = (kmax + AT_BN - 1) / AT_BN;
+  const int wrow0 = row0 + wave * 16 * MT;
+  const int w_first_ti = min(wrow0, rows - 1) / a.r + shift;               // smallest time index in the wave
+  const int w_last_ti = min(wrow0 + 16 * MT - 1, rows - 1) / a.r + shift;  // largest
+
+  auto issue = [&](int it) {
+    char* st = smem + (it % AT_NST) * STAGE;
+    const int j0 = it * AT_BN;
+    async_load_tile<CPR, AT_BN>(st, [&](int row) { return Kg + (long)min(j0 + row, a.tk - 1) * kstride; });
+    async_load_tile<CPR, AT_BN>(st + TILE, [&](int row) { return Vg + (long)min(j0 + row, a.tk - 1) * kstride; });
+    if (Gg && tid < 64) async_copy4(Gg + (long)min(j0 + tid, a.tk - 1) * a.h, st + 2 * TILE);
+  };
+  issue(0);
+  if (ntiles > 1) issue(1);
 
   v8 Qf[MT][KS];
   int ti[MT];
   long qoff[MT];
   bool live[MT];
-  float Gq[MT], mx[MT], lsum[MT];
+  float Gq[MT], mx[MT];
 #pragma unroll
   for (int mi = 0; mi < MT; mi++) {
-    const int row = row0 + wave * 16 * MT + 16 * mi + tcol;
+    const int row = wrow0 + 16 * mi + tcol;
     live[mi] = row < rows;
     const int rr = live[mi] ? row : 0;
     const int t = rr / a.r;
@@ -78,137 +104,155 @@ __global__ __launch_bounds__(256) void attention_fwd_kernel(AttnFwdArgs a) {
     }
     Gq[mi] = Gg ? Gg[(long)ti[mi] * a.h] : 0.f;
     mx[mi] = 0.f;
-    lsum[mi] = 0.f;
   }
-  f32x4 acc[MT][NT];
+  f32x4 acc[MT][NT], accl[MT];
 #pragma unroll
-  for (int mi = 0; mi < MT; mi++)
+  for (int mi = 0; mi < MT; mi++) {
 #pragma unroll
     for (int nt = 0; nt < NT; nt++) acc[mi][nt] = (f32x4){0, 0, 0, 0};
+    accl[mi] = (f32x4){0, 0, 0, 0};
+  }
+  const f32x4 epsv = {eps_s, eps_s, eps_s, eps_s};
+  const uint32_t one2 = OnesBits<T>::v;
+  v8 ones = __builtin_bit_cast(v8, (u32x4){one2, one2, one2, one2});
+  asm volatile("" : "+v"(ones));   // keep the four registers instead of rebuilding them at every use
 
-  const int last_row = min(row0 + ROWS, rows) - 1;
-  const int kmax = min(a.tk, last_row / a.r + shift + 1);   // keys any row of the workgroup can see
-  const int first_ti = row0 / a.r + shift;                   // smallest time index in the workgroup
-  const int ntiles = (kmax + AT_BN - 1) / AT_BN;
-
-  u32x4 rk[PT], rv[PT];
-  float rg = 0.f, rR = 0.f;
-  auto fetch = [&](int j0) {
+  // Per-lane LDS byte offsets; the swizzle depends only on the lane's row inside a 16-row group.
+  int koff[KS], voff[NT];
 #pragma unroll
-    for (int i = 0; i < PT; i++) {
-      const int ch = tid + 256 * i;
-      const int key = j0 + ch / (DH / 8), col = (ch % (DH / 8)) * 8;
-      rk[i] = (u32x4){0, 0, 0, 0};
-      rv[i] = (u32x4){0, 0, 0, 0};
-      if (ch < CH && key < a.tk) {
-        rk[i] = *(const u32x4*)(Kg + key * kstride + col);
-        rv[i] = *(const u32x4*)(Vg + key * kstride + col);
-      }
-    }
-    if (tid < AT_BN && Gg) {
-      rg = Gg[(long)min(j0 + tid, a.tk - 1) * a.h];
-      rR = Gg[(long)min(j0 + AT_BN - 1, a.tk - 1) * a.h];
-    }
-  };
-  auto stash = [&](int stage) {
+  for (int ks = 0; ks < KS; ks++) koff[ks] = tcol * RB + (((4 * ks + g) ^ swz<CPR>(tcol)) * 16);
+  {
+    const int vr = 4 * g + (tcol >> 2);   // V^T operand: row 4g + (s>>2) of a 16-key group, columns 16*nt + 4*(s&3) ..
 #pragma unroll
-    for (int i = 0; i < PT; i++) {
-      const int ch = tid + 256 * i;
-      if (ch < CH) {
-        const int o = stage * AT_BN * LD + (ch / (DH / 8)) * LD + (ch % (DH / 8)) * 8;
-        *(u32x4*)(Kt + o) = rk[i];
-        *(u32x4*)(Vt + o) = rv[i];
-      }
-    }
-    if (tid < AT_BN) {
-      gk[stage * GS + tid] = rg;
-      gk[stage * GS + AT_BN + tid] = __expf(fminf(rR - rg, AT_EXP_CLAMP));
-      if (tid == 0) gk[stage * GS + 2 * AT_BN] = rR;
-    }
-  };
-
-  fetch(0);
-  for (int it = 0; it < ntiles; it++) {
-    const int j0 = it * AT_BN, stage = it & 1;
-    stash(stage);
-    __syncthreads();
-    if (it + 1 < ntiles) fetch(j0 + AT_BN);
-    const T* kt_ = Kt + stage * AT_BN * LD;
-    const T* vt_ = Vt + stage * AT_BN * LD;
-    const float* gk_ = gk + stage * GS;
-    const bool diag = (j0 + AT_BN - 1 > first_ti) || (j0 + AT_BN > a.tk);   // some pair of the tile is masked
-    const float R = gk_[2 * AT_BN];
-
-    v8 kf[KT][KS];
-#pragma unroll
-    for (int kt = 0; kt < KT; kt++)
-#pragma unroll
-      for (int ks = 0; ks < KS; ks++) kf[kt][ks] = lds_frag<T>(kt_, LD, 16 * kt, 32 * ks);
-    f32x4 gkv[KT];
-#pragma unroll
-    for (int kt = 0; kt < KT; kt++) gkv[kt] = *(const f32x4*)(gk_ + (diag ? 0 : AT_BN) + 16 * kt + 4 * g);
-
-    v8 pf[MT][KT / 2];
-#pragma unroll
-    for (int mi = 0; mi < MT; mi++) {
-      const float eu = scale_p * (diag ? 1.f : __expf(fminf(Gq[mi] - R, AT_EXP_CLAMP)));
-      float p[KT][4];
-#pragma unroll
-      for (int kt = 0; kt < KT; kt++) {
-        f32x4 s = {0, 0, 0, 0};
-#pragma unroll
-        for (int ks = 0; ks < KS; ks++) s = mfma16(kf[kt][ks], Qf[mi][ks], s);
-#pragma unroll
-        for (int v = 0; v < 4; v++) {
-          const float pw = pow_even<DEG2>(fabsf(s[v]) + eps_s, half_deg);
-          float w;
-          if (diag) {
-            const int key = j0 + 16 * kt + 4 * g + v;
-            w = pw * eu * __expf(fminf(Gq[mi] - gkv[kt][v], AT_EXP_CLAMP));
-            if (key > ti[mi] || key >= a.tk) w = 0.f;
-          } else {
-            w = pw * gkv[kt][v] * eu;
-          }
-          p[kt][v] = w;
-          mx[mi] = fmaxf(mx[mi], w);
-        }
-      }
-      // the row sum is taken over the weights as the matrix cores will see them (rounded to 16 bit), so that
-      // o / l is an exact average (ref rounds p before summing: retention/_attention/reference.py:52-55)
-#pragma unroll
-      for (int kp = 0; kp < KT / 2; kp++) {
-        float q8[8];
-#pragma unroll
-        for (int v = 0; v < 4; v++) {
-          q8[v] = p[2 * kp][v];
-          q8[4 + v] = p[2 * kp + 1][v];
-        }
-        pf[mi][kp] = pack8<T>(q8);
-        unpack8(pf[mi][kp], q8);
-#pragma unroll
-        for (int v = 0; v < 8; v++) lsum[mi] += q8[v];
-      }
-    }
-    // O^T += V^T P^T, 32 keys per step: elements 0-3 are keys 4g.. of the first 16, 4-7 of the second 16
-#pragma unroll
-    for (int kp = 0; kp < KT / 2; kp++) {
-#pragma unroll
-      for (int nt = 0; nt < NT; nt++) {
-        v4 lo = lds_frag_tr4<T>(vt_, LD, 32 * kp + 4 * g, 16 * nt);
-        v4 hi = lds_frag_tr4<T>(vt_, LD, 32 * kp + 16 + 4 * g, 16 * nt);
-        v8 vf = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-#pragma unroll
-        for (int mi = 0; mi < MT; mi++) acc[mi][nt] = mfma16(vf, pf[mi][kp], acc[mi][nt]);
-      }
+    for (int nt = 0; nt < NT; nt++) {
+      const int col = 16 * nt + 4 * (tcol & 3);
+      voff[nt] = vr * RB + (((col / 8) ^ swz<CPR>(vr)) * 16) + (col % 8) * 2;
     }
   }
+
+  // Every wave runs ntiles steps with one barrier each, split by what the tile is to THIS wave: tiles entirely in
+  // its past (no masking code at all), tiles that cross its diagonal, and tiles entirely in its future, for
+  // which it only takes part in the copies and the barrier.  Three loops instead of one loop with branches keep
+  // the accumulators in place (no copies between control-flow paths).
+  const int n_past = min(ntiles, min(w_first_ti + 1, a.tk) / AT_BN);   // tiles with every pair visible
+  const int n_seen = min(ntiles, w_last_ti / AT_BN + 1);               // tiles with at least one visible pair
+
+  auto sync_step = [&](int it) -> char* {   // make tile `it` visible to the workgroup, start the copy of tile it+2
+    char* st = smem + (it % AT_NST) * STAGE;
+    if (it + 1 < ntiles) wait_vmcnt<LOADS>(); else wait_vmcnt<0>();
+    float* graw = (float*)(st + 2 * TILE);
+    if (tid < 64) {   // wave 0 issued the gate copy, so the values are visible to it once its own counter drained
+      const int rpos = min(AT_BN - 1, a.tk - 1 - it * AT_BN);
+      const float gv = Gg ? graw[tid] : 0.f;
+      const float R_ = Gg ? graw[rpos] : 0.f, Rs = Gg ? graw[tid & ~15] : 0.f;
+      graw[AT_BN + tid] = __expf(fminf(R_ - gv, AT_EXP_CLAMP));       // relative to the tile's last key   (<= 1)
+      graw[2 * AT_BN + tid] = __expf(fminf(Rs - gv, AT_EXP_CLAMP));   // relative to the first key of its 16 (>= 1)
+      if (!Gg) graw[tid] = 0.f;
+    }
+    lds_barrier();
+    if (it + 2 < ntiles) issue(it + 2);
+    return st;
+  };
+
+  // One 64-key tile.  Past tiles use one reference gate (the tile's last key), so both gate factors are <= 1.
+  // Diagonal tiles use the first key of every 16-key group instead: for every visible pair the row factor is
+  // then <= 1 and the key factor spans only 16 steps of decay, so neither leaves the fp32 range.
+  auto tile = [&](int it, const char* st, auto diag_c) {
+    constexpr bool DIAG = decltype(diag_c)::value != 0;
+    const int j0 = it * AT_BN;
+    const float* graw = (const float*)(st + 2 * TILE);
+    // LDS byte addresses of this lane's operands; opaque, so that the per-group and per-column-tile displacements
+    // stay immediate offsets of the loads instead of one address register each
+    uint32_t kb[KS], vb[NT], eb;
+    {
+      const uint32_t sa = (uint32_t)(uintptr_t)(lds_char*)st;
+#pragma unroll
+      for (int ks = 0; ks < KS; ks++) { kb[ks] = sa + koff[ks]; asm volatile("" : "+v"(kb[ks])); }
+#pragma unroll
+      for (int nt = 0; nt < NT; nt++) { vb[nt] = sa + TILE + voff[nt]; asm volatile("" : "+v"(vb[nt])); }
+      eb = sa + 2 * TILE + (DIAG ? 2 * AT_BN : AT_BN) * 4 + 16 * g;
+      asm volatile("" : "+v"(eb));
+    }
+    float eu[MT];
+    int lim[MT];
+#pragma unroll
+    for (int mi = 0; mi < MT; mi++) {
+      if (DIAG) lim[mi] = min(ti[mi], a.tk - 1) - j0 - 4 * g;   // pair (row, key 16*kt + 4g + v) visible iff 16*kt + v <= lim
+      else eu[mi] = scale_p * __expf(fminf(Gq[mi] - graw[min(AT_BN - 1, a.tk - 1 - j0)], AT_EXP_CLAMP));
+    }
+#pragma unroll
+    for (int kp = 0; kp < KT / 2; kp++) {
+      // S^T for 32 keys: operands first, then every product, so the matrix pipe runs back to back
+      v8 kf[2][KS];
+      f32x4 ev[2];
+#pragma unroll
+      for (int half = 0; half < 2; half++) {
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) kf[half][ks] = *(const lds_v8*)(kb[ks] + (2 * kp + half) * 16 * RB);
+        ev[half] = *(const lds_f32x4*)(eb + 64 * (2 * kp + half));
+      }
+      f32x4 sc[2][MT];
+#pragma unroll
+      for (int half = 0; half < 2; half++)
+#pragma unroll
+        for (int mi = 0; mi < MT; mi++) sc[half][mi] = epsv;   // start at eps: (s + eps)^deg stands in for (|s| + eps)^deg
+#pragma unroll
+      for (int ks = 0; ks < KS; ks++)
+#pragma unroll
+        for (int half = 0; half < 2; half++)
+#pragma unroll
+          for (int mi = 0; mi < MT; mi++) sc[half][mi] = mfma16(kf[half][ks], Qf[mi][ks], sc[half][mi]);
+      // V^T operands for the same 32 keys, in flight while the weights are formed
+      v8 vf[NT];
+#pragma unroll
+      for (int nt = 0; nt < NT; nt++) {
+        const uint32_t vp = vb[nt] + kp * 32 * RB;
+        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)vp);
+        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(vp + 16 * RB));
+        const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        vf[nt] = __builtin_bit_cast(v8, both);
+      }
+      v8 pf[MT];
+#pragma unroll
+      for (int mi = 0; mi < MT; mi++) {
+        float p[8];
+#pragma unroll
+        for (int half = 0; half < 2; half++) {
+          float e = eu[mi];
+          if (DIAG) e = scale_p * __expf(fminf(Gq[mi] - graw[16 * (2 * kp + half)], AT_EXP_CLAMP));
+#pragma unroll
+          for (int v = 0; v < 4; v++) {
+            float w = pow_even<DEG2>(sc[half][mi][v], half_deg) * ev[half][v] * e;
+            if (DIAG) w = (32 * kp + 16 * half + v <= lim[mi]) ? w : 0.f;
+            p[4 * half + v] = w;
+          }
+        }
+#pragma unroll
+        for (int e = 0; e < 8; e++) mx[mi] = fmaxf(mx[mi], p[e]);
+        pf[mi] = pack8<T>(p);
+      }
+      // O^T += V^T P^T over these 32 keys (elements 0-3 are keys 4g.. of the first 16, 4-7 of the second 16);
+      // the all-ones operand adds the row sums of the rounded weights
+#pragma unroll
+      for (int mi = 0; mi < MT; mi++) accl[mi] = mfma16(ones, pf[mi], accl[mi]);
+#pragma unroll
+      for (int nt = 0; nt < NT; nt++)
+#pragma unroll
+        for (int mi = 0; mi < MT; mi++) acc[mi][nt] = mfma16(vf[nt], pf[mi], acc[mi][nt]);
+    }
+  };
+
+  int it = 0;
+  for (; it < n_past; it++) tile(it, sync_step(it), IC<0>{});
+  for (; it < n_seen; it++) tile(it, sync_step(it), IC<1>{});
+  for (; it < ntiles; it++) sync_step(it);
 
   T* Og = (T*)a.O + (long)b * a.tq * hq * DH;
 #pragma unroll
   for (int mi = 0; mi < MT; mi++) {
-    const float wmax = max_over_rows(mx[mi]);          // = exp(rowmax)
-    const float wsum = sum_over_rows(lsum[mi]);
+    const float wmax = max_over_rows(mx[mi]);   // = exp(rowmax)
     if (!live[mi]) continue;
+    const float wsum = accl[mi][0];             // every accumulator row of the all-ones product holds the row sum
     const float inv = 1.f / wmax;
     const float lrow = wsum * inv + AT_SUM_EPS;
     const float f = a.norm ? inv / lrow : inv;
@@ -227,29 +271,35 @@ __global__ __launch_bounds__(256) void attention_fwd_kernel(AttnFwdArgs a) {
   }
 }
 
-template <typename T, int DH> static int attn_fwd_launch(const AttnFwdArgs& a, int B, hipStream_t st) {
-  constexpr int MT = DH <= 64 ? 2 : 1;
-  constexpr size_t smem = 2 * 2 * AT_BN * (DH + 8) * sizeof(T) + 2 * (2 * AT_BN + 4) * sizeof(float);
+template <typename T, int DH, bool DEG2> static int attn_fwd_launch(const AttnFwdArgs& a, int B, hipStream_t st) {
   const int rows = a.tq * a.r;
-  dim3 grid((rows + 64 * MT - 1) / (64 * MT), (unsigned)(B * a.h));
-  if (a.deg == 2.f) {
-    auto kern = attention_fwd_kernel<T, DH, MT, true>;
+  auto go = [&](auto mt, auto occ) {
+    constexpr int MT = decltype(mt)::value, OCC = decltype(occ)::value;
+    constexpr size_t smem = AT_NST * (2 * AT_BN * DH * 2 + 4 * AT_BN * 4);
+    dim3 grid((rows + 64 * MT - 1) / (64 * MT), (unsigned)(B * a.h));
+    auto kern = attention_fwd_kernel<T, DH, MT, DEG2, OCC>;
     allow_big_lds((const void*)kern, smem);
     hipLaunchKernelGGL(kern, grid, dim3(256), smem, st, a);
-  } else {
-    auto kern = attention_fwd_kernel<T, DH, MT, false>;
-    allow_big_lds((const void*)kern, smem);
-    hipLaunchKernelGGL(kern, grid, dim3(256), smem, st, a);
-  }
+  };
+  const char* e = getenv("PR_AT_VARIANT");
+  const int var = e ? atoi(e) : 0;
+  if (var == 1 && DH <= 64) go(IC<2>{}, IC<3>{});
+  else if (var == 2 && DH <= 64) go(IC<2>{}, IC<4>{});
+  else if (var == 3 && DH <= 64) go(IC<1>{}, IC<4>{});
+  else if (var == 4 && DH <= 64) go(IC<2>{}, IC<2>{});
+  else if (DH <= 64 && rows >= 256) go(IC<4>{}, IC<2>{});
+  else if (rows > 64) go(IC<2>{}, IC<2>{});
+  else go(IC<1>{}, IC<2>{});
   return (int)hipGetLastError();
 }
 
 int attention_fwd(const AttnFwdArgs& a, int B, int d, int dtype, hipStream_t st) {
+  const bool deg2 = a.deg == 2.f;
 #define PR_AF(T)                                                                                                       \
   switch (d) {                                                                                                         \
-    case 32: return attn_fwd_launch<T, 32>(a, B, st);                                                                  \
-    case 64: return attn_fwd_launch<T, 64>(a, B, st);                                                                  \
-    case 128: return attn_fwd_launch<T, 128>(a, B, st);                                                                \
+    case 32: return deg2 ? attn_fwd_launch<T, 32, true>(a, B, st) : attn_fwd_launch<T, 32, false>(a, B, st);           \
+    case 64: return deg2 ? attn_fwd_launch<T, 64, true>(a, B, st) : attn_fwd_launch<T, 64, false>(a, B, st);           \
+    case 128: return deg2 ? attn_fwd_launch<T, 128, true>(a, B, st) : attn_fwd_launch<T, 128, false>(a, B, st);        \
     default: return -2;                                                                                                \
   }
   if (dtype == DT_BF16) { PR_AF(bf16_t) }

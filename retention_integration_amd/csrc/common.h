@@ -140,6 +140,14 @@ __device__ __forceinline__ void async_copy4(const void* gsrc, void* lds_wave_bas
                                    (__attribute__((address_space(3))) void*)lds_wave_base, 4, 0, 0);
 }
 
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also drains the vector-memory counter, which
+// would make every asynchronous global->LDS copy (and every register prefetch) in flight complete at each barrier;
+// here only this wave's LDS operations are waited for, and copies are tracked by wait_vmcnt<N>() alone.  The asm
+// memory clobber keeps the compiler from moving LDS accesses across it.
+__device__ __forceinline__ void lds_barrier() {
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
 // Issue the copies of a tile of R rows (R*CPR a multiple of 256) by a 256-thread workgroup: every thread
 // issues exactly R*CPR/256 copies.  row_ptr(row) returns the global address of the row's first byte and
 // must be valid for every row (clamp out-of-range rows; zero them afterwards with zero_tile_rows).

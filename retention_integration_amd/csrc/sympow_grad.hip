@@ -133,7 +133,7 @@ __global__ __launch_bounds__(256, 2) void sympow_grad_kernel(GradArgs a, int row
   for (int step = 0; step < NSTEP; step++) {
     const char* st = ring + (step % GR_NST) * STAGE;
     if (step + 1 < NSTEP) wait_vmcnt<LOADS>(); else wait_vmcnt<0>();
-    __syncthreads();
+    lds_barrier();
     if (step + 2 < NSTEP) issue(step + 2);
     const int f0 = step * GR_FR;
     int y = 0;
@@ -190,7 +190,7 @@ __global__ __launch_bounds__(256, 2) void sympow_grad_kernel(GradArgs a, int row
   // (now idle) ring memory.
   T* Mt = (T*)ring;   // [DK][LDM]
   for (int part = 0; part < 2; part++) {
-    __syncthreads();
+    lds_barrier();
     for (int idx = tid; idx < DK * DK; idx += 256) {
       const int w = idx / DK, aa = idx % DK, yw = w / 16, ya = aa / 16;
       float val;
@@ -204,7 +204,7 @@ __global__ __launch_bounds__(256, 2) void sympow_grad_kernel(GradArgs a, int row
       const T hi16 = (T)val;
       Mt[w * LDM + aa] = part == 0 ? hi16 : (T)(val - (float)hi16);
     }
-    __syncthreads();
+    lds_barrier();
 #pragma unroll
     for (int mi = 0; mi < MT; mi++) {
       v8 xf[KX];

@@ -118,7 +118,7 @@ __global__ __launch_bounds__(256, 2) void sympow_nn_kernel(NNArgs a, int row_blo
   async_load_tile<CX, ROWS>(xt, [&](int row) { return (const char*)(Xg + row_off(row0 + row) * DK); });
   if (skip) {
     wait_vmcnt<0>();
-    __syncthreads();
+    lds_barrier();
   } else {
     FeatIter<MULT> cur, nxt;
     cur.init(TT);
@@ -133,7 +133,7 @@ __global__ __launch_bounds__(256, 2) void sympow_nn_kernel(NNArgs a, int row_blo
     while (!cur.done()) {
       const char* st = ring + (step % NN_NST) * STAGE;
       if (issued > step + 1) wait_vmcnt<LOADS>(); else wait_vmcnt<0>();
-      __syncthreads();
+      lds_barrier();
       if (!nxt.done()) {
         issue(nxt.f0(), issued % NN_NST);
         nxt.next();
@@ -171,7 +171,7 @@ __global__ __launch_bounds__(256, 2) void sympow_nn_kernel(NNArgs a, int row_blo
       // and a low 16-bit part), then a dot with x[row, b] down the accumulator rows.
       T* Mt = (T*)ring;   // [DK (b)][LDM (a)]
       for (int part = 0; part < 2; part++) {
-        __syncthreads();
+        lds_barrier();
         for (int idx = tid; idx < DK * DK; idx += 256) {
           const int b_ = idx / DK, aa = idx % DK, yb = b_ / 16;
           float val = 0.f;
@@ -179,7 +179,7 @@ __global__ __launch_bounds__(256, 2) void sympow_nn_kernel(NNArgs a, int row_blo
           const T hi16 = (T)val;
           Mt[b_ * LDM + aa] = part == 0 ? hi16 : (T)(val - (float)hi16);
         }
-        __syncthreads();
+        lds_barrier();
 #pragma unroll
         for (int mi = 0; mi < MT; mi++) {
           const int lrow = wave * 16 * MT + 16 * mi + tcol;
@@ -205,13 +205,13 @@ __global__ __launch_bounds__(256, 2) void sympow_nn_kernel(NNArgs a, int row_blo
   if (EPI == NN_EPI_MERGE) {
     // hand aux from the lane that holds the row as a column to the lanes that hold it as accumulator rows
     float* ax = (float*)ring;
-    __syncthreads();
+    lds_barrier();
 #pragma unroll
     for (int mi = 0; mi < MT; mi++) {
       const float tot = sum_over_rows(aux[mi]) * ScaleS<T>::up;
       if (g == 0) ax[wave * 16 * MT + 16 * mi + tcol] = tot;
     }
-    __syncthreads();
+    lds_barrier();
     constexpr float log_gamma_2 = 0.f;
     (void)log_gamma_2;
     const float log_gamma = 0.5f * __logf((float)D);

@@ -81,7 +81,7 @@ __device__ __forceinline__ void tn_body(const T* __restrict__ A, const T* __rest
     char* st = smem + (step % TN_NST) * STAGE;
     if (step + 1 < steps) wait_vmcnt<LOADS>(); else wait_vmcnt<0>();
     if ((step + 1) * TN_KT > rows) zero_tile_rows<CA, TN_KT>(st, rows - step * TN_KT);
-    __syncthreads();
+    lds_barrier();
     if (step + 2 < steps) issue(step + 2);
     if (active) {
       const float* wt = (const float*)(st + A_BYTES + B_BYTES);
