@@ -30,8 +30,10 @@ template <typename T> struct OnesBits;
 template <> struct OnesBits<bf16_t> { static constexpr uint32_t v = 0x3F803F80u; };
 template <> struct OnesBits<f16_t> { static constexpr uint32_t v = 0x3C003C00u; };
 
-template <bool DEG2> __device__ __forceinline__ float pow_even(float a, int half_deg) {  // a^(2*half_deg)
-  const float a2 = a * a;
+// (s^2 + eps^2)^half_deg, which stands in for (|s| + eps)^(2*half_deg): equal at s = 0 and within a relative
+// 2*eps/|s| elsewhere, and it needs neither the absolute value nor a separate addition.
+template <bool DEG2> __device__ __forceinline__ float pow_even(float sv, float eps2, int half_deg) {
+  const float a2 = __builtin_fmaf(sv, sv, eps2);
   float p = a2;
   if (!DEG2)
     for (int k = 1; k < half_deg; k++) p *= a2;
@@ -39,7 +41,7 @@ template <bool DEG2> __device__ __forceinline__ float pow_even(float a, int half
 }
 
 template <typename T, int DH, int MT, bool DEG2, int OCC>
-__global__ __launch_bounds__(256, OCC) void attention_fwd_kernel(AttnFwdArgs a) {
+__global__ __launch_bounds__(256, OCC) void attention_fwd_kernel(AttnFwdArgs a, int row_blocks, int npairs) {
   typedef typename VecOf<T>::v8 v8;
   typedef typename VecOf<T>::v4 v4;
   typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
@@ -54,9 +56,19 @@ __global__ __launch_bounds__(256, OCC) void attention_fwd_kernel(AttnFwdArgs a) 
 
   const int tid = threadIdx.x, l = tid & 63, g = l >> 4, tcol = l & 15;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform, so branches on it are scalar
-  const int b = blockIdx.y / a.h, hh = blockIdx.y % a.h;
+  // Workgroups are dealt round-robin by their linear index: to the 8 XCDs first, then inside an XCD to its 4
+  // shader engines (index / 8 % 4); only the CU inside a shader engine is chosen by load.  Row blocks differ in
+  // length (causal), so each of the 32 (XCD, shader engine) groups is given whole (batch, kv head) pairs: every
+  // group then gets the same mix of long and short row blocks and the K/V of a pair stay in one L2.  Inside a
+  // group the longest row blocks of all its pairs come first and the shortest last (they fill the tail).
+  const int grp = blockIdx.x % 32, u = blockIdx.x / 32, ppg = (npairs + 31) / 32;
+  const int pair = (u % ppg) * 32 + grp, rblk = row_blocks - 1 - u / ppg;
+  if (pair >= npairs) return;
+  const int b = pair / a.h, hh = pair % a.h;
   const int hq = a.h * a.r, rows = a.tq * a.r, shift = a.tk - a.tq;
-  const int row0 = blockIdx.x * ROWS;
+  // every other workgroup hands its 16*MT-row slices to the waves in reverse order: the wave nearest the
+  // diagonal has the most tiles, and co-resident workgroups then load the four SIMDs evenly
+  const int row0 = rblk * ROWS;
   const T* Qg = (const T*)a.Q + (long)b * a.tq * hq * DH;
   const char* Kg = (const char*)((const T*)a.K + (long)b * a.tk * a.h * DH + hh * DH);
   const char* Vg = (const char*)((const T*)a.V + (long)b * a.tk * a.h * DH + hh * DH);
@@ -69,16 +81,34 @@ __global__ __launch_bounds__(256, OCC) void attention_fwd_kernel(AttnFwdArgs a) 
   const int last_row = min(row0 + ROWS, rows) - 1;
   const int kmax = min(a.tk, last_row / a.r + shift + 1);   // keys any row of the workgroup can see
   const int ntiles = (kmax + AT_BN - 1) / AT_BN;
-  const int wrow0 = row0 + wave * 16 * MT;
+  const int wslice = (u & 1) ? 3 - wave : wave;
+  const int wrow0 = row0 + wslice * 16 * MT;
   const int w_first_ti = min(wrow0, rows - 1) / a.r + shift;               // smallest time index in the wave
   const int w_last_ti = min(wrow0 + 16 * MT - 1, rows - 1) / a.r + shift;  // largest
 
+  // Copies of one stage: every thread owns LOADS/2 16-byte chunks of the K tile and the same chunks of the V tile.
+  // Its byte offsets inside a tile are fixed, so a full tile costs no address arithmetic beyond a scalar base.
+  uint32_t goff[LOADS / 2];
+#pragma unroll
+  for (int ii = 0; ii < LOADS / 2; ii++) {
+    const int pos = (ii * 4 + wave) * 64 + l, row = pos / CPR;
+    goff[ii] = (uint32_t)(row * (int)kstride + 16 * ((pos % CPR) ^ swz<CPR>(row)));
+  }
   auto issue = [&](int it) {
     char* st = smem + (it % AT_NST) * STAGE;
     const int j0 = it * AT_BN;
-    async_load_tile<CPR, AT_BN>(st, [&](int row) { return Kg + (long)min(j0 + row, a.tk - 1) * kstride; });
-    async_load_tile<CPR, AT_BN>(st + TILE, [&](int row) { return Vg + (long)min(j0 + row, a.tk - 1) * kstride; });
-    if (Gg && tid < 64) async_copy4(Gg + (long)min(j0 + tid, a.tk - 1) * a.h, st + 2 * TILE);
+    if (j0 + AT_BN <= a.tk) {
+      const char* kb_ = Kg + (long)j0 * kstride;
+      const char* vb_ = Vg + (long)j0 * kstride;
+#pragma unroll
+      for (int ii = 0; ii < LOADS / 2; ii++) async_copy16(kb_ + goff[ii], st + (ii * 4 + wave) * 1024);
+#pragma unroll
+      for (int ii = 0; ii < LOADS / 2; ii++) async_copy16(vb_ + goff[ii], st + TILE + (ii * 4 + wave) * 1024);
+    } else {   // last, partial tile: rows past the end repeat the last key (they are masked)
+      async_load_tile<CPR, AT_BN>(st, [&](int row) { return Kg + (long)min(j0 + row, a.tk - 1) * kstride; });
+      async_load_tile<CPR, AT_BN>(st + TILE, [&](int row) { return Vg + (long)min(j0 + row, a.tk - 1) * kstride; });
+    }
+    if (Gg && wave == 0) async_copy4(Gg + (long)min(j0 + l, a.tk - 1) * a.h, st + 2 * TILE);
   };
   issue(0);
   if (ntiles > 1) issue(1);
@@ -112,7 +142,8 @@ __global__ __launch_bounds__(256, OCC) void attention_fwd_kernel(AttnFwdArgs a) 
     for (int nt = 0; nt < NT; nt++) acc[mi][nt] = (f32x4){0, 0, 0, 0};
     accl[mi] = (f32x4){0, 0, 0, 0};
   }
-  const f32x4 epsv = {eps_s, eps_s, eps_s, eps_s};
+  const float eps2 = eps_s * eps_s;
+  const float Rw = Gg ? Gg[(long)w_first_ti * a.h] : 0.f;   // gate at the wave's first row
   const uint32_t one2 = OnesBits<T>::v;
   v8 ones = __builtin_bit_cast(v8, (u32x4){one2, one2, one2, one2});
   asm volatile("" : "+v"(ones));   // keep the four registers instead of rebuilding them at every use
@@ -137,20 +168,32 @@ __global__ __launch_bounds__(256, OCC) void attention_fwd_kernel(AttnFwdArgs a) 
   const int n_past = min(ntiles, min(w_first_ti + 1, a.tk) / AT_BN);   // tiles with every pair visible
   const int n_seen = min(ntiles, w_last_ti / AT_BN + 1);               // tiles with at least one visible pair
 
-  auto sync_step = [&](int it) -> char* {   // make tile `it` visible to the workgroup, start the copy of tile it+2
+  // Gate factors of tile `it`, written by wave 0 (it issued the gate copy, so it alone can wait for it):
+  // exp(R - gate) relative to the tile's last key (<= 1) and relative to the first key of each 16-key group (>= 1).
+  auto gate_factors = [&](int it) {
+    float* graw = (float*)(smem + (it % AT_NST) * STAGE + 2 * TILE);
+    const int rpos = min(AT_BN - 1, a.tk - 1 - it * AT_BN);
+    const float gv = Gg ? graw[l] : 0.f;
+    const float R_ = Gg ? graw[rpos] : 0.f, Rs = Gg ? graw[l & ~15] : 0.f;
+    graw[AT_BN + l] = __expf(fminf(R_ - gv, AT_EXP_CLAMP));
+    graw[2 * AT_BN + l] = __expf(fminf(Rs - gv, AT_EXP_CLAMP));
+    if (!Gg) graw[l] = 0.f;
+  };
+  if (wave == 0) {
+    wait_vmcnt<0>();
+    gate_factors(0);
+  }
+  // Make tile `it` visible to the workgroup, start the copy of tile it+2, and (wave 0) prepare the gate factors of
+  // tile it+1 while the others already compute.
+  auto sync_step = [&](int it) -> char* {
     char* st = smem + (it % AT_NST) * STAGE;
     if (it + 1 < ntiles) wait_vmcnt<LOADS>(); else wait_vmcnt<0>();
-    float* graw = (float*)(st + 2 * TILE);
-    if (tid < 64) {   // wave 0 issued the gate copy, so the values are visible to it once its own counter drained
-      const int rpos = min(AT_BN - 1, a.tk - 1 - it * AT_BN);
-      const float gv = Gg ? graw[tid] : 0.f;
-      const float R_ = Gg ? graw[rpos] : 0.f, Rs = Gg ? graw[tid & ~15] : 0.f;
-      graw[AT_BN + tid] = __expf(fminf(R_ - gv, AT_EXP_CLAMP));       // relative to the tile's last key   (<= 1)
-      graw[2 * AT_BN + tid] = __expf(fminf(Rs - gv, AT_EXP_CLAMP));   // relative to the first key of its 16 (>= 1)
-      if (!Gg) graw[tid] = 0.f;
-    }
     lds_barrier();
     if (it + 2 < ntiles) issue(it + 2);
+    if (wave == 0 && it + 1 < ntiles) {
+      if (it + 2 < ntiles) wait_vmcnt<LOADS + 1>(); else wait_vmcnt<0>();   // all but the stage just issued
+      gate_factors(it + 1);
+    }
     return st;
   };
 
@@ -178,8 +221,10 @@ __global__ __launch_bounds__(256, OCC) void attention_fwd_kernel(AttnFwdArgs a) 
 #pragma unroll
     for (int mi = 0; mi < MT; mi++) {
       if (DIAG) lim[mi] = min(ti[mi], a.tk - 1) - j0 - 4 * g;   // pair (row, key 16*kt + 4g + v) visible iff 16*kt + v <= lim
-      else eu[mi] = scale_p * __expf(fminf(Gq[mi] - graw[min(AT_BN - 1, a.tk - 1 - j0)], AT_EXP_CLAMP));
+      else eu[mi] = 1.f;
     }
+    // past tiles: key factors relative to the gate at the wave's first row (<= 1 for every past key)
+    const float cw = DIAG ? 1.f : __expf(fminf(Rw - graw[AT_BN - 1], AT_EXP_CLAMP));
 #pragma unroll
     for (int kp = 0; kp < KT / 2; kp++) {
       // S^T for 32 keys: operands first, then every product, so the matrix pipe runs back to back
@@ -190,12 +235,13 @@ __global__ __launch_bounds__(256, OCC) void attention_fwd_kernel(AttnFwdArgs a) 
 #pragma unroll
         for (int ks = 0; ks < KS; ks++) kf[half][ks] = *(const lds_v8*)(kb[ks] + (2 * kp + half) * 16 * RB);
         ev[half] = *(const lds_f32x4*)(eb + 64 * (2 * kp + half));
+        if (!DIAG) ev[half] *= cw;
       }
       f32x4 sc[2][MT];
 #pragma unroll
       for (int half = 0; half < 2; half++)
 #pragma unroll
-        for (int mi = 0; mi < MT; mi++) sc[half][mi] = epsv;   // start at eps: (s + eps)^deg stands in for (|s| + eps)^deg
+        for (int mi = 0; mi < MT; mi++) sc[half][mi] = (f32x4){0, 0, 0, 0};
 #pragma unroll
       for (int ks = 0; ks < KS; ks++)
 #pragma unroll
@@ -222,7 +268,8 @@ __global__ __launch_bounds__(256, OCC) void attention_fwd_kernel(AttnFwdArgs a) 
           if (DIAG) e = scale_p * __expf(fminf(Gq[mi] - graw[16 * (2 * kp + half)], AT_EXP_CLAMP));
 #pragma unroll
           for (int v = 0; v < 4; v++) {
-            float w = pow_even<DEG2>(sc[half][mi][v], half_deg) * ev[half][v] * e;
+            float w = pow_even<DEG2>(sc[half][mi][v], eps2, half_deg) * ev[half][v];
+            if (DIAG) w *= e;
             if (DIAG) w = (32 * kp + 16 * half + v <= lim[mi]) ? w : 0.f;
             p[4 * half + v] = w;
           }
@@ -238,12 +285,23 @@ __global__ __launch_bounds__(256, OCC) void attention_fwd_kernel(AttnFwdArgs a) 
 #pragma unroll
       for (int nt = 0; nt < NT; nt++)
 #pragma unroll
-        for (int mi = 0; mi < MT; mi++) acc[mi][nt] = mfma16(vf[nt], pf[mi], acc[mi][nt]);
+        for (int mi = 0; mi < MT; mi++) {
+          acc[mi][nt] = mfma16(vf[nt], pf[mi], acc[mi][nt]);
+        }
     }
   };
 
   int it = 0;
   for (; it < n_past; it++) tile(it, sync_step(it), IC<0>{});
+  // the past tiles were accumulated without the row factor exp(G_q - Rw) * scale^deg; apply it once
+#pragma unroll
+  for (int mi = 0; mi < MT; mi++) {
+    const float f = scale_p * __expf(fminf(Gq[mi] - Rw, AT_EXP_CLAMP));
+#pragma unroll
+    for (int nt = 0; nt < NT; nt++) acc[mi][nt] *= f;
+    accl[mi] *= f;
+    mx[mi] *= f;
+  }
   for (; it < n_seen; it++) tile(it, sync_step(it), IC<1>{});
   for (; it < ntiles; it++) sync_step(it);
 
@@ -276,19 +334,17 @@ template <typename T, int DH, bool DEG2> static int attn_fwd_launch(const AttnFw
   auto go = [&](auto mt, auto occ) {
     constexpr int MT = decltype(mt)::value, OCC = decltype(occ)::value;
     constexpr size_t smem = AT_NST * (2 * AT_BN * DH * 2 + 4 * AT_BN * 4);
-    dim3 grid((rows + 64 * MT - 1) / (64 * MT), (unsigned)(B * a.h));
+    const int row_blocks = (rows + 64 * MT - 1) / (64 * MT), npairs = B * a.h;
+    dim3 grid((unsigned)(((npairs + 31) / 32) * 32 * row_blocks));
     auto kern = attention_fwd_kernel<T, DH, MT, DEG2, OCC>;
     allow_big_lds((const void*)kern, smem);
-    hipLaunchKernelGGL(kern, grid, dim3(256), smem, st, a);
+    hipLaunchKernelGGL(kern, grid, dim3(256), smem, st, a, row_blocks, npairs);
   };
-  const char* e = getenv("PR_AT_VARIANT");
-  const int var = e ? atoi(e) : 0;
-  if (var == 1 && DH <= 64) go(IC<2>{}, IC<3>{});
-  else if (var == 2 && DH <= 64) go(IC<2>{}, IC<4>{});
-  else if (var == 3 && DH <= 64) go(IC<1>{}, IC<4>{});
-  else if (var == 4 && DH <= 64) go(IC<2>{}, IC<2>{});
-  else if (DH <= 64 && rows >= 256) go(IC<4>{}, IC<2>{});
-  else if (rows > 64) go(IC<2>{}, IC<2>{});
+  constexpr bool BIG = DH <= 32 || (DH <= 64 && DEG2);   // 64 rows per wave fit the register file
+  if constexpr (BIG) {
+    if (rows >= 256) { go(IC<4>{}, IC<2>{}); return (int)hipGetLastError(); }
+  }
+  if (rows > 64) go(IC<2>{}, IC<2>{});
   else go(IC<1>{}, IC<2>{});
   return (int)hipGetLastError();
 }

@@ -27,7 +27,8 @@ def hipcc():
 
 def compile_one(name):
     obj = os.path.join(HERE, "build", name + ".o")
-    cmd = [hipcc(), *FLAGS, "-c", os.path.join(HERE, name + ".hip"), "-o", obj]
+    extra = os.environ.get("PR_HIPCC_EXTRA_FLAGS", "").split()
+    cmd = [hipcc(), *FLAGS, *extra, "-c", os.path.join(HERE, name + ".hip"), "-o", obj]
     p = subprocess.run(cmd, capture_output=True, text=True)
     err = "\n".join(l for l in p.stderr.splitlines() if "not a recognized feature" not in l)
     if p.returncode != 0:
