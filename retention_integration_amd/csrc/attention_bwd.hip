@@ -45,7 +45,7 @@ __device__ __forceinline__ void pair_grad(float s, float E, float dpl, float eps
 
 // ------------------------------------------------------------------ dQ, dGq
 template <typename T, int DH, int MT, bool DEG2>
-__global__ __launch_bounds__(256, 2) void attention_bwd_dq_kernel(AttnBwdArgs a) {
+__global__ __launch_bounds__(256, 2) void attention_bwd_dq_kernel(AttnBwdArgs a, int nblocks, int npairs) {
   typedef typename VecOf<T>::v8 v8;
   typedef typename VecOf<T>::v4 v4;
   constexpr int LD = DH + 8, KS = DH / 32, NT = DH / 16, KT = AB_BN / 16, ROWS = 64 * MT;
@@ -56,10 +56,16 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dq_kernel(AttnBwdArgs a)
   T* Vt = Kt + 2 * AB_BN * LD;
   float* gk = (float*)(Vt + 2 * AB_BN * LD);   // [2][GS]: raw gate [BN], exp(R - gate) [BN], R
 
+  // Workgroups are dealt round-robin by their linear index to the 8 XCDs and then to the 4 shader engines of an
+  // XCD; only the CU inside a shader engine is chosen by load.  Blocks differ in length (causal), so each of the 32
+  // (XCD, shader engine) groups gets whole (batch, kv head) pairs, the longest blocks of all its pairs first.
+  const int grp = blockIdx.x % 32, u = blockIdx.x / 32, ppg = (npairs + 31) / 32;
+  const int pair = (u % ppg) * 32 + grp;
+  if (pair >= npairs) return;
   const int tid = threadIdx.x, l = tid & 63, g = l >> 4, wave = tid >> 6, tcol = l & 15;
-  const int b = blockIdx.y / a.h, hh = blockIdx.y % a.h;
+  const int b = pair / a.h, hh = pair % a.h;
   const int hq = a.h * a.r, rows = a.tq * a.r, shift = a.tk - a.tq;
-  const int row0 = blockIdx.x * ROWS;
+  const int row0 = (nblocks - 1 - u / ppg) * ROWS;   // late rows see the most keys
   const T* Qg = (const T*)a.Q + (long)b * a.tq * hq * DH;
   const T* dOg = (const T*)a.dO + (long)b * a.tq * hq * DH;
   const T* Kg = (const T*)a.K + (long)b * a.tk * a.h * DH + hh * DH;
@@ -68,7 +74,7 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dq_kernel(AttnBwdArgs a)
   const long kstride = (long)a.h * DH;
   const int half_deg = (int)a.deg / 2;
   const float eps_s = AB_LOG_EPS / a.scale;
-  const float scale_p = __powf(a.scale, a.deg);
+  const float scale_p = __expf(a.deg * __logf(a.scale));
 
   v8 Qf[MT][KS], dOf[MT][KS];
   int ti[MT];
@@ -235,7 +241,7 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dq_kernel(AttnBwdArgs a)
 
 // ------------------------------------------------------------------ dK, dV, dGk
 template <typename T, int DH, int MK, bool DEG2>
-__global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a) {
+__global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a, int nblocks, int npairs) {
   typedef typename VecOf<T>::v8 v8;
   typedef typename VecOf<T>::v4 v4;
   constexpr int LD = DH + 8, KS = DH / 32, NT = DH / 16, QT = AB_BM / 16, KEYS = 64 * MK;
@@ -245,10 +251,16 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
   T* dOt = Qt + 2 * AB_BM * LD;           // [2][BM][LD]
   float* rowv = (float*)(dOt + 2 * AB_BM * LD);  // [2][5][BM]: G_q - m, dl, time index, scale^deg exp(G_q - m - R), dO scale
 
+  // Workgroups are dealt round-robin by their linear index to the 8 XCDs and then to the 4 shader engines of an
+  // XCD; only the CU inside a shader engine is chosen by load.  Blocks differ in length (causal), so each of the 32
+  // (XCD, shader engine) groups gets whole (batch, kv head) pairs, the longest blocks of all its pairs first.
+  const int grp = blockIdx.x % 32, u = blockIdx.x / 32, ppg = (npairs + 31) / 32;
+  const int pair = (u % ppg) * 32 + grp;
+  if (pair >= npairs) return;
   const int tid = threadIdx.x, l = tid & 63, g = l >> 4, wave = tid >> 6, kcol = l & 15;
-  const int b = blockIdx.y / a.h, hh = blockIdx.y % a.h;
+  const int b = pair / a.h, hh = pair % a.h;
   const int hq = a.h * a.r, rows = a.tq * a.r, shift = a.tk - a.tq;
-  const int key0 = blockIdx.x * KEYS;
+  const int key0 = (u / ppg) * KEYS;                 // early keys are seen by the most rows
   const T* Qg = (const T*)a.Q + (long)b * a.tq * hq * DH;
   const T* dOg = (const T*)a.dO + (long)b * a.tq * hq * DH;
   const T* Kg = (const T*)a.K + (long)b * a.tk * a.h * DH + hh * DH;
@@ -257,7 +269,7 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
   const long kstride = (long)a.h * DH;
   const int half_deg = (int)a.deg / 2;
   const float eps_s = AB_LOG_EPS / a.scale;
-  const float scale_p = __powf(a.scale, a.deg);
+  const float scale_p = __expf(a.deg * __logf(a.scale));
   const int last_key = min(key0 + KEYS, a.tk) - 1;
   const float R = Gg ? Gg[(long)last_key * a.h] : 0.f;   // reference gate of this key block
 
@@ -446,18 +458,20 @@ template <typename T, int DH, bool DEG2> static int attn_bwd_launch(const AttnBw
     constexpr int MT = DH <= 64 ? 2 : 1;
     constexpr size_t smem = 2 * 2 * AB_BN * (DH + 8) * sizeof(T) + 2 * (2 * AB_BN + 4) * sizeof(float);
     const int rows = a.tq * a.r;
-    dim3 grid((rows + 64 * MT - 1) / (64 * MT), (unsigned)(B * a.h));
+    const int nblocks = (rows + 64 * MT - 1) / (64 * MT), npairs = B * a.h;
+    dim3 grid((unsigned)((npairs + 31) / 32 * 32 * nblocks));
     auto kern = attention_bwd_dq_kernel<T, DH, MT, DEG2>;
     allow_big_lds((const void*)kern, smem);
-    hipLaunchKernelGGL(kern, grid, dim3(256), smem, st, a);
+    hipLaunchKernelGGL(kern, grid, dim3(256), smem, st, a, nblocks, npairs);
   }
   {
     constexpr int MK = DH <= 64 ? 2 : 1;
     constexpr size_t smem = 2 * 2 * AB_BM * (DH + 8) * sizeof(T) + 2 * 5 * AB_BM * sizeof(float);
-    dim3 grid((a.tk + 64 * MK - 1) / (64 * MK), (unsigned)(B * a.h));
+    const int nblocks = (a.tk + 64 * MK - 1) / (64 * MK), npairs = B * a.h;
+    dim3 grid((unsigned)((npairs + 31) / 32 * 32 * nblocks));
     auto kern = attention_bwd_dkv_kernel<T, DH, MK, DEG2>;
     allow_big_lds((const void*)kern, smem);
-    hipLaunchKernelGGL(kern, grid, dim3(256), smem, st, a);
+    hipLaunchKernelGGL(kern, grid, dim3(256), smem, st, a, nblocks, npairs);
   }
   return (int)hipGetLastError();
 }
