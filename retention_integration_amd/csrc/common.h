@@ -131,13 +131,19 @@ template <int N> __device__ __forceinline__ void wait_vmcnt() {
   __builtin_amdgcn_s_waitcnt((N & 0xF) | ((N >> 4) << 14) | (0x7 << 4) | (0xF << 8));
 }
 
+// The copies are written as inline assembly on purpose: the compiler tracks copies it knows about and makes every
+// later LDS read it cannot prove disjoint wait for ALL of them (vmcnt(0)), which serialises the ring.  Written
+// this way they are invisible to that tracking; completion is handled by wait_vmcnt<N>() alone, which counts
+// instructions and is therefore safe whatever other vector-memory operations the compiler interleaves.
 __device__ __forceinline__ void async_copy16(const void* gsrc, void* lds_wave_base) {
-  __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)gsrc,
-                                   (__attribute__((address_space(3))) void*)lds_wave_base, 16, 0, 0);
+  const uint32_t base = __builtin_amdgcn_readfirstlane(
+      (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)lds_wave_base);
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(base), "v"(gsrc) : "memory", "m0");
 }
 __device__ __forceinline__ void async_copy4(const void* gsrc, void* lds_wave_base) {
-  __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)gsrc,
-                                   (__attribute__((address_space(3))) void*)lds_wave_base, 4, 0, 0);
+  const uint32_t base = __builtin_amdgcn_readfirstlane(
+      (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)lds_wave_base);
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" ::"s"(base), "v"(gsrc) : "memory", "m0");
 }
 
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() also drains the vector-memory counter, which

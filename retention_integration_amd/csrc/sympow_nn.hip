@@ -9,7 +9,7 @@
 //                                                (ref: retention/_update_state/reference.py:61)
 //
 // A workgroup = 4 waves owns 64*MT rows; each wave 16*MT rows and all DV columns.  B streams through a
-// 3-deep ring of asynchronous global->LDS copies in its memory order, 64 features (four x columns of one
+// 2-deep ring of asynchronous global->LDS copies in its memory order, 64 features (four x columns of one
 // 16-wide y strip) per stage, and is read with the transposing LDS load; the phi operand is built in
 // registers from the wave's own rows (one scalar x[X] times eight x[16y+..] values per lane).
 // aux is a quadratic form, aux[row] = x_row^T M x_row with M[a, b] = sB[f(a, b)] on the stored pairs, so it
@@ -19,9 +19,10 @@
 #include "kernels.h"
 
 namespace pr {
+#define PR_STAMP(k)
 
 constexpr int NN_FR = 64;   // feature rows per stage
-constexpr int NN_NST = 3;
+constexpr int NN_NST = 2;   // two stages keep three workgroups (12 waves) resident per CU, which hides more than a deeper ring
 
 // Stage order over (strip y, first x column X0, a multiple of 4).  With the key-side multiplier the tiles
 // below the block diagonal come first so that the accumulators can be doubled once.
@@ -71,7 +72,7 @@ template <> struct PhiRow<f16_t> {
 };
 
 template <typename T, int DK, int DV, int MT, bool MULT, int EPI>
-__global__ __launch_bounds__(256, 2) void sympow_nn_kernel(NNArgs a, int row_blocks, int npairs) {
+__global__ __launch_bounds__(256, DK <= 64 ? 3 : 2) void sympow_nn_kernel(NNArgs a, int row_blocks, int npairs) {
   typedef typename VecOf<T>::v8 v8;
   typedef typename VecOf<T>::v4 v4;
   constexpr int NT = DV / 16, TT = DK / 16, KX = DK / 32, CB = DV / 8, CX = DK / 8;
@@ -79,7 +80,8 @@ __global__ __launch_bounds__(256, 2) void sympow_nn_kernel(NNArgs a, int row_blo
   constexpr int ROWS = 64 * MT, STAGE = NN_FR * DV * 2, LOADS = NN_FR * CB / 256, LDM = DK + 8;
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   char* ring = smem;                          // [NST][STAGE]; reused for M and the aux exchange at the end
-  char* xt = ring + NN_NST * STAGE;           // [ROWS][DK] T, swizzled
+  constexpr int RING_BYTES = NN_NST * STAGE > DK * LDM * 2 ? NN_NST * STAGE : DK * LDM * 2;   // the ring later holds M
+  char* xt = ring + (RING_BYTES + 1023) / 1024 * 1024;   // [ROWS][DK] T, swizzled
 
   const int xcd = blockIdx.x % 8, slot = blockIdx.x / 8;
   const int pair = (slot / row_blocks) * 8 + xcd;
@@ -124,14 +126,35 @@ __global__ __launch_bounds__(256, 2) void sympow_nn_kernel(NNArgs a, int row_blo
     cur.init(TT);
     nxt.init(TT);
     int issued = 0;
-    for (; issued < 2 && !nxt.done(); issued++) {
+    for (; issued < NN_NST - 1 && !nxt.done(); issued++) {
       issue(nxt.f0(), issued % NN_NST);
       nxt.next();
     }
     PhiRow<T> prow[MT];
     int y_loaded = -1, step = 0;
+    // Per-lane LDS byte addresses, hoisted out of the stage loop.  The swizzle of a row depends only on the row's
+    // position inside its group of 16 (8 for the transposing read), so a stage adds a scalar base and the
+    // displacements inside a stage are immediate offsets.
+    typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+    typedef __attribute__((address_space(3))) char lds_char;
+    typedef __attribute__((address_space(3))) unsigned short lds_u16;
+    const uint32_t ring_a = (uint32_t)(uintptr_t)(lds_char*)ring, xt_a = (uint32_t)(uintptr_t)(lds_char*)xt;
+    uint32_t boff[NT][2];      // B^T operand: rows 8g + (s>>2) (+4), columns 16*nt + 4*(s&3) ..
+#pragma unroll
+    for (int nt = 0; nt < NT; nt++)
+#pragma unroll
+      for (int hf = 0; hf < 2; hf++) {
+        const int row = 8 * g + 4 * hf + (tcol >> 2), col = 16 * nt + 4 * (tcol & 3);
+        boff[nt][hf] = row * (CB * 16) + (((col / 8) ^ swz<CB>(row)) * 16) + (col % 8) * 2;
+      }
+    uint32_t xrow_a[MT], xsw[MT];   // start of this lane's row of the X tile (+ the lane's column parity), its swizzle
+#pragma unroll
+    for (int mi = 0; mi < MT; mi++) {
+      const int lrow = wave * 16 * MT + 16 * mi + tcol;
+      xrow_a[mi] = xt_a + lrow * (DK * 2) + 2 * (g >> 1);
+      xsw[mi] = swz<CX>(lrow);
+    }
     while (!cur.done()) {
-      const char* st = ring + (step % NN_NST) * STAGE;
       if (issued > step + 1) wait_vmcnt<LOADS>(); else wait_vmcnt<0>();
       lds_barrier();
       if (!nxt.done()) {
@@ -144,14 +167,32 @@ __global__ __launch_bounds__(256, 2) void sympow_nn_kernel(NNArgs a, int row_blo
 #pragma unroll
         for (int mi = 0; mi < MT; mi++) prow[mi].load(x_ptr(wave * 16 * MT + 16 * mi + tcol, 16 * cur.y + 8 * (g & 1)));
       }
+      uint32_t ba[NT][2], xa[MT];
+      {
+        const uint32_t sa = ring_a + (step % NN_NST) * STAGE;
+#pragma unroll
+        for (int nt = 0; nt < NT; nt++)
+#pragma unroll
+          for (int hf = 0; hf < 2; hf++) { ba[nt][hf] = sa + boff[nt][hf]; asm volatile("" : "+v"(ba[nt][hf])); }
+        // x[row, X0 + 2*ks + parity]: X0 is a multiple of 4, so the 16-byte chunk is X0/8 and the rest is immediate
+        const int xc = cur.X0 >> 3, xo = (cur.X0 & 7) * 2;
+#pragma unroll
+        for (int mi = 0; mi < MT; mi++) { xa[mi] = xrow_a[mi] + ((xc ^ xsw[mi]) << 4) + xo; asm volatile("" : "+v"(xa[mi])); }
+      }
 #pragma unroll
       for (int ks = 0; ks < NN_FR / 32; ks++) {
         v8 vf[NT];
 #pragma unroll
-        for (int nt = 0; nt < NT; nt++) vf[nt] = sw_frag_tr<T, CB>(st, 32 * ks, 16 * nt);
+        for (int nt = 0; nt < NT; nt++) {
+          const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(ba[nt][0] + ks * 32 * (CB * 16)));
+          const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(ba[nt][1] + ks * 32 * (CB * 16)));
+          const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+          vf[nt] = __builtin_bit_cast(v8, both);
+        }
 #pragma unroll
         for (int mi = 0; mi < MT; mi++) {
-          const T xs = *(const T*)x_ptr(wave * 16 * MT + 16 * mi + tcol, cur.X0 + 2 * ks + (g >> 1));
+          const unsigned short xbits = *(const lds_u16*)(xa[mi] + 4 * ks);
+          const T xs = __builtin_bit_cast(T, xbits);
           const v8 af = prow[mi].make(xs);
 #pragma unroll
           for (int nt = 0; nt < NT; nt++) acc[mi][nt] = mfma16(af, vf[nt], acc[mi][nt]);
@@ -265,15 +306,17 @@ template <typename T, int DK, int DV, bool MULT, int EPI> static int nn_launch(c
   auto go = [&](auto mt) {
     constexpr int MT = decltype(mt)::value;
     constexpr size_t ring = NN_NST * NN_FR * DV * 2, mtile = (size_t)DK * (DK + 8) * 2;
-    constexpr size_t smem = (ring > mtile ? ring : mtile) + 64 * MT * DK * 2;
+    constexpr size_t smem = ((ring > mtile ? ring : mtile) + 1023) / 1024 * 1024 + 64 * MT * DK * 2;
     const int row_blocks = (rows + 64 * MT - 1) / (64 * MT);
     dim3 grid((unsigned)(((npairs + 7) / 8) * 8 * row_blocks));
     auto kern = sympow_nn_kernel<T, DK, DV, MT, MULT, EPI>;
     allow_big_lds((const void*)kern, smem);
     hipLaunchKernelGGL(kern, grid, dim3(256), smem, st, a, row_blocks, npairs);
   };
-  if (DK <= 64 && rows >= 256) go(IC<4>{});
-  else if (rows > 64) go(IC<2>{});
+  if constexpr (DK <= 64) {
+    if (rows >= 256) { go(IC<4>{}); return (int)hipGetLastError(); }
+  }
+  if (rows > 64) go(IC<2>{});
   else go(IC<1>{});
   return (int)hipGetLastError();
 }
