@@ -6,41 +6,45 @@
 //   dGq_i = sum_j dz_ij,  dGk_j = -sum_i dz_ij,
 //   d(q.k) = dz * deg * sign(s) / (|q.k| + 1e-7/scale),  dQ = d(q.k) K,  dK = d(q.k)^T Q.
 //
-// Two kernels, each recomputing P: one owns query rows and walks the keys (dQ, dGq), the other owns keys
-// and walks the query rows (dK, dV, dGk).  Products are oriented so that every accumulator layout is
-// already the operand layout of the next contraction (see attention_fwd.hip).
+// Two kernels, each recomputing P: one owns query rows and walks the keys (dQ, dGq), the other owns keys and walks
+// the query rows (dK, dV, dGk).  Products are oriented so that every accumulator layout is already the operand
+// layout of the next contraction (see attention_fwd.hip), and the streamed operand goes through a 3-deep ring of
+// asynchronous global->LDS copies.
 //
-// No logarithm or division per pair: with a = |q.k| + eps/scale,
-//   P = a^deg * E,  E = scale^deg * exp(G_q - m - G_k),  d(q.k)/deg = sign(s) * a^(deg-1) * E * dP,
-// and away from the diagonal E factors into a per-row and a per-key exponential around a reference
-// gate R (the gate at the last key of the key tile, so both exponents are <= 0 for decaying gates).
+// No logarithm or division per pair.  As in the forward, a2 = (q.k)^2 + (eps/scale)^2 stands in for
+// (|q.k| + eps/scale)^2, so P = a2^(deg/2) * E with E = scale^deg * exp(G_q - m - G_k), and
+//   d(q.k)/deg = (q.k) * a2^(deg/2 - 1) * E * dP,      dz = a2^(deg/2) * E * dP.
+// E is split into a per-row and a per-key exponential around a reference gate chosen so that both stay in range:
+// pairs well off the diagonal share one reference per wave or workgroup and the factor that is constant along the
+// accumulation (per row for dQ, per key for dK/dV) is applied once to the accumulators; pairs near the diagonal
+// use a reference per group of 16 keys and are masked per pair.
 #include "common.h"
 #include "kernels.h"
 
 namespace pr {
 
-constexpr int AB_BN = 64;   // keys per step in the dQ kernel
-constexpr int AB_BM = 32;   // query rows per step in the dK/dV kernel
+constexpr int AB_BN = 64;    // keys per stage in the dQ kernel
+constexpr int AB_BM = 64;    // query rows per stage in the dK/dV kernel
+constexpr int AB_NST = 3;
 constexpr float AB_LOG_EPS = 1e-7f, AB_EXP_CLAMP = 80.f;
 
-// a^(deg-2) for even deg
-template <bool DEG2> __device__ __forceinline__ float pow_m2(float a, int half_deg) {
+// a2^(half_deg - 1)
+template <bool DEG2> __device__ __forceinline__ float pow_hm1(float a2, int half_deg) {
   if (DEG2) return 1.f;
-  const float a2 = a * a;
   float p = 1.f;
   for (int k = 1; k < half_deg; k++) p *= a2;
   return p;
 }
 
-// One pair: s = raw q.k, E as above, dpl = dP (incl. dl).  Returns P, dz and d(q.k)/deg.
-template <bool DEG2>
-__device__ __forceinline__ void pair_grad(float s, float E, float dpl, float eps_s, int half_deg, float& p, float& dz,
-                                          float& dsr) {
-  const float as = fabsf(s) + eps_s;
-  const float t1 = pow_m2<DEG2>(as, half_deg) * as * E;   // a^(deg-1) E
-  p = t1 * as;
-  dz = p * dpl;
-  dsr = copysignf(t1, s) * dpl;
+typedef __attribute__((address_space(3))) s16x4 ab_lds_s16x4;
+typedef __attribute__((address_space(3))) f32x4 ab_lds_f32x4;
+typedef __attribute__((address_space(3))) char ab_lds_char;
+
+template <typename T> __device__ __forceinline__ typename VecOf<T>::v8 ab_tr8(uint32_t lo_addr, uint32_t hi_addr) {
+  const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((ab_lds_s16x4*)lo_addr);
+  const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((ab_lds_s16x4*)hi_addr);
+  const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+  return __builtin_bit_cast(typename VecOf<T>::v8, both);
 }
 
 // ------------------------------------------------------------------ dQ, dGq
@@ -48,13 +52,12 @@ template <typename T, int DH, int MT, bool DEG2>
 __global__ __launch_bounds__(256, 2) void attention_bwd_dq_kernel(AttnBwdArgs a, int nblocks, int npairs) {
   typedef typename VecOf<T>::v8 v8;
   typedef typename VecOf<T>::v4 v4;
-  constexpr int LD = DH + 8, KS = DH / 32, NT = DH / 16, KT = AB_BN / 16, ROWS = 64 * MT;
-  constexpr int CH = AB_BN * DH / 8, PT = (CH + 255) / 256;
-  constexpr int GS = 2 * AB_BN + 4;
-  extern __shared__ __attribute__((aligned(16))) char smem[];
-  T* Kt = (T*)smem;
-  T* Vt = Kt + 2 * AB_BN * LD;
-  float* gk = (float*)(Vt + 2 * AB_BN * LD);   // [2][GS]: raw gate [BN], exp(R - gate) [BN], R
+  typedef __attribute__((address_space(3))) v8 lds_v8;
+  constexpr int KS = DH / 32, NT = DH / 16, KT = AB_BN / 16, ROWS = 64 * MT, CPR = DH / 8, RB = CPR * 16;
+  constexpr int TILE = AB_BN * RB;
+  constexpr int STAGE = 2 * TILE + 4 * AB_BN * 4;   // K, V, raw gates, two sets of key gate factors
+  constexpr int LOADS = 2 * AB_BN * CPR / 256;
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
 
   // Workgroups are dealt round-robin by their linear index to the 8 XCDs and then to the 4 shader engines of an
   // XCD; only the CU inside a shader engine is chosen by load.  Blocks differ in length (causal), so each of the 32
@@ -62,19 +65,53 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dq_kernel(AttnBwdArgs a,
   const int grp = blockIdx.x % 32, u = blockIdx.x / 32, ppg = (npairs + 31) / 32;
   const int pair = (u % ppg) * 32 + grp;
   if (pair >= npairs) return;
-  const int tid = threadIdx.x, l = tid & 63, g = l >> 4, wave = tid >> 6, tcol = l & 15;
+  const int tid = threadIdx.x, l = tid & 63, g = l >> 4, tcol = l & 15;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int b = pair / a.h, hh = pair % a.h;
   const int hq = a.h * a.r, rows = a.tq * a.r, shift = a.tk - a.tq;
   const int row0 = (nblocks - 1 - u / ppg) * ROWS;   // late rows see the most keys
   const T* Qg = (const T*)a.Q + (long)b * a.tq * hq * DH;
   const T* dOg = (const T*)a.dO + (long)b * a.tq * hq * DH;
-  const T* Kg = (const T*)a.K + (long)b * a.tk * a.h * DH + hh * DH;
-  const T* Vg = (const T*)a.V + (long)b * a.tk * a.h * DH + hh * DH;
+  const char* Kg = (const char*)((const T*)a.K + (long)b * a.tk * a.h * DH + hh * DH);
+  const char* Vg = (const char*)((const T*)a.V + (long)b * a.tk * a.h * DH + hh * DH);
   const float* Gg = a.G ? a.G + (long)b * a.tk * a.h + hh : nullptr;
-  const long kstride = (long)a.h * DH;
+  const long kstride = (long)a.h * DH * 2;
   const int half_deg = (int)a.deg / 2;
-  const float eps_s = AB_LOG_EPS / a.scale;
+  const float eps_s = AB_LOG_EPS / a.scale, eps2 = eps_s * eps_s;
   const float scale_p = __expf(a.deg * __logf(a.scale));
+
+  const int last_row = min(row0 + ROWS, rows) - 1;
+  const int kmax = min(a.tk, last_row / a.r + shift + 1);
+  const int ntiles = (kmax + AB_BN - 1) / AB_BN;
+  const int wslice = (u & 1) ? 3 - wave : wave;   // alternate which wave is nearest the diagonal
+  const int wrow0 = row0 + wslice * 16 * MT;
+  const int w_first_ti = min(wrow0, rows - 1) / a.r + shift;
+  const int w_last_ti = min(wrow0 + 16 * MT - 1, rows - 1) / a.r + shift;
+
+  uint32_t goff[LOADS / 2];
+#pragma unroll
+  for (int ii = 0; ii < LOADS / 2; ii++) {
+    const int pos = (ii * 4 + wave) * 64 + l, row = pos / CPR;
+    goff[ii] = (uint32_t)(row * (int)kstride + 16 * ((pos % CPR) ^ swz<CPR>(row)));
+  }
+  auto issue = [&](int it) {
+    char* st = smem + (it % AB_NST) * STAGE;
+    const int j0 = it * AB_BN;
+    if (j0 + AB_BN <= a.tk) {
+      const char* kb_ = Kg + (long)j0 * kstride;
+      const char* vb_ = Vg + (long)j0 * kstride;
+#pragma unroll
+      for (int ii = 0; ii < LOADS / 2; ii++) async_copy16(kb_ + goff[ii], st + (ii * 4 + wave) * 1024);
+#pragma unroll
+      for (int ii = 0; ii < LOADS / 2; ii++) async_copy16(vb_ + goff[ii], st + TILE + (ii * 4 + wave) * 1024);
+    } else {   // last, partial tile: rows past the end repeat the last key (they are masked)
+      async_load_tile<CPR, AB_BN>(st, [&](int row) { return Kg + (long)min(j0 + row, a.tk - 1) * kstride; });
+      async_load_tile<CPR, AB_BN>(st + TILE, [&](int row) { return Vg + (long)min(j0 + row, a.tk - 1) * kstride; });
+    }
+    if (Gg && wave == 0) async_copy4(Gg + (long)min(j0 + l, a.tk - 1) * a.h, st + 2 * TILE);
+  };
+  issue(0);
+  if (ntiles > 1) issue(1);
 
   v8 Qf[MT][KS], dOf[MT][KS];
   int ti[MT];
@@ -83,7 +120,7 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dq_kernel(AttnBwdArgs a,
   float base[MT], dlr[MT], dgq[MT], osc[MT];   // base = G_q - m
 #pragma unroll
   for (int mi = 0; mi < MT; mi++) {
-    const int row = row0 + wave * 16 * MT + 16 * mi + tcol;
+    const int row = wrow0 + 16 * mi + tcol;
     live[mi] = row < rows;
     const int rr = live[mi] ? row : 0;
     const int t = rr / a.r;
@@ -105,123 +142,161 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dq_kernel(AttnBwdArgs a,
     osc[mi] = a.dO_scale ? a.dO_scale[so] : 1.f;
     dgq[mi] = 0.f;
   }
+  const float Rw = Gg ? Gg[(long)w_first_ti * a.h] : 0.f;   // gate at the wave's first row
   f32x4 acc[MT][NT];
 #pragma unroll
   for (int mi = 0; mi < MT; mi++)
 #pragma unroll
     for (int nt = 0; nt < NT; nt++) acc[mi][nt] = (f32x4){0, 0, 0, 0};
 
-  const int last_row = min(row0 + ROWS, rows) - 1;
-  const int kmax = min(a.tk, last_row / a.r + shift + 1);
-  const int first_ti = row0 / a.r + shift;
-  const int ntiles = (kmax + AB_BN - 1) / AB_BN;
-
-  u32x4 rk[PT], rv[PT];
-  float rg = 0.f, rR = 0.f;
-  auto fetch = [&](int j0) {
+  // per-lane LDS byte offsets inside a tile (the swizzle depends only on the row inside a 16-row group)
+  int koff[KS], toff[NT];
 #pragma unroll
-    for (int i = 0; i < PT; i++) {
-      const int ch = tid + 256 * i;
-      const int key = j0 + ch / (DH / 8), col = (ch % (DH / 8)) * 8;
-      rk[i] = (u32x4){0, 0, 0, 0};
-      rv[i] = (u32x4){0, 0, 0, 0};
-      if (ch < CH && key < a.tk) {
-        rk[i] = *(const u32x4*)(Kg + key * kstride + col);
-        rv[i] = *(const u32x4*)(Vg + key * kstride + col);
-      }
-    }
-    if (tid < AB_BN && Gg) {
-      rg = Gg[(long)min(j0 + tid, a.tk - 1) * a.h];
-      rR = Gg[(long)min(j0 + AB_BN - 1, a.tk - 1) * a.h];
-    }
-  };
-  auto stash = [&](int stage) {
+  for (int ks = 0; ks < KS; ks++) koff[ks] = tcol * RB + (((4 * ks + g) ^ swz<CPR>(tcol)) * 16);
+  {
+    const int vr = 4 * g + (tcol >> 2);
 #pragma unroll
-    for (int i = 0; i < PT; i++) {
-      const int ch = tid + 256 * i;
-      if (ch < CH) {
-        const int o = stage * AB_BN * LD + (ch / (DH / 8)) * LD + (ch % (DH / 8)) * 8;
-        *(u32x4*)(Kt + o) = rk[i];
-        *(u32x4*)(Vt + o) = rv[i];
-      }
-    }
-    if (tid < AB_BN) {
-      gk[stage * GS + tid] = rg;
-      gk[stage * GS + AB_BN + tid] = __expf(fminf(rR - rg, AB_EXP_CLAMP));
-      if (tid == 0) gk[stage * GS + 2 * AB_BN] = rR;
-    }
-  };
-
-  fetch(0);
-  for (int it = 0; it < ntiles; it++) {
-    const int j0 = it * AB_BN, stage = it & 1;
-    stash(stage);
-    lds_barrier();
-    if (it + 1 < ntiles) fetch(j0 + AB_BN);
-    const T* kt_ = Kt + stage * AB_BN * LD;
-    const T* vt_ = Vt + stage * AB_BN * LD;
-    const float* gk_ = gk + stage * GS;
-    const bool diag = (j0 + AB_BN - 1 > first_ti) || (j0 + AB_BN > a.tk);
-    const float R = gk_[2 * AB_BN];
-    float eu[MT];
-#pragma unroll
-    for (int mi = 0; mi < MT; mi++) eu[mi] = scale_p * (diag ? 1.f : __expf(fminf(base[mi] - R, AB_EXP_CLAMP)));
-
-    v8 dsf[MT][KT / 2];
-#pragma unroll
-    for (int kp = 0; kp < KT / 2; kp++) {
-      float d8[MT][8];
-#pragma unroll
-      for (int half = 0; half < 2; half++) {
-        const int kt = 2 * kp + half;
-        v8 kf[KS], vf[KS];
-#pragma unroll
-        for (int ks = 0; ks < KS; ks++) {
-          kf[ks] = lds_frag<T>(kt_, LD, 16 * kt, 32 * ks);
-          vf[ks] = lds_frag<T>(vt_, LD, 16 * kt, 32 * ks);
-        }
-        const f32x4 gkv = *(const f32x4*)(gk_ + (diag ? 0 : AB_BN) + 16 * kt + 4 * g);
-#pragma unroll
-        for (int mi = 0; mi < MT; mi++) {
-          f32x4 s = {0, 0, 0, 0}, dp = {0, 0, 0, 0};
-#pragma unroll
-          for (int ks = 0; ks < KS; ks++) {
-            s = mfma16(kf[ks], Qf[mi][ks], s);
-            dp = mfma16(vf[ks], dOf[mi][ks], dp);
-          }
-#pragma unroll
-          for (int v = 0; v < 4; v++) {
-            float E;
-            if (diag) {
-              const int key = j0 + 16 * kt + 4 * g + v;
-              E = eu[mi] * __expf(fminf(base[mi] - gkv[v], AB_EXP_CLAMP));
-              if (key > ti[mi] || key >= a.tk) E = 0.f;
-            } else {
-              E = eu[mi] * gkv[v];
-            }
-            float p, dz, dsr;
-            pair_grad<DEG2>(s[v], E, dp[v] * osc[mi] + dlr[mi], eps_s, half_deg, p, dz, dsr);
-            dgq[mi] += dz;
-            d8[mi][4 * half + v] = dsr;
-          }
-        }
-      }
-#pragma unroll
-      for (int mi = 0; mi < MT; mi++) dsf[mi][kp] = pack8<T>(d8[mi]);
-    }
-    // dQ^T[d, row] += K^T[d, key] dsr^T[key, row]
-#pragma unroll
-    for (int kp = 0; kp < KT / 2; kp++) {
-#pragma unroll
-      for (int nt = 0; nt < NT; nt++) {
-        v4 lo = lds_frag_tr4<T>(kt_, LD, 32 * kp + 4 * g, 16 * nt);
-        v4 hi = lds_frag_tr4<T>(kt_, LD, 32 * kp + 16 + 4 * g, 16 * nt);
-        v8 kT = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-#pragma unroll
-        for (int mi = 0; mi < MT; mi++) acc[mi][nt] = mfma16(kT, dsf[mi][kp], acc[mi][nt]);
-      }
+    for (int nt = 0; nt < NT; nt++) {
+      const int col = 16 * nt + 4 * (tcol & 3);
+      toff[nt] = vr * RB + (((col / 8) ^ swz<CPR>(vr)) * 16) + (col % 8) * 2;
     }
   }
+
+  const int n_past = min(ntiles, min(w_first_ti + 1, a.tk) / AB_BN);   // tiles with every pair visible
+  const int n_seen = min(ntiles, w_last_ti / AB_BN + 1);               // tiles with at least one visible pair
+
+  // exp(R - gate) relative to the tile's last key (<= 1) and to the first key of each 16-key group (>= 1);
+  // written by wave 0, which issued the gate copy and so is the one that can wait for it
+  auto gate_factors = [&](int it) {
+    float* graw = (float*)(smem + (it % AB_NST) * STAGE + 2 * TILE);
+    const int rpos = min(AB_BN - 1, a.tk - 1 - it * AB_BN);
+    const float gv = Gg ? graw[l] : 0.f;
+    const float R_ = Gg ? graw[rpos] : 0.f, Rs = Gg ? graw[l & ~15] : 0.f;
+    graw[AB_BN + l] = __expf(fminf(R_ - gv, AB_EXP_CLAMP));
+    graw[2 * AB_BN + l] = __expf(fminf(Rs - gv, AB_EXP_CLAMP));
+    if (!Gg) graw[l] = 0.f;
+  };
+  if (wave == 0) {
+    wait_vmcnt<0>();
+    gate_factors(0);
+  }
+  auto sync_step = [&](int it) -> char* {
+    char* st = smem + (it % AB_NST) * STAGE;
+    if (it + 1 < ntiles) wait_vmcnt<LOADS>(); else wait_vmcnt<0>();
+    lds_barrier();
+    if (it + 2 < ntiles) issue(it + 2);
+    if (wave == 0 && it + 1 < ntiles) {
+      if (it + 2 < ntiles) wait_vmcnt<LOADS + 1>(); else wait_vmcnt<0>();   // all but the stage just issued
+      gate_factors(it + 1);
+    }
+    return st;
+  };
+
+  // One 64-key tile.  Past tiles: key factors relative to the gate at the wave's first row (<= 1), the row factor
+  // is applied to the accumulators after the past tiles.  Diagonal tiles: per-group reference, per-pair mask.
+  auto tile = [&](int it, const char* st, auto diag_c) {
+    constexpr bool DIAG = decltype(diag_c)::value != 0;
+    const int j0 = it * AB_BN;
+    const float* graw = (const float*)(st + 2 * TILE);
+    uint32_t kb[KS], vb[KS], tb[NT], eb;
+    {
+      const uint32_t sa = (uint32_t)(uintptr_t)(ab_lds_char*)st;
+#pragma unroll
+      for (int ks = 0; ks < KS; ks++) {
+        kb[ks] = sa + koff[ks];
+        vb[ks] = sa + TILE + koff[ks];
+        asm volatile("" : "+v"(kb[ks]));
+        asm volatile("" : "+v"(vb[ks]));
+      }
+#pragma unroll
+      for (int nt = 0; nt < NT; nt++) { tb[nt] = sa + toff[nt]; asm volatile("" : "+v"(tb[nt])); }
+      eb = sa + 2 * TILE + (DIAG ? 2 * AB_BN : AB_BN) * 4 + 16 * g;
+      asm volatile("" : "+v"(eb));
+    }
+    int lim[MT];
+#pragma unroll
+    for (int mi = 0; mi < MT; mi++) lim[mi] = DIAG ? min(ti[mi], a.tk - 1) - j0 - 4 * g : 0;
+    const float cw = DIAG ? 1.f : __expf(fminf(Rw - graw[AB_BN - 1], AB_EXP_CLAMP));
+#pragma unroll
+    for (int kp = 0; kp < KT / 2; kp++) {
+      v8 kf[2][KS], vf[2][KS];
+      f32x4 ev[2];
+#pragma unroll
+      for (int half = 0; half < 2; half++) {
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) {
+          kf[half][ks] = *(const lds_v8*)(kb[ks] + (2 * kp + half) * 16 * RB);
+          vf[half][ks] = *(const lds_v8*)(vb[ks] + (2 * kp + half) * 16 * RB);
+        }
+        ev[half] = *(const ab_lds_f32x4*)(eb + 64 * (2 * kp + half));
+        if (!DIAG) ev[half] *= cw;
+      }
+      f32x4 sc[2][MT], dp[2][MT];
+#pragma unroll
+      for (int half = 0; half < 2; half++)
+#pragma unroll
+        for (int mi = 0; mi < MT; mi++) {
+          sc[half][mi] = (f32x4){0, 0, 0, 0};
+          dp[half][mi] = (f32x4){0, 0, 0, 0};
+        }
+#pragma unroll
+      for (int ks = 0; ks < KS; ks++)
+#pragma unroll
+        for (int half = 0; half < 2; half++)
+#pragma unroll
+          for (int mi = 0; mi < MT; mi++) {
+            sc[half][mi] = mfma16(kf[half][ks], Qf[mi][ks], sc[half][mi]);
+            dp[half][mi] = mfma16(vf[half][ks], dOf[mi][ks], dp[half][mi]);
+          }
+      // K^T operands for the same 32 keys, in flight while the pair gradients are formed
+      v8 kT[NT];
+#pragma unroll
+      for (int nt = 0; nt < NT; nt++) kT[nt] = ab_tr8<T>(tb[nt] + kp * 32 * RB, tb[nt] + kp * 32 * RB + 16 * RB);
+      v8 dsf[MT];
+#pragma unroll
+      for (int mi = 0; mi < MT; mi++) {
+        float d8[8];
+#pragma unroll
+        for (int half = 0; half < 2; half++) {
+          float e = 1.f;
+          if (DIAG) e = scale_p * __expf(fminf(base[mi] - graw[16 * (2 * kp + half)], AB_EXP_CLAMP));
+#pragma unroll
+          for (int v = 0; v < 4; v++) {
+            const float s = sc[half][mi][v];
+            const float dpl = __builtin_fmaf(dp[half][mi][v], osc[mi], dlr[mi]);
+            float q = ev[half][v] * dpl;                       // E * dP without the row factor
+            if (!DEG2) q *= pow_hm1<DEG2>(__builtin_fmaf(s, s, eps2), half_deg);
+            if (DIAG) {
+              q *= e;
+              q = (32 * kp + 16 * half + v <= lim[mi]) ? q : 0.f;
+            }
+            const float dsr = s * q;
+            dgq[mi] = DEG2 ? __builtin_fmaf(s, dsr, dgq[mi]) : __builtin_fmaf(__builtin_fmaf(s, s, eps2), q, dgq[mi]);
+            d8[4 * half + v] = dsr;
+          }
+        }
+        dsf[mi] = pack8<T>(d8);
+      }
+      // dQ^T[d, row] += K^T[d, key] dsr^T[key, row]
+#pragma unroll
+      for (int nt = 0; nt < NT; nt++)
+#pragma unroll
+        for (int mi = 0; mi < MT; mi++) acc[mi][nt] = mfma16(kT[nt], dsf[mi], acc[mi][nt]);
+    }
+  };
+
+  int it = 0;
+  for (; it < n_past; it++) tile(it, sync_step(it), IC<0>{});
+  // the past tiles were accumulated without the row factor scale^deg * exp(G_q - m - Rw); apply it once
+#pragma unroll
+  for (int mi = 0; mi < MT; mi++) {
+    const float f = scale_p * __expf(fminf(base[mi] - Rw, AB_EXP_CLAMP));
+#pragma unroll
+    for (int nt = 0; nt < NT; nt++) acc[mi][nt] *= f;
+    dgq[mi] *= f;
+  }
+  for (; it < n_seen; it++) tile(it, sync_step(it), IC<1>{});
+  for (; it < ntiles; it++) sync_step(it);
 
   T* dQg = (T*)a.dQ + (long)b * a.tq * hq * DH;
 #pragma unroll
@@ -240,47 +315,107 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dq_kernel(AttnBwdArgs a,
 }
 
 // ------------------------------------------------------------------ dK, dV, dGk
+// A workgroup owns 64*MK keys (16*MK per wave, keys on the lanes) and walks the query-row tiles that can see them
+// from the LAST row tile down to the tiles on its diagonal.  Far tiles (every row after every key of the workgroup)
+// use one reference gate R for the workgroup: the row factors scale^deg exp(G_q - m - R) (times the dO scale and
+// times dl) are prepared once per tile in LDS, and the key factor exp(R - G_k) <= 1 is applied to the accumulators
+// once after the far tiles; the tiles near the diagonal then add absolute terms (reference: last key of each 16).
 template <typename T, int DH, int MK, bool DEG2>
 __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a, int nblocks, int npairs) {
   typedef typename VecOf<T>::v8 v8;
   typedef typename VecOf<T>::v4 v4;
-  constexpr int LD = DH + 8, KS = DH / 32, NT = DH / 16, QT = AB_BM / 16, KEYS = 64 * MK;
-  constexpr int CH = AB_BM * DH / 8, PT = (CH + 255) / 256;
-  extern __shared__ __attribute__((aligned(16))) char smem[];
-  T* Qt = (T*)smem;                       // [2][BM][LD]
-  T* dOt = Qt + 2 * AB_BM * LD;           // [2][BM][LD]
-  float* rowv = (float*)(dOt + 2 * AB_BM * LD);  // [2][5][BM]: G_q - m, dl, time index, scale^deg exp(G_q - m - R), dO scale
+  typedef __attribute__((address_space(3))) v8 lds_v8;
+  constexpr int KS = DH / 32, NT = DH / 16, QT = AB_BM / 16, KEYS = 64 * MK, CPR = DH / 8, RB = CPR * 16;
+  constexpr int TILE = AB_BM * RB;
+  // row vectors of a stage, AB_BM floats each: [0] G_q (raw) -> G_q - m, [1] m (raw) -> time index (as a float),
+  // [2] dl, [3] dO scale, [4] far-tile factor * dO scale, [5] far-tile factor * dl
+  constexpr int NV = 6;
+  constexpr int STAGE = 2 * TILE + NV * AB_BM * 4;
+  constexpr int LOADS = 2 * AB_BM * CPR / 256;
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
 
-  // Workgroups are dealt round-robin by their linear index to the 8 XCDs and then to the 4 shader engines of an
-  // XCD; only the CU inside a shader engine is chosen by load.  Blocks differ in length (causal), so each of the 32
-  // (XCD, shader engine) groups gets whole (batch, kv head) pairs, the longest blocks of all its pairs first.
   const int grp = blockIdx.x % 32, u = blockIdx.x / 32, ppg = (npairs + 31) / 32;
   const int pair = (u % ppg) * 32 + grp;
   if (pair >= npairs) return;
-  const int tid = threadIdx.x, l = tid & 63, g = l >> 4, wave = tid >> 6, kcol = l & 15;
+  const int tid = threadIdx.x, l = tid & 63, g = l >> 4, kcol = l & 15;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int b = pair / a.h, hh = pair % a.h;
   const int hq = a.h * a.r, rows = a.tq * a.r, shift = a.tk - a.tq;
   const int key0 = (u / ppg) * KEYS;                 // early keys are seen by the most rows
-  const T* Qg = (const T*)a.Q + (long)b * a.tq * hq * DH;
-  const T* dOg = (const T*)a.dO + (long)b * a.tq * hq * DH;
+  const char* Qg = (const char*)((const T*)a.Q + (long)b * a.tq * hq * DH);
+  const char* dOg = (const char*)((const T*)a.dO + (long)b * a.tq * hq * DH);
   const T* Kg = (const T*)a.K + (long)b * a.tk * a.h * DH + hh * DH;
   const T* Vg = (const T*)a.V + (long)b * a.tk * a.h * DH + hh * DH;
   const float* Gg = a.G ? a.G + (long)b * a.tk * a.h + hh : nullptr;
+  const float* rmg = a.rowmax + (long)b * a.tq * hq;
+  const float* dlg = a.dl ? a.dl + (long)b * a.tq * hq : nullptr;
+  const float* osg = a.dO_scale ? a.dO_scale + (long)b * a.tq * hq : nullptr;
   const long kstride = (long)a.h * DH;
   const int half_deg = (int)a.deg / 2;
-  const float eps_s = AB_LOG_EPS / a.scale;
+  const float eps_s = AB_LOG_EPS / a.scale, eps2 = eps_s * eps_s;
   const float scale_p = __expf(a.deg * __logf(a.scale));
   const int last_key = min(key0 + KEYS, a.tk) - 1;
-  const float R = Gg ? Gg[(long)last_key * a.h] : 0.f;   // reference gate of this key block
+  const float Rblk = Gg ? Gg[(long)last_key * a.h] : 0.f;   // reference gate of the workgroup's far tiles
+
+  const int wslice = (u & 1) ? 3 - wave : wave;
+  const int wkey0 = key0 + wslice * 16 * MK;
+
+  // row tiles, walked downwards from the last one
+  const int ntile_total = (rows + AB_BM - 1) / AB_BM;
+  const int tile_lo = max(0, (key0 - shift) * a.r) / AB_BM;               // first tile that sees any key of the block
+  const int nsteps = max(0, ntile_total - tile_lo);
+  // far tiles: every row's time index >= last_key  <=>  tile >= ceil((last_key - shift) * r / BM)
+  const int tile_far = max(tile_lo, (max(0, (last_key - shift) * a.r) + AB_BM - 1) / AB_BM);
+  const int n_far = max(0, ntile_total - tile_far);
+  // tiles with at least one row that sees the wave's first key
+  const int tile_w = max(tile_lo, max(0, (wkey0 - shift) * a.r) / AB_BM);
+  const int n_seen = max(n_far, ntile_total - tile_w);
+
+  // copies of one stage
+  uint32_t grow[LOADS / 2], gchk[LOADS / 2];   // row inside the tile and byte offset of the 16-byte chunk in its row
+#pragma unroll
+  for (int ii = 0; ii < LOADS / 2; ii++) {
+    const int pos = (ii * 4 + wave) * 64 + l, row = pos / CPR;
+    grow[ii] = row;
+    gchk[ii] = 16 * ((pos % CPR) ^ swz<CPR>(row));
+  }
+  auto row_elem = [&](int row) -> long {   // element offset of a (clamped) folded row in a [tq, hq] array
+    row = min(row, rows - 1);
+    const int t = row / a.r;
+    return (long)t * hq + hh * a.r + (row - t * a.r);
+  };
+  auto issue = [&](int step) {
+    char* st = smem + (step % AB_NST) * STAGE;
+    const int rbase = (ntile_total - 1 - step) * AB_BM;
+#pragma unroll
+    for (int ii = 0; ii < LOADS / 2; ii++) {
+      const long ro = row_elem(rbase + grow[ii]) * (DH * 2) + gchk[ii];
+      async_copy16(Qg + ro, st + (ii * 4 + wave) * 1024);
+      async_copy16(dOg + ro, st + TILE + (ii * 4 + wave) * 1024);
+    }
+    if (wave == 0) {   // always four copies so that the count per stage is fixed
+      const int row = min(rbase + l, rows - 1);
+      const long ro = row_elem(row);
+      const int t = row / a.r + shift;
+      float* rv = (float*)(st + 2 * TILE);
+      async_copy4(Gg ? Gg + (long)t * a.h : rmg + ro, rv);
+      async_copy4(rmg + ro, rv + AB_BM);
+      async_copy4(dlg ? dlg + ro : rmg + ro, rv + 2 * AB_BM);
+      async_copy4(osg ? osg + ro : rmg + ro, rv + 3 * AB_BM);
+    }
+  };
+  if (nsteps > 0) issue(0);
+  if (nsteps > 1) issue(1);
 
   v8 Kf[MK][KS], Vf[MK][KS];
   int key[MK];
   bool live[MK];
-  float Gk[MK], ev[MK], dgk[MK];
+  float Gk[MK], Rk[MK], evg[MK], dgk[MK], keyf[MK];
 #pragma unroll
   for (int kj = 0; kj < MK; kj++) {
-    key[kj] = key0 + wave * 16 * MK + 16 * kj + kcol;
+    key[kj] = wkey0 + 16 * kj + kcol;
     live[kj] = key[kj] < a.tk;
+    keyf[kj] = (float)key[kj];
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) {
       u32x4 z = {0, 0, 0, 0}, z2 = {0, 0, 0, 0};
@@ -291,8 +426,9 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
       Kf[kj][ks] = __builtin_bit_cast(v8, z);
       Vf[kj][ks] = __builtin_bit_cast(v8, z2);
     }
-    Gk[kj] = (Gg && live[kj]) ? Gg[(long)key[kj] * a.h] : 0.f;
-    ev[kj] = __expf(fminf(R - Gk[kj], AB_EXP_CLAMP));
+    Gk[kj] = Gg ? Gg[(long)min(key[kj], a.tk - 1) * a.h] : 0.f;
+    Rk[kj] = Gg ? Gg[(long)min(wkey0 + 16 * kj + 15, a.tk - 1) * a.h] : 0.f;   // gate at the group's last key
+    evg[kj] = __expf(fminf(Rk[kj] - Gk[kj], AB_EXP_CLAMP));   // key factor inside its group of 16, <= 1
     dgk[kj] = 0.f;
   }
   f32x4 accK[MK][NT], accV[MK][NT];
@@ -304,133 +440,177 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
       accV[kj][nt] = (f32x4){0, 0, 0, 0};
     }
 
-  // folded rows that can see any key of this workgroup: time index >= key0
-  const int row_begin = max(0, (key0 - shift) * a.r) / AB_BM * AB_BM;
-  const int nsteps = (rows - row_begin + AB_BM - 1) / AB_BM;
-
-  u32x4 rq[PT], rdo[PT];
-  float r0 = 0.f, r1 = 0.f, r2 = 0.f, r3 = 1.f;
-  auto fetch = [&](int rbase) {
+  int qoff_[KS], toff[NT];
 #pragma unroll
-    for (int i = 0; i < PT; i++) {
-      const int ch = tid + 256 * i;
-      const int row = rbase + ch / (DH / 8), col = (ch % (DH / 8)) * 8;
-      rq[i] = (u32x4){0, 0, 0, 0};
-      rdo[i] = (u32x4){0, 0, 0, 0};
-      if (ch < CH && row < rows) {
-        const int t = row / a.r;
-        const long qo = (long)t * hq + hh * a.r + (row - t * a.r);
-        rq[i] = *(const u32x4*)(Qg + qo * DH + col);
-        rdo[i] = *(const u32x4*)(dOg + qo * DH + col);
-      }
-    }
-    if (tid < AB_BM) {
-      const int row = rbase + tid;
-      r0 = 0.f; r1 = 0.f; r2 = -1.f; r3 = 1.f;  // time index -1: sees no key
-      if (row < rows) {
-        const int t = row / a.r;
-        const long so = (long)b * a.tq * hq + (long)t * hq + hh * a.r + (row - t * a.r);
-        r0 = (Gg ? Gg[(long)(t + shift) * a.h] : 0.f) - a.rowmax[so];
-        r1 = a.dl ? a.dl[so] : 0.f;
-        r2 = (float)(t + shift);
-        r3 = a.dO_scale ? a.dO_scale[so] : 1.f;
-      }
-    }
-  };
-  auto stash = [&](int stage) {
-#pragma unroll
-    for (int i = 0; i < PT; i++) {
-      const int ch = tid + 256 * i;
-      if (ch < CH) {
-        const int o = stage * AB_BM * LD + (ch / (DH / 8)) * LD + (ch % (DH / 8)) * 8;
-        *(u32x4*)(Qt + o) = rq[i];
-        *(u32x4*)(dOt + o) = rdo[i];
-      }
-    }
-    if (tid < AB_BM) {
-      float* rv = rowv + stage * 5 * AB_BM;
-      rv[tid] = r0;
-      rv[AB_BM + tid] = r1;
-      rv[2 * AB_BM + tid] = r2;
-      rv[3 * AB_BM + tid] = scale_p * __expf(fminf(r0 - R, AB_EXP_CLAMP));
-      rv[4 * AB_BM + tid] = r3;
-    }
-  };
-
-  if (nsteps > 0) fetch(row_begin);
-  for (int it = 0; it < nsteps; it++) {
-    const int rbase = row_begin + it * AB_BM, stage = it & 1;
-    stash(stage);
-    lds_barrier();
-    if (it + 1 < nsteps) fetch(rbase + AB_BM);
-    const T* qt_ = Qt + stage * AB_BM * LD;
-    const T* dot_ = dOt + stage * AB_BM * LD;
-    const float* rv = rowv + stage * 5 * AB_BM;
-    // exact per-pair path unless every row of the step is real and sees every (real) key of the workgroup
-    const bool diag = (rbase / a.r + shift < last_key) || (rbase + AB_BM > rows) || (key0 + KEYS > a.tk);
-
-    v8 pf[MK], dsf[MK];
-    {
-      float p8[MK][8], d8[MK][8];
-#pragma unroll
-      for (int qt = 0; qt < QT; qt++) {
-        v8 qf[KS], dof[KS];
-#pragma unroll
-        for (int ks = 0; ks < KS; ks++) {
-          qf[ks] = lds_frag<T>(qt_, LD, 16 * qt, 32 * ks);
-          dof[ks] = lds_frag<T>(dot_, LD, 16 * qt, 32 * ks);
-        }
-        const f32x4 gm = *(const f32x4*)(rv + (diag ? 0 : 3 * AB_BM) + 16 * qt + 4 * g);
-        const f32x4 dlv = *(const f32x4*)(rv + AB_BM + 16 * qt + 4 * g);
-        const f32x4 tiv = *(const f32x4*)(rv + 2 * AB_BM + 16 * qt + 4 * g);
-        const f32x4 osv = *(const f32x4*)(rv + 4 * AB_BM + 16 * qt + 4 * g);
-#pragma unroll
-        for (int kj = 0; kj < MK; kj++) {
-          f32x4 s = {0, 0, 0, 0}, dp = {0, 0, 0, 0};
-#pragma unroll
-          for (int ks = 0; ks < KS; ks++) {
-            s = mfma16(qf[ks], Kf[kj][ks], s);
-            dp = mfma16(dof[ks], Vf[kj][ks], dp);
-          }
-#pragma unroll
-          for (int v = 0; v < 4; v++) {
-            float E;
-            if (diag) {
-              E = scale_p * __expf(fminf(gm[v] - Gk[kj], AB_EXP_CLAMP));
-              if ((float)key[kj] > tiv[v] || !live[kj]) E = 0.f;
-            } else {
-              E = gm[v] * ev[kj];
-            }
-            float p, dz, dsr;
-            pair_grad<DEG2>(s[v], E, dp[v] * osv[v] + dlv[v], eps_s, half_deg, p, dz, dsr);
-            dgk[kj] -= dz;
-            p8[kj][4 * qt + v] = p * osv[v];
-            d8[kj][4 * qt + v] = dsr;
-          }
-        }
-      }
-#pragma unroll
-      for (int kj = 0; kj < MK; kj++) {
-        pf[kj] = pack8<T>(p8[kj]);
-        dsf[kj] = pack8<T>(d8[kj]);
-      }
-    }
-    // dV^T[e, key] += dO^T[e, row] P[row, key];  dK^T[d, key] += Q^T[d, row] dsr[row, key]
+  for (int ks = 0; ks < KS; ks++) qoff_[ks] = kcol * RB + (((4 * ks + g) ^ swz<CPR>(kcol)) * 16);
+  {
+    const int vr = 4 * g + (kcol >> 2);
 #pragma unroll
     for (int nt = 0; nt < NT; nt++) {
-      v4 lo = lds_frag_tr4<T>(dot_, LD, 4 * g, 16 * nt);
-      v4 hi = lds_frag_tr4<T>(dot_, LD, 16 + 4 * g, 16 * nt);
-      v8 doT = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-      lo = lds_frag_tr4<T>(qt_, LD, 4 * g, 16 * nt);
-      hi = lds_frag_tr4<T>(qt_, LD, 16 + 4 * g, 16 * nt);
-      v8 qT = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-#pragma unroll
-      for (int kj = 0; kj < MK; kj++) {
-        accV[kj][nt] = mfma16(doT, pf[kj], accV[kj][nt]);
-        accK[kj][nt] = mfma16(qT, dsf[kj], accK[kj][nt]);
-      }
+      const int col = 16 * nt + 4 * (kcol & 3);
+      toff[nt] = vr * RB + (((col / 8) ^ swz<CPR>(vr)) * 16) + (col % 8) * 2;
     }
   }
+
+  // Row vectors of a tile (wave 0 issued their copies): G_q - m, time index (-1 for rows past the end), dl, dO
+  // scale, and the far-tile factors scale^deg exp(G_q - m - R) * {dO scale, dl} (zero for rows past the end).
+  auto row_factors = [&](int step) {
+    float* rv = (float*)(smem + (step % AB_NST) * STAGE + 2 * TILE);
+    const int row = (ntile_total - 1 - step) * AB_BM + l;
+    const bool real = row < rows;
+    const float bs = (Gg ? rv[l] : 0.f) - rv[AB_BM + l];
+    const float dl_ = (dlg && real) ? rv[2 * AB_BM + l] : 0.f;
+    const float os_ = osg ? rv[3 * AB_BM + l] : 1.f;
+    const float eu = real ? scale_p * __expf(fminf(bs - Rblk, AB_EXP_CLAMP)) : 0.f;
+    rv[l] = bs;
+    rv[AB_BM + l] = real ? (float)(min(row, rows - 1) / a.r + shift) : -1.f;
+    rv[2 * AB_BM + l] = dl_;
+    rv[3 * AB_BM + l] = real ? os_ : 0.f;
+    rv[4 * AB_BM + l] = eu * os_;
+    rv[5 * AB_BM + l] = eu * dl_;
+  };
+  if (wave == 0 && nsteps > 0) {
+    wait_vmcnt<0>();
+    row_factors(0);
+  }
+  auto sync_step = [&](int step) -> char* {
+    char* st = smem + (step % AB_NST) * STAGE;
+    if (step + 1 < nsteps) wait_vmcnt<LOADS>(); else wait_vmcnt<0>();
+    lds_barrier();
+    if (step + 2 < nsteps) issue(step + 2);
+    if (wave == 0 && step + 1 < nsteps) {
+      if (step + 2 < nsteps) wait_vmcnt<LOADS + 4>(); else wait_vmcnt<0>();   // all but the stage just issued
+      row_factors(step + 1);
+    }
+    return st;
+  };
+
+  auto tile = [&](const char* st, auto far_c) {
+    constexpr bool FAR = decltype(far_c)::value != 0;
+    uint32_t qb[KS], ob[KS], qtb[NT], otb[NT], fb;
+    {
+      const uint32_t sa = (uint32_t)(uintptr_t)(ab_lds_char*)st;
+#pragma unroll
+      for (int ks = 0; ks < KS; ks++) {
+        qb[ks] = sa + qoff_[ks];
+        ob[ks] = sa + TILE + qoff_[ks];
+        asm volatile("" : "+v"(qb[ks]));
+        asm volatile("" : "+v"(ob[ks]));
+      }
+#pragma unroll
+      for (int nt = 0; nt < NT; nt++) {
+        qtb[nt] = sa + toff[nt];
+        otb[nt] = sa + TILE + toff[nt];
+        asm volatile("" : "+v"(qtb[nt]));
+        asm volatile("" : "+v"(otb[nt]));
+      }
+      fb = sa + 2 * TILE + 16 * g;
+      asm volatile("" : "+v"(fb));
+    }
+#pragma unroll
+    for (int qp = 0; qp < QT / 2; qp++) {
+      v8 qf[2][KS], dof[2][KS];
+      f32x4 fa[2], fc[2], fd[2], fe[2];   // FAR: factor*scale, factor*dl;  near: G_q - m, time index, dl, dO scale
+#pragma unroll
+      for (int half = 0; half < 2; half++) {
+        const int qt = 2 * qp + half;
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) {
+          qf[half][ks] = *(const lds_v8*)(qb[ks] + qt * 16 * RB);
+          dof[half][ks] = *(const lds_v8*)(ob[ks] + qt * 16 * RB);
+        }
+        if (FAR) {
+          fa[half] = *(const ab_lds_f32x4*)(fb + (4 * AB_BM + 16 * qt) * 4);
+          fc[half] = *(const ab_lds_f32x4*)(fb + (5 * AB_BM + 16 * qt) * 4);
+        } else {
+          fa[half] = *(const ab_lds_f32x4*)(fb + (16 * qt) * 4);
+          fc[half] = *(const ab_lds_f32x4*)(fb + (AB_BM + 16 * qt) * 4);
+          fd[half] = *(const ab_lds_f32x4*)(fb + (2 * AB_BM + 16 * qt) * 4);
+          fe[half] = *(const ab_lds_f32x4*)(fb + (3 * AB_BM + 16 * qt) * 4);
+        }
+      }
+      f32x4 sc[2][MK], dp[2][MK];
+#pragma unroll
+      for (int half = 0; half < 2; half++)
+#pragma unroll
+        for (int kj = 0; kj < MK; kj++) {
+          sc[half][kj] = (f32x4){0, 0, 0, 0};
+          dp[half][kj] = (f32x4){0, 0, 0, 0};
+        }
+#pragma unroll
+      for (int ks = 0; ks < KS; ks++)
+#pragma unroll
+        for (int half = 0; half < 2; half++)
+#pragma unroll
+          for (int kj = 0; kj < MK; kj++) {
+            sc[half][kj] = mfma16(qf[half][ks], Kf[kj][ks], sc[half][kj]);
+            dp[half][kj] = mfma16(dof[half][ks], Vf[kj][ks], dp[half][kj]);
+          }
+      v8 pf[MK], dsf[MK];
+#pragma unroll
+      for (int kj = 0; kj < MK; kj++) {
+        float p8[8], d8[8];
+#pragma unroll
+        for (int half = 0; half < 2; half++) {
+#pragma unroll
+          for (int v = 0; v < 4; v++) {
+            const float s = sc[half][kj][v];
+            const float a2 = __builtin_fmaf(s, s, eps2);
+            float q, pw;   // q = E * dP, pw = P * (dO scale), both without the key factor
+            if (FAR) {
+              q = __builtin_fmaf(dp[half][kj][v], fa[half][v], fc[half][v]);
+              pw = a2 * fa[half][v];
+              if (!DEG2) {
+                const float h1 = pow_hm1<DEG2>(a2, half_deg);
+                q *= h1;
+                pw *= h1;
+              }
+            } else {
+              const bool vis = (keyf[kj] <= fc[half][v]) && live[kj];
+              float E = scale_p * __expf(fminf(fa[half][v] - Rk[kj], AB_EXP_CLAMP)) * evg[kj] * pow_hm1<DEG2>(a2, half_deg);
+              E = vis ? E : 0.f;
+              q = E * __builtin_fmaf(dp[half][kj][v], fe[half][v], fd[half][v]);
+              pw = a2 * E * fe[half][v];
+            }
+            const float dsr = s * q;
+            dgk[kj] = DEG2 ? __builtin_fmaf(s, dsr, dgk[kj]) : __builtin_fmaf(a2, q, dgk[kj]);
+            p8[4 * half + v] = pw;
+            d8[4 * half + v] = dsr;
+          }
+        }
+        pf[kj] = pack8<T>(p8);
+        dsf[kj] = pack8<T>(d8);
+      }
+      // dV^T[e, key] += dO^T[e, row] P[row, key];  dK^T[d, key] += Q^T[d, row] dsr[row, key]
+#pragma unroll
+      for (int nt = 0; nt < NT; nt++) {
+        const v8 doT = ab_tr8<T>(otb[nt] + qp * 32 * RB, otb[nt] + qp * 32 * RB + 16 * RB);
+        const v8 qT = ab_tr8<T>(qtb[nt] + qp * 32 * RB, qtb[nt] + qp * 32 * RB + 16 * RB);
+#pragma unroll
+        for (int kj = 0; kj < MK; kj++) {
+          accV[kj][nt] = mfma16(doT, pf[kj], accV[kj][nt]);
+          accK[kj][nt] = mfma16(qT, dsf[kj], accK[kj][nt]);
+        }
+      }
+    }
+  };
+
+  int step = 0;
+  for (; step < n_far; step++) tile(sync_step(step), IC<1>{});
+  // the far tiles were accumulated without the key factor exp(R - G_k) (<= 1); apply it once.  The tiles near
+  // the diagonal are accumulated in absolute terms (their packed weights stay <= the true ones).
+#pragma unroll
+  for (int kj = 0; kj < MK; kj++) {
+    const float c = __expf(fminf(Rblk - Gk[kj], AB_EXP_CLAMP));
+#pragma unroll
+    for (int nt = 0; nt < NT; nt++) {
+      accK[kj][nt] *= c;
+      accV[kj][nt] *= c;
+    }
+    dgk[kj] *= c;
+  }
+  for (; step < n_seen; step++) tile(sync_step(step), IC<0>{});
+  for (; step < nsteps; step++) sync_step(step);
 
   T* dKg = (T*)a.dK + (long)b * a.tk * a.h * DH + hh * DH;
   T* dVg = (T*)a.dV + (long)b * a.tk * a.h * DH + hh * DH;
@@ -449,16 +629,17 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
       *(v4*)(dKg + key[kj] * kstride + 16 * nt + 4 * g) = pack4<T>(k4);
       *(v4*)(dVg + key[kj] * kstride + 16 * nt + 4 * g) = pack4<T>(v4f);
     }
-    if (g == 0 && a.dGk) a.dGk[((long)b * a.tk + key[kj]) * a.h + hh] = tot;
+    if (g == 0 && a.dGk) a.dGk[((long)b * a.tk + key[kj]) * a.h + hh] = -tot;
   }
 }
 
 template <typename T, int DH, bool DEG2> static int attn_bwd_launch(const AttnBwdArgs& a, int B, hipStream_t st) {
+  const int npairs = B * a.h;
   {
     constexpr int MT = DH <= 64 ? 2 : 1;
-    constexpr size_t smem = 2 * 2 * AB_BN * (DH + 8) * sizeof(T) + 2 * (2 * AB_BN + 4) * sizeof(float);
+    constexpr size_t smem = AB_NST * (2 * AB_BN * DH * 2 + 4 * AB_BN * 4);
     const int rows = a.tq * a.r;
-    const int nblocks = (rows + 64 * MT - 1) / (64 * MT), npairs = B * a.h;
+    const int nblocks = (rows + 64 * MT - 1) / (64 * MT);
     dim3 grid((unsigned)((npairs + 31) / 32 * 32 * nblocks));
     auto kern = attention_bwd_dq_kernel<T, DH, MT, DEG2>;
     allow_big_lds((const void*)kern, smem);
@@ -466,8 +647,8 @@ template <typename T, int DH, bool DEG2> static int attn_bwd_launch(const AttnBw
   }
   {
     constexpr int MK = DH <= 64 ? 2 : 1;
-    constexpr size_t smem = 2 * 2 * AB_BM * (DH + 8) * sizeof(T) + 2 * 5 * AB_BM * sizeof(float);
-    const int nblocks = (a.tk + 64 * MK - 1) / (64 * MK), npairs = B * a.h;
+    constexpr size_t smem = AB_NST * (2 * AB_BM * DH * 2 + 6 * AB_BM * 4);
+    const int nblocks = (a.tk + 64 * MK - 1) / (64 * MK);
     dim3 grid((unsigned)((npairs + 31) / 32 * 32 * nblocks));
     auto kern = attention_bwd_dkv_kernel<T, DH, MK, DEG2>;
     allow_big_lds((const void*)kern, smem);
@@ -477,11 +658,12 @@ template <typename T, int DH, bool DEG2> static int attn_bwd_launch(const AttnBw
 }
 
 int attention_bwd(const AttnBwdArgs& a, int B, int d, int dtype, hipStream_t st) {
+  const bool deg2 = a.deg == 2.f;
 #define PR_AB(T)                                                                                                       \
   switch (d) {                                                                                                         \
-    case 32: return a.deg == 2.f ? attn_bwd_launch<T, 32, true>(a, B, st) : attn_bwd_launch<T, 32, false>(a, B, st);   \
-    case 64: return a.deg == 2.f ? attn_bwd_launch<T, 64, true>(a, B, st) : attn_bwd_launch<T, 64, false>(a, B, st);   \
-    case 128: return a.deg == 2.f ? attn_bwd_launch<T, 128, true>(a, B, st) : attn_bwd_launch<T, 128, false>(a, B, st);\
+    case 32: return deg2 ? attn_bwd_launch<T, 32, true>(a, B, st) : attn_bwd_launch<T, 32, false>(a, B, st);           \
+    case 64: return deg2 ? attn_bwd_launch<T, 64, true>(a, B, st) : attn_bwd_launch<T, 64, false>(a, B, st);           \
+    case 128: return deg2 ? attn_bwd_launch<T, 128, true>(a, B, st) : attn_bwd_launch<T, 128, false>(a, B, st);        \
     default: return -2;                                                                                                \
   }
   if (dtype == DT_BF16) { PR_AB(bf16_t) }
