@@ -34,6 +34,19 @@ template <typename T> struct OnePair;   // two packed 1.0 values
 template <> struct OnePair<bf16_t> { static constexpr uint32_t v = 0x3F803F80u; static constexpr float down = 1.f, up = 1.f; };
 template <> struct OnePair<f16_t> { static constexpr uint32_t v = 0x3C003C00u; static constexpr float down = 1.f / 256.f, up = 256.f; };
 
+// the two 16-bit values of one dword as floats
+template <typename T> __device__ __forceinline__ void unpack2(uint32_t u, float& lo, float& hi);
+template <> __device__ __forceinline__ void unpack2<bf16_t>(uint32_t u, float& lo, float& hi) {
+  lo = __builtin_bit_cast(float, u << 16);
+  hi = __builtin_bit_cast(float, u & 0xffff0000u);
+}
+template <> __device__ __forceinline__ void unpack2<f16_t>(uint32_t u, float& lo, float& hi) {
+  typedef __attribute__((ext_vector_type(2))) _Float16 h2;
+  const h2 p = __builtin_bit_cast(h2, u);
+  lo = (float)p[0];
+  hi = (float)p[1];
+}
+
 template <typename T, int DK, int DV, int MT, bool MULT>
 __global__ __launch_bounds__(256, 2) void sympow_grad_kernel(GradArgs a, int row_blocks, int npairs) {
   typedef typename VecOf<T>::v8 v8;
@@ -45,7 +58,8 @@ __global__ __launch_bounds__(256, 2) void sympow_grad_kernel(GradArgs a, int row
   constexpr int LDM = DK + 8;
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   char* ring = smem;                                         // [NST][STAGE]; reused for M at the end
-  char* xt = ring + GR_NST * STAGE;                          // [ROWS][DK] T, swizzled
+  constexpr int RING_BYTES = GR_NST * STAGE > DK * LDM * 2 ? GR_NST * STAGE : DK * LDM * 2;   // the ring later holds M
+  char* xt = ring + (RING_BYTES + 1023) / 1024 * 1024;       // [ROWS][DK] T, swizzled
 
   // XCD-aware placement: consecutive workgroup ids go to different XCDs, so id % 8 picks the XCD
   const int xcd = blockIdx.x % 8, slot = blockIdx.x / 8;
@@ -82,7 +96,7 @@ __global__ __launch_bounds__(256, 2) void sympow_grad_kernel(GradArgs a, int row
   // X rows of this workgroup (waited for together with stage 0), then the first two stages
   async_load_tile<CX, ROWS>(xt, [&](int row) { return (const char*)(Xg + row_off(row0 + row) * DK); });
   issue(0);
-  issue(1);
+  if (GR_NST > 2) issue(1);
 
   // per-lane row data (row = this lane's column of the dphi^T tiles)
   v8 Gf[MT][KS];
@@ -107,84 +121,106 @@ __global__ __launch_bounds__(256, 2) void sympow_grad_kernel(GradArgs a, int row
   };
 
   f32x4 acc[MT][TT];            // dX^T[16*blk + 4g + v, row]
-  f32x4 accA[MT], accB[MT];     // contributions of the current 16x16 feature block (y, xb)
-  float xr[MT][4];              // X[row, 16y + 4g + v]
 #pragma unroll
-  for (int mi = 0; mi < MT; mi++) {
+  for (int mi = 0; mi < MT; mi++)
 #pragma unroll
     for (int k = 0; k < TT; k++) acc[mi][k] = (f32x4){0, 0, 0, 0};
-    accA[mi] = (f32x4){0, 0, 0, 0};
-    accB[mi] = (f32x4){0, 0, 0, 0};
-  }
-  int y_cur = 0, xb_cur = 0;
-  auto commit_block = [&]() {
-    const float m = (MULT && xb_cur < y_cur) ? 2.f : 1.f;
-#pragma unroll
-    for (int mi = 0; mi < MT; mi++) {
-      static_for<TT>([&](auto k) {
-        if (k.value == y_cur) acc[mi][k.value] += accA[mi] * m;
-        if (k.value == xb_cur) acc[mi][k.value] += accB[mi] * m;
-      });
-      accA[mi] = (f32x4){0, 0, 0, 0};
-      accB[mi] = (f32x4){0, 0, 0, 0};
-    }
-  };
 
-  for (int step = 0; step < NSTEP; step++) {
-    const char* st = ring + (step % GR_NST) * STAGE;
-    if (step + 1 < NSTEP) wait_vmcnt<LOADS>(); else wait_vmcnt<0>();
-    lds_barrier();
-    if (step + 2 < NSTEP) issue(step + 2);
-    const int f0 = step * GR_FR;
-    int y = 0;
-    while (128 * (y + 1) * (y + 2) <= f0) y++;
-    const int X0 = (f0 - 128 * y * (y + 1)) / 16, xb = X0 / 16;
-    if (step == 0 || y != y_cur || xb != xb_cur) {
-      if (step > 0) commit_block();
-      if (step == 0 || y != y_cur) {
+  // Per-lane LDS byte addresses, hoisted out of the stage loop (the swizzle of a row depends only on its position
+  // inside a group of 16 rows, so a stage adds a scalar base and the rest are immediate offsets).
+  typedef __attribute__((address_space(3))) char lds_char;
+  typedef __attribute__((address_space(3))) v8 lds_v8;
+  typedef __attribute__((address_space(3))) uint32_t lds_u32;
+  const uint32_t ring_a = (uint32_t)(uintptr_t)(lds_char*)ring, xt_a = (uint32_t)(uintptr_t)(lds_char*)xt;
+  uint32_t aoff[KS];            // B rows as the A operand: row tcol of a 16-row group, chunk 4*ks + g
 #pragma unroll
-        for (int mi = 0; mi < MT; mi++) {
-          const v4 h4 = *(const v4*)x_ptr(mi, 16 * y + 4 * g);
+  for (int ks = 0; ks < KS; ks++) aoff[ks] = tcol * (CB * 16) + (((4 * ks + g) ^ swz<CB>(tcol)) * 16);
+  uint32_t xrow_a[MT], xsw[MT];
 #pragma unroll
-          for (int v = 0; v < 4; v++) xr[mi][v] = (float)h4[v];
-        }
-      }
-      y_cur = y;
-      xb_cur = xb;
-    }
-#pragma unroll
-    for (int pr2 = 0; pr2 < GR_FR / 32; pr2++) {
-      const int X = X0 + 2 * pr2, m0 = X % 16;
-      v8 af0[KS], af1[KS];
-#pragma unroll
-      for (int ks = 0; ks < KS; ks++) {
-        af0[ks] = sw_frag<T, CB>(st, 32 * pr2, 32 * ks);
-        af1[ks] = sw_frag<T, CB>(st, 32 * pr2 + 16, 32 * ks);
-      }
-      // selector: accumulator row m0 sums the first 16 contraction slots (column X), row m0+1 the last 16
-      const uint32_t s_lo = (tcol == m0) ? OnePair<T>::v : 0u, s_hi = (tcol == m0 + 1) ? OnePair<T>::v : 0u;
-      const v8 sel = __builtin_bit_cast(v8, (u32x4){s_lo, s_lo, s_hi, s_hi});
-#pragma unroll
-      for (int mi = 0; mi < MT; mi++) {
-        f32x4 d0 = {0, 0, 0, 0}, d1 = {0, 0, 0, 0};
-#pragma unroll
-        for (int ks = 0; ks < KS; ks++) {
-          d0 = mfma16(af0[ks], Gf[mi][ks], d0);
-          d1 = mfma16(af1[ks], Gf[mi][ks], d1);
-        }
-        const float x0 = (float)*(const T*)x_ptr(mi, X), x1 = (float)*(const T*)x_ptr(mi, X + 1);
-        accA[mi] += d0 * x0 + d1 * x1;
-        float w8[8];
-#pragma unroll
-        for (int v = 0; v < 4; v++) {
-          w8[v] = xr[mi][v] * d0[v];
-          w8[4 + v] = xr[mi][v] * d1[v];
-        }
-        accB[mi] = mfma16(sel, pack8<T>(w8), accB[mi]);
-      }
-    }
+  for (int mi = 0; mi < MT; mi++) {
+    xrow_a[mi] = xt_a + lrow[mi] * (DK * 2);
+    xsw[mi] = swz<CX>(lrow[mi]);
   }
-  commit_block();
+
+  // Blocks (y, xb) in memory order, both compile-time indices so that the two folds accumulate straight into the
+  // accumulators of strip y and strip xb; only the four stages of a block are a run-time loop.  With the key-side
+  // multiplier (2 below the block diagonal) the strip-y accumulator is doubled once before the diagonal block and
+  // the other fold uses doubled X values.
+  int step = 0;
+  static_for<TT>([&](auto yc) {
+    constexpr int y = decltype(yc)::value;
+    float xr[MT][4];              // X[row, 16y + 4g + v]
+    static_for<y + 1>([&](auto xc) {
+      constexpr int xb = decltype(xc)::value;
+      constexpr bool diag = xb == y;
+#pragma unroll 1
+      for (int sb = 0; sb < 256 / GR_FR; sb++, step++) {
+        if (GR_NST > 2 && step + 1 < NSTEP) wait_vmcnt<LOADS>(); else wait_vmcnt<0>();
+        lds_barrier();
+        if (step + GR_NST - 1 < NSTEP) issue(step + GR_NST - 1);
+        if (sb == 0 && (xb == 0 || (MULT && diag))) {   // (re)load the strip's X values; X tile is visible after the barrier
+          const float m = (MULT && !diag) ? 2.f : 1.f;
+#pragma unroll
+          for (int mi = 0; mi < MT; mi++) {
+            const v4 h4 = *(const v4*)x_ptr(mi, 16 * y + 4 * g);
+#pragma unroll
+            for (int v = 0; v < 4; v++) xr[mi][v] = (float)h4[v] * m;
+            if (MULT && diag) acc[mi][y] *= 2.f;
+          }
+        }
+        uint32_t ab[KS], xa[MT];
+        {
+          const uint32_t sa = ring_a + (step % GR_NST) * STAGE;
+#pragma unroll
+          for (int ks = 0; ks < KS; ks++) { ab[ks] = sa + aoff[ks]; asm volatile("" : "+v"(ab[ks])); }
+          // X[row, 16*xb + (GR_FR/16)*sb + 2*pr2 (+1)]: one 32-bit read per pair of columns
+          const int X0 = 16 * xb + (GR_FR / 16) * sb, xc = X0 >> 3, xo = (X0 & 7) * 2;
+#pragma unroll
+          for (int mi = 0; mi < MT; mi++) { xa[mi] = xrow_a[mi] + ((xc ^ xsw[mi]) << 4) + xo; asm volatile("" : "+v"(xa[mi])); }
+        }
+#pragma unroll
+        for (int pr2 = 0; pr2 < GR_FR / 32; pr2++) {
+          const int m0 = ((GR_FR / 16) * sb + 2 * pr2) % 16;
+          v8 af0[KS], af1[KS];
+#pragma unroll
+          for (int ks = 0; ks < KS; ks++) {
+            af0[ks] = *(const lds_v8*)(ab[ks] + (32 * pr2) * (CB * 16));
+            af1[ks] = *(const lds_v8*)(ab[ks] + (32 * pr2 + 16) * (CB * 16));
+          }
+          // selector: accumulator row m0 sums the first 16 contraction slots (column X), row m0+1 the last 16
+          const uint32_t s_lo = (tcol == m0) ? OnePair<T>::v : 0u, s_hi = (tcol == m0 + 1) ? OnePair<T>::v : 0u;
+          const v8 sel = __builtin_bit_cast(v8, (u32x4){s_lo, s_lo, s_hi, s_hi});
+          f32x4 d0[MT], d1[MT];
+#pragma unroll
+          for (int mi = 0; mi < MT; mi++) {
+            d0[mi] = (f32x4){0, 0, 0, 0};
+            d1[mi] = (f32x4){0, 0, 0, 0};
+          }
+#pragma unroll
+          for (int ks = 0; ks < KS; ks++)
+#pragma unroll
+            for (int mi = 0; mi < MT; mi++) {
+              d0[mi] = mfma16(af0[ks], Gf[mi][ks], d0[mi]);
+              d1[mi] = mfma16(af1[ks], Gf[mi][ks], d1[mi]);
+            }
+#pragma unroll
+          for (int mi = 0; mi < MT; mi++) {
+            float x0, x1;
+            unpack2<T>(*(const lds_u32*)(xa[mi] + 4 * pr2), x0, x1);
+            acc[mi][y] = acc[mi][y] + d0[mi] * x0;   // each line contracts to one fused multiply-add per element
+            acc[mi][y] = acc[mi][y] + d1[mi] * x1;
+            float w8[8];
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+              w8[v] = xr[mi][v] * d0[mi][v];
+              w8[4 + v] = xr[mi][v] * d1[mi][v];
+            }
+            acc[mi][xb] = mfma16(sel, pack8<T>(w8), acc[mi][xb]);   // fold into dX[row, 16*xb + X]
+          }
+        }
+      }
+    });
+  });
 
   // sB term: dX_s^T[w, row] = cvec[row] * sum_a M[w, a] X[row, a], M in two 16-bit parts (high, low) built in the
   // (now idle) ring memory.
@@ -239,16 +275,18 @@ template <typename T, int DK, int DV, bool MULT> static int grad_launch(const Gr
   auto go = [&](auto mt) {
     constexpr int MT = decltype(mt)::value;
     constexpr size_t ring = GR_NST * GR_FR * DV * 2, mtile = (size_t)DK * (DK + 8) * 2;
-    constexpr size_t smem = (ring > mtile ? ring : mtile) + 64 * MT * DK * 2;
+    constexpr size_t smem = ((ring > mtile ? ring : mtile) + 1023) / 1024 * 1024 + 64 * MT * DK * 2;
     const int row_blocks = (rows + 64 * MT - 1) / (64 * MT);
     dim3 grid((unsigned)(((npairs + 7) / 8) * 8 * row_blocks));
     auto kern = sympow_grad_kernel<T, DK, DV, MT, MULT>;
     allow_big_lds((const void*)kern, smem);
     hipLaunchKernelGGL(kern, grid, dim3(256), smem, st, a, row_blocks, npairs);
   };
-  if (DK <= 64 && rows >= 256) go(IC<4>{});
-  else if (DK <= 64 && rows > 64) go(IC<2>{});
-  else go(IC<1>{});
+  if constexpr (DK <= 64) {
+    if (rows >= 256) { go(IC<4>{}); return (int)hipGetLastError(); }
+    if (rows > 64) { go(IC<2>{}); return (int)hipGetLastError(); }
+  }
+  go(IC<1>{});
   return (int)hipGetLastError();
 }
 
