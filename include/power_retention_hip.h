@@ -132,6 +132,23 @@ int pr_chunk_glue_bwd(const float* A, const float* lcs, const void* Kd, const vo
                       void* dQ, void* dV, float* dlog_G, void* workspace, int BN, int c, int h, int r, int d, int deg,
                       int dtype, void* stream);
 
+/* Single-token inference step on the state -- query: retention/power_retention_maker.py:358-363 with
+ * retention/_query_state/reference.py:36-96 (one query position per sequence); update:
+ * retention/power_retention_maker.py:366-382 with retention/_update_state/reference.py:33-52 for ONE new token.
+ *   Q [B,tq,h*r,d] with tq*r <= 8, gq [B,h] fp32 or NULL: accumulated log gate at the query position
+ *   (Q is used as Q * exp(gq/deg), rounded to dtype), S [B,h,D,d], s [B,h,D] fp32,
+ *   Y_attn [B,tq,h*r,d], l_attn, rowmax [B,tq,h*r] fp32 or all NULL (attention over the not yet folded cache)
+ *   -> out [B,tq,h*r,d] = the merged, normalised output.
+ *   If K_new is not NULL: K_new, V_new [B,h,d], log_decay [B,h] fp32 or NULL (= 0)
+ *   -> S_out = exp(log_decay) * S + phi(K_new)^T V_new, s_out = exp(log_decay) * s + phi(K_new), read in the same
+ *      pass as the query (which sees the OLD state).  S_out/s_out must not alias S/s.
+ *   workspace: pr_decode_step_workspace() bytes. */
+size_t pr_decode_step_workspace(int B, int tq, int h, int r, int d);
+int pr_decode_step(const void* Q, const float* gq, const void* S, const float* s, const void* Y_attn,
+                   const float* l_attn, const float* rowmax, const void* K_new, const void* V_new,
+                   const float* log_decay, void* S_out, float* s_out, void* out, void* workspace, int B, int tq, int h,
+                   int r, int d, float scale_p, int deg, int dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

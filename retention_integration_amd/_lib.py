@@ -37,6 +37,8 @@ SIGNATURES = {
     "pr_chunk_prep_fwd": (c_int, [_P] * 7 + [_I] * 7 + [_P]),
     "pr_chunk_glue_bwd_workspace": (c_size_t, [_I] * 3),
     "pr_chunk_glue_bwd": (c_int, [_P] * 18 + [_I] * 7 + [_P]),
+    "pr_decode_step_workspace": (c_size_t, [_I] * 5),
+    "pr_decode_step": (c_int, [_P] * 14 + [_I] * 5 + [_F, _I, _I, _P]),
 }
 
 _lib = None

@@ -92,4 +92,11 @@ int chunk_glue_bwd(const float* A, const float* lcs, const void* Kd, const void*
                    float* dlogG, float* workspace, int BN, int c, int h, int r, int d, int deg, int dtype,
                    hipStream_t st);
 
+// decode.hip (return -3: more than 8 query rows per (batch, kv head))
+long decode_workspace_floats(int B, int h, int r, int tq, int d);
+int decode_step(const void* Q, const float* gq, const void* S, const float* s, const void* Y_attn, const float* l_attn,
+                const float* rowmax, const void* Knew, const void* Vnew, const float* decay, void* Sout, float* sout,
+                void* out, float* workspace, int B, int tq, int h, int r, int d, int deg, float scale_p, int dtype,
+                hipStream_t st);
+
 }  // namespace pr

@@ -1,0 +1,56 @@
+"""``power_retention_inference`` with the single-token step fused (ref: retention/power_retention_maker.py:284-395).
+
+Same signature, results and state layout as the maker-assembled function; calls with a state and at most 8 query
+rows per (batch, kv head) -- the decode step -- go through one pass over the state (query, and the fold of a
+single new token when ``switch_over_seq_len`` is reached with a one-token cache) instead of the operator chain.
+Everything else is delegated to the composed function.
+"""
+import torch
+
+from . import ops
+
+
+def make_fused_inference(composed):
+    def power_retention_inference(Q, K, V, log_G=None, initial_state=None, sum_of_keys=None, deg=2, scale=None,
+                                  switch_over_seq_len=512):
+        has_cache = K is not None and V is not None
+        fast = (initial_state is not None and sum_of_keys is not None and deg == 2 and Q.dim() == 4
+                and Q.dtype in (torch.bfloat16, torch.float16) and initial_state.dtype == Q.dtype
+                and Q.shape[1] * (Q.shape[2] // initial_state.shape[1]) <= 8
+                and Q.shape[3] in (32, 64, 128))
+        if has_cache:
+            fast = fast and K.shape[1] >= Q.shape[1] and K.dtype == Q.dtype == V.dtype and K.shape[0] == Q.shape[0] \
+                and K.shape[2] == initial_state.shape[1]
+        if not fast:
+            return composed(Q, K, V, log_G, initial_state, sum_of_keys, deg, scale, switch_over_seq_len)
+        b, tq, hq, d = Q.shape
+        assert initial_state.shape[0] == b, "initial_state must have a batch size of the same as the query"
+        scale = 1.0 / d ** 0.5 if scale is None else scale
+        tk = K.shape[1] if has_cache else 0
+        A = log_G.to(torch.float32).cumsum(1) if (log_G is not None and has_cache) else None
+        Ya = la = rm = None
+        if tk > 0:
+            Ya, la, rm = ops.attention(Q, K, V, A, deg, scale=scale, norm=False)
+        a_last = A[:, -1].contiguous() if A is not None else None
+        fold = switch_over_seq_len is not None and tk >= switch_over_seq_len
+        S32 = sum_of_keys.to(torch.float32).contiguous()
+        if fold and tk == 1:
+            Y, new_S, new_s = ops.decode_step(Q.contiguous(), a_last, initial_state.contiguous(), S32, Ya, la, rm,
+                                              K[:, 0].contiguous(), V[:, 0].contiguous(), a_last, float(scale) ** deg)
+            return Y, new_S, new_s.to(sum_of_keys.dtype)
+        Y, _, _ = ops.decode_step(Q.contiguous(), a_last, initial_state.contiguous(), S32, Ya, la, rm, None, None,
+                                  None, float(scale) ** deg)
+        if not fold:
+            return Y, initial_state, sum_of_keys
+        # fold of a longer cache: the operator chain of the composed function
+        Kd = K
+        if A is not None:
+            Kd = (K * torch.exp((A[:, -1:] - A) / deg).unsqueeze(-1)).to(K.dtype)
+        dS, ds = ops.update_state(Kd.contiguous(), V.contiguous(), deg)
+        if A is None:
+            return Y, initial_state + dS, sum_of_keys + ds
+        decay = torch.exp(A[:, -1, :])
+        return (Y, initial_state * decay[..., None, None].to(initial_state.dtype) + dS,
+                sum_of_keys * decay[..., None].to(sum_of_keys.dtype) + ds)
+
+    return power_retention_inference

@@ -359,3 +359,38 @@ def query_state(Q, S, s, Y_attn, l_attn, rowmax, deg, scale, zero_initial_state)
     O, _den = query_state_fwd(Q.contiguous(), S.contiguous(), f32(s), _cont(Y_attn), f32(l_attn), f32(rowmax),
                               float(scale) ** deg, bool(zero_initial_state))
     return O
+
+
+# ----------------------------------------------------------------------------
+# single-token inference step on the state (no autograd: inference only)
+# ----------------------------------------------------------------------------
+@torch.library.custom_op("pr::decode_step", mutates_args=(), device_types="cuda")
+def decode_step(Q: Tensor, gq: Optional[Tensor], S: Tensor, s: Tensor, Y_attn: Optional[Tensor],
+                l_attn: Optional[Tensor], rowmax: Optional[Tensor], K_new: Optional[Tensor], V_new: Optional[Tensor],
+                log_decay: Optional[Tensor], scale_p: float) -> Tuple[Tensor, Tensor, Tensor]:
+    """Q [b, tq, hq, d] (tq * hq/h <= 8), gq [b, h] fp32 or None, S [b, h, D, d], s [b, h, D] fp32, attention part or
+    None, and optionally one new token K_new, V_new [b, h, d] with log_decay [b, h] -> (out [b, tq, hq, d],
+    S_new, s_new); without a new token S_new, s_new are empty tensors."""
+    b, tq, hq, d = Q.shape
+    h = S.shape[1]
+    out = torch.empty_like(Q)
+    lib = _lib.load()
+    ws = torch.empty(lib.pr_decode_step_workspace(b, tq, h, hq // h, d), dtype=torch.uint8, device=Q.device)
+    if K_new is not None:
+        S_new, s_new = torch.empty_like(S), torch.empty_like(s)
+    else:
+        S_new, s_new = S.new_empty(0), s.new_empty(0)
+    _lib.check(lib.pr_decode_step(_lib.ptr(Q), _lib.ptr(gq), _lib.ptr(S), _lib.ptr(s), _lib.ptr(Y_attn),
+                                  _lib.ptr(l_attn), _lib.ptr(rowmax), _lib.ptr(K_new), _lib.ptr(V_new),
+                                  _lib.ptr(log_decay), _lib.ptr(S_new) if K_new is not None else None,
+                                  _lib.ptr(s_new) if K_new is not None else None, _lib.ptr(out), _lib.ptr(ws),
+                                  b, tq, h, hq // h, d, float(scale_p), 2, _lib.dtype_code(Q.dtype), _lib.stream()),
+               "decode_step")
+    return out, S_new, s_new
+
+
+@decode_step.register_fake
+def _(Q, gq, S, s, Y_attn, l_attn, rowmax, K_new, V_new, log_decay, scale_p):
+    if K_new is not None:
+        return torch.empty_like(Q), torch.empty_like(S), torch.empty_like(s)
+    return torch.empty_like(Q), S.new_empty(0), s.new_empty(0)

@@ -211,3 +211,49 @@ def test_large_shape_invariants(pra):
     # the first chunk sees no state: it must equal quadratic attention on that chunk alone
     Yq = pra.power_retention(Q[:, :c], K[:, :c], V[:, :c], lg[:, :c], deg=2, chunk_size=None)
     check("chunk 0 vs quadratic", Y[:, :c], Yq, 1e-2)
+
+
+@pytest.mark.parametrize("dtype,d,r,gated", [(torch.bfloat16, 64, 1, True), (torch.bfloat16, 32, 4, True),
+                                             (torch.float16, 128, 2, False), (torch.bfloat16, 64, 8, True)])
+def test_fused_decode_step_equals_operator_chain(pra, dtype, d, r, gated):
+    """The one-pass decode step (query + fold of one token) against the maker-assembled operator chain and the
+    oracle: with a growing cache (no fold), with a one-token cache folded every step, and from the state alone."""
+    b, h, t0, steps = 3, 2, 128, 3
+    std = 0.5 if dtype == torch.float16 else 1.0
+    Q, K, V, lg = make_inputs(b, t0 + steps, h, r, d, dtype, gated, seed=21 + d, std=std)
+    dv = lambda x: None if x is None else x.to(DEV)  # noqa: E731
+    sl = lambda x, a, e: None if x is None else x[:, a:e]  # noqa: E731
+    f32 = lambda x: None if x is None else x.float()  # noqa: E731
+    _, st, sk = pra.power_retention_inference(dv(Q[:, :t0]), dv(K[:, :t0]), dv(V[:, :t0]), dv(sl(lg, 0, t0)), None, None,
+                                              deg=2, switch_over_seq_len=t0)
+    sto, sko = st.float().cpu(), sk.float().cpu()
+    # (i) cache grows, the state is only queried
+    for n_cached in (1, 3):
+        a = (dv(Q[:, t0 + n_cached - 1:t0 + n_cached]), dv(K[:, t0:t0 + n_cached]), dv(V[:, t0:t0 + n_cached]),
+             dv(sl(lg, t0, t0 + n_cached)))
+        Yf, sf, kf = pra.power_retention_inference(*a, st, sk, deg=2, switch_over_seq_len=64)
+        Yc, _, _ = pra.power_retention_inference_composed(*a, st, sk, deg=2, switch_over_seq_len=64)
+        Yo, _, _ = oracle.power_retention_inference(f32(Q[:, t0 + n_cached - 1:t0 + n_cached]), f32(K[:, t0:t0 + n_cached]),
+                                                    f32(V[:, t0:t0 + n_cached]), sl(lg, t0, t0 + n_cached), sto, sko,
+                                                    deg=2, switch_over_seq_len=64)
+        assert sf is st and kf is sk
+        check(f"cache of {n_cached}: fused vs chain", Yf, Yc, OUT_TOL)
+        check(f"cache of {n_cached}: fused vs oracle", Yf, Yo, OUT_TOL)
+    # (ii) one-token cache folded into the state at every step
+    st_f, sk_f, st_c, sk_c = st, sk, st, sk
+    for i in range(t0, t0 + steps):
+        a = (dv(Q[:, i:i + 1]), dv(K[:, i:i + 1]), dv(V[:, i:i + 1]), dv(sl(lg, i, i + 1)))
+        Yf, st_f, sk_f = pra.power_retention_inference(*a, st_f, sk_f, deg=2, switch_over_seq_len=1)
+        Yc, st_c, sk_c = pra.power_retention_inference_composed(*a, st_c, sk_c, deg=2, switch_over_seq_len=1)
+        Yo, sto, sko = oracle.power_retention_inference(f32(Q[:, i:i + 1]), f32(K[:, i:i + 1]), f32(V[:, i:i + 1]),
+                                                        sl(lg, i, i + 1), sto, sko, deg=2, switch_over_seq_len=1)
+        check(f"step {i}: fused vs chain", Yf, Yc, OUT_TOL)
+        check(f"step {i}: fused vs oracle", Yf, Yo, OUT_TOL)
+    check("state: fused vs chain", st_f, st_c, OUT_TOL)
+    check("state: fused vs oracle", st_f, sto, OUT_TOL)
+    check("sum_of_keys: fused vs oracle", sk_f, sko, OUT_TOL)
+    # (iii) no cache at all
+    q = dv(Q[:, -1:])
+    Yf, _, _ = pra.power_retention_inference(q, None, None, None, st_f, sk_f, deg=2)
+    Yc, _, _ = pra.power_retention_inference_composed(q, None, None, None, st_f, sk_f, deg=2)
+    check("state only: fused vs chain", Yf, Yc, OUT_TOL)
