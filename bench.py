@@ -2,7 +2,7 @@
 (b=1, t=65536, h=8, d=64, bf16, deg=2, chunk_size=1024, gated; ref: perf/benchmark.py:58-61,335-343)
 on one MI355X.  Prints ONE JSON line.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-breakdown]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-breakdown] [--no-decode]
 
 A step = one forward + one backward over one synthetic batch already resident in HBM.
 """
@@ -84,7 +84,64 @@ def op_breakdown(pra, Q, K, V, lg, dO, cfg, iters=5):
     res["attention_bwd"] = event_time_ms(lambda: ops.attention_bwd(Qf, Kf, Vf, Af, rm, dOf, la, None, 2, scale), iters)
     res["discumsum_bwd(S)"] = event_time_ms(lambda: ops.discumsum_bwd(Sc, Sc, lcs), iters)
     res["update_state_bwd"] = event_time_ms(lambda: ops.update_state_bwd(Kc, Vc, S, s), iters)
+    # the single kernel with the largest share of a step: the feature-gradient contraction (sympow_grad), here as
+    # the dK half of update_state backward, launched alone through the C ABI (dV = NULL skips the other half)
+    from retention_integration_amd import _lib
+    lib = _lib.load()
+    dK = torch.empty_like(Kc)
+    grad_only = lambda: _lib.check(lib.pr_update_state_bwd(  # noqa: E731
+        _lib.ptr(Kc), _lib.ptr(Vc), _lib.ptr(S), _lib.ptr(s), _lib.ptr(dK), None, b * n, c, h, d, 2,
+        _lib.dtype_code(Kc.dtype), _lib.stream()), "update_state_bwd(dK)")
+    res["sympow_grad(dK)"] = event_time_ms(grad_only, iters)
     return {k: round(v, 4) for k, v in res.items()}
+
+
+def decode_bench(pra, dev, steps=512):
+    """BASELINE configs[3]: b=32, h=8, d=64 bf16; prefill of 2048 tokens with switch_over_seq_len=1024, then
+    `steps` single-token steps.  Two loops are timed: the recurrent one (every token is folded into the state,
+    switch_over_seq_len=1) and the API-faithful one of the reference's caller (the cache grows, the state is only
+    queried; ref: deploy/models/powercoder/modeling_powercoder.py:181-196)."""
+    b, h, d = 32, 8, 64
+    g = torch.Generator().manual_seed(4)
+    mk = lambda *shape: torch.randn(*shape, generator=g).to(torch.bfloat16).to(dev)  # noqa: E731
+    K, V, Q = mk(b, 2048, h, d), mk(b, 2048, h, d), mk(b, 1, h, d)
+    lg = torch.nn.functional.logsigmoid(torch.randn(b, 2048, h, generator=g)).to(dev)
+    qs, ks, vs = mk(steps, b, 1, h, d), mk(steps, b, 1, h, d), mk(steps, b, 1, h, d)
+    lgs = torch.nn.functional.logsigmoid(torch.randn(steps, b, 1, h, generator=g)).to(dev)
+    out = {}
+    with torch.no_grad():
+        pra.power_retention_inference(Q, K, V, lg, switch_over_seq_len=1024)   # warm-up
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        _, S, s = pra.power_retention_inference(Q, K, V, lg, switch_over_seq_len=1024)
+        torch.cuda.synchronize()
+        out["prefill_ms"] = round((time.perf_counter() - t0) * 1e3, 3)
+        St, st = S, s
+        for i in range(8):
+            _, St, st = pra.power_retention_inference(qs[i], ks[i], vs[i], lgs[i], St, st, switch_over_seq_len=1)
+        St, st = S, s
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(steps):
+            _, St, st = pra.power_retention_inference(qs[i], ks[i], vs[i], lgs[i], St, st, switch_over_seq_len=1)
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        out["recurrent"] = {"us_per_step": round(dt / steps * 1e6, 1), "tokens_per_s": round(b * steps / dt, 1)}
+        Kc = torch.empty(b, 0, h, d, dtype=torch.bfloat16, device=dev)
+        Vc, Gc = Kc.clone(), torch.empty(b, 0, h, device=dev)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(steps):
+            Kc, Vc, Gc = torch.cat([Kc, ks[i]], 1), torch.cat([Vc, vs[i]], 1), torch.cat([Gc, lgs[i]], 1)
+            pra.power_retention_inference(qs[i], Kc, Vc, Gc, S, s, switch_over_seq_len=1024)
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        out["growing_cache"] = {"us_per_step": round(dt / steps * 1e6, 1), "tokens_per_s": round(b * steps / dt, 1)}
+    state_bytes = b * h * (pra.expanded_dim(d) * d * 2 + pra.expanded_dim(d) * 4)
+    out["state_bytes"] = state_bytes
+    out["recurrent"]["state_GBps"] = round(2 * state_bytes / (out["recurrent"]["us_per_step"] * 1e-6) / 1e9, 1)
+    out["workload"] = f"power_retention_inference bf16 b={b} h={h} d={d}: prefill 2048 (switch_over_seq_len=1024), {steps} decode steps"
+    return out
 
 
 def cpu_baseline(cfg, seconds_hint=20):
@@ -113,6 +170,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-oracle baseline leg")
     ap.add_argument("--no-breakdown", action="store_true", help="skip the per-operator timings")
+    ap.add_argument("--no-decode", action="store_true", help="skip the inference (prefill + decode) leg")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs on one GPU; --gpus N with N > 1 is not supported", file=sys.stderr)
@@ -160,15 +218,24 @@ def main():
         out["breakdown_ms"] = bd
         n = cfg["t"] // cfg["chunk"]
         bh = cfg["b"] * cfg["h"]
-        # dominant single kernel: the update_state forward contraction (sympow_tn), one launch = all chunks
+        # dominant single kernel (two launches per step, the largest share of the step): the feature-gradient
+        # contraction sympow_grad; one launch = all n chunks, algorithmic flops = the d(phi) product 2*c*D*d per
+        # (chunk, head) with the compact D
         k_flops = 2.0 * bh * n * cfg["chunk"] * D_compact * cfg["d"]
-        k_ms = bd["update_state_fwd"]
-        out["roofline"] = {"kernel": "sympow_tn_kernel (update_state forward)", "bound": "mfma",
+        k_ms = bd["sympow_grad(dK)"]
+        out["roofline"] = {"kernel": "sympow_grad_kernel (dK of update_state backward)", "bound": "mfma",
                            "achieved": round(k_flops / k_ms / 1e9, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                            "frac": round(k_flops / k_ms / 1e9 / PEAK_BF16_TFLOPS, 4), "traffic": None}
+        t_ms = bd["update_state_fwd"]
+        out["roofline_update_state_fwd"] = {"kernel": "sympow_tn_kernel", "bound": "mfma",
+                                            "achieved": round(k_flops / t_ms / 1e9, 2), "peak": PEAK_BF16_TFLOPS,
+                                            "unit": "TFLOP/s", "frac": round(k_flops / t_ms / 1e9 / PEAK_BF16_TFLOPS, 4)}
         scan_bytes = bh * expanded_dim(cfg["d"]) * cfg["d"] * (2 * n - 1) * 2
         out["discumsum_hbm"] = {"achieved": round(scan_bytes / bd["discumsum_fwd(S)"] / 1e6, 1), "peak": PEAK_HBM_GBS,
                                 "unit": "GB/s", "frac": round(scan_bytes / bd["discumsum_fwd(S)"] / 1e6 / PEAK_HBM_GBS, 4)}
+    if not args.no_decode:
+        with torch.no_grad():
+            out["decode"] = decode_bench(pra, dev)
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(cfg)
     print(json.dumps(out))

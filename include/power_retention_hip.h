@@ -71,7 +71,7 @@ int pr_update_state_fwd(const void* K, const void* V, void* S, float* s, int BN,
                         int dtype, void* stream);
 
 /* Backward -- retention/_update_state/reference.py:55-83, Triton twin retention/_update_state/triton.py:148-260.
- *   dS [BN,h,D,d], ds [BN,h,D] fp32 -> dK, dV [BN,c,h,d]. */
+ *   dS [BN,h,D,d], ds [BN,h,D] fp32 -> dK, dV [BN,c,h,d]; one of dK, dV may be NULL (that gradient is skipped). */
 int pr_update_state_bwd(const void* K, const void* V, const void* dS, const float* ds, void* dK, void* dV, int BN,
                         int c, int h, int d, int deg, int dtype, void* stream);
 

@@ -86,11 +86,14 @@ int pr_update_state_fwd(const void* K, const void* V, void* S, float* s, int BN,
 int pr_update_state_bwd(const void* K, const void* V, const void* dS, const float* ds, void* dK, void* dV, int BN,
                         int c, int h, int d, int deg, int dtype, void* stream) {
   if (int rc = check_common("update_state_bwd", d, deg, dtype, true)) return rc;
-  if (bad_ptr(K) || bad_ptr(V) || bad_ptr(dS) || bad_ptr(ds) || bad_ptr(dK) || bad_ptr(dV))
+  if (bad_ptr(K) || bad_ptr(V) || bad_ptr(dS) || bad_ptr(ds) || bad_opt(dK) || bad_opt(dV) || (!dK && !dV))
     return fail(PR_ERR_ARG, "update_state_bwd: null or misaligned pointer");
   if (BN <= 0 || c <= 0 || h <= 0) return fail(PR_ERR_ARG, "update_state_bwd: need BN,c,h > 0");
-  pr::NNArgs nn{K, dS, nullptr, dV, nullptr, nullptr, nullptr, nullptr, 1.f, c, h, 1, 1, 0};
-  if (int rc = finish(pr::sympow_nn(nn, BN, d, 1, 0, dtype, (hipStream_t)stream), "update_state_bwd(dV)")) return rc;
+  if (dV) {
+    pr::NNArgs nn{K, dS, nullptr, dV, nullptr, nullptr, nullptr, nullptr, 1.f, c, h, 1, 1, 0};
+    if (int rc = finish(pr::sympow_nn(nn, BN, d, 1, 0, dtype, (hipStream_t)stream), "update_state_bwd(dV)")) return rc;
+  }
+  if (!dK) return 0;
   pr::GradArgs g{K, V, nullptr, dS, ds, dK, c, h, 1, 1, 0};
   return finish(pr::sympow_grad(g, BN, d, 1, dtype, (hipStream_t)stream), "update_state_bwd(dK)");
 }
