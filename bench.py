@@ -96,6 +96,27 @@ def op_breakdown(pra, Q, K, V, lg, dO, cfg, iters=5):
     return {k: round(v, 4) for k, v in res.items()}
 
 
+def counter_run(pra, Q, K, V, cfg, dev):
+    """Three launches of sympow_grad alone and three plain copies of 256 MiB (read 256 MiB + write 256 MiB)."""
+    from retention_integration_amd import _lib, ops
+    b, t, h, d, c = cfg["b"], cfg["t"], cfg["h"], cfg["d"], cfg["chunk"]
+    n = t // c
+    with torch.no_grad():
+        Kc, Vc = K.view(b, n, c, h, d), V.view(b, n, c, h, d)
+        S, s = ops.update_state_fwd(Kc, Vc)
+        dK = torch.empty_like(Kc)
+        lib = _lib.load()
+        src = torch.empty(256 * 1024 * 1024, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        for _ in range(3):
+            _lib.check(lib.pr_update_state_bwd(_lib.ptr(Kc), _lib.ptr(Vc), _lib.ptr(S), _lib.ptr(s), _lib.ptr(dK), None,
+                                               b * n, c, h, d, 2, _lib.dtype_code(Kc.dtype), _lib.stream()), "grad")
+            dst.copy_(src)
+        torch.cuda.synchronize()
+    print("counter run done: 3 x sympow_grad, 3 x 256 MiB device copy")
+
+
 def decode_bench(pra, dev, steps=512):
     """BASELINE configs[3]: b=32, h=8, d=64 bf16; prefill of 2048 tokens with switch_over_seq_len=1024, then
     `steps` single-token steps.  Two loops are timed: the recurrent one (every token is folded into the state,
@@ -171,6 +192,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-oracle baseline leg")
     ap.add_argument("--no-breakdown", action="store_true", help="skip the per-operator timings")
     ap.add_argument("--no-decode", action="store_true", help="skip the inference (prefill + decode) leg")
+    ap.add_argument("--counter-run", action="store_true",
+                    help="for rocprofv3 --pmc: launch only the dominant kernel (sympow_grad, dK of update_state "
+                         "backward) a few times, and a plain device copy of 256 MiB for calibrating byte counters")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs on one GPU; --gpus N with N > 1 is not supported", file=sys.stderr)
@@ -182,6 +206,9 @@ def main():
     cfg = CFG
     dev = torch.device("cuda:0")
     Q, K, V, lg, dO = make_inputs(cfg["b"], cfg["t"], cfg["h"], cfg["d"], dev)
+    if args.counter_run:
+        counter_run(pra, Q, K, V, cfg, dev)
+        return
     leaves = [x.requires_grad_(True) for x in (Q, K, V, lg)]
 
     def step():
@@ -225,7 +252,10 @@ def main():
         k_ms = bd["sympow_grad(dK)"]
         out["roofline"] = {"kernel": "sympow_grad_kernel (dK of update_state backward)", "bound": "mfma",
                            "achieved": round(k_flops / k_ms / 1e9, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                           "frac": round(k_flops / k_ms / 1e9 / PEAK_BF16_TFLOPS, 4), "traffic": None}
+                           "frac": round(k_flops / k_ms / 1e9 / PEAK_BF16_TFLOPS, 4),
+                           # HBM bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE, calibrated with a plain
+                           # 256 MiB copy (profiles/sympow_grad_t65536_hbm_traffic.txt); algorithmic: 374.3 MB
+                           "traffic": 374.8e6}
         t_ms = bd["update_state_fwd"]
         out["roofline_update_state_fwd"] = {"kernel": "sympow_tn_kernel", "bound": "mfma",
                                             "achieved": round(k_flops / t_ms / 1e9, 2), "peak": PEAK_BF16_TFLOPS,
