@@ -12,7 +12,8 @@
 
 namespace pr {
 
-template <typename T> struct Pack16 { enum { N = 16 / sizeof(T) }; typedef __attribute__((ext_vector_type(16 / sizeof(T)))) T type; };
+template <typename T, int BYTES = 16> struct Pack16 { enum { N = BYTES / sizeof(T) }; typedef __attribute__((ext_vector_type(BYTES / sizeof(T)))) T type; };
+template <typename T> struct Pack16<T, 4> { enum { N = 1 }; struct type { T v; __device__ T& operator[](int) { return v; } __device__ const T& operator[](int) const { return v; } }; };
 
 // Sum over the 64 lanes of a wave without LDS traffic inside a row: four rotate-adds (DPP) give every lane its
 // row total, two cross-row exchanges finish.
@@ -26,11 +27,11 @@ __device__ __forceinline__ float wave_sum_dpp(float x) {
   return sum_over_rows(x);
 }
 
-template <typename T, int AHEAD>
+template <typename T, int AHEAD, int BYTES = 16>
 __global__ __launch_bounds__(256) void discumsum_fwd_kernel(const T* __restrict__ X, const float* __restrict__ logG,
                                                             T* __restrict__ Y, int n, int n_out, int H, long F) {
-  constexpr int N = Pack16<T>::N;
-  typedef typename Pack16<T>::type vec;
+  constexpr int N = Pack16<T, BYTES>::N;
+  typedef typename Pack16<T, BYTES>::type vec;
   const long per_bh = F / N;
   const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
   const int bh = blockIdx.y;
@@ -78,13 +79,13 @@ __global__ __launch_bounds__(256) void discumsum_fwd_kernel(const T* __restrict_
 // dlog_G[k] = exp(log_G[k]) * sum_F Y[k] * r_k, written as one partial per wave (summed by
 // discumsum_reduce_kernel in a fixed order, so the result is deterministic).
 // partial layout: [BH][n][waves_per_bh]
-template <typename T, int AHEAD>
+template <typename T, int AHEAD, int BYTES = 16>
 __global__ __launch_bounds__(256) void discumsum_bwd_kernel(const T* __restrict__ dY, const T* __restrict__ Y,
                                                             const float* __restrict__ logG, T* __restrict__ dX,
                                                             float* __restrict__ partial, int n, int n_out, int H,
                                                             long F, int waves_per_bh) {
-  constexpr int N = Pack16<T>::N;
-  typedef typename Pack16<T>::type vec;
+  constexpr int N = Pack16<T, BYTES>::N;
+  typedef typename Pack16<T, BYTES>::type vec;
   const long per_bh = F / N;
   const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
   const int bh = blockIdx.y;
@@ -164,6 +165,13 @@ static int launch_fwd(const void* X, const float* logG, void* Y, int B, int n, i
   constexpr int N = Pack16<T>::N;
   const long per_bh = F / N;
   dim3 grid((unsigned)((per_bh + 255) / 256), (unsigned)(B * H));
+  // very few elements (the fp32 key sums): one element per thread and every chunk's load in flight at once, so the
+  // walk costs one memory round trip instead of n
+  if (sizeof(T) == 4 && F * B * H < 256 * 1024) {
+    dim3 g1((unsigned)((F + 255) / 256), (unsigned)(B * H));
+    hipLaunchKernelGGL((discumsum_fwd_kernel<T, 64, 4>), g1, dim3(256), 0, st, (const T*)X, logG, (T*)Y, n, n_out, H, F);
+    return (int)hipGetLastError();
+  }
   // few threads in flight (small F): keep many chunks' loads outstanding per thread instead
   if (per_bh * B * H < 256 * 1024)
     hipLaunchKernelGGL((discumsum_fwd_kernel<T, 16>), grid, dim3(256), 0, st, (const T*)X, logG, (T*)Y, n, n_out, H, F);
@@ -176,6 +184,15 @@ static int launch_bwd(const void* dY, const void* Y, const float* logG, void* dX
                       int n, int n_out, int H, long F, hipStream_t st) {
   constexpr int N = Pack16<T>::N;
   const long per_bh = F / N;
+  const int tot = B * H * n;
+  if (sizeof(T) == 4 && F * B * H < 256 * 1024) {   // see launch_fwd: one element per thread, all chunks in flight
+    const unsigned b1 = (unsigned)((F + 255) / 256);
+    hipLaunchKernelGGL((discumsum_bwd_kernel<T, 64, 4>), dim3(b1, (unsigned)(B * H)), dim3(256), 0, st, (const T*)dY,
+                       (const T*)Y, logG, (T*)dX, partial, n, n_out, H, F, (int)b1 * 4);
+    hipLaunchKernelGGL(discumsum_reduce_kernel, dim3((tot * 64 + 255) / 256), dim3(256), 0, st, partial, dlogG, n, H,
+                       (int)b1 * 4, B * H);
+    return (int)hipGetLastError();
+  }
   const unsigned blocks = (unsigned)((per_bh + 255) / 256);
   const int waves = blocks * 4;
   dim3 grid(blocks, (unsigned)(B * H));
@@ -185,7 +202,6 @@ static int launch_bwd(const void* dY, const void* Y, const float* logG, void* dX
   else
     hipLaunchKernelGGL((discumsum_bwd_kernel<T, 2>), grid, dim3(256), 0, st, (const T*)dY, (const T*)Y, logG, (T*)dX,
                        partial, n, n_out, H, F, waves);
-  const int tot = B * H * n;
   hipLaunchKernelGGL(discumsum_reduce_kernel, dim3((tot * 64 + 255) / 256), dim3(256), 0, st, partial, dlogG, n, H,
                      waves, B * H);
   return (int)hipGetLastError();
@@ -201,7 +217,7 @@ int discumsum_fwd(const void* X, const float* logG, void* Y, int B, int n, int n
   return -1;
 }
 long discumsum_bwd_workspace_floats(int B, int n, int H, long F, int dtype) {
-  const int N = dtype == DT_F32 ? 4 : 8;
+  const int N = dtype == DT_F32 ? 1 : 8;   // fp32 may run one element per thread (small tensors)
   const long blocks = (F / N + 255) / 256;
   return (long)B * H * blocks * 4 * n;
 }
