@@ -119,18 +119,23 @@ int pr_chunk_prep_fwd(const float* log_G, const void* K, const void* Q, float* A
                       int c, int h, int r, int d, int deg, int dtype, void* stream);
 
 /* Backward of the same glue plus the final gradient sums (autograd of retention/power_retention_maker.py:143-193).
- *   A, lcs as above, or A = NULL for the ungated path (then lcs, dG_attn, dlcs_*, dlog_G, workspace are ignored);
- *   dKd, dQg: gradients w.r.t. Kd, Qg; dK_attn, dQ_attn, dV_attn: from the attention backward; dV_state: from the
- *   update_state backward; dG_attn [BN,c,h]: gradient w.r.t. A from the attention backward; dlcs_a, dlcs_b [BN,h]:
- *   gradients w.r.t. lcs from the two scans
- *   -> dK, dQ, dV (may alias dK_attn, dQ_attn, dV_attn), dlog_G [BN,c,h].
- *   workspace: pr_chunk_glue_bwd_workspace() bytes. */
-size_t pr_chunk_glue_bwd_workspace(int BN, int c, int h);
-int pr_chunk_glue_bwd(const float* A, const float* lcs, const void* Kd, const void* dKd, const void* Qg,
-                      const void* dQg, const void* dK_attn, const void* dQ_attn, const void* dV_attn,
-                      const void* dV_state, const float* dG_attn, const float* dlcs_a, const float* dlcs_b, void* dK,
-                      void* dQ, void* dV, float* dlog_G, void* workspace, int BN, int c, int h, int r, int d, int deg,
-                      int dtype, void* stream);
+ * The row-wise part rides in the attention backward's epilogue (no extra pass over the gradients):
+ * pr_chunk_attention_bwd is pr_attention_bwd on the chunks (B = BN, tq = tk = c, G = A) that also adds the gradients
+ * arriving through the gated copies (retention/power_retention_maker.py:163-164, 183-186):
+ *   dQ = dQ_attn + dQ_state * exp(A/deg),  dK = dK_attn + dK_state * exp((A[c-1] - A)/deg),  dV = dV_attn + dV_state,
+ *   dGq [BN,c,h*r] and dGk [BN,c,h]: gradients w.r.t. A, including (Q.dQ_state) exp(A/deg)/deg and
+ *   -(K.dK_state) exp((A[c-1]-A)/deg)/deg,  dotk [BN,c,h] = (K.dK_state) exp((A[c-1]-A)/deg).
+ *   dQ_state = gradient w.r.t. Qg (query_state backward), dK_state, dV_state = gradients w.r.t. Kd, V
+ *   (update_state backward).  With A = NULL the factors are 1 and dGq, dGk, dotk are not written.
+ * pr_chunk_gate_scan_bwd finishes the gate gradient: dlog_G holds dGk + sum over the r query heads of dGq on entry,
+ *   dlog_G[c-1] += (sum_t dotk)/deg + dlcs_a + dlcs_b, then the reverse cumulative sum over the chunk, in place. */
+int pr_chunk_attention_bwd(const void* Q, const void* K, const void* V, const float* A, const float* rowmax,
+                           const void* dO, const float* dl, const float* dO_scale, const void* dQ_state,
+                           const void* dK_state, const void* dV_state, void* dQ, void* dK, void* dV, float* dGq,
+                           float* dGk, float* dotk, int BN, int c, int h, int r, int d, float scale, int deg,
+                           int dtype, void* stream);
+int pr_chunk_gate_scan_bwd(float* dlog_G, const float* dotk, const float* dlcs_a, const float* dlcs_b, int BN, int c,
+                           int h, int deg, void* stream);
 
 /* Single-token inference step on the state -- query: retention/power_retention_maker.py:358-363 with
  * retention/_query_state/reference.py:36-96 (one query position per sequence); update:

@@ -53,6 +53,7 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dq_kernel(AttnBwdArgs a,
   typedef typename VecOf<T>::v8 v8;
   typedef typename VecOf<T>::v4 v4;
   typedef __attribute__((address_space(3))) v8 lds_v8;
+  typedef __attribute__((address_space(3))) v4 lds_v4;
   constexpr int KS = DH / 32, NT = DH / 16, KT = AB_BN / 16, ROWS = 64 * MT, CPR = DH / 8, RB = CPR * 16;
   constexpr int TILE = AB_BN * RB;
   constexpr int STAGE = 2 * TILE + 4 * AB_BN * 4;   // K, V, raw gates, two sets of key gate factors
@@ -94,8 +95,24 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dq_kernel(AttnBwdArgs a,
     const int pos = (ii * 4 + wave) * 64 + l, row = pos / CPR;
     goff[ii] = (uint32_t)(row * (int)kstride + 16 * ((pos % CPR) ^ swz<CPR>(row)));
   }
+  // With the chunked epilogue the workgroup's rows of dQs ride through the ring as one more stage after the last
+  // key tile (rows 0..63 in the K area, 64..127 in the V area), so that they arrive under the last tiles' work.
+  const T* dQsg = a.dQs ? (const T*)a.dQs + (long)b * a.tq * hq * DH : nullptr;
+  const int ntot = ntiles + (dQsg ? 1 : 0);
   auto issue = [&](int it) {
     char* st = smem + (it % AB_NST) * STAGE;
+    if (it >= ntiles) {
+#pragma unroll
+      for (int ii = 0; ii < LOADS; ii++) {
+        const int pos = ((ii % (LOADS / 2)) * 4 + wave) * 64 + l, row = pos / CPR;
+        const int fr = min(row0 + (ii / (LOADS / 2)) * AB_BN + row, rows - 1), t = fr / a.r;
+        const long eo = ((long)t * hq + hh * a.r + (fr - t * a.r)) * DH;
+        async_copy16((const char*)(dQsg + eo) + 16 * ((pos % CPR) ^ swz<CPR>(row)),
+                     st + (ii / (LOADS / 2)) * TILE + ((ii % (LOADS / 2)) * 4 + wave) * 1024);
+      }
+      if (Gg && wave == 0) async_copy4(Gg, st + 2 * TILE);   // keeps the count of copies per stage fixed
+      return;
+    }
     const int j0 = it * AB_BN;
     if (j0 + AB_BN <= a.tk) {
       const char* kb_ = Kg + (long)j0 * kstride;
@@ -111,7 +128,7 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dq_kernel(AttnBwdArgs a,
     if (Gg && wave == 0) async_copy4(Gg + (long)min(j0 + l, a.tk - 1) * a.h, st + 2 * TILE);
   };
   issue(0);
-  if (ntiles > 1) issue(1);
+  if (ntot > 1) issue(1);
 
   v8 Qf[MT][KS], dOf[MT][KS];
   int ti[MT];
@@ -182,11 +199,11 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dq_kernel(AttnBwdArgs a,
   }
   auto sync_step = [&](int it) -> char* {
     char* st = smem + (it % AB_NST) * STAGE;
-    if (it + 1 < ntiles) wait_vmcnt<LOADS>(); else wait_vmcnt<0>();
+    if (it + 1 < ntot) wait_vmcnt<LOADS>(); else wait_vmcnt<0>();
     lds_barrier();
-    if (it + 2 < ntiles) issue(it + 2);
+    if (it + 2 < ntot) issue(it + 2);
     if (wave == 0 && it + 1 < ntiles) {
-      if (it + 2 < ntiles) wait_vmcnt<LOADS + 1>(); else wait_vmcnt<0>();   // all but the stage just issued
+      if (it + 2 < ntot) wait_vmcnt<LOADS + 1>(); else wait_vmcnt<0>();   // all but the stage just issued
       gate_factors(it + 1);
     }
     return st;
@@ -299,15 +316,44 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dq_kernel(AttnBwdArgs a,
   for (; it < ntiles; it++) sync_step(it);
 
   T* dQg = (T*)a.dQ + (long)b * a.tq * hq * DH;
+  uint32_t ep = 0;
+  if (dQsg) {
+    wait_vmcnt<0>();
+    lds_barrier();
+    ep = (uint32_t)(uintptr_t)(ab_lds_char*)(smem + (ntiles % AB_NST) * STAGE);
+  }
 #pragma unroll
   for (int mi = 0; mi < MT; mi++) {
-    const float tot = sum_over_rows(dgq[mi]);
+    float tot = sum_over_rows(dgq[mi]);
+    float u = 1.f;
+    v4 add4[NT];
+    if (dQsg) {   // gradient through the gated copy of Q: dQs * u, and (Q . dQs) u / deg for the gate
+      const int lr = wslice * 16 * MT + 16 * mi;
+      const uint32_t rb = ep + (lr / AB_BN) * TILE + (lr % AB_BN) * RB;
+      u = Gg ? __expf(Gg[(long)ti[mi] * a.h] / a.deg) : 1.f;
+      float dotq = 0.f;
+#pragma unroll
+      for (int ks = 0; ks < KS; ks++) {
+        float q8[8], d8[8];
+        unpack8(Qf[mi][ks], q8);
+        unpack8((v8)(*(const lds_v8*)(rb + koff[ks])), d8);
+#pragma unroll
+        for (int i = 0; i < 8; i++) dotq = __builtin_fmaf(q8[i], d8[i], dotq);
+      }
+#pragma unroll
+      for (int nt = 0; nt < NT; nt++)
+        add4[nt] = *(const lds_v4*)(rb + tcol * RB + (((2 * nt + (g >> 1)) ^ swz<CPR>(tcol)) * 16) + (g & 1) * 8);
+      tot += sum_over_rows(dotq) * u / a.deg;
+    }
     if (!live[mi]) continue;
 #pragma unroll
     for (int nt = 0; nt < NT; nt++) {
       float o4[4];
 #pragma unroll
-      for (int v = 0; v < 4; v++) o4[v] = acc[mi][nt][v] * a.deg;
+      for (int v = 0; v < 4; v++) {
+        o4[v] = acc[mi][nt][v] * a.deg;
+        if (dQsg) o4[v] = __builtin_fmaf((float)add4[nt][v], u, o4[v]);
+      }
       *(v4*)(dQg + qoff[mi] * DH + 16 * nt + 4 * g) = pack4<T>(o4);
     }
     if (g == 0 && a.dGq) a.dGq[(long)b * a.tq * hq + qoff[mi]] = tot;
@@ -325,6 +371,7 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
   typedef typename VecOf<T>::v8 v8;
   typedef typename VecOf<T>::v4 v4;
   typedef __attribute__((address_space(3))) v8 lds_v8;
+  typedef __attribute__((address_space(3))) v4 lds_v4;
   constexpr int KS = DH / 32, NT = DH / 16, QT = AB_BM / 16, KEYS = 64 * MK, CPR = DH / 8, RB = CPR * 16;
   constexpr int TILE = AB_BM * RB;
   // row vectors of a stage, AB_BM floats each: [0] G_q (raw) -> G_q - m, [1] m (raw) -> time index (as a float),
@@ -384,8 +431,28 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
     const int t = row / a.r;
     return (long)t * hq + hh * a.r + (row - t * a.r);
   };
+  // With the chunked epilogue the workgroup's rows of dKs and dVs ride through the ring as two more stages after
+  // the last row tile (keys 0..63 in the Q area, 64..127 in the dO area): they arrive under the last tiles' work.
+  const T* dKsg = a.dKs ? (const T*)a.dKs + (long)b * a.tk * a.h * DH + hh * DH : nullptr;
+  const T* dVsg = a.dVs ? (const T*)a.dVs + (long)b * a.tk * a.h * DH + hh * DH : nullptr;
+  const int ntot = nsteps + (dKsg ? 2 : 0);
   auto issue = [&](int step) {
     char* st = smem + (step % AB_NST) * STAGE;
+    if (step >= nsteps) {
+      const T* src = step == nsteps ? dKsg : dVsg;
+#pragma unroll
+      for (int ii = 0; ii < LOADS; ii++) {
+        const int half = ii / (LOADS / 2), i2 = ii % (LOADS / 2);
+        const long eo = (long)min(key0 + half * AB_BM + (int)grow[i2], a.tk - 1) * kstride;
+        async_copy16((const char*)(src + eo) + gchk[i2], st + half * TILE + (i2 * 4 + wave) * 1024);
+      }
+      if (wave == 0) {   // keeps the count of copies per stage fixed
+        float* rv = (float*)(st + 2 * TILE);
+#pragma unroll
+        for (int i = 0; i < 4; i++) async_copy4(rmg, rv + i * AB_BM);
+      }
+      return;
+    }
     const int rbase = (ntile_total - 1 - step) * AB_BM;
 #pragma unroll
     for (int ii = 0; ii < LOADS / 2; ii++) {
@@ -404,8 +471,8 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
       async_copy4(osg ? osg + ro : rmg + ro, rv + 3 * AB_BM);
     }
   };
-  if (nsteps > 0) issue(0);
-  if (nsteps > 1) issue(1);
+  if (ntot > 0) issue(0);
+  if (ntot > 1) issue(1);
 
   v8 Kf[MK][KS], Vf[MK][KS];
   int key[MK];
@@ -475,11 +542,11 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
   }
   auto sync_step = [&](int step) -> char* {
     char* st = smem + (step % AB_NST) * STAGE;
-    if (step + 1 < nsteps) wait_vmcnt<LOADS>(); else wait_vmcnt<0>();
+    if (step + 1 < ntot) wait_vmcnt<LOADS>(); else wait_vmcnt<0>();
     lds_barrier();
-    if (step + 2 < nsteps) issue(step + 2);
+    if (step + 2 < ntot) issue(step + 2);
     if (wave == 0 && step + 1 < nsteps) {
-      if (step + 2 < nsteps) wait_vmcnt<LOADS + 4>(); else wait_vmcnt<0>();   // all but the stage just issued
+      if (step + 2 < ntot) wait_vmcnt<LOADS + 4>(); else wait_vmcnt<0>();   // all but the stage just issued
       row_factors(step + 1);
     }
     return st;
@@ -614,9 +681,40 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
 
   T* dKg = (T*)a.dK + (long)b * a.tk * a.h * DH + hh * DH;
   T* dVg = (T*)a.dV + (long)b * a.tk * a.h * DH + hh * DH;
+  uint32_t epk = 0, epv = 0;
+  if (dKsg) {
+    wait_vmcnt<0>();
+    lds_barrier();
+    epk = (uint32_t)(uintptr_t)(ab_lds_char*)(smem + (nsteps % AB_NST) * STAGE);
+    epv = (uint32_t)(uintptr_t)(ab_lds_char*)(smem + ((nsteps + 1) % AB_NST) * STAGE);
+  }
+  const float Glast = Gg ? Gg[(long)(a.tk - 1) * a.h] : 0.f;
 #pragma unroll
   for (int kj = 0; kj < MK; kj++) {
-    const float tot = sum_over_rows(dgk[kj]);
+    float tot = sum_over_rows(dgk[kj]);
+    float w = 1.f, dotk = 0.f;
+    v4 addk[NT], addv[NT];
+    if (dKsg) {   // gradient through the discounted copy of K: dKs * w, and -(K . dKs) w / deg for the gate
+      const int lr = wslice * 16 * MK + 16 * kj;
+      const uint32_t ro = (lr / AB_BM) * TILE + (lr % AB_BM) * RB;
+      w = Gg ? __expf((Glast - Gk[kj]) / a.deg) : 1.f;
+#pragma unroll
+      for (int ks = 0; ks < KS; ks++) {
+        float k8[8], d8[8];
+        unpack8(Kf[kj][ks], k8);
+        unpack8((v8)(*(const lds_v8*)(epk + ro + qoff_[ks])), d8);
+#pragma unroll
+        for (int i = 0; i < 8; i++) dotk = __builtin_fmaf(k8[i], d8[i], dotk);
+      }
+#pragma unroll
+      for (int nt = 0; nt < NT; nt++) {
+        const uint32_t co = ro + kcol * RB + (((2 * nt + (g >> 1)) ^ swz<CPR>(kcol)) * 16) + (g & 1) * 8;
+        addk[nt] = *(const lds_v4*)(epk + co);
+        addv[nt] = *(const lds_v4*)(epv + co);
+      }
+      dotk = sum_over_rows(dotk) * w;
+      tot += dotk / a.deg;
+    }
     if (!live[kj]) continue;
 #pragma unroll
     for (int nt = 0; nt < NT; nt++) {
@@ -625,11 +723,19 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
       for (int v = 0; v < 4; v++) {
         k4[v] = accK[kj][nt][v] * a.deg;
         v4f[v] = accV[kj][nt][v];
+        if (dKsg) {
+          k4[v] = __builtin_fmaf((float)addk[nt][v], w, k4[v]);
+          v4f[v] += (float)addv[nt][v];
+        }
       }
       *(v4*)(dKg + key[kj] * kstride + 16 * nt + 4 * g) = pack4<T>(k4);
       *(v4*)(dVg + key[kj] * kstride + 16 * nt + 4 * g) = pack4<T>(v4f);
     }
-    if (g == 0 && a.dGk) a.dGk[((long)b * a.tk + key[kj]) * a.h + hh] = -tot;
+    if (g == 0) {
+      const long go = ((long)b * a.tk + key[kj]) * a.h + hh;
+      if (a.dGk) a.dGk[go] = -tot;
+      if (a.dotk) a.dotk[go] = dotk;
+    }
   }
 }
 

@@ -71,8 +71,26 @@ int pr_attention_bwd(const void* Q, const void* K, const void* V, const float* G
   if (B <= 0 || tq <= 0 || tk <= 0 || h <= 0 || r <= 0 || tq > tk)
     return fail(PR_ERR_ARG, "attention_bwd: need B,tq,tk,h,r > 0 and tq <= tk");
   pr::AttnBwdArgs a{Q, K, V, G, rowmax, dO, dl, dO_scale, dQ, dK, dV, G ? dGq : nullptr, G ? dGk : nullptr,
-                    tq, tk, h, r, scale, (float)deg};
+                    tq, tk, h, r, scale, (float)deg, nullptr, nullptr, nullptr, nullptr};
   return finish(pr::attention_bwd(a, B, d, dtype, (hipStream_t)stream), "attention_bwd");
+}
+
+int pr_chunk_attention_bwd(const void* Q, const void* K, const void* V, const float* A, const float* rowmax,
+                           const void* dO, const float* dl, const float* dO_scale, const void* dQ_state,
+                           const void* dK_state, const void* dV_state, void* dQ, void* dK, void* dV, float* dGq,
+                           float* dGk, float* dotk, int BN, int c, int h, int r, int d, float scale, int deg,
+                           int dtype, void* stream) {
+  if (int rc = check_common("chunk_attention_bwd", d, deg, dtype, false)) return rc;
+  if (bad_ptr(Q) || bad_ptr(K) || bad_ptr(V) || bad_ptr(rowmax) || bad_ptr(dO) || bad_ptr(dQ) || bad_ptr(dK) ||
+      bad_ptr(dV) || bad_ptr(dQ_state) || bad_ptr(dK_state) || bad_ptr(dV_state) || bad_opt(A) || bad_opt(dl) ||
+      bad_opt(dGq) || bad_opt(dGk))
+    return fail(PR_ERR_ARG, "chunk_attention_bwd: null or misaligned pointer");
+  if (A && (!dGq || !dGk || !dotk))
+    return fail(PR_ERR_ARG, "chunk_attention_bwd: dGq, dGk and dotk are required when A is given");
+  if (BN <= 0 || c <= 0 || h <= 0 || r <= 0) return fail(PR_ERR_ARG, "chunk_attention_bwd: need BN,c,h,r > 0");
+  pr::AttnBwdArgs a{Q, K, V, A, rowmax, dO, dl, dO_scale, dQ, dK, dV, A ? dGq : nullptr, A ? dGk : nullptr,
+                    c, c, h, r, scale, (float)deg, dQ_state, dK_state, dV_state, A ? dotk : nullptr};
+  return finish(pr::attention_bwd(a, BN, d, dtype, (hipStream_t)stream), "chunk_attention_bwd");
 }
 
 int pr_update_state_fwd(const void* K, const void* V, void* S, float* s, int BN, int c, int h, int d, int deg,
@@ -180,28 +198,13 @@ int pr_chunk_prep_fwd(const float* log_G, const void* K, const void* Q, float* A
                 "chunk_prep_fwd");
 }
 
-size_t pr_chunk_glue_bwd_workspace(int BN, int c, int h) {
-  return (size_t)pr::chunk_glue_bwd_workspace_floats(BN, c, h) * sizeof(float);
+int pr_chunk_gate_scan_bwd(float* dlog_G, const float* dotk, const float* dlcs_a, const float* dlcs_b, int BN, int c,
+                           int h, int deg, void* stream) {
+  if (!dlog_G || !dotk || !dlcs_a || !dlcs_b) return fail(PR_ERR_ARG, "chunk_gate_scan_bwd: null pointer");
+  if (BN <= 0 || c <= 0 || h <= 0 || deg <= 0) return fail(PR_ERR_ARG, "chunk_gate_scan_bwd: need BN,c,h,deg > 0");
+  return finish(pr::chunk_gate_scan_bwd(dlog_G, dotk, dlcs_a, dlcs_b, BN, c, h, deg, (hipStream_t)stream),
+                "chunk_gate_scan_bwd");
 }
-
-int pr_chunk_glue_bwd(const float* A, const float* lcs, const void* Kd, const void* dKd, const void* Qg,
-                      const void* dQg, const void* dK_attn, const void* dQ_attn, const void* dV_attn,
-                      const void* dV_state, const float* dG_attn, const float* dlcs_a, const float* dlcs_b, void* dK,
-                      void* dQ, void* dV, float* dlog_G, void* workspace, int BN, int c, int h, int r, int d, int deg,
-                      int dtype, void* stream) {
-  if (int rc = check_common("chunk_glue_bwd", d, deg, dtype, false)) return rc;
-  if (bad_ptr(Kd) || bad_ptr(dKd) || bad_ptr(Qg) || bad_ptr(dQg) || bad_ptr(dK_attn) || bad_ptr(dQ_attn) ||
-      bad_ptr(dV_attn) || bad_ptr(dV_state) || bad_ptr(dK) || bad_ptr(dQ) || bad_ptr(dV))
-    return fail(PR_ERR_ARG, "chunk_glue_bwd: null or misaligned pointer");
-  if (A && (!lcs || !dG_attn || !dlcs_a || !dlcs_b || !dlog_G || !workspace))
-    return fail(PR_ERR_ARG, "chunk_glue_bwd: gated call needs lcs, dG_attn, dlcs_a, dlcs_b, dlog_G and workspace");
-  if (BN <= 0 || c <= 0 || h <= 0 || r <= 0) return fail(PR_ERR_ARG, "chunk_glue_bwd: need BN,c,h,r > 0");
-  return finish(pr::chunk_glue_bwd(A, lcs, Kd, dKd, Qg, dQg, dK_attn, dQ_attn, dV_attn, dV_state, dG_attn, dlcs_a,
-                                   dlcs_b, dK, dQ, dV, dlog_G, (float*)workspace, BN, c, h, r, d, deg, dtype,
-                                   (hipStream_t)stream),
-                "chunk_glue_bwd");
-}
-
 
 size_t pr_decode_step_workspace(int B, int tq, int h, int r, int d) {
   return align256((size_t)pr::decode_workspace_floats(B, h, r, tq, d) * sizeof(float));

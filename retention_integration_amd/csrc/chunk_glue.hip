@@ -83,90 +83,6 @@ __global__ __launch_bounds__(256) void gate_apply_fwd_kernel(const float* __rest
   }
 }
 
-struct GlueBwdArgs {
-  const float* A;       // [BN, c, h] or null (ungated)
-  const float* lcs;     // [BN, h]
-  const void* Kd;       // [BN, c, h, d]
-  const void* dKd;      // [BN, c, h, d]
-  const void* Qg;       // [BN, c, hq, d]
-  const void* dQg;      // [BN, c, hq, d]
-  const void* dK_attn;  // [BN, c, h, d]
-  const void* dQ_attn;  // [BN, c, hq, d]
-  const void* dV_attn;  // [BN, c, h, d]
-  const void* dV_state; // [BN, c, h, d]
-  const float* dG_attn; // [BN, c, h]
-  void* dK;
-  void* dQ;
-  void* dV;
-  float* dA;            // [BN, c, h]  (the dlog_G buffer; scanned in place afterwards)
-  float* dotk;          // [BN, c, h]  workspace: sum_d dKd.Kd per row
-  long groups;
-  int c, h, r;
-  float inv_deg;
-};
-
-template <typename T, int DH> __global__ __launch_bounds__(256) void glue_rows_bwd_kernel(GlueBwdArgs g) {
-  typedef typename VecOf<T>::v8 v8;
-  constexpr int LPR = DH / 8;
-  const long gid = ((long)blockIdx.x * 256 + threadIdx.x) / LPR;
-  const bool live = gid < g.groups;
-  const long gi = live ? gid : 0;
-  const int sub = threadIdx.x % LPR, col = sub * 8;
-  const int hh = (int)(gi % g.h);
-  const long bn = gi / ((long)g.c * g.h);
-  const bool gated = g.A != nullptr;
-  float w = 1.f, u = 1.f;
-  if (gated) {
-    const float at = g.A[gi], al = g.lcs[bn * g.h + hh];
-    w = __expf((al - at) * g.inv_deg);
-    u = __expf(at * g.inv_deg);
-  }
-  float dotk = 0.f, dotq = 0.f;
-  {
-    const long o = gi * DH + col;
-    float kd[8], dkd[8], dka[8], dva[8], dvs[8], ok[8], ov[8];
-    unpack8(*(const v8*)((const T*)g.Kd + o), kd);
-    unpack8(*(const v8*)((const T*)g.dKd + o), dkd);
-    unpack8(*(const v8*)((const T*)g.dK_attn + o), dka);
-    unpack8(*(const v8*)((const T*)g.dV_attn + o), dva);
-    unpack8(*(const v8*)((const T*)g.dV_state + o), dvs);
-#pragma unroll
-    for (int i = 0; i < 8; i++) {
-      dotk += kd[i] * dkd[i];
-      ok[i] = dka[i] + dkd[i] * w;
-      ov[i] = dva[i] + dvs[i];
-    }
-    if (live) {
-      *(v8*)((T*)g.dK + o) = pack8<T>(ok);
-      *(v8*)((T*)g.dV + o) = pack8<T>(ov);
-    }
-  }
-  for (int rr = 0; rr < g.r; rr++) {
-    const long o = (gi * g.r + rr) * DH + col;
-    float qg[8], dqg[8], dqa[8], oq[8];
-    unpack8(*(const v8*)((const T*)g.Qg + o), qg);
-    unpack8(*(const v8*)((const T*)g.dQg + o), dqg);
-    unpack8(*(const v8*)((const T*)g.dQ_attn + o), dqa);
-#pragma unroll
-    for (int i = 0; i < 8; i++) {
-      dotq += qg[i] * dqg[i];
-      oq[i] = dqa[i] + dqg[i] * u;
-    }
-    if (live) *(v8*)((T*)g.dQ + o) = pack8<T>(oq);
-  }
-  if (gated) {
-#pragma unroll
-    for (int m = 1; m < LPR; m <<= 1) {
-      dotk += __shfl_xor(dotk, m);
-      dotq += __shfl_xor(dotq, m);
-    }
-    if (live && sub == 0) {
-      g.dA[gi] = g.dG_attn[gi] + (dotq - dotk) * g.inv_deg;
-      g.dotk[gi] = dotk;
-    }
-  }
-}
-
 // dA[c-1] += (sum_t dotk)/deg + dlcs_a + dlcs_b, then dlog_G = reverse cumsum of dA (in place)
 __global__ __launch_bounds__(256) void gate_scan_bwd_kernel(float* __restrict__ dA, const float* __restrict__ dotk,
                                                             const float* __restrict__ dlcs_a,
@@ -218,34 +134,12 @@ int chunk_prep_fwd(const float* logG, const void* K, const void* Q, float* A, fl
   return -1;
 }
 
-long chunk_glue_bwd_workspace_floats(int BN, int c, int h) { return (long)BN * c * h; }
-
-int chunk_glue_bwd(const float* A, const float* lcs, const void* Kd, const void* dKd, const void* Qg, const void* dQg,
-                   const void* dK_attn, const void* dQ_attn, const void* dV_attn, const void* dV_state,
-                   const float* dG_attn, const float* dlcs_a, const float* dlcs_b, void* dK, void* dQ, void* dV,
-                   float* dlogG, float* workspace, int BN, int c, int h, int r, int d, int deg, int dtype,
-                   hipStream_t st) {
+int chunk_gate_scan_bwd(float* dA, const float* dotk, const float* dlcs_a, const float* dlcs_b, int BN, int c, int h,
+                        int deg, hipStream_t st) {
   if (c > GLUE_MAX_C) return -5;
-  const long groups = (long)BN * c * h;
-  GlueBwdArgs g{A, lcs, Kd, dKd, Qg, dQg, dK_attn, dQ_attn, dV_attn, dV_state, dG_attn,
-                dK, dQ, dV, dlogG, workspace, groups, c, h, r, 1.f / deg};
-#define PR_GB(T, DD)                                                                                                   \
-  case DD:                                                                                                             \
-    hipLaunchKernelGGL((glue_rows_bwd_kernel<T, DD>), dim3((unsigned)((groups * (DD / 8) + 255) / 256)), dim3(256), 0,  \
-                       st, g);                                                                                         \
-    break;
-#define PR_GBT(T)                                                                                                      \
-  switch (d) { PR_GB(T, 32) PR_GB(T, 64) PR_GB(T, 128) default: return -2; }
-  if (dtype == DT_BF16) { PR_GBT(bf16_t) }
-  else if (dtype == DT_F16) { PR_GBT(f16_t) }
-  else return -1;
-#undef PR_GBT
-#undef PR_GB
-  if (A) {
-    const size_t smem = (size_t)(c + 256) * sizeof(float);
-    hipLaunchKernelGGL(gate_scan_bwd_kernel, dim3((unsigned)(BN * h)), dim3(256), smem, st, dlogG, workspace, dlcs_a,
-                       dlcs_b, c, h, 1.f / deg);
-  }
+  const size_t smem = (size_t)(c + 256) * sizeof(float);
+  hipLaunchKernelGGL(gate_scan_bwd_kernel, dim3((unsigned)(BN * h)), dim3(256), smem, st, dA, dotk, dlcs_a, dlcs_b, c,
+                     h, 1.f / deg);
   return (int)hipGetLastError();
 }
 

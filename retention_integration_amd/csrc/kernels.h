@@ -75,6 +75,12 @@ struct AttnBwdArgs {
   float* dGk;           // [B, tk, h]     (only when G; already negated)
   int tq, tk, h, r;
   float scale, deg;
+  // optional epilogue of the chunked algorithm (all null otherwise): gradients that arrive through the gated
+  // copies Q*exp(G/deg) and K*exp((G_last - G)/deg) and the value gradient of the state path
+  const void* dQs;      // [B, tq, h*r, d]: dQ = dQ_attn + dQs * exp(G_q/deg);  dGq += (Q.dQs) exp(G_q/deg) / deg
+  const void* dKs;      // [B, tk, h, d]:   dK = dK_attn + dKs * w, w = exp((G_last - G_k)/deg); dGk -= (K.dKs) w / deg
+  const void* dVs;      // [B, tk, h, d]:   dV = dV_attn + dVs
+  float* dotk;          // [B, tk, h]:      (K.dKs) w
 };
 int attention_bwd(const AttnBwdArgs& a, int B, int d, int dtype, hipStream_t st);
 
@@ -85,12 +91,8 @@ int qs_bwd_prep(const void* O, const void* dO, const float* den, const float* ro
 // chunk_glue.hip (return -5: chunk longer than the LDS-resident gate vector allows)
 int chunk_prep_fwd(const float* logG, const void* K, const void* Q, float* A, float* lcs, void* Kd, void* Qg, int BN,
                    int c, int h, int r, int d, int deg, int dtype, hipStream_t st);
-long chunk_glue_bwd_workspace_floats(int BN, int c, int h);
-int chunk_glue_bwd(const float* A, const float* lcs, const void* Kd, const void* dKd, const void* Qg, const void* dQg,
-                   const void* dK_attn, const void* dQ_attn, const void* dV_attn, const void* dV_state,
-                   const float* dG_attn, const float* dlcs_a, const float* dlcs_b, void* dK, void* dQ, void* dV,
-                   float* dlogG, float* workspace, int BN, int c, int h, int r, int d, int deg, int dtype,
-                   hipStream_t st);
+int chunk_gate_scan_bwd(float* dA, const float* dotk, const float* dlcs_a, const float* dlcs_b, int BN, int c, int h,
+                        int deg, hipStream_t st);
 
 // decode.hip (return -3: more than 8 query rows per (batch, kv head))
 long decode_workspace_floats(int B, int h, int r, int tq, int d);

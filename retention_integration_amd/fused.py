@@ -87,16 +87,6 @@ class _ChunkedPowerRetention(torch.autograd.Function):
         _lib.check(lib.pr_query_state_bwd(p(Qg), p(Sc), p(sc), p(rm), p(O), p(den), p(dO), p(dQg), p(dSc), p(dsc),
                                           p(dYa), p(dla), p(ws), BN, n, c, h, r, d, scale ** deg, 2, 1, code, st),
                    "query_state_bwd")
-        dQa, dKa, dVa = torch.empty_like(Q), torch.empty_like(K), torch.empty_like(V)
-        dGq = _empty((BN, c, hq), f32, dev) if gated else None
-        dGk = _empty((BN, c, h), f32, dev) if gated else None
-        _lib.check(lib.pr_attention_bwd(p(Q), p(K), p(V), p(A), p(rm), p(dYa), p(dla), None, p(dQa), p(dKa), p(dVa),
-                                        p(dGq), p(dGk), BN, c, c, h, r, d, scale, deg, code, st), "attention_bwd")
-        if gated:
-            dGa = dGk.add_(dGq.view(BN, c, h, r).sum(-1)) if r > 1 else dGk.add_(dGq)
-        else:
-            dGa = None
-
         dS, ds = torch.empty_like(Sc), torch.empty_like(sc)
         dl1, dl2 = torch.empty_like(lcs), torch.empty_like(lcs)
         ws = _empty((max(lib.pr_discumsum_bwd_workspace(b, n, h, D * d, code),
@@ -108,12 +98,20 @@ class _ChunkedPowerRetention(torch.autograd.Function):
         dKd, dVs = torch.empty_like(K), torch.empty_like(V)
         _lib.check(lib.pr_update_state_bwd(p(Kd), p(V), p(dS), p(ds), p(dKd), p(dVs), BN, c, h, d, 2, code, st),
                    "update_state_bwd")
-        dlg = _empty((b, t, h), f32, dev) if gated else None
-        # results are written in place over the attention gradients
-        ws = _empty((lib.pr_chunk_glue_bwd_workspace(BN, c, h),), u8, dev) if gated else None
-        _lib.check(lib.pr_chunk_glue_bwd(p(A), p(lcs), p(Kd), p(dKd), p(Qg), p(dQg), p(dKa), p(dQa), p(dVa), p(dVs),
-                                         p(dGa), p(dl1), p(dl2), p(dKa), p(dQa), p(dVa), p(dlg), p(ws), BN, c, h, r, d,
-                                         deg, code, st), "chunk_glue_bwd")
+
+        # the attention backward adds the state-path gradients in its epilogue and writes the final dQ, dK, dV
+        dQa, dKa, dVa = torch.empty_like(Q), torch.empty_like(K), torch.empty_like(V)
+        dGq = _empty((BN, c, hq), f32, dev) if gated else None
+        dGk = _empty((b, t, h), f32, dev) if gated else None
+        dotk = _empty((BN, c, h), f32, dev) if gated else None
+        _lib.check(lib.pr_chunk_attention_bwd(p(Q), p(K), p(V), p(A), p(rm), p(dYa), p(dla), None, p(dQg), p(dKd),
+                                              p(dVs), p(dQa), p(dKa), p(dVa), p(dGq), p(dGk), p(dotk), BN, c, h, r, d,
+                                              scale, deg, code, st), "chunk_attention_bwd")
+        dlg = None
+        if gated:
+            dlg = dGk.add_(dGq.view(b, t, h, r).sum(-1)) if r > 1 else dGk.add_(dGq.view(b, t, h))
+            _lib.check(lib.pr_chunk_gate_scan_bwd(p(dlg), p(dotk), p(dl1), p(dl2), BN, c, h, deg, st),
+                       "chunk_gate_scan_bwd")
         return dQa, dKa, dVa, dlg, None, None, None
 
 
