@@ -146,6 +146,23 @@ __device__ __forceinline__ void async_copy4(const void* gsrc, void* lds_wave_bas
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" ::"s"(base), "v"(gsrc) : "memory", "m0");
 }
 
+// The same copies with the global address split into a wave-uniform base (scalar registers) and a per-lane byte
+// offset, so that stepping the base through memory costs no vector instruction.  lds_wave_base is the wave-uniform
+// LDS byte address (lane i's bytes land at lds_wave_base + 16*i, resp. 4*i).
+__device__ __forceinline__ void async_copy16_sv(const void* uniform_base, uint32_t lane_off, uint32_t lds_wave_base) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_wave_base), "v"(lane_off),
+               "s"(uniform_base)
+               : "memory", "m0");
+}
+__device__ __forceinline__ void async_copy4_sv(const void* uniform_base, uint32_t lane_off, uint32_t lds_wave_base) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" ::"s"(lds_wave_base), "v"(lane_off),
+               "s"(uniform_base)
+               : "memory", "m0");
+}
+__device__ __forceinline__ uint32_t lds_addr(const void* p) {
+  return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char*)p;
+}
+
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() also drains the vector-memory counter, which
 // would make every asynchronous global->LDS copy (and every register prefetch) in flight complete at each barrier;
 // here only this wave's LDS operations are waited for, and copies are tracked by wait_vmcnt<N>() alone.  The asm

@@ -45,11 +45,16 @@ __device__ __forceinline__ void tn_body(const T* __restrict__ A, const T* __rest
                                         T* __restrict__ S, float* __restrict__ s, int c, int hA, int r, int hh,
                                         int bn, int h, int y, int xb, bool active, bool use_mult, char* smem) {
   typedef typename VecOf<T>::v8 v8;
+  typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+  typedef __attribute__((address_space(3))) f32x4 lds_f32x4;
   constexpr int NT = DV / 16, CA = DK / 8, CB = DV / 8;            // 16-byte chunks per row
   constexpr int A_BYTES = TN_KT * DK * 2, B_BYTES = TN_KT * DV * 2, W_BYTES = TN_KT * 4;
   constexpr int STAGE = A_BYTES + B_BYTES + W_BYTES;
-  constexpr int LOADS = (TN_KT * CA + TN_KT * CB) / 256;           // copies per thread per stage (w rides on wave 0)
+  constexpr int LA = TN_KT * CA / 256, LB = TN_KT * CB / 256;      // copies per thread per stage (w rides on wave 0)
+  constexpr int LOADS = LA + LB;
+  static_assert(CA == CB && TN_KT == 64 && TN_NST == 3, "the loop below is written for this shape");
   const int tid = threadIdx.x, l = tid & 63, g = l >> 4;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int rows = c * r;
   const char* a_base = (const char*)(A + (long)bn * c * hA * DK);
   const char* b_base = (const char*)(Bm + (long)bn * c * hA * DV);
@@ -59,12 +64,38 @@ __device__ __forceinline__ void tn_body(const T* __restrict__ A, const T* __rest
     const int t = row / r, rr = row - t * r;
     return (long)t * hA + hh * r + rr;
   };
+  // Copies of one stage.  When a stage is a whole number of time steps (TN_KT % r == 0) the folded rows of stage
+  // k+1 are those of stage k moved by a fixed distance: lane offsets are computed once, the base moves in scalar
+  // registers.  Other shapes and the partial last stage take the general path.
+  const bool regular = (TN_KT % r) == 0;
+  static_assert(DK == DV, "the A and B tiles share the copy offsets");
+  uint32_t voffA[LA], voffW = 0;
+#pragma unroll
+  for (int ii = 0; ii < LA; ii++) {
+    const int pos = (ii * 4 + wave) * 64 + l, row = pos / CA;
+    voffA[ii] = (uint32_t)(row_index(row) * (DK * 2) + 16 * ((pos % CA) ^ swz<CA>(row)));
+  }
+  if (HAS_W) voffW = (uint32_t)(row_index(l) * 4);
+  const long stage_rows = (long)(TN_KT / max(r, 1)) * hA;   // rows of the [c, hA] arrays per stage (regular shapes)
+  const uint32_t smem_a = lds_addr(smem);
   auto issue = [&](int step) {
-    char* st = smem + (step % TN_NST) * STAGE;
+    const int slot = step % TN_NST;
     const int r0 = step * TN_KT;
+    if (regular && r0 + TN_KT <= rows) {
+      const uint32_t sa = smem_a + slot * STAGE + wave * 1024;
+      const char* ab = a_base + step * stage_rows * (DK * 2);
+      const char* bb = b_base + step * stage_rows * (DV * 2);
+#pragma unroll
+      for (int ii = 0; ii < LA; ii++) async_copy16_sv(ab, voffA[ii], sa + ii * 4096);
+#pragma unroll
+      for (int ii = 0; ii < LB; ii++) async_copy16_sv(bb, voffA[ii], sa + A_BYTES + ii * 4096);
+      if (HAS_W && wave == 0) async_copy4_sv(w_base + step * stage_rows, voffW, smem_a + slot * STAGE + A_BYTES + B_BYTES);
+      return;
+    }
+    char* st = smem + slot * STAGE;
     async_load_tile<CA, TN_KT>(st, [&](int row) { return a_base + row_index(r0 + row) * (DK * 2); });
     async_load_tile<CB, TN_KT>(st + A_BYTES, [&](int row) { return b_base + row_index(r0 + row) * (DV * 2); });
-    if (HAS_W && tid < 64) async_copy4(w_base + row_index(r0 + tid), st + A_BYTES + B_BYTES);
+    if (HAS_W && wave == 0) async_copy4(w_base + row_index(r0 + l), st + A_BYTES + B_BYTES);
   };
 
   f32x4 acc[XPW][NT];
@@ -74,42 +105,138 @@ __device__ __forceinline__ void tn_body(const T* __restrict__ A, const T* __rest
     for (int j = 0; j < NT; j++) acc[i][j] = (f32x4){0, 0, 0, 0};
   f32x4 sacc = {0, 0, 0, 0};
 
+  // Operand fragments of one contraction step (32 rows).  With PREFETCH they are fetched one step ahead of the
+  // matrix-core work that uses them, and a stage's slot is free for the next copy as soon as every wave holds the
+  // stage's last fragments in registers.  Every vector instruction in this loop competes with the matrix cores
+  // for the SIMD, so the LDS addresses are per-lane registers set up once plus immediates (the stage loop is
+  // unrolled over the three slots of the ring).
+  struct Frags {
+    v8 kfy, kfx, vf[NT];
+  };
+  constexpr bool PREFETCH = DV <= 64;   // two sets of fragments and their addresses do not fit beyond that
+  uint32_t ay[2], ax[2], av[NT][2], aw = smem_a + A_BYTES + B_BYTES + 32 * g;
+  if constexpr (PREFETCH) {
+    const int sl = l & 15;
+#pragma unroll
+    for (int hf = 0; hf < 2; hf++) {
+      const int row = 8 * g + 4 * hf + (sl >> 2);
+      const int cy = 16 * y + 4 * (sl & 3), cx = 16 * xb + 4 * (sl & 3);
+      ay[hf] = smem_a + row * (CA * 16) + (((cy / 8) ^ swz<CA>(row)) * 16) + (cy % 8) * 2;
+      ax[hf] = smem_a + row * (CA * 16) + (((cx / 8) ^ swz<CA>(row)) * 16) + (cx % 8) * 2;
+      asm volatile("" : "+v"(ay[hf]));
+      asm volatile("" : "+v"(ax[hf]));
+#pragma unroll
+      for (int nt = 0; nt < NT; nt++) {
+        const int cv = 16 * nt + 4 * (sl & 3);
+        av[nt][hf] = smem_a + A_BYTES + row * (CB * 16) + (((cv / 8) ^ swz<CB>(row)) * 16) + (cv % 8) * 2;
+        asm volatile("" : "+v"(av[nt][hf]));
+      }
+    }
+    asm volatile("" : "+v"(aw));
+  }
+  auto tr8 = [&](uint32_t lo, uint32_t hi) -> v8 {
+    const s16x4 a = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)lo);
+    const s16x4 b = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)hi);
+    return __builtin_bit_cast(v8, __builtin_shufflevector(a, b, 0, 1, 2, 3, 4, 5, 6, 7));
+  };
+  auto load_frags = [&](Frags& F, auto slot_c, auto ks_c) {
+    constexpr int OFF = decltype(slot_c)::value * STAGE + decltype(ks_c)::value * 32 * (CA * 16);
+    F.kfy = tr8(ay[0] + OFF, ay[1] + OFF);
+    F.kfx = tr8(ax[0] + OFF, ax[1] + OFF);
+#pragma unroll
+    for (int nt = 0; nt < NT; nt++) F.vf[nt] = tr8(av[nt][0] + OFF, av[nt][1] + OFF);
+  };
+  auto compute = [&](const Frags& F, f32x4 w0, f32x4 w1) {
+    float rowf[8], srcf[8];
+    unpack8(F.kfy, rowf);
+    unpack8(F.kfx, srcf);
+    if (HAS_W) {
+      float sc[8];
+#pragma unroll
+      for (int q = 0; q < 4; q++) {
+        sc[q] = srcf[q] * w0[q];
+        sc[4 + q] = srcf[4 + q] * w1[q];
+      }
+      sacc = mfma16(F.kfy, pack8<T>(sc), sacc);
+    } else {
+      sacc = mfma16(F.kfy, F.kfx, sacc);
+    }
+    dpp_fence();  // srcf is read through DPP below
+    static_for<XPW>([&](auto xi) {
+      v8 a = PhiTile<T, PART * XPW + xi.value>::make(F.kfy, F.kfx, rowf, srcf);
+#pragma unroll
+      for (int nt = 0; nt < NT; nt++) acc[xi.value][nt] = mfma16(a, F.vf[nt], acc[xi.value][nt]);
+    });
+  };
+  // w of a step is fetched at the end of the previous step's work, when few registers are live
+  f32x4 wv0 = {0, 0, 0, 0}, wv1 = {0, 0, 0, 0};
+  auto load_w = [&](auto slot_c, auto ks_c) {
+    if (HAS_W) {
+      constexpr int WOFF = decltype(slot_c)::value * STAGE + decltype(ks_c)::value * 128;
+      wv0 = *(const lds_f32x4*)(aw + WOFF);
+      wv1 = *(const lds_f32x4*)(aw + WOFF + 16);
+    }
+  };
+
   const int steps = (rows + TN_KT - 1) / TN_KT;
-  issue(0);
-  if (steps > 1) issue(1);
-  for (int step = 0; step < steps; step++) {
-    char* st = smem + (step % TN_NST) * STAGE;
-    if (step + 1 < steps) wait_vmcnt<LOADS>(); else wait_vmcnt<0>();
-    if ((step + 1) * TN_KT > rows) zero_tile_rows<CA, TN_KT>(st, rows - step * TN_KT);
+  if constexpr (PREFETCH) {
+    issue(0);
+    if (steps > 1) issue(1);
+    if (steps > 2) issue(2);
+    if (steps > 2) wait_vmcnt<2 * LOADS>(); else if (steps > 1) wait_vmcnt<LOADS>(); else wait_vmcnt<0>();
+    if (TN_KT > rows) zero_tile_rows<CA, TN_KT>(smem, rows);
     lds_barrier();
-    if (step + 2 < steps) issue(step + 2);
-    if (active) {
-      const float* wt = (const float*)(st + A_BYTES + B_BYTES);
+    Frags F0, F1;
+    load_frags(F0, IC<0>{}, IC<0>{});
+    load_w(IC<0>{}, IC<0>{});
+    // one stage held in slot SL; returns false after the last stage
+    auto stage = [&](int step, auto sl_c) -> bool {
+      constexpr int SL = decltype(sl_c)::value, NX = (SL + 1) % TN_NST;
+      load_frags(F1, IC<SL>{}, IC<1>{});
+      if (active) compute(F0, wv0, wv1);
+      __builtin_amdgcn_sched_barrier(0);
+      load_w(IC<SL>{}, IC<1>{});
+      const bool more = step + 1 < steps;
+      if (more) {
+        if (step + 2 < steps) wait_vmcnt<LOADS>(); else wait_vmcnt<0>();
+        if ((step + 2) * TN_KT > rows) zero_tile_rows<CA, TN_KT>(smem + NX * STAGE, rows - (step + 1) * TN_KT);
+        lds_barrier();   // every wave holds the last fragments of this stage: its slot can be refilled
+        if (step + 3 < steps) issue(step + 3);
+        load_frags(F0, IC<NX>{}, IC<0>{});
+      }
+      if (active) compute(F1, wv0, wv1);
+      __builtin_amdgcn_sched_barrier(0);
+      if (more) load_w(IC<NX>{}, IC<0>{});
+      return more;
+    };
+    for (int step = 0;; step += 3) {
+      if (!stage(step, IC<0>{})) break;
+      if (!stage(step + 1, IC<1>{})) break;
+      if (!stage(step + 2, IC<2>{})) break;
+    }
+  } else {
+    issue(0);
+    if (steps > 1) issue(1);
+    Frags F;
+    for (int step = 0; step < steps; step++) {
+      const char* st = smem + (step % TN_NST) * STAGE;
+      if (step + 1 < steps) wait_vmcnt<LOADS>(); else wait_vmcnt<0>();
+      if ((step + 1) * TN_KT > rows) zero_tile_rows<CA, TN_KT>(smem + (step % TN_NST) * STAGE, rows - step * TN_KT);
+      lds_barrier();
+      if (step + 2 < steps) issue(step + 2);
 #pragma unroll 1
       for (int ks = 0; ks < TN_KT / 32; ks++) {
-        v8 kfy = sw_frag_tr<T, CA>(st, 32 * ks, 16 * y);
-        v8 kfx = (xb == y) ? kfy : sw_frag_tr<T, CA>(st, 32 * ks, 16 * xb);
-        v8 vf[NT];
+        F.kfy = sw_frag_tr<T, CA>(st, 32 * ks, 16 * y);
+        F.kfx = (xb == y) ? F.kfy : sw_frag_tr<T, CA>(st, 32 * ks, 16 * xb);
 #pragma unroll
-        for (int nt = 0; nt < NT; nt++) vf[nt] = sw_frag_tr<T, CB>(st + A_BYTES, 32 * ks, 16 * nt);
-        float rowf[8], srcf[8];
-        unpack8(kfy, rowf);
-        unpack8(kfx, srcf);
+        for (int nt = 0; nt < NT; nt++) F.vf[nt] = sw_frag_tr<T, CB>(st + A_BYTES, 32 * ks, 16 * nt);
+        f32x4 w0 = {0, 0, 0, 0}, w1 = {0, 0, 0, 0};
         if (HAS_W) {
-          float sc[8];
-          const float* wp = wt + 32 * ks + 8 * g;
-#pragma unroll
-          for (int q = 0; q < 8; q++) sc[q] = srcf[q] * wp[q];
-          sacc = mfma16(kfy, pack8<T>(sc), sacc);
-        } else {
-          sacc = mfma16(kfy, kfx, sacc);
+          const float* wp = (const float*)(st + A_BYTES + B_BYTES) + 32 * ks + 8 * g;
+          w0 = *(const f32x4*)wp;
+          w1 = *(const f32x4*)(wp + 4);
         }
-        dpp_fence();  // srcf is read through DPP below
-        static_for<XPW>([&](auto xi) {
-          v8 a = PhiTile<T, PART * XPW + xi.value>::make(kfy, kfx, rowf, srcf);
-#pragma unroll
-          for (int nt = 0; nt < NT; nt++) acc[xi.value][nt] = mfma16(a, vf[nt], acc[xi.value][nt]);
-        });
+        if (active) compute(F, w0, w1);
       }
     }
   }
@@ -142,7 +269,7 @@ __global__ __launch_bounds__(256, 2) void sympow_tn_kernel(const T* __restrict__
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   constexpr int PARTS = 16 / XPW;
   constexpr int NB = (DK / 16) * (DK / 16 + 1) / 2;
-  const int task = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int task = blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const bool active = task < NB * PARTS;
   const int t2 = active ? task : 0;
   const int part = t2 % PARTS;
