@@ -2,12 +2,19 @@
 
 Same arithmetic as composing the four operators through ``make_power_retention``
 (ref: retention/power_retention_maker.py:142-197), but the glue between the operators (chunk-local
-cumsum of the gates, key discounting, query gating, and their gradients) runs in two fused HIP kernels
+cumsum of the gates, key discounting, query gating, and their gradients) runs inside fused HIP kernels
 instead of a dozen elementwise launches, and only the first n entries of the scans are produced.
+
+Forward and backward are ``torch.library.custom_op``s (``pr::chunked_fwd`` / ``pr::chunked_bwd``) with fake
+implementations, like the per-kernel operators (the convention of the reference's CUDA wrappers,
+ref: retention/_attention/cuda.py:10-43,129-245), so the node survives ``torch.compile`` without a graph break.
 """
 from __future__ import annotations
 
+from typing import Optional, Tuple
+
 import torch
+from torch import Tensor
 
 from . import _lib
 from .ops import expanded_dim
@@ -17,104 +24,148 @@ def _empty(shape, dtype, device):
     return torch.empty(shape, dtype=dtype, device=device)
 
 
-class _ChunkedPowerRetention(torch.autograd.Function):
-    @staticmethod
-    def forward(ctx, Q, K, V, log_G, deg, scale, c):
-        lib = _lib.load()
-        st = _lib.stream()
-        b, t, hq, d = Q.shape
-        h = K.shape[2]
-        r = hq // h
-        n = t // c
-        BN = b * n
-        D = expanded_dim(d)
-        dev, dt = Q.device, Q.dtype
-        code = _lib.dtype_code(dt)
-        f32 = torch.float32
-        gated = log_G is not None
-        p = _lib.ptr
+@torch.library.custom_op("pr::chunked_fwd", mutates_args=(), device_types="cuda")
+def chunked_fwd(Q: Tensor, K: Tensor, V: Tensor, log_G: Optional[Tensor], deg: int, scale: float,
+                c: int) -> Tuple[Tensor, Tensor, Tensor, Tensor, Tensor, Tensor, Tensor, Tensor, Tensor]:
+    """-> O, and what the backward needs: A, lcs, Kd, Qg (empty when ungated), Sc, sc, rowmax, den."""
+    lib = _lib.load()
+    st = _lib.stream()
+    b, t, hq, d = Q.shape
+    h = K.shape[2]
+    r = hq // h
+    n = t // c
+    BN = b * n
+    D = expanded_dim(d)
+    dev, dt = Q.device, Q.dtype
+    code = _lib.dtype_code(dt)
+    f32 = torch.float32
+    gated = log_G is not None
+    p = _lib.ptr
 
-        if gated:
-            A, lcs = _empty((BN, c, h), f32, dev), _empty((BN, h), f32, dev)
-            Kd, Qg = torch.empty_like(K), torch.empty_like(Q)
-            _lib.check(lib.pr_chunk_prep_fwd(p(log_G), p(K), p(Q), p(A), p(lcs), p(Kd), p(Qg), BN, c, h, r, d, deg, code,
-                                             st), "chunk_prep_fwd")
-        else:
-            A, Kd, Qg = None, K, Q
-            lcs = torch.zeros((BN, h), dtype=f32, device=dev)
+    if gated:
+        A, lcs = _empty((BN, c, h), f32, dev), _empty((BN, h), f32, dev)
+        Kd, Qg = torch.empty_like(K), torch.empty_like(Q)
+        _lib.check(lib.pr_chunk_prep_fwd(p(log_G), p(K), p(Q), p(A), p(lcs), p(Kd), p(Qg), BN, c, h, r, d, deg, code,
+                                         st), "chunk_prep_fwd")
+        Kd_, Qg_ = Kd, Qg
+    else:
+        A, Kd, Qg = _empty((0,), f32, dev), _empty((0,), dt, dev), _empty((0,), dt, dev)
+        Kd_, Qg_ = K, Q
+        lcs = torch.zeros((BN, h), dtype=f32, device=dev)
 
-        S, s = _empty((BN, h, D, d), dt, dev), _empty((BN, h, D), f32, dev)
-        _lib.check(lib.pr_update_state_fwd(p(Kd), p(V), p(S), p(s), BN, c, h, d, 2, code, st), "update_state_fwd")
-        Sc, sc = torch.empty_like(S), torch.empty_like(s)
-        _lib.check(lib.pr_discumsum_fwd(p(S), p(lcs), p(Sc), b, n, n, h, D * d, code, st), "discumsum_fwd")
-        _lib.check(lib.pr_discumsum_fwd(p(s), p(lcs), p(sc), b, n, n, h, D, _lib.PR_F32, st), "discumsum_fwd")
-        del S, s
+    S, s = _empty((BN, h, D, d), dt, dev), _empty((BN, h, D), f32, dev)
+    _lib.check(lib.pr_update_state_fwd(p(Kd_), p(V), p(S), p(s), BN, c, h, d, 2, code, st), "update_state_fwd")
+    Sc, sc = torch.empty_like(S), torch.empty_like(s)
+    _lib.check(lib.pr_discumsum_fwd(p(S), p(lcs), p(Sc), b, n, n, h, D * d, code, st), "discumsum_fwd")
+    _lib.check(lib.pr_discumsum_fwd(p(s), p(lcs), p(sc), b, n, n, h, D, _lib.PR_F32, st), "discumsum_fwd")
+    del S, s
 
-        Ya = torch.empty_like(Q)
-        la, rm = _empty((BN, c, hq), f32, dev), _empty((BN, c, hq), f32, dev)
-        _lib.check(lib.pr_attention_fwd(p(Q), p(K), p(V), p(A), p(Ya), p(la), p(rm), BN, c, c, h, r, d, scale, deg, 0,
-                                        code, st), "attention_fwd")
-        O, den = torch.empty_like(Q), _empty((BN, c, hq), f32, dev)
-        _lib.check(lib.pr_query_state_fwd(p(Qg), p(Sc), p(sc), p(Ya), p(la), p(rm), p(O), p(den), BN, n, c, h, r, d,
-                                          scale ** deg, 2, 1, code, st), "query_state_fwd")
-        ctx.save_for_backward(Q, K, V, A, lcs, Kd if gated else None, Qg if gated else None, Sc, sc, rm, O, den)
-        ctx.meta = (deg, scale, c, gated)
-        return O
+    Ya = torch.empty_like(Q)
+    la, rm = _empty((BN, c, hq), f32, dev), _empty((BN, c, hq), f32, dev)
+    _lib.check(lib.pr_attention_fwd(p(Q), p(K), p(V), p(A) if gated else None, p(Ya), p(la), p(rm), BN, c, c, h, r, d,
+                                    scale, deg, 0, code, st), "attention_fwd")
+    O, den = torch.empty_like(Q), _empty((BN, c, hq), f32, dev)
+    _lib.check(lib.pr_query_state_fwd(p(Qg_), p(Sc), p(sc), p(Ya), p(la), p(rm), p(O), p(den), BN, n, c, h, r, d,
+                                      scale ** deg, 2, 1, code, st), "query_state_fwd")
+    return O, A, lcs, Kd, Qg, Sc, sc, rm, den
 
-    @staticmethod
-    def backward(ctx, dO):
-        Q, K, V, A, lcs, Kd, Qg, Sc, sc, rm, O, den = ctx.saved_tensors
-        deg, scale, c, gated = ctx.meta
-        if not gated:
-            Kd, Qg = K, Q
-        lib = _lib.load()
-        st = _lib.stream()
-        b, t, hq, d = Q.shape
-        h = K.shape[2]
-        r = hq // h
-        n = t // c
-        BN = b * n
-        D = expanded_dim(d)
-        dev, dt = Q.device, Q.dtype
-        code = _lib.dtype_code(dt)
-        f32, u8 = torch.float32, torch.uint8
-        p = _lib.ptr
-        dO = dO.contiguous()
 
-        dQg, dSc, dsc = torch.empty_like(Q), torch.empty_like(Sc), torch.empty_like(sc)
-        dYa, dla = torch.empty_like(Q), torch.empty_like(den)
-        ws = _empty((lib.pr_query_state_bwd_workspace(BN, c, h, r, d, code),), u8, dev)
-        _lib.check(lib.pr_query_state_bwd(p(Qg), p(Sc), p(sc), p(rm), p(O), p(den), p(dO), p(dQg), p(dSc), p(dsc),
-                                          p(dYa), p(dla), p(ws), BN, n, c, h, r, d, scale ** deg, 2, 1, code, st),
-                   "query_state_bwd")
-        dS, ds = torch.empty_like(Sc), torch.empty_like(sc)
-        dl1, dl2 = torch.empty_like(lcs), torch.empty_like(lcs)
-        ws = _empty((max(lib.pr_discumsum_bwd_workspace(b, n, h, D * d, code),
-                         lib.pr_discumsum_bwd_workspace(b, n, h, D, _lib.PR_F32)),), u8, dev)
-        _lib.check(lib.pr_discumsum_bwd(p(dSc), p(Sc), p(lcs), p(dS), p(dl1), p(ws), b, n, n, h, D * d, code, st),
-                   "discumsum_bwd")
-        _lib.check(lib.pr_discumsum_bwd(p(dsc), p(sc), p(lcs), p(ds), p(dl2), p(ws), b, n, n, h, D, _lib.PR_F32, st),
-                   "discumsum_bwd")
-        dKd, dVs = torch.empty_like(K), torch.empty_like(V)
-        _lib.check(lib.pr_update_state_bwd(p(Kd), p(V), p(dS), p(ds), p(dKd), p(dVs), BN, c, h, d, 2, code, st),
-                   "update_state_bwd")
+@chunked_fwd.register_fake
+def _(Q, K, V, log_G, deg, scale, c):
+    b, t, hq, d = Q.shape
+    h = K.shape[2]
+    BN, D = b * (t // c), expanded_dim(d)
+    f32 = torch.float32
+    gated = log_G is not None
+    A = Q.new_empty((BN, c, h) if gated else (0,), dtype=f32)
+    return (torch.empty_like(Q), A, Q.new_empty((BN, h), dtype=f32),
+            torch.empty_like(K) if gated else K.new_empty((0,)), torch.empty_like(Q) if gated else Q.new_empty((0,)),
+            Q.new_empty((BN, h, D, d)), Q.new_empty((BN, h, D), dtype=f32), Q.new_empty((BN, c, hq), dtype=f32),
+            Q.new_empty((BN, c, hq), dtype=f32))
 
-        # the attention backward adds the state-path gradients in its epilogue and writes the final dQ, dK, dV
-        dQa, dKa, dVa = torch.empty_like(Q), torch.empty_like(K), torch.empty_like(V)
-        dGq = _empty((BN, c, hq), f32, dev) if gated else None
-        dGk = _empty((b, t, h), f32, dev) if gated else None
-        dotk = _empty((BN, c, h), f32, dev) if gated else None
-        _lib.check(lib.pr_chunk_attention_bwd(p(Q), p(K), p(V), p(A), p(rm), p(dYa), p(dla), None, p(dQg), p(dKd),
-                                              p(dVs), p(dQa), p(dKa), p(dVa), p(dGq), p(dGk), p(dotk), BN, c, h, r, d,
-                                              scale, deg, code, st), "chunk_attention_bwd")
-        dlg = None
-        if gated:
-            dlg = dGk.add_(dGq.view(b, t, h, r).sum(-1)) if r > 1 else dGk.add_(dGq.view(b, t, h))
-            _lib.check(lib.pr_chunk_gate_scan_bwd(p(dlg), p(dotk), p(dl1), p(dl2), BN, c, h, deg, st),
-                       "chunk_gate_scan_bwd")
-        return dQa, dKa, dVa, dlg, None, None, None
+
+@torch.library.custom_op("pr::chunked_bwd", mutates_args=(), device_types="cuda")
+def chunked_bwd(Q: Tensor, K: Tensor, V: Tensor, A: Tensor, lcs: Tensor, Kd: Tensor, Qg: Tensor, Sc: Tensor,
+                sc: Tensor, rm: Tensor, O: Tensor, den: Tensor, dO: Tensor, deg: int, scale: float, c: int,
+                gated: bool) -> Tuple[Tensor, Tensor, Tensor, Tensor]:
+    """-> dQ, dK, dV, dlog_G (empty when ungated)."""
+    if not gated:
+        Kd, Qg = K, Q
+    lib = _lib.load()
+    st = _lib.stream()
+    b, t, hq, d = Q.shape
+    h = K.shape[2]
+    r = hq // h
+    n = t // c
+    BN = b * n
+    D = expanded_dim(d)
+    dev, dt = Q.device, Q.dtype
+    code = _lib.dtype_code(dt)
+    f32, u8 = torch.float32, torch.uint8
+    p = _lib.ptr
+    dO = dO.contiguous()
+    dQg, dSc, dsc = torch.empty_like(Q), torch.empty_like(Sc), torch.empty_like(sc)
+    dYa, dla = torch.empty_like(Q), torch.empty_like(den)
+    ws = _empty((lib.pr_query_state_bwd_workspace(BN, c, h, r, d, code),), u8, dev)
+    _lib.check(lib.pr_query_state_bwd(p(Qg), p(Sc), p(sc), p(rm), p(O), p(den), p(dO), p(dQg), p(dSc), p(dsc),
+                                      p(dYa), p(dla), p(ws), BN, n, c, h, r, d, scale ** deg, 2, 1, code, st),
+               "query_state_bwd")
+    dS, ds = torch.empty_like(Sc), torch.empty_like(sc)
+    dl1, dl2 = torch.empty_like(lcs), torch.empty_like(lcs)
+    ws = _empty((max(lib.pr_discumsum_bwd_workspace(b, n, h, D * d, code),
+                     lib.pr_discumsum_bwd_workspace(b, n, h, D, _lib.PR_F32)),), u8, dev)
+    _lib.check(lib.pr_discumsum_bwd(p(dSc), p(Sc), p(lcs), p(dS), p(dl1), p(ws), b, n, n, h, D * d, code, st),
+               "discumsum_bwd")
+    _lib.check(lib.pr_discumsum_bwd(p(dsc), p(sc), p(lcs), p(ds), p(dl2), p(ws), b, n, n, h, D, _lib.PR_F32, st),
+               "discumsum_bwd")
+    dKd, dVs = torch.empty_like(K), torch.empty_like(V)
+    _lib.check(lib.pr_update_state_bwd(p(Kd), p(V), p(dS), p(ds), p(dKd), p(dVs), BN, c, h, d, 2, code, st),
+               "update_state_bwd")
+
+    # the attention backward adds the state-path gradients in its epilogue and writes the final dQ, dK, dV
+    dQa, dKa, dVa = torch.empty_like(Q), torch.empty_like(K), torch.empty_like(V)
+    dGq = _empty((BN, c, hq), f32, dev) if gated else None
+    dGk = _empty((b, t, h), f32, dev) if gated else None
+    dotk = _empty((BN, c, h), f32, dev) if gated else None
+    _lib.check(lib.pr_chunk_attention_bwd(p(Q), p(K), p(V), p(A) if gated else None, p(rm), p(dYa), p(dla), None, p(dQg), p(dKd),
+                                          p(dVs), p(dQa), p(dKa), p(dVa), p(dGq), p(dGk), p(dotk), BN, c, h, r, d,
+                                          scale, deg, code, st), "chunk_attention_bwd")
+    dlg = _empty((0,), f32, dev)
+    if gated:
+        dlg = dGk.add_(dGq.view(b, t, h, r).sum(-1)) if r > 1 else dGk.add_(dGq.view(b, t, h))
+        _lib.check(lib.pr_chunk_gate_scan_bwd(p(dlg), p(dotk), p(dl1), p(dl2), BN, c, h, deg, st),
+                   "chunk_gate_scan_bwd")
+    return dQa, dKa, dVa, dlg
+
+
+@chunked_bwd.register_fake
+def _(Q, K, V, A, lcs, Kd, Qg, Sc, sc, rm, O, den, dO, deg, scale, c, gated):
+    b, t, _, _ = Q.shape
+    h = K.shape[2]
+    return (torch.empty_like(Q), torch.empty_like(K), torch.empty_like(V),
+            Q.new_empty((b, t, h) if gated else (0,), dtype=torch.float32))
+
+
+def _chunked_setup(ctx, inputs, output):
+    Q, K, V, log_G, deg, scale, c = inputs
+    O, A, lcs, Kd, Qg, Sc, sc, rm, den = output
+    ctx.save_for_backward(Q, K, V, A, lcs, Kd, Qg, Sc, sc, rm, O, den)
+    ctx.meta = (deg, scale, c, log_G is not None)
+    ctx.set_materialize_grads(False)
+
+
+def _chunked_backward(ctx, dO, *unused):
+    Q, K, V, A, lcs, Kd, Qg, Sc, sc, rm, O, den = ctx.saved_tensors
+    deg, scale, c, gated = ctx.meta
+    if dO is None:
+        return None, None, None, None, None, None, None
+    dQ, dK, dV, dlg = chunked_bwd(Q, K, V, A, lcs, Kd, Qg, Sc, sc, rm, O, den, dO, deg, scale, c, gated)
+    return dQ, dK, dV, (dlg if gated else None), None, None, None
+
+
+torch.library.register_autograd("pr::chunked_fwd", _chunked_backward, setup_context=_chunked_setup)
 
 
 def chunked_power_retention(Q, K, V, log_G, deg, scale, chunk_size):
     """Q [b,t,hq,d], K, V [b,t,h,d] contiguous, t a multiple of chunk_size, log_G [b,t,h] fp32 or None."""
-    return _ChunkedPowerRetention.apply(Q, K, V, log_G, int(deg), float(scale), int(chunk_size))
+    return chunked_fwd(Q, K, V, log_G, int(deg), float(scale), int(chunk_size))[0]
