@@ -113,7 +113,7 @@ __global__ __launch_bounds__(256, DK <= 64 ? 3 : 2) void sympow_nn_kernel(NNArgs
   for (int i = 0; i < MT; i++)
 #pragma unroll
     for (int j = 0; j < NT; j++) acc[i][j] = (f32x4){0, 0, 0, 0};
-  float aux[MT];   // aux of the row this lane holds as an accumulator COLUMN (row0 + wave*16*MT + 16*mi + tcol)
+  float aux[MT];   // partial aux of the lane's row (row0 + wave*16*MT + 16*mi + tcol), summed over the lane groups at the end
 #pragma unroll
   for (int mi = 0; mi < MT; mi++) aux[mi] = 0.f;
 
@@ -195,7 +195,7 @@ __global__ __launch_bounds__(256, DK <= 64 ? 3 : 2) void sympow_nn_kernel(NNArgs
           const T xs = __builtin_bit_cast(T, xbits);
           const v8 af = prow[mi].make(xs);
 #pragma unroll
-          for (int nt = 0; nt < NT; nt++) acc[mi][nt] = mfma16(af, vf[nt], acc[mi][nt]);
+          for (int nt = 0; nt < NT; nt++) acc[mi][nt] = mfma16(vf[nt], af, acc[mi][nt]);   // out^T[e, row]
         }
       }
       if (cur.next()) {
@@ -210,15 +210,31 @@ __global__ __launch_bounds__(256, DK <= 64 ? 3 : 2) void sympow_nn_kernel(NNArgs
     if (EPI == NN_EPI_MERGE) {
       // aux[row] = sum_{a,b} x[a] M[a,b] x[b]: U^T[b, row] = sum_a M[a,b] x[row,a] on the matrix cores (M in a high
       // and a low 16-bit part), then a dot with x[row, b] down the accumulator rows.
-      T* Mt = (T*)ring;   // [DK (b)][LDM (a)]
+      T* Mt = (T*)ring;   // [DK (a)][LDM (b)]: sB of the stored pair (a, b), read transposed as the A operand
       for (int part = 0; part < 2; part++) {
         lds_barrier();
-        for (int idx = tid; idx < DK * DK; idx += 256) {
-          const int b_ = idx / DK, aa = idx % DK, yb = b_ / 16;
-          float val = 0.f;
-          if (aa < 16 * (yb + 1)) val = sBg[128 * yb * (yb + 1) + 16 * aa + (b_ - 16 * yb)] * ScaleS<T>::down;
-          const T hi16 = (T)val;
-          Mt[b_ * LDM + aa] = part == 0 ? hi16 : (T)(val - (float)hi16);
+        // one thread per (a, strip of 16 b): 16 consecutive floats of sB, 16 consecutive elements of M
+        for (int idx = tid; idx < DK * TT; idx += 256) {
+          const int aa = idx % DK, yb = idx / DK;
+          float v16[16];
+          if (aa < 16 * (yb + 1)) {
+            const f32x4* src = (const f32x4*)(sBg + 128 * yb * (yb + 1) + 16 * aa);
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+              const f32x4 t4 = src[q];
+#pragma unroll
+              for (int v = 0; v < 4; v++) v16[4 * q + v] = t4[v] * ScaleS<T>::down;
+            }
+          } else {
+#pragma unroll
+            for (int q = 0; q < 16; q++) v16[q] = 0.f;
+          }
+          if (part == 1) {
+#pragma unroll
+            for (int q = 0; q < 16; q++) v16[q] -= (float)(T)v16[q];
+          }
+          *(v8*)(Mt + aa * LDM + 16 * yb) = pack8<T>(v16);
+          *(v8*)(Mt + aa * LDM + 16 * yb + 8) = pack8<T>(v16 + 8);
         }
         lds_barrier();
 #pragma unroll
@@ -231,7 +247,7 @@ __global__ __launch_bounds__(256, DK <= 64 ? 3 : 2) void sympow_nn_kernel(NNArgs
           for (int wt = 0; wt < TT; wt++) {
             f32x4 t = {0, 0, 0, 0};
 #pragma unroll
-            for (int ks = 0; ks < KX; ks++) t = mfma16(lds_frag<T>(Mt, LDM, 16 * wt, 32 * ks), xf[ks], t);
+            for (int ks = 0; ks < KX; ks++) t = mfma16(lds_frag_tr<T>(Mt, LDM, 32 * ks, 16 * wt), xf[ks], t);
             const v4 xb4 = *(const v4*)x_ptr(lrow, 16 * wt + 4 * g);
 #pragma unroll
             for (int v = 0; v < 4; v++) aux[mi] += t[v] * (float)xb4[v];
@@ -241,63 +257,55 @@ __global__ __launch_bounds__(256, DK <= 64 ? 3 : 2) void sympow_nn_kernel(NNArgs
     }
   }
 
-  // epilogue: accumulator element v of lane l is row 4*(l/16)+v, column 16*nt + l%16
+  // epilogue: the accumulators hold out^T, element v of lane l is column 16*nt + 4*(l/16) + v of the lane's row
+  // (row0 + wave*16*MT + 16*mi + l%16): one row per lane, 8-byte loads and stores
   T* out = (T*)a.out + (long)bn * a.c * hA * DV;
-  if (EPI == NN_EPI_MERGE) {
-    // hand aux from the lane that holds the row as a column to the lanes that hold it as accumulator rows
-    float* ax = (float*)ring;
-    lds_barrier();
+  const float log_gamma = 0.5f * __logf((float)D);
 #pragma unroll
-    for (int mi = 0; mi < MT; mi++) {
-      const float tot = sum_over_rows(aux[mi]) * ScaleS<T>::up;
-      if (g == 0) ax[wave * 16 * MT + 16 * mi + tcol] = tot;
-    }
-    lds_barrier();
-    constexpr float log_gamma_2 = 0.f;
-    (void)log_gamma_2;
-    const float log_gamma = 0.5f * __logf((float)D);
+  for (int mi = 0; mi < MT; mi++) {
+    const int row = row0 + wave * 16 * MT + 16 * mi + tcol;
+    const bool live = row < rows;
+    const long ro = row_off(row);   // clamped
+    if (EPI == NN_EPI_MERGE) {
+      const float lqs = sum_over_rows(aux[mi]) * ScaleS<T>::up;
+      float wa = 0.f, wq = 1.f, la = 0.f;
+      v4 ya4[NT];
+      if (a.Y_attn) {
+        const long go = (long)bn * a.c * hA + ro;
+        const float m = a.rowmax[go];
+        la = a.l_attn[go];
+        const T* ya = (const T*)a.Y_attn + (long)bn * a.c * hA * DV + ro * DV;
 #pragma unroll
-    for (int mi = 0; mi < MT; mi++) {
+        for (int nt = 0; nt < NT; nt++) ya4[nt] = *(const v4*)(ya + 16 * nt + 4 * g);
+        const float beta = fmaxf(m, log_gamma);
+        wa = __expf(m - beta);
+        wq = a.scale_p * __expf(-beta);
+      }
+      const float den = la * wa + lqs * wq;
+      const float inv = 1.f / den;
+      if (!live) continue;
 #pragma unroll
-      for (int v = 0; v < 4; v++) {
-        const int lrow = wave * 16 * MT + 16 * mi + 4 * g + v, row = row0 + lrow;
-        if (row >= rows) continue;
-        const long ro = row_off(row);
-        const float lqs = ax[lrow];
-        float wa = 0.f, wq = 1.f, la = 0.f;
-        const T* ya = nullptr;
-        if (a.Y_attn) {
-          const long go = (long)bn * a.c * hA + ro;
-          const float m = a.rowmax[go];
-          la = a.l_attn[go];
-          const float beta = fmaxf(m, log_gamma);
-          wa = __expf(m - beta);
-          wq = a.scale_p * __expf(-beta);
-          ya = (const T*)a.Y_attn + (long)bn * a.c * hA * DV + ro * DV;
-        }
-        const float den = la * wa + lqs * wq;
-        const float inv = 1.f / den;
+      for (int nt = 0; nt < NT; nt++) {
+        float o4[4];
 #pragma unroll
-        for (int nt = 0; nt < NT; nt++) {
-          const int e = 16 * nt + tcol;
+        for (int v = 0; v < 4; v++) {
           float num = acc[mi][nt][v] * wq;
-          if (ya) num += (float)ya[e] * wa;
-          out[ro * DV + e] = (T)(num * inv);
+          if (a.Y_attn) num += (float)ya4[nt][v] * wa;
+          o4[v] = num * inv;
         }
-        if (tcol == 0) a.den[(long)bn * a.c * hA + ro] = den;
+        *(v4*)(out + ro * DV + 16 * nt + 4 * g) = pack4<T>(o4);
+      }
+      if (g == 0) a.den[(long)bn * a.c * hA + ro] = den;
+    } else {
+      if (!live) continue;
+#pragma unroll
+      for (int nt = 0; nt < NT; nt++) {
+        float o4[4];
+#pragma unroll
+        for (int v = 0; v < 4; v++) o4[v] = acc[mi][nt][v];
+        *(v4*)(out + ro * DV + 16 * nt + 4 * g) = pack4<T>(o4);
       }
     }
-  } else {
-#pragma unroll
-    for (int mi = 0; mi < MT; mi++)
-#pragma unroll
-      for (int v = 0; v < 4; v++) {
-        const int row = row0 + wave * 16 * MT + 16 * mi + 4 * g + v;
-        if (row >= rows) continue;
-        const long ro = row_off(row);
-#pragma unroll
-        for (int nt = 0; nt < NT; nt++) out[ro * DV + 16 * nt + tcol] = (T)acc[mi][nt][v];
-      }
   }
 }
 
