@@ -222,23 +222,35 @@ __global__ __launch_bounds__(256, 2) void sympow_grad_kernel(GradArgs a, int row
     });
   });
 
-  // sB term: dX_s^T[w, row] = cvec[row] * sum_a M[w, a] X[row, a], M in two 16-bit parts (high, low) built in the
-  // (now idle) ring memory.
-  T* Mt = (T*)ring;   // [DK][LDM]
+  // sB term: dX_s[row, w] = cvec[row] * sum_a (U[a, w] + U[w, a]) X[row, a] with U[a, w] = m_f sB[f] for the stored
+  // pair f = (a, w) and 0 elsewhere.  U is built in the (now idle) ring memory in two 16-bit parts (high, low), one
+  // thread per (a, strip of 16 w): 16 consecutive floats of sB, 16 consecutive elements of U; U and U^T are both
+  // read from the one tile (plain and transposing operand loads).
+  T* Mt = (T*)ring;   // [DK (a)][LDM (w)]
   for (int part = 0; part < 2; part++) {
     lds_barrier();
-    for (int idx = tid; idx < DK * DK; idx += 256) {
-      const int w = idx / DK, aa = idx % DK, yw = w / 16, ya = aa / 16;
-      float val;
-      if (ya == yw) {
-        val = sBg[128 * yw * (yw + 1) + 16 * aa + (w - 16 * yw)] + sBg[128 * yw * (yw + 1) + 16 * w + (aa - 16 * yw)];
+    for (int idx = tid; idx < DK * TT; idx += 256) {
+      const int aa = idx % DK, yb = idx / DK;
+      float v16[16];
+      if (aa < 16 * (yb + 1)) {
+        const float m = ((MULT && aa < 16 * yb) ? 2.f : 1.f) * OnePair<T>::down;
+        const f32x4* src = (const f32x4*)(sBg + 128 * yb * (yb + 1) + 16 * aa);
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+          const f32x4 t4 = src[q];
+#pragma unroll
+          for (int v = 0; v < 4; v++) v16[4 * q + v] = t4[v] * m;
+        }
       } else {
-        const int lo = ya < yw ? aa : w, hi = ya < yw ? w : aa, yh = hi / 16;
-        val = sBg[128 * yh * (yh + 1) + 16 * lo + (hi - 16 * yh)] * (MULT ? 2.f : 1.f);
+#pragma unroll
+        for (int q = 0; q < 16; q++) v16[q] = 0.f;
       }
-      val *= OnePair<T>::down;
-      const T hi16 = (T)val;
-      Mt[w * LDM + aa] = part == 0 ? hi16 : (T)(val - (float)hi16);
+      if (part == 1) {
+#pragma unroll
+        for (int q = 0; q < 16; q++) v16[q] -= (float)(T)v16[q];
+      }
+      *(v8*)(Mt + aa * LDM + 16 * yb) = pack8<T>(v16);
+      *(v8*)(Mt + aa * LDM + 16 * yb + 8) = pack8<T>(v16 + 8);
     }
     lds_barrier();
 #pragma unroll
@@ -250,7 +262,10 @@ __global__ __launch_bounds__(256, 2) void sympow_grad_kernel(GradArgs a, int row
       for (int wt = 0; wt < TT; wt++) {
         f32x4 t = {0, 0, 0, 0};
 #pragma unroll
-        for (int ks = 0; ks < KX; ks++) t = mfma16(lds_frag<T>(Mt, LDM, 16 * wt, 32 * ks), xf[ks], t);
+        for (int ks = 0; ks < KX; ks++) {
+          t = mfma16(lds_frag_tr<T>(Mt, LDM, 32 * ks, 16 * wt), xf[ks], t);   // sum_a U[a, w] x[a]
+          t = mfma16(lds_frag<T>(Mt, LDM, 16 * wt, 32 * ks), xf[ks], t);      // sum_a U[w, a] x[a]
+        }
         acc[mi][wt] += t * (cv[mi] * OnePair<T>::up);
       }
     }
