@@ -381,14 +381,15 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
   constexpr int LOADS = 2 * AB_BM * CPR / 256;
   extern __shared__ __attribute__((aligned(1024))) char smem[];
 
+  // (integer division runs on the vector unit: readfirstlane brings the uniform results back to scalar registers)
   const int grp = blockIdx.x % 32, u = blockIdx.x / 32, ppg = (npairs + 31) / 32;
-  const int pair = (u % ppg) * 32 + grp;
+  const int pair = __builtin_amdgcn_readfirstlane((u % ppg) * 32 + grp);
   if (pair >= npairs) return;
   const int tid = threadIdx.x, l = tid & 63, g = l >> 4, kcol = l & 15;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int b = pair / a.h, hh = pair % a.h;
+  const int b = __builtin_amdgcn_readfirstlane(pair / a.h), hh = pair - b * a.h;
   const int hq = a.h * a.r, rows = a.tq * a.r, shift = a.tk - a.tq;
-  const int key0 = (u / ppg) * KEYS;                 // early keys are seen by the most rows
+  const int key0 = __builtin_amdgcn_readfirstlane(u / ppg) * KEYS;   // early keys are seen by the most rows
   const char* Qg = (const char*)((const T*)a.Q + (long)b * a.tq * hq * DH);
   const char* dOg = (const char*)((const T*)a.dO + (long)b * a.tq * hq * DH);
   const T* Kg = (const T*)a.K + (long)b * a.tk * a.h * DH + hh * DH;
@@ -418,14 +419,13 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
   const int tile_w = max(tile_lo, max(0, (wkey0 - shift) * a.r) / AB_BM);
   const int n_seen = max(n_far, ntile_total - tile_w);
 
-  // copies of one stage
-  uint32_t grow[LOADS / 2], gchk[LOADS / 2];   // row inside the tile and byte offset of the 16-byte chunk in its row
-#pragma unroll
-  for (int ii = 0; ii < LOADS / 2; ii++) {
-    const int pos = (ii * 4 + wave) * 64 + l, row = pos / CPR;
-    grow[ii] = row;
-    gchk[ii] = 16 * ((pos % CPR) ^ swz<CPR>(row));
-  }
+  // copies of one stage: row inside the tile and byte offset of the 16-byte chunk in its row for this thread's
+  // copy number ii (recomputed where needed: only the irregular paths use them)
+  auto grow = [&](int ii) -> int { return ((ii * 4 + wave) * 64 + l) / CPR; };
+  auto gchk = [&](int ii) -> uint32_t {
+    const int pos = (ii * 4 + wave) * 64 + l;
+    return 16 * ((pos % CPR) ^ swz<CPR>(pos / CPR));
+  };
   auto row_elem = [&](int row) -> long {   // element offset of a (clamped) folded row in a [tq, hq] array
     row = min(row, rows - 1);
     const int t = row / a.r;
@@ -436,6 +436,15 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
   const T* dKsg = a.dKs ? (const T*)a.dKs + (long)b * a.tk * a.h * DH + hh * DH : nullptr;
   const T* dVsg = a.dVs ? (const T*)a.dVs + (long)b * a.tk * a.h * DH + hh * DH : nullptr;
   const int ntot = nsteps + (dKsg ? 2 : 0);
+  // lane offsets of the copies of a regular tile (r a power of two): folded row j of a tile is time step j / r, head
+  // hh * r + j % r, whatever the tile
+  const bool regular = (a.r & (a.r - 1)) == 0 && a.r <= AB_BM;
+  const int rsh = 31 - __builtin_clz(a.r);
+  const uint32_t smem_a = lds_addr(smem);
+  uint32_t voff[LOADS / 2];
+#pragma unroll
+  for (int ii = 0; ii < LOADS / 2; ii++)
+    voff[ii] = (uint32_t)((((grow(ii) >> rsh) * hq + hh * a.r + (grow(ii) & (a.r - 1))) * (DH * 2))) + gchk(ii);
   auto issue = [&](int step) {
     char* st = smem + (step % AB_NST) * STAGE;
     if (step >= nsteps) {
@@ -443,8 +452,8 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
 #pragma unroll
       for (int ii = 0; ii < LOADS; ii++) {
         const int half = ii / (LOADS / 2), i2 = ii % (LOADS / 2);
-        const long eo = (long)min(key0 + half * AB_BM + (int)grow[i2], a.tk - 1) * kstride;
-        async_copy16((const char*)(src + eo) + gchk[i2], st + half * TILE + (i2 * 4 + wave) * 1024);
+        const long eo = (long)min(key0 + half * AB_BM + grow(i2), a.tk - 1) * kstride;
+        async_copy16((const char*)(src + eo) + gchk(i2), st + half * TILE + (i2 * 4 + wave) * 1024);
       }
       if (wave == 0) {   // keeps the count of copies per stage fixed
         float* rv = (float*)(st + 2 * TILE);
@@ -454,9 +463,33 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
       return;
     }
     const int rbase = (ntile_total - 1 - step) * AB_BM;
+    if (regular && rbase + AB_BM <= rows) {
+      // a whole tile of whole time steps: lane offsets are fixed, the tile's base moves in scalar registers
+      const long tb = (long)(rbase >> rsh) * hq;   // first [t, hq] row of the tile
+      const uint32_t sa = __builtin_amdgcn_readfirstlane(smem_a + (step % AB_NST) * STAGE + wave * 1024);
+      const void* qb_ = uniform_ptr(Qg + tb * (DH * 2));
+      const void* ob_ = uniform_ptr(dOg + tb * (DH * 2));
+#pragma unroll
+      for (int ii = 0; ii < LOADS / 2; ii++) {
+        async_copy16_sv(qb_, voff[ii], sa + ii * 4096);
+        async_copy16_sv(ob_, voff[ii], sa + TILE + ii * 4096);
+      }
+      if (wave == 0) {   // always four copies so that the count per stage is fixed
+        const uint32_t rv = sa + 2 * TILE;
+        const uint32_t voffR = (uint32_t)((((l >> rsh) * hq + hh * a.r + (l & (a.r - 1)))) * 4);
+        const uint32_t voffG = (uint32_t)((l >> rsh) * a.h * 4);
+        const void* rb_ = uniform_ptr(rmg + tb);
+        if (Gg) async_copy4_sv(uniform_ptr(Gg + (long)((rbase >> rsh) + shift) * a.h), voffG, rv);
+        else async_copy4_sv(rb_, voffR, rv);
+        async_copy4_sv(rb_, voffR, rv + AB_BM * 4);
+        async_copy4_sv(uniform_ptr((dlg ? dlg : rmg) + tb), voffR, rv + 2 * AB_BM * 4);
+        async_copy4_sv(uniform_ptr((osg ? osg : rmg) + tb), voffR, rv + 3 * AB_BM * 4);
+      }
+      return;
+    }
 #pragma unroll
     for (int ii = 0; ii < LOADS / 2; ii++) {
-      const long ro = row_elem(rbase + grow[ii]) * (DH * 2) + gchk[ii];
+      const long ro = row_elem(rbase + grow(ii)) * (DH * 2) + gchk(ii);
       async_copy16(Qg + ro, st + (ii * 4 + wave) * 1024);
       async_copy16(dOg + ro, st + TILE + (ii * 4 + wave) * 1024);
     }

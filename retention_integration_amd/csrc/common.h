@@ -159,6 +159,13 @@ __device__ __forceinline__ void async_copy4_sv(const void* uniform_base, uint32_
                "s"(uniform_base)
                : "memory", "m0");
 }
+// For values that are uniform but were computed on the vector unit (anything behind an integer division): bring
+// them back to scalar registers, as the operands above require.
+__device__ __forceinline__ const void* uniform_ptr(const void* p) {
+  const uint64_t u = (uint64_t)(uintptr_t)p;
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)u), hi = __builtin_amdgcn_readfirstlane((uint32_t)(u >> 32));
+  return (const void*)(uintptr_t)(((uint64_t)hi << 32) | lo);
+}
 __device__ __forceinline__ uint32_t lds_addr(const void* p) {
   return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char*)p;
 }
