@@ -68,7 +68,8 @@ __global__ __launch_bounds__(256, 2) void sympow_grad_kernel(GradArgs a, int row
   const int row0 = (slot % row_blocks) * ROWS;
   const int bn = pair / a.h, hh = pair % a.h;
 
-  const int tid = threadIdx.x, l = tid & 63, g = l >> 4, wave = tid >> 6, tcol = l & 15;
+  const int tid = threadIdx.x, l = tid & 63, g = l >> 4, tcol = l & 15;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int hA = a.h * a.r, rows = a.c * a.r;
   const T* Xg = (const T*)a.X + (long)bn * a.c * hA * DK;
   const T* Gg = (const T*)a.G + (long)bn * a.c * hA * DV;
@@ -89,9 +90,18 @@ __global__ __launch_bounds__(256, 2) void sympow_grad_kernel(GradArgs a, int row
     return;
   }
 
+  // B rows are contiguous: the copies of a stage have fixed lane offsets and a base that moves in scalar registers
+  uint32_t boffs[LOADS];
+#pragma unroll
+  for (int ii = 0; ii < LOADS; ii++) {
+    const int pos = (ii * 4 + wave) * 64 + l, row = pos / CB;
+    boffs[ii] = (uint32_t)(row * (DV * 2) + 16 * ((pos % CB) ^ swz<CB>(row)));
+  }
+  const uint32_t ring_lds = lds_addr(ring) + wave * 1024;
   auto issue = [&](int step) {
     const char* src = Bg + (long)step * GR_FR * DV * 2;
-    async_load_tile<CB, GR_FR>(ring + (step % GR_NST) * STAGE, [&](int row) { return src + row * (DV * 2); });
+#pragma unroll
+    for (int ii = 0; ii < LOADS; ii++) async_copy16_sv(src, boffs[ii], ring_lds + (step % GR_NST) * STAGE + ii * 4096);
   };
   // X rows of this workgroup (waited for together with stage 0), then the first two stages
   async_load_tile<CX, ROWS>(xt, [&](int row) { return (const char*)(Xg + row_off(row0 + row) * DK); });

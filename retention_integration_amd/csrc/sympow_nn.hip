@@ -89,7 +89,8 @@ __global__ __launch_bounds__(256, DK <= 64 ? 3 : 2) void sympow_nn_kernel(NNArgs
   const int row0 = (slot % row_blocks) * ROWS;
   const int bn = pair / a.h, hh = pair % a.h;
 
-  const int tid = threadIdx.x, l = tid & 63, g = l >> 4, wave = tid >> 6, tcol = l & 15;
+  const int tid = threadIdx.x, l = tid & 63, g = l >> 4, tcol = l & 15;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int hA = a.h * a.r, rows = a.c * a.r;
   const T* Xg = (const T*)a.X + (long)bn * a.c * hA * DK;
   const char* Bg = (const char*)((const T*)a.B + ((long)bn * a.h + hh) * D * DV);
@@ -102,9 +103,18 @@ __global__ __launch_bounds__(256, DK <= 64 ? 3 : 2) void sympow_nn_kernel(NNArgs
   auto x_ptr = [&](int lrow, int col) -> const char* {
     return xt + lrow * (DK * 2) + (((col / 8) ^ swz<CX>(lrow)) * 16) + (col % 8) * 2;
   };
+  // B rows are contiguous: the copies of a stage have fixed lane offsets and a base that moves in scalar registers
+  uint32_t boffs[LOADS];
+#pragma unroll
+  for (int ii = 0; ii < LOADS; ii++) {
+    const int pos = (ii * 4 + wave) * 64 + l, row = pos / CB;
+    boffs[ii] = (uint32_t)(row * (DV * 2) + 16 * ((pos % CB) ^ swz<CB>(row)));
+  }
+  const uint32_t ring_lds = lds_addr(ring) + wave * 1024;
   auto issue = [&](int f0, int ringpos) {
     const char* src = Bg + (long)f0 * DV * 2;
-    async_load_tile<CB, NN_FR>(ring + ringpos * STAGE, [&](int row) { return src + row * (DV * 2); });
+#pragma unroll
+    for (int ii = 0; ii < LOADS; ii++) async_copy16_sv(src, boffs[ii], ring_lds + ringpos * STAGE + ii * 4096);
   };
 
   const bool skip = (EPI == NN_EPI_MERGE) && a.skip_first && (bn % a.n == 0);
