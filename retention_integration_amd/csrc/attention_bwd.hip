@@ -63,14 +63,15 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dq_kernel(AttnBwdArgs a,
   // Workgroups are dealt round-robin by their linear index to the 8 XCDs and then to the 4 shader engines of an
   // XCD; only the CU inside a shader engine is chosen by load.  Blocks differ in length (causal), so each of the 32
   // (XCD, shader engine) groups gets whole (batch, kv head) pairs, the longest blocks of all its pairs first.
+  // (integer division runs on the vector unit: readfirstlane brings the uniform results back to scalar registers)
   const int grp = blockIdx.x % 32, u = blockIdx.x / 32, ppg = (npairs + 31) / 32;
-  const int pair = (u % ppg) * 32 + grp;
+  const int pair = __builtin_amdgcn_readfirstlane((u % ppg) * 32 + grp);
   if (pair >= npairs) return;
   const int tid = threadIdx.x, l = tid & 63, g = l >> 4, tcol = l & 15;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int b = pair / a.h, hh = pair % a.h;
+  const int b = __builtin_amdgcn_readfirstlane(pair / a.h), hh = pair - b * a.h;
   const int hq = a.h * a.r, rows = a.tq * a.r, shift = a.tk - a.tq;
-  const int row0 = (nblocks - 1 - u / ppg) * ROWS;   // late rows see the most keys
+  const int row0 = (nblocks - 1 - __builtin_amdgcn_readfirstlane(u / ppg)) * ROWS;   // late rows see the most keys
   const T* Qg = (const T*)a.Q + (long)b * a.tq * hq * DH;
   const T* dOg = (const T*)a.dO + (long)b * a.tq * hq * DH;
   const char* Kg = (const char*)((const T*)a.K + (long)b * a.tk * a.h * DH + hh * DH);
@@ -117,10 +118,11 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dq_kernel(AttnBwdArgs a,
     if (j0 + AB_BN <= a.tk) {
       const char* kb_ = Kg + (long)j0 * kstride;
       const char* vb_ = Vg + (long)j0 * kstride;
+      const uint32_t sa = lds_addr(st) + wave * 1024;
 #pragma unroll
-      for (int ii = 0; ii < LOADS / 2; ii++) async_copy16(kb_ + goff[ii], st + (ii * 4 + wave) * 1024);
+      for (int ii = 0; ii < LOADS / 2; ii++) async_copy16_sv(kb_, goff[ii], sa + ii * 4096);
 #pragma unroll
-      for (int ii = 0; ii < LOADS / 2; ii++) async_copy16(vb_ + goff[ii], st + TILE + (ii * 4 + wave) * 1024);
+      for (int ii = 0; ii < LOADS / 2; ii++) async_copy16_sv(vb_, goff[ii], sa + TILE + ii * 4096);
     } else {   // last, partial tile: rows past the end repeat the last key (they are masked)
       async_load_tile<CPR, AB_BN>(st, [&](int row) { return Kg + (long)min(j0 + row, a.tk - 1) * kstride; });
       async_load_tile<CPR, AB_BN>(st + TILE, [&](int row) { return Vg + (long)min(j0 + row, a.tk - 1) * kstride; });

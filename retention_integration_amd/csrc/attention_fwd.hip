@@ -62,9 +62,11 @@ __global__ __launch_bounds__(256, OCC) void attention_fwd_kernel(AttnFwdArgs a, 
   // group then gets the same mix of long and short row blocks and the K/V of a pair stay in one L2.  Inside a
   // group the longest row blocks of all its pairs come first and the shortest last (they fill the tail).
   const int grp = blockIdx.x % 32, u = blockIdx.x / 32, ppg = (npairs + 31) / 32;
-  const int pair = (u % ppg) * 32 + grp, rblk = row_blocks - 1 - u / ppg;
+  // (integer division runs on the vector unit: readfirstlane brings the uniform results back to scalar registers)
+  const int pair = __builtin_amdgcn_readfirstlane((u % ppg) * 32 + grp);
+  const int rblk = row_blocks - 1 - __builtin_amdgcn_readfirstlane(u / ppg);
   if (pair >= npairs) return;
-  const int b = pair / a.h, hh = pair % a.h;
+  const int b = __builtin_amdgcn_readfirstlane(pair / a.h), hh = pair - b * a.h;
   const int hq = a.h * a.r, rows = a.tq * a.r, shift = a.tk - a.tq;
   // every other workgroup hands its 16*MT-row slices to the waves in reverse order: the wave nearest the
   // diagonal has the most tiles, and co-resident workgroups then load the four SIMDs evenly
@@ -100,10 +102,11 @@ __global__ __launch_bounds__(256, OCC) void attention_fwd_kernel(AttnFwdArgs a, 
     if (j0 + AT_BN <= a.tk) {
       const char* kb_ = Kg + (long)j0 * kstride;
       const char* vb_ = Vg + (long)j0 * kstride;
+      const uint32_t sa = lds_addr(st) + wave * 1024;
 #pragma unroll
-      for (int ii = 0; ii < LOADS / 2; ii++) async_copy16(kb_ + goff[ii], st + (ii * 4 + wave) * 1024);
+      for (int ii = 0; ii < LOADS / 2; ii++) async_copy16_sv(kb_, goff[ii], sa + ii * 4096);
 #pragma unroll
-      for (int ii = 0; ii < LOADS / 2; ii++) async_copy16(vb_ + goff[ii], st + TILE + (ii * 4 + wave) * 1024);
+      for (int ii = 0; ii < LOADS / 2; ii++) async_copy16_sv(vb_, goff[ii], sa + TILE + ii * 4096);
     } else {   // last, partial tile: rows past the end repeat the last key (they are masked)
       async_load_tile<CPR, AT_BN>(st, [&](int row) { return Kg + (long)min(j0 + row, a.tk - 1) * kstride; });
       async_load_tile<CPR, AT_BN>(st + TILE, [&](int row) { return Vg + (long)min(j0 + row, a.tk - 1) * kstride; });
