@@ -238,6 +238,7 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dq_kernel(AttnBwdArgs a,
     const float cw = DIAG ? 1.f : __expf(fminf(Rw - graw[AB_BN - 1], AB_EXP_CLAMP));
 #pragma unroll
     for (int kp = 0; kp < KT / 2; kp++) {
+      if (DIAG && j0 + 32 * kp > w_last_ti) continue;   // these 32 keys come after every row of the wave
       v8 kf[2][KS], vf[2][KS];
       f32x4 ev[2];
 #pragma unroll
@@ -415,8 +416,11 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
   const int tile_lo = max(0, (key0 - shift) * a.r) / AB_BM;               // first tile that sees any key of the block
   const int nsteps = max(0, ntile_total - tile_lo);
   // far tiles: every row's time index >= last_key  <=>  tile >= ceil((last_key - shift) * r / BM)
+  // (per workgroup, not per wave: the row factors in LDS are relative to the gate at the workgroup's last key and
+  // stay <= 1 only for rows after it)
   const int tile_far = max(tile_lo, (max(0, (last_key - shift) * a.r) + AB_BM - 1) / AB_BM);
   const int n_far = max(0, ntile_total - tile_far);
+  const int row_vis = (wkey0 - shift) * a.r;   // folded rows before this one see none of the wave's keys
   // tiles with at least one row that sees the wave's first key
   const int tile_w = max(tile_lo, max(0, (wkey0 - shift) * a.r) / AB_BM);
   const int n_seen = max(n_far, ntile_total - tile_w);
@@ -587,7 +591,7 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
     return st;
   };
 
-  auto tile = [&](const char* st, auto far_c) {
+  auto tile = [&](const char* st, int rbase, auto far_c) {
     constexpr bool FAR = decltype(far_c)::value != 0;
     uint32_t qb[KS], ob[KS], qtb[NT], otb[NT], fb;
     {
@@ -611,6 +615,7 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
     }
 #pragma unroll
     for (int qp = 0; qp < QT / 2; qp++) {
+      if (!FAR && rbase + 32 * qp + 31 < row_vis) continue;   // these 32 rows come before every key of the wave
       v8 qf[2][KS], dof[2][KS];
       f32x4 fa[2], fc[2], fd[2], fe[2];   // FAR: factor*scale, factor*dl;  near: G_q - m, time index, dl, dO scale
 #pragma unroll
@@ -698,7 +703,7 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
   };
 
   int step = 0;
-  for (; step < n_far; step++) tile(sync_step(step), IC<1>{});
+  for (; step < n_far; step++) tile(sync_step(step), (ntile_total - 1 - step) * AB_BM, IC<1>{});
   // the far tiles were accumulated without the key factor exp(R - G_k) (<= 1); apply it once.  The tiles near
   // the diagonal are accumulated in absolute terms (their packed weights stay <= the true ones).
 #pragma unroll
@@ -711,7 +716,7 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
     }
     dgk[kj] *= c;
   }
-  for (; step < n_seen; step++) tile(sync_step(step), IC<0>{});
+  for (; step < n_seen; step++) tile(sync_step(step), (ntile_total - 1 - step) * AB_BM, IC<0>{});
   for (; step < nsteps; step++) sync_step(step);
 
   T* dKg = (T*)a.dK + (long)b * a.tk * a.h * DH + hh * DH;

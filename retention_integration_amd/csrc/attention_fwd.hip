@@ -230,6 +230,7 @@ __global__ __launch_bounds__(256, OCC) void attention_fwd_kernel(AttnFwdArgs a, 
     const float cw = DIAG ? 1.f : __expf(fminf(Rw - graw[AT_BN - 1], AT_EXP_CLAMP));
 #pragma unroll
     for (int kp = 0; kp < KT / 2; kp++) {
+      if (DIAG && j0 + 32 * kp > w_last_ti) continue;   // these 32 keys come after every row of the wave
       // S^T for 32 keys: operands first, then every product, so the matrix pipe runs back to back
       v8 kf[2][KS];
       f32x4 ev[2];
