@@ -110,7 +110,6 @@ __global__ __launch_bounds__(256, 2) void sympow_grad_kernel(GradArgs a, int row
 
   // per-lane row data (row = this lane's column of the dphi^T tiles)
   v8 Gf[MT][KS];
-  float cv[MT];
   int lrow[MT];
   bool live[MT];
 #pragma unroll
@@ -124,7 +123,6 @@ __global__ __launch_bounds__(256, 2) void sympow_grad_kernel(GradArgs a, int row
       if (!live[mi]) z = (u32x4){0, 0, 0, 0};
       Gf[mi][ks] = __builtin_bit_cast(v8, z);
     }
-    cv[mi] = live[mi] ? (a.cvec ? a.cvec[(long)bn * a.c * hA + ro] : 1.f) : 0.f;
   }
   auto x_ptr = [&](int mi, int col) -> const char* {   // address of X[lrow[mi], col] in the swizzled tile
     return xt + lrow[mi] * (DK * 2) + (((col / 8) ^ swz<CX>(lrow[mi])) * 16) + (col % 8) * 2;
@@ -237,6 +235,17 @@ __global__ __launch_bounds__(256, 2) void sympow_grad_kernel(GradArgs a, int row
   // thread per (a, strip of 16 w): 16 consecutive floats of sB, 16 consecutive elements of U; U and U^T are both
   // read from the one tile (plain and transposing operand loads).
   T* Mt = (T*)ring;   // [DK (a)][LDM (w)]
+  // Row offsets and cvec are (re)computed here, from a copy of the row index the compiler cannot match with the one
+  // used before the sweep: nothing that is only needed now should stay in registers (or scratch) through it.
+  float cv[MT];
+  long rofs[MT];
+#pragma unroll
+  for (int mi = 0; mi < MT; mi++) {
+    int lr = lrow[mi];
+    asm volatile("" : "+v"(lr));
+    rofs[mi] = row_off(row0 + lr);
+    cv[mi] = live[mi] ? (a.cvec ? a.cvec[(long)bn * a.c * hA + rofs[mi]] : 1.f) : 0.f;
+  }
   for (int part = 0; part < 2; part++) {
     lds_barrier();
     for (int idx = tid; idx < DK * TT; idx += 256) {
@@ -278,13 +287,14 @@ __global__ __launch_bounds__(256, 2) void sympow_grad_kernel(GradArgs a, int row
         }
         acc[mi][wt] += t * (cv[mi] * OnePair<T>::up);
       }
+      __builtin_amdgcn_sched_barrier(0);   // one row tile at a time: the accumulators leave few registers free
     }
   }
 
 #pragma unroll
   for (int mi = 0; mi < MT; mi++) {
     if (!live[mi]) continue;
-    const long ro = row_off(row0 + lrow[mi]);
+    const long ro = rofs[mi];
 #pragma unroll
     for (int k = 0; k < TT; k++) {
       float o4[4];

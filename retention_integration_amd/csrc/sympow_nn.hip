@@ -205,7 +205,7 @@ __global__ __launch_bounds__(256, DK <= 64 ? 3 : 2) void sympow_nn_kernel(NNArgs
           const T xs = __builtin_bit_cast(T, xbits);
           const v8 af = prow[mi].make(xs);
 #pragma unroll
-          for (int nt = 0; nt < NT; nt++) acc[mi][nt] = mfma16(vf[nt], af, acc[mi][nt]);   // out^T[e, row]
+          for (int nt = 0; nt < NT; nt++) acc[mi][nt] = mfma16(af, vf[nt], acc[mi][nt]);   // phi first: see below
         }
       }
       if (cur.next()) {
@@ -267,10 +267,25 @@ __global__ __launch_bounds__(256, DK <= 64 ? 3 : 2) void sympow_nn_kernel(NNArgs
     }
   }
 
-  // epilogue: the accumulators hold out^T, element v of lane l is column 16*nt + 4*(l/16) + v of the lane's row
-  // (row0 + wave*16*MT + 16*mi + l%16): one row per lane, 8-byte loads and stores
+  // Epilogue.  The accumulators hold out[row 4*(l/16)+v, column 16*nt + l%16] (the phi operand stays the first
+  // matrix-core operand: in the sibling kernel sympow_tn the other order measured ~10 % slower).  Each 16-row tile
+  // goes through a private LDS buffer once so that a lane ends up with 4 consecutive columns of ONE row (its own:
+  // row0 + wave*16*MT + 16*mi + l%16): per-row scalars are computed once per lane, loads and stores are 8 bytes.
   T* out = (T*)a.out + (long)bn * a.c * hA * DV;
   const float log_gamma = 0.5f * __logf((float)D);
+  constexpr int TP = DV + 4;   // pitch of the transposition buffer in floats (conflict-free both ways)
+  static_assert(4 * 16 * TP * 4 <= RING_BYTES + 64 * MT * DK * 2, "transposition buffers fit the (idle) LDS");
+  float* tbuf = (float*)smem + wave * 16 * TP;
+  lds_barrier();   // every wave is done with the ring and the X tile
+#pragma unroll
+  for (int mi = 0; mi < MT; mi++) {
+#pragma unroll
+    for (int nt = 0; nt < NT; nt++)
+#pragma unroll
+      for (int v = 0; v < 4; v++) tbuf[(4 * g + v) * TP + 16 * nt + tcol] = acc[mi][nt][v];
+#pragma unroll
+    for (int nt = 0; nt < NT; nt++) acc[mi][nt] = *(const f32x4*)(tbuf + tcol * TP + 16 * nt + 4 * g);
+  }
 #pragma unroll
   for (int mi = 0; mi < MT; mi++) {
     const int row = row0 + wave * 16 * MT + 16 * mi + tcol;
