@@ -89,6 +89,18 @@ size_t pr_discumsum_bwd_workspace(int B, int n, int H, int64_t F, int dtype);
 int pr_discumsum_bwd(const void* dY, const void* Y, const float* log_G, void* dX, float* dlog_G, void* workspace,
                      int B, int n, int n_out, int H, int64_t F, int dtype, void* stream);
 
+/* The two scans of the chunked algorithm -- discumsum(S, lcs) and discumsum(s, lcs),
+ * retention/power_retention_maker.py:167-170 -- in one launch each way (the small fp32 scan is bound by latency and
+ * costs nothing next to the big one).  S [B,n,H,F] 16-bit, s [B,n,H,F2] fp32, same log_G [B,n,H].
+ * Backward: dlog_G [B,n,H] receives the SUM of both scans' gate gradients.
+ *   workspace: pr_state_scan_bwd_workspace() bytes. */
+int pr_state_scan_fwd(const void* S, const float* s, const float* log_G, void* S_out, float* s_out, int B, int n,
+                      int n_out, int H, int64_t F, int64_t F2, int dtype, void* stream);
+size_t pr_state_scan_bwd_workspace(int B, int n, int H, int64_t F, int64_t F2);
+int pr_state_scan_bwd(const void* dS_out, const void* S_out, const float* ds_out, const float* s_out,
+                      const float* log_G, void* dS, float* ds, float* dlog_G, void* workspace, int B, int n, int n_out,
+                      int H, int64_t F, int64_t F2, int dtype, void* stream);
+
 /* query_state(Q, S, s, Y_attn, l_attn, rowmax, deg, scale, zero_initial_state) --
  * retention/_query_state/reference.py:36-96,166-191, Triton twin retention/_query_state/triton.py:54-169,478-544.
  *   Q [BN,c,h*r,d] (already gated), S [BN,h,D,d], s [BN,h,D] fp32,
@@ -128,7 +140,8 @@ int pr_chunk_prep_fwd(const float* log_G, const void* K, const void* Q, float* A
  *   dQ_state = gradient w.r.t. Qg (query_state backward), dK_state, dV_state = gradients w.r.t. Kd, V
  *   (update_state backward).  With A = NULL the factors are 1 and dGq, dGk, dotk are not written.
  * pr_chunk_gate_scan_bwd finishes the gate gradient: dlog_G holds dGk + sum over the r query heads of dGq on entry,
- *   dlog_G[c-1] += (sum_t dotk)/deg + dlcs_a + dlcs_b, then the reverse cumulative sum over the chunk, in place. */
+ *   dlog_G[c-1] += (sum_t dotk)/deg + dlcs_a + dlcs_b (dlcs_b may be NULL), then the reverse cumulative sum over the
+ *   chunk, in place. */
 int pr_chunk_attention_bwd(const void* Q, const void* K, const void* V, const float* A, const float* rowmax,
                            const void* dO, const float* dl, const float* dO_scale, const void* dQ_state,
                            const void* dK_state, const void* dV_state, void* dQ, void* dK, void* dV, float* dGq,

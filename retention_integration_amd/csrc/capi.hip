@@ -142,6 +142,34 @@ int pr_discumsum_bwd(const void* dY, const void* Y, const float* log_G, void* dX
                                   (hipStream_t)stream), "discumsum_bwd");
 }
 
+int pr_state_scan_fwd(const void* S, const float* s, const float* log_G, void* S_out, float* s_out, int B, int n,
+                      int n_out, int H, int64_t F, int64_t F2, int dtype, void* stream) {
+  if (dtype != PR_BF16 && dtype != PR_F16) return fail(PR_ERR_DTYPE, "state_scan_fwd: unsupported dtype");
+  if (bad_ptr(S) || bad_ptr(s) || log_G == nullptr || bad_ptr(S_out) || bad_ptr(s_out))
+    return fail(PR_ERR_ARG, "state_scan_fwd: null or misaligned pointer");
+  if (B <= 0 || n <= 0 || H <= 0 || F <= 0 || F2 <= 0 || F % 8 != 0 || (n_out != n && n_out != n + 1))
+    return fail(PR_ERR_ARG, "state_scan_fwd: need B,n,H,F2 > 0, F a multiple of 8, n_out in {n, n+1}");
+  return finish(pr::discumsum_pair_fwd(S, s, log_G, S_out, s_out, B, n, n_out, H, (long)F, (long)F2, dtype,
+                                       (hipStream_t)stream), "state_scan_fwd");
+}
+
+size_t pr_state_scan_bwd_workspace(int B, int n, int H, int64_t F, int64_t F2) {
+  return (size_t)pr::discumsum_pair_bwd_workspace_floats(B, n, H, (long)F, (long)F2) * sizeof(float);
+}
+
+int pr_state_scan_bwd(const void* dS_out, const void* S_out, const float* ds_out, const float* s_out,
+                      const float* log_G, void* dS, float* ds, float* dlog_G, void* workspace, int B, int n, int n_out,
+                      int H, int64_t F, int64_t F2, int dtype, void* stream) {
+  if (dtype != PR_BF16 && dtype != PR_F16) return fail(PR_ERR_DTYPE, "state_scan_bwd: unsupported dtype");
+  if (bad_ptr(dS_out) || bad_ptr(S_out) || bad_ptr(ds_out) || bad_ptr(s_out) || log_G == nullptr || bad_ptr(dS) ||
+      bad_ptr(ds) || dlog_G == nullptr || bad_ptr(workspace))
+    return fail(PR_ERR_ARG, "state_scan_bwd: null or misaligned pointer");
+  if (B <= 0 || n <= 0 || H <= 0 || F <= 0 || F2 <= 0 || F % 8 != 0 || (n_out != n && n_out != n + 1))
+    return fail(PR_ERR_ARG, "state_scan_bwd: need B,n,H,F2 > 0, F a multiple of 8, n_out in {n, n+1}");
+  return finish(pr::discumsum_pair_bwd(dS_out, S_out, ds_out, s_out, log_G, dS, ds, dlog_G, (float*)workspace, B, n,
+                                       n_out, H, (long)F, (long)F2, dtype, (hipStream_t)stream), "state_scan_bwd");
+}
+
 int pr_query_state_fwd(const void* Q, const void* S, const float* s, const void* Y_attn, const float* l_attn,
                        const float* rowmax, void* O, float* den, int BN, int n, int c, int h, int r, int d,
                        float scale_p, int deg, int zero_initial_state, int dtype, void* stream) {
@@ -200,7 +228,7 @@ int pr_chunk_prep_fwd(const float* log_G, const void* K, const void* Q, float* A
 
 int pr_chunk_gate_scan_bwd(float* dlog_G, const float* dotk, const float* dlcs_a, const float* dlcs_b, int BN, int c,
                            int h, int deg, void* stream) {
-  if (!dlog_G || !dotk || !dlcs_a || !dlcs_b) return fail(PR_ERR_ARG, "chunk_gate_scan_bwd: null pointer");
+  if (!dlog_G || !dotk || !dlcs_a) return fail(PR_ERR_ARG, "chunk_gate_scan_bwd: null pointer");
   if (BN <= 0 || c <= 0 || h <= 0 || deg <= 0) return fail(PR_ERR_ARG, "chunk_gate_scan_bwd: need BN,c,h,deg > 0");
   return finish(pr::chunk_gate_scan_bwd(dlog_G, dotk, dlcs_a, dlcs_b, BN, c, h, deg, (hipStream_t)stream),
                 "chunk_gate_scan_bwd");

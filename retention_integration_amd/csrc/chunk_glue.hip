@@ -104,7 +104,7 @@ __global__ __launch_bounds__(256) void gate_scan_bwd_kernel(float* __restrict__ 
     if (tid < off) tot[tid] += tot[tid + off];
     __syncthreads();
   }
-  if (tid == 0) a[c - 1] += tot[0] * inv_deg + dlcs_a[(long)bn * h + hh] + dlcs_b[(long)bn * h + hh];
+  if (tid == 0) a[c - 1] += tot[0] * inv_deg + dlcs_a[(long)bn * h + hh] + (dlcs_b ? dlcs_b[(long)bn * h + hh] : 0.f);
   __syncthreads();
   block_scan(a, tot, c, true);
   for (int i = tid; i < c; i += 256) dA[base + (long)i * h] = a[i];

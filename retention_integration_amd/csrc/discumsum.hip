@@ -27,13 +27,13 @@ __device__ __forceinline__ float wave_sum_dpp(float x) {
   return sum_over_rows(x);
 }
 
-template <typename T, int AHEAD, int BYTES = 16>
-__global__ __launch_bounds__(256) void discumsum_fwd_kernel(const T* __restrict__ X, const float* __restrict__ logG,
-                                                            T* __restrict__ Y, int n, int n_out, int H, long F) {
+template <typename T, int AHEAD, int BYTES>
+__device__ __forceinline__ void discumsum_fwd_body(const T* __restrict__ X, const float* __restrict__ logG,
+                                                   T* __restrict__ Y, int n, int n_out, int H, long F, int block) {
   constexpr int N = Pack16<T, BYTES>::N;
   typedef typename Pack16<T, BYTES>::type vec;
   const long per_bh = F / N;
-  const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  const long idx = (long)block * blockDim.x + threadIdx.x;
   const int bh = blockIdx.y;
   if (idx >= per_bh) return;
   const int b = bh / H, hh = bh % H;
@@ -75,19 +75,36 @@ __global__ __launch_bounds__(256) void discumsum_fwd_kernel(const T* __restrict_
   }
 }
 
+template <typename T, int AHEAD, int BYTES = 16>
+__global__ __launch_bounds__(256) void discumsum_fwd_kernel(const T* __restrict__ X, const float* __restrict__ logG,
+                                                            T* __restrict__ Y, int n, int n_out, int H, long F) {
+  discumsum_fwd_body<T, AHEAD, BYTES>(X, logG, Y, n, n_out, H, F, blockIdx.x);
+}
+// Two tensors that share their gates in one launch: a 16-bit one (16 bytes per lane) in the first nblk blocks of a
+// row of the grid, a small fp32 one (one element per lane, every chunk in flight) in the rest.  The small scan is
+// bound by latency; next to the big one it costs nothing.
+template <typename T, int AHEAD>
+__global__ __launch_bounds__(256) void discumsum_pair_fwd_kernel(const T* __restrict__ X, const float* __restrict__ X2,
+                                                                 const float* __restrict__ logG, T* __restrict__ Y,
+                                                                 float* __restrict__ Y2, int n, int n_out, int H,
+                                                                 long F, long F2, int nblk) {
+  if ((int)blockIdx.x < nblk) discumsum_fwd_body<T, AHEAD, 16>(X, logG, Y, n, n_out, H, F, blockIdx.x);
+  else discumsum_fwd_body<float, 64, 4>(X2, logG, Y2, n, n_out, H, F2, blockIdx.x - nblk);
+}
+
 // Reverse scan: r_k = dY[k+1] + exp(log_G[k+1]) * r_{k+1};  dX[k] = r_k;
 // dlog_G[k] = exp(log_G[k]) * sum_F Y[k] * r_k, written as one partial per wave (summed by
 // discumsum_reduce_kernel in a fixed order, so the result is deterministic).
 // partial layout: [BH][n][waves_per_bh]
-template <typename T, int AHEAD, int BYTES = 16>
-__global__ __launch_bounds__(256) void discumsum_bwd_kernel(const T* __restrict__ dY, const T* __restrict__ Y,
-                                                            const float* __restrict__ logG, T* __restrict__ dX,
-                                                            float* __restrict__ partial, int n, int n_out, int H,
-                                                            long F, int waves_per_bh) {
+template <typename T, int AHEAD, int BYTES>
+__device__ __forceinline__ void discumsum_bwd_body(const T* __restrict__ dY, const T* __restrict__ Y,
+                                                   const float* __restrict__ logG, T* __restrict__ dX,
+                                                   float* __restrict__ partial, int n, int n_out, int H, long F,
+                                                   int waves_per_bh, int block, int wave0) {
   constexpr int N = Pack16<T, BYTES>::N;
   typedef typename Pack16<T, BYTES>::type vec;
   const long per_bh = F / N;
-  const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  const long idx = (long)block * blockDim.x + threadIdx.x;
   const int bh = blockIdx.y;
   const bool live = idx < per_bh;
   const int b = bh / H, hh = bh % H;
@@ -97,7 +114,7 @@ __global__ __launch_bounds__(256) void discumsum_bwd_kernel(const T* __restrict_
   vec* dx = (vec*)(dX + ((long)b * n * H + hh) * F) + safe;
   const long xs = (long)H * F / N;
   const float* lg = logG + (long)b * n * H + hh;
-  const int wave = (blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+  const int wave = wave0 + ((block * blockDim.x + threadIdx.x) >> 6);
   float* part = partial + (long)bh * n * waves_per_bh + wave;
 
   float r[N];
@@ -144,6 +161,30 @@ __global__ __launch_bounds__(256) void discumsum_bwd_kernel(const T* __restrict_
       }
     }
   }
+}
+
+template <typename T, int AHEAD, int BYTES = 16>
+__global__ __launch_bounds__(256) void discumsum_bwd_kernel(const T* __restrict__ dY, const T* __restrict__ Y,
+                                                            const float* __restrict__ logG, T* __restrict__ dX,
+                                                            float* __restrict__ partial, int n, int n_out, int H,
+                                                            long F, int waves_per_bh) {
+  discumsum_bwd_body<T, AHEAD, BYTES>(dY, Y, logG, dX, partial, n, n_out, H, F, waves_per_bh, blockIdx.x, 0);
+}
+// The pair of tensors of discumsum_pair_fwd_kernel; their gate gradients land in one set of partials, so dlog_G is
+// the sum of both.
+template <typename T, int AHEAD>
+__global__ __launch_bounds__(256) void discumsum_pair_bwd_kernel(const T* __restrict__ dY, const T* __restrict__ Y,
+                                                                 const float* __restrict__ dY2,
+                                                                 const float* __restrict__ Y2,
+                                                                 const float* __restrict__ logG, T* __restrict__ dX,
+                                                                 float* __restrict__ dX2, float* __restrict__ partial,
+                                                                 int n, int n_out, int H, long F, long F2, int nblk,
+                                                                 int waves_per_bh) {
+  if ((int)blockIdx.x < nblk)
+    discumsum_bwd_body<T, AHEAD, 16>(dY, Y, logG, dX, partial, n, n_out, H, F, waves_per_bh, blockIdx.x, 0);
+  else
+    discumsum_bwd_body<float, 64, 4>(dY2, Y2, logG, dX2, partial, n, n_out, H, F2, waves_per_bh, blockIdx.x - nblk,
+                                     nblk * 4);
 }
 
 // one wave per (bh, k): sums the waves_per_bh partials in a fixed order
@@ -205,6 +246,56 @@ static int launch_bwd(const void* dY, const void* Y, const float* logG, void* dX
   hipLaunchKernelGGL(discumsum_reduce_kernel, dim3((tot * 64 + 255) / 256), dim3(256), 0, st, partial, dlogG, n, H,
                      waves, B * H);
   return (int)hipGetLastError();
+}
+
+template <typename T>
+static int launch_pair_fwd(const void* X, const float* X2, const float* logG, void* Y, float* Y2, int B, int n,
+                           int n_out, int H, long F, long F2, hipStream_t st) {
+  const int nblk = (int)((F / Pack16<T>::N + 255) / 256), nblk2 = (int)((F2 + 255) / 256);
+  dim3 grid((unsigned)(nblk + nblk2), (unsigned)(B * H));
+  if ((F / Pack16<T>::N) * B * H < 256 * 1024)
+    hipLaunchKernelGGL((discumsum_pair_fwd_kernel<T, 16>), grid, dim3(256), 0, st, (const T*)X, X2, logG, (T*)Y, Y2, n,
+                       n_out, H, F, F2, nblk);
+  else
+    hipLaunchKernelGGL((discumsum_pair_fwd_kernel<T, 4>), grid, dim3(256), 0, st, (const T*)X, X2, logG, (T*)Y, Y2, n,
+                       n_out, H, F, F2, nblk);
+  return (int)hipGetLastError();
+}
+template <typename T>
+static int launch_pair_bwd(const void* dY, const void* Y, const float* dY2, const float* Y2, const float* logG,
+                           void* dX, float* dX2, float* dlogG, float* partial, int B, int n, int n_out, int H, long F,
+                           long F2, hipStream_t st) {
+  const int nblk = (int)((F / Pack16<T>::N + 255) / 256), nblk2 = (int)((F2 + 255) / 256);
+  const int waves = (nblk + nblk2) * 4, tot = B * H * n;
+  dim3 grid((unsigned)(nblk + nblk2), (unsigned)(B * H));
+  if ((F / Pack16<T>::N) * B * H < 256 * 1024)
+    hipLaunchKernelGGL((discumsum_pair_bwd_kernel<T, 8>), grid, dim3(256), 0, st, (const T*)dY, (const T*)Y, dY2, Y2,
+                       logG, (T*)dX, dX2, partial, n, n_out, H, F, F2, nblk, waves);
+  else
+    hipLaunchKernelGGL((discumsum_pair_bwd_kernel<T, 2>), grid, dim3(256), 0, st, (const T*)dY, (const T*)Y, dY2, Y2,
+                       logG, (T*)dX, dX2, partial, n, n_out, H, F, F2, nblk, waves);
+  hipLaunchKernelGGL(discumsum_reduce_kernel, dim3((tot * 64 + 255) / 256), dim3(256), 0, st, partial, dlogG, n, H,
+                     waves, B * H);
+  return (int)hipGetLastError();
+}
+
+int discumsum_pair_fwd(const void* X, const float* X2, const float* logG, void* Y, float* Y2, int B, int n, int n_out,
+                       int H, long F, long F2, int dtype, hipStream_t st) {
+  if (dtype == DT_BF16) return launch_pair_fwd<bf16_t>(X, X2, logG, Y, Y2, B, n, n_out, H, F, F2, st);
+  if (dtype == DT_F16) return launch_pair_fwd<f16_t>(X, X2, logG, Y, Y2, B, n, n_out, H, F, F2, st);
+  return -1;
+}
+long discumsum_pair_bwd_workspace_floats(int B, int n, int H, long F, long F2) {
+  return (long)B * H * ((F / 8 + 255) / 256 + (F2 + 255) / 256) * 4 * n;
+}
+int discumsum_pair_bwd(const void* dY, const void* Y, const float* dY2, const float* Y2, const float* logG, void* dX,
+                       float* dX2, float* dlogG, float* partial, int B, int n, int n_out, int H, long F, long F2,
+                       int dtype, hipStream_t st) {
+  if (dtype == DT_BF16)
+    return launch_pair_bwd<bf16_t>(dY, Y, dY2, Y2, logG, dX, dX2, dlogG, partial, B, n, n_out, H, F, F2, st);
+  if (dtype == DT_F16)
+    return launch_pair_bwd<f16_t>(dY, Y, dY2, Y2, logG, dX, dX2, dlogG, partial, B, n, n_out, H, F, F2, st);
+  return -1;
 }
 
 int discumsum_fwd(const void* X, const float* logG, void* Y, int B, int n, int n_out, int H, long F, int dtype,

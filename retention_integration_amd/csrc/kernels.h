@@ -9,6 +9,13 @@ int discumsum_fwd(const void* X, const float* logG, void* Y, int B, int n, int n
                   hipStream_t st);
 int discumsum_bwd(const void* dY, const void* Y, const float* logG, void* dX, float* dlogG, float* partial, int B,
                   int n, int n_out, int H, long F, int dtype, hipStream_t st);
+// the state and its fp32 key sums (same gates) in one launch each way; dlogG is the sum of both contributions
+int discumsum_pair_fwd(const void* X, const float* X2, const float* logG, void* Y, float* Y2, int B, int n, int n_out,
+                       int H, long F, long F2, int dtype, hipStream_t st);
+long discumsum_pair_bwd_workspace_floats(int B, int n, int H, long F, long F2);
+int discumsum_pair_bwd(const void* dY, const void* Y, const float* dY2, const float* Y2, const float* logG, void* dX,
+                       float* dX2, float* dlogG, float* partial, int B, int n, int n_out, int H, long F, long F2,
+                       int dtype, hipStream_t st);
 long discumsum_bwd_workspace_floats(int B, int n, int H, long F, int dtype);
 
 // sympow_tn.hip: A [BN,c,h*r,d], Bm [BN,c,h*r,d], w [BN,c,h*r] or null -> S [BN,h,D,d], s [BN,h,D]

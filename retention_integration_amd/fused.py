@@ -56,8 +56,8 @@ def chunked_fwd(Q: Tensor, K: Tensor, V: Tensor, log_G: Optional[Tensor], deg: i
     S, s = _empty((BN, h, D, d), dt, dev), _empty((BN, h, D), f32, dev)
     _lib.check(lib.pr_update_state_fwd(p(Kd_), p(V), p(S), p(s), BN, c, h, d, 2, code, st), "update_state_fwd")
     Sc, sc = torch.empty_like(S), torch.empty_like(s)
-    _lib.check(lib.pr_discumsum_fwd(p(S), p(lcs), p(Sc), b, n, n, h, D * d, code, st), "discumsum_fwd")
-    _lib.check(lib.pr_discumsum_fwd(p(s), p(lcs), p(sc), b, n, n, h, D, _lib.PR_F32, st), "discumsum_fwd")
+    _lib.check(lib.pr_state_scan_fwd(p(S), p(s), p(lcs), p(Sc), p(sc), b, n, n, h, D * d, D, code, st),
+               "state_scan_fwd")
     del S, s
 
     Ya = torch.empty_like(Q)
@@ -111,13 +111,10 @@ def chunked_bwd(Q: Tensor, K: Tensor, V: Tensor, A: Tensor, lcs: Tensor, Kd: Ten
                                       p(dYa), p(dla), p(ws), BN, n, c, h, r, d, scale ** deg, 2, 1, code, st),
                "query_state_bwd")
     dS, ds = torch.empty_like(Sc), torch.empty_like(sc)
-    dl1, dl2 = torch.empty_like(lcs), torch.empty_like(lcs)
-    ws = _empty((max(lib.pr_discumsum_bwd_workspace(b, n, h, D * d, code),
-                     lib.pr_discumsum_bwd_workspace(b, n, h, D, _lib.PR_F32)),), u8, dev)
-    _lib.check(lib.pr_discumsum_bwd(p(dSc), p(Sc), p(lcs), p(dS), p(dl1), p(ws), b, n, n, h, D * d, code, st),
-               "discumsum_bwd")
-    _lib.check(lib.pr_discumsum_bwd(p(dsc), p(sc), p(lcs), p(ds), p(dl2), p(ws), b, n, n, h, D, _lib.PR_F32, st),
-               "discumsum_bwd")
+    dlcs = torch.empty_like(lcs)   # gate gradient of both scans
+    ws = _empty((lib.pr_state_scan_bwd_workspace(b, n, h, D * d, D),), u8, dev)
+    _lib.check(lib.pr_state_scan_bwd(p(dSc), p(Sc), p(dsc), p(sc), p(lcs), p(dS), p(ds), p(dlcs), p(ws), b, n, n, h,
+                                     D * d, D, code, st), "state_scan_bwd")
     dKd, dVs = torch.empty_like(K), torch.empty_like(V)
     _lib.check(lib.pr_update_state_bwd(p(Kd), p(V), p(dS), p(ds), p(dKd), p(dVs), BN, c, h, d, 2, code, st),
                "update_state_bwd")
@@ -133,7 +130,7 @@ def chunked_bwd(Q: Tensor, K: Tensor, V: Tensor, A: Tensor, lcs: Tensor, Kd: Ten
     dlg = _empty((0,), f32, dev)
     if gated:
         dlg = dGk.add_(dGq.view(b, t, h, r).sum(-1)) if r > 1 else dGk.add_(dGq.view(b, t, h))
-        _lib.check(lib.pr_chunk_gate_scan_bwd(p(dlg), p(dotk), p(dl1), p(dl2), BN, c, h, deg, st),
+        _lib.check(lib.pr_chunk_gate_scan_bwd(p(dlg), p(dotk), p(dlcs), None, BN, c, h, deg, st),
                    "chunk_gate_scan_bwd")
     return dQa, dKa, dVa, dlg
 

@@ -84,6 +84,40 @@ def test_discumsum_1d_features(pra):
     check("Y", pra.discumsum(dev(X), dev(lg)), oracle.discumsum(X, lg), 1e-5)
 
 
+@pytest.mark.parametrize("n_out_extra", [0, 1])
+@pytest.mark.parametrize("dtype,F", [(torch.bfloat16, 768 * 32), (torch.float16, 2560 * 64)])
+def test_state_scan_pair_equals_separate_scans(pra, dtype, F, n_out_extra):
+    """The one-launch scan of (state, key sums) through the C ABI: same values as the two discumsum launches, and a
+    gate gradient equal to the sum of theirs (ref: retention/power_retention_maker.py:167-170)."""
+    from retention_integration_amd import _lib
+    lib, st, p = _lib.load(), _lib.stream(), _lib.ptr
+    b, n, h = 2, 6, 3
+    F2 = F // (32 if F == 768 * 32 else 64)
+    n_out = n + n_out_extra
+    S, s, lg = dev(rnd(b, n, h, F, dtype=dtype, seed=11)), dev(rnd(b, n, h, F2, dtype=torch.float32, seed=12)), dev(gates(b, n, h, seed=13))
+    code = _lib.dtype_code(dtype)
+    Sc, sc = torch.empty(b, n_out, h, F, dtype=dtype, device=DEV), torch.empty(b, n_out, h, F2, device=DEV)
+    Sc1, sc1 = torch.empty_like(Sc), torch.empty_like(sc)
+    _lib.check(lib.pr_state_scan_fwd(p(S), p(s), p(lg), p(Sc), p(sc), b, n, n_out, h, F, F2, code, st), "pair fwd")
+    _lib.check(lib.pr_discumsum_fwd(p(S), p(lg), p(Sc1), b, n, n_out, h, F, code, st), "fwd")
+    _lib.check(lib.pr_discumsum_fwd(p(s), p(lg), p(sc1), b, n, n_out, h, F2, _lib.PR_F32, st), "fwd")
+    assert torch.equal(Sc, Sc1) and torch.equal(sc, sc1)
+
+    dSc, dsc = dev(rnd(b, n_out, h, F, dtype=dtype, seed=14)), dev(rnd(b, n_out, h, F2, dtype=torch.float32, seed=15))
+    u8 = torch.uint8
+    dS, ds, dlg = torch.empty_like(S), torch.empty_like(s), torch.empty_like(lg)
+    ws = torch.empty(lib.pr_state_scan_bwd_workspace(b, n, h, F, F2), dtype=u8, device=DEV)
+    _lib.check(lib.pr_state_scan_bwd(p(dSc), p(Sc), p(dsc), p(sc), p(lg), p(dS), p(ds), p(dlg), p(ws), b, n, n_out, h,
+                                     F, F2, code, st), "pair bwd")
+    dS1, ds1, dl1, dl2 = torch.empty_like(S), torch.empty_like(s), torch.empty_like(lg), torch.empty_like(lg)
+    ws1 = torch.empty(max(lib.pr_discumsum_bwd_workspace(b, n, h, F, code),
+                          lib.pr_discumsum_bwd_workspace(b, n, h, F2, _lib.PR_F32)), dtype=u8, device=DEV)
+    _lib.check(lib.pr_discumsum_bwd(p(dSc), p(Sc), p(lg), p(dS1), p(dl1), p(ws1), b, n, n_out, h, F, code, st), "bwd")
+    _lib.check(lib.pr_discumsum_bwd(p(dsc), p(sc), p(lg), p(ds1), p(dl2), p(ws1), b, n, n_out, h, F2, _lib.PR_F32, st), "bwd")
+    assert torch.equal(dS, dS1) and torch.equal(ds, ds1)
+    check("dlog_G", dlg, dl1 + dl2, 1e-5)
+
+
 # ---------------------------------------------------------------- update_state
 @pytest.mark.parametrize("dtype,d,c", [(torch.bfloat16, 64, 128), (torch.bfloat16, 32, 48), (torch.float16, 128, 64),
                                        (torch.float16, 64, 32), (torch.bfloat16, 128, 32)])
