@@ -139,16 +139,16 @@ int pr_chunk_prep_fwd(const float* log_G, const void* K, const void* Q, float* A
  *   -(K.dK_state) exp((A[c-1]-A)/deg)/deg,  dotk [BN,c,h] = (K.dK_state) exp((A[c-1]-A)/deg).
  *   dQ_state = gradient w.r.t. Qg (query_state backward), dK_state, dV_state = gradients w.r.t. Kd, V
  *   (update_state backward).  With A = NULL the factors are 1 and dGq, dGk, dotk are not written.
- * pr_chunk_gate_scan_bwd finishes the gate gradient: dlog_G holds dGk + sum over the r query heads of dGq on entry,
- *   dlog_G[c-1] += (sum_t dotk)/deg + dlcs_a + dlcs_b (dlcs_b may be NULL), then the reverse cumulative sum over the
- *   chunk, in place. */
+ * pr_chunk_gate_scan_bwd finishes the gate gradient: dlog_G holds dGk on entry; the r query heads' dGq [BN,c,h*r]
+ *   are added (dGq may be NULL), dlog_G[c-1] += (sum_t dotk)/deg + dlcs_a + dlcs_b (dlcs_b may be NULL), then the
+ *   reverse cumulative sum over the chunk, in place. */
 int pr_chunk_attention_bwd(const void* Q, const void* K, const void* V, const float* A, const float* rowmax,
                            const void* dO, const float* dl, const float* dO_scale, const void* dQ_state,
                            const void* dK_state, const void* dV_state, void* dQ, void* dK, void* dV, float* dGq,
                            float* dGk, float* dotk, int BN, int c, int h, int r, int d, float scale, int deg,
                            int dtype, void* stream);
-int pr_chunk_gate_scan_bwd(float* dlog_G, const float* dotk, const float* dlcs_a, const float* dlcs_b, int BN, int c,
-                           int h, int deg, void* stream);
+int pr_chunk_gate_scan_bwd(float* dlog_G, const float* dGq, const float* dotk, const float* dlcs_a, const float* dlcs_b,
+                           int BN, int c, int h, int r, int deg, void* stream);
 
 /* Single-token inference step on the state -- query: retention/power_retention_maker.py:358-363 with
  * retention/_query_state/reference.py:36-96 (one query position per sequence); update:

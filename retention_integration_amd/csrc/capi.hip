@@ -226,11 +226,12 @@ int pr_chunk_prep_fwd(const float* log_G, const void* K, const void* Q, float* A
                 "chunk_prep_fwd");
 }
 
-int pr_chunk_gate_scan_bwd(float* dlog_G, const float* dotk, const float* dlcs_a, const float* dlcs_b, int BN, int c,
-                           int h, int deg, void* stream) {
+int pr_chunk_gate_scan_bwd(float* dlog_G, const float* dGq, const float* dotk, const float* dlcs_a, const float* dlcs_b,
+                           int BN, int c, int h, int r, int deg, void* stream) {
   if (!dlog_G || !dotk || !dlcs_a) return fail(PR_ERR_ARG, "chunk_gate_scan_bwd: null pointer");
-  if (BN <= 0 || c <= 0 || h <= 0 || deg <= 0) return fail(PR_ERR_ARG, "chunk_gate_scan_bwd: need BN,c,h,deg > 0");
-  return finish(pr::chunk_gate_scan_bwd(dlog_G, dotk, dlcs_a, dlcs_b, BN, c, h, deg, (hipStream_t)stream),
+  if (BN <= 0 || c <= 0 || h <= 0 || r <= 0 || deg <= 0)
+    return fail(PR_ERR_ARG, "chunk_gate_scan_bwd: need BN,c,h,r,deg > 0");
+  return finish(pr::chunk_gate_scan_bwd(dlog_G, dGq, dotk, dlcs_a, dlcs_b, BN, c, h, r, deg, (hipStream_t)stream),
                 "chunk_gate_scan_bwd");
 }
 

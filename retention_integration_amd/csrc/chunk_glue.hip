@@ -83,10 +83,12 @@ __global__ __launch_bounds__(256) void gate_apply_fwd_kernel(const float* __rest
   }
 }
 
-// dA[c-1] += (sum_t dotk)/deg + dlcs_a + dlcs_b, then dlog_G = reverse cumsum of dA (in place)
-__global__ __launch_bounds__(256) void gate_scan_bwd_kernel(float* __restrict__ dA, const float* __restrict__ dotk,
+// dA += sum over the r query heads of dGq (when given); dA[c-1] += (sum_t dotk)/deg + dlcs_a + dlcs_b, then
+// dlog_G = reverse cumsum of dA (in place)
+__global__ __launch_bounds__(256) void gate_scan_bwd_kernel(float* __restrict__ dA, const float* __restrict__ dGq,
+                                                            const float* __restrict__ dotk,
                                                             const float* __restrict__ dlcs_a,
-                                                            const float* __restrict__ dlcs_b, int c, int h,
+                                                            const float* __restrict__ dlcs_b, int c, int h, int r,
                                                             float inv_deg) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   float* a = (float*)smem;
@@ -95,7 +97,10 @@ __global__ __launch_bounds__(256) void gate_scan_bwd_kernel(float* __restrict__ 
   const long base = (long)bn * c * h + hh;
   float ks = 0.f;
   for (int i = tid; i < c; i += 256) {
-    a[i] = dA[base + (long)i * h];
+    float v = dA[base + (long)i * h];
+    if (dGq)
+      for (int rr = 0; rr < r; rr++) v += dGq[(base + (long)i * h) * r + rr];
+    a[i] = v;
     ks += dotk[base + (long)i * h];
   }
   tot[tid] = ks;
@@ -134,12 +139,12 @@ int chunk_prep_fwd(const float* logG, const void* K, const void* Q, float* A, fl
   return -1;
 }
 
-int chunk_gate_scan_bwd(float* dA, const float* dotk, const float* dlcs_a, const float* dlcs_b, int BN, int c, int h,
-                        int deg, hipStream_t st) {
+int chunk_gate_scan_bwd(float* dA, const float* dGq, const float* dotk, const float* dlcs_a, const float* dlcs_b, int BN,
+                        int c, int h, int r, int deg, hipStream_t st) {
   if (c > GLUE_MAX_C) return -5;
   const size_t smem = (size_t)(c + 256) * sizeof(float);
-  hipLaunchKernelGGL(gate_scan_bwd_kernel, dim3((unsigned)(BN * h)), dim3(256), smem, st, dA, dotk, dlcs_a, dlcs_b, c,
-                     h, 1.f / deg);
+  hipLaunchKernelGGL(gate_scan_bwd_kernel, dim3((unsigned)(BN * h)), dim3(256), smem, st, dA, dGq, dotk, dlcs_a, dlcs_b,
+                     c, h, r, 1.f / deg);
   return (int)hipGetLastError();
 }
 

@@ -98,8 +98,8 @@ int qs_bwd_prep(const void* O, const void* dO, const float* den, const float* ro
 // chunk_glue.hip (return -5: chunk longer than the LDS-resident gate vector allows)
 int chunk_prep_fwd(const float* logG, const void* K, const void* Q, float* A, float* lcs, void* Kd, void* Qg, int BN,
                    int c, int h, int r, int d, int deg, int dtype, hipStream_t st);
-int chunk_gate_scan_bwd(float* dA, const float* dotk, const float* dlcs_a, const float* dlcs_b, int BN, int c, int h,
-                        int deg, hipStream_t st);
+int chunk_gate_scan_bwd(float* dA, const float* dGq, const float* dotk, const float* dlcs_a, const float* dlcs_b, int BN,
+                        int c, int h, int r, int deg, hipStream_t st);
 
 // decode.hip (return -3: more than 8 query rows per (batch, kv head))
 long decode_workspace_floats(int B, int h, int r, int tq, int d);

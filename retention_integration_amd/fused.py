@@ -129,8 +129,8 @@ def chunked_bwd(Q: Tensor, K: Tensor, V: Tensor, A: Tensor, lcs: Tensor, Kd: Ten
                                           scale, deg, code, st), "chunk_attention_bwd")
     dlg = _empty((0,), f32, dev)
     if gated:
-        dlg = dGk.add_(dGq.view(b, t, h, r).sum(-1)) if r > 1 else dGk.add_(dGq.view(b, t, h))
-        _lib.check(lib.pr_chunk_gate_scan_bwd(p(dlg), p(dotk), p(dlcs), None, BN, c, h, deg, st),
+        dlg = dGk
+        _lib.check(lib.pr_chunk_gate_scan_bwd(p(dlg), p(dGq), p(dotk), p(dlcs), None, BN, c, h, r, deg, st),
                    "chunk_gate_scan_bwd")
     return dQa, dKa, dVa, dlg
 
