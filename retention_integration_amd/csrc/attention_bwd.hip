@@ -100,7 +100,7 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dq_kernel(AttnBwdArgs a,
   // key tile (rows 0..63 in the K area, 64..127 in the V area), so that they arrive under the last tiles' work.
   const T* dQsg = a.dQs ? (const T*)a.dQs + (long)b * a.tq * hq * DH : nullptr;
   const int ntot = ntiles + (dQsg ? 1 : 0);
-  auto issue = [&](int it) {
+  auto issue = [&](int it) __attribute__((always_inline)) {
     char* st = smem + (it % AB_NST) * STAGE;
     if (it >= ntiles) {
 #pragma unroll
@@ -186,7 +186,7 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dq_kernel(AttnBwdArgs a,
 
   // exp(R - gate) relative to the tile's last key (<= 1) and to the first key of each 16-key group (>= 1);
   // written by wave 0, which issued the gate copy and so is the one that can wait for it
-  auto gate_factors = [&](int it) {
+  auto gate_factors = [&](int it) __attribute__((always_inline)) {
     float* graw = (float*)(smem + (it % AB_NST) * STAGE + 2 * TILE);
     const int rpos = min(AB_BN - 1, a.tk - 1 - it * AB_BN);
     const float gv = Gg ? graw[l] : 0.f;
@@ -199,7 +199,7 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dq_kernel(AttnBwdArgs a,
     wait_vmcnt<0>();
     gate_factors(0);
   }
-  auto sync_step = [&](int it) -> char* {
+  auto sync_step = [&](int it) __attribute__((always_inline)) -> char* {
     char* st = smem + (it % AB_NST) * STAGE;
     if (it + 1 < ntot) wait_vmcnt<LOADS>(); else wait_vmcnt<0>();
     lds_barrier();
@@ -213,7 +213,7 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dq_kernel(AttnBwdArgs a,
 
   // One 64-key tile.  Past tiles: key factors relative to the gate at the wave's first row (<= 1), the row factor
   // is applied to the accumulators after the past tiles.  Diagonal tiles: per-group reference, per-pair mask.
-  auto tile = [&](int it, const char* st, auto diag_c) {
+  auto tile = [&](int it, const char* st, auto diag_c) __attribute__((always_inline)) {
     constexpr bool DIAG = decltype(diag_c)::value != 0;
     const int j0 = it * AB_BN;
     const float* graw = (const float*)(st + 2 * TILE);
@@ -427,12 +427,12 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
 
   // copies of one stage: row inside the tile and byte offset of the 16-byte chunk in its row for this thread's
   // copy number ii (recomputed where needed: only the irregular paths use them)
-  auto grow = [&](int ii) -> int { return ((ii * 4 + wave) * 64 + l) / CPR; };
-  auto gchk = [&](int ii) -> uint32_t {
+  auto grow = [&](int ii) __attribute__((always_inline)) -> int { return ((ii * 4 + wave) * 64 + l) / CPR; };
+  auto gchk = [&](int ii) __attribute__((always_inline)) -> uint32_t {
     const int pos = (ii * 4 + wave) * 64 + l;
     return 16 * ((pos % CPR) ^ swz<CPR>(pos / CPR));
   };
-  auto row_elem = [&](int row) -> long {   // element offset of a (clamped) folded row in a [tq, hq] array
+  auto row_elem = [&](int row) __attribute__((always_inline)) -> long {   // element offset of a (clamped) folded row in a [tq, hq] array
     row = min(row, rows - 1);
     const int t = row / a.r;
     return (long)t * hq + hh * a.r + (row - t * a.r);
@@ -451,7 +451,7 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
 #pragma unroll
   for (int ii = 0; ii < LOADS / 2; ii++)
     voff[ii] = (uint32_t)((((grow(ii) >> rsh) * hq + hh * a.r + (grow(ii) & (a.r - 1))) * (DH * 2))) + gchk(ii);
-  auto issue = [&](int step) {
+  auto issue = [&](int step) __attribute__((always_inline)) {
     char* st = smem + (step % AB_NST) * STAGE;
     if (step >= nsteps) {
       const T* src = step == nsteps ? dKsg : dVsg;
@@ -560,7 +560,7 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
 
   // Row vectors of a tile (wave 0 issued their copies): G_q - m, time index (-1 for rows past the end), dl, dO
   // scale, and the far-tile factors scale^deg exp(G_q - m - R) * {dO scale, dl} (zero for rows past the end).
-  auto row_factors = [&](int step) {
+  auto row_factors = [&](int step) __attribute__((always_inline)) {
     float* rv = (float*)(smem + (step % AB_NST) * STAGE + 2 * TILE);
     const int row = (ntile_total - 1 - step) * AB_BM + l;
     const bool real = row < rows;
@@ -579,7 +579,7 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
     wait_vmcnt<0>();
     row_factors(0);
   }
-  auto sync_step = [&](int step) -> char* {
+  auto sync_step = [&](int step) __attribute__((always_inline)) -> char* {
     char* st = smem + (step % AB_NST) * STAGE;
     if (step + 1 < ntot) wait_vmcnt<LOADS>(); else wait_vmcnt<0>();
     lds_barrier();
@@ -591,7 +591,7 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
     return st;
   };
 
-  auto tile = [&](const char* st, int rbase, auto far_c) {
+  auto tile = [&](const char* st, int rbase, auto far_c) __attribute__((always_inline)) {
     constexpr bool FAR = decltype(far_c)::value != 0;
     uint32_t qb[KS], ob[KS], qtb[NT], otb[NT], fb;
     {

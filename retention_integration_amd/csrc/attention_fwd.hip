@@ -96,7 +96,7 @@ __global__ __launch_bounds__(256, OCC) void attention_fwd_kernel(AttnFwdArgs a, 
     const int pos = (ii * 4 + wave) * 64 + l, row = pos / CPR;
     goff[ii] = (uint32_t)(row * (int)kstride + 16 * ((pos % CPR) ^ swz<CPR>(row)));
   }
-  auto issue = [&](int it) {
+  auto issue = [&](int it) __attribute__((always_inline)) {
     char* st = smem + (it % AT_NST) * STAGE;
     const int j0 = it * AT_BN;
     if (j0 + AT_BN <= a.tk) {
@@ -173,7 +173,7 @@ __global__ __launch_bounds__(256, OCC) void attention_fwd_kernel(AttnFwdArgs a, 
 
   // Gate factors of tile `it`, written by wave 0 (it issued the gate copy, so it alone can wait for it):
   // exp(R - gate) relative to the tile's last key (<= 1) and relative to the first key of each 16-key group (>= 1).
-  auto gate_factors = [&](int it) {
+  auto gate_factors = [&](int it) __attribute__((always_inline)) {
     float* graw = (float*)(smem + (it % AT_NST) * STAGE + 2 * TILE);
     const int rpos = min(AT_BN - 1, a.tk - 1 - it * AT_BN);
     const float gv = Gg ? graw[l] : 0.f;
@@ -188,7 +188,7 @@ __global__ __launch_bounds__(256, OCC) void attention_fwd_kernel(AttnFwdArgs a, 
   }
   // Make tile `it` visible to the workgroup, start the copy of tile it+2, and (wave 0) prepare the gate factors of
   // tile it+1 while the others already compute.
-  auto sync_step = [&](int it) -> char* {
+  auto sync_step = [&](int it) __attribute__((always_inline)) -> char* {
     char* st = smem + (it % AT_NST) * STAGE;
     if (it + 1 < ntiles) wait_vmcnt<LOADS>(); else wait_vmcnt<0>();
     lds_barrier();
@@ -203,7 +203,7 @@ __global__ __launch_bounds__(256, OCC) void attention_fwd_kernel(AttnFwdArgs a, 
   // One 64-key tile.  Past tiles use one reference gate (the tile's last key), so both gate factors are <= 1.
   // Diagonal tiles use the first key of every 16-key group instead: for every visible pair the row factor is
   // then <= 1 and the key factor spans only 16 steps of decay, so neither leaves the fp32 range.
-  auto tile = [&](int it, const char* st, auto diag_c) {
+  auto tile = [&](int it, const char* st, auto diag_c) __attribute__((always_inline)) {
     constexpr bool DIAG = decltype(diag_c)::value != 0;
     const int j0 = it * AT_BN;
     const float* graw = (const float*)(st + 2 * TILE);

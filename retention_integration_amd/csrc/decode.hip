@@ -131,16 +131,20 @@ __global__ __launch_bounds__(256) void decode_step_kernel(DecodeArgs a) {
 
   // reduce over the FPP feature-row groups of the workgroup, one query row at a time
   float* part = a.part + ((long)pair * a.split + sp) * rows * (DH + 1);
-  for (int r_ = 0; r_ < rows; r_++) {
-    __syncthreads();
+  // (compile-time row index: a run-time index would put the accumulators in scratch memory for the whole kernel)
 #pragma unroll
-    for (int i = 0; i < 8; i++) red[fr][8 * sub + i] = acc[r_][i];
-    if (sub == 0) red[fr][DH] = lq[r_];
-    __syncthreads();
-    if (tid <= DH) {
-      float t = 0.f;
-      for (int k = 0; k < FPP; k++) t += red[k][tid];
-      part[r_ * (DH + 1) + tid] = t;
+  for (int r_ = 0; r_ < DEC_MAXROWS; r_++) {
+    if (r_ < rows) {
+      __syncthreads();
+#pragma unroll
+      for (int i = 0; i < 8; i++) red[fr][8 * sub + i] = acc[r_][i];
+      if (sub == 0) red[fr][DH] = lq[r_];
+      __syncthreads();
+      if (tid <= DH) {
+        float t = 0.f;
+        for (int k = 0; k < FPP; k++) t += red[k][tid];
+        part[r_ * (DH + 1) + tid] = t;
+      }
     }
   }
 }
