@@ -160,12 +160,15 @@ int pr_chunk_gate_scan_bwd(float* dlog_G, const float* dGq, const float* dotk, c
  *   If K_new is not NULL: K_new, V_new [B,h,d], log_decay [B,h] fp32 or NULL (= 0)
  *   -> S_out = exp(log_decay) * S + phi(K_new)^T V_new, s_out = exp(log_decay) * s + phi(K_new), read in the same
  *      pass as the query (which sees the OLD state).  S_out/s_out must not alias S/s.
+ *   attend_new != 0 (needs K_new, tq == 1, Y_attn == NULL): the attention part is that of the new token attending to
+ *      itself -- the recurrent loop that folds every token (switch_over_seq_len = 1) in one call: Y_attn = V_new,
+ *      l_attn = 1 + 1e-6, rowmax = log((scale q.k)^deg), retention/_attention/reference.py:42-69 with one key.
  *   workspace: pr_decode_step_workspace() bytes. */
 size_t pr_decode_step_workspace(int B, int tq, int h, int r, int d);
 int pr_decode_step(const void* Q, const float* gq, const void* S, const float* s, const void* Y_attn,
                    const float* l_attn, const float* rowmax, const void* K_new, const void* V_new,
                    const float* log_decay, void* S_out, float* s_out, void* out, void* workspace, int B, int tq, int h,
-                   int r, int d, float scale_p, int deg, int dtype, void* stream);
+                   int r, int d, float scale_p, int deg, int dtype, int attend_new, void* stream);
 
 #ifdef __cplusplus
 }

@@ -242,8 +242,10 @@ size_t pr_decode_step_workspace(int B, int tq, int h, int r, int d) {
 int pr_decode_step(const void* Q, const float* gq, const void* S, const float* s, const void* Y_attn,
                    const float* l_attn, const float* rowmax, const void* K_new, const void* V_new,
                    const float* log_decay, void* S_out, float* s_out, void* out, void* workspace, int B, int tq, int h,
-                   int r, int d, float scale_p, int deg, int dtype, void* stream) {
+                   int r, int d, float scale_p, int deg, int dtype, int attend_new, void* stream) {
   if (int rc = check_common("decode_step", d, deg, dtype, true)) return rc;
+  if (attend_new && (!K_new || tq != 1 || Y_attn))
+    return fail(PR_ERR_ARG, "decode_step: attend_new needs K_new, V_new, tq == 1 and no separate attention part");
   if (bad_ptr(Q) || bad_ptr(S) || bad_ptr(s) || bad_ptr(out) || bad_ptr(workspace) || bad_opt(Y_attn) ||
       bad_opt(K_new) || bad_opt(V_new) || bad_opt(S_out))
     return fail(PR_ERR_ARG, "decode_step: null or misaligned pointer");
@@ -254,7 +256,8 @@ int pr_decode_step(const void* Q, const float* gq, const void* S, const float* s
   if (B <= 0 || tq <= 0 || h <= 0 || r <= 0) return fail(PR_ERR_ARG, "decode_step: need B,tq,h,r > 0");
   if (tq * r > 8) return fail(PR_ERR_ARG, "decode_step: at most 8 query rows per (batch, kv head) (got %d)", tq * r);
   return finish(pr::decode_step(Q, gq, S, s, Y_attn, l_attn, rowmax, K_new, V_new, log_decay, S_out, s_out, out,
-                                (float*)workspace, B, tq, h, r, d, deg, scale_p, dtype, (hipStream_t)stream),
+                                (float*)workspace, B, tq, h, r, d, deg, scale_p, dtype, attend_new ? 1 : 0,
+                                (hipStream_t)stream),
                 "decode_step");
 }
 

@@ -151,11 +151,16 @@ __global__ __launch_bounds__(256) void decode_step_kernel(DecodeArgs a) {
 
 // out[row, e] = (Y_attn * wa + y * wq) / (l_attn * wa + lq * wq), the merge of the chunked kernel
 // (sympow_nn.hip); without an attention part out = y / lq.
+// With Qn/Kn/Vn the attention part is that of the ONE new token attending to itself (tq = 1): one weight
+// (scale q.k)^deg, so Y_attn = v, l_attn = 1 + 1e-6 and rowmax = log of the weight
+// (ref: retention/_attention/reference.py:42-69 with a single key).
 template <typename T, int DH>
 __global__ __launch_bounds__(64) void decode_merge_kernel(const float* __restrict__ part, const T* __restrict__ Y_attn,
                                                           const float* __restrict__ l_attn,
-                                                          const float* __restrict__ rowmax, T* __restrict__ out, int h,
-                                                          int r, int tq, int split, float scale_p) {
+                                                          const float* __restrict__ rowmax, const T* __restrict__ Qn,
+                                                          const T* __restrict__ Kn, const T* __restrict__ Vn,
+                                                          T* __restrict__ out, int h, int r, int tq, int split,
+                                                          float scale_p, float deg) {
   constexpr int D = 128 * (DH / 16) * (DH / 16 + 1);
   const int pair = blockIdx.x, row = blockIdx.y, rows = tq * r, hq = h * r;
   const int b = pair / h, hh = pair % h, t = row / r, rr = row % r;
@@ -164,7 +169,19 @@ __global__ __launch_bounds__(64) void decode_merge_kernel(const float* __restric
   float lq = 0.f;
   for (int k = 0; k < split; k++) lq += p[(long)k * rows * (DH + 1) + DH];
   float wa = 0.f, wq = 1.f, la = 0.f;
-  if (Y_attn) {
+  const T* ya = Y_attn ? Y_attn + ro * DH : nullptr;
+  if (Kn) {
+    float dot = 0.f;
+    for (int e = threadIdx.x; e < DH; e += 64) dot += (float)Qn[ro * DH + e] * (float)Kn[(long)pair * DH + e];
+    dot = sum_over_rows(sum_in_row(dot));
+    const float scale = __expf(__logf(scale_p) / deg), eps = 1e-7f / scale;
+    const float m = 0.5f * deg * __logf(dot * dot + eps * eps) + __logf(scale_p);
+    const float beta = fmaxf(m, 0.5f * __logf((float)D));
+    la = 1.f + 1e-6f;
+    wa = __expf(m - beta);
+    wq = scale_p * __expf(-beta);
+    ya = Vn + (long)pair * DH;
+  } else if (Y_attn) {
     const float m = rowmax[ro], beta = fmaxf(m, 0.5f * __logf((float)D));
     la = l_attn[ro];
     wa = __expf(m - beta);
@@ -175,7 +192,7 @@ __global__ __launch_bounds__(64) void decode_merge_kernel(const float* __restric
     float y = 0.f;
     for (int k = 0; k < split; k++) y += p[(long)k * rows * (DH + 1) + e];
     float num = y * wq;
-    if (Y_attn) num += (float)Y_attn[ro * DH + e] * wa;
+    if (ya) num += (float)ya[e] * wa;
     out[ro * DH + e] = (T)(num * inv);
   }
 }
@@ -192,26 +209,28 @@ long decode_workspace_floats(int B, int h, int r, int tq, int d) {
 
 template <typename T, int DH>
 static int decode_launch(const DecodeArgs& a0, const void* Y_attn, const float* l_attn, const float* rowmax, void* out,
-                         int B, float scale_p, hipStream_t st) {
+                         int B, float scale_p, int attend_new, hipStream_t st) {
   DecodeArgs a = a0;
   a.split = decode_split(B, a.h);
   hipLaunchKernelGGL((decode_step_kernel<T, DH>), dim3((unsigned)(B * a.h), (unsigned)a.split), dim3(256), 0, st, a);
   hipLaunchKernelGGL((decode_merge_kernel<T, DH>), dim3((unsigned)(B * a.h), (unsigned)(a.tq * a.r)), dim3(64), 0, st,
-                     a.part, (const T*)Y_attn, l_attn, rowmax, (T*)out, a.h, a.r, a.tq, a.split, scale_p);
+                     a.part, (const T*)Y_attn, l_attn, rowmax, attend_new ? (const T*)a.Q : nullptr,
+                     attend_new ? (const T*)a.Knew : nullptr, attend_new ? (const T*)a.Vnew : nullptr, (T*)out, a.h,
+                     a.r, a.tq, a.split, scale_p, (float)a.deg);
   return (int)hipGetLastError();
 }
 
 int decode_step(const void* Q, const float* gq, const void* S, const float* s, const void* Y_attn, const float* l_attn,
                 const float* rowmax, const void* Knew, const void* Vnew, const float* decay, void* Sout, float* sout,
                 void* out, float* workspace, int B, int tq, int h, int r, int d, int deg, float scale_p, int dtype,
-                hipStream_t st) {
+                int attend_new, hipStream_t st) {
   if (tq * r > DEC_MAXROWS) return -3;
   DecodeArgs a{Q, gq, S, s, Knew, Vnew, decay, Sout, sout, workspace, h, r, tq, 1, deg};
 #define PR_DEC(T)                                                                                                      \
   switch (d) {                                                                                                         \
-    case 32: return decode_launch<T, 32>(a, Y_attn, l_attn, rowmax, out, B, scale_p, st);                              \
-    case 64: return decode_launch<T, 64>(a, Y_attn, l_attn, rowmax, out, B, scale_p, st);                              \
-    case 128: return decode_launch<T, 128>(a, Y_attn, l_attn, rowmax, out, B, scale_p, st);                            \
+    case 32: return decode_launch<T, 32>(a, Y_attn, l_attn, rowmax, out, B, scale_p, attend_new, st);                              \
+    case 64: return decode_launch<T, 64>(a, Y_attn, l_attn, rowmax, out, B, scale_p, attend_new, st);                              \
+    case 128: return decode_launch<T, 128>(a, Y_attn, l_attn, rowmax, out, B, scale_p, attend_new, st);                            \
     default: return -2;                                                                                                \
   }
   if (dtype == DT_BF16) { PR_DEC(bf16_t) }

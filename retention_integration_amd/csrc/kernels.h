@@ -106,6 +106,6 @@ long decode_workspace_floats(int B, int h, int r, int tq, int d);
 int decode_step(const void* Q, const float* gq, const void* S, const float* s, const void* Y_attn, const float* l_attn,
                 const float* rowmax, const void* Knew, const void* Vnew, const float* decay, void* Sout, float* sout,
                 void* out, float* workspace, int B, int tq, int h, int r, int d, int deg, float scale_p, int dtype,
-                hipStream_t st);
+                int attend_new, hipStream_t st);
 
 }  // namespace pr

@@ -27,17 +27,21 @@ def make_fused_inference(composed):
         assert initial_state.shape[0] == b, "initial_state must have a batch size of the same as the query"
         scale = 1.0 / d ** 0.5 if scale is None else scale
         tk = K.shape[1] if has_cache else 0
+        fold = switch_over_seq_len is not None and tk >= switch_over_seq_len
+        if fold and tk == 1:   # (then tq == 1 as well)
+            # the recurrent loop (every token folded as it arrives): the new token attends to itself, queries the old
+            # state and is folded, all in one pass over the state
+            g1 = log_G.to(torch.float32)[:, 0].contiguous() if log_G is not None else None
+            Y, new_S, new_s = ops.decode_step(Q.contiguous(), g1, initial_state.contiguous(),
+                                              sum_of_keys.to(torch.float32).contiguous(), None, None, None,
+                                              K[:, 0].contiguous(), V[:, 0].contiguous(), g1, float(scale) ** deg, True)
+            return Y, new_S, new_s.to(sum_of_keys.dtype)
         A = log_G.to(torch.float32).cumsum(1) if (log_G is not None and has_cache) else None
         Ya = la = rm = None
         if tk > 0:
             Ya, la, rm = ops.attention(Q, K, V, A, deg, scale=scale, norm=False)
         a_last = A[:, -1].contiguous() if A is not None else None
-        fold = switch_over_seq_len is not None and tk >= switch_over_seq_len
         S32 = sum_of_keys.to(torch.float32).contiguous()
-        if fold and tk == 1:
-            Y, new_S, new_s = ops.decode_step(Q.contiguous(), a_last, initial_state.contiguous(), S32, Ya, la, rm,
-                                              K[:, 0].contiguous(), V[:, 0].contiguous(), a_last, float(scale) ** deg)
-            return Y, new_S, new_s.to(sum_of_keys.dtype)
         Y, _, _ = ops.decode_step(Q.contiguous(), a_last, initial_state.contiguous(), S32, Ya, la, rm, None, None,
                                   None, float(scale) ** deg)
         if not fold:

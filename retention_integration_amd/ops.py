@@ -367,10 +367,11 @@ def query_state(Q, S, s, Y_attn, l_attn, rowmax, deg, scale, zero_initial_state)
 @torch.library.custom_op("pr::decode_step", mutates_args=(), device_types="cuda")
 def decode_step(Q: Tensor, gq: Optional[Tensor], S: Tensor, s: Tensor, Y_attn: Optional[Tensor],
                 l_attn: Optional[Tensor], rowmax: Optional[Tensor], K_new: Optional[Tensor], V_new: Optional[Tensor],
-                log_decay: Optional[Tensor], scale_p: float) -> Tuple[Tensor, Tensor, Tensor]:
+                log_decay: Optional[Tensor], scale_p: float, attend_new: bool = False) -> Tuple[Tensor, Tensor, Tensor]:
     """Q [b, tq, hq, d] (tq * hq/h <= 8), gq [b, h] fp32 or None, S [b, h, D, d], s [b, h, D] fp32, attention part or
     None, and optionally one new token K_new, V_new [b, h, d] with log_decay [b, h] -> (out [b, tq, hq, d],
-    S_new, s_new); without a new token S_new, s_new are empty tensors."""
+    S_new, s_new); without a new token S_new, s_new are empty tensors.  attend_new: the attention part is the new
+    token attending to itself (tq == 1, no Y_attn)."""
     b, tq, hq, d = Q.shape
     h = S.shape[1]
     out = torch.empty_like(Q)
@@ -384,13 +385,14 @@ def decode_step(Q: Tensor, gq: Optional[Tensor], S: Tensor, s: Tensor, Y_attn: O
                                   _lib.ptr(l_attn), _lib.ptr(rowmax), _lib.ptr(K_new), _lib.ptr(V_new),
                                   _lib.ptr(log_decay), _lib.ptr(S_new) if K_new is not None else None,
                                   _lib.ptr(s_new) if K_new is not None else None, _lib.ptr(out), _lib.ptr(ws),
-                                  b, tq, h, hq // h, d, float(scale_p), 2, _lib.dtype_code(Q.dtype), _lib.stream()),
+                                  b, tq, h, hq // h, d, float(scale_p), 2, _lib.dtype_code(Q.dtype), int(attend_new),
+                                  _lib.stream()),
                "decode_step")
     return out, S_new, s_new
 
 
 @decode_step.register_fake
-def _(Q, gq, S, s, Y_attn, l_attn, rowmax, K_new, V_new, log_decay, scale_p):
+def _(Q, gq, S, s, Y_attn, l_attn, rowmax, K_new, V_new, log_decay, scale_p, attend_new=False):
     if K_new is not None:
         return torch.empty_like(Q), torch.empty_like(S), torch.empty_like(s)
     return torch.empty_like(Q), S.new_empty(0), s.new_empty(0)
