@@ -123,6 +123,10 @@ int pr_query_state_bwd(const void* Q, const void* S, const float* s, const float
                        float* dl_attn, void* workspace, int BN, int n, int c, int h, int r, int d, float scale_p,
                        int deg, int zero_initial_state, int dtype, void* stream);
 
+/* Accumulated gates of the quadratic / inference paths -- log_G.cumsum(1), retention/power_retention_maker.py:129,
+ * 348-349.  log_G, A [B,t,h] fp32, t <= 8192. */
+int pr_gate_cumsum(const float* log_G, float* A, int B, int t, int h, void* stream);
+
 /* Gate arithmetic of the chunked algorithm, forward -- retention/power_retention_maker.py:146-153,163-164,183-186.
  *   log_G [BN,c,h] fp32 (BN = b*n chunks of length c <= 8192), K [BN,c,h,d], Q [BN,c,h*r,d]
  *   -> A [BN,c,h] = cumsum over the chunk, lcs [BN,h] = A[c-1],

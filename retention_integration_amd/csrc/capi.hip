@@ -216,6 +216,13 @@ int pr_query_state_bwd(const void* Q, const void* S, const float* s, const float
 }
 
 
+int pr_gate_cumsum(const float* log_G, float* A, int B, int t, int h, void* stream) {
+  if (!log_G || !A) return fail(PR_ERR_ARG, "gate_cumsum: null pointer");
+  if (B <= 0 || t <= 0 || h <= 0) return fail(PR_ERR_ARG, "gate_cumsum: need B,t,h > 0");
+  if (t > 8192) return fail(PR_ERR_ARG, "gate_cumsum: at most 8192 positions (got %d)", t);
+  return finish(pr::gate_cumsum(log_G, A, B, t, h, (hipStream_t)stream), "gate_cumsum");
+}
+
 int pr_chunk_prep_fwd(const float* log_G, const void* K, const void* Q, float* A, float* lcs, void* Kd, void* Qg, int BN,
                       int c, int h, int r, int d, int deg, int dtype, void* stream) {
   if (int rc = check_common("chunk_prep_fwd", d, deg, dtype, false)) return rc;

@@ -51,7 +51,7 @@ __global__ __launch_bounds__(256) void gate_scan_fwd_kernel(const float* __restr
   __syncthreads();
   block_scan(a, tot, c, false);
   for (int i = tid; i < c; i += 256) A[base + (long)i * h] = a[i];
-  if (tid == 0) lcs[(long)bn * h + hh] = a[c - 1];
+  if (tid == 0 && lcs) lcs[(long)bn * h + hh] = a[c - 1];
 }
 
 // one group of DH/8 lanes per (chunk, position, kv head)
@@ -128,6 +128,13 @@ static int prep_launch(const float* logG, const void* K, const void* Q, float* A
     break;
   switch (d) { PR_CP(32) PR_CP(64) PR_CP(128) default: return -2; }
 #undef PR_CP
+  return (int)hipGetLastError();
+}
+
+int gate_cumsum(const float* logG, float* A, int B, int t, int h, hipStream_t st) {
+  if (t > GLUE_MAX_C) return -5;
+  const size_t smem = (size_t)(t + 256) * sizeof(float);
+  hipLaunchKernelGGL(gate_scan_fwd_kernel, dim3((unsigned)(B * h)), dim3(256), smem, st, logG, A, (float*)nullptr, t, h);
   return (int)hipGetLastError();
 }
 

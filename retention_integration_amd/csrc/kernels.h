@@ -96,6 +96,7 @@ int qs_bwd_prep(const void* O, const void* dO, const float* den, const float* ro
                 void* dY_attn, float* dl_attn, long rows, int d, float scale_p, int dtype, hipStream_t st);
 
 // chunk_glue.hip (return -5: chunk longer than the LDS-resident gate vector allows)
+int gate_cumsum(const float* logG, float* A, int B, int t, int h, hipStream_t st);
 int chunk_prep_fwd(const float* logG, const void* K, const void* Q, float* A, float* lcs, void* Kd, void* Qg, int BN,
                    int c, int h, int r, int d, int deg, int dtype, hipStream_t st);
 int chunk_gate_scan_bwd(float* dA, const float* dGq, const float* dotk, const float* dlcs_a, const float* dlcs_b, int BN,

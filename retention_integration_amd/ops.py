@@ -361,6 +361,20 @@ def query_state(Q, S, s, Y_attn, l_attn, rowmax, deg, scale, zero_initial_state)
     return O
 
 
+@torch.library.custom_op("pr::gate_cumsum", mutates_args=(), device_types="cuda")
+def gate_cumsum(log_G: Tensor) -> Tensor:
+    """log_G [b, t, h] fp32 contiguous, t <= 8192 -> cumulative sum over t (inference only: no autograd)."""
+    b, t, h = log_G.shape
+    A = torch.empty_like(log_G)
+    _lib.check(_lib.load().pr_gate_cumsum(_lib.ptr(log_G), _lib.ptr(A), b, t, h, _lib.stream()), "gate_cumsum")
+    return A
+
+
+@gate_cumsum.register_fake
+def _(log_G):
+    return torch.empty_like(log_G)
+
+
 # ----------------------------------------------------------------------------
 # single-token inference step on the state (no autograd: inference only)
 # ----------------------------------------------------------------------------
