@@ -78,6 +78,8 @@ def run_both(pra, Q, K, V, lg, chunk, dO=None, **kw):
     (torch.float16, 1, 512, 2, 1, 128, 128, False),     # config 5 flavour: fp16, d = 128, ungated
     (torch.bfloat16, 1, 2048, 1, 1, 64, 1024, True),    # headline chunk size
     (torch.bfloat16, 1, 96, 2, 1, 64, None, True),      # quadratic path
+    (torch.bfloat16, 1, 384, 2, 3, 64, 128, True),      # GQA ratio that is not a power of two (irregular tile copies)
+    (torch.float16, 2, 320, 1, 3, 32, 64, True),        # the same with d = 32, fp16, padding
 ])
 def test_power_retention_fwd_bwd(pra, dtype, b, t, h, r, d, chunk, gated):
     std = 0.5 if dtype == torch.float16 else 1.0
@@ -101,6 +103,17 @@ def test_fused_node_equals_operator_composition(pra, gated, r):
         outs.append([Y] + [x.grad for x in xs if x is not None])
     for nm, a, b_ in zip(["Y", "dQ", "dK", "dV", "dlog_G"], *outs):
         check(f"fused vs composed {nm}", a, b_, 4e-3)
+
+
+def test_strong_gates(pra):
+    """log_G around -3 per step: weights across a chunk span e^-300, the reference gates of the kernels must keep
+    every intermediate in range (same bar as the other cases)."""
+    b, t, h, r, d, chunk = 1, 512, 2, 1, 64, 128
+    Q, K, V, _ = make_inputs(b, t, h, r, d, torch.bfloat16, False, seed=5)
+    g = torch.Generator().manual_seed(6)
+    lg = -3.0 + 0.5 * torch.randn(b, t, h, generator=g)
+    dO = torch.randn(b, t, h * r, d, generator=g).to(torch.bfloat16)
+    run_both(pra, Q, K, V, lg.clamp(max=-0.01), chunk, dO)
 
 
 def test_fp32_inputs_are_rejected_loudly(pra):
