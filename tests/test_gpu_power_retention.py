@@ -105,6 +105,37 @@ def test_fused_node_equals_operator_composition(pra, gated, r):
         check(f"fused vs composed {nm}", a, b_, 4e-3)
 
 
+def test_shape_sweep_fused_vs_composed_vs_oracle(pra):
+    """A seeded sweep over shapes the kernels treat differently (row counts that are not multiples of a tile, GQA
+    ratios, head dims, chunk sizes from one tile to several, both dtypes, gated or not): the fused node against the
+    operator composition (tight bar: same arithmetic, different kernels for the glue) and against the oracle."""
+    rng = torch.Generator().manual_seed(1234)
+    pick = lambda xs: xs[int(torch.randint(len(xs), (1,), generator=rng))]  # noqa: E731
+    for case in range(10):
+        dtype = pick([torch.bfloat16, torch.float16])
+        d, r, h, b = pick([32, 64, 128]), pick([1, 2, 3, 4]), pick([1, 2]), pick([1, 2])
+        chunk = pick([32, 64, 128, 256])
+        n = pick([2, 3, 5])
+        t = chunk * n - pick([0, 0, 1, 17])          # ragged lengths are padded up to a chunk multiple
+        gated = pick([True, True, False])
+        print(f"case {case}: {dtype} b={b} t={t} h={h} r={r} d={d} chunk={chunk} gated={gated}", flush=True)
+        Q, K, V, lg = make_inputs(b, t, h, r, d, dtype, gated, seed=100 + case, std=0.5 if dtype == torch.float16 else 1.0)
+        dO = torch.randn(b, t, h * r, d, generator=rng).to(dtype)
+        outs = []
+        for fn in (pra.power_retention, pra.power_retention_composed):
+            xs = [x.to(DEV).requires_grad_(True) if x is not None else None for x in (Q, K, V, lg)]
+            Y = fn(*xs, deg=2, chunk_size=chunk)
+            Y.backward(dO.to(DEV))
+            outs.append([Y] + [x.grad for x in xs if x is not None])
+        for nm, a, b_ in zip(["Y", "dQ", "dK", "dV", "dlog_G"], *outs):
+            check(f"fused vs composed {nm}", a, b_, 5e-3)
+        xo = [x.float().clone().requires_grad_(True) if x is not None else None for x in (Q, K, V, lg)]
+        Yo = oracle.power_retention(*xo, deg=2, chunk_size=chunk)
+        Yo.backward(dO.float())
+        for nm, a, b_ in zip(["Y", "dQ", "dK", "dV", "dlog_G"], outs[0], [Yo] + [x.grad for x in xo if x is not None]):
+            check(f"fused vs oracle {nm}", a, b_, OUT_TOL if nm == "Y" else GRAD_TOL)
+
+
 def test_strong_gates(pra):
     """log_G around -3 per step: weights across a chunk span e^-300, the reference gates of the kernels must keep
     every intermediate in range (same bar as the other cases)."""
