@@ -115,13 +115,15 @@ int pr_query_state_fwd(const void* Q, const void* S, const float* s, const void*
 /* Backward -- formulas of retention/_query_state/triton.py:546-553 (kernels :184-448).
  *   O, den from the forward; dO [BN,c,h*r,d]
  *   -> dQ [BN,c,h*r,d], dS [BN,h,D,d], ds [BN,h,D] fp32, and, when rowmax != NULL,
- *      dY_attn [BN,c,h*r,d], dl_attn [BN,c,h*r] fp32.
+ *      dY_attn [BN,c,h*r,d], dl_attn [BN,c,h*r] fp32.  dY_attn is dO times a per-row factor; a consumer that scales
+ *      on the fly (the dO_scale argument of the attention backward) can ask for that factor instead:
+ *      dY_scale [BN,c,h*r] fp32 (then dY_attn may be NULL).
  *   workspace: pr_query_state_bwd_workspace() bytes (scaled dO and two fp32 row vectors). */
 size_t pr_query_state_bwd_workspace(int BN, int c, int h, int r, int d, int dtype);
 int pr_query_state_bwd(const void* Q, const void* S, const float* s, const float* rowmax, const void* O,
                        const float* den, const void* dO, void* dQ, void* dS, float* ds, void* dY_attn,
-                       float* dl_attn, void* workspace, int BN, int n, int c, int h, int r, int d, float scale_p,
-                       int deg, int zero_initial_state, int dtype, void* stream);
+                       float* dl_attn, float* dY_scale, void* workspace, int BN, int n, int c, int h, int r, int d,
+                       float scale_p, int deg, int zero_initial_state, int dtype, void* stream);
 
 /* Accumulated gates of the quadratic / inference paths -- log_G.cumsum(1), retention/power_retention_maker.py:129,
  * 348-349.  log_G, A [B,t,h] fp32, t <= 8192. */

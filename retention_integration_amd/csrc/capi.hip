@@ -193,13 +193,14 @@ size_t pr_query_state_bwd_workspace(int BN, int c, int h, int r, int d, int dtyp
 
 int pr_query_state_bwd(const void* Q, const void* S, const float* s, const float* rowmax, const void* O,
                        const float* den, const void* dO, void* dQ, void* dS, float* ds, void* dY_attn,
-                       float* dl_attn, void* workspace, int BN, int n, int c, int h, int r, int d, float scale_p,
-                       int deg, int zero_initial_state, int dtype, void* stream) {
+                       float* dl_attn, float* dY_scale, void* workspace, int BN, int n, int c, int h, int r, int d,
+                       float scale_p, int deg, int zero_initial_state, int dtype, void* stream) {
   if (int rc = check_common("query_state_bwd", d, deg, dtype, true)) return rc;
   if (bad_ptr(Q) || bad_ptr(S) || bad_ptr(s) || bad_ptr(O) || bad_ptr(den) || bad_ptr(dO) || bad_ptr(dQ) ||
       bad_ptr(dS) || bad_ptr(ds) || bad_ptr(workspace) || bad_opt(rowmax) || bad_opt(dY_attn) || bad_opt(dl_attn))
     return fail(PR_ERR_ARG, "query_state_bwd: null or misaligned pointer");
-  if (rowmax && (!dY_attn || !dl_attn)) return fail(PR_ERR_ARG, "query_state_bwd: dY_attn and dl_attn are required when rowmax is given");
+  if (rowmax && ((!dY_attn && !dY_scale) || !dl_attn))
+    return fail(PR_ERR_ARG, "query_state_bwd: dl_attn and one of dY_attn, dY_scale are required when rowmax is given");
   if (BN <= 0 || n <= 0 || c <= 0 || h <= 0 || r <= 0 || BN % n != 0)
     return fail(PR_ERR_ARG, "query_state_bwd: need BN,n,c,h,r > 0 and BN a multiple of n");
   const size_t rows = (size_t)BN * c * h * r;
@@ -207,7 +208,8 @@ int pr_query_state_bwd(const void* Q, const void* S, const float* s, const float
   float* cvec = (float*)((char*)workspace + align256(rows * d * 2));
   hipStream_t st = (hipStream_t)stream;
   if (int rc = finish(pr::qs_bwd_prep(O, dO, den, rowmax, dOs, cvec, rowmax ? dY_attn : nullptr,
-                                      rowmax ? dl_attn : nullptr, (long)rows, d, scale_p, dtype, st),
+                                      rowmax ? dl_attn : nullptr, rowmax ? dY_scale : nullptr, (long)rows, d, scale_p,
+                                      dtype, st),
                       "query_state_bwd(prep)"))
     return rc;
   if (int rc = finish(pr::sympow_tn(Q, dOs, cvec, dS, ds, BN, c, h, r, d, 0, dtype, st), "query_state_bwd(dS)")) return rc;

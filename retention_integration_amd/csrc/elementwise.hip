@@ -12,7 +12,8 @@ __global__ __launch_bounds__(256) void qs_bwd_prep_kernel(const T* __restrict__ 
                                                           const float* __restrict__ den,
                                                           const float* __restrict__ rowmax, T* __restrict__ dOs,
                                                           float* __restrict__ cvec, T* __restrict__ dYa,
-                                                          float* __restrict__ dla, long rows, float scale_p) {
+                                                          float* __restrict__ dla, float* __restrict__ dYscale,
+                                                          long rows, float scale_p) {
   typedef typename VecOf<T>::v8 v8;
   constexpr int LPR = DH / 8;  // lanes per row
   const long gid = (long)blockIdx.x * blockDim.x + threadIdx.x;
@@ -48,18 +49,22 @@ __global__ __launch_bounds__(256) void qs_bwd_prep_kernel(const T* __restrict__ 
   if (col == 0) {
     cvec[r] = -wq * f * delta;
     if (dla) dla[r] = -wa * f * delta;
+    // dY_attn = dO * dYscale[row], for consumers that scale on the fly.  The factor is <= 1/l_attn, i.e. <= ~1 unless
+    // every weight of the row underflowed (a zero query, e.g. a padded row, in fp16: l_attn = 1e-6); it is capped so
+    // that weight * factor stays inside the fp16 range there too.
+    if (dYscale) dYscale[r] = fminf(wa * f, 3.0e4f);
   }
 }
 
 template <typename T>
 static int prep_launch(const void* O, const void* dO, const float* den, const float* rowmax, void* dOs, float* cvec,
-                       void* dYa, float* dla, long rows, int d, float scale_p, hipStream_t st) {
+                       void* dYa, float* dla, float* dYscale, long rows, int d, float scale_p, hipStream_t st) {
   const long threads = rows * (d / 8);
   dim3 grid((unsigned)((threads + 255) / 256));
 #define PR_PREP(DD)                                                                                                    \
   case DD:                                                                                                             \
     hipLaunchKernelGGL((qs_bwd_prep_kernel<T, DD>), grid, dim3(256), 0, st, (const T*)O, (const T*)dO, den, rowmax,    \
-                       (T*)dOs, cvec, (T*)dYa, dla, rows, scale_p);                                                    \
+                       (T*)dOs, cvec, (T*)dYa, dla, dYscale, rows, scale_p);                                                    \
     break;
   switch (d) { PR_PREP(32) PR_PREP(64) PR_PREP(128) default: return -2; }
 #undef PR_PREP
@@ -67,9 +72,12 @@ static int prep_launch(const void* O, const void* dO, const float* den, const fl
 }
 
 int qs_bwd_prep(const void* O, const void* dO, const float* den, const float* rowmax, void* dOs, float* cvec,
-                void* dY_attn, float* dl_attn, long rows, int d, float scale_p, int dtype, hipStream_t st) {
-  if (dtype == DT_BF16) return prep_launch<bf16_t>(O, dO, den, rowmax, dOs, cvec, dY_attn, dl_attn, rows, d, scale_p, st);
-  if (dtype == DT_F16) return prep_launch<f16_t>(O, dO, den, rowmax, dOs, cvec, dY_attn, dl_attn, rows, d, scale_p, st);
+                void* dY_attn, float* dl_attn, float* dY_scale, long rows, int d, float scale_p, int dtype,
+                hipStream_t st) {
+  if (dtype == DT_BF16)
+    return prep_launch<bf16_t>(O, dO, den, rowmax, dOs, cvec, dY_attn, dl_attn, dY_scale, rows, d, scale_p, st);
+  if (dtype == DT_F16)
+    return prep_launch<f16_t>(O, dO, den, rowmax, dOs, cvec, dY_attn, dl_attn, dY_scale, rows, d, scale_p, st);
   return -1;
 }
 

@@ -93,7 +93,7 @@ int attention_bwd(const AttnBwdArgs& a, int B, int d, int dtype, hipStream_t st)
 
 // elementwise.hip
 int qs_bwd_prep(const void* O, const void* dO, const float* den, const float* rowmax, void* dOs, float* cvec,
-                void* dY_attn, float* dl_attn, long rows, int d, float scale_p, int dtype, hipStream_t st);
+                void* dY_attn, float* dl_attn, float* dY_scale, long rows, int d, float scale_p, int dtype, hipStream_t st);
 
 // chunk_glue.hip (return -5: chunk longer than the LDS-resident gate vector allows)
 int gate_cumsum(const float* logG, float* A, int B, int t, int h, hipStream_t st);

@@ -105,10 +105,11 @@ def chunked_bwd(Q: Tensor, K: Tensor, V: Tensor, A: Tensor, lcs: Tensor, Kd: Ten
     p = _lib.ptr
     dO = dO.contiguous()
     dQg, dSc, dsc = torch.empty_like(Q), torch.empty_like(Sc), torch.empty_like(sc)
-    dYa, dla = torch.empty_like(Q), torch.empty_like(den)
+    # the attention part's output gradient is dO times a per-row factor: the attention backward applies it on the fly
+    dla, dys = torch.empty_like(den), torch.empty_like(den)
     ws = _empty((lib.pr_query_state_bwd_workspace(BN, c, h, r, d, code),), u8, dev)
     _lib.check(lib.pr_query_state_bwd(p(Qg), p(Sc), p(sc), p(rm), p(O), p(den), p(dO), p(dQg), p(dSc), p(dsc),
-                                      p(dYa), p(dla), p(ws), BN, n, c, h, r, d, scale ** deg, 2, 1, code, st),
+                                      None, p(dla), p(dys), p(ws), BN, n, c, h, r, d, scale ** deg, 2, 1, code, st),
                "query_state_bwd")
     dS, ds = torch.empty_like(Sc), torch.empty_like(sc)
     dlcs = torch.empty_like(lcs)   # gate gradient of both scans
@@ -124,7 +125,7 @@ def chunked_bwd(Q: Tensor, K: Tensor, V: Tensor, A: Tensor, lcs: Tensor, Kd: Ten
     dGq = _empty((BN, c, hq), f32, dev) if gated else None
     dGk = _empty((b, t, h), f32, dev) if gated else None
     dotk = _empty((BN, c, h), f32, dev) if gated else None
-    _lib.check(lib.pr_chunk_attention_bwd(p(Q), p(K), p(V), p(A) if gated else None, p(rm), p(dYa), p(dla), None, p(dQg), p(dKd),
+    _lib.check(lib.pr_chunk_attention_bwd(p(Q), p(K), p(V), p(A) if gated else None, p(rm), p(dO), p(dla), p(dys), p(dQg), p(dKd),
                                           p(dVs), p(dQa), p(dKa), p(dVa), p(dGq), p(dGk), p(dotk), BN, c, h, r, d,
                                           scale, deg, code, st), "chunk_attention_bwd")
     dlg = _empty((0,), f32, dev)

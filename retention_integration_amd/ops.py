@@ -305,7 +305,7 @@ def query_state_bwd(Q: Tensor, S: Tensor, s: Tensor, rowmax: Optional[Tensor], O
     ws = torch.empty((lib.pr_query_state_bwd_workspace(b * n, c, h, r, d, code),), dtype=torch.uint8, device=Q.device)
     _lib.check(lib.pr_query_state_bwd(_lib.ptr(Q), _lib.ptr(S), _lib.ptr(s), _lib.ptr(rowmax), _lib.ptr(O),
                                       _lib.ptr(den), _lib.ptr(dO), _lib.ptr(dQ), _lib.ptr(dS), _lib.ptr(ds),
-                                      _lib.ptr(dYa), _lib.ptr(dla), _lib.ptr(ws), b * n, n, c, h, r, d,
+                                      _lib.ptr(dYa), _lib.ptr(dla), None, _lib.ptr(ws), b * n, n, c, h, r, d,
                                       float(scale_p), 2, int(zero_initial_state), code, _lib.stream()),
                "query_state_bwd")
     if not has_attn:
