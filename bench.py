@@ -118,7 +118,7 @@ def counter_run(pra, Q, K, V, cfg, dev):
 
 
 def decode_bench(pra, dev, steps=512):
-    """BASELINE configs[3]: b=32, h=8, d=64 bf16; prefill of 2048 tokens with switch_over_seq_len=1024, then
+    """The inference configuration of the benchmark contract (configs[3]): b=32, h=8, d=64 bf16; prefill of 2048 tokens with switch_over_seq_len=1024, then
     `steps` single-token steps.  Two loops are timed: the recurrent one (every token is folded into the state,
     switch_over_seq_len=1) and the API-faithful one of the reference's caller (the cache grows, the state is only
     queried; ref: deploy/models/powercoder/modeling_powercoder.py:181-196)."""

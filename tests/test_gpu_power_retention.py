@@ -72,7 +72,7 @@ def run_both(pra, Q, K, V, lg, chunk, dO=None, **kw):
 
 
 @pytest.mark.parametrize("dtype,b,t,h,r,d,chunk,gated", [
-    (torch.bfloat16, 2, 1024, 8, 1, 64, 128, True),     # BASELINE config 1 shape (there in fp32 on the CPU)
+    (torch.bfloat16, 2, 1024, 8, 1, 64, 128, True),     # the benchmark contract's CPU-runnable shape (there in fp32)
     (torch.bfloat16, 1, 512, 2, 2, 64, 128, True),      # GQA
     (torch.bfloat16, 1, 300, 2, 1, 32, 64, True),       # padding (300 -> 320), d = 32
     (torch.float16, 1, 512, 2, 1, 128, 128, False),     # config 5 flavour: fp16, d = 128, ungated
