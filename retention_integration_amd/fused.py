@@ -20,6 +20,24 @@ from . import _lib
 from .ops import expanded_dim
 
 
+# Optional in-step timing of the two kernels a benchmark reports on their own: set to a dict and every call appends a
+# pair of events (recorded on the launch stream around that kernel alone) under "sympow_grad(dK)" and
+# "sympow_tn(update_state)".  None (the default) records nothing.
+KERNEL_TIMERS = None
+
+
+def _timed(name, launch):
+    tm = KERNEL_TIMERS
+    if tm is None:
+        return launch()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    rc = launch()
+    e1.record()
+    tm.setdefault(name, []).append((e0, e1))
+    return rc
+
+
 def _empty(shape, dtype, device):
     return torch.empty(shape, dtype=dtype, device=device)
 
@@ -54,7 +72,8 @@ def chunked_fwd(Q: Tensor, K: Tensor, V: Tensor, log_G: Optional[Tensor], deg: i
         lcs = torch.zeros((BN, h), dtype=f32, device=dev)
 
     S, s = _empty((BN, h, D, d), dt, dev), _empty((BN, h, D), f32, dev)
-    _lib.check(lib.pr_update_state_fwd(p(Kd_), p(V), p(S), p(s), BN, c, h, d, 2, code, st), "update_state_fwd")
+    _lib.check(_timed("sympow_tn(update_state)", lambda: lib.pr_update_state_fwd(
+        p(Kd_), p(V), p(S), p(s), BN, c, h, d, 2, code, st)), "update_state_fwd")
     Sc, sc = torch.empty_like(S), torch.empty_like(s)
     _lib.check(lib.pr_state_scan_fwd(p(S), p(s), p(lcs), p(Sc), p(sc), b, n, n, h, D * d, D, code, st),
                "state_scan_fwd")
@@ -117,8 +136,11 @@ def chunked_bwd(Q: Tensor, K: Tensor, V: Tensor, A: Tensor, lcs: Tensor, Kd: Ten
     _lib.check(lib.pr_state_scan_bwd(p(dSc), p(Sc), p(dsc), p(sc), p(lcs), p(dS), p(ds), p(dlcs), p(ws), b, n, n, h,
                                      D * d, D, code, st), "state_scan_bwd")
     dKd, dVs = torch.empty_like(K), torch.empty_like(V)
-    _lib.check(lib.pr_update_state_bwd(p(Kd), p(V), p(dS), p(ds), p(dKd), p(dVs), BN, c, h, d, 2, code, st),
-               "update_state_bwd")
+    # (two calls: the value gradient and the key gradient are separate kernels, and the latter is timed on its own)
+    _lib.check(lib.pr_update_state_bwd(p(Kd), p(V), p(dS), p(ds), None, p(dVs), BN, c, h, d, 2, code, st),
+               "update_state_bwd(dV)")
+    _lib.check(_timed("sympow_grad(dK)", lambda: lib.pr_update_state_bwd(
+        p(Kd), p(V), p(dS), p(ds), p(dKd), None, BN, c, h, d, 2, code, st)), "update_state_bwd(dK)")
 
     # the attention backward adds the state-path gradients in its epilogue and writes the final dQ, dK, dV
     dQa, dKa, dVa = torch.empty_like(Q), torch.empty_like(K), torch.empty_like(V)
