@@ -165,7 +165,8 @@ int pr_chunk_gate_scan_bwd(float* dlog_G, const float* dGq, const float* dotk, c
  *   -> out [B,tq,h*r,d] = the merged, normalised output.
  *   If K_new is not NULL: K_new, V_new [B,h,d], log_decay [B,h] fp32 or NULL (= 0)
  *   -> S_out = exp(log_decay) * S + phi(K_new)^T V_new, s_out = exp(log_decay) * s + phi(K_new), read in the same
- *      pass as the query (which sees the OLD state).  S_out/s_out must not alias S/s.
+ *      pass as the query (which sees the OLD state).  S_out/s_out may be S/s themselves (in-place update: every
+ *      element is read and written by the same thread) or separate buffers, both or neither.
  *   attend_new != 0 (needs K_new, tq == 1, Y_attn == NULL): the attention part is that of the new token attending to
  *      itself -- the recurrent loop that folds every token (switch_over_seq_len = 1) in one call: Y_attn = V_new,
  *      l_attn = 1 + 1e-6, rowmax = log((scale q.k)^deg), retention/_attention/reference.py:42-69 with one key.

@@ -261,7 +261,8 @@ int pr_decode_step(const void* Q, const float* gq, const void* S, const float* s
   if ((Y_attn != nullptr) != (l_attn != nullptr) || (Y_attn != nullptr) != (rowmax != nullptr))
     return fail(PR_ERR_ARG, "decode_step: Y_attn, l_attn and rowmax must be given together");
   if (K_new && (!V_new || !S_out || !s_out)) return fail(PR_ERR_ARG, "decode_step: V_new, S_out and s_out are required with K_new");
-  if (K_new && (S_out == S || s_out == s)) return fail(PR_ERR_ARG, "decode_step: the updated state must not alias the old one");
+  if (K_new && ((S_out == S) != (s_out == s)))
+    return fail(PR_ERR_ARG, "decode_step: update S and s both in place or both out of place");
   if (B <= 0 || tq <= 0 || h <= 0 || r <= 0) return fail(PR_ERR_ARG, "decode_step: need B,tq,h,r > 0");
   if (tq * r > 8) return fail(PR_ERR_ARG, "decode_step: at most 8 query rows per (batch, kv head) (got %d)", tq * r);
   return finish(pr::decode_step(Q, gq, S, s, Y_attn, l_attn, rowmax, K_new, V_new, log_decay, S_out, s_out, out,

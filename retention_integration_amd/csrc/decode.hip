@@ -11,7 +11,8 @@
 //           retention/_update_state/reference.py:33-52):
 //       S'[f, e] = decay * S[f, e] + m_f phi(k)[f] v[e],   s'[f] = decay * s[f] + m_f phi(k)[f].
 //
-// The query reads the OLD state, so one pass serves both: every workgroup owns a slice of the features of one
+// The query reads the OLD state, so one pass serves both (and the update may be in place: a state element is read and
+// then written by the same thread, the key sum of a feature row by the lanes of one wave before its lane 0 writes it): every workgroup owns a slice of the features of one
 // (batch, kv head), streams its rows of S once (16 bytes per lane, fully coalesced), accumulates the query partials
 // in registers and writes the updated rows.  A second, tiny kernel adds the partials of the slices and merges.
 #include "common.h"

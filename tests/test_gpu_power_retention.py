@@ -303,3 +303,24 @@ def test_fused_decode_step_equals_operator_chain(pra, dtype, d, r, gated):
     Yf, _, _ = pra.power_retention_inference(q, None, None, None, st_f, sk_f, deg=2)
     Yc, _, _ = pra.power_retention_inference_composed(q, None, None, None, st_f, sk_f, deg=2)
     check("state only: fused vs chain", Yf, Yc, OUT_TOL)
+
+
+def test_decode_step_in_place_through_the_c_abi(pra):
+    """pr_decode_step with S_out = S, s_out = s (the serving loop's in-place state) gives the out-of-place results."""
+    from retention_integration_amd import _lib, ops
+    lib, st, p = _lib.load(), _lib.stream(), _lib.ptr
+    b, h, r, d = 3, 2, 2, 64
+    D = pra.expanded_dim(d)
+    g = torch.Generator().manual_seed(21)
+    dt = torch.bfloat16
+    S = (torch.randn(b, h, D, d, generator=g) * 0.3).to(dt).to(DEV)
+    s = torch.rand(b, h, D, generator=g).to(DEV) + 0.5
+    Q = torch.randn(b, 1, h * r, d, generator=g).to(dt).to(DEV)
+    K, V = (torch.randn(b, h, d, generator=g).to(dt).to(DEV) for _ in range(2))
+    lg = torch.nn.functional.logsigmoid(torch.randn(b, h, generator=g)).to(DEV)
+    out, S2, s2 = ops.decode_step(Q, lg, S, s, None, None, None, K, V, lg, 0.125 ** 2, True)
+    Si, si, oi = S.clone(), s.clone(), torch.empty_like(Q)
+    ws = torch.empty(lib.pr_decode_step_workspace(b, 1, h, r, d), dtype=torch.uint8, device=DEV)
+    _lib.check(lib.pr_decode_step(p(Q), p(lg), p(Si), p(si), None, None, None, p(K), p(V), p(lg), p(Si), p(si), p(oi),
+                                  p(ws), b, 1, h, r, d, 0.125 ** 2, 2, _lib.dtype_code(dt), 1, st), "decode_step")
+    assert torch.equal(oi, out) and torch.equal(Si, S2) and torch.equal(si, s2)
