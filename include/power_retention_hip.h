@@ -101,6 +101,29 @@ int pr_state_scan_bwd(const void* dS_out, const void* S_out, const float* ds_out
                       const float* log_G, void* dS, float* ds, float* dlog_G, void* workspace, int B, int n, int n_out,
                       int H, int64_t F, int64_t F2, int dtype, void* stream);
 
+/* Short chunks: update_state followed by the scan that keeps its first n entries
+ * (retention/power_retention_maker.py:156,167-170) as ONE pass that never writes the per-chunk states:
+ *   K, V [B,n*c,h,d] (keys already discounted), log_G [B,n,h] fp32 chunk gate sums or NULL (no decay)
+ *   -> S_out [B*n,h,D,d], s_out [B*n,h,D] fp32 with S_out[b,0] = 0, S_out[b,k+1] = e^{log_G[b,k]} S_out[b,k] + phi(K_k)^T V_k.
+ * A workgroup walks the chunks of a batch element serially, so this pays only when B*h is large and the chunks are
+ * short.  pr_state_chain_supported() returns 0 when the shape is not supported (it needs c*r a multiple of 64, r a
+ * divisor of 64, n >= 2), 1 when it is, 2 when it also has enough independent work to be the faster form
+ * (r = 1 on the key side, the query-head ratio on the query side). */
+int pr_state_chain_supported(int B, int n, int c, int h, int r, int d);
+int pr_update_state_scan_fwd(const void* K, const void* V, const float* log_G, void* S_out, float* s_out, int B, int n,
+                             int c, int h, int d, int deg, int dtype, void* stream);
+
+/* The backward of query_state (below, with zero_initial_state) chained with the backward of that scan: from dO to
+ * dQ, to the gradient of the PER-CHUNK states dS_in [B*n,h,D,d], ds_in [B*n,h,D] (what update_state's backward
+ * consumes) and, when log_G is given, to dlog_G [B,n,h]; formulas retention/_query_state/triton.py:546-553 and
+ * retention/_discumsum/reference.py:3-15 differentiated.  S, s are the scanned states the forward used.
+ *   workspace: pr_query_state_scan_bwd_workspace() bytes. */
+size_t pr_query_state_scan_bwd_workspace(int B, int n, int c, int h, int r, int d, int dtype);
+int pr_query_state_scan_bwd(const void* Q, const void* S, const float* s, const float* rowmax, const void* O,
+                            const float* den, const void* dO, const float* log_G, void* dQ, void* dS_in, float* ds_in,
+                            void* dY_attn, float* dl_attn, float* dY_scale, float* dlog_G, void* workspace, int B,
+                            int n, int c, int h, int r, int d, float scale_p, int deg, int dtype, void* stream);
+
 /* query_state(Q, S, s, Y_attn, l_attn, rowmax, deg, scale, zero_initial_state) --
  * retention/_query_state/reference.py:36-96,166-191, Triton twin retention/_query_state/triton.py:54-169,478-544.
  *   Q [BN,c,h*r,d] (already gated), S [BN,h,D,d], s [BN,h,D] fp32,

@@ -218,6 +218,64 @@ int pr_query_state_bwd(const void* Q, const void* S, const float* s, const float
 }
 
 
+int pr_state_chain_supported(int B, int n, int c, int h, int r, int d) {
+  return pr::sympow_tn_chain_ok(B, n, c, h, r, d);
+}
+
+int pr_update_state_scan_fwd(const void* K, const void* V, const float* log_G, void* S_out, float* s_out, int B, int n,
+                             int c, int h, int d, int deg, int dtype, void* stream) {
+  if (int rc = check_common("update_state_scan_fwd", d, deg, dtype, true)) return rc;
+  if (bad_ptr(K) || bad_ptr(V) || bad_ptr(S_out) || bad_ptr(s_out))
+    return fail(PR_ERR_ARG, "update_state_scan_fwd: null or misaligned pointer");
+  if (B <= 0 || n <= 0 || c <= 0 || h <= 0 || c % 64 != 0)
+    return fail(PR_ERR_ARG, "update_state_scan_fwd: need B,n,h > 0 and c a positive multiple of 64");
+  return finish(pr::sympow_tn_chain(K, V, nullptr, log_G, S_out, s_out, B, n, c, h, 1, d, 1, 0, dtype,
+                                    (hipStream_t)stream), "update_state_scan_fwd");
+}
+
+size_t pr_query_state_scan_bwd_workspace(int B, int n, int c, int h, int r, int d, int dtype) {
+  const long D = 128L * (d / 16) * (d / 16 + 1);
+  return pr_query_state_bwd_workspace(B * n, c, h, r, d, dtype) +
+         align256((size_t)pr::scan_gate_grad_workspace_floats(B, n, h, D * d, D) * sizeof(float));
+}
+
+int pr_query_state_scan_bwd(const void* Q, const void* S, const float* s, const float* rowmax, const void* O,
+                            const float* den, const void* dO, const float* log_G, void* dQ, void* dS_in, float* ds_in,
+                            void* dY_attn, float* dl_attn, float* dY_scale, float* dlog_G, void* workspace, int B,
+                            int n, int c, int h, int r, int d, float scale_p, int deg, int dtype, void* stream) {
+  if (int rc = check_common("query_state_scan_bwd", d, deg, dtype, true)) return rc;
+  if (bad_ptr(Q) || bad_ptr(S) || bad_ptr(s) || bad_ptr(O) || bad_ptr(den) || bad_ptr(dO) || bad_ptr(dQ) ||
+      bad_ptr(dS_in) || bad_ptr(ds_in) || bad_ptr(workspace) || bad_opt(rowmax) || bad_opt(dY_attn) || bad_opt(dl_attn))
+    return fail(PR_ERR_ARG, "query_state_scan_bwd: null or misaligned pointer");
+  if (rowmax && ((!dY_attn && !dY_scale) || !dl_attn))
+    return fail(PR_ERR_ARG, "query_state_scan_bwd: dl_attn and one of dY_attn, dY_scale are required when rowmax is given");
+  if ((log_G != nullptr) != (dlog_G != nullptr))
+    return fail(PR_ERR_ARG, "query_state_scan_bwd: log_G and dlog_G must be given together");
+  if (B <= 0 || n <= 0 || c <= 0 || h <= 0 || r <= 0 || 64 % r != 0 || ((long)c * r) % 64 != 0)
+    return fail(PR_ERR_ARG, "query_state_scan_bwd: need B,n,c,h > 0, r a divisor of 64 and c*r a multiple of 64");
+  const int BN = B * n;
+  const size_t rows = (size_t)BN * c * h * r;
+  const long D = 128L * (d / 16) * (d / 16 + 1);
+  void* dOs = workspace;
+  float* cvec = (float*)((char*)workspace + align256(rows * d * 2));
+  float* part = (float*)((char*)workspace + pr_query_state_bwd_workspace(BN, c, h, r, d, dtype));
+  hipStream_t st = (hipStream_t)stream;
+  if (int rc = finish(pr::qs_bwd_prep(O, dO, den, rowmax, dOs, cvec, rowmax ? dY_attn : nullptr,
+                                      rowmax ? dl_attn : nullptr, rowmax ? dY_scale : nullptr, (long)rows, d, scale_p,
+                                      dtype, st),
+                      "query_state_scan_bwd(prep)"))
+    return rc;
+  if (int rc = finish(pr::sympow_tn_chain(Q, dOs, cvec, log_G, dS_in, ds_in, B, n, c, h, r, d, 0, 1, dtype, st),
+                      "query_state_scan_bwd(dS)"))
+    return rc;
+  if (log_G)
+    if (int rc = finish(pr::scan_gate_grad(S, dS_in, s, ds_in, log_G, dlog_G, part, B, n, h, D * d, D, dtype, st),
+                        "query_state_scan_bwd(dlog_G)"))
+      return rc;
+  pr::GradArgs g{Q, dOs, cvec, S, s, dQ, c, h, r, n, 1};
+  return finish(pr::sympow_grad(g, BN, d, 0, dtype, st), "query_state_scan_bwd(dQ)");
+}
+
 int pr_gate_cumsum(const float* log_G, float* A, int B, int t, int h, void* stream) {
   if (!log_G || !A) return fail(PR_ERR_ARG, "gate_cumsum: null pointer");
   if (B <= 0 || t <= 0 || h <= 0) return fail(PR_ERR_ARG, "gate_cumsum: need B,t,h > 0");

@@ -298,6 +298,67 @@ int discumsum_pair_bwd(const void* dY, const void* Y, const float* dY2, const fl
   return -1;
 }
 
+// Gate gradient of a scan whose backward pass has already been formed elsewhere: given the scan Y and
+// R[k] = dL/dX[k] (both [B, n, H, F], and the fp32 pair Y2, R2 [B, n, H, F2]),
+//   dlog_G[k] = exp(log_G[k]) * (sum_F Y[k] R[k] + sum_F2 Y2[k] R2[k]).
+// grid (blocks, B*H, n); a thread of the first nblk blocks owns four 16-byte vectors of the 16-bit tensors, a thread
+// of the others four floats.  Partials as in discumsum_bwd_body.
+template <typename T>
+__global__ __launch_bounds__(256) void scan_gate_grad_kernel(const T* __restrict__ Y, const T* __restrict__ R,
+                                                             const float* __restrict__ Y2, const float* __restrict__ R2,
+                                                             const float* __restrict__ logG, float* __restrict__ partial,
+                                                             int n, int H, long F, long F2, int nblk, int waves_per_bh) {
+  typedef typename Pack16<T, 16>::type vec;
+  const int bh = blockIdx.y, k = blockIdx.z, b = bh / H, hh = bh % H;
+  const long row = ((long)b * n + k) * H + hh;
+  float dot = 0.f;
+  if ((int)blockIdx.x < nblk) {
+    const vec* y = (const vec*)(Y + row * F);
+    const vec* rr = (const vec*)(R + row * F);
+    const long nv = F / 8, i0 = (long)blockIdx.x * 1024 + threadIdx.x;
+    vec a[4], c4[4];
+#pragma unroll
+    for (int u = 0; u < 4; u++)
+      if (i0 + 256 * u < nv) {
+        a[u] = y[i0 + 256 * u];
+        c4[u] = rr[i0 + 256 * u];
+      }
+#pragma unroll
+    for (int u = 0; u < 4; u++)
+      if (i0 + 256 * u < nv)
+#pragma unroll
+        for (int i = 0; i < 8; i++) dot += to_f32(a[u][i]) * to_f32(c4[u][i]);
+  } else {
+    const long i0 = (long)(blockIdx.x - nblk) * 1024 + threadIdx.x;
+#pragma unroll
+    for (int u = 0; u < 4; u++)
+      if (i0 + 256 * u < F2) dot += Y2[row * F2 + i0 + 256 * u] * R2[row * F2 + i0 + 256 * u];
+  }
+  dot = wave_sum_dpp(dot);
+  const int wave = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (lane_id() == 0) partial[((long)bh * n + k) * waves_per_bh + wave] = dot * __expf(logG[row]);
+}
+long scan_gate_grad_workspace_floats(int B, int n, int H, long F, long F2) {
+  return (long)B * H * n * ((F / 8 + 1023) / 1024 + (F2 + 1023) / 1024) * 4;
+}
+int scan_gate_grad(const void* Y, const void* R, const float* Y2, const float* R2, const float* logG, float* dlogG,
+                   float* partial, int B, int n, int H, long F, long F2, int dtype, hipStream_t st) {
+  const int nblk = (int)((F / 8 + 1023) / 1024), nblk2 = (int)((F2 + 1023) / 1024);
+  const int waves = (nblk + nblk2) * 4, tot = B * H * n;
+  dim3 grid((unsigned)(nblk + nblk2), (unsigned)(B * H), (unsigned)n);
+  if (dtype == DT_BF16)
+    hipLaunchKernelGGL(scan_gate_grad_kernel<bf16_t>, grid, dim3(256), 0, st, (const bf16_t*)Y, (const bf16_t*)R, Y2, R2,
+                       logG, partial, n, H, F, F2, nblk, waves);
+  else if (dtype == DT_F16)
+    hipLaunchKernelGGL(scan_gate_grad_kernel<f16_t>, grid, dim3(256), 0, st, (const f16_t*)Y, (const f16_t*)R, Y2, R2,
+                       logG, partial, n, H, F, F2, nblk, waves);
+  else
+    return -1;
+  hipLaunchKernelGGL(discumsum_reduce_kernel, dim3((tot * 64 + 255) / 256), dim3(256), 0, st, partial, dlogG, n, H,
+                     waves, B * H);
+  return (int)hipGetLastError();
+}
+
 int discumsum_fwd(const void* X, const float* logG, void* Y, int B, int n, int n_out, int H, long F, int dtype,
                   hipStream_t st) {
   switch (dtype) {

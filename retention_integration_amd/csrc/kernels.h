@@ -17,10 +17,20 @@ int discumsum_pair_bwd(const void* dY, const void* Y, const float* dY2, const fl
                        float* dX2, float* dlogG, float* partial, int B, int n, int n_out, int H, long F, long F2,
                        int dtype, hipStream_t st);
 long discumsum_bwd_workspace_floats(int B, int n, int H, long F, int dtype);
+// gate gradient of the pair of scans from the scans Y, Y2 and the already formed input gradients R, R2 ([B,n,H,*])
+long scan_gate_grad_workspace_floats(int B, int n, int H, long F, long F2);
+int scan_gate_grad(const void* Y, const void* R, const float* Y2, const float* R2, const float* logG, float* dlogG,
+                   float* partial, int B, int n, int H, long F, long F2, int dtype, hipStream_t st);
 
 // sympow_tn.hip: A [BN,c,h*r,d], Bm [BN,c,h*r,d], w [BN,c,h*r] or null -> S [BN,h,D,d], s [BN,h,D]
 int sympow_tn(const void* A, const void* Bm, const float* w, void* S, float* s, int BN, int c, int h, int r, int d,
               int use_mult, int dtype, hipStream_t st);
+// The same contraction chained with the gated scan over the n chunks of a batch element (A, Bm [B,n*c,h*r,d],
+// lcs [B,n,h] or null): entry k of S, s [B*n,h,D,*] is the scan's k-th value (forward) or the scan's input gradient
+// (reverse).  sympow_tn_chain_ok: 0 = shape not supported, 1 = supported, 2 = and enough independent work to pay.
+int sympow_tn_chain_ok(int B, int n, int c, int h, int r, int d);
+int sympow_tn_chain(const void* A, const void* Bm, const float* w, const float* lcs, void* S, float* s, int B, int n,
+                    int c, int h, int r, int d, int use_mult, int reverse, int dtype, hipStream_t st);
 
 // sympow_nn.hip
 enum { NN_EPI_PLAIN = 0, NN_EPI_MERGE = 1 };

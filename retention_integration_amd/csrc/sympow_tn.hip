@@ -291,6 +291,301 @@ __global__ __launch_bounds__(256, 2) void sympow_tn_kernel(const T* __restrict__
 #undef PR_TN_CASE
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// Chained form (short chunks).  The per-chunk sums S_k of the kernel above are only ever consumed through the gated
+// scan over the chunk axis (discumsum.hip).  When a batch element has many short chunks the scan's traffic -- S
+// written, read back, and the scanned tensor written -- is what the pair of kernels costs.  Here one workgroup
+// walks the chunks of a batch element in order, keeps the running sum in its accumulators and writes only the
+// scanned tensor:
+//   forward:  Y[0] = 0,    Y[k+1] = e^{g_k} Y[k] + S_k        (the first n entries of the scan)
+//   reverse:  R[n-1] = 0,  R[k-1] = e^{g_k} R[k] + S_k        (the scan's backward applied to S_k = per-chunk gradient)
+// Rows of all chunks form one stream of stages through the ring; at each chunk boundary the accumulators are
+// written (through a small per-wave LDS buffer, so that a wave stores whole contiguous kilobytes) and decayed.
+// What bounds it: the scanned tensor is written once, and while a compute unit's burst of stores drains, the copies
+// queued behind it wait -- measured, the stores add their drain time to the contraction's instead of hiding under it.
+template <typename T, int DK, int DV, int XPW, int NW, int KT, int PART, bool HAS_W, bool REVERSE>
+__device__ __forceinline__ void tn_chain_body(const T* __restrict__ A, const T* __restrict__ Bm,
+                                              const float* __restrict__ w, const float* __restrict__ lcs,
+                                              T* __restrict__ S, float* __restrict__ s, int n, int c, int hA, int r,
+                                              int hh, int b, int h, int y, int xb, bool active, bool use_mult,
+                                              char* smem) {
+  typedef typename VecOf<T>::v8 v8;
+  typedef __attribute__((address_space(3))) unsigned short lds_u16;
+  typedef __attribute__((address_space(3))) u32x4 lds_u32x4;
+  constexpr int NT = DV / 16, CA = DK / 8, CB = DV / 8;
+  constexpr int A_BYTES = KT * DK * 2, B_BYTES = KT * DV * 2, W_BYTES = KT * 4;
+  constexpr int STAGE = A_BYTES + B_BYTES + W_BYTES;
+  constexpr int LA = KT * CA / (64 * NW), LB = KT * CB / (64 * NW);   // copies per thread per stage
+  constexpr int LOADS = LA + LB;
+  constexpr int NSTORE = XPW * (DV / 32);   // 16-byte stores of a boundary per wave (the key sums add one more)
+  static_assert(16 * DV * 2 / 1024 == DV / 32, "one kilobyte per store instruction");
+  static_assert(LOADS + 2 * NSTORE <= 63, "the wait counter has six bits");
+  constexpr int D = 128 * (DK / 16) * (DK / 16 + 1);
+  static_assert(DK == DV, "the A and B tiles share the copy offsets");
+  const int tid = threadIdx.x, l = tid & 63, g = l >> 4, sl = l & 15;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const char* a_base = (const char*)(A + (long)b * n * c * hA * DK);
+  const char* b_base = (const char*)(Bm + (long)b * n * c * hA * DV);
+  const float* w_base = w + (long)b * n * c * hA;
+  // every stage is KT whole folded rows = KT / r time steps (checked by the host)
+  auto row_index = [&](int row) -> long {
+    const int t = row / r, rr = row - t * r;
+    return (long)t * hA + hh * r + rr;
+  };
+  uint32_t voffA[LA], voffW = 0;
+#pragma unroll
+  for (int ii = 0; ii < LA; ii++) {
+    const int pos = (ii * NW + wave) * 64 + l, row = pos / CA;
+    voffA[ii] = (uint32_t)(row_index(row) * (DK * 2) + 16 * ((pos % CA) ^ swz<CA>(row)));
+  }
+  if (HAS_W) voffW = (uint32_t)(row_index(l % KT) * 4);
+  const long stage_rows = (long)(KT / r) * hA;
+  const uint32_t smem_a = lds_addr(smem);
+  auto issue = [&](int slot, int stage) {
+    const uint32_t sa = smem_a + slot * STAGE + wave * 1024;
+    const char* ab = a_base + stage * stage_rows * (DK * 2);
+    const char* bb = b_base + stage * stage_rows * (DV * 2);
+#pragma unroll
+    for (int ii = 0; ii < LA; ii++) async_copy16_sv(ab, voffA[ii], sa + ii * (NW * 1024));
+#pragma unroll
+    for (int ii = 0; ii < LB; ii++) async_copy16_sv(bb, voffA[ii], sa + A_BYTES + ii * (NW * 1024));
+    if (HAS_W && wave == 0 && l < KT) async_copy4_sv(w_base + stage * stage_rows, voffW, smem_a + slot * STAGE + A_BYTES + B_BYTES);
+  };
+
+  f32x4 acc[XPW][NT];
+#pragma unroll
+  for (int i = 0; i < XPW; i++)
+#pragma unroll
+    for (int j = 0; j < NT; j++) acc[i][j] = (f32x4){0, 0, 0, 0};
+  f32x4 sacc = {0, 0, 0, 0};
+
+  const float mul = (use_mult && xb < y) ? 2.f : 1.f;
+  const int fbase = 128 * y * (y + 1) + 256 * xb;
+  // per-wave staging buffer behind the ring: the 16 feature rows of one x, row-major with padded rows, so that the
+  // tile leaves as whole contiguous kilobytes (the rows of one x are adjacent in S)
+  constexpr int TP = DV * 2 + 16;
+  const uint32_t tb = smem_a + TN_NST * STAGE + wave * (16 * TP);
+  const uint32_t tb_w = tb + 4 * g * TP + sl * 2;   // + 32*nt (+ v*TP): rows 4g+v of column 16nt+sl
+  auto write_out = [&](int k) {
+    if (!active) return;
+    const long so = ((long)(b * n + k) * h + hh) * D + fbase;
+    static_for<XPW>([&](auto xi) {
+      constexpr int X = PART * XPW + decltype(xi)::value;
+#pragma unroll
+      for (int nt = 0; nt < NT; nt++) {
+        float o[4];
+#pragma unroll
+        for (int v = 0; v < 4; v++) o[v] = acc[xi.value][nt][v] * mul;
+        const u32x2 pk = __builtin_bit_cast(u32x2, pack4<T>(o));
+        *(lds_u16*)(tb_w + 32 * nt) = (unsigned short)pk[0];
+        *(lds_u16*)(tb_w + 32 * nt + TP) = (unsigned short)(pk[0] >> 16);
+        *(lds_u16*)(tb_w + 32 * nt + 2 * TP) = (unsigned short)pk[1];
+        *(lds_u16*)(tb_w + 32 * nt + 3 * TP) = (unsigned short)(pk[1] >> 16);
+      }
+      asm volatile("" ::: "memory");   // (LDS operations of one wave execute in order)
+      char* dst = (char*)(S + (so + 16 * X) * DV);
+#pragma unroll
+      for (int j = 0; j < 16 * DV * 2 / 1024; j++) {
+        const int q = j * 1024 + l * 16;
+        const u32x4 val = *(const lds_u32x4*)(tb + (q / (DV * 2)) * TP + q % (DV * 2));
+        *(u32x4*)(dst + q) = val;
+      }
+      asm volatile("" ::: "memory");   // the buffer is rewritten for the next x
+    });
+    if (sl >= PART * XPW && sl < (PART + 1) * XPW) *(f32x4*)(s + so + 16 * sl + 4 * g) = sacc * mul;
+  };
+  auto decay = [&](int k) {
+    if (lcs == nullptr) return;
+    const float gk = __expf(lcs[((long)b * n + k) * h + hh]);
+#pragma unroll
+    for (int i = 0; i < XPW; i++)
+#pragma unroll
+      for (int j = 0; j < NT; j++) acc[i][j] *= gk;
+    sacc *= gk;
+  };
+
+  struct Frags {
+    v8 kfy, kfx, vf[NT];
+  };
+  auto compute = [&](const Frags& F, f32x4 w0, f32x4 w1) {
+    float rowf[8], srcf[8];
+    unpack8(F.kfy, rowf);
+    unpack8(F.kfx, srcf);
+    if (HAS_W) {
+      float sc[8];
+#pragma unroll
+      for (int q = 0; q < 4; q++) {
+        sc[q] = srcf[q] * w0[q];
+        sc[4 + q] = srcf[4 + q] * w1[q];
+      }
+      sacc = mfma16(F.kfy, pack8<T>(sc), sacc);
+    } else {
+      sacc = mfma16(F.kfy, F.kfx, sacc);
+    }
+    dpp_fence();
+    static_for<XPW>([&](auto xi) {
+      v8 a = PhiTile<T, PART * XPW + xi.value>::make(F.kfy, F.kfx, rowf, srcf);
+#pragma unroll
+      for (int nt = 0; nt < NT; nt++) acc[xi.value][nt] = mfma16(a, F.vf[nt], acc[xi.value][nt]);
+    });
+  };
+
+  // Step st of the walk: chunk ordinal st / spc (chunk index n-1-ordinal when walking backwards).  The last chunk of
+  // the walk contributes to no output and is not read.
+  const int spc = (c * r) / KT, steps = (n - 1) * spc;
+  int ik = 0, iw = 0;   // chunk ordinal and stage within the chunk of the next stage to copy
+  auto issue_next = [&](int st) {
+    issue(st % TN_NST, (REVERSE ? n - 1 - ik : ik) * spc + iw);
+    if (++iw == spc) {
+      iw = 0;
+      ik++;
+    }
+  };
+  if (steps > 0) issue_next(0);
+  if (steps > 1) issue_next(1);
+  int kk = 0, wi = 0;
+  int b1 = 0, b2 = 0;   // whether the previous step / the one before wrote a boundary (this wave's stores)
+  Frags F;
+  for (int step = 0; step < steps; step++) {
+    const char* st = smem + (step % TN_NST) * STAGE;
+    // Copies and stores of a wave complete in the order issued and share one counter.  Younger than this stage's
+    // copies are: the next stage's copies, and the stores of a boundary written in one of the last two steps (at
+    // least NSTORE each) -- the boundary's stores are never waited for.
+    const int nb = b1 + b2;
+    if (step + 1 < steps) {
+      if (nb == 0) wait_vmcnt<LOADS>(); else if (nb == 1) wait_vmcnt<LOADS + NSTORE>(); else wait_vmcnt<LOADS + 2 * NSTORE>();
+    } else {
+      if (nb == 0) wait_vmcnt<0>(); else if (nb == 1) wait_vmcnt<NSTORE>(); else wait_vmcnt<2 * NSTORE>();
+    }
+    lds_barrier();
+    if (step + 2 < steps) issue_next(step + 2);
+    b2 = b1;
+    b1 = 0;
+    if (wi == 0) {
+      const int k = REVERSE ? n - 1 - kk : kk;
+      write_out(k);
+      decay(k);
+      b1 = active ? 1 : 0;
+    }
+#pragma unroll 1
+    for (int ks = 0; ks < KT / 32; ks++) {
+      F.kfy = sw_frag_tr<T, CA>(st, 32 * ks, 16 * y);
+      F.kfx = (xb == y) ? F.kfy : sw_frag_tr<T, CA>(st, 32 * ks, 16 * xb);
+#pragma unroll
+      for (int nt = 0; nt < NT; nt++) F.vf[nt] = sw_frag_tr<T, CB>(st + A_BYTES, 32 * ks, 16 * nt);
+      f32x4 w0 = {0, 0, 0, 0}, w1 = {0, 0, 0, 0};
+      if (HAS_W) {
+        const float* wp = (const float*)(st + A_BYTES + B_BYTES) + 32 * ks + 8 * g;
+        w0 = *(const f32x4*)wp;
+        w1 = *(const f32x4*)(wp + 4);
+      }
+      if (active) compute(F, w0, w1);
+    }
+    if (++wi == spc) {
+      wi = 0;
+      kk++;
+    }
+  }
+  write_out(REVERSE ? 0 : n - 1);
+}
+
+template <typename T, int DK, int DV, int XPW, int NW, int KT, bool HAS_W, bool REVERSE>
+__global__ __launch_bounds__(64 * NW, 2) void sympow_tn_chain_kernel(
+    const T* __restrict__ A, const T* __restrict__ Bm, const float* __restrict__ w, const float* __restrict__ lcs,
+    T* __restrict__ S, float* __restrict__ s, int n, int c, int hA, int r, int h, int use_mult) {
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  constexpr int PARTS = 16 / XPW;
+  constexpr int NB = (DK / 16) * (DK / 16 + 1) / 2;
+  // Workgroups are handed to the 8 XCDs (each with its own L2) round-robin by linear id.  All workgroups of a
+  // (batch, head) read the same rows, so ids are permuted to put them on one XCD: XCD x takes the x-th eighth.
+  int bx = blockIdx.x, by = blockIdx.y;
+  const int total = gridDim.x * gridDim.y;
+  if (total % 8 == 0) {
+    const int lin = by * gridDim.x + bx, v = (lin % 8) * (total / 8) + lin / 8;
+    by = v / gridDim.x;
+    bx = v - by * gridDim.x;
+  }
+  const int task = bx * NW + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const bool active = task < NB * PARTS;
+  const int t2 = active ? task : 0;
+  const int part = t2 % PARTS;
+  int y, xb;
+  block_to_yx(t2 / PARTS, y, xb);
+  const int b = by / h, hh = by % h;
+#define PR_TN_CASE(P)                                                                                                  \
+  case P:                                                                                                              \
+    if (P < PARTS)                                                                                                     \
+      tn_chain_body<T, DK, DV, XPW, NW, KT, (P < PARTS ? P : 0), HAS_W, REVERSE>(A, Bm, w, lcs, S, s, n, c, hA, r, hh, \
+                                                                                 b, h, y, xb, active, use_mult != 0,   \
+                                                                                 smem);                                \
+    break;
+  switch (part) {
+    PR_TN_CASE(0)
+    PR_TN_CASE(1)
+    PR_TN_CASE(2)
+    PR_TN_CASE(3)
+  }
+#undef PR_TN_CASE
+}
+
+constexpr int chain_stage_rows(int d) { return d <= 64 ? 64 : 32; }
+
+template <typename T, int DK, int DV>
+static int tn_chain_launch(const void* A, const void* Bm, const float* w, const float* lcs, void* S, float* s, int B,
+                           int n, int c, int h, int r, int use_mult, int reverse, hipStream_t st) {
+  constexpr int XPW = DV <= 64 ? 8 : 4;
+  constexpr int NB = (DK / 16) * (DK / 16 + 1) / 2;
+  constexpr int TASKS = NB * (16 / XPW);
+  constexpr int NW = 4;                         // waves that share a stage of rows
+  constexpr int KT = chain_stage_rows(DV);      // rows per stage: two workgroups per compute unit must fit
+  constexpr size_t smem = TN_NST * (KT * DK * 2 + KT * DV * 2 + KT * 4) + NW * 16 * (DV * 2 + 16);
+  dim3 grid((TASKS + NW - 1) / NW, (unsigned)(B * h));
+#define PR_TN_CHAIN(W, R)                                                                                              \
+  {                                                                                                                    \
+    auto kern = sympow_tn_chain_kernel<T, DK, DV, XPW, NW, KT, W, R>;                                                          \
+    allow_big_lds((const void*)kern, smem);                                                                            \
+    hipLaunchKernelGGL(kern, grid, dim3(64 * NW), smem, st, (const T*)A, (const T*)Bm, w, lcs, (T*)S, s, n, c, h * r, \
+                       r, h, use_mult);                                                                                \
+  }
+  if (w) {
+    if (reverse) PR_TN_CHAIN(true, true) else PR_TN_CHAIN(true, false)
+  } else {
+    if (reverse) PR_TN_CHAIN(false, true) else PR_TN_CHAIN(false, false)
+  }
+#undef PR_TN_CHAIN
+  return (int)hipGetLastError();
+}
+
+// 0: the chained form does not apply (it needs whole stages per chunk); 1: it applies; 2: it applies and there are
+// enough workgroups to fill the chip although the chunk axis is walked serially.
+int sympow_tn_chain_ok(int B, int n, int c, int h, int r, int d) {
+  if (d != 32 && d != 64 && d != 128) return 0;
+  const int kt = chain_stage_rows(d);
+  if (n < 2 || r < 1 || kt % r != 0 || ((long)c * r) % kt != 0) return 0;
+  const int xpw = d <= 64 ? 8 : 4;
+  const long wgs = (long)B * h * (((d / 16) * (d / 16 + 1) / 2 * (16 / xpw) + 3) / 4);
+  return wgs >= 512 ? 2 : 1;
+}
+
+// A: [B, n*c, h*r, d], Bm the same, w: [B, n*c, h*r] or null, lcs: [B, n, h] or null (no decay)
+// -> S: [B*n, h, D, d], s: [B*n, h, D], entry k of a batch element being the scan value described above
+int sympow_tn_chain(const void* A, const void* Bm, const float* w, const float* lcs, void* S, float* s, int B, int n,
+                    int c, int h, int r, int d, int use_mult, int reverse, int dtype, hipStream_t st) {
+  if (d != 32 && d != 64 && d != 128) return -2;
+  if (n < 1 || r < 1 || chain_stage_rows(d) % r != 0 || ((long)c * r) % chain_stage_rows(d) != 0) return -3;
+#define PR_TN_DISPATCH(T)                                                                                              \
+  switch (d) {                                                                                                         \
+    case 32: return tn_chain_launch<T, 32, 32>(A, Bm, w, lcs, S, s, B, n, c, h, r, use_mult, reverse, st);             \
+    case 64: return tn_chain_launch<T, 64, 64>(A, Bm, w, lcs, S, s, B, n, c, h, r, use_mult, reverse, st);             \
+    case 128: return tn_chain_launch<T, 128, 128>(A, Bm, w, lcs, S, s, B, n, c, h, r, use_mult, reverse, st);          \
+    default: return -2;                                                                                                \
+  }
+  if (dtype == DT_BF16) { PR_TN_DISPATCH(bf16_t) }
+  if (dtype == DT_F16) { PR_TN_DISPATCH(f16_t) }
+#undef PR_TN_DISPATCH
+  return -1;
+}
+
 template <typename T, int DK, int DV>
 static int tn_launch(const void* A, const void* Bm, const float* w, void* S, float* s, int BN, int c, int h, int r,
                      int use_mult, hipStream_t st) {

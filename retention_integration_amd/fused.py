@@ -38,6 +38,17 @@ def _timed(name, launch):
     return rc
 
 
+# The state kernels chained with the scan over the chunk axis (short chunks, many batch elements x heads).
+# None: where the library says it is the faster form; True: wherever the shape allows it; False: never.
+CHAIN = None
+
+
+def _chained(lib, b, n, c, h, r, d):
+    if CHAIN is False:
+        return False
+    return lib.pr_state_chain_supported(b, n, c, h, r, d) >= (1 if CHAIN else 2)
+
+
 def _empty(shape, dtype, device):
     return torch.empty(shape, dtype=dtype, device=device)
 
@@ -71,13 +82,18 @@ def chunked_fwd(Q: Tensor, K: Tensor, V: Tensor, log_G: Optional[Tensor], deg: i
         Kd_, Qg_ = K, Q
         lcs = torch.zeros((BN, h), dtype=f32, device=dev)
 
-    S, s = _empty((BN, h, D, d), dt, dev), _empty((BN, h, D), f32, dev)
-    _lib.check(_timed("sympow_tn(update_state)", lambda: lib.pr_update_state_fwd(
-        p(Kd_), p(V), p(S), p(s), BN, c, h, d, 2, code, st)), "update_state_fwd")
-    Sc, sc = torch.empty_like(S), torch.empty_like(s)
-    _lib.check(lib.pr_state_scan_fwd(p(S), p(s), p(lcs), p(Sc), p(sc), b, n, n, h, D * d, D, code, st),
-               "state_scan_fwd")
-    del S, s
+    Sc, sc = _empty((BN, h, D, d), dt, dev), _empty((BN, h, D), f32, dev)
+    if _chained(lib, b, n, c, h, 1, d):
+        # short chunks: the chunk states are scanned as they are formed and never written on their own
+        _lib.check(lib.pr_update_state_scan_fwd(p(Kd_), p(V), p(lcs) if gated else None, p(Sc), p(sc), b, n, c, h, d,
+                                                2, code, st), "update_state_scan_fwd")
+    else:
+        S, s = torch.empty_like(Sc), torch.empty_like(sc)
+        _lib.check(_timed("sympow_tn(update_state)", lambda: lib.pr_update_state_fwd(
+            p(Kd_), p(V), p(S), p(s), BN, c, h, d, 2, code, st)), "update_state_fwd")
+        _lib.check(lib.pr_state_scan_fwd(p(S), p(s), p(lcs), p(Sc), p(sc), b, n, n, h, D * d, D, code, st),
+                   "state_scan_fwd")
+        del S, s
 
     Ya = torch.empty_like(Q)
     la, rm = _empty((BN, c, hq), f32, dev), _empty((BN, c, hq), f32, dev)
@@ -123,18 +139,27 @@ def chunked_bwd(Q: Tensor, K: Tensor, V: Tensor, A: Tensor, lcs: Tensor, Kd: Ten
     f32, u8 = torch.float32, torch.uint8
     p = _lib.ptr
     dO = dO.contiguous()
-    dQg, dSc, dsc = torch.empty_like(Q), torch.empty_like(Sc), torch.empty_like(sc)
+    dQg = torch.empty_like(Q)
     # the attention part's output gradient is dO times a per-row factor: the attention backward applies it on the fly
     dla, dys = torch.empty_like(den), torch.empty_like(den)
-    ws = _empty((lib.pr_query_state_bwd_workspace(BN, c, h, r, d, code),), u8, dev)
-    _lib.check(lib.pr_query_state_bwd(p(Qg), p(Sc), p(sc), p(rm), p(O), p(den), p(dO), p(dQg), p(dSc), p(dsc),
-                                      None, p(dla), p(dys), p(ws), BN, n, c, h, r, d, scale ** deg, 2, 1, code, st),
-               "query_state_bwd")
     dS, ds = torch.empty_like(Sc), torch.empty_like(sc)
     dlcs = torch.empty_like(lcs)   # gate gradient of both scans
-    ws = _empty((lib.pr_state_scan_bwd_workspace(b, n, h, D * d, D),), u8, dev)
-    _lib.check(lib.pr_state_scan_bwd(p(dSc), p(Sc), p(dsc), p(sc), p(lcs), p(dS), p(ds), p(dlcs), p(ws), b, n, n, h,
-                                     D * d, D, code, st), "state_scan_bwd")
+    if _chained(lib, b, n, c, h, r, d):
+        ws = _empty((lib.pr_query_state_scan_bwd_workspace(b, n, c, h, r, d, code),), u8, dev)
+        _lib.check(lib.pr_query_state_scan_bwd(p(Qg), p(Sc), p(sc), p(rm), p(O), p(den), p(dO),
+                                               p(lcs) if gated else None, p(dQg), p(dS), p(ds), None, p(dla), p(dys),
+                                               p(dlcs) if gated else None, p(ws), b, n, c, h, r, d, scale ** deg, 2,
+                                               code, st), "query_state_scan_bwd")
+    else:
+        dSc, dsc = torch.empty_like(Sc), torch.empty_like(sc)
+        ws = _empty((lib.pr_query_state_bwd_workspace(BN, c, h, r, d, code),), u8, dev)
+        _lib.check(lib.pr_query_state_bwd(p(Qg), p(Sc), p(sc), p(rm), p(O), p(den), p(dO), p(dQg), p(dSc), p(dsc),
+                                          None, p(dla), p(dys), p(ws), BN, n, c, h, r, d, scale ** deg, 2, 1, code, st),
+                   "query_state_bwd")
+        ws = _empty((lib.pr_state_scan_bwd_workspace(b, n, h, D * d, D),), u8, dev)
+        _lib.check(lib.pr_state_scan_bwd(p(dSc), p(Sc), p(dsc), p(sc), p(lcs), p(dS), p(ds), p(dlcs), p(ws), b, n, n, h,
+                                         D * d, D, code, st), "state_scan_bwd")
+        del dSc, dsc
     dKd, dVs = torch.empty_like(K), torch.empty_like(V)
     # (two calls: the value gradient and the key gradient are separate kernels, and the latter is timed on its own)
     _lib.check(lib.pr_update_state_bwd(p(Kd), p(V), p(dS), p(ds), None, p(dVs), BN, c, h, d, 2, code, st),

@@ -138,6 +138,52 @@ def test_shape_sweep_fused_vs_composed_vs_oracle(pra):
             check(f"fused vs oracle {nm}", a, b_, OUT_TOL if nm == "Y" else GRAD_TOL)
 
 
+@pytest.mark.parametrize("dtype,b,t,h,r,d,chunk,gated", [
+    (torch.bfloat16, 2, 512, 2, 1, 64, 64, True),      # one stage per chunk
+    (torch.bfloat16, 1, 640, 3, 2, 64, 128, True),     # GQA: 4 stages of folded rows per chunk, odd chunk count
+    (torch.float16, 2, 512, 2, 1, 128, 128, False),    # BASELINE config 5's kind: d = 128, no gates
+    (torch.bfloat16, 2, 384, 1, 4, 32, 64, True),
+    (torch.float16, 1, 256, 2, 1, 32, 128, True),      # two chunks: only chunk 0 is ever accumulated
+])
+def test_chained_state_kernels(pra, dtype, b, t, h, r, d, chunk, gated):
+    """Short chunks: update_state + scan, and the scan's backward + query_state's dS, as single passes that keep
+    the running state in registers, against the separate kernels (tight bar: same products, but the running state
+    is not rounded to 16 bits between the two steps) and against the oracle."""
+    from retention_integration_amd import fused
+    Q, K, V, lg = make_inputs(b, t, h, r, d, dtype, gated, seed=31, std=0.5 if dtype == torch.float16 else 1.0)
+    dO = torch.randn(b, t, h * r, d, generator=torch.Generator().manual_seed(32)).to(dtype)
+    outs = []
+    try:
+        for chain in (True, False):
+            fused.CHAIN = chain
+            xs = [x.to(DEV).requires_grad_(True) if x is not None else None for x in (Q, K, V, lg)]
+            Y = pra.power_retention(*xs, deg=2, chunk_size=chunk)
+            Y.backward(dO.to(DEV))
+            outs.append([Y] + [x.grad for x in xs if x is not None])
+    finally:
+        fused.CHAIN = None
+    names = ["Y", "dQ", "dK", "dV", "dlog_G"]
+    for nm, a, b_ in zip(names, *outs):
+        check(f"chained vs separate {nm}", a, b_, 6e-3)
+    xo = [x.float().clone().requires_grad_(True) if x is not None else None for x in (Q, K, V, lg)]
+    Yo = oracle.power_retention(*xo, deg=2, chunk_size=chunk)
+    Yo.backward(dO.float())
+    for nm, a, b_ in zip(names, outs[0], [Yo] + [x.grad for x in xo if x is not None]):
+        check(f"chained vs oracle {nm}", a, b_, OUT_TOL if nm == "Y" else GRAD_TOL)
+
+
+def test_chained_form_is_chosen_for_many_short_chunks(pra):
+    """The library's own choice: chained where batch x heads x feature blocks fill the chip, separate kernels at the
+    headline shape (8 heads, one batch element), nothing where a chunk is not a whole number of 64-row stages."""
+    from retention_integration_amd import _lib
+    lib = _lib.load()
+    assert lib.pr_state_chain_supported(4, 128, 128, 16, 1, 128) == 2
+    assert lib.pr_state_chain_supported(1, 64, 1024, 8, 1, 64) == 1
+    assert lib.pr_state_chain_supported(2, 4, 96, 2, 1, 64) == 0
+    assert lib.pr_state_chain_supported(2, 4, 64, 2, 3, 64) == 0
+    assert lib.pr_state_chain_supported(2, 1, 64, 2, 1, 64) == 0
+
+
 def test_strong_gates(pra):
     """log_G around -3 per step: weights across a chunk span e^-300, the reference gates of the kernels must keep
     every intermediate in range (same bar as the other cases)."""
