@@ -40,6 +40,43 @@ template <int X> struct PhiTile<f16_t, X> {
   }
 };
 
+// Writes a wave's accumulators -- for each of its XPW x values the 16 feature rows (4g+v) x DV value columns
+// (16nt + lane%16) of S, times mul -- and its key sums.  Each x goes through a per-wave LDS buffer of 16 padded rows
+// (tb, 16 * (2 DV + 16) bytes) so that the tile leaves as whole contiguous kilobytes: the rows of one x are adjacent
+// in S.  S, s point at feature fbase of the (chunk, head).
+template <typename T, int DV, int XPW, int PART>
+__device__ __forceinline__ void tn_store_rows(const f32x4 (&acc)[XPW][DV / 16], const f32x4& sacc, float mul,
+                                              uint32_t tb, T* __restrict__ S, float* __restrict__ s) {
+  typedef __attribute__((address_space(3))) unsigned short lds_u16;
+  typedef __attribute__((address_space(3))) u32x4 lds_u32x4;
+  constexpr int NT = DV / 16, TP = DV * 2 + 16;
+  const int l = lane_id(), g = l >> 4, sl = l & 15;
+  const uint32_t tb_w = tb + 4 * g * TP + sl * 2;   // + 32*nt (+ v*TP): rows 4g+v of column 16nt+sl
+  static_for<XPW>([&](auto xi) {
+    constexpr int X = PART * XPW + decltype(xi)::value;
+#pragma unroll
+    for (int nt = 0; nt < NT; nt++) {
+      float o[4];
+#pragma unroll
+      for (int v = 0; v < 4; v++) o[v] = acc[xi.value][nt][v] * mul;
+      const u32x2 pk = __builtin_bit_cast(u32x2, pack4<T>(o));
+      *(lds_u16*)(tb_w + 32 * nt) = (unsigned short)pk[0];
+      *(lds_u16*)(tb_w + 32 * nt + TP) = (unsigned short)(pk[0] >> 16);
+      *(lds_u16*)(tb_w + 32 * nt + 2 * TP) = (unsigned short)pk[1];
+      *(lds_u16*)(tb_w + 32 * nt + 3 * TP) = (unsigned short)(pk[1] >> 16);
+    }
+    asm volatile("" ::: "memory");   // (LDS operations of one wave execute in order)
+    char* dst = (char*)(S + 16 * X * DV);
+#pragma unroll
+    for (int j = 0; j < DV / 32; j++) {   // one kilobyte per store instruction
+      const int q = j * 1024 + l * 16;
+      *(u32x4*)(dst + q) = *(const lds_u32x4*)(tb + (q / (DV * 2)) * TP + q % (DV * 2));
+    }
+    asm volatile("" ::: "memory");   // the buffer is rewritten for the next x
+  });
+  if (sl >= PART * XPW && sl < (PART + 1) * XPW) *(f32x4*)(s + 16 * sl + 4 * g) = sacc * mul;
+}
+
 template <typename T, int DK, int DV, int XPW, int PART, bool HAS_W>
 __device__ __forceinline__ void tn_body(const T* __restrict__ A, const T* __restrict__ Bm, const float* __restrict__ w,
                                         T* __restrict__ S, float* __restrict__ s, int c, int hA, int r, int hh,
@@ -240,25 +277,12 @@ __device__ __forceinline__ void tn_body(const T* __restrict__ A, const T* __rest
       }
     }
   }
+  lds_barrier();   // every wave is done with the ring: its memory stages the stores
   if (!active) return;
   const float mul = (use_mult && xb < y) ? 2.f : 1.f;
   constexpr int D = 128 * (DK / 16) * (DK / 16 + 1);
-  const int fbase = 128 * y * (y + 1) + 256 * xb;
-  const long so = ((long)bn * h + hh) * D;
-#pragma unroll
-  for (int xi = 0; xi < XPW; xi++) {
-    const int X = PART * XPW + xi;
-#pragma unroll
-    for (int nt = 0; nt < NT; nt++)
-#pragma unroll
-      for (int v = 0; v < 4; v++)
-        S[(so + fbase + 16 * X + 4 * g + v) * DV + 16 * nt + (l & 15)] = (T)(acc[xi][nt][v] * mul);
-  }
-  const int Xc = l & 15;
-  if (Xc >= PART * XPW && Xc < (PART + 1) * XPW) {
-#pragma unroll
-    for (int v = 0; v < 4; v++) s[so + fbase + 16 * Xc + 4 * g + v] = sacc[v] * mul;
-  }
+  const long so = ((long)bn * h + hh) * D + 128 * y * (y + 1) + 256 * xb;
+  tn_store_rows<T, DV, XPW, PART>(acc, sacc, mul, smem_a + wave * (16 * (DV * 2 + 16)), S + so * DV, s + so);
 }
 
 template <typename T, int DK, int DV, int XPW, bool HAS_W>
@@ -310,15 +334,12 @@ __device__ __forceinline__ void tn_chain_body(const T* __restrict__ A, const T* 
                                               int hh, int b, int h, int y, int xb, bool active, bool use_mult,
                                               char* smem) {
   typedef typename VecOf<T>::v8 v8;
-  typedef __attribute__((address_space(3))) unsigned short lds_u16;
-  typedef __attribute__((address_space(3))) u32x4 lds_u32x4;
   constexpr int NT = DV / 16, CA = DK / 8, CB = DV / 8;
   constexpr int A_BYTES = KT * DK * 2, B_BYTES = KT * DV * 2, W_BYTES = KT * 4;
   constexpr int STAGE = A_BYTES + B_BYTES + W_BYTES;
   constexpr int LA = KT * CA / (64 * NW), LB = KT * CB / (64 * NW);   // copies per thread per stage
   constexpr int LOADS = LA + LB;
   constexpr int NSTORE = XPW * (DV / 32);   // 16-byte stores of a boundary per wave (the key sums add one more)
-  static_assert(16 * DV * 2 / 1024 == DV / 32, "one kilobyte per store instruction");
   static_assert(LOADS + 2 * NSTORE <= 63, "the wait counter has six bits");
   constexpr int D = 128 * (DK / 16) * (DK / 16 + 1);
   static_assert(DK == DV, "the A and B tiles share the copy offsets");
@@ -361,38 +382,12 @@ __device__ __forceinline__ void tn_chain_body(const T* __restrict__ A, const T* 
 
   const float mul = (use_mult && xb < y) ? 2.f : 1.f;
   const int fbase = 128 * y * (y + 1) + 256 * xb;
-  // per-wave staging buffer behind the ring: the 16 feature rows of one x, row-major with padded rows, so that the
-  // tile leaves as whole contiguous kilobytes (the rows of one x are adjacent in S)
-  constexpr int TP = DV * 2 + 16;
-  const uint32_t tb = smem_a + TN_NST * STAGE + wave * (16 * TP);
-  const uint32_t tb_w = tb + 4 * g * TP + sl * 2;   // + 32*nt (+ v*TP): rows 4g+v of column 16nt+sl
+  // per-wave staging buffer of the boundary's stores, behind the ring
+  const uint32_t tb = smem_a + TN_NST * STAGE + wave * (16 * (DV * 2 + 16));
   auto write_out = [&](int k) {
     if (!active) return;
     const long so = ((long)(b * n + k) * h + hh) * D + fbase;
-    static_for<XPW>([&](auto xi) {
-      constexpr int X = PART * XPW + decltype(xi)::value;
-#pragma unroll
-      for (int nt = 0; nt < NT; nt++) {
-        float o[4];
-#pragma unroll
-        for (int v = 0; v < 4; v++) o[v] = acc[xi.value][nt][v] * mul;
-        const u32x2 pk = __builtin_bit_cast(u32x2, pack4<T>(o));
-        *(lds_u16*)(tb_w + 32 * nt) = (unsigned short)pk[0];
-        *(lds_u16*)(tb_w + 32 * nt + TP) = (unsigned short)(pk[0] >> 16);
-        *(lds_u16*)(tb_w + 32 * nt + 2 * TP) = (unsigned short)pk[1];
-        *(lds_u16*)(tb_w + 32 * nt + 3 * TP) = (unsigned short)(pk[1] >> 16);
-      }
-      asm volatile("" ::: "memory");   // (LDS operations of one wave execute in order)
-      char* dst = (char*)(S + (so + 16 * X) * DV);
-#pragma unroll
-      for (int j = 0; j < 16 * DV * 2 / 1024; j++) {
-        const int q = j * 1024 + l * 16;
-        const u32x4 val = *(const lds_u32x4*)(tb + (q / (DV * 2)) * TP + q % (DV * 2));
-        *(u32x4*)(dst + q) = val;
-      }
-      asm volatile("" ::: "memory");   // the buffer is rewritten for the next x
-    });
-    if (sl >= PART * XPW && sl < (PART + 1) * XPW) *(f32x4*)(s + so + 16 * sl + 4 * g) = sacc * mul;
+    tn_store_rows<T, DV, XPW, PART>(acc, sacc, mul, tb, S + so * DV, s + so);
   };
   auto decay = [&](int k) {
     if (lcs == nullptr) return;
