@@ -184,6 +184,40 @@ def cpu_baseline(cfg, seconds_hint=20):
                                       f"{dt:.1f} s wall"}
 
 
+def short_chunks(pra, dev, steps, warmup):
+    """BASELINE configs[4]: many short chunks of a wide head -- the state tensors (19.3 GB each) dominate, and the
+    chained state kernels apply."""
+    b, t, h, d, c = 4, 16384, 16, 128, 128
+    g = torch.Generator().manual_seed(42)
+    Q, K, V = ((0.5 * torch.randn(b, t, h, d, generator=g)).to(torch.float16).to(dev).requires_grad_(True)
+               for _ in range(3))
+    dO = torch.randn(b, t, h, d, generator=g).to(torch.float16).to(dev)
+
+    def step():
+        for x in (Q, K, V):
+            x.grad = None
+        pra.power_retention(Q, K, V, None, deg=2, chunk_size=c).backward(dO)
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / steps
+    f_fwd, f_bwd = flops(b, t, h, d, c, d * (d + 1) // 2)
+    print(json.dumps({
+        "metric": "fwd+bwd tokens/s at b=4,t=16384,h=16,d=128,deg=2,chunk=128 (no gating, fp16)",
+        "value": round(b * t / dt, 1), "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+        "ms_per_step": round(dt * 1e3, 3), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "fp16", "data": "synthetic",
+        "config": {"workload": "power_retention fwd+bwd b=4 t=16384 h=16 d=128 deg=2 chunk_size=128 gating=False "
+                               "(BASELINE configs[4])"},
+        "tflops": round((f_fwd + f_bwd) / dt / 1e12, 2),
+        "state_bytes_per_tensor": b * (t // c) * h * 128 * (d // 16) * (d // 16 + 1) * d * 2}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -195,6 +229,9 @@ def main():
     ap.add_argument("--counter-run", action="store_true",
                     help="for rocprofv3 --pmc: launch only the dominant kernel (sympow_grad, dK of update_state "
                          "backward) a few times, and a plain device copy of 256 MiB for calibrating byte counters")
+    ap.add_argument("--short-chunks", action="store_true",
+                    help="instead of the headline workload: BASELINE configs[4] (fp16, b=4, t=16384, h=16, d=128, "
+                         "chunk 128, no gating, inputs N(0,1)*0.5), fwd+bwd; prints its own JSON line")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs on one GPU; --gpus N with N > 1 is not supported", file=sys.stderr)
@@ -203,8 +240,11 @@ def main():
     import retention_integration_amd as pra
     from retention_integration_amd import expanded_dim
 
-    cfg = CFG
     dev = torch.device("cuda:0")
+    if args.short_chunks:
+        short_chunks(pra, dev, args.steps, args.warmup)
+        return
+    cfg = CFG
     Q, K, V, lg, dO = make_inputs(cfg["b"], cfg["t"], cfg["h"], cfg["d"], dev)
     if args.counter_run:
         counter_run(pra, Q, K, V, cfg, dev)
