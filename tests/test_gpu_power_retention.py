@@ -144,13 +144,40 @@ def test_shape_sweep_fused_vs_composed_vs_oracle(pra):
     (torch.float16, 2, 512, 2, 1, 128, 128, False),    # BASELINE config 5's kind: d = 128, no gates
     (torch.bfloat16, 2, 384, 1, 4, 32, 64, True),
     (torch.float16, 1, 256, 2, 1, 32, 128, True),      # two chunks: only chunk 0 is ever accumulated
+    (torch.bfloat16, 1, 512, 2, 2, 128, 128, True),    # d = 128 (32-row stages) with GQA and gates
 ])
 def test_chained_state_kernels(pra, dtype, b, t, h, r, d, chunk, gated):
+    _chained_case(pra, dtype, b, t, h, r, d, chunk, gated, 1.0)
+
+
+@pytest.mark.parametrize("dtype,b,t,h,r,d,chunk", [
+    (torch.bfloat16, 2, 512, 2, 1, 64, 64),
+    (torch.float16, 1, 640, 2, 2, 128, 128),
+    (torch.bfloat16, 1, 384, 2, 4, 32, 64),
+])
+def test_chained_state_kernels_weak_gates(pra, dtype, b, t, h, r, d, chunk):
+    """Gates close to 1 (a chunk keeps 30-50 % of the state): every earlier chunk matters to every later one, so a
+    decay applied with the wrong chunk's gate, or in the wrong order, shows (with logsigmoid(N(0,1)) gates a chunk of
+    64 tokens forgets the state entirely and the scan degenerates to a shift)."""
+    _chained_case(pra, dtype, b, t, h, r, d, chunk, True, 0.02)
+
+
+def test_weak_gates(pra):
+    """The same for the separate scan kernels (the default path at this shape)."""
+    b, t, h, r, d, chunk = 2, 1024, 2, 2, 64, 128
+    Q, K, V, lg = make_inputs(b, t, h, r, d, torch.bfloat16, True, seed=41)
+    dO = torch.randn(b, t, h * r, d, generator=torch.Generator().manual_seed(42)).to(torch.bfloat16)
+    run_both(pra, Q, K, V, lg * 0.01, chunk, dO)
+
+
+def _chained_case(pra, dtype, b, t, h, r, d, chunk, gated, gate_scale):
     """Short chunks: update_state + scan, and the scan's backward + query_state's dS, as single passes that keep
     the running state in registers, against the separate kernels (tight bar: same products, but the running state
     is not rounded to 16 bits between the two steps) and against the oracle."""
     from retention_integration_amd import fused
     Q, K, V, lg = make_inputs(b, t, h, r, d, dtype, gated, seed=31, std=0.5 if dtype == torch.float16 else 1.0)
+    if gated:
+        lg = lg * gate_scale
     dO = torch.randn(b, t, h * r, d, generator=torch.Generator().manual_seed(32)).to(dtype)
     outs = []
     try:
@@ -170,6 +197,36 @@ def test_chained_state_kernels(pra, dtype, b, t, h, r, d, chunk, gated):
     Yo.backward(dO.float())
     for nm, a, b_ in zip(names, outs[0], [Yo] + [x.grad for x in xo if x is not None]):
         check(f"chained vs oracle {nm}", a, b_, OUT_TOL if nm == "Y" else GRAD_TOL)
+
+
+def test_chained_state_kernels_at_full_size(pra):
+    """BASELINE configs[4] at its full size (fp16, b=4, t=16384, h=16, d=128, chunk 128, no gating; 19.3 GB per
+    state tensor): the chained kernels, which the library picks there, against the separate ones."""
+    from retention_integration_amd import fused
+    b, t, h, d, c = 4, 16384, 16, 128, 128
+    g = torch.Generator(device=DEV).manual_seed(7)
+    Q, K, V = ((0.5 * torch.randn(b, t, h, d, generator=g, device=DEV)).half().requires_grad_(True) for _ in range(3))
+    dO = torch.randn(b, t, h, d, generator=g, device=DEV).half()
+    assert fused._chained(__import__("retention_integration_amd")._lib.load(), b, t // c, c, h, 1, d)
+    outs = []
+    try:
+        for chain in (None, False):
+            fused.CHAIN = chain
+            for x in (Q, K, V):
+                x.grad = None
+            Y = pra.power_retention(Q, K, V, None, deg=2, chunk_size=c)
+            Y.backward(dO)
+            outs.append([Y.detach()] + [x.grad for x in (Q, K, V)])
+            del Y
+    finally:
+        fused.CHAIN = None
+    for nm, a, b_ in zip(["Y", "dQ", "dK", "dV"], *outs):
+        assert torch.isfinite(a).all()
+        err = ((a.float() - b_.float()).norm() / b_.float().norm()).item()
+        print(f"  chained vs separate {nm}: rel-L2 {err:.3e}", flush=True)
+        assert err <= 6e-3, (nm, err)
+    del outs
+    torch.cuda.empty_cache()
 
 
 def test_chained_form_is_chosen_for_many_short_chunks(pra):
