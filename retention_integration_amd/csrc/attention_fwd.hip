@@ -60,11 +60,12 @@ __global__ __launch_bounds__(256, OCC) void attention_fwd_kernel(AttnFwdArgs a, 
   // shader engines (index / 8 % 4); only the CU inside a shader engine is chosen by load.  Row blocks differ in
   // length (causal), so each of the 32 (XCD, shader engine) groups is given whole (batch, kv head) pairs: every
   // group then gets the same mix of long and short row blocks and the K/V of a pair stay in one L2.  Inside a
-  // group the longest row blocks of all its pairs come first and the shortest last (they fill the tail).
+  // group the pairs follow one another, longest row block first, so that the row blocks of a pair run together.
   const int grp = blockIdx.x % 32, u = blockIdx.x / 32, ppg = (npairs + 31) / 32;
   // (integer division runs on the vector unit: readfirstlane brings the uniform results back to scalar registers)
-  const int pair = __builtin_amdgcn_readfirstlane((u % ppg) * 32 + grp);
-  const int rblk = row_blocks - 1 - __builtin_amdgcn_readfirstlane(u / ppg);
+  const int pig = __builtin_amdgcn_readfirstlane(u / row_blocks);
+  const int pair = pig * 32 + grp;
+  const int rblk = row_blocks - 1 - (u - pig * row_blocks);
   if (pair >= npairs) return;
   const int b = __builtin_amdgcn_readfirstlane(pair / a.h), hh = pair - b * a.h;
   const int hq = a.h * a.r, rows = a.tq * a.r, shift = a.tk - a.tq;

@@ -48,7 +48,7 @@ template <> __device__ __forceinline__ void unpack2<f16_t>(uint32_t u, float& lo
 }
 
 template <typename T, int DK, int DV, int MT, bool MULT>
-__global__ __launch_bounds__(256, 2) void sympow_grad_kernel(GradArgs a, int row_blocks, int npairs) {
+__global__ __launch_bounds__(256, (MT == 2 && DK <= 64) ? 4 : 2) void sympow_grad_kernel(GradArgs a, int row_blocks, int npairs) {
   typedef typename VecOf<T>::v8 v8;
   typedef typename VecOf<T>::v4 v4;
   constexpr int TT = DK / 16, KS = DV / 32, KX = DK / 32, ROWS = 64 * MT, CB = DV / 8, CX = DK / 8;
@@ -318,7 +318,10 @@ template <typename T, int DK, int DV, bool MULT> static int grad_launch(const Gr
     hipLaunchKernelGGL(kern, grid, dim3(256), smem, st, a, row_blocks, npairs);
   };
   if constexpr (DK <= 64) {
-    if (rows >= 256) { go(IC<4>{}); return (int)hipGetLastError(); }
+    // 128 rows per workgroup at d = 64: half the reuse of a state tile, but four workgroups (16 waves) share a
+    // compute unit and the vector instructions of the two folds issue at twice the rate (measured 7 % faster than
+    // 256 rows at two workgroups)
+    if (rows >= 256 && DK < 64) { go(IC<4>{}); return (int)hipGetLastError(); }
     if (rows > 64) { go(IC<2>{}); return (int)hipGetLastError(); }
   }
   go(IC<1>{});

@@ -293,13 +293,22 @@ __global__ __launch_bounds__(256, 2) void sympow_tn_kernel(const T* __restrict__
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   constexpr int PARTS = 16 / XPW;
   constexpr int NB = (DK / 16) * (DK / 16 + 1) / 2;
-  const int task = blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  // Workgroups are handed to the 8 XCDs (each with its own L2) round-robin by linear id.  The workgroups of a
+  // (chunk, head) read the same rows, so ids are permuted to put them on one XCD: XCD x takes the x-th eighth.
+  int bx = blockIdx.x, by = blockIdx.y;
+  const int total = gridDim.x * gridDim.y;
+  if (total % 8 == 0) {
+    const int lin = by * gridDim.x + bx, v = (lin % 8) * (total / 8) + lin / 8;
+    by = v / gridDim.x;
+    bx = v - by * gridDim.x;
+  }
+  const int task = bx * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const bool active = task < NB * PARTS;
   const int t2 = active ? task : 0;
   const int part = t2 % PARTS;
   int y, xb;
   block_to_yx(t2 / PARTS, y, xb);
-  const int bn = blockIdx.y / h, hh = blockIdx.y % h;
+  const int bn = by / h, hh = by % h;
 #define PR_TN_CASE(P)                                                                                                  \
   case P:                                                                                                              \
     if (P < PARTS)                                                                                                     \
