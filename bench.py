@@ -297,7 +297,7 @@ def main():
                        "frac": round(k_flops / k_ms / 1e9 / PEAK_BF16_TFLOPS, 4), "ms_per_launch": round(k_ms, 4),
                        # HBM bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE, calibrated with a plain
                        # 256 MiB copy (profiles/sympow_grad_t65536_hbm_traffic.txt); algorithmic: 374.3 MB
-                       "traffic": 374.8e6}
+                       "traffic": 374.6e6}
     t_ms = in_step_ms["sympow_tn(update_state)"]
     out["roofline_update_state_fwd"] = {"kernel": "sympow_tn_kernel", "bound": "mfma",
                                         "achieved": round(k_flops / t_ms / 1e9, 2), "peak": PEAK_BF16_TFLOPS,
