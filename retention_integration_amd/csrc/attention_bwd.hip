@@ -25,7 +25,8 @@ namespace pr {
 
 constexpr int AB_BN = 64;    // keys per stage in the dQ kernel
 constexpr int AB_BM = 64;    // query rows per stage in the dK/dV kernel
-constexpr int AB_NST = 3;
+// stages in the ring: three up to d = 64; two at d = 128, where three would leave room for one workgroup per CU
+constexpr int ab_stages(int d) { return d <= 64 ? 3 : 2; }
 constexpr float AB_LOG_EPS = 1e-7f, AB_EXP_CLAMP = 80.f;
 
 // a2^(half_deg - 1)
@@ -57,6 +58,7 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dq_kernel(AttnBwdArgs a,
   constexpr int KS = DH / 32, NT = DH / 16, KT = AB_BN / 16, ROWS = 64 * MT, CPR = DH / 8, RB = CPR * 16;
   constexpr int TILE = AB_BN * RB;
   constexpr int STAGE = 2 * TILE + 4 * AB_BN * 4;   // K, V, raw gates, two sets of key gate factors
+  constexpr int NST = ab_stages(DH);
   constexpr int LOADS = 2 * AB_BN * CPR / 256;
   extern __shared__ __attribute__((aligned(1024))) char smem[];
 
@@ -104,7 +106,7 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dq_kernel(AttnBwdArgs a,
   const T* dQsg = a.dQs ? (const T*)a.dQs + (long)b * a.tq * hq * DH : nullptr;
   const int ntot = ntiles + (dQsg ? 1 : 0);
   auto issue = [&](int it) __attribute__((always_inline)) {
-    char* st = smem + (it % AB_NST) * STAGE;
+    char* st = smem + (it % NST) * STAGE;
     if (it >= ntiles) {
 #pragma unroll
       for (int ii = 0; ii < LOADS; ii++) {
@@ -133,7 +135,7 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dq_kernel(AttnBwdArgs a,
     if (Gg && wave == 0) async_copy4(Gg + (long)min(j0 + l, a.tk - 1) * a.h, st + 2 * TILE);
   };
   issue(0);
-  if (ntot > 1) issue(1);
+  if (NST == 3 && ntot > 1) issue(1);
 
   v8 Qf[MT][KS], dOf[MT][KS];
   int ti[MT];
@@ -190,7 +192,7 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dq_kernel(AttnBwdArgs a,
   // exp(R - gate) relative to the tile's last key (<= 1) and to the first key of each 16-key group (>= 1);
   // written by wave 0, which issued the gate copy and so is the one that can wait for it
   auto gate_factors = [&](int it) __attribute__((always_inline)) {
-    float* graw = (float*)(smem + (it % AB_NST) * STAGE + 2 * TILE);
+    float* graw = (float*)(smem + (it % NST) * STAGE + 2 * TILE);
     const int rpos = min(AB_BN - 1, a.tk - 1 - it * AB_BN);
     const float gv = Gg ? graw[l] : 0.f;
     const float R_ = Gg ? graw[rpos] : 0.f, Rs = Gg ? graw[l & ~15] : 0.f;
@@ -203,15 +205,31 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dq_kernel(AttnBwdArgs a,
     gate_factors(0);
   }
   auto sync_step = [&](int it) __attribute__((always_inline)) -> char* {
-    char* st = smem + (it % AB_NST) * STAGE;
-    if (it + 1 < ntot) wait_vmcnt<LOADS>(); else wait_vmcnt<0>();
-    lds_barrier();
-    if (it + 2 < ntot) issue(it + 2);
-    if (wave == 0 && it + 1 < ntiles) {
-      if (it + 2 < ntot) wait_vmcnt<LOADS + 1>(); else wait_vmcnt<0>();   // all but the stage just issued
-      gate_factors(it + 1);
+    char* st = smem + (it % NST) * STAGE;
+    if constexpr (NST == 3) {
+      if (it + 1 < ntot) wait_vmcnt<LOADS>(); else wait_vmcnt<0>();
+      lds_barrier();
+      if (it + 2 < ntot) issue(it + 2);
+      if (wave == 0 && it + 1 < ntiles) {
+        if (it + 2 < ntot) wait_vmcnt<LOADS + 1>(); else wait_vmcnt<0>();   // all but the stage just issued
+        gate_factors(it + 1);
+      }
+    } else {
+      wait_vmcnt<0>();   // one stage in flight
+      lds_barrier();
+      if (it + 1 < ntot) issue(it + 1);
     }
     return st;
+  };
+  // two-stage ring: wave 0 prepares the next tile's factors after its own work on this one, when the copy issued at
+  // the start of the step has had a tile's time to arrive
+  auto after_step = [&](int it) __attribute__((always_inline)) {
+    if constexpr (NST == 2) {
+      if (wave == 0 && it + 1 < ntiles) {
+        wait_vmcnt<0>();
+        gate_factors(it + 1);
+      }
+    }
   };
 
   // One 64-key tile.  Past tiles: key factors relative to the gate at the wave's first row (<= 1), the row factor
@@ -309,7 +327,10 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dq_kernel(AttnBwdArgs a,
   };
 
   int it = 0;
-  for (; it < n_past; it++) tile(it, sync_step(it), IC<0>{});
+  for (; it < n_past; it++) {
+    tile(it, sync_step(it), IC<0>{});
+    after_step(it);
+  }
   // the past tiles were accumulated without the row factor scale^deg * exp(G_q - m - Rw); apply it once
 #pragma unroll
   for (int mi = 0; mi < MT; mi++) {
@@ -318,15 +339,21 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dq_kernel(AttnBwdArgs a,
     for (int nt = 0; nt < NT; nt++) acc[mi][nt] *= f;
     dgq[mi] *= f;
   }
-  for (; it < n_seen; it++) tile(it, sync_step(it), IC<1>{});
-  for (; it < ntiles; it++) sync_step(it);
+  for (; it < n_seen; it++) {
+    tile(it, sync_step(it), IC<1>{});
+    after_step(it);
+  }
+  for (; it < ntiles; it++) {
+    sync_step(it);
+    after_step(it);
+  }
 
   T* dQg = (T*)a.dQ + (long)b * a.tq * hq * DH;
   uint32_t ep = 0;
   if (dQsg) {
     wait_vmcnt<0>();
     lds_barrier();
-    ep = (uint32_t)(uintptr_t)(ab_lds_char*)(smem + (ntiles % AB_NST) * STAGE);
+    ep = (uint32_t)(uintptr_t)(ab_lds_char*)(smem + (ntiles % NST) * STAGE);
   }
 #pragma unroll
   for (int mi = 0; mi < MT; mi++) {
@@ -384,6 +411,7 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
   // [2] dl, [3] dO scale, [4] far-tile factor * dO scale, [5] far-tile factor * dl
   constexpr int NV = 6;
   constexpr int STAGE = 2 * TILE + NV * AB_BM * 4;
+  constexpr int NST = ab_stages(DH);
   constexpr int LOADS = 2 * AB_BM * CPR / 256;
   extern __shared__ __attribute__((aligned(1024))) char smem[];
 
@@ -456,7 +484,7 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
   for (int ii = 0; ii < LOADS / 2; ii++)
     voff[ii] = (uint32_t)((((grow(ii) >> rsh) * hq + hh * a.r + (grow(ii) & (a.r - 1))) * (DH * 2))) + gchk(ii);
   auto issue = [&](int step) __attribute__((always_inline)) {
-    char* st = smem + (step % AB_NST) * STAGE;
+    char* st = smem + (step % NST) * STAGE;
     if (step >= nsteps) {
       const T* src = step == nsteps ? dKsg : dVsg;
 #pragma unroll
@@ -476,7 +504,7 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
     if (regular && rbase + AB_BM <= rows) {
       // a whole tile of whole time steps: lane offsets are fixed, the tile's base moves in scalar registers
       const long tb = (long)(rbase >> rsh) * hq;   // first [t, hq] row of the tile
-      const uint32_t sa = __builtin_amdgcn_readfirstlane(smem_a + (step % AB_NST) * STAGE + wave * 1024);
+      const uint32_t sa = __builtin_amdgcn_readfirstlane(smem_a + (step % NST) * STAGE + wave * 1024);
       const void* qb_ = uniform_ptr(Qg + tb * (DH * 2));
       const void* ob_ = uniform_ptr(dOg + tb * (DH * 2));
 #pragma unroll
@@ -515,7 +543,7 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
     }
   };
   if (ntot > 0) issue(0);
-  if (ntot > 1) issue(1);
+  if (NST == 3 && ntot > 1) issue(1);
 
   v8 Kf[MK][KS], Vf[MK][KS];
   int key[MK];
@@ -565,7 +593,7 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
   // Row vectors of a tile (wave 0 issued their copies): G_q - m, time index (-1 for rows past the end), dl, dO
   // scale, and the far-tile factors scale^deg exp(G_q - m - R) * {dO scale, dl} (zero for rows past the end).
   auto row_factors = [&](int step) __attribute__((always_inline)) {
-    float* rv = (float*)(smem + (step % AB_NST) * STAGE + 2 * TILE);
+    float* rv = (float*)(smem + (step % NST) * STAGE + 2 * TILE);
     const int row = (ntile_total - 1 - step) * AB_BM + l;
     const bool real = row < rows;
     const float bs = (Gg ? rv[l] : 0.f) - rv[AB_BM + l];
@@ -584,15 +612,30 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
     row_factors(0);
   }
   auto sync_step = [&](int step) __attribute__((always_inline)) -> char* {
-    char* st = smem + (step % AB_NST) * STAGE;
-    if (step + 1 < ntot) wait_vmcnt<LOADS>(); else wait_vmcnt<0>();
-    lds_barrier();
-    if (step + 2 < ntot) issue(step + 2);
-    if (wave == 0 && step + 1 < nsteps) {
-      if (step + 2 < ntot) wait_vmcnt<LOADS + 4>(); else wait_vmcnt<0>();   // all but the stage just issued
-      row_factors(step + 1);
+    char* st = smem + (step % NST) * STAGE;
+    if constexpr (NST == 3) {
+      if (step + 1 < ntot) wait_vmcnt<LOADS>(); else wait_vmcnt<0>();
+      lds_barrier();
+      if (step + 2 < ntot) issue(step + 2);
+      if (wave == 0 && step + 1 < nsteps) {
+        if (step + 2 < ntot) wait_vmcnt<LOADS + 4>(); else wait_vmcnt<0>();   // all but the stage just issued
+        row_factors(step + 1);
+      }
+    } else {
+      wait_vmcnt<0>();   // one stage in flight
+      lds_barrier();
+      if (step + 1 < ntot) issue(step + 1);
     }
     return st;
+  };
+  // two-stage ring: wave 0 prepares the next tile's row vectors after its own work on this one
+  auto after_step = [&](int step) __attribute__((always_inline)) {
+    if constexpr (NST == 2) {
+      if (wave == 0 && step + 1 < nsteps) {
+        wait_vmcnt<0>();
+        row_factors(step + 1);
+      }
+    }
   };
 
   auto tile = [&](const char* st, int rbase, auto far_c) __attribute__((always_inline)) {
@@ -707,7 +750,10 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
   };
 
   int step = 0;
-  for (; step < n_far; step++) tile(sync_step(step), (ntile_total - 1 - step) * AB_BM, IC<1>{});
+  for (; step < n_far; step++) {
+    tile(sync_step(step), (ntile_total - 1 - step) * AB_BM, IC<1>{});
+    after_step(step);
+  }
   // the far tiles were accumulated without the key factor exp(R - G_k) (<= 1); apply it once.  The tiles near
   // the diagonal are accumulated in absolute terms (their packed weights stay <= the true ones).
 #pragma unroll
@@ -720,8 +766,18 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
     }
     dgk[kj] *= c;
   }
-  for (; step < n_seen; step++) tile(sync_step(step), (ntile_total - 1 - step) * AB_BM, IC<0>{});
-  for (; step < nsteps; step++) sync_step(step);
+  for (; step < n_seen; step++) {
+    tile(sync_step(step), (ntile_total - 1 - step) * AB_BM, IC<0>{});
+    after_step(step);
+  }
+  for (; step < nsteps; step++) {
+    sync_step(step);
+    after_step(step);
+  }
+  if (NST == 2 && nsteps + 1 < ntot) {   // the second of the two epilogue stages has no step that would copy it
+    lds_barrier();
+    issue(nsteps + 1);
+  }
 
   T* dKg = (T*)a.dK + (long)b * a.tk * a.h * DH + hh * DH;
   T* dVg = (T*)a.dV + (long)b * a.tk * a.h * DH + hh * DH;
@@ -729,8 +785,8 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
   if (dKsg) {
     wait_vmcnt<0>();
     lds_barrier();
-    epk = (uint32_t)(uintptr_t)(ab_lds_char*)(smem + (nsteps % AB_NST) * STAGE);
-    epv = (uint32_t)(uintptr_t)(ab_lds_char*)(smem + ((nsteps + 1) % AB_NST) * STAGE);
+    epk = (uint32_t)(uintptr_t)(ab_lds_char*)(smem + (nsteps % NST) * STAGE);
+    epv = (uint32_t)(uintptr_t)(ab_lds_char*)(smem + ((nsteps + 1) % NST) * STAGE);
   }
   const float Glast = Gg ? Gg[(long)(a.tk - 1) * a.h] : 0.f;
 #pragma unroll
@@ -787,7 +843,7 @@ template <typename T, int DH, bool DEG2> static int attn_bwd_launch(const AttnBw
   const int npairs = B * a.h;
   {
     constexpr int MT = DH <= 64 ? 2 : 1;
-    constexpr size_t smem = AB_NST * (2 * AB_BN * DH * 2 + 4 * AB_BN * 4);
+    constexpr size_t smem = ab_stages(DH) * (2 * AB_BN * DH * 2 + 4 * AB_BN * 4);
     const int rows = a.tq * a.r;
     const int nblocks = (rows + 64 * MT - 1) / (64 * MT);
     dim3 grid((unsigned)((npairs + 31) / 32 * 32 * nblocks));
@@ -797,7 +853,7 @@ template <typename T, int DH, bool DEG2> static int attn_bwd_launch(const AttnBw
   }
   {
     constexpr int MK = DH <= 64 ? 2 : 1;
-    constexpr size_t smem = AB_NST * (2 * AB_BM * DH * 2 + 6 * AB_BM * 4);
+    constexpr size_t smem = ab_stages(DH) * (2 * AB_BM * DH * 2 + 6 * AB_BM * 4);
     const int nblocks = (a.tk + 64 * MK - 1) / (64 * MK);
     dim3 grid((unsigned)((npairs + 31) / 32 * 32 * nblocks));
     auto kern = attention_bwd_dkv_kernel<T, DH, MK, DEG2>;

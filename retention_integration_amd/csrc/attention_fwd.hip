@@ -23,7 +23,9 @@
 
 namespace pr {
 
-constexpr int AT_BN = 64, AT_NST = 3;
+constexpr int AT_BN = 64;
+// stages in the ring: three up to d = 64; two at d = 128, where three would leave room for one workgroup per CU
+constexpr int at_stages(int d) { return d <= 64 ? 3 : 2; }
 constexpr float AT_LOG_EPS = 1e-7f, AT_SUM_EPS = 1e-6f, AT_EXP_CLAMP = 80.f;
 
 template <typename T> struct OnesBits;
@@ -52,6 +54,7 @@ __global__ __launch_bounds__(256, OCC) void attention_fwd_kernel(AttnFwdArgs a, 
   constexpr int TILE = AT_BN * RB;                  // bytes of one K or V tile
   constexpr int STAGE = 2 * TILE + 4 * AT_BN * 4;   // K, V, raw gates, two sets of key gate factors
   constexpr int LOADS = 2 * AT_BN * CPR / 256;      // tile copies per thread per stage
+  constexpr int NST = at_stages(DH);
   extern __shared__ __attribute__((aligned(1024))) char smem[];
 
   const int tid = threadIdx.x, l = tid & 63, g = l >> 4, tcol = l & 15;
@@ -98,7 +101,7 @@ __global__ __launch_bounds__(256, OCC) void attention_fwd_kernel(AttnFwdArgs a, 
     goff[ii] = (uint32_t)(row * (int)kstride + 16 * ((pos % CPR) ^ swz<CPR>(row)));
   }
   auto issue = [&](int it) __attribute__((always_inline)) {
-    char* st = smem + (it % AT_NST) * STAGE;
+    char* st = smem + (it % NST) * STAGE;
     const int j0 = it * AT_BN;
     if (j0 + AT_BN <= a.tk) {
       const char* kb_ = Kg + (long)j0 * kstride;
@@ -115,7 +118,7 @@ __global__ __launch_bounds__(256, OCC) void attention_fwd_kernel(AttnFwdArgs a, 
     if (Gg && wave == 0) async_copy4(Gg + (long)min(j0 + l, a.tk - 1) * a.h, st + 2 * TILE);
   };
   issue(0);
-  if (ntiles > 1) issue(1);
+  if (NST == 3 && ntiles > 1) issue(1);
 
   v8 Qf[MT][KS];
   int ti[MT];
@@ -175,7 +178,7 @@ __global__ __launch_bounds__(256, OCC) void attention_fwd_kernel(AttnFwdArgs a, 
   // Gate factors of tile `it`, written by wave 0 (it issued the gate copy, so it alone can wait for it):
   // exp(R - gate) relative to the tile's last key (<= 1) and relative to the first key of each 16-key group (>= 1).
   auto gate_factors = [&](int it) __attribute__((always_inline)) {
-    float* graw = (float*)(smem + (it % AT_NST) * STAGE + 2 * TILE);
+    float* graw = (float*)(smem + (it % NST) * STAGE + 2 * TILE);
     const int rpos = min(AT_BN - 1, a.tk - 1 - it * AT_BN);
     const float gv = Gg ? graw[l] : 0.f;
     const float R_ = Gg ? graw[rpos] : 0.f, Rs = Gg ? graw[l & ~15] : 0.f;
@@ -190,15 +193,30 @@ __global__ __launch_bounds__(256, OCC) void attention_fwd_kernel(AttnFwdArgs a, 
   // Make tile `it` visible to the workgroup, start the copy of tile it+2, and (wave 0) prepare the gate factors of
   // tile it+1 while the others already compute.
   auto sync_step = [&](int it) __attribute__((always_inline)) -> char* {
-    char* st = smem + (it % AT_NST) * STAGE;
-    if (it + 1 < ntiles) wait_vmcnt<LOADS>(); else wait_vmcnt<0>();
-    lds_barrier();
-    if (it + 2 < ntiles) issue(it + 2);
-    if (wave == 0 && it + 1 < ntiles) {
-      if (it + 2 < ntiles) wait_vmcnt<LOADS + 1>(); else wait_vmcnt<0>();   // all but the stage just issued
-      gate_factors(it + 1);
+    char* st = smem + (it % NST) * STAGE;
+    if constexpr (NST == 3) {
+      if (it + 1 < ntiles) wait_vmcnt<LOADS>(); else wait_vmcnt<0>();
+      lds_barrier();
+      if (it + 2 < ntiles) issue(it + 2);
+      if (wave == 0 && it + 1 < ntiles) {
+        if (it + 2 < ntiles) wait_vmcnt<LOADS + 1>(); else wait_vmcnt<0>();   // all but the stage just issued
+        gate_factors(it + 1);
+      }
+    } else {
+      wait_vmcnt<0>();   // one stage in flight
+      lds_barrier();
+      if (it + 1 < ntiles) issue(it + 1);
     }
     return st;
+  };
+  // two-stage ring: wave 0 prepares the next tile's factors after its own work on this one
+  auto after_step = [&](int it) __attribute__((always_inline)) {
+    if constexpr (NST == 2) {
+      if (wave == 0 && it + 1 < ntiles) {
+        wait_vmcnt<0>();
+        gate_factors(it + 1);
+      }
+    }
   };
 
   // One 64-key tile.  Past tiles use one reference gate (the tile's last key), so both gate factors are <= 1.
@@ -297,7 +315,10 @@ __global__ __launch_bounds__(256, OCC) void attention_fwd_kernel(AttnFwdArgs a, 
   };
 
   int it = 0;
-  for (; it < n_past; it++) tile(it, sync_step(it), IC<0>{});
+  for (; it < n_past; it++) {
+    tile(it, sync_step(it), IC<0>{});
+    after_step(it);
+  }
   // the past tiles were accumulated without the row factor exp(G_q - Rw) * scale^deg; apply it once
 #pragma unroll
   for (int mi = 0; mi < MT; mi++) {
@@ -307,8 +328,14 @@ __global__ __launch_bounds__(256, OCC) void attention_fwd_kernel(AttnFwdArgs a, 
     accl[mi] *= f;
     mx[mi] *= f;
   }
-  for (; it < n_seen; it++) tile(it, sync_step(it), IC<1>{});
-  for (; it < ntiles; it++) sync_step(it);
+  for (; it < n_seen; it++) {
+    tile(it, sync_step(it), IC<1>{});
+    after_step(it);
+  }
+  for (; it < ntiles; it++) {
+    sync_step(it);
+    after_step(it);
+  }
 
   T* Og = (T*)a.O + (long)b * a.tq * hq * DH;
 #pragma unroll
@@ -338,7 +365,7 @@ template <typename T, int DH, bool DEG2> static int attn_fwd_launch(const AttnFw
   const int rows = a.tq * a.r;
   auto go = [&](auto mt, auto occ) {
     constexpr int MT = decltype(mt)::value, OCC = decltype(occ)::value;
-    constexpr size_t smem = AT_NST * (2 * AT_BN * DH * 2 + 4 * AT_BN * 4);
+    constexpr size_t smem = at_stages(DH) * (2 * AT_BN * DH * 2 + 4 * AT_BN * 4);
     const int row_blocks = (rows + 64 * MT - 1) / (64 * MT), npairs = B * a.h;
     dim3 grid((unsigned)(((npairs + 31) / 32) * 32 * row_blocks));
     auto kern = attention_fwd_kernel<T, DH, MT, DEG2, OCC>;

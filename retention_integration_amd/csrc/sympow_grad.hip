@@ -323,6 +323,9 @@ template <typename T, int DK, int DV, bool MULT> static int grad_launch(const Gr
     // 256 rows at two workgroups)
     if (rows >= 256 && DK < 64) { go(IC<4>{}); return (int)hipGetLastError(); }
     if (rows > 64) { go(IC<2>{}); return (int)hipGetLastError(); }
+  } else {
+    // d = 128: a workgroup streams the whole 2.4 MB state from L2; 128 rows halve that traffic
+    if (rows > 64) { go(IC<2>{}); return (int)hipGetLastError(); }
   }
   go(IC<1>{});
   return (int)hipGetLastError();

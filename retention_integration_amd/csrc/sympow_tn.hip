@@ -19,8 +19,10 @@
 
 namespace pr {
 
-constexpr int TN_KT = 64;   // rows per pipeline stage (two contraction steps of 32)
 constexpr int TN_NST = 3;   // stages in the ring
+// rows per pipeline stage: two contraction steps of 32 up to d = 64, one at d = 128 (so that the ring of two
+// workgroups fits a compute unit's LDS)
+constexpr int tn_stage_rows(int d) { return d <= 64 ? 64 : 32; }
 
 template <typename T, int X> struct PhiTile;
 template <int X> struct PhiTile<bf16_t, X> {
@@ -84,12 +86,13 @@ __device__ __forceinline__ void tn_body(const T* __restrict__ A, const T* __rest
   typedef typename VecOf<T>::v8 v8;
   typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
   typedef __attribute__((address_space(3))) f32x4 lds_f32x4;
+  constexpr int KT = tn_stage_rows(DV);                            // rows per pipeline stage
   constexpr int NT = DV / 16, CA = DK / 8, CB = DV / 8;            // 16-byte chunks per row
-  constexpr int A_BYTES = TN_KT * DK * 2, B_BYTES = TN_KT * DV * 2, W_BYTES = TN_KT * 4;
+  constexpr int A_BYTES = KT * DK * 2, B_BYTES = KT * DV * 2, W_BYTES = KT * 4;
   constexpr int STAGE = A_BYTES + B_BYTES + W_BYTES;
-  constexpr int LA = TN_KT * CA / 256, LB = TN_KT * CB / 256;      // copies per thread per stage (w rides on wave 0)
+  constexpr int LA = KT * CA / 256, LB = KT * CB / 256;      // copies per thread per stage (w rides on wave 0)
   constexpr int LOADS = LA + LB;
-  static_assert(CA == CB && TN_KT == 64 && TN_NST == 3, "the loop below is written for this shape");
+  static_assert(CA == CB && TN_NST == 3 && (KT == 64 || DV > 64), "the loops below are written for these shapes");
   const int tid = threadIdx.x, l = tid & 63, g = l >> 4;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int rows = c * r;
@@ -101,10 +104,10 @@ __device__ __forceinline__ void tn_body(const T* __restrict__ A, const T* __rest
     const int t = row / r, rr = row - t * r;
     return (long)t * hA + hh * r + rr;
   };
-  // Copies of one stage.  When a stage is a whole number of time steps (TN_KT % r == 0) the folded rows of stage
+  // Copies of one stage.  When a stage is a whole number of time steps (KT % r == 0) the folded rows of stage
   // k+1 are those of stage k moved by a fixed distance: lane offsets are computed once, the base moves in scalar
   // registers.  Other shapes and the partial last stage take the general path.
-  const bool regular = (TN_KT % r) == 0;
+  const bool regular = (KT % r) == 0;
   static_assert(DK == DV, "the A and B tiles share the copy offsets");
   uint32_t voffA[LA], voffW = 0;
 #pragma unroll
@@ -113,12 +116,12 @@ __device__ __forceinline__ void tn_body(const T* __restrict__ A, const T* __rest
     voffA[ii] = (uint32_t)(row_index(row) * (DK * 2) + 16 * ((pos % CA) ^ swz<CA>(row)));
   }
   if (HAS_W) voffW = (uint32_t)(row_index(l) * 4);
-  const long stage_rows = (long)(TN_KT / max(r, 1)) * hA;   // rows of the [c, hA] arrays per stage (regular shapes)
+  const long stage_rows = (long)(KT / max(r, 1)) * hA;   // rows of the [c, hA] arrays per stage (regular shapes)
   const uint32_t smem_a = lds_addr(smem);
   auto issue = [&](int step) {
     const int slot = step % TN_NST;
-    const int r0 = step * TN_KT;
-    if (regular && r0 + TN_KT <= rows) {
+    const int r0 = step * KT;
+    if (regular && r0 + KT <= rows) {
       const uint32_t sa = smem_a + slot * STAGE + wave * 1024;
       const char* ab = a_base + step * stage_rows * (DK * 2);
       const char* bb = b_base + step * stage_rows * (DV * 2);
@@ -126,13 +129,13 @@ __device__ __forceinline__ void tn_body(const T* __restrict__ A, const T* __rest
       for (int ii = 0; ii < LA; ii++) async_copy16_sv(ab, voffA[ii], sa + ii * 4096);
 #pragma unroll
       for (int ii = 0; ii < LB; ii++) async_copy16_sv(bb, voffA[ii], sa + A_BYTES + ii * 4096);
-      if (HAS_W && wave == 0) async_copy4_sv(w_base + step * stage_rows, voffW, smem_a + slot * STAGE + A_BYTES + B_BYTES);
+      if (HAS_W && wave == 0 && l < KT) async_copy4_sv(w_base + step * stage_rows, voffW, smem_a + slot * STAGE + A_BYTES + B_BYTES);
       return;
     }
     char* st = smem + slot * STAGE;
-    async_load_tile<CA, TN_KT>(st, [&](int row) { return a_base + row_index(r0 + row) * (DK * 2); });
-    async_load_tile<CB, TN_KT>(st + A_BYTES, [&](int row) { return b_base + row_index(r0 + row) * (DV * 2); });
-    if (HAS_W && wave == 0) async_copy4(w_base + row_index(r0 + l), st + A_BYTES + B_BYTES);
+    async_load_tile<CA, KT>(st, [&](int row) { return a_base + row_index(r0 + row) * (DK * 2); });
+    async_load_tile<CB, KT>(st + A_BYTES, [&](int row) { return b_base + row_index(r0 + row) * (DV * 2); });
+    if (HAS_W && wave == 0 && l < KT) async_copy4(w_base + row_index(r0 + l), st + A_BYTES + B_BYTES);
   };
 
   f32x4 acc[XPW][NT];
@@ -215,13 +218,13 @@ __device__ __forceinline__ void tn_body(const T* __restrict__ A, const T* __rest
     }
   };
 
-  const int steps = (rows + TN_KT - 1) / TN_KT;
+  const int steps = (rows + KT - 1) / KT;
   if constexpr (PREFETCH) {
     issue(0);
     if (steps > 1) issue(1);
     if (steps > 2) issue(2);
     if (steps > 2) wait_vmcnt<2 * LOADS>(); else if (steps > 1) wait_vmcnt<LOADS>(); else wait_vmcnt<0>();
-    if (TN_KT > rows) zero_tile_rows<CA, TN_KT>(smem, rows);
+    if (KT > rows) zero_tile_rows<CA, KT>(smem, rows);
     lds_barrier();
     Frags F0, F1;
     load_frags(F0, IC<0>{}, IC<0>{});
@@ -236,7 +239,7 @@ __device__ __forceinline__ void tn_body(const T* __restrict__ A, const T* __rest
       const bool more = step + 1 < steps;
       if (more) {
         if (step + 2 < steps) wait_vmcnt<LOADS>(); else wait_vmcnt<0>();
-        if ((step + 2) * TN_KT > rows) zero_tile_rows<CA, TN_KT>(smem + NX * STAGE, rows - (step + 1) * TN_KT);
+        if ((step + 2) * KT > rows) zero_tile_rows<CA, KT>(smem + NX * STAGE, rows - (step + 1) * KT);
         lds_barrier();   // every wave holds the last fragments of this stage: its slot can be refilled
         if (step + 3 < steps) issue(step + 3);
         load_frags(F0, IC<NX>{}, IC<0>{});
@@ -258,11 +261,11 @@ __device__ __forceinline__ void tn_body(const T* __restrict__ A, const T* __rest
     for (int step = 0; step < steps; step++) {
       const char* st = smem + (step % TN_NST) * STAGE;
       if (step + 1 < steps) wait_vmcnt<LOADS>(); else wait_vmcnt<0>();
-      if ((step + 1) * TN_KT > rows) zero_tile_rows<CA, TN_KT>(smem + (step % TN_NST) * STAGE, rows - step * TN_KT);
+      if ((step + 1) * KT > rows) zero_tile_rows<CA, KT>(smem + (step % TN_NST) * STAGE, rows - step * KT);
       lds_barrier();
       if (step + 2 < steps) issue(step + 2);
 #pragma unroll 1
-      for (int ks = 0; ks < TN_KT / 32; ks++) {
+      for (int ks = 0; ks < KT / 32; ks++) {
         F.kfy = sw_frag_tr<T, CA>(st, 32 * ks, 16 * y);
         F.kfx = (xb == y) ? F.kfy : sw_frag_tr<T, CA>(st, 32 * ks, 16 * xb);
 #pragma unroll
@@ -532,8 +535,6 @@ __global__ __launch_bounds__(64 * NW, 2) void sympow_tn_chain_kernel(
 #undef PR_TN_CASE
 }
 
-constexpr int chain_stage_rows(int d) { return d <= 64 ? 64 : 32; }
-
 template <typename T, int DK, int DV>
 static int tn_chain_launch(const void* A, const void* Bm, const float* w, const float* lcs, void* S, float* s, int B,
                            int n, int c, int h, int r, int use_mult, int reverse, hipStream_t st) {
@@ -541,7 +542,7 @@ static int tn_chain_launch(const void* A, const void* Bm, const float* w, const 
   constexpr int NB = (DK / 16) * (DK / 16 + 1) / 2;
   constexpr int TASKS = NB * (16 / XPW);
   constexpr int NW = 4;                         // waves that share a stage of rows
-  constexpr int KT = chain_stage_rows(DV);      // rows per stage: two workgroups per compute unit must fit
+  constexpr int KT = tn_stage_rows(DV);      // rows per stage: two workgroups per compute unit must fit
   constexpr size_t smem = TN_NST * (KT * DK * 2 + KT * DV * 2 + KT * 4) + NW * 16 * (DV * 2 + 16);
   dim3 grid((TASKS + NW - 1) / NW, (unsigned)(B * h));
 #define PR_TN_CHAIN(W, R)                                                                                              \
@@ -564,7 +565,7 @@ static int tn_chain_launch(const void* A, const void* Bm, const float* w, const 
 // enough workgroups to fill the chip although the chunk axis is walked serially.
 int sympow_tn_chain_ok(int B, int n, int c, int h, int r, int d) {
   if (d != 32 && d != 64 && d != 128) return 0;
-  const int kt = chain_stage_rows(d);
+  const int kt = tn_stage_rows(d);
   if (n < 2 || r < 1 || kt % r != 0 || ((long)c * r) % kt != 0) return 0;
   const int xpw = d <= 64 ? 8 : 4;
   const long wgs = (long)B * h * (((d / 16) * (d / 16 + 1) / 2 * (16 / xpw) + 3) / 4);
@@ -576,7 +577,7 @@ int sympow_tn_chain_ok(int B, int n, int c, int h, int r, int d) {
 int sympow_tn_chain(const void* A, const void* Bm, const float* w, const float* lcs, void* S, float* s, int B, int n,
                     int c, int h, int r, int d, int use_mult, int reverse, int dtype, hipStream_t st) {
   if (d != 32 && d != 64 && d != 128) return -2;
-  if (n < 1 || r < 1 || chain_stage_rows(d) % r != 0 || ((long)c * r) % chain_stage_rows(d) != 0) return -3;
+  if (n < 1 || r < 1 || tn_stage_rows(d) % r != 0 || ((long)c * r) % tn_stage_rows(d) != 0) return -3;
 #define PR_TN_DISPATCH(T)                                                                                              \
   switch (d) {                                                                                                         \
     case 32: return tn_chain_launch<T, 32, 32>(A, Bm, w, lcs, S, s, B, n, c, h, r, use_mult, reverse, st);             \
@@ -596,7 +597,8 @@ static int tn_launch(const void* A, const void* Bm, const float* w, void* S, flo
   constexpr int XPW = DV <= 64 ? 8 : 4;
   constexpr int NB = (DK / 16) * (DK / 16 + 1) / 2;
   constexpr int TASKS = NB * (16 / XPW);
-  constexpr size_t smem = TN_NST * (TN_KT * DK * 2 + TN_KT * DV * 2 + TN_KT * 4);
+  constexpr int KT = tn_stage_rows(DV);
+  constexpr size_t smem = TN_NST * (KT * DK * 2 + KT * DV * 2 + KT * 4);
   dim3 grid((TASKS + 3) / 4, (unsigned)(BN * h));
   if (w) {
     auto kern = sympow_tn_kernel<T, DK, DV, XPW, true>;
