@@ -374,7 +374,8 @@ template <typename T, int DH, bool DEG2> static int attn_fwd_launch(const AttnFw
   };
   constexpr bool BIG = DH <= 32 || (DH <= 64 && DEG2);   // 64 rows per wave fit the register file
   if constexpr (BIG) {
-    if (rows >= 256) { go(IC<4>{}, IC<2>{}); return (int)hipGetLastError(); }
+    // (at d = 32 the 128-row tiling needs 123 registers: four workgroups per CU, 9 % faster than 256 rows at two)
+    if (rows >= 256 && DH > 32) { go(IC<4>{}, IC<2>{}); return (int)hipGetLastError(); }
   }
   if (rows > 64) go(IC<2>{}, IC<2>{});
   else go(IC<1>{}, IC<2>{});

@@ -317,16 +317,11 @@ template <typename T, int DK, int DV, bool MULT> static int grad_launch(const Gr
     allow_big_lds((const void*)kern, smem);
     hipLaunchKernelGGL(kern, grid, dim3(256), smem, st, a, row_blocks, npairs);
   };
-  if constexpr (DK <= 64) {
-    // 128 rows per workgroup at d = 64: half the reuse of a state tile, but four workgroups (16 waves) share a
-    // compute unit and the vector instructions of the two folds issue at twice the rate (measured 7 % faster than
-    // 256 rows at two workgroups)
-    if (rows >= 256 && DK < 64) { go(IC<4>{}); return (int)hipGetLastError(); }
-    if (rows > 64) { go(IC<2>{}); return (int)hipGetLastError(); }
-  } else {
-    // d = 128: a workgroup streams the whole 2.4 MB state from L2; 128 rows halve that traffic
-    if (rows > 64) { go(IC<2>{}); return (int)hipGetLastError(); }
-  }
+  // 128 rows per workgroup.  Up to d = 64 that is four workgroups (16 waves) per compute unit, and the vector
+  // instructions of the two folds issue at twice the rate of a 256-row tiling at two workgroups (measured 7 %
+  // faster at d = 64 although a state tile is reused half as often, equal at d = 32).  At d = 128 a workgroup
+  // streams the whole 2.4 MB state from L2, and 128 rows instead of 64 halve that traffic (27 % faster).
+  if (rows > 64) { go(IC<2>{}); return (int)hipGetLastError(); }
   go(IC<1>{});
   return (int)hipGetLastError();
 }
