@@ -312,7 +312,8 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dq_kernel(AttnBwdArgs a,
               q = (32 * kp + 16 * half + v <= lim[mi]) ? q : 0.f;
             }
             const float dsr = s * q;
-            dgq[mi] = DEG2 ? __builtin_fmaf(s, dsr, dgq[mi]) : __builtin_fmaf(__builtin_fmaf(s, s, eps2), q, dgq[mi]);
+            // dz = (s^2 + eps^2) q: the eps^2 part is all there is for a key with q.k = 0 (an all-zero key)
+            dgq[mi] = __builtin_fmaf(__builtin_fmaf(s, s, eps2), q, dgq[mi]);
             d8[4 * half + v] = dsr;
           }
         }
@@ -727,7 +728,7 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
               pw = a2 * E * fe[half][v];
             }
             const float dsr = s * q;
-            dgk[kj] = DEG2 ? __builtin_fmaf(s, dsr, dgk[kj]) : __builtin_fmaf(a2, q, dgk[kj]);
+            dgk[kj] = __builtin_fmaf(a2, q, dgk[kj]);
             p8[4 * half + v] = pw;
             d8[4 * half + v] = dsr;
           }

@@ -125,6 +125,8 @@ __global__ __launch_bounds__(256, OCC) void attention_fwd_kernel(AttnFwdArgs a, 
   long qoff[MT];
   bool live[MT];
   float Gq[MT], mx[MT];
+  constexpr bool TWO_PASS = sizeof(T) == 2 && !__is_same(T, bf16_t);   // fp16
+  float pn[MT], prow[MT];   // (second pass) 1 / row maximum, and that times the past tiles' row factor
 #pragma unroll
   for (int mi = 0; mi < MT; mi++) {
     const int row = wrow0 + 16 * mi + tcol;
@@ -222,8 +224,13 @@ __global__ __launch_bounds__(256, OCC) void attention_fwd_kernel(AttnFwdArgs a, 
   // One 64-key tile.  Past tiles use one reference gate (the tile's last key), so both gate factors are <= 1.
   // Diagonal tiles use the first key of every 16-key group instead: for every visible pair the row factor is
   // then <= 1 and the key factor spans only 16 steps of decay, so neither leaves the fp32 range.
-  auto tile = [&](int it, const char* st, auto diag_c) __attribute__((always_inline)) {
+  // MODE 0: weights in absolute terms, the row maximum divides the result at the end (bf16: its exponent range
+  // covers any row).  fp16 needs the reference's normalisation -- weights relative to the row maximum, <= 1 -- or
+  // a row whose largest weight is below 6e-8 would lose all of them: it runs the tiles twice, MODE 1 only for the
+  // row maxima (no V, no packing, no accumulation), then MODE 2 with every weight divided by its row's maximum.
+  auto tile = [&](int it, const char* st, auto diag_c, auto mode_c) __attribute__((always_inline)) {
     constexpr bool DIAG = decltype(diag_c)::value != 0;
+    constexpr int MODE = decltype(mode_c)::value;
     const int j0 = it * AT_BN;
     const float* graw = (const float*)(st + 2 * TILE);
     // LDS byte addresses of this lane's operands; opaque, so that the per-group and per-column-tile displacements
@@ -243,7 +250,7 @@ __global__ __launch_bounds__(256, OCC) void attention_fwd_kernel(AttnFwdArgs a, 
 #pragma unroll
     for (int mi = 0; mi < MT; mi++) {
       if (DIAG) lim[mi] = min(ti[mi], a.tk - 1) - j0 - 4 * g;   // pair (row, key 16*kt + 4g + v) visible iff 16*kt + v <= lim
-      else eu[mi] = 1.f;
+      else eu[mi] = MODE == 2 ? prow[mi] : 1.f;
     }
     // past tiles: key factors relative to the gate at the wave's first row (<= 1 for every past key)
     const float cw = DIAG ? 1.f : __expf(fminf(Rw - graw[AT_BN - 1], AT_EXP_CLAMP));
@@ -274,7 +281,7 @@ __global__ __launch_bounds__(256, OCC) void attention_fwd_kernel(AttnFwdArgs a, 
       // V^T operands for the same 32 keys, in flight while the weights are formed
       v8 vf[NT];
 #pragma unroll
-      for (int nt = 0; nt < NT; nt++) {
+      for (int nt = 0; MODE != 1 && nt < NT; nt++) {
         const uint32_t vp = vb[nt] + kp * 32 * RB;
         const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)vp);
         const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(vp + 16 * RB));
@@ -289,61 +296,92 @@ __global__ __launch_bounds__(256, OCC) void attention_fwd_kernel(AttnFwdArgs a, 
         for (int half = 0; half < 2; half++) {
           float e = eu[mi];
           if (DIAG) e = scale_p * __expf(fminf(Gq[mi] - graw[16 * (2 * kp + half)], AT_EXP_CLAMP));
+          if (DIAG && MODE == 2) e *= pn[mi];
 #pragma unroll
           for (int v = 0; v < 4; v++) {
             float w = pow_even<DEG2>(sc[half][mi][v], eps2, half_deg) * ev[half][v];
-            if (DIAG) w *= e;
+            if (DIAG || MODE == 2) w *= e;
             if (DIAG) w = (32 * kp + 16 * half + v <= lim[mi]) ? w : 0.f;
             p[4 * half + v] = w;
           }
         }
+        if (MODE != 2) {
 #pragma unroll
-        for (int e = 0; e < 8; e++) mx[mi] = fmaxf(mx[mi], p[e]);
-        pf[mi] = pack8<T>(p);
-      }
-      // O^T += V^T P^T over these 32 keys (elements 0-3 are keys 4g.. of the first 16, 4-7 of the second 16);
-      // the all-ones operand adds the row sums of the rounded weights
-#pragma unroll
-      for (int mi = 0; mi < MT; mi++) accl[mi] = mfma16(ones, pf[mi], accl[mi]);
-#pragma unroll
-      for (int nt = 0; nt < NT; nt++)
-#pragma unroll
-        for (int mi = 0; mi < MT; mi++) {
-          acc[mi][nt] = mfma16(vf[nt], pf[mi], acc[mi][nt]);
+          for (int e = 0; e < 8; e++) mx[mi] = fmaxf(mx[mi], p[e]);
         }
+        if (MODE != 1) pf[mi] = pack8<T>(p);
+      }
+      if constexpr (MODE != 1) {
+        // O^T += V^T P^T over these 32 keys (elements 0-3 are keys 4g.. of the first 16, 4-7 of the second 16);
+        // the all-ones operand adds the row sums of the rounded weights
+#pragma unroll
+        for (int mi = 0; mi < MT; mi++) accl[mi] = mfma16(ones, pf[mi], accl[mi]);
+#pragma unroll
+        for (int nt = 0; nt < NT; nt++)
+#pragma unroll
+          for (int mi = 0; mi < MT; mi++) {
+            acc[mi][nt] = mfma16(vf[nt], pf[mi], acc[mi][nt]);
+          }
+      }
     }
   };
 
-  int it = 0;
-  for (; it < n_past; it++) {
-    tile(it, sync_step(it), IC<0>{});
-    after_step(it);
-  }
-  // the past tiles were accumulated without the row factor exp(G_q - Rw) * scale^deg; apply it once
+  auto run_pass = [&](auto mode_c) __attribute__((always_inline)) {
+    constexpr int MODE = decltype(mode_c)::value;
+    int it = 0;
+    for (; it < n_past; it++) {
+      tile(it, sync_step(it), IC<0>{}, mode_c);
+      after_step(it);
+    }
+    // the past tiles were accumulated without the row factor exp(G_q - Rw) * scale^deg; apply it once
+    if constexpr (MODE != 2) {
 #pragma unroll
-  for (int mi = 0; mi < MT; mi++) {
-    const float f = scale_p * __expf(fminf(Gq[mi] - Rw, AT_EXP_CLAMP));
+      for (int mi = 0; mi < MT; mi++) {
+        const float f = scale_p * __expf(fminf(Gq[mi] - Rw, AT_EXP_CLAMP));
+        if (MODE == 0) {
 #pragma unroll
-    for (int nt = 0; nt < NT; nt++) acc[mi][nt] *= f;
-    accl[mi] *= f;
-    mx[mi] *= f;
-  }
-  for (; it < n_seen; it++) {
-    tile(it, sync_step(it), IC<1>{});
-    after_step(it);
-  }
-  for (; it < ntiles; it++) {
-    sync_step(it);
-    after_step(it);
+          for (int nt = 0; nt < NT; nt++) acc[mi][nt] *= f;
+          accl[mi] *= f;
+        }
+        mx[mi] *= f;
+      }
+    }
+    for (; it < n_seen; it++) {
+      tile(it, sync_step(it), IC<1>{}, mode_c);
+      after_step(it);
+    }
+    for (; it < ntiles; it++) {
+      sync_step(it);
+      after_step(it);
+    }
+  };
+  if constexpr (TWO_PASS) {
+    run_pass(IC<1>{});
+#pragma unroll
+    for (int mi = 0; mi < MT; mi++) {
+      mx[mi] = max_over_rows(mx[mi]);
+      pn[mi] = mx[mi] > 0.f ? 1.f / mx[mi] : 0.f;
+      prow[mi] = scale_p * __expf(fminf(Gq[mi] - Rw, AT_EXP_CLAMP)) * pn[mi];
+    }
+    lds_barrier();   // every wave is done with the ring: start the copies over
+    issue(0);
+    if (NST == 3 && ntiles > 1) issue(1);
+    if (wave == 0) {
+      wait_vmcnt<0>();
+      gate_factors(0);
+    }
+    run_pass(IC<2>{});
+  } else {
+    run_pass(IC<0>{});
   }
 
   T* Og = (T*)a.O + (long)b * a.tq * hq * DH;
 #pragma unroll
   for (int mi = 0; mi < MT; mi++) {
-    const float wmax = max_over_rows(mx[mi]);   // = exp(rowmax)
+    const float wmax = TWO_PASS ? mx[mi] : max_over_rows(mx[mi]);   // = exp(rowmax)
     if (!live[mi]) continue;
     const float wsum = accl[mi][0];             // every accumulator row of the all-ones product holds the row sum
-    const float inv = 1.f / wmax;
+    const float inv = TWO_PASS ? 1.f : 1.f / wmax;
     const float lrow = wsum * inv + AT_SUM_EPS;
     const float f = a.norm ? inv / lrow : inv;
 #pragma unroll

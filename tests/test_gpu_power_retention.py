@@ -252,6 +252,44 @@ def test_strong_gates(pra):
     run_both(pra, Q, K, V, lg.clamp(max=-0.01), chunk, dO)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("chunk", [None, 128])
+def test_rows_whose_every_weight_is_tiny(pra, dtype, chunk):
+    """Rows that see only keys with |q.k| ~ 1e-4 or exactly 0 (a first token orthogonal to its own key; leading
+    all-zero keys).  The reference normalises the weights by the row maximum before it rounds them to 16 bits
+    (retention/_attention/reference.py:50-52), so such a row is an exact average of the values it sees; in fp16 an
+    unnormalised weight of 1e-8 would round to zero.  Checked row by row, not as a norm over the tensor."""
+    b, t, h, r, d = 2, 256, 2, 2, 64
+    Q, K, V, lg = make_inputs(b, t, h, r, d, dtype, True, seed=51, std=0.5 if dtype == torch.float16 else 1.0)
+    Qf, Kf = Q.float(), K.float()
+    K0 = Kf[:, 0].repeat_interleave(r, dim=1)                       # [b, hq, d]
+    Qf[:, 0] -= (Qf[:, 0] * K0).sum(-1, keepdim=True) / (K0 * K0).sum(-1, keepdim=True) * K0   # q_0 orthogonal to k_0
+    Kf[1, :3] = 0.0                                                 # batch 1: the first three keys are zero
+    Q, K = Qf.to(dtype), Kf.to(dtype)
+    dO = torch.randn(b, t, h * r, d, generator=torch.Generator().manual_seed(52)).to(dtype)
+    xs = [x.to(DEV).requires_grad_(True) for x in (Q, K, V, lg)]
+    xo = [x.float().clone().requires_grad_(True) for x in (Q, K, V, lg)]
+    Y = pra.power_retention(*xs, deg=2, chunk_size=chunk)
+    Yo = oracle.power_retention(*xo, deg=2, chunk_size=chunk)
+    Y.backward(dO.to(DEV))
+    Yo.backward(dO.float())
+    row_err = (Y.float().cpu() - Yo).norm(dim=-1) / Yo.norm(dim=-1).clamp_min(1e-6)
+    print(f"  worst row of Y: {row_err.max().item():.3e} (rows 0-3: {row_err[:, :4].max().item():.3e})", flush=True)
+    assert row_err.max().item() <= 5e-2, "a row of Y is off"
+    # Gradients.  The orthogonal first row's own dQ and dK are left out of the norm: its output does not depend on
+    # its one weight, so they are a cancellation to ~0 (of dO.v against rowsum(O dO) with O rounded to 16 bits)
+    # multiplied by 1/|q.k| ~ 1e4 -- any run that keeps O in 16 bits leaves a residual there.  They must be finite.
+    for nm, x, o in zip(["dQ", "dK", "dV", "dlog_G"], xs, xo):
+        got, want = x.grad, o.grad
+        assert torch.isfinite(got.float()).all(), f"{nm}: non-finite values"
+        if nm in ("dQ", "dK"):
+            got, want = got[:, 1:], want[:, 1:]
+        check(nm, got, want, GRAD_TOL)
+    # the gate gradient of the rows that see only all-zero keys comes from the eps term of the weights alone
+    got, want = xs[3].grad[1, 1:3].float().cpu(), xo[3].grad[1, 1:3]
+    assert torch.allclose(got, want, rtol=5e-2, atol=1e-3), (got, want)
+
+
 def test_fp32_inputs_are_rejected_loudly(pra):
     Q, K, V, lg = make_inputs(1, 256, 1, 1, 64, torch.float32, True)
     with pytest.raises((AssertionError, TypeError, RuntimeError)):
