@@ -410,11 +410,9 @@ template <typename T, int DH, bool DEG2> static int attn_fwd_launch(const AttnFw
     allow_big_lds((const void*)kern, smem);
     hipLaunchKernelGGL(kern, grid, dim3(256), smem, st, a, row_blocks, npairs);
   };
-  constexpr bool BIG = DH <= 32 || (DH <= 64 && DEG2);   // 64 rows per wave fit the register file
-  if constexpr (BIG) {
-    // (at d = 32 the 128-row tiling needs 123 registers: four workgroups per CU, 9 % faster than 256 rows at two)
-    if (rows >= 256 && DH > 32) { go(IC<4>{}, IC<2>{}); return (int)hipGetLastError(); }
-  }
+  // 128 rows per workgroup: 123 registers at d = 32 (four workgroups per CU), 166 at d = 64 (three); measured 9 % and
+  // 6 % faster than 256 rows at two workgroups -- the kernel is mostly vector work, which issues faster with more
+  // waves resident, and that outweighs streaming K and V twice as often
   if (rows > 64) go(IC<2>{}, IC<2>{});
   else go(IC<1>{}, IC<2>{});
   return (int)hipGetLastError();
