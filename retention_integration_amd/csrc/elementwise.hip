@@ -38,21 +38,29 @@ __global__ __launch_bounds__(256) void qs_bwd_prep_kernel(const T* __restrict__ 
     wq = scale_p * __expf(-beta);
   }
   if (!live) return;
+  // Row factors of the two parts.  They are ~1e-3..1 unless the row's total weight is ~0 (a zero query: 1/den is
+  // then ~1e14 and multiplies a feature vector that is exactly zero).  fp16 cannot hold dO times such a factor, so
+  // there it is capped far above any regular value; the products with the zero features stay zero instead of NaN.
+  float cq = wq * f, ca = wa * f;
+  if (!__is_same(T, bf16_t)) {
+    cq = fminf(cq, 4096.f);
+    ca = fminf(ca, 4096.f);
+  }
   float a[8], b[8];
 #pragma unroll
   for (int i = 0; i < 8; i++) {
-    a[i] = g[i] * (wq * f);
-    b[i] = g[i] * (wa * f);
+    a[i] = g[i] * cq;
+    b[i] = g[i] * ca;
   }
   *(v8*)(dOs + r * DH + col) = pack8<T>(a);
   if (dYa) *(v8*)(dYa + r * DH + col) = pack8<T>(b);
   if (col == 0) {
-    cvec[r] = -wq * f * delta;
-    if (dla) dla[r] = -wa * f * delta;
+    cvec[r] = -cq * delta;
+    if (dla) dla[r] = -ca * delta;
     // dY_attn = dO * dYscale[row], for consumers that scale on the fly.  The factor is <= 1/l_attn, i.e. <= ~1 unless
     // every weight of the row underflowed (a zero query, e.g. a padded row, in fp16: l_attn = 1e-6); it is capped so
     // that weight * factor stays inside the fp16 range there too.
-    if (dYscale) dYscale[r] = fminf(wa * f, 3.0e4f);
+    if (dYscale) dYscale[r] = fminf(ca, 3.0e4f);
   }
 }
 

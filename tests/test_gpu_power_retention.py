@@ -265,6 +265,8 @@ def test_rows_whose_every_weight_is_tiny(pra, dtype, chunk):
     K0 = Kf[:, 0].repeat_interleave(r, dim=1)                       # [b, hq, d]
     Qf[:, 0] -= (Qf[:, 0] * K0).sum(-1, keepdim=True) / (K0 * K0).sum(-1, keepdim=True) * K0   # q_0 orthogonal to k_0
     Kf[1, :3] = 0.0                                                 # batch 1: the first three keys are zero
+    Qf[0, 5] = 0.0                                                  # a zero query: every weight is the eps term
+    Qf[1, 200] = 0.0                                                # ... also deep inside a later chunk
     Q, K = Qf.to(dtype), Kf.to(dtype)
     dO = torch.randn(b, t, h * r, d, generator=torch.Generator().manual_seed(52)).to(dtype)
     xs = [x.to(DEV).requires_grad_(True) for x in (Q, K, V, lg)]
