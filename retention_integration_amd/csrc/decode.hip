@@ -42,18 +42,69 @@ struct DecodeArgs {
   const float* decay;   // [B, h] log of the decay applied to the old state, or null (= 0)
   void* Sout;           // [B, h, D, d]
   float* sout;          // [B, h, D]
-  float* part;          // [B*h, split, rows, d + 1] partial query sums
+  float* part;          // [B*h, split, rows, d + 1] partial query sums (unused when one workgroup owns a pair)
   int h, r, tq, split, deg;
+  // the merge with the attention part
+  const void* Y_attn;   // [B, tq, h*r, d] or null
+  const float* l_attn;  // [B, tq, h*r]
+  const float* rowmax;  // [B, tq, h*r]
+  void* out;            // [B, tq, h*r, d]
+  float scale_p;
+  int attend_new;       // the attention part is the one new token attending to itself
 };
 
-template <typename T, int DH>
-__global__ __launch_bounds__(256) void decode_step_kernel(DecodeArgs a) {
-  typedef typename VecOf<T>::v8 v8;
-  constexpr int LPR = DH / 8, FPP = 256 / LPR;            // lanes per feature row, feature rows per pass
+// out[row, e] = (Y_attn * wa + y * wq) / (l_attn * wa + lq * wq), the merge of the chunked kernel
+// (sympow_nn.hip); without an attention part out = y / lq.  Run by one wave; y(e) gives the query sums.
+// With Qn/Kn/Vn the attention part is that of the ONE new token attending to itself (tq = 1): one weight
+// (scale q.k)^deg, so Y_attn = v, l_attn = 1 + 1e-6 and rowmax = log of the weight
+// (ref: retention/_attention/reference.py:42-69 with a single key).
+template <typename T, int DH, typename YF>
+__device__ __forceinline__ void decode_merge_row(int lane, YF y, float lq, const T* __restrict__ Y_attn,
+                                                 const float* __restrict__ l_attn, const float* __restrict__ rowmax,
+                                                 const T* __restrict__ Qn, const T* __restrict__ Kn,
+                                                 const T* __restrict__ Vn, T* __restrict__ out, long ro, int pair,
+                                                 float scale_p, float deg) {
   constexpr int D = 128 * (DH / 16) * (DH / 16 + 1);
-  __shared__ float qs[DEC_MAXROWS][DH];
+  float wa = 0.f, wq = 1.f, la = 0.f;
+  const T* ya = Y_attn ? Y_attn + ro * DH : nullptr;
+  if (Kn) {
+    float dot = 0.f;
+    for (int e = lane; e < DH; e += 64) dot += (float)Qn[ro * DH + e] * (float)Kn[(long)pair * DH + e];
+    dot = sum_over_rows(sum_in_row(dot));
+    const float scale = __expf(__logf(scale_p) / deg), eps = 1e-7f / scale;
+    const float m = 0.5f * deg * __logf(dot * dot + eps * eps) + __logf(scale_p);
+    const float beta = fmaxf(m, 0.5f * __logf((float)D));
+    la = 1.f + 1e-6f;
+    wa = __expf(m - beta);
+    wq = scale_p * __expf(-beta);
+    ya = Vn + (long)pair * DH;
+  } else if (Y_attn) {
+    const float m = rowmax[ro], beta = fmaxf(m, 0.5f * __logf((float)D));
+    la = l_attn[ro];
+    wa = __expf(m - beta);
+    wq = scale_p * __expf(-beta);
+  }
+  const float inv = 1.f / (la * wa + lq * wq);
+  for (int e = lane; e < DH; e += 64) {
+    float num = y(e) * wq;
+    if (ya) num += (float)ya[e] * wa;
+    out[ro * DH + e] = (T)(num * inv);
+  }
+}
+
+// One workgroup of NTHR threads streams the feature rows [f_lo, f_hi) of one (batch, kv head).
+// WHOLE: the workgroup owns every feature of its pair and merges the result itself; otherwise it writes the
+// partial sums of its slice for decode_merge_kernel.
+template <typename T, int DH, int MAXR, int NTHR, bool WHOLE>
+__global__ __launch_bounds__(NTHR) void decode_step_kernel(DecodeArgs a) {
+  typedef typename VecOf<T>::v8 v8;
+  constexpr int LPR = DH / 8, FPP = NTHR / LPR;            // lanes per feature row, feature rows per pass
+  constexpr int RPW = 64 / LPR, NW = NTHR / 64;            // feature rows per wave and pass, waves
+  constexpr int D = 128 * (DH / 16) * (DH / 16 + 1);
+  __shared__ float qs[MAXR][DH];
   __shared__ float ks[DH];
-  __shared__ float red[FPP][DH + 1];
+  __shared__ float red[NW][DH + 1];
+  __shared__ float tot[DH + 1];
 
   const int pair = blockIdx.x, sp = blockIdx.y;
   const int b = pair / a.h, hh = pair % a.h;
@@ -63,29 +114,29 @@ __global__ __launch_bounds__(256) void decode_step_kernel(DecodeArgs a) {
 
   // gated, rounded query rows and the new key in LDS as floats
   const float qg = a.gq ? __expf(a.gq[b * a.h + hh] / (float)a.deg) : 1.f;
-  for (int i = tid; i < rows * DH; i += 256) {
+  for (int i = tid; i < rows * DH; i += NTHR) {
     const int row = i / DH, e = i % DH, t = row / a.r, rr = row % a.r;
     const float q = (float)((const T*)a.Q)[(((long)b * a.tq + t) * hq + hh * a.r + rr) * DH + e];
     qs[row][e] = (float)(T)(q * qg);
   }
   if (upd)
-    for (int i = tid; i < DH; i += 256) ks[i] = (float)((const T*)a.Knew)[((long)b * a.h + hh) * DH + i];
+    for (int i = tid; i < DH; i += NTHR) ks[i] = (float)((const T*)a.Knew)[((long)b * a.h + hh) * DH + i];
   __syncthreads();
 
   const float dec = (upd && a.decay) ? __expf(a.decay[b * a.h + hh]) : 1.f;
   float vnew[8];
   if (upd) unpack8(*(const v8*)((const T*)a.Vnew + ((long)b * a.h + hh) * DH + 8 * sub), vnew);
 
-  const int per = (D + a.split - 1) / a.split;
-  const int f_lo = sp * per, f_hi = min(D, f_lo + per);
+  const int per = WHOLE ? D : (D + a.split - 1) / a.split;
+  const int f_lo = WHOLE ? 0 : sp * per, f_hi = min(D, f_lo + per);
   const T* Sg = (const T*)a.S + (long)pair * D * DH;
   T* So = upd ? (T*)a.Sout + (long)pair * D * DH : nullptr;
   const float* sg = a.s + (long)pair * D;
   float* so = upd ? a.sout + (long)pair * D : nullptr;
 
-  float acc[DEC_MAXROWS][8], lq[DEC_MAXROWS];
+  float acc[MAXR][8], lq[MAXR];
 #pragma unroll
-  for (int r_ = 0; r_ < DEC_MAXROWS; r_++) {
+  for (int r_ = 0; r_ < MAXR; r_++) {
     lq[r_] = 0.f;
 #pragma unroll
     for (int i = 0; i < 8; i++) acc[r_][i] = 0.f;
@@ -111,7 +162,7 @@ __global__ __launch_bounds__(256) void decode_step_kernel(DecodeArgs a) {
       float sv[8];
       unpack8(raw[u], sv);
 #pragma unroll
-      for (int r_ = 0; r_ < DEC_MAXROWS; r_++) {
+      for (int r_ = 0; r_ < MAXR; r_++) {
         if (r_ < rows) {
           const float ph = qs[r_][x] * qs[r_][w];
 #pragma unroll
@@ -130,94 +181,108 @@ __global__ __launch_bounds__(256) void decode_step_kernel(DecodeArgs a) {
     }
   }
 
-  // reduce over the FPP feature-row groups of the workgroup, one query row at a time
-  float* part = a.part + ((long)pair * a.split + sp) * rows * (DH + 1);
+  // Sum over the feature rows: first over the RPW rows a wave holds (lanes LPR apart), then over the waves through
+  // LDS, one query row at a time.
   // (compile-time row index: a run-time index would put the accumulators in scratch memory for the whole kernel)
+  const int wave = tid >> 6, lane = tid & 63;
+  float* part = WHOLE ? nullptr : a.part + ((long)pair * a.split + sp) * rows * (DH + 1);
 #pragma unroll
-  for (int r_ = 0; r_ < DEC_MAXROWS; r_++) {
+  for (int r_ = 0; r_ < MAXR; r_++) {
     if (r_ < rows) {
-      __syncthreads();
+      float v[9];
 #pragma unroll
-      for (int i = 0; i < 8; i++) red[fr][8 * sub + i] = acc[r_][i];
-      if (sub == 0) red[fr][DH] = lq[r_];
+      for (int i = 0; i < 8; i++) v[i] = acc[r_][i];
+      v[8] = lq[r_];
+#pragma unroll
+      for (int off = LPR; off < 64; off <<= 1)
+#pragma unroll
+        for (int i = 0; i < 9; i++) v[i] += __shfl_xor(v[i], off);
+      __syncthreads();   // red and tot of the previous row have been read
+      if (lane < LPR) {
+#pragma unroll
+        for (int i = 0; i < 8; i++) red[wave][8 * lane + i] = v[i];
+        if (lane == 0) red[wave][DH] = v[8];
+      }
       __syncthreads();
       if (tid <= DH) {
         float t = 0.f;
-        for (int k = 0; k < FPP; k++) t += red[k][tid];
-        part[r_ * (DH + 1) + tid] = t;
+#pragma unroll
+        for (int k = 0; k < NW; k++) t += red[k][tid];
+        if (WHOLE) tot[tid] = t;
+        else part[r_ * (DH + 1) + tid] = t;
+      }
+      if (WHOLE) {
+        __syncthreads();
+        if (wave == 0) {
+          const int t = r_ / a.r, rr = r_ % a.r;
+          const long ro = ((long)b * a.tq + t) * hq + hh * a.r + rr;
+          const bool an = a.attend_new != 0;
+          decode_merge_row<T, DH>(lane, [&](int e) { return tot[e]; }, tot[DH], (const T*)a.Y_attn, a.l_attn,
+                                  a.rowmax, an ? (const T*)a.Q : nullptr, an ? (const T*)a.Knew : nullptr,
+                                  an ? (const T*)a.Vnew : nullptr, (T*)a.out, ro, pair, a.scale_p, (float)a.deg);
+        }
       }
     }
   }
 }
 
-// out[row, e] = (Y_attn * wa + y * wq) / (l_attn * wa + lq * wq), the merge of the chunked kernel
-// (sympow_nn.hip); without an attention part out = y / lq.
-// With Qn/Kn/Vn the attention part is that of the ONE new token attending to itself (tq = 1): one weight
-// (scale q.k)^deg, so Y_attn = v, l_attn = 1 + 1e-6 and rowmax = log of the weight
-// (ref: retention/_attention/reference.py:42-69 with a single key).
+// Adds the partial sums of the feature slices of a (batch, kv head) and merges: one wave per query row.
 template <typename T, int DH>
-__global__ __launch_bounds__(64) void decode_merge_kernel(const float* __restrict__ part, const T* __restrict__ Y_attn,
-                                                          const float* __restrict__ l_attn,
-                                                          const float* __restrict__ rowmax, const T* __restrict__ Qn,
-                                                          const T* __restrict__ Kn, const T* __restrict__ Vn,
-                                                          T* __restrict__ out, int h, int r, int tq, int split,
-                                                          float scale_p, float deg) {
-  constexpr int D = 128 * (DH / 16) * (DH / 16 + 1);
-  const int pair = blockIdx.x, row = blockIdx.y, rows = tq * r, hq = h * r;
-  const int b = pair / h, hh = pair % h, t = row / r, rr = row % r;
-  const long ro = ((long)b * tq + t) * hq + hh * r + rr;
-  const float* p = part + (long)pair * split * rows * (DH + 1) + row * (DH + 1);
+__global__ __launch_bounds__(64) void decode_merge_kernel(DecodeArgs a) {
+  const int pair = blockIdx.x, row = blockIdx.y, rows = a.tq * a.r, hq = a.h * a.r;
+  const int b = pair / a.h, hh = pair % a.h, t = row / a.r, rr = row % a.r;
+  const long ro = ((long)b * a.tq + t) * hq + hh * a.r + rr;
+  const int split = a.split;
+  const float* p = a.part + (long)pair * split * rows * (DH + 1) + row * (DH + 1);
   float lq = 0.f;
   for (int k = 0; k < split; k++) lq += p[(long)k * rows * (DH + 1) + DH];
-  float wa = 0.f, wq = 1.f, la = 0.f;
-  const T* ya = Y_attn ? Y_attn + ro * DH : nullptr;
-  if (Kn) {
-    float dot = 0.f;
-    for (int e = threadIdx.x; e < DH; e += 64) dot += (float)Qn[ro * DH + e] * (float)Kn[(long)pair * DH + e];
-    dot = sum_over_rows(sum_in_row(dot));
-    const float scale = __expf(__logf(scale_p) / deg), eps = 1e-7f / scale;
-    const float m = 0.5f * deg * __logf(dot * dot + eps * eps) + __logf(scale_p);
-    const float beta = fmaxf(m, 0.5f * __logf((float)D));
-    la = 1.f + 1e-6f;
-    wa = __expf(m - beta);
-    wq = scale_p * __expf(-beta);
-    ya = Vn + (long)pair * DH;
-  } else if (Y_attn) {
-    const float m = rowmax[ro], beta = fmaxf(m, 0.5f * __logf((float)D));
-    la = l_attn[ro];
-    wa = __expf(m - beta);
-    wq = scale_p * __expf(-beta);
-  }
-  const float inv = 1.f / (la * wa + lq * wq);
-  for (int e = threadIdx.x; e < DH; e += 64) {
-    float y = 0.f;
-    for (int k = 0; k < split; k++) y += p[(long)k * rows * (DH + 1) + e];
-    float num = y * wq;
-    if (ya) num += (float)ya[e] * wa;
-    out[ro * DH + e] = (T)(num * inv);
-  }
+  const bool an = a.attend_new != 0;
+  decode_merge_row<T, DH>(
+      threadIdx.x,
+      [&](int e) {
+        float y = 0.f;
+        for (int k = 0; k < split; k++) y += p[(long)k * rows * (DH + 1) + e];
+        return y;
+      },
+      lq, (const T*)a.Y_attn, a.l_attn, a.rowmax, an ? (const T*)a.Q : nullptr, an ? (const T*)a.Knew : nullptr,
+      an ? (const T*)a.Vnew : nullptr, (T*)a.out, ro, pair, a.scale_p, (float)a.deg);
 }
 
 int decode_split(int B, int h) {
-  // enough workgroups to fill the chip a few times over, at most 16 slices per (batch, kv head)
+  // about a thousand workgroups of 256 threads (four per compute unit, resident together); at most 16 slices per
+  // (batch, kv head)
   const int pairs = B * h;
-  int split = (2048 + pairs - 1) / pairs;
+  const int split = (1024 + pairs - 1) / pairs;
   return split < 1 ? 1 : (split > 16 ? 16 : split);
 }
 long decode_workspace_floats(int B, int h, int r, int tq, int d) {
   return (long)B * h * decode_split(B, h) * tq * r * (d + 1);
 }
 
+// With at least one (batch, kv head) per compute unit and few query rows, one workgroup of 1024 threads takes a whole
+// pair and merges in the same kernel (no partial sums, no second launch).
+static bool decode_whole_pair(int B, int h, int rows) { return B * h >= 256 && rows <= 2; }
+
 template <typename T, int DH>
-static int decode_launch(const DecodeArgs& a0, const void* Y_attn, const float* l_attn, const float* rowmax, void* out,
-                         int B, float scale_p, int attend_new, hipStream_t st) {
+static int decode_launch(const DecodeArgs& a0, int B, hipStream_t st) {
   DecodeArgs a = a0;
+  const int rows = a.tq * a.r;
+  // the accumulators of all query rows live in registers: a kernel per power of two keeps the common single-row
+  // step small
+  if (decode_whole_pair(B, a.h, rows)) {
+    a.split = 1;
+    const dim3 grid((unsigned)(B * a.h));
+    if (rows <= 1) hipLaunchKernelGGL((decode_step_kernel<T, DH, 1, 1024, true>), grid, dim3(1024), 0, st, a);
+    else hipLaunchKernelGGL((decode_step_kernel<T, DH, 2, 1024, true>), grid, dim3(1024), 0, st, a);
+    return (int)hipGetLastError();
+  }
   a.split = decode_split(B, a.h);
-  hipLaunchKernelGGL((decode_step_kernel<T, DH>), dim3((unsigned)(B * a.h), (unsigned)a.split), dim3(256), 0, st, a);
-  hipLaunchKernelGGL((decode_merge_kernel<T, DH>), dim3((unsigned)(B * a.h), (unsigned)(a.tq * a.r)), dim3(64), 0, st,
-                     a.part, (const T*)Y_attn, l_attn, rowmax, attend_new ? (const T*)a.Q : nullptr,
-                     attend_new ? (const T*)a.Knew : nullptr, attend_new ? (const T*)a.Vnew : nullptr, (T*)out, a.h,
-                     a.r, a.tq, a.split, scale_p, (float)a.deg);
+  const dim3 grid((unsigned)(B * a.h), (unsigned)a.split);
+  if (rows <= 1) hipLaunchKernelGGL((decode_step_kernel<T, DH, 1, 256, false>), grid, dim3(256), 0, st, a);
+  else if (rows <= 2) hipLaunchKernelGGL((decode_step_kernel<T, DH, 2, 256, false>), grid, dim3(256), 0, st, a);
+  else if (rows <= 4) hipLaunchKernelGGL((decode_step_kernel<T, DH, 4, 256, false>), grid, dim3(256), 0, st, a);
+  else hipLaunchKernelGGL((decode_step_kernel<T, DH, DEC_MAXROWS, 256, false>), grid, dim3(256), 0, st, a);
+  hipLaunchKernelGGL((decode_merge_kernel<T, DH>), dim3((unsigned)(B * a.h), (unsigned)rows), dim3(64), 0, st, a);
   return (int)hipGetLastError();
 }
 
@@ -226,12 +291,13 @@ int decode_step(const void* Q, const float* gq, const void* S, const float* s, c
                 void* out, float* workspace, int B, int tq, int h, int r, int d, int deg, float scale_p, int dtype,
                 int attend_new, hipStream_t st) {
   if (tq * r > DEC_MAXROWS) return -3;
-  DecodeArgs a{Q, gq, S, s, Knew, Vnew, decay, Sout, sout, workspace, h, r, tq, 1, deg};
+  DecodeArgs a{Q, gq, S, s, Knew, Vnew, decay, Sout, sout, workspace, h, r, tq, 1, deg,
+               Y_attn, l_attn, rowmax, out, scale_p, attend_new};
 #define PR_DEC(T)                                                                                                      \
   switch (d) {                                                                                                         \
-    case 32: return decode_launch<T, 32>(a, Y_attn, l_attn, rowmax, out, B, scale_p, attend_new, st);                              \
-    case 64: return decode_launch<T, 64>(a, Y_attn, l_attn, rowmax, out, B, scale_p, attend_new, st);                              \
-    case 128: return decode_launch<T, 128>(a, Y_attn, l_attn, rowmax, out, B, scale_p, attend_new, st);                            \
+    case 32: return decode_launch<T, 32>(a, B, st);                                                                    \
+    case 64: return decode_launch<T, 64>(a, B, st);                                                                    \
+    case 128: return decode_launch<T, 128>(a, B, st);                                                                  \
     default: return -2;                                                                                                \
   }
   if (dtype == DT_BF16) { PR_DEC(bf16_t) }

@@ -467,3 +467,51 @@ def test_decode_step_in_place_through_the_c_abi(pra):
     _lib.check(lib.pr_decode_step(p(Q), p(lg), p(Si), p(si), None, None, None, p(K), p(V), p(lg), p(Si), p(si), p(oi),
                                   p(ws), b, 1, h, r, d, 0.125 ** 2, 2, _lib.dtype_code(dt), 1, st), "decode_step")
     assert torch.equal(oi, out) and torch.equal(Si, S2) and torch.equal(si, s2)
+
+
+@pytest.mark.parametrize("dtype,d,r,mode", [(torch.bfloat16, 64, 1, "new"), (torch.bfloat16, 64, 2, "cache"),
+                                            (torch.float16, 128, 1, "new"), (torch.bfloat16, 32, 2, "state"),
+                                            (torch.bfloat16, 64, 4, "new")])
+def test_decode_step_large_batch_equals_small_batches(pra, dtype, d, r, mode):
+    """With at least 256 (batch, kv head) pairs and at most two query rows the decode step runs as one kernel with a
+    workgroup per pair; smaller batches (and more rows: the r = 4 case) slice the features and merge in a second
+    kernel, the form the other tests pin to the oracle.  The same rows must come out of both, and the oracle's
+    recurrent step (ref: retention/power_retention_maker.py:358-382) must agree on a slice."""
+    from retention_integration_amd import ops
+    b, h, t0 = 32, 8, 64
+    std = 0.5 if dtype == torch.float16 else 1.0
+    Q, K, V, lg = make_inputs(b, t0 + 1, h, r, d, dtype, True, seed=77 + d + r, std=std)
+    Q, K, V, lg = (x.to(DEV) for x in (Q, K, V, lg))
+    S, s = pra.update_state(K[:, :t0].contiguous(), V[:, :t0].contiguous(), 2)
+    q = Q[:, t0:].contiguous()
+    kn, vn, g1 = K[:, t0].contiguous(), V[:, t0].contiguous(), lg[:, t0].contiguous()
+    gen = torch.Generator().manual_seed(5)
+    hq = h * r
+    scale_p = (1.0 / d ** 0.5) ** 2
+    if mode == "new":
+        args = lambda i: (q[i], g1[i], S[i], s[i], None, None, None, kn[i], vn[i], g1[i], scale_p, True)  # noqa: E731
+    elif mode == "cache":
+        Ya = torch.randn(b, 1, hq, d, generator=gen).to(dtype).to(DEV)
+        la = (torch.rand(b, 1, hq, generator=gen) + 0.5).to(DEV)
+        rm = torch.randn(b, 1, hq, generator=gen).to(DEV)
+        args = lambda i: (q[i], g1[i], S[i], s[i], Ya[i], la[i], rm[i], None, None, None, scale_p, False)  # noqa: E731
+    else:
+        args = lambda i: (q[i], None, S[i], s[i], None, None, None, None, None, None, scale_p, False)  # noqa: E731
+    out, S2, s2 = ops.decode_step(*args(slice(None)))
+    assert torch.isfinite(out.float()).all()
+    for sl in (slice(0, 3), slice(b - 3, b)):
+        o_s, S_s, s_s = ops.decode_step(*[x.contiguous() if torch.is_tensor(x) else x for x in args(sl)])
+        check(f"rows {sl.start}:{sl.stop} out", out[sl], o_s, 2e-3)
+        if mode == "new":
+            # same arithmetic element by element; in fp16 the compiler may fuse the final rounding into the multiply-add
+            # in one kernel and not in the other (a last-bit difference in a few elements per million)
+            check(f"rows {sl.start}:{sl.stop} state", S2[sl], S_s, 1e-4)
+            assert torch.equal(s2[sl], s_s)
+    if mode == "new":
+        sl = slice(0, 2)
+        f = lambda x: x[sl].float().cpu()  # noqa: E731
+        Yo, So, so = oracle.power_retention_inference(f(q), f(K[:, t0:]), f(V[:, t0:]), lg[sl, t0:].cpu(), f(S), f(s),
+                                                      deg=2, switch_over_seq_len=1)
+        check("oracle out", out[sl], Yo, OUT_TOL)
+        check("oracle state", S2[sl], So, OUT_TOL)
+        check("oracle sum_of_keys", s2[sl], so, OUT_TOL)
