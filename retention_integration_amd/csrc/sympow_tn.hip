@@ -42,6 +42,72 @@ template <int X> struct PhiTile<f16_t, X> {
   }
 };
 
+// Diagonal feature blocks (xb == y) hold every product of the strip's 16 columns twice, (a, b) and (b, a), with equal
+// sums.  They are therefore computed along the cyclic diagonals: fragment J holds a[i] * a[(i - J) mod 16] in lane i
+// (a row rotation instead of a row broadcast, still one vector op per element); J = 0..8 covers every unordered pair
+// (J = 8 covers its eight pairs twice), nine fragments instead of sixteen, and every sum is stored at both places.
+template <int J> __device__ __forceinline__ float mul_row_ror(float src, float row) {
+  if constexpr (J == 0) return src * row;
+  float r;
+  asm("v_mul_f32_dpp %0, %1, %2 row_ror:%3 row_mask:0xf bank_mask:0xf" : "=v"(r) : "v"(src), "v"(row), "n"(J));
+  return r;
+}
+template <typename T, int J> struct PhiDiag;
+template <int J> struct PhiDiag<bf16_t, J> {
+  static __device__ __forceinline__ bf16x8 make(const bf16x8&, const float* rowf) {
+    float p[8];
+#pragma unroll
+    for (int r = 0; r < 8; r++) p[r] = mul_row_ror<J>(rowf[r], rowf[r]);
+    return pack8<bf16_t>(p);
+  }
+};
+template <int J> struct PhiDiag<f16_t, J> {
+  static __device__ __forceinline__ f16x8 make(const f16x8& rows, const float*) {
+    if constexpr (J == 0) return rows * rows;
+    u32x4 u = __builtin_bit_cast(u32x4, rows), b;
+#pragma unroll
+    for (int i = 0; i < 4; i++) b[i] = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)u[i], 0x120 + J, 0xf, 0xf, true);
+    return rows * __builtin_bit_cast(f16x8, b);
+  }
+};
+constexpr int TN_NDIAG = 9;   // fragments of a diagonal block
+
+// The diagonal block's counterpart of tn_store_rows below: fragment J's row i is feature (i, i') with
+// i' = (i - J) mod 16, stored at 16 i + i' and at 16 i' + i.  S, s point at the block's first feature.
+template <typename T, int DV>
+__device__ __forceinline__ void tn_store_diag(const f32x4 (&acc)[TN_NDIAG][DV / 16], const f32x4& sacc, uint32_t tb,
+                                              T* __restrict__ S, float* __restrict__ s) {
+  typedef __attribute__((address_space(3))) unsigned short lds_u16;
+  typedef __attribute__((address_space(3))) u32x4 lds_u32x4;
+  constexpr int NT = DV / 16, TP = DV * 2 + 16;
+  const int l = lane_id(), g = l >> 4, sl = l & 15;
+  const uint32_t tb_w = tb + 4 * g * TP + sl * 2;
+  static_for<TN_NDIAG>([&](auto ji) {
+    constexpr int J = decltype(ji)::value;
+#pragma unroll
+    for (int nt = 0; nt < NT; nt++) {
+      float o[4];
+#pragma unroll
+      for (int v = 0; v < 4; v++) o[v] = acc[J][nt][v];
+      const u32x2 pk = __builtin_bit_cast(u32x2, pack4<T>(o));
+      *(lds_u16*)(tb_w + 32 * nt) = (unsigned short)pk[0];
+      *(lds_u16*)(tb_w + 32 * nt + TP) = (unsigned short)(pk[0] >> 16);
+      *(lds_u16*)(tb_w + 32 * nt + 2 * TP) = (unsigned short)pk[1];
+      *(lds_u16*)(tb_w + 32 * nt + 3 * TP) = (unsigned short)(pk[1] >> 16);
+    }
+    asm volatile("" ::: "memory");   // (LDS operations of one wave execute in order)
+#pragma unroll
+    for (int j = 0; j < DV / 32; j++) {
+      const int q = j * 1024 + l * 16, i = q / (DV * 2), col = q % (DV * 2), i2 = (i - J) & 15;
+      const u32x4 v = *(const lds_u32x4*)(tb + i * TP + col);
+      *(u32x4*)((char*)S + (16 * i + i2) * (DV * 2) + col) = v;
+      if (J != 0 && J != 8) *(u32x4*)((char*)S + (16 * i2 + i) * (DV * 2) + col) = v;
+    }
+    asm volatile("" ::: "memory");   // the buffer is rewritten for the next fragment
+  });
+  *(f32x4*)(s + 16 * sl + 4 * g) = sacc;
+}
+
 // Writes a wave's accumulators -- for each of its XPW x values the 16 feature rows (4g+v) x DV value columns
 // (16nt + lane%16) of S, times mul -- and its key sums.  Each x goes through a per-wave LDS buffer of 16 padded rows
 // (tb, 16 * (2 DV + 16) bytes) so that the tile leaves as whole contiguous kilobytes: the rows of one x are adjacent
@@ -79,7 +145,7 @@ __device__ __forceinline__ void tn_store_rows(const f32x4 (&acc)[XPW][DV / 16], 
   if (sl >= PART * XPW && sl < (PART + 1) * XPW) *(f32x4*)(s + 16 * sl + 4 * g) = sacc * mul;
 }
 
-template <typename T, int DK, int DV, int XPW, int PART, bool HAS_W>
+template <typename T, int DK, int DV, int XPW, int PART, bool HAS_W, bool DIAG = false>
 __device__ __forceinline__ void tn_body(const T* __restrict__ A, const T* __restrict__ Bm, const float* __restrict__ w,
                                         T* __restrict__ S, float* __restrict__ s, int c, int hA, int r, int hh,
                                         int bn, int h, int y, int xb, bool active, bool use_mult, char* smem) {
@@ -138,9 +204,10 @@ __device__ __forceinline__ void tn_body(const T* __restrict__ A, const T* __rest
     if (HAS_W && wave == 0 && l < KT) async_copy4(w_base + row_index(r0 + l), st + A_BYTES + B_BYTES);
   };
 
-  f32x4 acc[XPW][NT];
+  constexpr int NF = DIAG ? TN_NDIAG : XPW;   // operand fragments built per step
+  f32x4 acc[NF][NT];
 #pragma unroll
-  for (int i = 0; i < XPW; i++)
+  for (int i = 0; i < NF; i++)
 #pragma unroll
     for (int j = 0; j < NT; j++) acc[i][j] = (f32x4){0, 0, 0, 0};
   f32x4 sacc = {0, 0, 0, 0};
@@ -182,28 +249,30 @@ __device__ __forceinline__ void tn_body(const T* __restrict__ A, const T* __rest
   auto load_frags = [&](Frags& F, auto slot_c, auto ks_c) {
     constexpr int OFF = decltype(slot_c)::value * STAGE + decltype(ks_c)::value * 32 * (CA * 16);
     F.kfy = tr8(ay[0] + OFF, ay[1] + OFF);
-    F.kfx = tr8(ax[0] + OFF, ax[1] + OFF);
+    if constexpr (!DIAG) F.kfx = tr8(ax[0] + OFF, ax[1] + OFF);
 #pragma unroll
     for (int nt = 0; nt < NT; nt++) F.vf[nt] = tr8(av[nt][0] + OFF, av[nt][1] + OFF);
   };
   auto compute = [&](const Frags& F, f32x4 w0, f32x4 w1) {
     float rowf[8], srcf[8];
     unpack8(F.kfy, rowf);
-    unpack8(F.kfx, srcf);
+    if constexpr (!DIAG) unpack8(F.kfx, srcf);
     if (HAS_W) {
       float sc[8];
 #pragma unroll
       for (int q = 0; q < 4; q++) {
-        sc[q] = srcf[q] * w0[q];
-        sc[4 + q] = srcf[4 + q] * w1[q];
+        sc[q] = (DIAG ? rowf[q] : srcf[q]) * w0[q];
+        sc[4 + q] = (DIAG ? rowf[4 + q] : srcf[4 + q]) * w1[q];
       }
       sacc = mfma16(F.kfy, pack8<T>(sc), sacc);
     } else {
-      sacc = mfma16(F.kfy, F.kfx, sacc);
+      sacc = mfma16(F.kfy, DIAG ? F.kfy : F.kfx, sacc);
     }
-    dpp_fence();  // srcf is read through DPP below
-    static_for<XPW>([&](auto xi) {
-      v8 a = PhiTile<T, PART * XPW + xi.value>::make(F.kfy, F.kfx, rowf, srcf);
+    dpp_fence();  // srcf / rowf is read through DPP below
+    static_for<NF>([&](auto xi) {
+      v8 a;
+      if constexpr (DIAG) a = PhiDiag<T, xi.value>::make(F.kfy, rowf);
+      else a = PhiTile<T, PART * XPW + xi.value>::make(F.kfy, F.kfx, rowf, srcf);
 #pragma unroll
       for (int nt = 0; nt < NT; nt++) acc[xi.value][nt] = mfma16(a, F.vf[nt], acc[xi.value][nt]);
     });
@@ -285,7 +354,16 @@ __device__ __forceinline__ void tn_body(const T* __restrict__ A, const T* __rest
   const float mul = (use_mult && xb < y) ? 2.f : 1.f;
   constexpr int D = 128 * (DK / 16) * (DK / 16 + 1);
   const long so = ((long)bn * h + hh) * D + 128 * y * (y + 1) + 256 * xb;
-  tn_store_rows<T, DV, XPW, PART>(acc, sacc, mul, smem_a + wave * (16 * (DV * 2 + 16)), S + so * DV, s + so);
+  if constexpr (DIAG) tn_store_diag<T, DV>(acc, sacc, smem_a + wave * (16 * (DV * 2 + 16)), S + so * DV, s + so);
+  else tn_store_rows<T, DV, XPW, PART>(acc, sacc, mul, smem_a + wave * (16 * (DV * 2 + 16)), S + so * DV, s + so);
+}
+
+// Wave tasks of a (chunk, head).  With eight x columns per wave (XPW == 8) the blocks below the block diagonal give
+// two tasks each, numbered first, and every diagonal block is ONE task of nine cyclic fragments; otherwise every
+// block, diagonal or not, is cut into 16 / XPW tasks.
+template <int DK, int XPW> constexpr int tn_tasks() {
+  constexpr int T = DK / 16;
+  return XPW == 8 ? T * (T - 1) + T : (T * (T + 1) / 2) * (16 / XPW);
 }
 
 template <typename T, int DK, int DV, int XPW, bool HAS_W>
@@ -306,12 +384,24 @@ __global__ __launch_bounds__(256, 2) void sympow_tn_kernel(const T* __restrict__
     bx = v - by * gridDim.x;
   }
   const int task = bx * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const bool active = task < NB * PARTS;
+  const bool active = task < tn_tasks<DK, XPW>();
   const int t2 = active ? task : 0;
-  const int part = t2 % PARTS;
+  int part = t2 % PARTS;
   int y, xb;
-  block_to_yx(t2 / PARTS, y, xb);
   const int bn = by / h, hh = by % h;
+  if constexpr (XPW == 8) {
+    constexpr int NOFF = (DK / 16) * (DK / 16 - 1);   // tasks below the block diagonal
+    if (t2 >= NOFF) {
+      y = xb = t2 - NOFF;
+      tn_body<T, DK, DV, XPW, 0, HAS_W, true>(A, Bm, w, S, s, c, hA, r, hh, bn, h, y, xb, active, use_mult != 0, smem);
+      return;
+    }
+    y = 1;
+    while (y * (y + 1) / 2 <= t2 / 2) y++;
+    xb = t2 / 2 - y * (y - 1) / 2;
+  } else {
+    block_to_yx(t2 / PARTS, y, xb);
+  }
 #define PR_TN_CASE(P)                                                                                                  \
   case P:                                                                                                              \
     if (P < PARTS)                                                                                                     \
@@ -596,7 +686,7 @@ static int tn_launch(const void* A, const void* Bm, const float* w, void* S, flo
                      int use_mult, hipStream_t st) {
   constexpr int XPW = DV <= 64 ? 8 : 4;
   constexpr int NB = (DK / 16) * (DK / 16 + 1) / 2;
-  constexpr int TASKS = NB * (16 / XPW);
+  constexpr int TASKS = tn_tasks<DK, XPW>();
   constexpr int KT = tn_stage_rows(DV);
   constexpr size_t smem = TN_NST * (KT * DK * 2 + KT * DV * 2 + KT * 4);
   dim3 grid((TASKS + 3) / 4, (unsigned)(BN * h));
