@@ -71,9 +71,13 @@ int pr_update_state_fwd(const void* K, const void* V, void* S, float* s, int BN,
                         int dtype, void* stream);
 
 /* Backward -- retention/_update_state/reference.py:55-83, Triton twin retention/_update_state/triton.py:148-260.
- *   dS [BN,h,D,d], ds [BN,h,D] fp32 -> dK, dV [BN,c,h,d]; one of dK, dV may be NULL (that gradient is skipped). */
+ *   dS [BN,h,D,d], ds [BN,h,D] fp32 -> dK, dV [BN,c,h,d]; one of dK, dV may be NULL (that gradient is skipped).
+ *   dS_symmetric != 0 is the caller's promise that dS[(a,b)] == dS[(b,a)] for the pairs the layout stores in both
+ *   orders (the 16x16 blocks on the diagonal); true of the dS that pr_query_state_bwd and the scans produce, not of
+ *   an arbitrary tensor.  The key gradient then takes a shorter path through those blocks; with 0 every feature is
+ *   used as given, as the reference does. */
 int pr_update_state_bwd(const void* K, const void* V, const void* dS, const float* ds, void* dK, void* dV, int BN,
-                        int c, int h, int d, int deg, int dtype, void* stream);
+                        int c, int h, int d, int deg, int dS_symmetric, int dtype, void* stream);
 
 /* discumsum(X, log_G) -- retention/_discumsum/reference.py:3-15, Triton twin retention/_discumsum/triton.py:34-94.
  *   X [B,n,H,F], log_G [B,n,H] fp32 -> Y [B,n_out,H,F], Y[0]=0, Y[k+1]=Y[k]*exp(log_G[k])+X[k];
@@ -141,12 +145,14 @@ int pr_query_state_fwd(const void* Q, const void* S, const float* s, const void*
  *      dY_attn [BN,c,h*r,d], dl_attn [BN,c,h*r] fp32.  dY_attn is dO times a per-row factor; a consumer that scales
  *      on the fly (the dO_scale argument of the attention backward) can ask for that factor instead:
  *      dY_scale [BN,c,h*r] fp32 (then dY_attn may be NULL).
- *   workspace: pr_query_state_bwd_workspace() bytes (scaled dO and two fp32 row vectors). */
+ *   workspace: pr_query_state_bwd_workspace() bytes (scaled dO and two fp32 row vectors).
+ *   S_symmetric != 0: the caller's promise that S[(a,b)] == S[(b,a)] in the blocks on the diagonal (true of every
+ *   state made by pr_update_state_fwd and the scans); the query gradient then takes a shorter path through them. */
 size_t pr_query_state_bwd_workspace(int BN, int c, int h, int r, int d, int dtype);
 int pr_query_state_bwd(const void* Q, const void* S, const float* s, const float* rowmax, const void* O,
                        const float* den, const void* dO, void* dQ, void* dS, float* ds, void* dY_attn,
                        float* dl_attn, float* dY_scale, void* workspace, int BN, int n, int c, int h, int r, int d,
-                       float scale_p, int deg, int zero_initial_state, int dtype, void* stream);
+                       float scale_p, int deg, int zero_initial_state, int S_symmetric, int dtype, void* stream);
 
 /* Accumulated gates of the quadratic / inference paths -- log_G.cumsum(1), retention/power_retention_maker.py:129,
  * 348-349.  log_G, A [B,t,h] fp32, t <= 8192. */

@@ -38,7 +38,7 @@ size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 
 extern "C" {
 
-int pr_abi_version(void) { return 1; }
+int pr_abi_version(void) { return 2; }
 const char* pr_last_error(void) { return g_err; }
 
 int pr_expanded_dim(int d, int deg) {
@@ -102,7 +102,7 @@ int pr_update_state_fwd(const void* K, const void* V, void* S, float* s, int BN,
 }
 
 int pr_update_state_bwd(const void* K, const void* V, const void* dS, const float* ds, void* dK, void* dV, int BN,
-                        int c, int h, int d, int deg, int dtype, void* stream) {
+                        int c, int h, int d, int deg, int dS_symmetric, int dtype, void* stream) {
   if (int rc = check_common("update_state_bwd", d, deg, dtype, true)) return rc;
   if (bad_ptr(K) || bad_ptr(V) || bad_ptr(dS) || bad_ptr(ds) || bad_opt(dK) || bad_opt(dV) || (!dK && !dV))
     return fail(PR_ERR_ARG, "update_state_bwd: null or misaligned pointer");
@@ -112,7 +112,7 @@ int pr_update_state_bwd(const void* K, const void* V, const void* dS, const floa
     if (int rc = finish(pr::sympow_nn(nn, BN, d, 1, 0, dtype, (hipStream_t)stream), "update_state_bwd(dV)")) return rc;
   }
   if (!dK) return 0;
-  pr::GradArgs g{K, V, nullptr, dS, ds, dK, c, h, 1, 1, 0};
+  pr::GradArgs g{K, V, nullptr, dS, ds, dK, c, h, 1, 1, 0, dS_symmetric ? 1 : 0};
   return finish(pr::sympow_grad(g, BN, d, 1, dtype, (hipStream_t)stream), "update_state_bwd(dK)");
 }
 
@@ -194,7 +194,7 @@ size_t pr_query_state_bwd_workspace(int BN, int c, int h, int r, int d, int dtyp
 int pr_query_state_bwd(const void* Q, const void* S, const float* s, const float* rowmax, const void* O,
                        const float* den, const void* dO, void* dQ, void* dS, float* ds, void* dY_attn,
                        float* dl_attn, float* dY_scale, void* workspace, int BN, int n, int c, int h, int r, int d,
-                       float scale_p, int deg, int zero_initial_state, int dtype, void* stream) {
+                       float scale_p, int deg, int zero_initial_state, int S_symmetric, int dtype, void* stream) {
   if (int rc = check_common("query_state_bwd", d, deg, dtype, true)) return rc;
   if (bad_ptr(Q) || bad_ptr(S) || bad_ptr(s) || bad_ptr(O) || bad_ptr(den) || bad_ptr(dO) || bad_ptr(dQ) ||
       bad_ptr(dS) || bad_ptr(ds) || bad_ptr(workspace) || bad_opt(rowmax) || bad_opt(dY_attn) || bad_opt(dl_attn))
@@ -213,7 +213,7 @@ int pr_query_state_bwd(const void* Q, const void* S, const float* s, const float
                       "query_state_bwd(prep)"))
     return rc;
   if (int rc = finish(pr::sympow_tn(Q, dOs, cvec, dS, ds, BN, c, h, r, d, 0, dtype, st), "query_state_bwd(dS)")) return rc;
-  pr::GradArgs g{Q, dOs, cvec, S, s, dQ, c, h, r, n, zero_initial_state ? 1 : 0};
+  pr::GradArgs g{Q, dOs, cvec, S, s, dQ, c, h, r, n, zero_initial_state ? 1 : 0, S_symmetric ? 1 : 0};
   return finish(pr::sympow_grad(g, BN, d, 0, dtype, st), "query_state_bwd(dQ)");
 }
 

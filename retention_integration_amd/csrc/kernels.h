@@ -59,6 +59,7 @@ struct GradArgs {
   void* dX;           // [BN, c, h*r, d]
   int c, h, r, n;
   int skip_first;     // chunk 0 of every batch entry has a zero state: dX = 0 there
+  int sym_diag;       // B[(a, b)] == B[(b, a)] in the blocks on the diagonal (the caller's promise)
 };
 int sympow_grad(const GradArgs& a, int BN, int d, int mult, int dtype, hipStream_t st);
 

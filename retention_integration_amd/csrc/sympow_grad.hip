@@ -47,7 +47,10 @@ template <> __device__ __forceinline__ void unpack2<f16_t>(uint32_t u, float& lo
   hi = (float)p[1];
 }
 
-template <typename T, int DK, int DV, int MT, bool MULT>
+// SYM: the caller guarantees B[(a, b)] == B[(b, a)] inside the blocks on the diagonal (true of every state and state
+// gradient this library forms: both orders of a pair are the same sum).  dphi is then symmetric there, the two folds
+// of a diagonal block are equal, and the block takes twice the first fold instead of both.
+template <typename T, int DK, int DV, int MT, bool MULT, bool SYM>
 __global__ __launch_bounds__(256, (MT == 2 && DK <= 64) ? 4 : 2) void sympow_grad_kernel(GradArgs a, int row_blocks, int npairs) {
   typedef typename VecOf<T>::v8 v8;
   typedef typename VecOf<T>::v4 v4;
@@ -215,8 +218,13 @@ __global__ __launch_bounds__(256, (MT == 2 && DK <= 64) ? 4 : 2) void sympow_gra
           for (int mi = 0; mi < MT; mi++) {
             float x0, x1;
             unpack2<T>(*(const lds_u32*)(xa[mi] + 4 * pr2), x0, x1);
+            if constexpr (SYM && diag) {
+              x0 += x0;
+              x1 += x1;
+            }
             acc[mi][y] = acc[mi][y] + d0[mi] * x0;   // each line contracts to one fused multiply-add per element
             acc[mi][y] = acc[mi][y] + d1[mi] * x1;
+            if constexpr (SYM && diag) continue;
             float w8[8];
 #pragma unroll
             for (int v = 0; v < 4; v++) {
@@ -305,7 +313,8 @@ __global__ __launch_bounds__(256, (MT == 2 && DK <= 64) ? 4 : 2) void sympow_gra
   }
 }
 
-template <typename T, int DK, int DV, bool MULT> static int grad_launch(const GradArgs& a, int BN, hipStream_t st) {
+template <typename T, int DK, int DV, bool MULT, bool SYM>
+static int grad_launch(const GradArgs& a, int BN, hipStream_t st) {
   const int rows = a.c * a.r, npairs = BN * a.h;
   auto go = [&](auto mt) {
     constexpr int MT = decltype(mt)::value;
@@ -313,7 +322,7 @@ template <typename T, int DK, int DV, bool MULT> static int grad_launch(const Gr
     constexpr size_t smem = ((ring > mtile ? ring : mtile) + 1023) / 1024 * 1024 + 64 * MT * DK * 2;
     const int row_blocks = (rows + 64 * MT - 1) / (64 * MT);
     dim3 grid((unsigned)(((npairs + 7) / 8) * 8 * row_blocks));
-    auto kern = sympow_grad_kernel<T, DK, DV, MT, MULT>;
+    auto kern = sympow_grad_kernel<T, DK, DV, MT, MULT, SYM>;
     allow_big_lds((const void*)kern, smem);
     hipLaunchKernelGGL(kern, grid, dim3(256), smem, st, a, row_blocks, npairs);
   };
@@ -328,7 +337,9 @@ template <typename T, int DK, int DV, bool MULT> static int grad_launch(const Gr
 
 int sympow_grad(const GradArgs& a, int BN, int d, int mult, int dtype, hipStream_t st) {
 #define PR_G_D(T, DD)                                                                                                  \
-  case DD: return mult ? grad_launch<T, DD, DD, true>(a, BN, st) : grad_launch<T, DD, DD, false>(a, BN, st);
+  case DD:                                                                                                             \
+    if (a.sym_diag) return mult ? grad_launch<T, DD, DD, true, true>(a, BN, st) : grad_launch<T, DD, DD, false, true>(a, BN, st); \
+    return mult ? grad_launch<T, DD, DD, true, false>(a, BN, st) : grad_launch<T, DD, DD, false, false>(a, BN, st);
 #define PR_G_T(T)                                                                                                      \
   switch (d) { PR_G_D(T, 32) PR_G_D(T, 64) PR_G_D(T, 128) default: return -2; }
   if (dtype == DT_BF16) { PR_G_T(bf16_t) }

@@ -154,7 +154,8 @@ def chunked_bwd(Q: Tensor, K: Tensor, V: Tensor, A: Tensor, lcs: Tensor, Kd: Ten
         dSc, dsc = torch.empty_like(Sc), torch.empty_like(sc)
         ws = _empty((lib.pr_query_state_bwd_workspace(BN, c, h, r, d, code),), u8, dev)
         _lib.check(lib.pr_query_state_bwd(p(Qg), p(Sc), p(sc), p(rm), p(O), p(den), p(dO), p(dQg), p(dSc), p(dsc),
-                                          None, p(dla), p(dys), p(ws), BN, n, c, h, r, d, scale ** deg, 2, 1, code, st),
+                                          None, p(dla), p(dys), p(ws), BN, n, c, h, r, d, scale ** deg, 2, 1, 1, code,
+                                          st),
                    "query_state_bwd")
         ws = _empty((lib.pr_state_scan_bwd_workspace(b, n, h, D * d, D),), u8, dev)
         _lib.check(lib.pr_state_scan_bwd(p(dSc), p(Sc), p(dsc), p(sc), p(lcs), p(dS), p(ds), p(dlcs), p(ws), b, n, n, h,
@@ -162,10 +163,11 @@ def chunked_bwd(Q: Tensor, K: Tensor, V: Tensor, A: Tensor, lcs: Tensor, Kd: Ten
         del dSc, dsc
     dKd, dVs = torch.empty_like(K), torch.empty_like(V)
     # (two calls: the value gradient and the key gradient are separate kernels, and the latter is timed on its own)
-    _lib.check(lib.pr_update_state_bwd(p(Kd), p(V), p(dS), p(ds), None, p(dVs), BN, c, h, d, 2, code, st),
+    # (dS comes from the kernels above, so both orders of a pair hold the same sum: the last flag says so)
+    _lib.check(lib.pr_update_state_bwd(p(Kd), p(V), p(dS), p(ds), None, p(dVs), BN, c, h, d, 2, 1, code, st),
                "update_state_bwd(dV)")
     _lib.check(_timed("sympow_grad(dK)", lambda: lib.pr_update_state_bwd(
-        p(Kd), p(V), p(dS), p(ds), p(dKd), None, BN, c, h, d, 2, code, st)), "update_state_bwd(dK)")
+        p(Kd), p(V), p(dS), p(ds), p(dKd), None, BN, c, h, d, 2, 1, code, st)), "update_state_bwd(dK)")
 
     # the attention backward adds the state-path gradients in its epilogue and writes the final dQ, dK, dV
     dQa, dKa, dVa = torch.empty_like(Q), torch.empty_like(K), torch.empty_like(V)

@@ -161,7 +161,7 @@ def update_state_bwd(K: Tensor, V: Tensor, dS: Tensor, ds: Tensor) -> Tuple[Tens
     dK, dV = torch.empty_like(K), torch.empty_like(V)
     lib = _lib.load()
     _lib.check(lib.pr_update_state_bwd(_lib.ptr(K), _lib.ptr(V), _lib.ptr(dS), _lib.ptr(ds), _lib.ptr(dK),
-                                       _lib.ptr(dV), b * n, c, h, d, 2, _lib.dtype_code(K.dtype), _lib.stream()),
+                                       _lib.ptr(dV), b * n, c, h, d, 2, 0, _lib.dtype_code(K.dtype), _lib.stream()),
                "update_state_bwd")
     return dK, dV
 
@@ -306,7 +306,7 @@ def query_state_bwd(Q: Tensor, S: Tensor, s: Tensor, rowmax: Optional[Tensor], O
     _lib.check(lib.pr_query_state_bwd(_lib.ptr(Q), _lib.ptr(S), _lib.ptr(s), _lib.ptr(rowmax), _lib.ptr(O),
                                       _lib.ptr(den), _lib.ptr(dO), _lib.ptr(dQ), _lib.ptr(dS), _lib.ptr(ds),
                                       _lib.ptr(dYa), _lib.ptr(dla), None, _lib.ptr(ws), b * n, n, c, h, r, d,
-                                      float(scale_p), 2, int(zero_initial_state), code, _lib.stream()),
+                                      float(scale_p), 2, int(zero_initial_state), 0, code, _lib.stream()),
                "query_state_bwd")
     if not has_attn:
         dYa = torch.empty((0,), dtype=Q.dtype, device=Q.device)
