@@ -218,3 +218,64 @@ def test_attention(pra, dtype, d, tq, tk, r, gated, norm, deg):
     for nm, a, b_ in zip(["dQ", "dK", "dV", "dG"], g_in, o_in):
         if a is not None:
             check(nm, a.grad, b_.grad, GRAD_TOL)
+
+
+# ---------------------------------------------------------------- symmetric-state promise of the C ABI
+def test_query_state_with_a_state_that_is_not_symmetric(pra):
+    """The layout stores the pairs of a diagonal block in both orders.  The operator makes no assumption about them
+    (ref: retention/_query_state/reference.py:27-31 expands every stored feature): a state whose two copies differ
+    must give the oracle's output and gradients."""
+    dtype, d, c, r = torch.bfloat16, 64, 128, 1
+    b, n, h = 1, 2, 2
+    Q = rnd(b, n, c, h * r, d, dtype=dtype, seed=40)
+    Ks = rnd(b, n, 48, h, d, dtype=torch.float32, scale=d ** -0.25, seed=41)
+    Vs = rnd(b, n, 48, h, d, dtype=torch.float32, seed=42)
+    S, s = oracle.update_state(Ks, Vs, 2)
+    S = (S + rnd(*S.shape, dtype=torch.float32, scale=S.std().item(), seed=43)).to(dtype)
+    scale = 1.0 / math.sqrt(d)
+    g_in = [dev(Q, True), dev(S, True), dev(s, True)]
+    o_in = [gold(Q, True), gold(S, True), gold(s, True)]
+    O = pra.query_state(*g_in, None, None, None, 2, scale, False)
+    Oo = oracle.query_state(*o_in, None, None, None, 2, scale, False)
+    check("O", O, Oo, OUT_TOL)
+    dO = rnd(*Oo.shape, dtype=dtype, seed=44)
+    O.backward(dev(dO))
+    Oo.backward(gold(dO))
+    for nm, a, b_ in zip(["dQ", "dS", "ds"], g_in, o_in):
+        check(nm, a.grad, b_.grad, GRAD_TOL)
+
+
+@pytest.mark.parametrize("dtype,d,c", [(torch.bfloat16, 64, 256), (torch.float16, 32, 128), (torch.bfloat16, 128, 128)])
+def test_symmetric_state_flag_changes_nothing_for_a_symmetric_state(pra, dtype, d, c):
+    """dS_symmetric / S_symmetric let the gradient kernels take one fold instead of two through the diagonal blocks.
+    For a state made by update_state (both copies of a pair are the same sum) the results with and without the
+    promise agree to rounding, and the state produced by the forward kernel is symmetric bit for bit."""
+    from retention_integration_amd import _lib, ops
+    lib, st, p = _lib.load(), _lib.stream(), _lib.ptr
+    b, n, h = 1, 3, 2
+    std = 0.5 if dtype == torch.float16 else 1.0
+    K = dev(rnd(b, n, c, h, d, dtype=dtype, scale=std, seed=50))
+    V = dev(rnd(b, n, c, h, d, dtype=dtype, scale=std, seed=51))
+    Q = dev(rnd(b, n, c, h, d, dtype=dtype, scale=std, seed=52))
+    dO = dev(rnd(b, n, c, h, d, dtype=dtype, seed=53))
+    S, s = ops.update_state_fwd(K, V)
+    for y in range(d // 16):   # diagonal block y: features 128 y (y+1) + 256 y + 16 a + i  <->  pair (16y + a, 16y + i)
+        f0 = 128 * y * (y + 1) + 256 * y
+        blk = S[..., f0:f0 + 256, :].reshape(b, n, h, 16, 16, d)
+        assert torch.equal(blk, blk.transpose(3, 4)), f"diagonal block {y} of the state is not symmetric"
+    code = _lib.dtype_code(dtype)
+    res = []
+    for flag in (0, 1):
+        dK, dV = torch.empty_like(K), torch.empty_like(V)
+        _lib.check(lib.pr_update_state_bwd(p(K), p(V), p(S), p(s), p(dK), p(dV), b * n, c, h, d, 2, flag, code, st),
+                   "update_state_bwd")
+        O, den = ops.query_state_fwd(Q, S, s, None, None, None, 1.0 / d, False)
+        dQ, dS, ds = torch.empty_like(Q), torch.empty_like(S), torch.empty_like(s)
+        ws = torch.empty(lib.pr_query_state_bwd_workspace(b * n, c, h, 1, d, code), dtype=torch.uint8, device=DEV)
+        _lib.check(lib.pr_query_state_bwd(p(Q), p(S), p(s), None, p(O), p(den), p(dO), p(dQ), p(dS), p(ds), None, None,
+                                          None, p(ws), b * n, n, c, h, 1, d, 1.0 / d, 2, 0, flag, code, st),
+                   "query_state_bwd")
+        res.append((dK, dV, dQ, dS, ds))
+    for nm, a, b_ in zip(["dK", "dV", "dQ", "dS", "ds"], res[1], res[0]):
+        check(f"{nm}: with the promise vs without", a, b_, 3e-3)
+    assert torch.equal(res[0][1], res[1][1]) and torch.equal(res[0][3], res[1][3])
