@@ -56,7 +56,10 @@ def event_time_ms(fn, iters, warmup=2):
 
 
 def op_breakdown(pra, Q, K, V, lg, dO, cfg, iters=5):
-    """Per-kernel-family timings of the pieces of one step, each launched alone (HIP events)."""
+    """Per-kernel-family timings of the pieces of one step, each launched alone (HIP events) through the operator
+    wrappers.  Those make no promise about the state's symmetry, so their query_state / update_state backward take
+    both folds through the diagonal feature blocks (the fused step promises it and is ~20 us per launch faster,
+    which the "sympow_grad(dK)" entry, launched as the step launches it, shows)."""
     from retention_integration_amd import ops
     b, t, h, d, c = cfg["b"], cfg["t"], cfg["h"], cfg["d"], cfg["chunk"]
     n = t // c
