@@ -66,10 +66,11 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dq_kernel(AttnBwdArgs a,
   // XCD; only the CU inside a shader engine is chosen by load.  Blocks differ in length (causal), so each of the 32
   // (XCD, shader engine) groups gets whole (batch, kv head) pairs, pair after pair with the longest block of a pair
   // first: the blocks of a pair run at the same time and share its rows in the XCD's L2 (dealing the longest blocks
-  // of all pairs first instead balances the tail no better and fetches 2.5x the bytes from HBM).
-  // (integer division runs on the vector unit: readfirstlane brings the uniform results back to scalar registers)
+  // of ALL pairs first instead fetches 2.5x the bytes from HBM); only the last few pairs of a group are interleaved,
+  // see deal_causal_blocks.
   const int grp = blockIdx.x % 32, u = blockIdx.x / 32, ppg = (npairs + 31) / 32;
-  const int pig = __builtin_amdgcn_readfirstlane(u / nblocks), blk = u - pig * nblocks;
+  int pig, blk;
+  deal_causal_blocks(u, nblocks, ppg, pig, blk);
   const int pair = pig * 32 + grp;
   if (pair >= npairs) return;
   const int tid = threadIdx.x, l = tid & 63, g = l >> 4, tcol = l & 15;
@@ -416,9 +417,9 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
   constexpr int LOADS = 2 * AB_BM * CPR / 256;
   extern __shared__ __attribute__((aligned(1024))) char smem[];
 
-  // (integer division runs on the vector unit: readfirstlane brings the uniform results back to scalar registers)
   const int grp = blockIdx.x % 32, u = blockIdx.x / 32, ppg = (npairs + 31) / 32;
-  const int pig = __builtin_amdgcn_readfirstlane(u / nblocks), blk = u - pig * nblocks;
+  int pig, blk;
+  deal_causal_blocks(u, nblocks, ppg, pig, blk);
   const int pair = pig * 32 + grp;
   if (pair >= npairs) return;
   const int tid = threadIdx.x, l = tid & 63, g = l >> 4, kcol = l & 15;

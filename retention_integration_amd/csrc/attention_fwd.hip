@@ -65,10 +65,11 @@ __global__ __launch_bounds__(256, OCC) void attention_fwd_kernel(AttnFwdArgs a, 
   // group then gets the same mix of long and short row blocks and the K/V of a pair stay in one L2.  Inside a
   // group the pairs follow one another, longest row block first, so that the row blocks of a pair run together.
   const int grp = blockIdx.x % 32, u = blockIdx.x / 32, ppg = (npairs + 31) / 32;
-  // (integer division runs on the vector unit: readfirstlane brings the uniform results back to scalar registers)
-  const int pig = __builtin_amdgcn_readfirstlane(u / row_blocks);
+  // (the last few pairs of a group are interleaved, see deal_causal_blocks)
+  int pig, blk;
+  deal_causal_blocks(u, row_blocks, ppg, pig, blk);
   const int pair = pig * 32 + grp;
-  const int rblk = row_blocks - 1 - (u - pig * row_blocks);
+  const int rblk = row_blocks - 1 - blk;
   if (pair >= npairs) return;
   const int b = __builtin_amdgcn_readfirstlane(pair / a.h), hh = pair - b * a.h;
   const int hq = a.h * a.r, rows = a.tq * a.r, shift = a.tk - a.tq;

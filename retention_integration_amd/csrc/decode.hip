@@ -14,7 +14,9 @@
 // The query reads the OLD state, so one pass serves both (and the update may be in place: a state element is read and
 // then written by the same thread, the key sum of a feature row by the lanes of one wave before its lane 0 writes it): every workgroup owns a slice of the features of one
 // (batch, kv head), streams its rows of S once (16 bytes per lane, fully coalesced), accumulates the query partials
-// in registers and writes the updated rows.  A second, tiny kernel adds the partials of the slices and merges.
+// in registers and writes the updated rows.  A second, tiny kernel adds the partials of the slices and merges; with
+// many (batch, kv head) pairs and one or two query rows a single 1024-thread workgroup takes a whole pair and merges
+// in the same kernel.
 #include "common.h"
 #include "kernels.h"
 

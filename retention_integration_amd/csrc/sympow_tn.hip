@@ -12,7 +12,9 @@
 // (y, xb) and all DV value columns, and contracts over the rows 32 at a time.  The phi tile is
 // never stored: the A-operand of each matrix-core op is produced in registers as the product of a
 // row-broadcast (DPP) of column x with the 16 columns 16*y..16*y+15, both read transposed from one
-// row-major LDS tile.  s uses the identity s[(x, j)] = (A^T diag(w) A)[x, j], one extra matrix-core op
+// row-major LDS tile.  Blocks on the diagonal (xb == y) hold every product twice; up to d = 64 one wave computes such
+// a block along its nine cyclic diagonals (row rotation instead of row broadcast) and stores each sum at both places.
+// s uses the identity s[(x, j)] = (A^T diag(w) A)[x, j], one extra matrix-core op
 // per step.  Row tiles of A and B arrive through a 3-deep ring of asynchronous global->LDS copies.
 #include "common.h"
 #include "kernels.h"
