@@ -36,6 +36,7 @@ enum {
   PR_ERR_DEG = -4        /* unsupported degree */
 };
 
+/* 2: pr_update_state_bwd and pr_query_state_bwd take the symmetric-state promise (dS_symmetric, S_symmetric). */
 int pr_abi_version(void);
 const char* pr_last_error(void);
 
