@@ -218,11 +218,21 @@ def power_retention(Q, K, V, log_G=None, initial_state=None, return_final_state=
     """Training-path power retention.
 
     ref: retention/power_retention_maker.py:71-90 (padding), :96-197 (body),
-    wired as in ref: retention/reference.py:8.  ``initial_state`` /
-    ``return_final_state`` are not restated (unused by every benchmark config).
+    wired as in ref: retention/reference.py:8.
+
+    ``initial_state`` / ``return_final_state`` do NOT follow the reference
+    (:131-140, :158-160, :168-172), whose handling is unfinished there: the
+    returned tensor is the state at the start of the last chunk, the carried
+    state is not decayed by the gates (":158 TODO") and no key sums travel with
+    it.  Here they carry the definition the product documents: the state is
+    the pair (S [b,h,D,d], sum_of_keys [b,h,D]) AFTER the last token, decayed
+    like any chunk state, so that two chained calls equal one call.  That
+    definition is pinned by exactly this property and by equality with the
+    state ``power_retention_inference`` forms over the same tokens
+    (tests/test_oracle_invariants.py), not by the reference.
     """
-    assert initial_state is None and not return_final_state, "not restated"
     assert deg % 2 == 0, f"deg must be even: {deg=}"
+    with_state = initial_state is not None or return_final_state
     t_orig = Q.shape[1]
     pad = 0
     if chunk_size is not None and t_orig % chunk_size != 0:
@@ -249,7 +259,7 @@ def power_retention(Q, K, V, log_G=None, initial_state=None, return_final_state=
     if not scale:
         scale = 1.0 / d ** 0.5
 
-    if switch_over_seq_len is None or t <= switch_over_seq_len:
+    if (switch_over_seq_len is None or t <= switch_over_seq_len) and not with_state:
         A = log_G.cumsum(1) if gating else None
         out = attention(Q, K, V, A, deg, scale=scale, norm=True)
         return out[:, :t_orig] if pad else out
@@ -265,8 +275,16 @@ def power_retention(Q, K, V, log_G=None, initial_state=None, return_final_state=
         Kd = Kc
         lcs = torch.zeros(b, n, h, dtype=torch.float32, device=Q.device)
     S, s = update_state(Kd.contiguous(), Vc.contiguous(), deg)
-    S = discumsum(S, lcs).narrow(1, 0, n)
-    s = discumsum(s, lcs).narrow(1, 0, n)
+    first = 0
+    if initial_state is not None:  # one more scan entry in front; chunk k's gate sum decays it like a chunk state
+        S0, s0 = initial_state
+        S = torch.cat([S0.unsqueeze(1).to(S.dtype), S], dim=1)
+        s = torch.cat([s0.unsqueeze(1).to(s.dtype), s], dim=1)
+        lcs = torch.cat([torch.zeros_like(lcs[:, :1]), lcs], dim=1)
+        first = 1
+    S, s = discumsum(S, lcs), discumsum(s, lcs)
+    final = (S[:, first + n], s[:, first + n])
+    S, s = S.narrow(1, first, n), s.narrow(1, first, n)
 
     Ya, la, rm = attention(Qc.reshape(b * n, c, hq, d), Kc.reshape(b * n, c, h, d), Vc.reshape(b * n, c, h, d),
                            A.reshape(b * n, c, h) if gating else None, deg, scale=scale, norm=False)
@@ -277,9 +295,10 @@ def power_retention(Q, K, V, log_G=None, initial_state=None, return_final_state=
     else:
         Qg = Qc
     Y = query_state(Qg.contiguous(), S.contiguous(), s.contiguous(), Ya.contiguous(), la.contiguous(),
-                    rm.contiguous(), deg, scale, True)
+                    rm.contiguous(), deg, scale, initial_state is None)
     out = Y.contiguous().view(b, t, hq, d).to(dtype)
-    return out[:, :t_orig] if pad else out
+    out = out[:, :t_orig] if pad else out
+    return (out, final) if return_final_state else out
 
 
 def power_retention_inference(Q, K, V, log_G=None, initial_state=None, sum_of_keys=None,

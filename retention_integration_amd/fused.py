@@ -86,11 +86,11 @@ def chunked_fwd(Q: Tensor, K: Tensor, V: Tensor, log_G: Optional[Tensor], deg: i
     if _chained(lib, b, n, c, h, 1, d):
         # short chunks: the chunk states are scanned as they are formed and never written on their own
         _lib.check(lib.pr_update_state_scan_fwd(p(Kd_), p(V), p(lcs) if gated else None, p(Sc), p(sc), b, n, c, h, d,
-                                                2, code, st), "update_state_scan_fwd")
+                                                deg, code, st), "update_state_scan_fwd")
     else:
         S, s = torch.empty_like(Sc), torch.empty_like(sc)
         _lib.check(_timed("sympow_tn(update_state)", lambda: lib.pr_update_state_fwd(
-            p(Kd_), p(V), p(S), p(s), BN, c, h, d, 2, code, st)), "update_state_fwd")
+            p(Kd_), p(V), p(S), p(s), BN, c, h, d, deg, code, st)), "update_state_fwd")
         _lib.check(lib.pr_state_scan_fwd(p(S), p(s), p(lcs), p(Sc), p(sc), b, n, n, h, D * d, D, code, st),
                    "state_scan_fwd")
         del S, s
@@ -101,7 +101,7 @@ def chunked_fwd(Q: Tensor, K: Tensor, V: Tensor, log_G: Optional[Tensor], deg: i
                                     scale, deg, 0, code, st), "attention_fwd")
     O, den = torch.empty_like(Q), _empty((BN, c, hq), f32, dev)
     _lib.check(lib.pr_query_state_fwd(p(Qg_), p(Sc), p(sc), p(Ya), p(la), p(rm), p(O), p(den), BN, n, c, h, r, d,
-                                      scale ** deg, 2, 1, code, st), "query_state_fwd")
+                                      scale ** deg, deg, 1, code, st), "query_state_fwd")
     return O, A, lcs, Kd, Qg, Sc, sc, rm, den
 
 
@@ -148,13 +148,13 @@ def chunked_bwd(Q: Tensor, K: Tensor, V: Tensor, A: Tensor, lcs: Tensor, Kd: Ten
         ws = _empty((lib.pr_query_state_scan_bwd_workspace(b, n, c, h, r, d, code),), u8, dev)
         _lib.check(lib.pr_query_state_scan_bwd(p(Qg), p(Sc), p(sc), p(rm), p(O), p(den), p(dO),
                                                p(lcs) if gated else None, p(dQg), p(dS), p(ds), None, p(dla), p(dys),
-                                               p(dlcs) if gated else None, p(ws), b, n, c, h, r, d, scale ** deg, 2,
+                                               p(dlcs) if gated else None, p(ws), b, n, c, h, r, d, scale ** deg, deg,
                                                code, st), "query_state_scan_bwd")
     else:
         dSc, dsc = torch.empty_like(Sc), torch.empty_like(sc)
         ws = _empty((lib.pr_query_state_bwd_workspace(BN, c, h, r, d, code),), u8, dev)
         _lib.check(lib.pr_query_state_bwd(p(Qg), p(Sc), p(sc), p(rm), p(O), p(den), p(dO), p(dQg), p(dSc), p(dsc),
-                                          None, p(dla), p(dys), p(ws), BN, n, c, h, r, d, scale ** deg, 2, 1, 1, code,
+                                          None, p(dla), p(dys), p(ws), BN, n, c, h, r, d, scale ** deg, deg, 1, 1, code,
                                           st),
                    "query_state_bwd")
         ws = _empty((lib.pr_state_scan_bwd_workspace(b, n, h, D * d, D),), u8, dev)
@@ -164,10 +164,10 @@ def chunked_bwd(Q: Tensor, K: Tensor, V: Tensor, A: Tensor, lcs: Tensor, Kd: Ten
     dKd, dVs = torch.empty_like(K), torch.empty_like(V)
     # (two calls: the value gradient and the key gradient are separate kernels, and the latter is timed on its own)
     # (dS comes from the kernels above, so both orders of a pair hold the same sum: the last flag says so)
-    _lib.check(lib.pr_update_state_bwd(p(Kd), p(V), p(dS), p(ds), None, p(dVs), BN, c, h, d, 2, 1, code, st),
+    _lib.check(lib.pr_update_state_bwd(p(Kd), p(V), p(dS), p(ds), None, p(dVs), BN, c, h, d, deg, 1, code, st),
                "update_state_bwd(dV)")
     _lib.check(_timed("sympow_grad(dK)", lambda: lib.pr_update_state_bwd(
-        p(Kd), p(V), p(dS), p(ds), p(dKd), None, BN, c, h, d, 2, 1, code, st)), "update_state_bwd(dK)")
+        p(Kd), p(V), p(dS), p(ds), p(dKd), None, BN, c, h, d, deg, 1, code, st)), "update_state_bwd(dK)")
 
     # the attention backward adds the state-path gradients in its epilogue and writes the final dQ, dK, dV
     dQa, dKa, dVa = torch.empty_like(Q), torch.empty_like(K), torch.empty_like(V)
@@ -214,5 +214,8 @@ torch.library.register_autograd("pr::chunked_fwd", _chunked_backward, setup_cont
 
 
 def chunked_power_retention(Q, K, V, log_G, deg, scale, chunk_size):
-    """Q [b,t,hq,d], K, V [b,t,h,d] contiguous, t a multiple of chunk_size, log_G [b,t,h] fp32 or None."""
+    """Q [b,t,hq,d], K, V [b,t,h,d] contiguous, t a multiple of chunk_size, log_G [b,t,h] fp32 or None.
+    Only deg = 2 has a state (ref: retention/_update_state/triton.py:310-311 raises the same way)."""
+    if deg != 2:
+        raise NotImplementedError(f"the chunked algorithm needs the degree-2 state layout (got deg={deg})")
     return chunked_fwd(Q, K, V, log_G, int(deg), float(scale), int(chunk_size))[0]

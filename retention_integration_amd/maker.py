@@ -17,14 +17,26 @@ def _pad_time(x, pad, dims_after):
 
 
 def make_power_retention(update_state_impl, query_state_impl, discumsum_impl, attention_impl, *,
-                         scan_keeps_last=True, chunked_impl=None):
+                         scan_keeps_last=True, chunked_impl=None, full_scan_impl=None):
     """Build ``power_retention`` from operator implementations.
 
     ``scan_keeps_last=False`` declares that ``discumsum_impl(X, log_G)`` already returns only the first n
     entries of the scan (the composed path never reads the last one).  ``chunked_impl(Q, K, V, log_G, deg,
     scale, chunk_size)``, when given, replaces the composition of the four operators on the chunked branch
-    (same result; used for the fused single-node path).
+    (same result; used for the fused single-node path).  ``full_scan_impl(X, log_G)`` must return all n + 1
+    entries; it is needed for ``return_final_state`` when ``discumsum_impl`` drops the last one.
+
+    State across calls.  ``initial_state`` is a pair ``(state [b,h,D,d], sum_of_keys [b,h,D])`` -- what
+    ``power_retention_inference`` takes and returns -- and ``return_final_state=True`` returns
+    ``(out, (state, sum_of_keys))`` with the state AFTER the last token of this call, every chunk's decay
+    applied to what came before it.  One call over t tokens therefore equals two calls over t/2 chained
+    through the returned pair.  This departs from the reference on purpose: there the returned tensor is the
+    state at the START of the last chunk, the initial state is not decayed by the gates ("TODO", ref:
+    retention/power_retention_maker.py:158, 168-172) and no key sums travel with it, so its normaliser
+    forgets the earlier call.
     """
+    if full_scan_impl is None and scan_keeps_last:
+        full_scan_impl = discumsum_impl
 
     def power_retention(Q, K, V, log_G=None, initial_state=None, return_final_state=False,
                         deg=2, scale=None, chunk_size=None, switch_over_seq_len=None):
@@ -39,7 +51,7 @@ def make_power_retention(update_state_impl, query_state_impl, discumsum_impl, at
         out = _body(Q, K, V, log_G, initial_state, return_final_state, deg, scale, chunk_size, switch_over_seq_len)
         if not pad:
             return out
-        if return_final_state:
+        if return_final_state:   # (padded keys are zero and padded gates are log 1: the state is not touched by them)
             return out[0][:, :t_in], out[1]
         return out[:, :t_in]
 
@@ -47,8 +59,6 @@ def make_power_retention(update_state_impl, query_state_impl, discumsum_impl, at
         # ref: retention/power_retention_maker.py:96-197
         assert deg % 2 == 0, f"deg must be even: {deg=}"
         assert Q.dtype == K.dtype == V.dtype, f"dtypes of inputs must match: {Q.dtype=}, {K.dtype=}, {V.dtype=}"
-        if initial_state is not None or return_final_state:
-            raise NotImplementedError("initial_state / return_final_state are not provided by this build")
         dtype = Q.dtype
         b, t, hq, d = Q.shape
         h = K.shape[2]
@@ -66,12 +76,25 @@ def make_power_retention(update_state_impl, query_state_impl, discumsum_impl, at
             log_G = log_G.to(torch.float32)
         if not scale:
             scale = 1.0 / d ** 0.5
+        with_state = initial_state is not None or return_final_state
+        if initial_state is not None:
+            assert isinstance(initial_state, (tuple, list)) and len(initial_state) == 2, \
+                "initial_state must be the pair (state [b,h,D,d], sum_of_keys [b,h,D])"
+            S0, s0 = initial_state
+            assert S0.dim() == 4 and S0.shape[:2] == (b, h) and S0.shape[3] == d and s0.shape == S0.shape[:3], \
+                f"initial_state shapes {tuple(S0.shape)}, {tuple(s0.shape)} do not fit {b=} {h=} {d=}"
+            assert S0.dtype == dtype, f"initial_state dtype {S0.dtype} must match the inputs' {dtype}"
 
-        if switch_over_seq_len is None or t <= switch_over_seq_len:  # quadratic form (:128-140)
+        if (switch_over_seq_len is None or t <= switch_over_seq_len) and not with_state:   # quadratic form (:128-140)
             A = log_G.cumsum(1) if gated else None
             return attention_impl(Q, K, V, A, deg, scale=scale, norm=True)
 
-        if chunked_impl is not None:
+        # Everything below goes through the state, which exists for degree 2 only: refuse here, before anything is
+        # launched, whichever implementation follows (ref: retention/_update_state/triton.py:310-311).
+        if deg != 2:
+            raise NotImplementedError(f"the chunked algorithm needs the degree-2 state layout (got deg={deg})")
+
+        if chunked_impl is not None and not with_state:
             return chunked_impl(Q.contiguous(), K.contiguous(), V.contiguous(),
                                 log_G.contiguous() if gated else None, deg, scale, c)
 
@@ -85,9 +108,26 @@ def make_power_retention(update_state_impl, query_state_impl, discumsum_impl, at
             A, Kd = None, Kc
             lcs = torch.zeros(b, n, h, device=Q.device, dtype=torch.float32)              # (:166)
         S, s = update_state_impl(Kd.contiguous(), Vc.contiguous(), deg)                    # (:156)
-        S, s = discumsum_impl(S, lcs), discumsum_impl(s, lcs)                              # (:167-170)
-        if scan_keeps_last:
-            S, s = S.narrow(1, 0, n), s.narrow(1, 0, n)
+        final = None
+        if with_state:
+            if full_scan_impl is None:
+                raise NotImplementedError("initial_state / return_final_state need a scan that keeps its last entry")
+            first = 0
+            if initial_state is not None:
+                # the carried state is one more entry in front of the chunk states; its own gate is never applied
+                # (entry 0 of the scan is zero), and chunk k's gate sum then decays it like any other chunk's state
+                S = torch.cat([S0.unsqueeze(1), S], 1)
+                s = torch.cat([s0.unsqueeze(1).to(s.dtype), s], 1)
+                lcs = torch.cat([torch.zeros_like(lcs[:, :1]), lcs], 1)
+                first = 1
+            S, s = full_scan_impl(S, lcs), full_scan_impl(s, lcs)
+            if return_final_state:
+                final = (S[:, first + n], s[:, first + n])
+            S, s = S.narrow(1, first, n), s.narrow(1, first, n)
+        else:
+            S, s = discumsum_impl(S, lcs), discumsum_impl(s, lcs)                          # (:167-170)
+            if scan_keeps_last:
+                S, s = S.narrow(1, 0, n), s.narrow(1, 0, n)
 
         flat = lambda x: x.reshape(b * n, *x.shape[2:])  # noqa: E731
         Ya, la, rm = attention_impl(flat(Qc), flat(Kc), flat(Vc), flat(A) if gated else None, deg,
@@ -99,8 +139,9 @@ def make_power_retention(update_state_impl, query_state_impl, discumsum_impl, at
         else:
             Qg = Qc
         Y = query_state_impl(Qg.contiguous(), S.contiguous(), s.contiguous(), Ya.contiguous(), la.contiguous(),
-                             rm.contiguous(), deg, scale, True)                            # (:190)
-        return Y.contiguous().view(b, t, hq, d).to(dtype)
+                             rm.contiguous(), deg, scale, initial_state is None)           # (:190)
+        out = Y.contiguous().view(b, t, hq, d).to(dtype)
+        return (out, final) if return_final_state else out
 
     return power_retention
 

@@ -260,9 +260,14 @@ torch.library.register_autograd("pr::discumsum_fwd", _discumsum_backward, setup_
 def discumsum(X, log_G, keep_last=True):
     """Gated exclusive scan over axis 1: X [b, n, h, ...], log_G [b, n, h] fp32 -> [b, n+1, h, ...]
     (ref: retention/_discumsum/reference.py:3-15).  ``keep_last=False`` returns only the first n entries,
-    which is what the composed function keeps (ref: retention/power_retention_maker.py:167-170)."""
-    assert X.dim() >= 4 and log_G is not None and log_G.shape == X.shape[:3]
-    assert X.dtype in (*_HALF, torch.float32)
+    which is what the composed function keeps (ref: retention/power_retention_maker.py:167-170).
+    ``log_G=None`` is the reference's other branch (:4-5): the plain inclusive cumulative sum, n entries --
+    the same scan with every gate log 1, minus its leading zero."""
+    assert X.dim() >= 4 and X.dtype in (*_HALF, torch.float32)
+    if log_G is None:
+        zeros = torch.zeros(X.shape[:3], dtype=torch.float32, device=X.device)
+        return discumsum_fwd(X.contiguous(), zeros, X.shape[1] + 1)[:, 1:]
+    assert log_G.shape == X.shape[:3]
     n = X.shape[1]
     return discumsum_fwd(X.contiguous(), log_G.to(torch.float32).contiguous(), n + 1 if keep_last else n)
 

@@ -279,3 +279,23 @@ def test_symmetric_state_flag_changes_nothing_for_a_symmetric_state(pra, dtype, 
     for nm, a, b_ in zip(["dK", "dV", "dQ", "dS", "ds"], res[1], res[0]):
         check(f"{nm}: with the promise vs without", a, b_, 3e-3)
     assert torch.equal(res[0][1], res[1][1]) and torch.equal(res[0][3], res[1][3])
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_discumsum_without_gates_is_the_plain_cumsum(dtype):
+    """log_G = None: the reference's other branch (ref: retention/_discumsum/reference.py:4-5), n entries."""
+    import retention_integration_amd as pra
+    g = torch.Generator().manual_seed(3)
+    X = torch.randn(2, 6, 3, 40, 16, generator=g).to(dtype)
+    Xg = X.to("cuda").requires_grad_(True)
+    Y = pra.discumsum(Xg, None)
+    Xo = X.float().clone().requires_grad_(True)
+    Yo = oracle.discumsum(Xo, None)
+    assert Y.shape == Yo.shape == X.shape
+    W = torch.randn(X.shape, generator=g)
+    (Y.float() * W.to("cuda")).sum().backward()
+    (Yo * W).sum().backward()
+    for nm, a, b in (("Y", Y, Yo), ("dX", Xg.grad, Xo.grad)):
+        err = ((a.detach().float().cpu() - b.detach()).norm() / b.detach().norm()).item()
+        print(f"  {nm}: rel-L2 {err:.3e}", flush=True)
+        assert err <= (1e-2 if dtype == torch.bfloat16 else 1e-5)

@@ -192,3 +192,54 @@ def test_inference_state_parity():
     Y2, st2, sk2 = oracle.power_retention_inference(Q[:, -1:], None, None, None, st, sk, deg=2, switch_over_seq_len=9)
     torch.testing.assert_close(Y, Y2, rtol=1e-5, atol=1e-6)
     assert st2 is st and sk2 is sk
+
+
+# --------------------------------------------------------------------------
+# state carried across calls (initial_state / return_final_state): the product's own definition, pinned by the
+# closed form over the whole history and by the state the (golden-pinned) inference function forms
+# --------------------------------------------------------------------------
+@pytest.mark.parametrize("gated,r,chunk", [(True, 1, 8), (False, 2, 8), (True, 2, None)])
+def test_two_chained_calls_equal_the_closed_form_over_the_whole_sequence(gated, r, chunk):
+    b, t, h, d = 2, 32, 2, 16
+    Q, K, V, G = inputs(b, t, h, r, d, gated)
+    scale = 1.0 / math.sqrt(d)
+    want = closed_form(Q, K, V, G, scale)
+    half = t // 2
+    sl = lambda x, a, e: None if x is None else x[:, a:e]  # noqa: E731
+    y1, st = oracle.power_retention(Q[:, :half], K[:, :half], V[:, :half], sl(G, 0, half), return_final_state=True,
+                                    deg=2, chunk_size=chunk)
+    y2, st2 = oracle.power_retention(Q[:, half:], K[:, half:], V[:, half:], sl(G, half, t), initial_state=st,
+                                     return_final_state=True, deg=2, chunk_size=chunk)
+    torch.testing.assert_close(torch.cat([y1, y2], 1), want, rtol=1e-5, atol=1e-6)   # the eps terms are ~1e-6 relative
+    # one call over everything returns the same final state, and so does the inference function's prefill
+    _, st_all = oracle.power_retention(Q, K, V, G, return_final_state=True, deg=2, chunk_size=chunk or t)
+    _, S_inf, s_inf = oracle.power_retention_inference(Q[:, -1:], K, V, G, None, None, deg=2, switch_over_seq_len=t)
+    for a, b_, c_ in zip(st2, st_all, (S_inf, s_inf)):
+        # (the scan's first entry passes through fp32, as in the reference: retention/_discumsum/reference.py:10)
+        torch.testing.assert_close(a, b_, rtol=1e-5, atol=1e-5)
+        # (the training function rounds the gates to fp32 as the reference does, the inference function does not)
+        torch.testing.assert_close(a.double(), c_.double(), rtol=1e-5, atol=1e-5)
+
+
+def test_chained_calls_with_ragged_lengths_and_gradients():
+    """Padding must not touch the carried state, and gradients flow through it: the gradient of a loss over both
+    calls equals the gradient of the same loss over one call."""
+    b, t, h, r, d, chunk = 1, 27, 2, 2, 16, 8
+    Q, K, V, G = inputs(b, t, h, r, d, True)
+    W = torch.randn(b, t, h * r, d, dtype=torch.float64)
+    xs = [x.clone().requires_grad_(True) for x in (Q, K, V, G)]
+    (oracle.power_retention(*xs, deg=2, chunk_size=chunk) * W).sum().backward()
+    ys = [x.clone().requires_grad_(True) for x in (Q, K, V, G)]
+    cut = 13   # neither part is a chunk multiple
+    y1, st = oracle.power_retention(*(x[:, :cut] for x in ys), return_final_state=True, deg=2, chunk_size=chunk)
+    y2 = oracle.power_retention(*(x[:, cut:] for x in ys), initial_state=st, deg=2, chunk_size=chunk)
+    (torch.cat([y1, y2], 1) * W).sum().backward()
+    for a, b_ in zip(xs, ys):
+        # (the chunk boundaries differ between the two runs, and with them where the 1e-6 / 1e-7 terms enter)
+        torch.testing.assert_close(b_.grad, a.grad, rtol=1e-3, atol=1e-5)
+
+
+def test_discumsum_without_gates_is_the_inclusive_cumsum():
+    X = torch.randn(2, 5, 3, 4, 6, dtype=torch.float64)
+    torch.testing.assert_close(oracle.discumsum(X, None), X.cumsum(1))
+    torch.testing.assert_close(oracle.discumsum(X, torch.zeros(2, 5, 3, dtype=torch.float64))[:, 1:], X.cumsum(1))
