@@ -83,7 +83,7 @@ int pr_chunk_attention_bwd(const void* Q, const void* K, const void* V, const fl
   if (int rc = check_common("chunk_attention_bwd", d, deg, dtype, false)) return rc;
   if (bad_ptr(Q) || bad_ptr(K) || bad_ptr(V) || bad_ptr(rowmax) || bad_ptr(dO) || bad_ptr(dQ) || bad_ptr(dK) ||
       bad_ptr(dV) || bad_ptr(dQ_state) || bad_ptr(dK_state) || bad_ptr(dV_state) || bad_opt(A) || bad_opt(dl) ||
-      bad_opt(dGq) || bad_opt(dGk))
+      bad_opt(dGq) || bad_opt(dGk) || bad_opt(dotk))
     return fail(PR_ERR_ARG, "chunk_attention_bwd: null or misaligned pointer");
   if (A && (!dGq || !dGk || !dotk))
     return fail(PR_ERR_ARG, "chunk_attention_bwd: dGq, dGk and dotk are required when A is given");
@@ -227,8 +227,9 @@ int pr_update_state_scan_fwd(const void* K, const void* V, const float* log_G, v
   if (int rc = check_common("update_state_scan_fwd", d, deg, dtype, true)) return rc;
   if (bad_ptr(K) || bad_ptr(V) || bad_ptr(S_out) || bad_ptr(s_out))
     return fail(PR_ERR_ARG, "update_state_scan_fwd: null or misaligned pointer");
-  if (B <= 0 || n <= 0 || c <= 0 || h <= 0 || c % 64 != 0)
-    return fail(PR_ERR_ARG, "update_state_scan_fwd: need B,n,h > 0 and c a positive multiple of 64");
+  // (the same predicate as pr_state_chain_supported, so a shape the query accepts is never refused here)
+  if (B <= 0 || n <= 0 || c <= 0 || h <= 0 || !pr::sympow_tn_chain_ok(B, n < 2 ? 2 : n, c, h, 1, d))
+    return fail(PR_ERR_ARG, "update_state_scan_fwd: need B,n,h > 0 and c a positive multiple of the stage (64 rows, 32 at d = 128)");
   return finish(pr::sympow_tn_chain(K, V, nullptr, log_G, S_out, s_out, B, n, c, h, 1, d, 1, 0, dtype,
                                     (hipStream_t)stream), "update_state_scan_fwd");
 }
@@ -251,8 +252,9 @@ int pr_query_state_scan_bwd(const void* Q, const void* S, const float* s, const 
     return fail(PR_ERR_ARG, "query_state_scan_bwd: dl_attn and one of dY_attn, dY_scale are required when rowmax is given");
   if ((log_G != nullptr) != (dlog_G != nullptr))
     return fail(PR_ERR_ARG, "query_state_scan_bwd: log_G and dlog_G must be given together");
-  if (B <= 0 || n <= 0 || c <= 0 || h <= 0 || r <= 0 || 64 % r != 0 || ((long)c * r) % 64 != 0)
-    return fail(PR_ERR_ARG, "query_state_scan_bwd: need B,n,c,h > 0, r a divisor of 64 and c*r a multiple of 64");
+  if (B <= 0 || n <= 0 || c <= 0 || h <= 0 || r <= 0 || !pr::sympow_tn_chain_ok(B, n < 2 ? 2 : n, c, h, r, d))
+    return fail(PR_ERR_ARG, "query_state_scan_bwd: need B,n,c,h > 0, r a divisor of the stage (64 rows, 32 at d = 128) and "
+                            "c*r a multiple of it");
   const int BN = B * n;
   const size_t rows = (size_t)BN * c * h * r;
   const long D = 128L * (d / 16) * (d / 16 + 1);
