@@ -36,7 +36,8 @@ enum {
   PR_ERR_DEG = -4        /* unsupported degree */
 };
 
-/* 2: pr_update_state_bwd and pr_query_state_bwd take the symmetric-state promise (dS_symmetric, S_symmetric). */
+/* 2: pr_update_state_bwd and pr_query_state_bwd take the symmetric-state promise (dS_symmetric, S_symmetric).
+ * 3: pr_decode_step_noalloc. */
 int pr_abi_version(void);
 const char* pr_last_error(void);
 
@@ -111,8 +112,8 @@ int pr_state_scan_bwd(const void* dS_out, const void* S_out, const float* ds_out
  *   K, V [B,n*c,h,d] (keys already discounted), log_G [B,n,h] fp32 chunk gate sums or NULL (no decay)
  *   -> S_out [B*n,h,D,d], s_out [B*n,h,D] fp32 with S_out[b,0] = 0, S_out[b,k+1] = e^{log_G[b,k]} S_out[b,k] + phi(K_k)^T V_k.
  * A workgroup walks the chunks of a batch element serially, so this pays only when B*h is large and the chunks are
- * short.  pr_state_chain_supported() returns 0 when the shape is not supported (it needs c*r a multiple of 64, r a
- * divisor of 64, n >= 2), 1 when it is, 2 when it also has enough independent work to be the faster form
+ * short.  pr_state_chain_supported() returns 0 when the shape is not supported (it needs c*r a multiple of the 64-row
+ * stage and r a divisor of it -- 32 rows at d = 128 -- and n >= 2), 1 when it is, 2 when it also has enough independent work to be the faster form
  * (r = 1 on the key side, the query-head ratio on the query side). */
 int pr_state_chain_supported(int B, int n, int c, int h, int r, int d);
 int pr_update_state_scan_fwd(const void* K, const void* V, const float* log_G, void* S_out, float* s_out, int B, int n,
@@ -206,6 +207,19 @@ int pr_decode_step(const void* Q, const float* gq, const void* S, const float* s
                    const float* l_attn, const float* rowmax, const void* K_new, const void* V_new,
                    const float* log_decay, void* S_out, float* s_out, void* out, void* workspace, int B, int tq, int h,
                    int r, int d, float scale_p, int deg, int dtype, int attend_new, void* stream);
+
+/* pr_decode_step without a workspace argument.  No counterpart in the reference: it is for callers that cannot
+ * allocate device memory -- code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.
+ * The partial query sums live in an array of pr_decode_step_noalloc_max_workspace() bytes (8 MiB) that the library
+ * holds on every GPU it runs on until the process ends; the call allocates and frees nothing.  A step whose
+ * pr_decode_step_workspace() exceeds that size is refused with PR_ERR_ARG (use pr_decode_step).  All calls on one
+ * GPU share the array: calls that overlap in time on one GPU (two streams) race; calls on one stream do not.
+ * Same arguments, results and in-place rules as pr_decode_step. */
+size_t pr_decode_step_noalloc_max_workspace(void);
+int pr_decode_step_noalloc(const void* Q, const float* gq, const void* S, const float* s, const void* Y_attn,
+                           const float* l_attn, const float* rowmax, const void* K_new, const void* V_new,
+                           const float* log_decay, void* S_out, float* s_out, void* out, int B, int tq, int h, int r,
+                           int d, float scale_p, int deg, int dtype, int attend_new, void* stream);
 
 #ifdef __cplusplus
 }

@@ -47,6 +47,8 @@ SIGNATURES = {
     "pr_chunk_gate_scan_bwd": (c_int, [_P] * 5 + [_I] * 5 + [_P]),
     "pr_decode_step_workspace": (c_size_t, [_I] * 5),
     "pr_decode_step": (c_int, [_P] * 14 + [_I] * 5 + [_F, _I, _I, _I, _P]),
+    "pr_decode_step_noalloc_max_workspace": (c_size_t, []),
+    "pr_decode_step_noalloc": (c_int, [_P] * 13 + [_I] * 5 + [_F, _I, _I, _I, _P]),
 }
 
 _lib = None

@@ -38,7 +38,7 @@ size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 
 extern "C" {
 
-int pr_abi_version(void) { return 2; }
+int pr_abi_version(void) { return 3; }
 const char* pr_last_error(void) { return g_err; }
 
 int pr_expanded_dim(int d, int deg) {
@@ -308,27 +308,59 @@ size_t pr_decode_step_workspace(int B, int tq, int h, int r, int d) {
   return align256((size_t)pr::decode_workspace_floats(B, h, r, tq, d) * sizeof(float));
 }
 
+namespace {
+// argument checks shared by pr_decode_step and pr_decode_step_noalloc
+int check_decode(const char* what, const void* Q, const void* S, const float* s, const void* Y_attn, const float* l_attn,
+                 const float* rowmax, const void* K_new, const void* V_new, const void* S_out, const float* s_out,
+                 const void* out, int B, int tq, int h, int r, int d, int deg, int dtype, int attend_new) {
+  if (int rc = check_common(what, d, deg, dtype, true)) return rc;
+  if (attend_new && (!K_new || tq != 1 || Y_attn))
+    return fail(PR_ERR_ARG, "%s: attend_new needs K_new, V_new, tq == 1 and no separate attention part", what);
+  if (bad_ptr(Q) || bad_ptr(S) || bad_ptr(s) || bad_ptr(out) || bad_opt(Y_attn) || bad_opt(K_new) || bad_opt(V_new) ||
+      bad_opt(S_out))
+    return fail(PR_ERR_ARG, "%s: null or misaligned pointer", what);
+  if ((Y_attn != nullptr) != (l_attn != nullptr) || (Y_attn != nullptr) != (rowmax != nullptr))
+    return fail(PR_ERR_ARG, "%s: Y_attn, l_attn and rowmax must be given together", what);
+  if (K_new && (!V_new || !S_out || !s_out)) return fail(PR_ERR_ARG, "%s: V_new, S_out and s_out are required with K_new", what);
+  if (K_new && ((S_out == S) != (s_out == s)))
+    return fail(PR_ERR_ARG, "%s: update S and s both in place or both out of place", what);
+  if (B <= 0 || tq <= 0 || h <= 0 || r <= 0) return fail(PR_ERR_ARG, "%s: need B,tq,h,r > 0", what);
+  if (tq * r > 8) return fail(PR_ERR_ARG, "%s: at most 8 query rows per (batch, kv head) (got %d)", what, tq * r);
+  return 0;
+}
+}  // namespace
+
 int pr_decode_step(const void* Q, const float* gq, const void* S, const float* s, const void* Y_attn,
                    const float* l_attn, const float* rowmax, const void* K_new, const void* V_new,
                    const float* log_decay, void* S_out, float* s_out, void* out, void* workspace, int B, int tq, int h,
                    int r, int d, float scale_p, int deg, int dtype, int attend_new, void* stream) {
-  if (int rc = check_common("decode_step", d, deg, dtype, true)) return rc;
-  if (attend_new && (!K_new || tq != 1 || Y_attn))
-    return fail(PR_ERR_ARG, "decode_step: attend_new needs K_new, V_new, tq == 1 and no separate attention part");
-  if (bad_ptr(Q) || bad_ptr(S) || bad_ptr(s) || bad_ptr(out) || bad_ptr(workspace) || bad_opt(Y_attn) ||
-      bad_opt(K_new) || bad_opt(V_new) || bad_opt(S_out))
-    return fail(PR_ERR_ARG, "decode_step: null or misaligned pointer");
-  if ((Y_attn != nullptr) != (l_attn != nullptr) || (Y_attn != nullptr) != (rowmax != nullptr))
-    return fail(PR_ERR_ARG, "decode_step: Y_attn, l_attn and rowmax must be given together");
-  if (K_new && (!V_new || !S_out || !s_out)) return fail(PR_ERR_ARG, "decode_step: V_new, S_out and s_out are required with K_new");
-  if (K_new && ((S_out == S) != (s_out == s)))
-    return fail(PR_ERR_ARG, "decode_step: update S and s both in place or both out of place");
-  if (B <= 0 || tq <= 0 || h <= 0 || r <= 0) return fail(PR_ERR_ARG, "decode_step: need B,tq,h,r > 0");
-  if (tq * r > 8) return fail(PR_ERR_ARG, "decode_step: at most 8 query rows per (batch, kv head) (got %d)", tq * r);
+  if (int rc = check_decode("decode_step", Q, S, s, Y_attn, l_attn, rowmax, K_new, V_new, S_out, s_out, out, B, tq, h, r,
+                            d, deg, dtype, attend_new))
+    return rc;
+  if (bad_ptr(workspace)) return fail(PR_ERR_ARG, "decode_step: null or misaligned workspace");
   return finish(pr::decode_step(Q, gq, S, s, Y_attn, l_attn, rowmax, K_new, V_new, log_decay, S_out, s_out, out,
                                 (float*)workspace, B, tq, h, r, d, deg, scale_p, dtype, attend_new ? 1 : 0,
                                 (hipStream_t)stream),
                 "decode_step");
+}
+
+size_t pr_decode_step_noalloc_max_workspace(void) { return (size_t)pr::decode_static_floats() * sizeof(float); }
+
+int pr_decode_step_noalloc(const void* Q, const float* gq, const void* S, const float* s, const void* Y_attn,
+                           const float* l_attn, const float* rowmax, const void* K_new, const void* V_new,
+                           const float* log_decay, void* S_out, float* s_out, void* out, int B, int tq, int h, int r,
+                           int d, float scale_p, int deg, int dtype, int attend_new, void* stream) {
+  if (int rc = check_decode("decode_step_noalloc", Q, S, s, Y_attn, l_attn, rowmax, K_new, V_new, S_out, s_out, out, B,
+                            tq, h, r, d, deg, dtype, attend_new))
+    return rc;
+  const size_t need = pr_decode_step_workspace(B, tq, h, r, d);
+  if (need > pr_decode_step_noalloc_max_workspace())
+    return fail(PR_ERR_ARG, "decode_step_noalloc: this step needs %zu bytes of partial sums, the library's array holds %zu "
+                            "(use pr_decode_step with a workspace)", need, pr_decode_step_noalloc_max_workspace());
+  const int rc = pr::decode_step_static(Q, gq, S, s, Y_attn, l_attn, rowmax, K_new, V_new, log_decay, S_out, s_out, out,
+                                        B, tq, h, r, d, deg, scale_p, dtype, attend_new ? 1 : 0, (hipStream_t)stream);
+  if (rc == -6) return fail(PR_ERR_ARG, "decode_step_noalloc: the step needs more partial sums than the library's array holds");
+  return finish(rc, "decode_step_noalloc");
 }
 
 }  // extern "C"

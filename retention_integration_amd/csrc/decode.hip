@@ -17,10 +17,18 @@
 // in registers and writes the updated rows.  A second, tiny kernel adds the partials of the slices and merges; with
 // many (batch, kv head) pairs and one or two query rows a single 1024-thread workgroup takes a whole pair and merges
 // in the same kernel.
+#include <mutex>
+
 #include "common.h"
 #include "kernels.h"
 
 namespace pr {
+
+// Partial query sums of decode_step_static() (below): device memory that belongs to the library, one copy per GPU,
+// held until the process ends.  In host code this name is only a handle for hipGetSymbolAddress -- never a device
+// address: kernels get the address that call returns.
+constexpr long DEC_STATIC_FLOATS = 2L << 20;   // 8 MiB
+static __device__ __align__(256) float scratch[DEC_STATIC_FLOATS];
 
 constexpr int DEC_MAXROWS = 8;   // query rows (positions x query heads per kv head) handled per (batch, kv head)
 
@@ -306,6 +314,39 @@ int decode_step(const void* Q, const float* gq, const void* S, const float* s, c
   if (dtype == DT_F16) { PR_DEC(f16_t) }
 #undef PR_DEC
   return -1;
+}
+
+long decode_static_floats() { return DEC_STATIC_FLOATS; }
+
+// decode_step with the partial sums in the library's own per-GPU array instead of a caller's workspace: nothing is
+// allocated here or below.  Every slice of every (batch, kv head) writes all of its partial sums before the merge
+// kernel reads them, so nothing has to be cleared between calls; two calls in flight on one GPU at the same time
+// would share the array and race.  Returns -6 when the step needs more than the array holds, or a positive
+// hipError_t if the array's address cannot be obtained.
+int decode_step_static(const void* Q, const float* gq, const void* S, const float* s, const void* Y_attn,
+                       const float* l_attn, const float* rowmax, const void* Knew, const void* Vnew,
+                       const float* decay, void* Sout, float* sout, void* out, int B, int tq, int h, int r, int d,
+                       int deg, float scale_p, int dtype, int attend_new, hipStream_t st) {
+  constexpr int MAX_DEVICES = 64;
+  static std::mutex mu;
+  static float* ptr[MAX_DEVICES] = {};   // the array's address on each GPU (each holds its own copy)
+  if (decode_workspace_floats(B, h, r, tq, d) > DEC_STATIC_FLOATS) return -6;
+  int dev = -1;
+  if (hipError_t e = hipGetDevice(&dev)) return (int)e;
+  if (dev < 0 || dev >= MAX_DEVICES) return (int)hipErrorInvalidDevice;
+  float* part;
+  {
+    std::lock_guard<std::mutex> lock(mu);
+    if (!ptr[dev]) {   // first call on this GPU, which is the current one
+      float* p = nullptr;
+      if (hipError_t e = hipGetSymbolAddress((void**)&p, HIP_SYMBOL(scratch))) return (int)e;
+      if (!p) return (int)hipErrorInvalidSymbol;
+      ptr[dev] = p;
+    }
+    part = ptr[dev];
+  }
+  return decode_step(Q, gq, S, s, Y_attn, l_attn, rowmax, Knew, Vnew, decay, Sout, sout, out, part, B, tq, h, r, d, deg,
+                     scale_p, dtype, attend_new, st);
 }
 
 }  // namespace pr

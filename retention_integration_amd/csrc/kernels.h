@@ -120,4 +120,12 @@ int decode_step(const void* Q, const float* gq, const void* S, const float* s, c
                 void* out, float* workspace, int B, int tq, int h, int r, int d, int deg, float scale_p, int dtype,
                 int attend_new, hipStream_t st);
 
+// the same step with its partial sums in a per-GPU array of the library (return -6: the step needs more than
+// decode_static_floats() floats of partial sums)
+long decode_static_floats();
+int decode_step_static(const void* Q, const float* gq, const void* S, const float* s, const void* Y_attn,
+                       const float* l_attn, const float* rowmax, const void* Knew, const void* Vnew,
+                       const float* decay, void* Sout, float* sout, void* out, int B, int tq, int h, int r, int d,
+                       int deg, float scale_p, int dtype, int attend_new, hipStream_t st);
+
 }  // namespace pr
