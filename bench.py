@@ -93,7 +93,7 @@ def op_breakdown(pra, Q, K, V, lg, dO, cfg, iters=5):
     lib = _lib.load()
     dK = torch.empty_like(Kc)
     grad_only = lambda: _lib.check(lib.pr_update_state_bwd(  # noqa: E731
-        _lib.ptr(Kc), _lib.ptr(Vc), _lib.ptr(S), _lib.ptr(s), _lib.ptr(dK), None, b * n, c, h, d, 2, 1,
+        _lib.ptr(Kc), _lib.ptr(Vc), _lib.ptr(S), _lib.ptr(s), _lib.ptr(dK), None, b * n, c, h, d, 2, 1, 0,
         _lib.dtype_code(Kc.dtype), _lib.stream()), "update_state_bwd(dK)")
     res["sympow_grad(dK)"] = event_time_ms(grad_only, iters)
     return {k: round(v, 4) for k, v in res.items()}
@@ -114,7 +114,7 @@ def counter_run(pra, Q, K, V, cfg, dev):
         torch.cuda.synchronize()
         for _ in range(3):
             _lib.check(lib.pr_update_state_bwd(_lib.ptr(Kc), _lib.ptr(Vc), _lib.ptr(S), _lib.ptr(s), _lib.ptr(dK), None,
-                                               b * n, c, h, d, 2, 1, _lib.dtype_code(Kc.dtype), _lib.stream()), "grad")
+                                               b * n, c, h, d, 2, 1, 0, _lib.dtype_code(Kc.dtype), _lib.stream()), "grad")
             dst.copy_(src)
         torch.cuda.synchronize()
     print("counter run done: 3 x sympow_grad, 3 x 256 MiB device copy")

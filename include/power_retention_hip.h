@@ -37,7 +37,8 @@ enum {
 };
 
 /* 2: pr_update_state_bwd and pr_query_state_bwd take the symmetric-state promise (dS_symmetric, S_symmetric).
- * 3: pr_decode_step_noalloc. */
+ * 3: pr_decode_step_noalloc.  4: pr_cache_append, pr_cache_attention_fwd; pr_update_state_fwd takes skip_last_of and
+ * pr_update_state_bwd zero_last_of. */
 int pr_abi_version(void);
 const char* pr_last_error(void);
 
@@ -68,18 +69,22 @@ int pr_attention_bwd(const void* Q, const void* K, const void* V, const float* G
 
 /* update_state(K, V, deg) -- retention/_update_state/reference.py:33-52,86-94,
  * Triton twin retention/_update_state/triton.py:61-133,280-320.
- *   K, V [BN,c,h,d] (BN = b*n chunks) -> S [BN,h,D,d], s [BN,h,D] fp32. */
+ *   K, V [BN,c,h,d] (BN = b*n chunks) -> S [BN,h,D,d], s [BN,h,D] fp32.
+ *   skip_last_of = n > 0: the last of every n chunks is not computed and its S, s are left unwritten (the composed
+ *   function never reads the last chunk's state, retention/power_retention_maker.py:168-170); 0 computes every chunk. */
 int pr_update_state_fwd(const void* K, const void* V, void* S, float* s, int BN, int c, int h, int d, int deg,
-                        int dtype, void* stream);
+                        int skip_last_of, int dtype, void* stream);
 
 /* Backward -- retention/_update_state/reference.py:55-83, Triton twin retention/_update_state/triton.py:148-260.
  *   dS [BN,h,D,d], ds [BN,h,D] fp32 -> dK, dV [BN,c,h,d]; one of dK, dV may be NULL (that gradient is skipped).
  *   dS_symmetric != 0 is the caller's promise that dS[(a,b)] == dS[(b,a)] for the pairs the layout stores in both
  *   orders (the 16x16 blocks on the diagonal); true of the dS that pr_query_state_bwd and the scans produce, not of
  *   an arbitrary tensor.  The key gradient then takes a shorter path through those blocks; with 0 every feature is
- *   used as given, as the reference does. */
+ *   used as given, as the reference does.
+ *   zero_last_of = n > 0 is the promise that dS, ds of the last of every n chunks are zero (that chunk's state feeds
+ *   nothing): they are not read and dK, dV are written as zeros there; 0 makes no such promise. */
 int pr_update_state_bwd(const void* K, const void* V, const void* dS, const float* ds, void* dK, void* dV, int BN,
-                        int c, int h, int d, int deg, int dS_symmetric, int dtype, void* stream);
+                        int c, int h, int d, int deg, int dS_symmetric, int zero_last_of, int dtype, void* stream);
 
 /* discumsum(X, log_G) -- retention/_discumsum/reference.py:3-15, Triton twin retention/_discumsum/triton.py:34-94.
  *   X [B,n,H,F], log_G [B,n,H] fp32 -> Y [B,n_out,H,F], Y[0]=0, Y[k+1]=Y[k]*exp(log_G[k])+X[k];
@@ -147,6 +152,9 @@ int pr_query_state_fwd(const void* Q, const void* S, const float* s, const void*
  *      dY_attn [BN,c,h*r,d], dl_attn [BN,c,h*r] fp32.  dY_attn is dO times a per-row factor; a consumer that scales
  *      on the fly (the dO_scale argument of the attention backward) can ask for that factor instead:
  *      dY_scale [BN,c,h*r] fp32 (then dY_attn may be NULL).
+ *   zero_initial_state: 1 as in the forward; 2 additionally declares that nobody needs the gradient of the first
+ *   chunk's (zero) state: dS, ds of the first of every n chunks are then written as zeros instead of computed (the
+ *   composed function discards them, retention/power_retention_maker.py:167-170).
  *   workspace: pr_query_state_bwd_workspace() bytes (scaled dO and two fp32 row vectors).
  *   S_symmetric != 0: the caller's promise that S[(a,b)] == S[(b,a)] in the blocks on the diagonal (true of every
  *   state made by pr_update_state_fwd and the scans); the query gradient then takes a shorter path through them. */
@@ -207,6 +215,22 @@ int pr_decode_step(const void* Q, const float* gq, const void* S, const float* s
                    const float* l_attn, const float* rowmax, const void* K_new, const void* V_new,
                    const float* log_decay, void* S_out, float* s_out, void* out, void* workspace, int B, int tq, int h,
                    int r, int d, float scale_p, int deg, int dtype, int attend_new, void* stream);
+
+/* Preallocated K / V / gate cache of the decode loop -- replaces the three torch.cat per layer and step of
+ * deploy/models/powercoder/kvgs_dynamic_cache.py:131-161 (DynamicLayer.update_kv) and the cumulative sum over the whole
+ * cache of retention/power_retention_maker.py:347.
+ *   K_cache, V_cache [B,capacity,h,d], A_cache [B,capacity,h] fp32: ACCUMULATED log gates since the start of the cache;
+ *   K_new, V_new [B,t_new,h,d], log_G_new [B,t_new,h] fp32 or NULL (no gates: zeros are written)
+ *   -> rows pos .. pos+t_new-1 of the three buffers (A_cache[pos+i] = A_cache[pos-1] + log_G_new[0] + ... + log_G_new[i],
+ *      A_cache[-1] = 0); A_last [B,h] fp32 or NULL also receives the last of them (dense: the gq argument of
+ *      pr_decode_step).  The caller keeps the length; rows beyond it are never read.
+ * pr_cache_attention_fwd is pr_attention_fwd over the first tk rows of such buffers (batch stride = capacity rows). */
+int pr_cache_append(void* K_cache, void* V_cache, float* A_cache, const void* K_new, const void* V_new,
+                    const float* log_G_new, float* A_last, int B, int capacity, int pos, int t_new, int h, int d,
+                    int dtype, void* stream);
+int pr_cache_attention_fwd(const void* Q, const void* K_cache, const void* V_cache, const float* A_cache, void* O, float* l,
+                           float* rowmax, int B, int tq, int tk, int capacity, int h, int r, int d, float scale, int deg,
+                           int norm, int dtype, void* stream);
 
 /* pr_decode_step without a workspace argument.  No counterpart in the reference: it is for callers that cannot
  * allocate device memory -- code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.

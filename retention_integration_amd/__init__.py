@@ -13,6 +13,7 @@ maker-assembled form.
 """
 from functools import partial
 
+from .cache import RetentionCache
 from .fused import chunked_power_retention
 from .inference import make_fused_inference
 from .maker import make_power_retention, make_power_retention_inference
@@ -31,4 +32,5 @@ __all__ = [
     "power_retention", "power_retention_composed", "power_retention_inference",
     "power_retention_inference_composed", "make_power_retention",
     "make_power_retention_inference", "attention", "update_state", "discumsum", "query_state", "expanded_dim",
+    "RetentionCache",
 ]

@@ -77,9 +77,9 @@ __global__ __launch_bounds__(256, OCC) void attention_fwd_kernel(AttnFwdArgs a, 
   // diagonal has the most tiles, and co-resident workgroups then load the four SIMDs evenly
   const int row0 = rblk * ROWS;
   const T* Qg = (const T*)a.Q + (long)b * a.tq * hq * DH;
-  const char* Kg = (const char*)((const T*)a.K + (long)b * a.tk * a.h * DH + hh * DH);
-  const char* Vg = (const char*)((const T*)a.V + (long)b * a.tk * a.h * DH + hh * DH);
-  const float* Gg = a.G ? a.G + (long)b * a.tk * a.h + hh : nullptr;
+  const char* Kg = (const char*)((const T*)a.K + (long)b * a.kv_rows * a.h * DH + hh * DH);
+  const char* Vg = (const char*)((const T*)a.V + (long)b * a.kv_rows * a.h * DH + hh * DH);
+  const float* Gg = a.G ? a.G + (long)b * a.kv_rows * a.h + hh : nullptr;
   const long kstride = (long)a.h * DH * 2;
   const int half_deg = (int)a.deg / 2;
   const float eps_s = AT_LOG_EPS / a.scale;          // |scale*x| + eps = scale * (|x| + eps/scale)

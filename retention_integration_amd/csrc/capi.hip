@@ -38,7 +38,7 @@ size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 
 extern "C" {
 
-int pr_abi_version(void) { return 3; }
+int pr_abi_version(void) { return 4; }
 const char* pr_last_error(void) { return g_err; }
 
 int pr_expanded_dim(int d, int deg) {
@@ -55,7 +55,7 @@ int pr_attention_fwd(const void* Q, const void* K, const void* V, const float* G
   if (!norm && (!l || !rowmax)) return fail(PR_ERR_ARG, "attention_fwd: l and rowmax are required when norm == 0");
   if (B <= 0 || tq <= 0 || tk <= 0 || h <= 0 || r <= 0 || tq > tk)
     return fail(PR_ERR_ARG, "attention_fwd: need B,tq,tk,h,r > 0 and tq <= tk (got %d %d %d %d %d)", B, tq, tk, h, r);
-  pr::AttnFwdArgs a{Q, K, V, G, O, l, rowmax, tq, tk, h, r, scale, (float)deg, norm};
+  pr::AttnFwdArgs a{Q, K, V, G, O, l, rowmax, tq, tk, h, r, scale, (float)deg, norm, tk};
   return finish(pr::attention_fwd(a, B, d, dtype, (hipStream_t)stream), "attention_fwd");
 }
 
@@ -94,25 +94,31 @@ int pr_chunk_attention_bwd(const void* Q, const void* K, const void* V, const fl
 }
 
 int pr_update_state_fwd(const void* K, const void* V, void* S, float* s, int BN, int c, int h, int d, int deg,
-                        int dtype, void* stream) {
+                        int skip_last_of, int dtype, void* stream) {
   if (int rc = check_common("update_state_fwd", d, deg, dtype, true)) return rc;
   if (bad_ptr(K) || bad_ptr(V) || bad_ptr(S) || bad_ptr(s)) return fail(PR_ERR_ARG, "update_state_fwd: null or misaligned pointer");
   if (BN <= 0 || c <= 0 || h <= 0) return fail(PR_ERR_ARG, "update_state_fwd: need BN,c,h > 0");
-  return finish(pr::sympow_tn(K, V, nullptr, S, s, BN, c, h, 1, d, 1, dtype, (hipStream_t)stream), "update_state_fwd");
+  if (skip_last_of < 0 || (skip_last_of > 0 && BN % skip_last_of != 0))
+    return fail(PR_ERR_ARG, "update_state_fwd: skip_last_of must be 0 or a divisor of BN (got %d, BN %d)", skip_last_of, BN);
+  return finish(pr::sympow_tn(K, V, nullptr, S, s, BN, c, h, 1, d, 1, skip_last_of, dtype, (hipStream_t)stream),
+                "update_state_fwd");
 }
 
 int pr_update_state_bwd(const void* K, const void* V, const void* dS, const float* ds, void* dK, void* dV, int BN,
-                        int c, int h, int d, int deg, int dS_symmetric, int dtype, void* stream) {
+                        int c, int h, int d, int deg, int dS_symmetric, int zero_last_of, int dtype, void* stream) {
   if (int rc = check_common("update_state_bwd", d, deg, dtype, true)) return rc;
   if (bad_ptr(K) || bad_ptr(V) || bad_ptr(dS) || bad_ptr(ds) || bad_opt(dK) || bad_opt(dV) || (!dK && !dV))
     return fail(PR_ERR_ARG, "update_state_bwd: null or misaligned pointer");
   if (BN <= 0 || c <= 0 || h <= 0) return fail(PR_ERR_ARG, "update_state_bwd: need BN,c,h > 0");
+  if (zero_last_of < 0 || (zero_last_of > 0 && BN % zero_last_of != 0))
+    return fail(PR_ERR_ARG, "update_state_bwd: zero_last_of must be 0 or a divisor of BN (got %d, BN %d)", zero_last_of, BN);
+  const int nn_ = zero_last_of > 0 ? zero_last_of : 1, skl = zero_last_of > 0 ? 1 : 0;
   if (dV) {
-    pr::NNArgs nn{K, dS, nullptr, dV, nullptr, nullptr, nullptr, nullptr, 1.f, c, h, 1, 1, 0};
+    pr::NNArgs nn{K, dS, nullptr, dV, nullptr, nullptr, nullptr, nullptr, 1.f, c, h, 1, nn_, 0, skl};
     if (int rc = finish(pr::sympow_nn(nn, BN, d, 1, 0, dtype, (hipStream_t)stream), "update_state_bwd(dV)")) return rc;
   }
   if (!dK) return 0;
-  pr::GradArgs g{K, V, nullptr, dS, ds, dK, c, h, 1, 1, 0, dS_symmetric ? 1 : 0};
+  pr::GradArgs g{K, V, nullptr, dS, ds, dK, c, h, 1, nn_, 0, dS_symmetric ? 1 : 0, skl};
   return finish(pr::sympow_grad(g, BN, d, 1, dtype, (hipStream_t)stream), "update_state_bwd(dK)");
 }
 
@@ -181,7 +187,7 @@ int pr_query_state_fwd(const void* Q, const void* S, const float* s, const void*
     return fail(PR_ERR_ARG, "query_state_fwd: Y_attn, l_attn and rowmax must be given together");
   if (BN <= 0 || n <= 0 || c <= 0 || h <= 0 || r <= 0 || BN % n != 0)
     return fail(PR_ERR_ARG, "query_state_fwd: need BN,n,c,h,r > 0 and BN a multiple of n");
-  pr::NNArgs a{Q, S, s, O, den, Y_attn, l_attn, rowmax, scale_p, c, h, r, n, zero_initial_state ? 1 : 0};
+  pr::NNArgs a{Q, S, s, O, den, Y_attn, l_attn, rowmax, scale_p, c, h, r, n, zero_initial_state ? 1 : 0, 0};
   return finish(pr::sympow_nn(a, BN, d, 0, 1, dtype, (hipStream_t)stream), "query_state_fwd");
 }
 
@@ -212,8 +218,11 @@ int pr_query_state_bwd(const void* Q, const void* S, const float* s, const float
                                       dtype, st),
                       "query_state_bwd(prep)"))
     return rc;
-  if (int rc = finish(pr::sympow_tn(Q, dOs, cvec, dS, ds, BN, c, h, r, d, 0, dtype, st), "query_state_bwd(dS)")) return rc;
-  pr::GradArgs g{Q, dOs, cvec, S, s, dQ, c, h, r, n, zero_initial_state ? 1 : 0, S_symmetric ? 1 : 0};
+  // (zero_initial_state == 2: the caller does not want the gradient of the first chunk's (zero) state either)
+  if (int rc = finish(pr::sympow_tn(Q, dOs, cvec, dS, ds, BN, c, h, r, d, 0, zero_initial_state == 2 ? -n : 0, dtype, st),
+                      "query_state_bwd(dS)"))
+    return rc;
+  pr::GradArgs g{Q, dOs, cvec, S, s, dQ, c, h, r, n, zero_initial_state ? 1 : 0, S_symmetric ? 1 : 0, 0};
   return finish(pr::sympow_grad(g, BN, d, 0, dtype, st), "query_state_bwd(dQ)");
 }
 
@@ -274,7 +283,7 @@ int pr_query_state_scan_bwd(const void* Q, const void* S, const float* s, const 
     if (int rc = finish(pr::scan_gate_grad(S, dS_in, s, ds_in, log_G, dlog_G, part, B, n, h, D * d, D, dtype, st),
                         "query_state_scan_bwd(dlog_G)"))
       return rc;
-  pr::GradArgs g{Q, dOs, cvec, S, s, dQ, c, h, r, n, 1};
+  pr::GradArgs g{Q, dOs, cvec, S, s, dQ, c, h, r, n, 1, 0, 0};
   return finish(pr::sympow_grad(g, BN, d, 0, dtype, st), "query_state_scan_bwd(dQ)");
 }
 
@@ -302,6 +311,34 @@ int pr_chunk_gate_scan_bwd(float* dlog_G, const float* dGq, const float* dotk, c
     return fail(PR_ERR_ARG, "chunk_gate_scan_bwd: need BN,c,h,r,deg > 0");
   return finish(pr::chunk_gate_scan_bwd(dlog_G, dGq, dotk, dlcs_a, dlcs_b, BN, c, h, r, deg, (hipStream_t)stream),
                 "chunk_gate_scan_bwd");
+}
+
+int pr_cache_append(void* K_cache, void* V_cache, float* A_cache, const void* K_new, const void* V_new,
+                    const float* log_G_new, float* A_last, int B, int capacity, int pos, int t_new, int h, int d,
+                    int dtype, void* stream) {
+  if (dtype != PR_BF16 && dtype != PR_F16) return fail(PR_ERR_DTYPE, "cache_append: dtype must be bf16 or fp16");
+  if (d <= 0 || d % 8 != 0) return fail(PR_ERR_HEAD_DIM, "cache_append: head dim must be a positive multiple of 8 (got %d)", d);
+  if (bad_ptr(K_cache) || bad_ptr(V_cache) || !A_cache || bad_ptr(K_new) || bad_ptr(V_new))
+    return fail(PR_ERR_ARG, "cache_append: null or misaligned pointer");
+  if (B <= 0 || h <= 0 || t_new <= 0 || pos < 0 || (long)pos + t_new > capacity)
+    return fail(PR_ERR_ARG, "cache_append: need B,h,t_new > 0 and 0 <= pos, pos + t_new <= capacity (got pos %d + %d, "
+                            "capacity %d)", pos, t_new, capacity);
+  return finish(pr::cache_append(K_cache, V_cache, A_cache, K_new, V_new, log_G_new, A_last, B, capacity, pos, t_new, h, d, dtype,
+                                 (hipStream_t)stream), "cache_append");
+}
+
+int pr_cache_attention_fwd(const void* Q, const void* K_cache, const void* V_cache, const float* A_cache, void* O, float* l,
+                           float* rowmax, int B, int tq, int tk, int capacity, int h, int r, int d, float scale, int deg,
+                           int norm, int dtype, void* stream) {
+  if (int rc = check_common("cache_attention_fwd", d, deg, dtype, false)) return rc;
+  if (bad_ptr(Q) || bad_ptr(K_cache) || bad_ptr(V_cache) || bad_ptr(O) || bad_opt(A_cache) || bad_opt(l) || bad_opt(rowmax))
+    return fail(PR_ERR_ARG, "cache_attention_fwd: null or misaligned pointer");
+  if (!norm && (!l || !rowmax)) return fail(PR_ERR_ARG, "cache_attention_fwd: l and rowmax are required when norm == 0");
+  if (B <= 0 || tq <= 0 || tk <= 0 || h <= 0 || r <= 0 || tq > tk || tk > capacity)
+    return fail(PR_ERR_ARG, "cache_attention_fwd: need B,tq,tk,h,r > 0 and tq <= tk <= capacity (got %d %d %d %d)", B, tq, tk,
+                capacity);
+  pr::AttnFwdArgs a{Q, K_cache, V_cache, A_cache, O, l, rowmax, tq, tk, h, r, scale, (float)deg, norm, capacity};
+  return finish(pr::attention_fwd(a, B, d, dtype, (hipStream_t)stream), "cache_attention_fwd");
 }
 
 size_t pr_decode_step_workspace(int B, int tq, int h, int r, int d) {

@@ -23,8 +23,10 @@ int scan_gate_grad(const void* Y, const void* R, const float* Y2, const float* R
                    float* partial, int B, int n, int H, long F, long F2, int dtype, hipStream_t st);
 
 // sympow_tn.hip: A [BN,c,h*r,d], Bm [BN,c,h*r,d], w [BN,c,h*r] or null -> S [BN,h,D,d], s [BN,h,D]
+// skip: 0 = every chunk; +n = the last chunk of every n is not computed and its S, s are left unwritten (nobody reads
+// them); -n = the first chunk of every n is not computed and its S, s are written as zeros.
 int sympow_tn(const void* A, const void* Bm, const float* w, void* S, float* s, int BN, int c, int h, int r, int d,
-              int use_mult, int dtype, hipStream_t st);
+              int use_mult, int skip, int dtype, hipStream_t st);
 // The same contraction chained with the gated scan over the n chunks of a batch element (A, Bm [B,n*c,h*r,d],
 // lcs [B,n,h] or null): entry k of S, s [B*n,h,D,*] is the scan's k-th value (forward) or the scan's input gradient
 // (reverse).  sympow_tn_chain_ok: 0 = shape not supported, 1 = supported, 2 = and enough independent work to pay.
@@ -46,6 +48,7 @@ struct NNArgs {
   float scale_p;        // scale^deg
   int c, h, r, n;       // n: chunks per batch entry
   int skip_first;       // chunk 0 of every batch entry has a zero state
+  int skip_last;        // chunk n-1 of every batch entry has a zero B: the output there is zero (nothing is read)
 };
 int sympow_nn(const NNArgs& a, int BN, int d, int mult, int epi, int dtype, hipStream_t st);
 
@@ -60,6 +63,7 @@ struct GradArgs {
   int c, h, r, n;
   int skip_first;     // chunk 0 of every batch entry has a zero state: dX = 0 there
   int sym_diag;       // B[(a, b)] == B[(b, a)] in the blocks on the diagonal (the caller's promise)
+  int skip_last;      // chunk n-1 of every batch entry has a zero B: dX = 0 there (nothing is read)
 };
 int sympow_grad(const GradArgs& a, int BN, int d, int mult, int dtype, hipStream_t st);
 
@@ -75,6 +79,7 @@ struct AttnFwdArgs {
   int tq, tk, h, r;
   float scale, deg;
   int norm;
+  int kv_rows;      // rows per batch entry of the K, V, G buffers (tk for dense tensors, the capacity of a cache)
 };
 int attention_fwd(const AttnFwdArgs& a, int B, int d, int dtype, hipStream_t st);
 struct AttnBwdArgs {
@@ -112,6 +117,10 @@ int chunk_prep_fwd(const float* logG, const void* K, const void* Q, float* A, fl
                    int c, int h, int r, int d, int deg, int dtype, hipStream_t st);
 int chunk_gate_scan_bwd(float* dA, const float* dGq, const float* dotk, const float* dlcs_a, const float* dlcs_b, int BN,
                         int c, int h, int r, int deg, hipStream_t st);
+
+// cache.hip
+int cache_append(void* Kc, void* Vc, float* Ac, const void* k, const void* v, const float* g, float* a_last, int B,
+                 int cap, int pos, int t_new, int h, int d, int dtype, hipStream_t st);
 
 // decode.hip (return -3: more than 8 query rows per (batch, kv head))
 long decode_workspace_floats(int B, int h, int r, int tq, int d);

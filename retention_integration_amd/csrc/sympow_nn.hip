@@ -117,7 +117,7 @@ __global__ __launch_bounds__(256, DK <= 64 ? 3 : 2) void sympow_nn_kernel(NNArgs
     for (int ii = 0; ii < LOADS; ii++) async_copy16_sv(src, boffs[ii], ring_lds + ringpos * STAGE + ii * 4096);
   };
 
-  const bool skip = (EPI == NN_EPI_MERGE) && a.skip_first && (bn % a.n == 0);
+  const bool skip = ((EPI == NN_EPI_MERGE) && a.skip_first && (bn % a.n == 0)) || (a.skip_last && (bn % a.n == a.n - 1));
   f32x4 acc[MT][NT];
 #pragma unroll
   for (int i = 0; i < MT; i++)

@@ -372,7 +372,7 @@ template <typename T, int DK, int DV, int XPW, bool HAS_W>
 __global__ __launch_bounds__(256, 2) void sympow_tn_kernel(const T* __restrict__ A, const T* __restrict__ Bm,
                                                            const float* __restrict__ w, T* __restrict__ S,
                                                            float* __restrict__ s, int c, int hA, int r, int h,
-                                                           int use_mult) {
+                                                           int use_mult, int skip) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   constexpr int PARTS = 16 / XPW;
   constexpr int NB = (DK / 16) * (DK / 16 + 1) / 2;
@@ -391,6 +391,34 @@ __global__ __launch_bounds__(256, 2) void sympow_tn_kernel(const T* __restrict__
   int part = t2 % PARTS;
   int y, xb;
   const int bn = by / h, hh = by % h;
+  // Chunks whose result nobody reads (skip = +n: the last of every n chunks, left unwritten; skip = -n: the first of
+  // every n, whose result is zero by definition and is written as zeros).  Uniform over the workgroup.
+  if (skip > 0 && bn % skip == skip - 1) return;
+  if (skip < 0 && bn % (-skip) == 0) {
+    if (!active) return;
+    constexpr int D = 128 * (DK / 16) * (DK / 16 + 1);
+    int f0, nf;   // the feature rows this wave owns
+    if (XPW == 8 && t2 >= (DK / 16) * (DK / 16 - 1)) {
+      y = t2 - (DK / 16) * (DK / 16 - 1);
+      f0 = 128 * y * (y + 1) + 256 * y;
+      nf = 256;
+    } else {
+      if (XPW == 8) {
+        y = 1;
+        while (y * (y + 1) / 2 <= t2 / 2) y++;
+        xb = t2 / 2 - y * (y - 1) / 2;
+      } else {
+        block_to_yx(t2 / PARTS, y, xb);
+      }
+      f0 = 128 * y * (y + 1) + 256 * xb + 16 * XPW * part;
+      nf = 16 * XPW;
+    }
+    const long so = ((long)bn * h + hh) * D + f0;
+    const int l = threadIdx.x & 63;
+    for (int q = l * 8; q < nf * DV; q += 512) *(u32x4*)(S + so * DV + q) = (u32x4){0, 0, 0, 0};
+    for (int q = l; q < nf; q += 64) s[so + q] = 0.f;
+    return;
+  }
   if constexpr (XPW == 8) {
     constexpr int NOFF = (DK / 16) * (DK / 16 - 1);   // tasks below the block diagonal
     if (t2 >= NOFF) {
@@ -685,7 +713,7 @@ int sympow_tn_chain(const void* A, const void* Bm, const float* w, const float* 
 
 template <typename T, int DK, int DV>
 static int tn_launch(const void* A, const void* Bm, const float* w, void* S, float* s, int BN, int c, int h, int r,
-                     int use_mult, hipStream_t st) {
+                     int use_mult, int skip, hipStream_t st) {
   constexpr int XPW = DV <= 64 ? 8 : 4;
   constexpr int NB = (DK / 16) * (DK / 16 + 1) / 2;
   constexpr int TASKS = tn_tasks<DK, XPW>();
@@ -695,23 +723,24 @@ static int tn_launch(const void* A, const void* Bm, const float* w, void* S, flo
   if (w) {
     auto kern = sympow_tn_kernel<T, DK, DV, XPW, true>;
     allow_big_lds((const void*)kern, smem);
-    hipLaunchKernelGGL(kern, grid, dim3(256), smem, st, (const T*)A, (const T*)Bm, w, (T*)S, s, c, h * r, r, h, use_mult);
+    hipLaunchKernelGGL(kern, grid, dim3(256), smem, st, (const T*)A, (const T*)Bm, w, (T*)S, s, c, h * r, r, h, use_mult, skip);
   } else {
     auto kern = sympow_tn_kernel<T, DK, DV, XPW, false>;
     allow_big_lds((const void*)kern, smem);
-    hipLaunchKernelGGL(kern, grid, dim3(256), smem, st, (const T*)A, (const T*)Bm, w, (T*)S, s, c, h * r, r, h, use_mult);
+    hipLaunchKernelGGL(kern, grid, dim3(256), smem, st, (const T*)A, (const T*)Bm, w, (T*)S, s, c, h * r, r, h, use_mult, skip);
   }
   return (int)hipGetLastError();
 }
 
 // A: [BN, c, h*r, d], Bm: [BN, c, h*r, d], w: [BN, c, h*r] or null -> S: [BN, h, D, d], s: [BN, h, D]
+// skip: 0, or +n / -n to skip the last / first chunk of every n (see the kernel)
 int sympow_tn(const void* A, const void* Bm, const float* w, void* S, float* s, int BN, int c, int h, int r, int d,
-              int use_mult, int dtype, hipStream_t st) {
+              int use_mult, int skip, int dtype, hipStream_t st) {
 #define PR_TN_DISPATCH(T)                                                                                              \
   switch (d) {                                                                                                         \
-    case 32: return tn_launch<T, 32, 32>(A, Bm, w, S, s, BN, c, h, r, use_mult, st);                                   \
-    case 64: return tn_launch<T, 64, 64>(A, Bm, w, S, s, BN, c, h, r, use_mult, st);                                   \
-    case 128: return tn_launch<T, 128, 128>(A, Bm, w, S, s, BN, c, h, r, use_mult, st);                                \
+    case 32: return tn_launch<T, 32, 32>(A, Bm, w, S, s, BN, c, h, r, use_mult, skip, st);                                   \
+    case 64: return tn_launch<T, 64, 64>(A, Bm, w, S, s, BN, c, h, r, use_mult, skip, st);                                   \
+    case 128: return tn_launch<T, 128, 128>(A, Bm, w, S, s, BN, c, h, r, use_mult, skip, st);                                \
     default: return -2;                                                                                                \
   }
   if (dtype == DT_BF16) { PR_TN_DISPATCH(bf16_t) }

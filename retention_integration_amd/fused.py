@@ -90,7 +90,7 @@ def chunked_fwd(Q: Tensor, K: Tensor, V: Tensor, log_G: Optional[Tensor], deg: i
     else:
         S, s = torch.empty_like(Sc), torch.empty_like(sc)
         _lib.check(_timed("sympow_tn(update_state)", lambda: lib.pr_update_state_fwd(
-            p(Kd_), p(V), p(S), p(s), BN, c, h, d, deg, code, st)), "update_state_fwd")
+            p(Kd_), p(V), p(S), p(s), BN, c, h, d, deg, n, code, st)), "update_state_fwd")
         _lib.check(lib.pr_state_scan_fwd(p(S), p(s), p(lcs), p(Sc), p(sc), b, n, n, h, D * d, D, code, st),
                    "state_scan_fwd")
         del S, s
@@ -154,7 +154,7 @@ def chunked_bwd(Q: Tensor, K: Tensor, V: Tensor, A: Tensor, lcs: Tensor, Kd: Ten
         dSc, dsc = torch.empty_like(Sc), torch.empty_like(sc)
         ws = _empty((lib.pr_query_state_bwd_workspace(BN, c, h, r, d, code),), u8, dev)
         _lib.check(lib.pr_query_state_bwd(p(Qg), p(Sc), p(sc), p(rm), p(O), p(den), p(dO), p(dQg), p(dSc), p(dsc),
-                                          None, p(dla), p(dys), p(ws), BN, n, c, h, r, d, scale ** deg, deg, 1, 1, code,
+                                          None, p(dla), p(dys), p(ws), BN, n, c, h, r, d, scale ** deg, deg, 2, 1, code,
                                           st),
                    "query_state_bwd")
         ws = _empty((lib.pr_state_scan_bwd_workspace(b, n, h, D * d, D),), u8, dev)
@@ -164,10 +164,10 @@ def chunked_bwd(Q: Tensor, K: Tensor, V: Tensor, A: Tensor, lcs: Tensor, Kd: Ten
     dKd, dVs = torch.empty_like(K), torch.empty_like(V)
     # (two calls: the value gradient and the key gradient are separate kernels, and the latter is timed on its own)
     # (dS comes from the kernels above, so both orders of a pair hold the same sum: the last flag says so)
-    _lib.check(lib.pr_update_state_bwd(p(Kd), p(V), p(dS), p(ds), None, p(dVs), BN, c, h, d, deg, 1, code, st),
+    _lib.check(lib.pr_update_state_bwd(p(Kd), p(V), p(dS), p(ds), None, p(dVs), BN, c, h, d, deg, 1, n, code, st),
                "update_state_bwd(dV)")
     _lib.check(_timed("sympow_grad(dK)", lambda: lib.pr_update_state_bwd(
-        p(Kd), p(V), p(dS), p(ds), p(dKd), None, BN, c, h, d, deg, 1, code, st)), "update_state_bwd(dK)")
+        p(Kd), p(V), p(dS), p(ds), p(dKd), None, BN, c, h, d, deg, 1, n, code, st)), "update_state_bwd(dK)")
 
     # the attention backward adds the state-path gradients in its epilogue and writes the final dQ, dK, dV
     dQa, dKa, dVa = torch.empty_like(Q), torch.empty_like(K), torch.empty_like(V)

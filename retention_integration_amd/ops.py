@@ -143,7 +143,7 @@ def update_state_fwd(K: Tensor, V: Tensor) -> Tuple[Tensor, Tensor]:
     S = torch.empty((b, n, h, D, d), dtype=K.dtype, device=K.device)
     s = torch.empty((b, n, h, D), dtype=torch.float32, device=K.device)
     lib = _lib.load()
-    _lib.check(lib.pr_update_state_fwd(_lib.ptr(K), _lib.ptr(V), _lib.ptr(S), _lib.ptr(s), b * n, c, h, d, 2,
+    _lib.check(lib.pr_update_state_fwd(_lib.ptr(K), _lib.ptr(V), _lib.ptr(S), _lib.ptr(s), b * n, c, h, d, 2, 0,
                                        _lib.dtype_code(K.dtype), _lib.stream()), "update_state_fwd")
     return S, s
 
@@ -161,7 +161,7 @@ def update_state_bwd(K: Tensor, V: Tensor, dS: Tensor, ds: Tensor) -> Tuple[Tens
     dK, dV = torch.empty_like(K), torch.empty_like(V)
     lib = _lib.load()
     _lib.check(lib.pr_update_state_bwd(_lib.ptr(K), _lib.ptr(V), _lib.ptr(dS), _lib.ptr(ds), _lib.ptr(dK),
-                                       _lib.ptr(dV), b * n, c, h, d, 2, 0, _lib.dtype_code(K.dtype), _lib.stream()),
+                                       _lib.ptr(dV), b * n, c, h, d, 2, 0, 0, _lib.dtype_code(K.dtype), _lib.stream()),
                "update_state_bwd")
     return dK, dV
 

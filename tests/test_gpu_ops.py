@@ -267,7 +267,7 @@ def test_symmetric_state_flag_changes_nothing_for_a_symmetric_state(pra, dtype, 
     res = []
     for flag in (0, 1):
         dK, dV = torch.empty_like(K), torch.empty_like(V)
-        _lib.check(lib.pr_update_state_bwd(p(K), p(V), p(S), p(s), p(dK), p(dV), b * n, c, h, d, 2, flag, code, st),
+        _lib.check(lib.pr_update_state_bwd(p(K), p(V), p(S), p(s), p(dK), p(dV), b * n, c, h, d, 2, flag, 0, code, st),
                    "update_state_bwd")
         O, den = ops.query_state_fwd(Q, S, s, None, None, None, 1.0 / d, False)
         dQ, dS, ds = torch.empty_like(Q), torch.empty_like(S), torch.empty_like(s)
