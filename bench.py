@@ -121,10 +121,14 @@ def counter_run(pra, Q, K, V, cfg, dev):
 
 
 def decode_bench(pra, dev, steps=512):
-    """The inference configuration of the benchmark contract (configs[3]): b=32, h=8, d=64 bf16; prefill of 2048 tokens with switch_over_seq_len=1024, then
-    `steps` single-token steps.  Two loops are timed: the recurrent one (every token is folded into the state,
-    switch_over_seq_len=1) and the API-faithful one of the reference's caller (the cache grows, the state is only
-    queried; ref: deploy/models/powercoder/modeling_powercoder.py:181-196)."""
+    """The inference configuration of the benchmark contract (configs[3]): b=32, h=8, d=64 bf16; prefill of 2048 tokens
+    with switch_over_seq_len=1024, then `steps` single-token steps.  Loops timed:
+      recurrent           every token folded into the state (switch_over_seq_len=1), one library call per token,
+                          through power_retention_inference;
+      recurrent_graph     the same steps through RetentionCache.step, captured once in a HIP graph and replayed;
+      growing_cache       the reference caller's loop: torch.cat of the cache + power_retention_inference with the whole
+                          cache, the state only queried (ref: deploy/models/powercoder/modeling_powercoder.py:181-196);
+      growing_cache_prealloc  the same arithmetic through RetentionCache.step (append in place, no torch.cat)."""
     b, h, d = 32, 8, 64
     g = torch.Generator().manual_seed(4)
     mk = lambda *shape: torch.randn(*shape, generator=g).to(torch.bfloat16).to(dev)  # noqa: E731
@@ -133,6 +137,15 @@ def decode_bench(pra, dev, steps=512):
     qs, ks, vs = mk(steps, b, 1, h, d), mk(steps, b, 1, h, d), mk(steps, b, 1, h, d)
     lgs = torch.nn.functional.logsigmoid(torch.randn(steps, b, 1, h, generator=g)).to(dev)
     out = {}
+
+    def timed(fn):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        fn()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        return {"us_per_step": round(dt / steps * 1e6, 1), "tokens_per_s": round(b * steps / dt, 1)}
+
     with torch.no_grad():
         pra.power_retention_inference(Q, K, V, lg, switch_over_seq_len=1024)   # warm-up
         torch.cuda.synchronize()
@@ -143,29 +156,71 @@ def decode_bench(pra, dev, steps=512):
         St, st = S, s
         for i in range(8):
             _, St, st = pra.power_retention_inference(qs[i], ks[i], vs[i], lgs[i], St, st, switch_over_seq_len=1)
-        St, st = S, s
+
+        def recurrent():
+            St, st = S, s
+            for i in range(steps):
+                _, St, st = pra.power_retention_inference(qs[i], ks[i], vs[i], lgs[i], St, st, switch_over_seq_len=1)
+        out["recurrent"] = timed(recurrent)
+
+        # the same steps captured in a HIP graph (state updated in place in the cache's own buffers)
+        cache = pra.RetentionCache(b, h, d, capacity=steps, device=dev)
+        ys = torch.empty(steps, b, 1, h, d, dtype=torch.bfloat16, device=dev)
+
+        def rec_steps():
+            for i in range(steps):
+                cache.step(qs[i], ks[i], vs[i], lgs[i], switch_over_seq_len=1, out=ys[i])
+        cache.update_state(S, s)
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            rec_steps()
+        torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for i in range(steps):
-            _, St, st = pra.power_retention_inference(qs[i], ks[i], vs[i], lgs[i], St, st, switch_over_seq_len=1)
-        torch.cuda.synchronize()
-        dt = time.perf_counter() - t0
-        out["recurrent"] = {"us_per_step": round(dt / steps * 1e6, 1), "tokens_per_s": round(b * steps / dt, 1)}
-        Kc = torch.empty(b, 0, h, d, dtype=torch.bfloat16, device=dev)
-        Vc, Gc = Kc.clone(), torch.empty(b, 0, h, device=dev)
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for i in range(steps):
-            Kc, Vc, Gc = torch.cat([Kc, ks[i]], 1), torch.cat([Vc, vs[i]], 1), torch.cat([Gc, lgs[i]], 1)
-            pra.power_retention_inference(qs[i], Kc, Vc, Gc, S, s, switch_over_seq_len=1024)
-        torch.cuda.synchronize()
-        dt = time.perf_counter() - t0
-        out["growing_cache"] = {"us_per_step": round(dt / steps * 1e6, 1), "tokens_per_s": round(b * steps / dt, 1)}
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            rec_steps()
+        cache.update_state(S, s)
+        graph.replay()
+        cache.update_state(S, s)
+        out["recurrent_graph"] = timed(graph.replay)
+
+        def growing():
+            Kc = torch.empty(b, 0, h, d, dtype=torch.bfloat16, device=dev)
+            Vc, Gc = Kc.clone(), torch.empty(b, 0, h, device=dev)
+            for i in range(steps):
+                Kc, Vc, Gc = torch.cat([Kc, ks[i]], 1), torch.cat([Vc, vs[i]], 1), torch.cat([Gc, lgs[i]], 1)
+                pra.power_retention_inference(qs[i], Kc, Vc, Gc, S, s, switch_over_seq_len=1024)
+        out["growing_cache"] = timed(growing)
+
+        def growing_prealloc():
+            cache.clean_kv()
+            for i in range(steps):
+                cache.step(qs[i], ks[i], vs[i], lgs[i], switch_over_seq_len=1024)
+        cache.update_state(S, s)
+        growing_prealloc()
+        out["growing_cache_prealloc"] = timed(growing_prealloc)
     state_bytes = b * h * (pra.expanded_dim(d) * d * 2 + pra.expanded_dim(d) * 4)
     out["state_bytes"] = state_bytes
-    out["recurrent"]["state_GBps"] = round(2 * state_bytes / (out["recurrent"]["us_per_step"] * 1e-6) / 1e9, 1)
+    for key in ("recurrent", "recurrent_graph"):
+        out[key]["state_GBps"] = round(2 * state_bytes / (out[key]["us_per_step"] * 1e-6) / 1e9, 1)
     out["workload"] = f"power_retention_inference bf16 b={b} h={h} d={d}: prefill 2048 (switch_over_seq_len=1024), {steps} decode steps"
     return out
+
+
+def measured_traffic(name):
+    """HBM bytes per launch of the roofline kernel as measured with rocprofv3 byte counters: read from the line
+    'total HBM traffic <x> MB' of the tracked summary profiles/<name> (which gives the commands and the calibration).
+    None when the file is absent or has no such line -- never a number typed in here."""
+    import re
+    path = os.path.join(ROOT, "profiles", name)
+    try:
+        m = re.search(r"total HBM traffic ([0-9.]+) MB", open(path).read())
+    except OSError:
+        return None, "profiles/" + name + " not found"
+    if not m:
+        return None, "profiles/" + name + " has no 'total HBM traffic' line"
+    return float(m.group(1)) * 1e6, "profiles/" + name + " (rocprofv3 FETCH_SIZE + WRITE_SIZE, calibrated with a plain copy)"
 
 
 def cpu_baseline(cfg, seconds_hint=20):
@@ -178,13 +233,18 @@ def cpu_baseline(cfg, seconds_hint=20):
     Q, K, V, dO = (torch.randn(cfg["b"], t_s, cfg["h"], cfg["d"], generator=g).to(torch.bfloat16).float() for _ in range(4))
     lg = torch.nn.functional.logsigmoid(torch.randn(cfg["b"], t_s, cfg["h"], generator=g))
     xs = [x.requires_grad_(True) for x in (Q, K, V, lg)]
+    # one untimed pass over two chunks first: thread pool, allocator and the oracle's cached index tables are warm
+    w = 2 * cfg["chunk"]
+    oracle.power_retention(*(x[:, :w] for x in xs), deg=2, chunk_size=cfg["chunk"]).backward(dO[:, :w])
+    for x in xs:
+        x.grad = None
     t0 = time.perf_counter()
     Y = oracle.power_retention(*xs, deg=2, chunk_size=cfg["chunk"])
     Y.backward(dO)
     dt = time.perf_counter() - t0
     return {"value": round(cfg["b"] * t_s / dt, 1), "unit": "tokens/s", "cores": torch.get_num_threads(),
             "kind": "port", "sample": f"fwd+bwd fp32, same shape with t={t_s} (32 chunks of {cfg['chunk']}), "
-                                      f"{dt:.1f} s wall"}
+                                      f"{dt:.1f} s wall after one untimed warm-up pass"}
 
 
 def short_chunks(pra, dev, steps, warmup):
@@ -264,16 +324,33 @@ def main():
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
-    # the two kernels of the roofline blocks are timed where they run: HIP events on the launch stream around each of
-    # their launches inside the timed steps (a few microseconds of host work per step)
+    # (a) K steps back to back between two synchronisations.  The two kernels of the roofline blocks are timed where
+    # they run: HIP events on the launch stream around each of their launches inside these steps.
     fused.KERNEL_TIMERS = {}
     t0 = time.perf_counter()
     for _ in range(args.steps):
         step()
     torch.cuda.synchronize()
-    dt = (time.perf_counter() - t0) / args.steps
+    dt_b2b = (time.perf_counter() - t0) / args.steps
     in_step_ms = {k: sum(a.elapsed_time(b_) for a, b_ in v) / len(v) for k, v in fused.KERNEL_TIMERS.items()}
     fused.KERNEL_TIMERS = None
+    # (b) the reference's protocol (ref: perf/_timing.py:77-110): before every step the caches are flushed (a fill of
+    # 512 MB: L2 and the 256 MB memory-side cache), the step is bracketed by HIP events of its own, and the MEDIAN over
+    # the K steps is the headline figure; the fill and a short device-side pause (which lets the host run ahead, so
+    # launch latency is not measured) sit outside the events.
+    flush = torch.empty(512 * 1024 * 1024, dtype=torch.int8, device=dev)
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    for e0, e1 in ev:
+        flush.zero_()
+        torch.cuda._sleep(200_000)
+        e0.record()
+        step()
+        e1.record()
+    torch.cuda.synchronize()
+    times = sorted(a.elapsed_time(b_) for a, b_ in ev)
+    del flush
+    dt = times[len(times) // 2] * 1e-3 if len(times) % 2 else 0.5e-3 * (times[len(times) // 2 - 1] + times[len(times) // 2])
 
     D_compact = cfg["d"] * (cfg["d"] + 1) // 2
     f_fwd, f_bwd = flops(cfg["b"], cfg["t"], cfg["h"], cfg["d"], cfg["chunk"], D_compact)
@@ -286,21 +363,27 @@ def main():
         "config": {"workload": "power_retention fwd+bwd b=1 t=65536 h=8 d=64 deg=2 chunk_size=1024 gating=True "
                                "(BASELINE configs[1]+[2])", "D_state": expanded_dim(cfg["d"])},
         "tflops": round(tflops, 2), "pct_bf16_mfma_peak": round(100 * tflops / PEAK_BF16_TFLOPS, 2),
+        "timing": {"protocol": "median over the K steps, each after a 512 MB cache flush, HIP events per step "
+                               "(ref: perf/_timing.py:77-110); back_to_back = wall clock of K consecutive steps / K",
+                   "flushed_ms": {"median": round(dt * 1e3, 4), "min": round(times[0], 4), "max": round(times[-1], 4)},
+                   "back_to_back_ms_per_step": round(dt_b2b * 1e3, 4)},
     }
     n = cfg["t"] // cfg["chunk"]
     bh = cfg["b"] * cfg["h"]
     # dominant single kernel (two launches per step, the largest share of the step): the feature-gradient contraction
-    # sympow_grad, here its dK launch of update_state backward; one launch = all n chunks, algorithmic flops = the
-    # d(phi) product 2*c*D*d per (chunk, head) with the compact D.  Duration: HIP events around that launch inside
-    # the timed steps (in_step_ms above), which is what the kernel trace of the same command shows.
-    k_flops = 2.0 * bh * n * cfg["chunk"] * D_compact * cfg["d"]
+    # sympow_grad, here its dK launch of update_state backward.  Algorithmic flops per launch = the d(phi) product
+    # 2*c*D*d per (chunk, head) with the compact D over the n-1 chunks whose state is read (the same convention as
+    # flops() above).  Duration: HIP events around that launch inside the back-to-back steps, which is what the kernel
+    # trace of the same command shows.
+    k_flops = 2.0 * bh * (n - 1) * cfg["chunk"] * D_compact * cfg["d"]
     k_ms = in_step_ms["sympow_grad(dK)"]
+    traffic, traffic_src = measured_traffic("sympow_grad_t65536_hbm_traffic.txt")
+    esz = 2
+    algo_bytes = bh * (n - 1) * (3 * cfg["chunk"] * cfg["d"] * esz + expanded_dim(cfg["d"]) * (cfg["d"] * esz + 4))
     out["roofline"] = {"kernel": "sympow_grad_kernel (dK of update_state backward)", "bound": "mfma",
                        "achieved": round(k_flops / k_ms / 1e9, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                        "frac": round(k_flops / k_ms / 1e9 / PEAK_BF16_TFLOPS, 4), "ms_per_launch": round(k_ms, 4),
-                       # HBM bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE, calibrated with a plain
-                       # 256 MiB copy (profiles/sympow_grad_t65536_hbm_traffic.txt); algorithmic: 374.3 MB
-                       "traffic": 374.6e6}
+                       "traffic": traffic, "traffic_source": traffic_src, "algorithmic_bytes": algo_bytes}
     t_ms = in_step_ms["sympow_tn(update_state)"]
     out["roofline_update_state_fwd"] = {"kernel": "sympow_tn_kernel", "bound": "mfma",
                                         "achieved": round(k_flops / t_ms / 1e9, 2), "peak": PEAK_BF16_TFLOPS,

@@ -93,12 +93,17 @@ class RetentionCache:
         self.sum_of_keys.zero_()
 
     # ---- the decode step ---------------------------------------------------------------------------------------
-    def step(self, q, k, v, log_g=None, scale=None, switch_over_seq_len=512):
-        """One token: ``q [b, 1, hq, d]``, ``k, v [b, 1, h, d]``, ``log_g [b, 1, h]`` fp32 or None -> ``[b, 1, hq, d]``
-        (a buffer of the cache, overwritten by the next step).  Same arithmetic as the reference caller's sequence
+    def step(self, q, k, v, log_g=None, scale=None, switch_over_seq_len=512, out=None):
+        """One token: ``q [b, 1, hq, d]``, ``k, v [b, 1, h, d]``, ``log_g [b, 1, h]`` fp32 or None -> ``[b, 1, hq, d]``,
+        written to ``out`` (contiguous, same shape and dtype as q) or, without it, to a buffer of the cache that the next
+        step overwrites.  Same arithmetic as the reference caller's sequence
         ``update_kv -> power_retention_inference(whole cache, state) -> clean_kv + update_state at the switch-over``."""
         lib, p, stream = self._lib, _lib.ptr, _lib.stream()
         assert q.shape == (self.b, 1, self.hq, self.d) and q.dtype == self.dtype
+        if out is None:
+            out = self._out
+        else:
+            assert out.shape == q.shape and out.dtype == q.dtype and out.is_contiguous()
         scale = float(scale) if scale else 1.0 / self.d ** 0.5
         r = self.hq // self.h
         fold = switch_over_seq_len is not None and self.length + 1 >= switch_over_seq_len
@@ -108,15 +113,15 @@ class RetentionCache:
             _lib.check(lib.pr_decode_step(p(q.contiguous()), p(g), p(self.state), p(self.sum_of_keys), None, None, None,
                                           p(k.reshape(self.b, self.h, self.d).contiguous()),
                                           p(v.reshape(self.b, self.h, self.d).contiguous()), p(g), p(self.state),
-                                          p(self.sum_of_keys), p(self._out), p(self._ws), self.b, 1, self.h, r, self.d,
+                                          p(self.sum_of_keys), p(out), p(self._ws), self.b, 1, self.h, r, self.d,
                                           scale ** 2, 2, self._code, 1, stream), "decode_step")
-            return self._out
+            return out
         self.update_kv(k, v, log_g)
         n = self.length
         if not self.has_state:
             # no state yet: normalised attention over the cache
             _lib.check(lib.pr_cache_attention_fwd(p(q.contiguous()), p(self.keys), p(self.values), p(self.gatings),
-                                                  p(self._out), p(self._la), p(self._rm), self.b, 1, n, self.capacity,
+                                                  p(out), p(self._la), p(self._rm), self.b, 1, n, self.capacity,
                                                   self.h, r, self.d, scale, 2, 1, self._code, stream), "cache_attention_fwd")
         else:
             _lib.check(lib.pr_cache_attention_fwd(p(q.contiguous()), p(self.keys), p(self.values), p(self.gatings),
@@ -124,12 +129,12 @@ class RetentionCache:
                                                   self.h, r, self.d, scale, 2, 0, self._code, stream), "cache_attention_fwd")
             # (the query is gated by the accumulated gate at the newest cache position, which the append left in _gq)
             _lib.check(lib.pr_decode_step(p(q.contiguous()), p(self._gq), p(self.state), p(self.sum_of_keys), p(self._ya),
-                                          p(self._la), p(self._rm), None, None, None, None, None, p(self._out),
+                                          p(self._la), p(self._rm), None, None, None, None, None, p(out),
                                           p(self._ws), self.b, 1, self.h, r, self.d, scale ** 2, 2, self._code, 0,
                                           stream), "decode_step")
         if fold:
             self._fold()
-        return self._out
+        return out
 
     def _fold(self):
         """Compress the cache into the state and clear it (ref: retention/power_retention_maker.py:366-382 and

@@ -62,6 +62,19 @@ def main():
     S, N = update_state(K, V, 2)
     npz("update_state_d32.npz", K=K, V=V, S=S, N=N)
 
+    # update_state at d=64 (four diagonal tiles, six below them: D = 2560) together with the one hand-written backward
+    # the reference's pure-torch backend has (SymmetricPowerUpdateStateReference.backward).  Inputs are multiples of
+    # 1/4, so every product and sum is exact in fp32 (and the file compresses); the upstream gradient of S is the outer
+    # product u w^T of two stored vectors, so it need not be stored itself.
+    g64 = torch.Generator().manual_seed(4321)   # (its own stream: the vectors below keep their values)
+    q4 = lambda *s: (torch.randn(*s, generator=g64, dtype=torch.float32) * 4).round().clamp(-8, 8) / 4  # noqa: E731
+    K64, V64 = q4(1, 1, 4, 1, 64).requires_grad_(True), q4(1, 1, 4, 1, 64).requires_grad_(True)
+    S64, N64 = update_state(K64, V64, 2)
+    u, wv, dN = q4(2560), q4(64), q4(1, 1, 1, 2560)
+    dS = (u[:, None] * wv[None, :]).view(1, 1, 1, 2560, 64)
+    dK64, dV64 = torch.autograd.grad((S64, N64), (K64, V64), (dS, dN))
+    npz("update_state_d64_bwd.npz", K=K64, V=V64, S=S64, N=N64, dS_u=u, dS_w=wv, dN=dN, dK=dK64, dV=dV64)
+
     # query_state with GQA ratio 2, second chunk uses gamma = sqrt(D)
     Q = rn(1, 2, 4, 2, 32)
     S_in = rn(1, 2, 1, 768, 32)

@@ -110,7 +110,7 @@ def test_recurrent_steps_captured_in_a_hip_graph_equal_the_eager_loop():
 
     def run():
         for i in range(n):
-            outs[i].copy_(cache.step(q[i], k[i], v[i], lg[i], switch_over_seq_len=1))
+            cache.step(q[i], k[i], v[i], lg[i], switch_over_seq_len=1, out=outs[i])
 
     cache.update_state(S0, s0)
     run()

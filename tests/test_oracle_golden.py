@@ -63,3 +63,17 @@ def test_inference_prefill_then_decode():
     Y1, st1, sk1 = oracle.power_retention_inference(v["Q1"], v["K1"], v["V1"], v["log_G1"], v["state0"],
                                                     v["sum_of_keys0"], deg=2, switch_over_seq_len=3)
     close(Y1, v["Y1"], rtol=1e-4, atol=1e-5); close(st1, v["state1"]); close(sk1, v["sum_of_keys1"])
+
+
+def test_update_state_d64_forward_and_the_references_hand_written_backward():
+    """d = 64: ten feature tiles (four on the diagonal), and the gradients of the one backward the reference's
+    pure-torch backend writes by hand (ref: retention/_update_state/reference.py:55-83) against the oracle's autograd.
+    The inputs are multiples of 1/4, so both sides are exact in fp32."""
+    v = load("update_state_d64_bwd.npz")
+    K, V = v["K"].clone().requires_grad_(True), v["V"].clone().requires_grad_(True)
+    S, N = oracle.update_state(K, V, 2)
+    assert torch.equal(S, v["S"]) and torch.equal(N, v["N"])
+    dS = (v["dS_u"][:, None] * v["dS_w"][None, :]).view(1, 1, 1, 2560, 64)
+    dK, dV = torch.autograd.grad((S, N), (K, V), (dS, v["dN"]))
+    close(dK, v["dK"], rtol=1e-6, atol=1e-4)
+    close(dV, v["dV"], rtol=1e-6, atol=1e-4)
