@@ -49,7 +49,23 @@ def build(jobs=8, verbose=True):
     return OUT
 
 
+def build_probe():
+    """The stand-alone issue microbenchmark (probe_issue.hip) as an executable next to the library; not part of it."""
+    out = os.path.join(os.path.dirname(HERE), "probe_issue")
+    cmd = [hipcc(), *[f for f in FLAGS if f != "-fPIC"], os.path.join(HERE, "probe_issue.hip"), "-o", out]
+    p = subprocess.run(cmd, capture_output=True, text=True)
+    if p.returncode != 0:
+        raise RuntimeError("hipcc failed for probe_issue.hip:\n" + p.stderr)
+    print("built", out)
+    return out
+
+
 if __name__ == "__main__":
     ap = argparse.ArgumentParser()
     ap.add_argument("--jobs", type=int, default=min(8, os.cpu_count() or 1))
-    build(ap.parse_args().jobs)
+    ap.add_argument("--probe", action="store_true", help="build only the stand-alone issue microbenchmark")
+    args = ap.parse_args()
+    if args.probe:
+        build_probe()
+    else:
+        build(args.jobs)
