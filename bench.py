@@ -120,6 +120,25 @@ def counter_run(pra, Q, K, V, cfg, dev):
     print("counter run done: 3 x sympow_grad, 3 x 256 MiB device copy")
 
 
+def attention_scaling(pra, dev, chunk):
+    """For a kernel trace: the three attention kernels alone (operator level, four forward + backward calls) on the
+    headline's 65536 x 8 rows cut into chunks of `chunk` keys.  The tile work of a launch is proportional to the chunk
+    length while everything per row and per workgroup (loading the block's own rows, storing its results, set-up) is
+    not, so two chunk lengths separate the two."""
+    from retention_integration_amd import ops
+    t, h, d = CFG["t"], CFG["h"], CFG["d"]
+    Q, K, V, lg, dO = make_inputs(1, t, h, d, dev)
+    n = t // chunk
+    Qf, Kf, Vf, dOf = (x.view(n, chunk, h, d) for x in (Q, K, V, dO))
+    A = lg.view(n, chunk, h).cumsum(1).contiguous()
+    with torch.no_grad():
+        for _ in range(4):
+            Ya, la, rm = ops.attention_fwd(Qf, Kf, Vf, A, 2, d ** -0.5, False)
+            ops.attention_bwd(Qf, Kf, Vf, A, rm, dOf, la, None, 2, d ** -0.5)
+        torch.cuda.synchronize()
+    print(f"attention scaling run done: 4 x (attention_fwd, attention_bwd) at chunk {chunk}, {n} chunks x {h} heads")
+
+
 def decode_bench(pra, dev, steps=512):
     """The inference configuration of the benchmark contract (configs[3]): b=32, h=8, d=64 bf16; prefill of 2048 tokens
     with switch_over_seq_len=1024, then `steps` single-token steps.  Loops timed:
@@ -292,6 +311,9 @@ def main():
     ap.add_argument("--counter-run", action="store_true",
                     help="for rocprofv3 --pmc: launch only the dominant kernel (sympow_grad, dK of update_state "
                          "backward) a few times, and a plain device copy of 256 MiB for calibrating byte counters")
+    ap.add_argument("--attention-chunk", type=int, default=0,
+                    help="for rocprofv3 --kernel-trace: run only the attention kernels, four times, with the headline's "
+                         "rows cut into chunks of this length")
     ap.add_argument("--short-chunks", action="store_true",
                     help="instead of the headline workload: BASELINE configs[4] (fp16, b=4, t=16384, h=16, d=128, "
                          "chunk 128, no gating, inputs N(0,1)*0.5), fwd+bwd; prints its own JSON line")
@@ -306,6 +328,9 @@ def main():
     dev = torch.device("cuda:0")
     if args.short_chunks:
         short_chunks(pra, dev, args.steps, args.warmup)
+        return
+    if args.attention_chunk:
+        attention_scaling(pra, dev, args.attention_chunk)
         return
     cfg = CFG
     Q, K, V, lg, dO = make_inputs(cfg["b"], cfg["t"], cfg["h"], cfg["d"], dev)
