@@ -38,7 +38,8 @@ enum {
 
 /* 2: pr_update_state_bwd and pr_query_state_bwd take the symmetric-state promise (dS_symmetric, S_symmetric).
  * 3: pr_decode_step_noalloc.  4: pr_cache_append, pr_cache_attention_fwd; pr_update_state_fwd takes skip_last_of and
- * pr_update_state_bwd zero_last_of. */
+ * pr_update_state_bwd zero_last_of; pr_query_state_fwd / _bwd / _scan_bwd take q_log_gate and
+ * pr_chunk_attention_bwd dQ_state_plain. */
 int pr_abi_version(void);
 const char* pr_last_error(void);
 
@@ -130,10 +131,10 @@ int pr_update_state_scan_fwd(const void* K, const void* V, const float* log_G, v
  * retention/_discumsum/reference.py:3-15 differentiated.  S, s are the scanned states the forward used.
  *   workspace: pr_query_state_scan_bwd_workspace() bytes. */
 size_t pr_query_state_scan_bwd_workspace(int B, int n, int c, int h, int r, int d, int dtype);
-int pr_query_state_scan_bwd(const void* Q, const void* S, const float* s, const float* rowmax, const void* O,
-                            const float* den, const void* dO, const float* log_G, void* dQ, void* dS_in, float* ds_in,
-                            void* dY_attn, float* dl_attn, float* dY_scale, float* dlog_G, void* workspace, int B,
-                            int n, int c, int h, int r, int d, float scale_p, int deg, int dtype, void* stream);
+int pr_query_state_scan_bwd(const void* Q, const void* S, const float* s, const float* rowmax, const float* q_log_gate,
+                            const void* O, const float* den, const void* dO, const float* log_G, void* dQ, void* dS_in,
+                            float* ds_in, void* dY_attn, float* dl_attn, float* dY_scale, float* dlog_G, void* workspace,
+                            int B, int n, int c, int h, int r, int d, float scale_p, int deg, int dtype, void* stream);
 
 /* query_state(Q, S, s, Y_attn, l_attn, rowmax, deg, scale, zero_initial_state) --
  * retention/_query_state/reference.py:36-96,166-191, Triton twin retention/_query_state/triton.py:54-169,478-544.
@@ -141,10 +142,15 @@ int pr_query_state_scan_bwd(const void* Q, const void* S, const float* s, const 
  *   Y_attn [BN,c,h*r,d] / l_attn, rowmax [BN,c,h*r] fp32, all three NULL when there is no attention part
  *   -> O [BN,c,h*r,d] and den [BN,c,h*r] fp32, the normaliser in the scaled units the backward expects.
  *   scale_p = scale^deg; n = chunks per batch entry; zero_initial_state != 0 declares S, s of chunk 0 of every
- *   batch entry to be zero (they are then not read). */
+ *   batch entry to be zero (they are then not read).
+ *   q_log_gate [BN,c,h] fp32 or NULL (needs the attention part): the query gating of
+ *   retention/power_retention_maker.py:183-186 without the gated copy -- with it, Q is the UNGATED query and the result
+ *   is that of Q * exp(q_log_gate / deg): the state part is homogeneous of degree deg in the query, so the gate is a
+ *   factor exp(q_log_gate) on that part of each row and is applied in the merge (exact; the reference rounds the gated
+ *   copy to 16 bits first). */
 int pr_query_state_fwd(const void* Q, const void* S, const float* s, const void* Y_attn, const float* l_attn,
-                       const float* rowmax, void* O, float* den, int BN, int n, int c, int h, int r, int d,
-                       float scale_p, int deg, int zero_initial_state, int dtype, void* stream);
+                       const float* rowmax, const float* q_log_gate, void* O, float* den, int BN, int n, int c, int h,
+                       int r, int d, float scale_p, int deg, int zero_initial_state, int dtype, void* stream);
 
 /* Backward -- formulas of retention/_query_state/triton.py:546-553 (kernels :184-448).
  *   O, den from the forward; dO [BN,c,h*r,d]
@@ -156,11 +162,13 @@ int pr_query_state_fwd(const void* Q, const void* S, const float* s, const void*
  *   chunk's (zero) state: dS, ds of the first of every n chunks are then written as zeros instead of computed (the
  *   composed function discards them, retention/power_retention_maker.py:167-170).
  *   workspace: pr_query_state_bwd_workspace() bytes (scaled dO and two fp32 row vectors).
+ *   q_log_gate as in the forward: Q is then the ungated query and dQ the gradient w.r.t. it through the state part
+ *   (the gate's own gradient is (Q . dQ) / deg per row, which pr_chunk_attention_bwd forms with dQ_state_plain).
  *   S_symmetric != 0: the caller's promise that S[(a,b)] == S[(b,a)] in the blocks on the diagonal (true of every
  *   state made by pr_update_state_fwd and the scans); the query gradient then takes a shorter path through them. */
 size_t pr_query_state_bwd_workspace(int BN, int c, int h, int r, int d, int dtype);
-int pr_query_state_bwd(const void* Q, const void* S, const float* s, const float* rowmax, const void* O,
-                       const float* den, const void* dO, void* dQ, void* dS, float* ds, void* dY_attn,
+int pr_query_state_bwd(const void* Q, const void* S, const float* s, const float* rowmax, const float* q_log_gate,
+                       const void* O, const float* den, const void* dO, void* dQ, void* dS, float* ds, void* dY_attn,
                        float* dl_attn, float* dY_scale, void* workspace, int BN, int n, int c, int h, int r, int d,
                        float scale_p, int deg, int zero_initial_state, int S_symmetric, int dtype, void* stream);
 
@@ -171,7 +179,7 @@ int pr_gate_cumsum(const float* log_G, float* A, int B, int t, int h, void* stre
 /* Gate arithmetic of the chunked algorithm, forward -- retention/power_retention_maker.py:146-153,163-164,183-186.
  *   log_G [BN,c,h] fp32 (BN = b*n chunks of length c <= 8192), K [BN,c,h,d], Q [BN,c,h*r,d]
  *   -> A [BN,c,h] = cumsum over the chunk, lcs [BN,h] = A[c-1],
- *      Kd = K * exp((A[c-1] - A)/deg), Qg = Q * exp(A/deg). */
+ *      Kd = K * exp((A[c-1] - A)/deg), Qg = Q * exp(A/deg) (Qg may be NULL: not formed). */
 int pr_chunk_prep_fwd(const float* log_G, const void* K, const void* Q, float* A, float* lcs, void* Kd, void* Qg, int BN,
                       int c, int h, int r, int d, int deg, int dtype, void* stream);
 
@@ -184,6 +192,8 @@ int pr_chunk_prep_fwd(const float* log_G, const void* K, const void* Q, float* A
  *   -(K.dK_state) exp((A[c-1]-A)/deg)/deg,  dotk [BN,c,h] = (K.dK_state) exp((A[c-1]-A)/deg).
  *   dQ_state = gradient w.r.t. Qg (query_state backward), dK_state, dV_state = gradients w.r.t. Kd, V
  *   (update_state backward).  With A = NULL the factors are 1 and dGq, dGk, dotk are not written.
+ *   dQ_state_plain != 0: dQ_state is already the gradient w.r.t. Q itself (pr_query_state_bwd with q_log_gate):
+ *   dQ = dQ_attn + dQ_state and dGq gets (Q.dQ_state)/deg.
  * pr_chunk_gate_scan_bwd finishes the gate gradient: dlog_G holds dGk on entry; the r query heads' dGq [BN,c,h*r]
  *   are added (dGq may be NULL), dlog_G[c-1] += (sum_t dotk)/deg + dlcs_a + dlcs_b (dlcs_b may be NULL), then the
  *   reverse cumulative sum over the chunk, in place. */
@@ -191,7 +201,7 @@ int pr_chunk_attention_bwd(const void* Q, const void* K, const void* V, const fl
                            const void* dO, const float* dl, const float* dO_scale, const void* dQ_state,
                            const void* dK_state, const void* dV_state, void* dQ, void* dK, void* dV, float* dGq,
                            float* dGk, float* dotk, int BN, int c, int h, int r, int d, float scale, int deg,
-                           int dtype, void* stream);
+                           int dQ_state_plain, int dtype, void* stream);
 int pr_chunk_gate_scan_bwd(float* dlog_G, const float* dGq, const float* dotk, const float* dlcs_a, const float* dlcs_b,
                            int BN, int c, int h, int r, int deg, void* stream);
 

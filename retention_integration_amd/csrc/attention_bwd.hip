@@ -365,7 +365,7 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dq_kernel(AttnBwdArgs a,
     if (dQsg) {   // gradient through the gated copy of Q: dQs * u, and (Q . dQs) u / deg for the gate
       const int lr = wslice * 16 * MT + 16 * mi;
       const uint32_t rb = ep + (lr / AB_BN) * TILE + (lr % AB_BN) * RB;
-      u = Gg ? __expf(Gg[(long)ti[mi] * a.h] / a.deg) : 1.f;
+      u = (Gg && !a.dQs_plain) ? __expf(Gg[(long)ti[mi] * a.h] / a.deg) : 1.f;
       float dotq = 0.f;
 #pragma unroll
       for (int ks = 0; ks < KS; ks++) {

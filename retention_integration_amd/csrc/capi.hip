@@ -71,7 +71,7 @@ int pr_attention_bwd(const void* Q, const void* K, const void* V, const float* G
   if (B <= 0 || tq <= 0 || tk <= 0 || h <= 0 || r <= 0 || tq > tk)
     return fail(PR_ERR_ARG, "attention_bwd: need B,tq,tk,h,r > 0 and tq <= tk");
   pr::AttnBwdArgs a{Q, K, V, G, rowmax, dO, dl, dO_scale, dQ, dK, dV, G ? dGq : nullptr, G ? dGk : nullptr,
-                    tq, tk, h, r, scale, (float)deg, nullptr, nullptr, nullptr, nullptr};
+                    tq, tk, h, r, scale, (float)deg, nullptr, nullptr, nullptr, nullptr, 0};
   return finish(pr::attention_bwd(a, B, d, dtype, (hipStream_t)stream), "attention_bwd");
 }
 
@@ -79,7 +79,7 @@ int pr_chunk_attention_bwd(const void* Q, const void* K, const void* V, const fl
                            const void* dO, const float* dl, const float* dO_scale, const void* dQ_state,
                            const void* dK_state, const void* dV_state, void* dQ, void* dK, void* dV, float* dGq,
                            float* dGk, float* dotk, int BN, int c, int h, int r, int d, float scale, int deg,
-                           int dtype, void* stream) {
+                           int dQ_state_plain, int dtype, void* stream) {
   if (int rc = check_common("chunk_attention_bwd", d, deg, dtype, false)) return rc;
   if (bad_ptr(Q) || bad_ptr(K) || bad_ptr(V) || bad_ptr(rowmax) || bad_ptr(dO) || bad_ptr(dQ) || bad_ptr(dK) ||
       bad_ptr(dV) || bad_ptr(dQ_state) || bad_ptr(dK_state) || bad_ptr(dV_state) || bad_opt(A) || bad_opt(dl) ||
@@ -89,7 +89,7 @@ int pr_chunk_attention_bwd(const void* Q, const void* K, const void* V, const fl
     return fail(PR_ERR_ARG, "chunk_attention_bwd: dGq, dGk and dotk are required when A is given");
   if (BN <= 0 || c <= 0 || h <= 0 || r <= 0) return fail(PR_ERR_ARG, "chunk_attention_bwd: need BN,c,h,r > 0");
   pr::AttnBwdArgs a{Q, K, V, A, rowmax, dO, dl, dO_scale, dQ, dK, dV, A ? dGq : nullptr, A ? dGk : nullptr,
-                    c, c, h, r, scale, (float)deg, dQ_state, dK_state, dV_state, A ? dotk : nullptr};
+                    c, c, h, r, scale, (float)deg, dQ_state, dK_state, dV_state, A ? dotk : nullptr, dQ_state_plain ? 1 : 0};
   return finish(pr::attention_bwd(a, BN, d, dtype, (hipStream_t)stream), "chunk_attention_bwd");
 }
 
@@ -114,7 +114,7 @@ int pr_update_state_bwd(const void* K, const void* V, const void* dS, const floa
     return fail(PR_ERR_ARG, "update_state_bwd: zero_last_of must be 0 or a divisor of BN (got %d, BN %d)", zero_last_of, BN);
   const int nn_ = zero_last_of > 0 ? zero_last_of : 1, skl = zero_last_of > 0 ? 1 : 0;
   if (dV) {
-    pr::NNArgs nn{K, dS, nullptr, dV, nullptr, nullptr, nullptr, nullptr, 1.f, c, h, 1, nn_, 0, skl};
+    pr::NNArgs nn{K, dS, nullptr, dV, nullptr, nullptr, nullptr, nullptr, 1.f, c, h, 1, nn_, 0, skl, nullptr};
     if (int rc = finish(pr::sympow_nn(nn, BN, d, 1, 0, dtype, (hipStream_t)stream), "update_state_bwd(dV)")) return rc;
   }
   if (!dK) return 0;
@@ -177,17 +177,18 @@ int pr_state_scan_bwd(const void* dS_out, const void* S_out, const float* ds_out
 }
 
 int pr_query_state_fwd(const void* Q, const void* S, const float* s, const void* Y_attn, const float* l_attn,
-                       const float* rowmax, void* O, float* den, int BN, int n, int c, int h, int r, int d,
-                       float scale_p, int deg, int zero_initial_state, int dtype, void* stream) {
+                       const float* rowmax, const float* q_log_gate, void* O, float* den, int BN, int n, int c, int h,
+                       int r, int d, float scale_p, int deg, int zero_initial_state, int dtype, void* stream) {
   if (int rc = check_common("query_state_fwd", d, deg, dtype, true)) return rc;
   if (bad_ptr(Q) || bad_ptr(S) || bad_ptr(s) || bad_ptr(O) || bad_ptr(den) || bad_opt(Y_attn) || bad_opt(l_attn) ||
       bad_opt(rowmax))
     return fail(PR_ERR_ARG, "query_state_fwd: null or misaligned pointer");
   if ((Y_attn != nullptr) != (l_attn != nullptr) || (Y_attn != nullptr) != (rowmax != nullptr))
     return fail(PR_ERR_ARG, "query_state_fwd: Y_attn, l_attn and rowmax must be given together");
+  if (q_log_gate && !Y_attn) return fail(PR_ERR_ARG, "query_state_fwd: q_log_gate needs the attention part (it enters the merge)");
   if (BN <= 0 || n <= 0 || c <= 0 || h <= 0 || r <= 0 || BN % n != 0)
     return fail(PR_ERR_ARG, "query_state_fwd: need BN,n,c,h,r > 0 and BN a multiple of n");
-  pr::NNArgs a{Q, S, s, O, den, Y_attn, l_attn, rowmax, scale_p, c, h, r, n, zero_initial_state ? 1 : 0, 0};
+  pr::NNArgs a{Q, S, s, O, den, Y_attn, l_attn, rowmax, scale_p, c, h, r, n, zero_initial_state ? 1 : 0, 0, q_log_gate};
   return finish(pr::sympow_nn(a, BN, d, 0, 1, dtype, (hipStream_t)stream), "query_state_fwd");
 }
 
@@ -197,8 +198,8 @@ size_t pr_query_state_bwd_workspace(int BN, int c, int h, int r, int d, int dtyp
   return align256(rows * d * 2) + align256(rows * sizeof(float));
 }
 
-int pr_query_state_bwd(const void* Q, const void* S, const float* s, const float* rowmax, const void* O,
-                       const float* den, const void* dO, void* dQ, void* dS, float* ds, void* dY_attn,
+int pr_query_state_bwd(const void* Q, const void* S, const float* s, const float* rowmax, const float* q_log_gate,
+                       const void* O, const float* den, const void* dO, void* dQ, void* dS, float* ds, void* dY_attn,
                        float* dl_attn, float* dY_scale, void* workspace, int BN, int n, int c, int h, int r, int d,
                        float scale_p, int deg, int zero_initial_state, int S_symmetric, int dtype, void* stream) {
   if (int rc = check_common("query_state_bwd", d, deg, dtype, true)) return rc;
@@ -207,15 +208,16 @@ int pr_query_state_bwd(const void* Q, const void* S, const float* s, const float
     return fail(PR_ERR_ARG, "query_state_bwd: null or misaligned pointer");
   if (rowmax && ((!dY_attn && !dY_scale) || !dl_attn))
     return fail(PR_ERR_ARG, "query_state_bwd: dl_attn and one of dY_attn, dY_scale are required when rowmax is given");
+  if (q_log_gate && !rowmax) return fail(PR_ERR_ARG, "query_state_bwd: q_log_gate needs the attention part");
   if (BN <= 0 || n <= 0 || c <= 0 || h <= 0 || r <= 0 || BN % n != 0)
     return fail(PR_ERR_ARG, "query_state_bwd: need BN,n,c,h,r > 0 and BN a multiple of n");
   const size_t rows = (size_t)BN * c * h * r;
   void* dOs = workspace;
   float* cvec = (float*)((char*)workspace + align256(rows * d * 2));
   hipStream_t st = (hipStream_t)stream;
-  if (int rc = finish(pr::qs_bwd_prep(O, dO, den, rowmax, dOs, cvec, rowmax ? dY_attn : nullptr,
-                                      rowmax ? dl_attn : nullptr, rowmax ? dY_scale : nullptr, (long)rows, d, scale_p,
-                                      dtype, st),
+  if (int rc = finish(pr::qs_bwd_prep(O, dO, den, rowmax, q_log_gate, dOs, cvec, rowmax ? dY_attn : nullptr,
+                                      rowmax ? dl_attn : nullptr, rowmax ? dY_scale : nullptr, (long)rows, h, r, d,
+                                      scale_p, dtype, st),
                       "query_state_bwd(prep)"))
     return rc;
   // (zero_initial_state == 2: the caller does not want the gradient of the first chunk's (zero) state either)
@@ -249,8 +251,9 @@ size_t pr_query_state_scan_bwd_workspace(int B, int n, int c, int h, int r, int 
          align256((size_t)pr::scan_gate_grad_workspace_floats(B, n, h, D * d, D) * sizeof(float));
 }
 
-int pr_query_state_scan_bwd(const void* Q, const void* S, const float* s, const float* rowmax, const void* O,
-                            const float* den, const void* dO, const float* log_G, void* dQ, void* dS_in, float* ds_in,
+int pr_query_state_scan_bwd(const void* Q, const void* S, const float* s, const float* rowmax, const float* q_log_gate,
+                            const void* O, const float* den, const void* dO, const float* log_G, void* dQ, void* dS_in,
+                            float* ds_in,
                             void* dY_attn, float* dl_attn, float* dY_scale, float* dlog_G, void* workspace, int B,
                             int n, int c, int h, int r, int d, float scale_p, int deg, int dtype, void* stream) {
   if (int rc = check_common("query_state_scan_bwd", d, deg, dtype, true)) return rc;
@@ -271,9 +274,10 @@ int pr_query_state_scan_bwd(const void* Q, const void* S, const float* s, const 
   float* cvec = (float*)((char*)workspace + align256(rows * d * 2));
   float* part = (float*)((char*)workspace + pr_query_state_bwd_workspace(BN, c, h, r, d, dtype));
   hipStream_t st = (hipStream_t)stream;
-  if (int rc = finish(pr::qs_bwd_prep(O, dO, den, rowmax, dOs, cvec, rowmax ? dY_attn : nullptr,
-                                      rowmax ? dl_attn : nullptr, rowmax ? dY_scale : nullptr, (long)rows, d, scale_p,
-                                      dtype, st),
+  if (q_log_gate && !rowmax) return fail(PR_ERR_ARG, "query_state_scan_bwd: q_log_gate needs the attention part");
+  if (int rc = finish(pr::qs_bwd_prep(O, dO, den, rowmax, q_log_gate, dOs, cvec, rowmax ? dY_attn : nullptr,
+                                      rowmax ? dl_attn : nullptr, rowmax ? dY_scale : nullptr, (long)rows, h, r, d,
+                                      scale_p, dtype, st),
                       "query_state_scan_bwd(prep)"))
     return rc;
   if (int rc = finish(pr::sympow_tn_chain(Q, dOs, cvec, log_G, dS_in, ds_in, B, n, c, h, r, d, 0, 1, dtype, st),
@@ -297,7 +301,7 @@ int pr_gate_cumsum(const float* log_G, float* A, int B, int t, int h, void* stre
 int pr_chunk_prep_fwd(const float* log_G, const void* K, const void* Q, float* A, float* lcs, void* Kd, void* Qg, int BN,
                       int c, int h, int r, int d, int deg, int dtype, void* stream) {
   if (int rc = check_common("chunk_prep_fwd", d, deg, dtype, false)) return rc;
-  if (log_G == nullptr || bad_ptr(K) || bad_ptr(Q) || A == nullptr || lcs == nullptr || bad_ptr(Kd) || bad_ptr(Qg))
+  if (log_G == nullptr || bad_ptr(K) || bad_ptr(Q) || A == nullptr || lcs == nullptr || bad_ptr(Kd) || bad_opt(Qg))
     return fail(PR_ERR_ARG, "chunk_prep_fwd: null or misaligned pointer");
   if (BN <= 0 || c <= 0 || h <= 0 || r <= 0) return fail(PR_ERR_ARG, "chunk_prep_fwd: need BN,c,h,r > 0");
   return finish(pr::chunk_prep_fwd(log_G, K, Q, A, lcs, Kd, Qg, BN, c, h, r, d, deg, dtype, (hipStream_t)stream),

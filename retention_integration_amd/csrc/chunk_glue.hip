@@ -74,7 +74,7 @@ __global__ __launch_bounds__(256) void gate_apply_fwd_kernel(const float* __rest
 #pragma unroll
   for (int i = 0; i < 8; i++) f[i] *= w;
   *(v8*)(Kd + gid * DH + col) = pack8<T>(f);
-  for (int rr = 0; rr < r; rr++) {
+  for (int rr = 0; Qg && rr < r; rr++) {
     const long o = (gid * r + rr) * DH + col;
     unpack8(*(const v8*)(Q + o), f);
 #pragma unroll

@@ -10,10 +10,11 @@ namespace pr {
 template <typename T, int DH>
 __global__ __launch_bounds__(256) void qs_bwd_prep_kernel(const T* __restrict__ O, const T* __restrict__ dO,
                                                           const float* __restrict__ den,
-                                                          const float* __restrict__ rowmax, T* __restrict__ dOs,
+                                                          const float* __restrict__ rowmax,
+                                                          const float* __restrict__ qgate, T* __restrict__ dOs,
                                                           float* __restrict__ cvec, T* __restrict__ dYa,
                                                           float* __restrict__ dla, float* __restrict__ dYscale,
-                                                          long rows, float scale_p) {
+                                                          long rows, int h, int rr, float scale_p) {
   typedef typename VecOf<T>::v8 v8;
   constexpr int LPR = DH / 8;  // lanes per row
   const long gid = (long)blockIdx.x * blockDim.x + threadIdx.x;
@@ -35,7 +36,9 @@ __global__ __launch_bounds__(256) void qs_bwd_prep_kernel(const T* __restrict__ 
     constexpr int D = 128 * (DH / 16) * (DH / 16 + 1);
     const float m = rowmax[r], beta = fmaxf(m, 0.5f * __logf((float)D));
     wa = __expf(m - beta);
-    wq = scale_p * __expf(-beta);
+    // the forward's log factor on the state part of this row: rows are (.., position, kv head, query head of it)
+    const float qg = qgate ? qgate[(r / ((long)h * rr)) * h + (r % ((long)h * rr)) / rr] : 0.f;
+    wq = scale_p * __expf(qg - beta);
   }
   if (!live) return;
   // Row factors of the two parts.  They are ~1e-3..1 unless the row's total weight is ~0 (a zero query: 1/den is
@@ -65,27 +68,29 @@ __global__ __launch_bounds__(256) void qs_bwd_prep_kernel(const T* __restrict__ 
 }
 
 template <typename T>
-static int prep_launch(const void* O, const void* dO, const float* den, const float* rowmax, void* dOs, float* cvec,
-                       void* dYa, float* dla, float* dYscale, long rows, int d, float scale_p, hipStream_t st) {
+static int prep_launch(const void* O, const void* dO, const float* den, const float* rowmax, const float* qgate, void* dOs,
+                       float* cvec, void* dYa, float* dla, float* dYscale, long rows, int h, int r, int d, float scale_p,
+                       hipStream_t st) {
   const long threads = rows * (d / 8);
   dim3 grid((unsigned)((threads + 255) / 256));
 #define PR_PREP(DD)                                                                                                    \
   case DD:                                                                                                             \
     hipLaunchKernelGGL((qs_bwd_prep_kernel<T, DD>), grid, dim3(256), 0, st, (const T*)O, (const T*)dO, den, rowmax,    \
-                       (T*)dOs, cvec, (T*)dYa, dla, dYscale, rows, scale_p);                                                    \
+                       qgate, (T*)dOs, cvec, (T*)dYa, dla, dYscale, rows, h, r, scale_p);                              \
     break;
   switch (d) { PR_PREP(32) PR_PREP(64) PR_PREP(128) default: return -2; }
 #undef PR_PREP
   return (int)hipGetLastError();
 }
 
-int qs_bwd_prep(const void* O, const void* dO, const float* den, const float* rowmax, void* dOs, float* cvec,
-                void* dY_attn, float* dl_attn, float* dY_scale, long rows, int d, float scale_p, int dtype,
-                hipStream_t st) {
+int qs_bwd_prep(const void* O, const void* dO, const float* den, const float* rowmax, const float* qgate, void* dOs,
+                float* cvec, void* dY_attn, float* dl_attn, float* dY_scale, long rows, int h, int r, int d, float scale_p,
+                int dtype, hipStream_t st) {
+  if (qgate && !rowmax) return -3;   // the gate enters through the merge weights
   if (dtype == DT_BF16)
-    return prep_launch<bf16_t>(O, dO, den, rowmax, dOs, cvec, dY_attn, dl_attn, dY_scale, rows, d, scale_p, st);
+    return prep_launch<bf16_t>(O, dO, den, rowmax, qgate, dOs, cvec, dY_attn, dl_attn, dY_scale, rows, h, r, d, scale_p, st);
   if (dtype == DT_F16)
-    return prep_launch<f16_t>(O, dO, den, rowmax, dOs, cvec, dY_attn, dl_attn, dY_scale, rows, d, scale_p, st);
+    return prep_launch<f16_t>(O, dO, den, rowmax, qgate, dOs, cvec, dY_attn, dl_attn, dY_scale, rows, h, r, d, scale_p, st);
   return -1;
 }
 

@@ -49,6 +49,8 @@ struct NNArgs {
   int c, h, r, n;       // n: chunks per batch entry
   int skip_first;       // chunk 0 of every batch entry has a zero state
   int skip_last;        // chunk n-1 of every batch entry has a zero B: the output there is zero (nothing is read)
+  const float* qgate;   // [BN, c, h] or null (merge only): log of a factor on the state part of every row of a kv head
+                        // at a position -- out and den are those of X * exp(qgate / 2) without forming that product
 };
 int sympow_nn(const NNArgs& a, int BN, int d, int mult, int epi, int dtype, hipStream_t st);
 
@@ -104,15 +106,19 @@ struct AttnBwdArgs {
   const void* dKs;      // [B, tk, h, d]:   dK = dK_attn + dKs * w, w = exp((G_last - G_k)/deg); dGk -= (K.dKs) w / deg
   const void* dVs;      // [B, tk, h, d]:   dV = dV_attn + dVs
   float* dotk;          // [B, tk, h]:      (K.dKs) w
+  int dQs_plain;        // dQs is already the gradient w.r.t. Q itself: dQ = dQ_attn + dQs, dGq += (Q.dQs) / deg
 };
 int attention_bwd(const AttnBwdArgs& a, int B, int d, int dtype, hipStream_t st);
 
 // elementwise.hip
-int qs_bwd_prep(const void* O, const void* dO, const float* den, const float* rowmax, void* dOs, float* cvec,
-                void* dY_attn, float* dl_attn, float* dY_scale, long rows, int d, float scale_p, int dtype, hipStream_t st);
+// qgate [rows / (h*r), h] or null: the forward's log factor on the state part (see NNArgs); rows are (.., position, h*r)
+int qs_bwd_prep(const void* O, const void* dO, const float* den, const float* rowmax, const float* qgate, void* dOs,
+                float* cvec, void* dY_attn, float* dl_attn, float* dY_scale, long rows, int h, int r, int d, float scale_p,
+                int dtype, hipStream_t st);
 
 // chunk_glue.hip (return -5: chunk longer than the LDS-resident gate vector allows)
 int gate_cumsum(const float* logG, float* A, int B, int t, int h, hipStream_t st);
+// (Qg may be null: the gated queries are then not formed)
 int chunk_prep_fwd(const float* logG, const void* K, const void* Q, float* A, float* lcs, void* Kd, void* Qg, int BN,
                    int c, int h, int r, int d, int deg, int dtype, hipStream_t st);
 int chunk_gate_scan_bwd(float* dA, const float* dGq, const float* dotk, const float* dlcs_a, const float* dlcs_b, int BN,

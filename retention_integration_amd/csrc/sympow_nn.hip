@@ -304,7 +304,10 @@ __global__ __launch_bounds__(256, DK <= 64 ? 3 : 2) void sympow_nn_kernel(NNArgs
         for (int nt = 0; nt < NT; nt++) ya4[nt] = *(const v4*)(ya + 16 * nt + 4 * g);
         const float beta = fmaxf(m, log_gamma);
         wa = __expf(m - beta);
-        wq = a.scale_p * __expf(-beta);
+        // (gates only decay, so the exponent only shrinks: no range problem; a row whose gate has decayed to nothing
+        // keeps its attention part alone, as a gated query rounded to zero would)
+        const float qg = a.qgate ? a.qgate[((long)bn * a.c + min(row, rows - 1) / a.r) * a.h + hh] : 0.f;
+        wq = a.scale_p * __expf(qg - beta);
       }
       const float den = la * wa + lqs * wq;
       const float inv = 1.f / den;

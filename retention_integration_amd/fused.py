@@ -55,8 +55,12 @@ def _empty(shape, dtype, device):
 
 @torch.library.custom_op("pr::chunked_fwd", mutates_args=(), device_types="cuda")
 def chunked_fwd(Q: Tensor, K: Tensor, V: Tensor, log_G: Optional[Tensor], deg: int, scale: float,
-                c: int) -> Tuple[Tensor, Tensor, Tensor, Tensor, Tensor, Tensor, Tensor, Tensor, Tensor]:
-    """-> O, and what the backward needs: A, lcs, Kd, Qg (empty when ungated), Sc, sc, rowmax, den."""
+                c: int) -> Tuple[Tensor, Tensor, Tensor, Tensor, Tensor, Tensor, Tensor, Tensor]:
+    """-> O, and what the backward needs: A, lcs, Kd (empty when ungated), Sc, sc, rowmax, den.
+
+    The gated queries Q * exp(A / deg) (ref: retention/power_retention_maker.py:183-186) are never formed: the state part
+    is homogeneous of degree deg in the query, so the gate is a per-row factor exp(A) on it, applied where the state
+    part is merged with the attention part (and, in the backward, in the per-row factor of dO)."""
     lib = _lib.load()
     st = _lib.stream()
     b, t, hq, d = Q.shape
@@ -73,13 +77,13 @@ def chunked_fwd(Q: Tensor, K: Tensor, V: Tensor, log_G: Optional[Tensor], deg: i
 
     if gated:
         A, lcs = _empty((BN, c, h), f32, dev), _empty((BN, h), f32, dev)
-        Kd, Qg = torch.empty_like(K), torch.empty_like(Q)
-        _lib.check(lib.pr_chunk_prep_fwd(p(log_G), p(K), p(Q), p(A), p(lcs), p(Kd), p(Qg), BN, c, h, r, d, deg, code,
+        Kd = torch.empty_like(K)
+        _lib.check(lib.pr_chunk_prep_fwd(p(log_G), p(K), p(Q), p(A), p(lcs), p(Kd), None, BN, c, h, r, d, deg, code,
                                          st), "chunk_prep_fwd")
-        Kd_, Qg_ = Kd, Qg
+        Kd_ = Kd
     else:
-        A, Kd, Qg = _empty((0,), f32, dev), _empty((0,), dt, dev), _empty((0,), dt, dev)
-        Kd_, Qg_ = K, Q
+        A, Kd = _empty((0,), f32, dev), _empty((0,), dt, dev)
+        Kd_ = K
         lcs = torch.zeros((BN, h), dtype=f32, device=dev)
 
     Sc, sc = _empty((BN, h, D, d), dt, dev), _empty((BN, h, D), f32, dev)
@@ -100,9 +104,9 @@ def chunked_fwd(Q: Tensor, K: Tensor, V: Tensor, log_G: Optional[Tensor], deg: i
     _lib.check(lib.pr_attention_fwd(p(Q), p(K), p(V), p(A) if gated else None, p(Ya), p(la), p(rm), BN, c, c, h, r, d,
                                     scale, deg, 0, code, st), "attention_fwd")
     O, den = torch.empty_like(Q), _empty((BN, c, hq), f32, dev)
-    _lib.check(lib.pr_query_state_fwd(p(Qg_), p(Sc), p(sc), p(Ya), p(la), p(rm), p(O), p(den), BN, n, c, h, r, d,
-                                      scale ** deg, deg, 1, code, st), "query_state_fwd")
-    return O, A, lcs, Kd, Qg, Sc, sc, rm, den
+    _lib.check(lib.pr_query_state_fwd(p(Q), p(Sc), p(sc), p(Ya), p(la), p(rm), p(A) if gated else None, p(O), p(den),
+                                      BN, n, c, h, r, d, scale ** deg, deg, 1, code, st), "query_state_fwd")
+    return O, A, lcs, Kd, Sc, sc, rm, den
 
 
 @chunked_fwd.register_fake
@@ -114,18 +118,19 @@ def _(Q, K, V, log_G, deg, scale, c):
     gated = log_G is not None
     A = Q.new_empty((BN, c, h) if gated else (0,), dtype=f32)
     return (torch.empty_like(Q), A, Q.new_empty((BN, h), dtype=f32),
-            torch.empty_like(K) if gated else K.new_empty((0,)), torch.empty_like(Q) if gated else Q.new_empty((0,)),
+            torch.empty_like(K) if gated else K.new_empty((0,)),
             Q.new_empty((BN, h, D, d)), Q.new_empty((BN, h, D), dtype=f32), Q.new_empty((BN, c, hq), dtype=f32),
             Q.new_empty((BN, c, hq), dtype=f32))
 
 
 @torch.library.custom_op("pr::chunked_bwd", mutates_args=(), device_types="cuda")
-def chunked_bwd(Q: Tensor, K: Tensor, V: Tensor, A: Tensor, lcs: Tensor, Kd: Tensor, Qg: Tensor, Sc: Tensor,
+def chunked_bwd(Q: Tensor, K: Tensor, V: Tensor, A: Tensor, lcs: Tensor, Kd: Tensor, Sc: Tensor,
                 sc: Tensor, rm: Tensor, O: Tensor, den: Tensor, dO: Tensor, deg: int, scale: float, c: int,
                 gated: bool) -> Tuple[Tensor, Tensor, Tensor, Tensor]:
     """-> dQ, dK, dV, dlog_G (empty when ungated)."""
     if not gated:
-        Kd, Qg = K, Q
+        Kd = K
+    qgate = _lib.ptr(A) if gated else None
     lib = _lib.load()
     st = _lib.stream()
     b, t, hq, d = Q.shape
@@ -146,14 +151,14 @@ def chunked_bwd(Q: Tensor, K: Tensor, V: Tensor, A: Tensor, lcs: Tensor, Kd: Ten
     dlcs = torch.empty_like(lcs)   # gate gradient of both scans
     if _chained(lib, b, n, c, h, r, d):
         ws = _empty((lib.pr_query_state_scan_bwd_workspace(b, n, c, h, r, d, code),), u8, dev)
-        _lib.check(lib.pr_query_state_scan_bwd(p(Qg), p(Sc), p(sc), p(rm), p(O), p(den), p(dO),
+        _lib.check(lib.pr_query_state_scan_bwd(p(Q), p(Sc), p(sc), p(rm), qgate, p(O), p(den), p(dO),
                                                p(lcs) if gated else None, p(dQg), p(dS), p(ds), None, p(dla), p(dys),
                                                p(dlcs) if gated else None, p(ws), b, n, c, h, r, d, scale ** deg, deg,
                                                code, st), "query_state_scan_bwd")
     else:
         dSc, dsc = torch.empty_like(Sc), torch.empty_like(sc)
         ws = _empty((lib.pr_query_state_bwd_workspace(BN, c, h, r, d, code),), u8, dev)
-        _lib.check(lib.pr_query_state_bwd(p(Qg), p(Sc), p(sc), p(rm), p(O), p(den), p(dO), p(dQg), p(dSc), p(dsc),
+        _lib.check(lib.pr_query_state_bwd(p(Q), p(Sc), p(sc), p(rm), qgate, p(O), p(den), p(dO), p(dQg), p(dSc), p(dsc),
                                           None, p(dla), p(dys), p(ws), BN, n, c, h, r, d, scale ** deg, deg, 2, 1, code,
                                           st),
                    "query_state_bwd")
@@ -176,7 +181,7 @@ def chunked_bwd(Q: Tensor, K: Tensor, V: Tensor, A: Tensor, lcs: Tensor, Kd: Ten
     dotk = _empty((BN, c, h), f32, dev) if gated else None
     _lib.check(lib.pr_chunk_attention_bwd(p(Q), p(K), p(V), p(A) if gated else None, p(rm), p(dO), p(dla), p(dys), p(dQg), p(dKd),
                                           p(dVs), p(dQa), p(dKa), p(dVa), p(dGq), p(dGk), p(dotk), BN, c, h, r, d,
-                                          scale, deg, code, st), "chunk_attention_bwd")
+                                          scale, deg, 1, code, st), "chunk_attention_bwd")
     dlg = _empty((0,), f32, dev)
     if gated:
         dlg = dGk
@@ -186,7 +191,7 @@ def chunked_bwd(Q: Tensor, K: Tensor, V: Tensor, A: Tensor, lcs: Tensor, Kd: Ten
 
 
 @chunked_bwd.register_fake
-def _(Q, K, V, A, lcs, Kd, Qg, Sc, sc, rm, O, den, dO, deg, scale, c, gated):
+def _(Q, K, V, A, lcs, Kd, Sc, sc, rm, O, den, dO, deg, scale, c, gated):
     b, t, _, _ = Q.shape
     h = K.shape[2]
     return (torch.empty_like(Q), torch.empty_like(K), torch.empty_like(V),
@@ -195,18 +200,18 @@ def _(Q, K, V, A, lcs, Kd, Qg, Sc, sc, rm, O, den, dO, deg, scale, c, gated):
 
 def _chunked_setup(ctx, inputs, output):
     Q, K, V, log_G, deg, scale, c = inputs
-    O, A, lcs, Kd, Qg, Sc, sc, rm, den = output
-    ctx.save_for_backward(Q, K, V, A, lcs, Kd, Qg, Sc, sc, rm, O, den)
+    O, A, lcs, Kd, Sc, sc, rm, den = output
+    ctx.save_for_backward(Q, K, V, A, lcs, Kd, Sc, sc, rm, O, den)
     ctx.meta = (deg, scale, c, log_G is not None)
     ctx.set_materialize_grads(False)
 
 
 def _chunked_backward(ctx, dO, *unused):
-    Q, K, V, A, lcs, Kd, Qg, Sc, sc, rm, O, den = ctx.saved_tensors
+    Q, K, V, A, lcs, Kd, Sc, sc, rm, O, den = ctx.saved_tensors
     deg, scale, c, gated = ctx.meta
     if dO is None:
         return None, None, None, None, None, None, None
-    dQ, dK, dV, dlg = chunked_bwd(Q, K, V, A, lcs, Kd, Qg, Sc, sc, rm, O, den, dO, deg, scale, c, gated)
+    dQ, dK, dV, dlg = chunked_bwd(Q, K, V, A, lcs, Kd, Sc, sc, rm, O, den, dO, deg, scale, c, gated)
     return dQ, dK, dV, (dlg if gated else None), None, None, None
 
 

@@ -284,7 +284,7 @@ def query_state_fwd(Q: Tensor, S: Tensor, s: Tensor, Y_attn: Optional[Tensor], l
     den = torch.empty((b, n, c, hq), dtype=torch.float32, device=Q.device)
     lib = _lib.load()
     _lib.check(lib.pr_query_state_fwd(_lib.ptr(Q), _lib.ptr(S), _lib.ptr(s), _lib.ptr(Y_attn), _lib.ptr(l_attn),
-                                      _lib.ptr(rowmax), _lib.ptr(O), _lib.ptr(den), b * n, n, c, h, hq // h, d,
+                                      _lib.ptr(rowmax), None, _lib.ptr(O), _lib.ptr(den), b * n, n, c, h, hq // h, d,
                                       float(scale_p), 2, int(zero_initial_state), _lib.dtype_code(Q.dtype),
                                       _lib.stream()), "query_state_fwd")
     return O, den
@@ -308,7 +308,7 @@ def query_state_bwd(Q: Tensor, S: Tensor, s: Tensor, rowmax: Optional[Tensor], O
     lib = _lib.load()
     code = _lib.dtype_code(Q.dtype)
     ws = torch.empty((lib.pr_query_state_bwd_workspace(b * n, c, h, r, d, code),), dtype=torch.uint8, device=Q.device)
-    _lib.check(lib.pr_query_state_bwd(_lib.ptr(Q), _lib.ptr(S), _lib.ptr(s), _lib.ptr(rowmax), _lib.ptr(O),
+    _lib.check(lib.pr_query_state_bwd(_lib.ptr(Q), _lib.ptr(S), _lib.ptr(s), _lib.ptr(rowmax), None, _lib.ptr(O),
                                       _lib.ptr(den), _lib.ptr(dO), _lib.ptr(dQ), _lib.ptr(dS), _lib.ptr(ds),
                                       _lib.ptr(dYa), _lib.ptr(dla), None, _lib.ptr(ws), b * n, n, c, h, r, d,
                                       float(scale_p), 2, int(zero_initial_state), 0, code, _lib.stream()),
