@@ -118,7 +118,7 @@ int pr_update_state_bwd(const void* K, const void* V, const void* dS, const floa
     if (int rc = finish(pr::sympow_nn(nn, BN, d, 1, 0, dtype, (hipStream_t)stream), "update_state_bwd(dV)")) return rc;
   }
   if (!dK) return 0;
-  pr::GradArgs g{K, V, nullptr, dS, ds, dK, c, h, 1, nn_, 0, dS_symmetric ? 1 : 0, skl};
+  pr::GradArgs g{K, V, nullptr, dS, ds, dK, c, h, 1, nn_, skl ? 2 : 0, dS_symmetric ? 1 : 0};
   return finish(pr::sympow_grad(g, BN, d, 1, dtype, (hipStream_t)stream), "update_state_bwd(dK)");
 }
 
@@ -224,7 +224,7 @@ int pr_query_state_bwd(const void* Q, const void* S, const float* s, const float
   if (int rc = finish(pr::sympow_tn(Q, dOs, cvec, dS, ds, BN, c, h, r, d, 0, zero_initial_state == 2 ? -n : 0, dtype, st),
                       "query_state_bwd(dS)"))
     return rc;
-  pr::GradArgs g{Q, dOs, cvec, S, s, dQ, c, h, r, n, zero_initial_state ? 1 : 0, S_symmetric ? 1 : 0, 0};
+  pr::GradArgs g{Q, dOs, cvec, S, s, dQ, c, h, r, n, zero_initial_state ? 1 : 0, S_symmetric ? 1 : 0};
   return finish(pr::sympow_grad(g, BN, d, 0, dtype, st), "query_state_bwd(dQ)");
 }
 
@@ -287,7 +287,7 @@ int pr_query_state_scan_bwd(const void* Q, const void* S, const float* s, const 
     if (int rc = finish(pr::scan_gate_grad(S, dS_in, s, ds_in, log_G, dlog_G, part, B, n, h, D * d, D, dtype, st),
                         "query_state_scan_bwd(dlog_G)"))
       return rc;
-  pr::GradArgs g{Q, dOs, cvec, S, s, dQ, c, h, r, n, 1, 0, 0};
+  pr::GradArgs g{Q, dOs, cvec, S, s, dQ, c, h, r, n, 1, 0};
   return finish(pr::sympow_grad(g, BN, d, 0, dtype, st), "query_state_scan_bwd(dQ)");
 }
 

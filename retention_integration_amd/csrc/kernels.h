@@ -63,9 +63,9 @@ struct GradArgs {
   const float* sB;    // [BN, h, D]
   void* dX;           // [BN, c, h*r, d]
   int c, h, r, n;
-  int skip_first;     // chunk 0 of every batch entry has a zero state: dX = 0 there
+  int skip_first;     // bit 0: chunk 0 of every batch entry has a zero state, bit 1: chunk n-1 has a zero B: dX = 0
+                      // there and nothing is read
   int sym_diag;       // B[(a, b)] == B[(b, a)] in the blocks on the diagonal (the caller's promise)
-  int skip_last;      // chunk n-1 of every batch entry has a zero B: dX = 0 there (nothing is read)
 };
 int sympow_grad(const GradArgs& a, int BN, int d, int mult, int dtype, hipStream_t st);
 

@@ -85,7 +85,8 @@ __global__ __launch_bounds__(256, (MT == 2 && DK <= 64) ? 4 : 2) void sympow_gra
     return (long)t * hA + hh * a.r + rr;
   };
 
-  if ((a.skip_first && (bn % a.n == 0)) || (a.skip_last && (bn % a.n == a.n - 1))) {
+  // (skip_first: bit 0 = the first, bit 1 = the last chunk of every n contributes nothing and is written as zeros)
+  if (a.skip_first && (((a.skip_first & 1) && bn % a.n == 0) || ((a.skip_first & 2) && bn % a.n == a.n - 1))) {
     for (int i = tid; i < ROWS * DK / 8; i += 256) {
       const int rl = i / (DK / 8), col = (i % (DK / 8)) * 8;
       if (row0 + rl < rows) *(u32x4*)(dXg + row_off(row0 + rl) * DK + col) = (u32x4){0, 0, 0, 0};
