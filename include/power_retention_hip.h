@@ -39,7 +39,7 @@ enum {
 /* 2: pr_update_state_bwd and pr_query_state_bwd take the symmetric-state promise (dS_symmetric, S_symmetric).
  * 3: pr_decode_step_noalloc.  4: pr_cache_append, pr_cache_attention_fwd; pr_update_state_fwd takes skip_last_of and
  * pr_update_state_bwd zero_last_of; pr_query_state_fwd / _bwd / _scan_bwd take q_log_gate and
- * pr_chunk_attention_bwd dQ_state_plain. */
+ * pr_chunk_attention_bwd dQ_state_plain.  5: pr_query_state_fwd takes S_symmetric. */
 int pr_abi_version(void);
 const char* pr_last_error(void);
 
@@ -147,10 +147,14 @@ int pr_query_state_scan_bwd(const void* Q, const void* S, const float* s, const 
  *   retention/power_retention_maker.py:183-186 without the gated copy -- with it, Q is the UNGATED query and the result
  *   is that of Q * exp(q_log_gate / deg): the state part is homogeneous of degree deg in the query, so the gate is a
  *   factor exp(q_log_gate) on that part of each row and is applied in the merge (exact; the reference rounds the gated
- *   copy to 16 bits first). */
+ *   copy to 16 bits first).
+ *   S_symmetric != 0: the caller's promise that S[(a,b)] == S[(b,a)] in the blocks on the diagonal (true of every
+ *   state made by pr_update_state_fwd and the scans): the mirrored quarter of each such block is then not read
+ *   (a tenth of the state less to contract). */
 int pr_query_state_fwd(const void* Q, const void* S, const float* s, const void* Y_attn, const float* l_attn,
                        const float* rowmax, const float* q_log_gate, void* O, float* den, int BN, int n, int c, int h,
-                       int r, int d, float scale_p, int deg, int zero_initial_state, int dtype, void* stream);
+                       int r, int d, float scale_p, int deg, int zero_initial_state, int S_symmetric, int dtype,
+                       void* stream);
 
 /* Backward -- formulas of retention/_query_state/triton.py:546-553 (kernels :184-448).
  *   O, den from the forward; dO [BN,c,h*r,d]

@@ -38,7 +38,7 @@ size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 
 extern "C" {
 
-int pr_abi_version(void) { return 4; }
+int pr_abi_version(void) { return 5; }
 const char* pr_last_error(void) { return g_err; }
 
 int pr_expanded_dim(int d, int deg) {
@@ -114,7 +114,7 @@ int pr_update_state_bwd(const void* K, const void* V, const void* dS, const floa
     return fail(PR_ERR_ARG, "update_state_bwd: zero_last_of must be 0 or a divisor of BN (got %d, BN %d)", zero_last_of, BN);
   const int nn_ = zero_last_of > 0 ? zero_last_of : 1, skl = zero_last_of > 0 ? 1 : 0;
   if (dV) {
-    pr::NNArgs nn{K, dS, nullptr, dV, nullptr, nullptr, nullptr, nullptr, 1.f, c, h, 1, nn_, 0, skl, nullptr};
+    pr::NNArgs nn{K, dS, nullptr, dV, nullptr, nullptr, nullptr, nullptr, 1.f, c, h, 1, nn_, 0, skl, dS_symmetric ? 1 : 0, nullptr};
     if (int rc = finish(pr::sympow_nn(nn, BN, d, 1, 0, dtype, (hipStream_t)stream), "update_state_bwd(dV)")) return rc;
   }
   if (!dK) return 0;
@@ -178,7 +178,8 @@ int pr_state_scan_bwd(const void* dS_out, const void* S_out, const float* ds_out
 
 int pr_query_state_fwd(const void* Q, const void* S, const float* s, const void* Y_attn, const float* l_attn,
                        const float* rowmax, const float* q_log_gate, void* O, float* den, int BN, int n, int c, int h,
-                       int r, int d, float scale_p, int deg, int zero_initial_state, int dtype, void* stream) {
+                       int r, int d, float scale_p, int deg, int zero_initial_state, int S_symmetric, int dtype,
+                       void* stream) {
   if (int rc = check_common("query_state_fwd", d, deg, dtype, true)) return rc;
   if (bad_ptr(Q) || bad_ptr(S) || bad_ptr(s) || bad_ptr(O) || bad_ptr(den) || bad_opt(Y_attn) || bad_opt(l_attn) ||
       bad_opt(rowmax))
@@ -188,7 +189,8 @@ int pr_query_state_fwd(const void* Q, const void* S, const float* s, const void*
   if (q_log_gate && !Y_attn) return fail(PR_ERR_ARG, "query_state_fwd: q_log_gate needs the attention part (it enters the merge)");
   if (BN <= 0 || n <= 0 || c <= 0 || h <= 0 || r <= 0 || BN % n != 0)
     return fail(PR_ERR_ARG, "query_state_fwd: need BN,n,c,h,r > 0 and BN a multiple of n");
-  pr::NNArgs a{Q, S, s, O, den, Y_attn, l_attn, rowmax, scale_p, c, h, r, n, zero_initial_state ? 1 : 0, 0, q_log_gate};
+  pr::NNArgs a{Q, S, s, O, den, Y_attn, l_attn, rowmax, scale_p, c, h, r, n, zero_initial_state ? 1 : 0, 0,
+               S_symmetric ? 1 : 0, q_log_gate};
   return finish(pr::sympow_nn(a, BN, d, 0, 1, dtype, (hipStream_t)stream), "query_state_fwd");
 }
 

@@ -49,6 +49,8 @@ struct NNArgs {
   int c, h, r, n;       // n: chunks per batch entry
   int skip_first;       // chunk 0 of every batch entry has a zero state
   int skip_last;        // chunk n-1 of every batch entry has a zero B: the output there is zero (nothing is read)
+  int sym_diag;         // B[(a, b)] == B[(b, a)] in the blocks on the diagonal (the caller's promise): the mirrored
+                        // quarter of every such block is not read
   const float* qgate;   // [BN, c, h] or null (merge only): log of a factor on the state part of every row of a kv head
                         // at a position -- out and den are those of X * exp(qgate / 2) without forming that product
 };

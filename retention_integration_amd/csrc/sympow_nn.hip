@@ -26,8 +26,16 @@ constexpr int NN_NST = 2;   // two stages keep three workgroups (12 waves) resid
 
 // Stage order over (strip y, first x column X0, a multiple of 4).  With the key-side multiplier the tiles
 // below the block diagonal come first so that the accumulators can be doubled once.
-template <bool MULT> struct FeatIter {
+//
+// SYM (the caller's promise that B[(a, b)] == B[(b, a)] inside the blocks on the diagonal): a diagonal block is cut
+// into its four 8 x 8 quarters (x half, w half).  Quarter (1, 0) is the mirror image of (0, 1) and is never read;
+// (0, 1) counts twice instead.  The block then takes three stages instead of four: x columns 0-3 and 4-7 as before
+// (with the w half 8..15 weighted 2) and ONE stage for quarter (1, 1), eight x columns times the eight w of the
+// upper half ("narrow" stage).
+template <bool MULT, bool SYM> struct FeatIter {
   int y, X0, phase, T;
+  __device__ bool narrow() const { return SYM && X0 == 16 * y + 8; }
+  __device__ bool enters_diag() const { return SYM && X0 == 16 * y; }
   __device__ void init(int T_) {
     T = T_;
     if (MULT && T > 1) { phase = 0; y = 1; X0 = 0; } else { phase = MULT ? 1 : 2; y = 0; X0 = 0; }
@@ -36,7 +44,7 @@ template <bool MULT> struct FeatIter {
   __device__ int f0() const { return 128 * y * (y + 1) + 16 * X0; }
   // returns true when the stage just consumed was the last one below the diagonal
   __device__ bool next() {
-    X0 += 4;
+    X0 += narrow() ? 8 : 4;
     if (phase == 0) {
       if (X0 == 16 * y) { y++; X0 = 0; }
       if (y == T) { phase = 1; y = 0; X0 = 0; return true; }
@@ -57,6 +65,10 @@ template <typename T> struct PhiRow;
 template <> struct PhiRow<bf16_t> {
   float row[8];
   __device__ __forceinline__ void load(const char* p) { unpack8(*(const bf16x8*)p, row); }
+  __device__ __forceinline__ void scale(float f) {
+#pragma unroll
+    for (int i = 0; i < 8; i++) row[i] *= f;
+  }
   __device__ __forceinline__ bf16x8 make(bf16_t x) const {
     const float xs = (float)x;
     float p[8];
@@ -68,10 +80,11 @@ template <> struct PhiRow<bf16_t> {
 template <> struct PhiRow<f16_t> {
   f16x8 row;
   __device__ __forceinline__ void load(const char* p) { row = *(const f16x8*)p; }
+  __device__ __forceinline__ void scale(float f) { row = row * (f16_t)f; }
   __device__ __forceinline__ f16x8 make(f16_t x) const { return row * x; }
 };
 
-template <typename T, int DK, int DV, int MT, bool MULT, int EPI>
+template <typename T, int DK, int DV, int MT, bool MULT, int EPI, bool SYM>
 __global__ __launch_bounds__(256, DK <= 64 ? 3 : 2) void sympow_nn_kernel(NNArgs a, int row_blocks, int npairs) {
   typedef typename VecOf<T>::v8 v8;
   typedef typename VecOf<T>::v4 v4;
@@ -110,11 +123,27 @@ __global__ __launch_bounds__(256, DK <= 64 ? 3 : 2) void sympow_nn_kernel(NNArgs
     const int pos = (ii * 4 + wave) * 64 + l, row = pos / CB;
     boffs[ii] = (uint32_t)(row * (DV * 2) + 16 * ((pos % CB) ^ swz<CB>(row)));
   }
+  // the narrow stage of a symmetric diagonal block: eight x columns, the upper eight w of each.  Contraction step
+  // ks, lane group g take x column 8 + 2*ks + (g & 1) + 4*(g >> 1), so that, as in every other stage, the x scalar of
+  // step ks sits 4*ks bytes past a lane constant; stage row j = 32*ks + 8*g + i is B row 16 * column + 8 + i.
+  uint32_t boffs_n[SYM ? LOADS : 1];
+  if constexpr (SYM) {
+#pragma unroll
+    for (int ii = 0; ii < LOADS; ii++) {
+      const int pos = (ii * 4 + wave) * 64 + l, row = pos / CB;
+      const int gg = (row / 8) % 4, xcol = 2 * (row / 32) + (gg & 1) + 4 * (gg >> 1);
+      boffs_n[ii] = (uint32_t)((16 * xcol + 8 + row % 8) * (DV * 2) + 16 * ((pos % CB) ^ swz<CB>(row)));
+    }
+  }
   const uint32_t ring_lds = lds_addr(ring) + wave * 1024;
-  auto issue = [&](int f0, int ringpos) {
+  auto issue = [&](int f0, int ringpos, bool narrow) {
     const char* src = Bg + (long)f0 * DV * 2;
 #pragma unroll
-    for (int ii = 0; ii < LOADS; ii++) async_copy16_sv(src, boffs[ii], ring_lds + ringpos * STAGE + ii * 4096);
+    for (int ii = 0; ii < LOADS; ii++) {
+      uint32_t bo = boffs[ii];
+      if constexpr (SYM) bo = narrow ? boffs_n[ii] : bo;
+      async_copy16_sv(src, bo, ring_lds + ringpos * STAGE + ii * 4096);
+    }
   };
 
   const bool skip = ((EPI == NN_EPI_MERGE) && a.skip_first && (bn % a.n == 0)) || (a.skip_last && (bn % a.n == a.n - 1));
@@ -132,12 +161,12 @@ __global__ __launch_bounds__(256, DK <= 64 ? 3 : 2) void sympow_nn_kernel(NNArgs
     wait_vmcnt<0>();
     lds_barrier();
   } else {
-    FeatIter<MULT> cur, nxt;
+    FeatIter<MULT, SYM> cur, nxt;
     cur.init(TT);
     nxt.init(TT);
     int issued = 0;
     for (; issued < NN_NST - 1 && !nxt.done(); issued++) {
-      issue(nxt.f0(), issued % NN_NST);
+      issue(nxt.f0(), issued % NN_NST, nxt.narrow());
       nxt.next();
     }
     PhiRow<T> prow[MT];
@@ -157,25 +186,34 @@ __global__ __launch_bounds__(256, DK <= 64 ? 3 : 2) void sympow_nn_kernel(NNArgs
         const int row = 8 * g + 4 * hf + (tcol >> 2), col = 16 * nt + 4 * (tcol & 3);
         boff[nt][hf] = row * (CB * 16) + (((col / 8) ^ swz<CB>(row)) * 16) + (col % 8) * 2;
       }
-    uint32_t xrow_a[MT], xsw[MT];   // start of this lane's row of the X tile (+ the lane's column parity), its swizzle
+    const int xlane = 2 * (g >> 1), xlane_n = 2 * ((g & 1) + 4 * (g >> 1));   // byte offsets of the lane's x column
+    uint32_t xrow_a[MT], xsw[MT];   // start of this lane's row of the X tile, its swizzle
 #pragma unroll
     for (int mi = 0; mi < MT; mi++) {
       const int lrow = wave * 16 * MT + 16 * mi + tcol;
-      xrow_a[mi] = xt_a + lrow * (DK * 2) + 2 * (g >> 1);
+      xrow_a[mi] = xt_a + lrow * (DK * 2);
       xsw[mi] = swz<CX>(lrow);
     }
     while (!cur.done()) {
       if (issued > step + 1) wait_vmcnt<LOADS>(); else wait_vmcnt<0>();
       lds_barrier();
       if (!nxt.done()) {
-        issue(nxt.f0(), issued % NN_NST);
+        issue(nxt.f0(), issued % NN_NST, nxt.narrow());
         nxt.next();
         issued++;
       }
-      if (cur.y != y_loaded) {
-        y_loaded = cur.y;
+      const bool narrow = cur.narrow();
+      if (cur.y != y_loaded || narrow) {
+        // (in the narrow stage every lane takes the upper eight w; the strip's values are loaded again afterwards)
+        y_loaded = narrow ? -1 : cur.y;
+        const int half = narrow ? 8 : 8 * (g & 1);
 #pragma unroll
-        for (int mi = 0; mi < MT; mi++) prow[mi].load(x_ptr(wave * 16 * MT + 16 * mi + tcol, 16 * cur.y + 8 * (g & 1)));
+        for (int mi = 0; mi < MT; mi++) prow[mi].load(x_ptr(wave * 16 * MT + 16 * mi + tcol, 16 * cur.y + half));
+      }
+      if (cur.enters_diag()) {   // quarter (0, 1) stands for (1, 0) as well
+        const float f = (g & 1) ? 2.f : 1.f;
+#pragma unroll
+        for (int mi = 0; mi < MT; mi++) prow[mi].scale(f);
       }
       uint32_t ba[NT][2], xa[MT];
       {
@@ -184,8 +222,9 @@ __global__ __launch_bounds__(256, DK <= 64 ? 3 : 2) void sympow_nn_kernel(NNArgs
         for (int nt = 0; nt < NT; nt++)
 #pragma unroll
           for (int hf = 0; hf < 2; hf++) { ba[nt][hf] = sa + boff[nt][hf]; asm volatile("" : "+v"(ba[nt][hf])); }
-        // x[row, X0 + 2*ks + parity]: X0 is a multiple of 4, so the 16-byte chunk is X0/8 and the rest is immediate
-        const int xc = cur.X0 >> 3, xo = (cur.X0 & 7) * 2;
+        // x[row, X0 + 2*ks + g/2] (narrow stage: x[row, X0 + 2*ks + (g & 1) + 4*(g >> 1)]): X0 is a multiple of 4 (8),
+        // so the 16-byte chunk is X0/8 and the rest is a lane constant plus an immediate
+        const int xc = cur.X0 >> 3, xo = (cur.X0 & 7) * 2 + ((SYM && narrow) ? xlane_n : xlane);
 #pragma unroll
         for (int mi = 0; mi < MT; mi++) { xa[mi] = xrow_a[mi] + ((xc ^ xsw[mi]) << 4) + xo; asm volatile("" : "+v"(xa[mi])); }
       }
@@ -337,7 +376,8 @@ __global__ __launch_bounds__(256, DK <= 64 ? 3 : 2) void sympow_nn_kernel(NNArgs
   }
 }
 
-template <typename T, int DK, int DV, bool MULT, int EPI> static int nn_launch(const NNArgs& a, int BN, hipStream_t st) {
+template <typename T, int DK, int DV, bool MULT, int EPI, bool SYM>
+static int nn_launch(const NNArgs& a, int BN, hipStream_t st) {
   const int rows = a.c * a.r, npairs = BN * a.h;
   auto go = [&](auto mt) {
     constexpr int MT = decltype(mt)::value;
@@ -345,7 +385,7 @@ template <typename T, int DK, int DV, bool MULT, int EPI> static int nn_launch(c
     constexpr size_t smem = ((ring > mtile ? ring : mtile) + 1023) / 1024 * 1024 + 64 * MT * DK * 2;
     const int row_blocks = (rows + 64 * MT - 1) / (64 * MT);
     dim3 grid((unsigned)(((npairs + 7) / 8) * 8 * row_blocks));
-    auto kern = sympow_nn_kernel<T, DK, DV, MT, MULT, EPI>;
+    auto kern = sympow_nn_kernel<T, DK, DV, MT, MULT, EPI, SYM>;
     allow_big_lds((const void*)kern, smem);
     hipLaunchKernelGGL(kern, grid, dim3(256), smem, st, a, row_blocks, npairs);
   };
@@ -360,8 +400,14 @@ template <typename T, int DK, int DV, bool MULT, int EPI> static int nn_launch(c
 int sympow_nn(const NNArgs& a, int BN, int d, int mult, int epi, int dtype, hipStream_t st) {
 #define PR_NN_D(T, DD)                                                                                                 \
   case DD:                                                                                                             \
-    if (epi == NN_EPI_MERGE) return nn_launch<T, DD, DD, false, NN_EPI_MERGE>(a, BN, st);                             \
-    return mult ? nn_launch<T, DD, DD, true, NN_EPI_PLAIN>(a, BN, st) : nn_launch<T, DD, DD, false, NN_EPI_PLAIN>(a, BN, st);
+    if (a.sym_diag) {                                                                                                  \
+      if (epi == NN_EPI_MERGE) return nn_launch<T, DD, DD, false, NN_EPI_MERGE, true>(a, BN, st);                     \
+      return mult ? nn_launch<T, DD, DD, true, NN_EPI_PLAIN, true>(a, BN, st)                                         \
+                  : nn_launch<T, DD, DD, false, NN_EPI_PLAIN, true>(a, BN, st);                                       \
+    }                                                                                                                  \
+    if (epi == NN_EPI_MERGE) return nn_launch<T, DD, DD, false, NN_EPI_MERGE, false>(a, BN, st);                      \
+    return mult ? nn_launch<T, DD, DD, true, NN_EPI_PLAIN, false>(a, BN, st)                                          \
+                : nn_launch<T, DD, DD, false, NN_EPI_PLAIN, false>(a, BN, st);
 #define PR_NN_T(T)                                                                                                     \
   switch (d) { PR_NN_D(T, 32) PR_NN_D(T, 64) PR_NN_D(T, 128) default: return -2; }
   if (dtype == DT_BF16) { PR_NN_T(bf16_t) }

@@ -105,7 +105,7 @@ def chunked_fwd(Q: Tensor, K: Tensor, V: Tensor, log_G: Optional[Tensor], deg: i
                                     scale, deg, 0, code, st), "attention_fwd")
     O, den = torch.empty_like(Q), _empty((BN, c, hq), f32, dev)
     _lib.check(lib.pr_query_state_fwd(p(Q), p(Sc), p(sc), p(Ya), p(la), p(rm), p(A) if gated else None, p(O), p(den),
-                                      BN, n, c, h, r, d, scale ** deg, deg, 1, code, st), "query_state_fwd")
+                                      BN, n, c, h, r, d, scale ** deg, deg, 1, 1, code, st), "query_state_fwd")
     return O, A, lcs, Kd, Sc, sc, rm, den
 
 

@@ -285,7 +285,7 @@ def query_state_fwd(Q: Tensor, S: Tensor, s: Tensor, Y_attn: Optional[Tensor], l
     lib = _lib.load()
     _lib.check(lib.pr_query_state_fwd(_lib.ptr(Q), _lib.ptr(S), _lib.ptr(s), _lib.ptr(Y_attn), _lib.ptr(l_attn),
                                       _lib.ptr(rowmax), None, _lib.ptr(O), _lib.ptr(den), b * n, n, c, h, hq // h, d,
-                                      float(scale_p), 2, int(zero_initial_state), _lib.dtype_code(Q.dtype),
+                                      float(scale_p), 2, int(zero_initial_state), 0, _lib.dtype_code(Q.dtype),
                                       _lib.stream()), "query_state_fwd")
     return O, den
 

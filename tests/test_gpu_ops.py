@@ -247,9 +247,11 @@ def test_query_state_with_a_state_that_is_not_symmetric(pra):
 
 @pytest.mark.parametrize("dtype,d,c", [(torch.bfloat16, 64, 256), (torch.float16, 32, 128), (torch.bfloat16, 128, 128)])
 def test_symmetric_state_flag_changes_nothing_for_a_symmetric_state(pra, dtype, d, c):
-    """dS_symmetric / S_symmetric let the gradient kernels take one fold instead of two through the diagonal blocks.
-    For a state made by update_state (both copies of a pair are the same sum) the results with and without the
-    promise agree to rounding, and the state produced by the forward kernel is symmetric bit for bit."""
+    """dS_symmetric / S_symmetric let the gradient kernels take one fold instead of two through the diagonal blocks
+    and the two contractions over the state (query_state forward, dV of update_state backward) skip the mirrored
+    quarter of every diagonal block.  For a state made by update_state (both copies of a pair are the same sum) the
+    results with and without the promise agree to rounding, and the state produced by the forward kernel is
+    symmetric bit for bit."""
     from retention_integration_amd import _lib, ops
     lib, st, p = _lib.load(), _lib.stream(), _lib.ptr
     b, n, h = 1, 3, 2
@@ -269,16 +271,20 @@ def test_symmetric_state_flag_changes_nothing_for_a_symmetric_state(pra, dtype, 
         dK, dV = torch.empty_like(K), torch.empty_like(V)
         _lib.check(lib.pr_update_state_bwd(p(K), p(V), p(S), p(s), p(dK), p(dV), b * n, c, h, d, 2, flag, 0, code, st),
                    "update_state_bwd")
-        O, den = ops.query_state_fwd(Q, S, s, None, None, None, 1.0 / d, False)
+        O, den = torch.empty_like(Q), torch.empty(b, n, c, h, dtype=torch.float32, device=DEV)
+        _lib.check(lib.pr_query_state_fwd(p(Q), p(S), p(s), None, None, None, None, p(O), p(den), b * n, n, c, h, 1, d,
+                                          1.0 / d, 2, 0, flag, code, st), "query_state_fwd")
         dQ, dS, ds = torch.empty_like(Q), torch.empty_like(S), torch.empty_like(s)
         ws = torch.empty(lib.pr_query_state_bwd_workspace(b * n, c, h, 1, d, code), dtype=torch.uint8, device=DEV)
         _lib.check(lib.pr_query_state_bwd(p(Q), p(S), p(s), None, None, p(O), p(den), p(dO), p(dQ), p(dS), p(ds), None, None,
                                           None, p(ws), b * n, n, c, h, 1, d, 1.0 / d, 2, 0, flag, code, st),
                    "query_state_bwd")
-        res.append((dK, dV, dQ, dS, ds))
-    for nm, a, b_ in zip(["dK", "dV", "dQ", "dS", "ds"], res[1], res[0]):
+        res.append((dK, dV, dQ, dS, ds, O, den))
+    for nm, a, b_ in zip(["dK", "dV", "dQ", "dS", "ds", "O", "den"], res[1], res[0]):
         check(f"{nm}: with the promise vs without", a, b_, 3e-3)
-    assert torch.equal(res[0][1], res[1][1]) and torch.equal(res[0][3], res[1][3])
+    assert torch.equal(res[0][3], res[1][3])
+    Oo = oracle.query_state(gold(Q.cpu()), gold(S.cpu()), gold(s.cpu()), None, None, None, 2, 1.0 / math.sqrt(d), False)
+    check("O with the promise vs the oracle", res[1][5], Oo, OUT_TOL)
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
