@@ -50,20 +50,24 @@ def build(jobs=8, verbose=True):
 
 
 def build_probe():
-    """The stand-alone issue microbenchmark (probe_issue.hip) as an executable next to the library; not part of it."""
-    out = os.path.join(os.path.dirname(HERE), "probe_issue")
-    cmd = [hipcc(), *[f for f in FLAGS if f != "-fPIC"], os.path.join(HERE, "probe_issue.hip"), "-o", out]
-    p = subprocess.run(cmd, capture_output=True, text=True)
-    if p.returncode != 0:
-        raise RuntimeError("hipcc failed for probe_issue.hip:\n" + p.stderr)
-    print("built", out)
-    return out
+    """The stand-alone probes (probe_issue.hip: the VALU / MFMA issue microbenchmark; probe_attention.hip: per-workgroup
+    phase timing of the attention kernels) as executables next to the library; not part of it."""
+    outs = []
+    for name in ("probe_issue", "probe_attention"):
+        out = os.path.join(os.path.dirname(HERE), name)
+        cmd = [hipcc(), *[f for f in FLAGS if f != "-fPIC"], os.path.join(HERE, name + ".hip"), "-o", out]
+        p = subprocess.run(cmd, capture_output=True, text=True)
+        if p.returncode != 0:
+            raise RuntimeError(f"hipcc failed for {name}.hip:\n" + p.stderr)
+        print("built", out)
+        outs.append(out)
+    return outs
 
 
 if __name__ == "__main__":
     ap = argparse.ArgumentParser()
     ap.add_argument("--jobs", type=int, default=min(8, os.cpu_count() or 1))
-    ap.add_argument("--probe", action="store_true", help="build only the stand-alone issue microbenchmark")
+    ap.add_argument("--probe", action="store_true", help="build only the stand-alone probes")
     args = ap.parse_args()
     if args.probe:
         build_probe()

@@ -83,7 +83,7 @@ int pr_chunk_attention_bwd(const void* Q, const void* K, const void* V, const fl
   if (int rc = check_common("chunk_attention_bwd", d, deg, dtype, false)) return rc;
   if (bad_ptr(Q) || bad_ptr(K) || bad_ptr(V) || bad_ptr(rowmax) || bad_ptr(dO) || bad_ptr(dQ) || bad_ptr(dK) ||
       bad_ptr(dV) || bad_ptr(dQ_state) || bad_ptr(dK_state) || bad_ptr(dV_state) || bad_opt(A) || bad_opt(dl) ||
-      bad_opt(dGq) || bad_opt(dGk) || bad_opt(dotk))
+      bad_opt(dO_scale) || bad_opt(dGq) || bad_opt(dGk) || bad_opt(dotk))
     return fail(PR_ERR_ARG, "chunk_attention_bwd: null or misaligned pointer");
   if (A && (!dGq || !dGk || !dotk))
     return fail(PR_ERR_ARG, "chunk_attention_bwd: dGq, dGk and dotk are required when A is given");

@@ -271,6 +271,13 @@ __device__ __forceinline__ float wave_sum(float x) {
   return sum_over_rows(sum_in_row(x));
 }
 
+// Hook points for a stand-alone timing probe (probe_attention.hip defines them to record wall-clock stamps per
+// workgroup); in the library they expand to nothing.
+#ifndef PR_STAMP
+#define PR_STAMP(i)
+#define PR_STAMP_VALUE(i, v)
+#endif
+
 // Kernels that use more than 64 KB of dynamic LDS must opt in once per function.
 static inline void allow_big_lds(const void* kernel, size_t bytes) {
   if (bytes > 48 * 1024) hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
