@@ -448,6 +448,7 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
   const float scale_p = __expf(a.deg * __logf(a.scale));
   const int last_key = min(key0 + KEYS, a.tk) - 1;
   const float Rblk = Gg ? Gg[(long)last_key * a.h] : 0.f;   // reference gate of the workgroup's far tiles
+  const float Glast = Gg ? Gg[(long)(a.tk - 1) * a.h] : 0.f;  // (for the epilogue; fetched here, where its latency hides)
 
   const int wslice = (u & 1) ? 3 - wave : wave;
   const int wkey0 = key0 + wslice * 16 * MK;
@@ -793,6 +794,12 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
 
   T* dKg = (T*)a.dK + (long)b * a.tk * a.h * DH + hh * DH;
   T* dVg = (T*)a.dV + (long)b * a.tk * a.h * DH + hh * DH;
+  // Indices of this lane for the epilogue, re-derived from a copy of the lane id that the compiler cannot match with
+  // the one used before the sweep: nothing that is only needed here should stay in registers (or in scratch memory,
+  // whose reload waits for every copy in flight) through it.
+  int le = threadIdx.x & 63;
+  asm volatile("" : "+v"(le));
+  const int ge = le >> 4, kce = le & 15;
   uint32_t epk = 0, epv = 0;
   if (dKsg) {
     wait_vmcnt<0>();
@@ -800,9 +807,9 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
     epk = (uint32_t)(uintptr_t)(ab_lds_char*)(smem + (nsteps % NST) * STAGE);
     epv = (uint32_t)(uintptr_t)(ab_lds_char*)(smem + ((nsteps + 1) % NST) * STAGE);
   }
-  const float Glast = Gg ? Gg[(long)(a.tk - 1) * a.h] : 0.f;
 #pragma unroll
   for (int kj = 0; kj < MK; kj++) {
+    const int key_e = wkey0 + 16 * kj + kce;
     float tot = sum_over_rows(dgk[kj]);
     float w = 1.f, dotk = 0.f;
     v4 addk[NT], addv[NT];
@@ -814,20 +821,20 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
       for (int ks = 0; ks < KS; ks++) {
         float k8[8], d8[8];
         unpack8(Kf[kj][ks], k8);
-        unpack8((v8)(*(const lds_v8*)(epk + ro + qoff_[ks])), d8);
+        unpack8((v8)(*(const lds_v8*)(epk + ro + kce * RB + (((4 * ks + ge) ^ swz<CPR>(kce)) * 16))), d8);
 #pragma unroll
         for (int i = 0; i < 8; i++) dotk = __builtin_fmaf(k8[i], d8[i], dotk);
       }
 #pragma unroll
       for (int nt = 0; nt < NT; nt++) {
-        const uint32_t co = ro + kcol * RB + (((2 * nt + (g >> 1)) ^ swz<CPR>(kcol)) * 16) + (g & 1) * 8;
+        const uint32_t co = ro + kce * RB + (((2 * nt + (ge >> 1)) ^ swz<CPR>(kce)) * 16) + (ge & 1) * 8;
         addk[nt] = *(const lds_v4*)(epk + co);
         addv[nt] = *(const lds_v4*)(epv + co);
       }
       dotk = sum_over_rows(dotk) * w;
       tot += dotk / a.deg;
     }
-    if (!live[kj]) continue;
+    if (key_e >= a.tk) continue;
 #pragma unroll
     for (int nt = 0; nt < NT; nt++) {
       float k4[4], v4f[4];
@@ -840,11 +847,11 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
           v4f[v] += (float)addv[nt][v];
         }
       }
-      *(v4*)(dKg + key[kj] * kstride + 16 * nt + 4 * g) = pack4<T>(k4);
-      *(v4*)(dVg + key[kj] * kstride + 16 * nt + 4 * g) = pack4<T>(v4f);
+      *(v4*)(dKg + key_e * kstride + 16 * nt + 4 * ge) = pack4<T>(k4);
+      *(v4*)(dVg + key_e * kstride + 16 * nt + 4 * ge) = pack4<T>(v4f);
     }
-    if (g == 0) {
-      const long go = ((long)b * a.tk + key[kj]) * a.h + hh;
+    if (ge == 0) {
+      const long go = ((long)b * a.tk + key_e) * a.h + hh;
       if (a.dGk) a.dGk[go] = -tot;
       if (a.dotk) a.dotk[go] = dotk;
     }
