@@ -44,16 +44,29 @@ static void report(const char* name, int base) {
   static int cnt[64];
   memset(sum, 0, sizeof(sum));
   memset(cnt, 0, sizeof(cnt));
-  unsigned long long t0 = ~0ull, t1 = 0;
+  unsigned long long t0 = ~0ull, t1 = 0, gend[32] = {0}, gbusy[32] = {0};
   for (int i = first_wg; i < first_wg + n_wg && i < PR_STAMP_MAX_WG; i++) {
     const unsigned long long* s = &st[(size_t)i * PR_STAMP_SLOTS + base];
     if (s[0] == 0 || s[4] == 0) continue;   // a workgroup without work
+    // workgroups go round-robin to the 8 XCDs and, inside an XCD, to its 4 shader engines: group = index % 32
+    if (s[4] > gend[i % 32]) gend[i % 32] = s[4];
+    gbusy[i % 32] += s[4] - s[0];
     const int nt = (int)s[5];
     if (nt < 0 || nt >= 64) continue;
     if (s[0] < t0) t0 = s[0];
     if (s[4] > t1) t1 = s[4];
     cnt[nt]++;
     for (int k = 0; k < 4; k++) sum[nt][k] += (double)(s[k + 1] - s[k]) * 0.01;
+  }
+  {
+    double lo = 1e30, hi = 0, sum = 0, blo = 1e30, bhi = 0;
+    for (int q = 0; q < 32; q++) {
+      const double e = (gend[q] - t0) * 0.01, bz = gbusy[q] * 0.01;
+      lo = e < lo ? e : lo; hi = e > hi ? e : hi; sum += e;
+      blo = bz < blo ? bz : blo; bhi = bz > bhi ? bz : bhi;
+    }
+    printf("%s: the 32 (XCD, shader engine) groups finish %.1f .. %.1f us after the first workgroup starts (mean %.1f); "
+           "workgroup time summed per group %.0f .. %.0f us\n", name, lo, hi, sum / 32, blo, bhi);
   }
   printf("%s: span of the launch %.1f us\n  steps  workgroups  set-up  first factors  tile loop  epilogue   total   (us, mean)\n", name,
          (t1 - t0) * 0.01);
