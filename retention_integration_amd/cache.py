@@ -62,6 +62,10 @@ class RetentionCache:
         the cache, i.e. what the reference computes from its ``gatings`` with ``cumsum(1)``."""
         t_new = key_states.shape[1]
         assert key_states.shape == (self.b, t_new, self.h, self.d) and value_states.shape == key_states.shape
+        assert key_states.dtype == self.dtype and value_states.dtype == self.dtype, \
+            f"the cache holds {self.dtype}; got {key_states.dtype} / {value_states.dtype}"
+        assert key_states.device == self.keys.device and value_states.device == self.keys.device
+        assert gate_states is None or gate_states.shape == (self.b, t_new, self.h)
         if self.length + t_new > self.capacity:
             raise ValueError(f"cache capacity {self.capacity} exceeded ({self.length} + {t_new})")
         p = _lib.ptr
@@ -99,7 +103,8 @@ class RetentionCache:
         step overwrites.  Same arithmetic as the reference caller's sequence
         ``update_kv -> power_retention_inference(whole cache, state) -> clean_kv + update_state at the switch-over``."""
         lib, p, stream = self._lib, _lib.ptr, _lib.stream()
-        assert q.shape == (self.b, 1, self.hq, self.d) and q.dtype == self.dtype
+        assert q.shape == (self.b, 1, self.hq, self.d) and q.dtype == self.dtype and q.device == self.keys.device
+        assert k.shape == (self.b, 1, self.h, self.d) and v.shape == k.shape and k.dtype == self.dtype and v.dtype == self.dtype
         if out is None:
             out = self._out
         else:

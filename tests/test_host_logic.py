@@ -50,3 +50,60 @@ def test_operators_refuse_degree_4_state():
         pra.update_state(K.view(1, 4, 16, 2, 32), V.view(1, 4, 16, 2, 32), 4)
     with pytest.raises(NotImplementedError):
         pra.query_state(Q.view(1, 4, 16, 2, 32), None, None, None, None, None, 4, 0.125, True)
+
+
+class _RecordingLibrary:
+    """Stands in for the shared library: every entry point returns success and is recorded, so the cache layer's
+    bookkeeping (ref: deploy/models/powercoder/kvgs_dynamic_cache.py:111-172) can be exercised without a GPU."""
+
+    def __init__(self):
+        self.calls = []
+
+    def __getattr__(self, name):
+        def entry(*args):
+            self.calls.append((name, args))
+            return 16 if name.endswith("_workspace") else 0
+        return entry
+
+
+@pytest.fixture
+def cpu_cache(monkeypatch):
+    from retention_integration_amd import _lib
+    lib = _RecordingLibrary()
+    monkeypatch.setattr(_lib, "load", lambda: lib)
+    monkeypatch.setattr(_lib, "stream", lambda: None)
+    cache = pra.RetentionCache(batch=2, kv_heads=2, head_dim=32, capacity=4, dtype=torch.bfloat16, device="cpu", q_heads=4)
+    return cache, lib
+
+
+def test_cache_layer_bookkeeping(cpu_cache):
+    cache, lib = cpu_cache
+    k = torch.zeros(2, 3, 2, 32, dtype=torch.bfloat16)
+    g = torch.zeros(2, 3, 2)
+    keys, values, gates, state, sk = cache.update_kv(k, k, g)
+    assert cache.get_seq_length() == 3 and keys.shape == (2, 3, 2, 32) and gates.shape == (2, 3, 2)
+    assert state is None and sk is None
+    name, args = lib.calls[-1]
+    assert name == "pr_cache_append" and args[7:14] == (2, 4, 0, 3, 2, 32, 0)   # B, capacity, pos, t_new, h, d, bf16
+    with pytest.raises(ValueError):                       # 3 + 3 tokens do not fit a capacity of 4
+        cache.update_kv(k, k, g)
+    assert cache.get_seq_length() == 3
+    with pytest.raises(AssertionError):                   # the cache holds bf16
+        cache.update_kv(k[:, :1].half(), k[:, :1].half(), g[:, :1])
+    cache.update_kv(k[:, :1], k[:, :1], None)             # ungated append at position 3
+    assert lib.calls[-1][1][9] == 3 and cache.get_seq_length() == 4
+    cache.clean_kv()
+    assert cache.get_seq_length() == 0 and not cache.has_state
+    S = torch.ones_like(cache.state)
+    cache.update_state(S, torch.ones_like(cache.sum_of_keys))
+    assert cache.has_state and torch.equal(cache.state, S)
+    assert cache.update_kv(k[:, :1], k[:, :1], g[:, :1])[3] is cache.state
+    cache.reset()
+    assert cache.get_seq_length() == 0 and not cache.has_state and float(cache.state.abs().sum()) == 0.0
+
+
+def test_cache_layer_refuses_more_than_eight_query_heads_per_kv_head(monkeypatch):
+    from retention_integration_amd import _lib
+    monkeypatch.setattr(_lib, "load", lambda: _RecordingLibrary())
+    with pytest.raises(AssertionError):
+        pra.RetentionCache(batch=1, kv_heads=1, head_dim=32, capacity=4, device="cpu", q_heads=16)
