@@ -49,8 +49,8 @@ template <typename T> __device__ __forceinline__ typename VecOf<T>::v8 ab_tr8(ui
 }
 
 // ------------------------------------------------------------------ dQ, dGq
-template <typename T, int DH, int MT, bool DEG2>
-__global__ __launch_bounds__(256, 2) void attention_bwd_dq_kernel(AttnBwdArgs a, int nblocks, int npairs) {
+template <typename T, int DH, int MT, bool DEG2, int OCC>
+__global__ __launch_bounds__(256, OCC) void attention_bwd_dq_kernel(AttnBwdArgs a, int nblocks, int npairs) {
   typedef typename VecOf<T>::v8 v8;
   typedef typename VecOf<T>::v4 v4;
   typedef __attribute__((address_space(3))) v8 lds_v8;
@@ -242,15 +242,13 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dq_kernel(AttnBwdArgs a,
     constexpr bool DIAG = decltype(diag_c)::value != 0;
     const int j0 = it * AB_BN;
     const float* graw = (const float*)(st + 2 * TILE);
-    uint32_t kb[KS], vb[KS], tb[NT], eb;
+    uint32_t kb[KS], tb[NT], eb;
     {
       const uint32_t sa = (uint32_t)(uintptr_t)(ab_lds_char*)st;
 #pragma unroll
       for (int ks = 0; ks < KS; ks++) {
         kb[ks] = sa + koff[ks];
-        vb[ks] = sa + TILE + koff[ks];
         asm volatile("" : "+v"(kb[ks]));
-        asm volatile("" : "+v"(vb[ks]));
       }
 #pragma unroll
       for (int nt = 0; nt < NT; nt++) { tb[nt] = sa + toff[nt]; asm volatile("" : "+v"(tb[nt])); }
@@ -264,65 +262,60 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dq_kernel(AttnBwdArgs a,
 #pragma unroll
     for (int kp = 0; kp < KT / 2; kp++) {
       if (DIAG && j0 + 32 * kp > w_last_ti) continue;   // these 32 keys come after every row of the wave
-      v8 kf[2][KS], vf[2][KS];
-      f32x4 ev[2];
+      v4 h4[2][MT];
 #pragma unroll
       for (int half = 0; half < 2; half++) {
+        v8 kf[KS], vf[KS];
 #pragma unroll
         for (int ks = 0; ks < KS; ks++) {
-          kf[half][ks] = *(const lds_v8*)(kb[ks] + (2 * kp + half) * 16 * RB);
-          vf[half][ks] = *(const lds_v8*)(vb[ks] + (2 * kp + half) * 16 * RB);
+          kf[ks] = *(const lds_v8*)(kb[ks] + (2 * kp + half) * 16 * RB);
+          vf[ks] = *(const lds_v8*)(kb[ks] + TILE + (2 * kp + half) * 16 * RB);
         }
-        ev[half] = *(const ab_lds_f32x4*)(eb + 64 * (2 * kp + half));
-        if (!DIAG) ev[half] *= cw;
-      }
-      f32x4 sc[2][MT], dp[2][MT];
-#pragma unroll
-      for (int half = 0; half < 2; half++)
+        f32x4 ev = *(const ab_lds_f32x4*)(eb + 64 * (2 * kp + half));
+        if (!DIAG) ev *= cw;
+        f32x4 sc[MT], dp[MT];
 #pragma unroll
         for (int mi = 0; mi < MT; mi++) {
-          sc[half][mi] = (f32x4){0, 0, 0, 0};
-          dp[half][mi] = (f32x4){0, 0, 0, 0};
+          sc[mi] = (f32x4){0, 0, 0, 0};
+          dp[mi] = (f32x4){0, 0, 0, 0};
         }
 #pragma unroll
-      for (int ks = 0; ks < KS; ks++)
-#pragma unroll
-        for (int half = 0; half < 2; half++)
+        for (int ks = 0; ks < KS; ks++)
 #pragma unroll
           for (int mi = 0; mi < MT; mi++) {
-            sc[half][mi] = mfma16(kf[half][ks], Qf[mi][ks], sc[half][mi]);
-            dp[half][mi] = mfma16(vf[half][ks], dOf[mi][ks], dp[half][mi]);
+            sc[mi] = mfma16(kf[ks], Qf[mi][ks], sc[mi]);
+            dp[mi] = mfma16(vf[ks], dOf[mi][ks], dp[mi]);
           }
-      // K^T operands for the same 32 keys, in flight while the pair gradients are formed
-      v8 kT[NT];
 #pragma unroll
-      for (int nt = 0; nt < NT; nt++) kT[nt] = ab_tr8<T>(tb[nt] + kp * 32 * RB, tb[nt] + kp * 32 * RB + 16 * RB);
-      v8 dsf[MT];
-#pragma unroll
-      for (int mi = 0; mi < MT; mi++) {
-        float d8[8];
-#pragma unroll
-        for (int half = 0; half < 2; half++) {
+        for (int mi = 0; mi < MT; mi++) {
+          float d4[4];
           float e = 1.f;
           if (DIAG) e = scale_p * __expf(fminf(base[mi] - graw[16 * (2 * kp + half)], AB_EXP_CLAMP));
 #pragma unroll
           for (int v = 0; v < 4; v++) {
-            const float s = sc[half][mi][v];
-            const float dpl = __builtin_fmaf(dp[half][mi][v], osc[mi], dlr[mi]);
-            float q = ev[half][v] * dpl;                       // E * dP without the row factor
+            const float s = sc[mi][v];
+            const float dpl = __builtin_fmaf(dp[mi][v], osc[mi], dlr[mi]);
+            float q = ev[v] * dpl;                       // E * dP without the row factor
             if (!DEG2) q *= pow_hm1<DEG2>(__builtin_fmaf(s, s, eps2), half_deg);
             if (DIAG) {
               q *= e;
               q = (32 * kp + 16 * half + v <= lim[mi]) ? q : 0.f;
             }
-            const float dsr = s * q;
             // dz = (s^2 + eps^2) q: the eps^2 part is all there is for a key with q.k = 0 (an all-zero key)
             dgq[mi] = __builtin_fmaf(__builtin_fmaf(s, s, eps2), q, dgq[mi]);
-            d8[4 * half + v] = dsr;
+            d4[v] = s * q;
           }
+          h4[half][mi] = pack4<T>(d4);
+          asm volatile("" : "+v"(h4[half][mi]));
         }
-        dsf[mi] = pack8<T>(d8);
       }
+      // K^T operands for the same 32 keys
+      v8 kT[NT];
+#pragma unroll
+      for (int nt = 0; nt < NT; nt++) kT[nt] = ab_tr8<T>(tb[nt] + kp * 32 * RB, tb[nt] + kp * 32 * RB + 16 * RB);
+      v8 dsf[MT];
+#pragma unroll
+      for (int mi = 0; mi < MT; mi++) dsf[mi] = __builtin_shufflevector(h4[0][mi], h4[1][mi], 0, 1, 2, 3, 4, 5, 6, 7);
       // dQ^T[d, row] += K^T[d, key] dsr^T[key, row]
 #pragma unroll
       for (int nt = 0; nt < NT; nt++)
@@ -355,6 +348,11 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dq_kernel(AttnBwdArgs a,
   PR_STAMP(3)
 
   T* dQg = (T*)a.dQ + (long)b * a.tq * hq * DH;
+  // Indices of this lane for the epilogue, re-derived from a copy of the lane id that the compiler cannot match with
+  // the one used before the sweep: nothing that is only needed here should stay in registers through it.
+  int le = threadIdx.x & 63;
+  asm volatile("" : "+v"(le));
+  const int ge = le >> 4, tce = le & 15;
   uint32_t ep = 0;
   if (dQsg) {
     wait_vmcnt<0>();
@@ -363,28 +361,32 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dq_kernel(AttnBwdArgs a,
   }
 #pragma unroll
   for (int mi = 0; mi < MT; mi++) {
+    const int row_e = wrow0 + 16 * mi + tce;
+    const bool live_e = row_e < rows;
+    const int rr_e = live_e ? row_e : 0, t_e = rr_e / a.r;
+    const long qoff_e = (long)t_e * hq + hh * a.r + (rr_e - t_e * a.r);
     float tot = sum_over_rows(dgq[mi]);
     float u = 1.f;
     v4 add4[NT];
     if (dQsg) {   // gradient through the gated copy of Q: dQs * u, and (Q . dQs) u / deg for the gate
       const int lr = wslice * 16 * MT + 16 * mi;
       const uint32_t rb = ep + (lr / AB_BN) * TILE + (lr % AB_BN) * RB;
-      u = (Gg && !a.dQs_plain) ? __expf(Gg[(long)ti[mi] * a.h] / a.deg) : 1.f;
+      u = (Gg && !a.dQs_plain) ? __expf(Gg[(long)(t_e + shift) * a.h] / a.deg) : 1.f;
       float dotq = 0.f;
 #pragma unroll
       for (int ks = 0; ks < KS; ks++) {
         float q8[8], d8[8];
         unpack8(Qf[mi][ks], q8);
-        unpack8((v8)(*(const lds_v8*)(rb + koff[ks])), d8);
+        unpack8((v8)(*(const lds_v8*)(rb + tce * RB + (((4 * ks + ge) ^ swz<CPR>(tce)) * 16))), d8);
 #pragma unroll
         for (int i = 0; i < 8; i++) dotq = __builtin_fmaf(q8[i], d8[i], dotq);
       }
 #pragma unroll
       for (int nt = 0; nt < NT; nt++)
-        add4[nt] = *(const lds_v4*)(rb + tcol * RB + (((2 * nt + (g >> 1)) ^ swz<CPR>(tcol)) * 16) + (g & 1) * 8);
+        add4[nt] = *(const lds_v4*)(rb + tce * RB + (((2 * nt + (ge >> 1)) ^ swz<CPR>(tce)) * 16) + (ge & 1) * 8);
       tot += sum_over_rows(dotq) * u / a.deg;
     }
-    if (!live[mi]) continue;
+    if (!live_e) continue;
 #pragma unroll
     for (int nt = 0; nt < NT; nt++) {
       float o4[4];
@@ -393,9 +395,9 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dq_kernel(AttnBwdArgs a,
         o4[v] = acc[mi][nt][v] * a.deg;
         if (dQsg) o4[v] = __builtin_fmaf((float)add4[nt][v], u, o4[v]);
       }
-      *(v4*)(dQg + qoff[mi] * DH + 16 * nt + 4 * g) = pack4<T>(o4);
+      *(v4*)(dQg + qoff_e * DH + 16 * nt + 4 * ge) = pack4<T>(o4);
     }
-    if (g == 0 && a.dGq) a.dGq[(long)b * a.tq * hq + qoff[mi]] = tot;
+    if (ge == 0 && a.dGq) a.dGq[(long)b * a.tq * hq + qoff_e] = tot;
   }
   PR_STAMP(4)
   PR_STAMP_VALUE(5, ntiles)
@@ -868,7 +870,10 @@ template <typename T, int DH, bool DEG2> static int attn_bwd_launch(const AttnBw
     const int rows = a.tq * a.r;
     const int nblocks = (rows + 64 * MT - 1) / (64 * MT);
     dim3 grid((unsigned)((npairs + 31) / 32 * 32 * nblocks));
-    auto kern = attention_bwd_dq_kernel<T, DH, MT, DEG2>;
+    // three workgroups per CU where the registers allow it without spilling (168 at d = 64 and degree 2, the
+    // stage-by-stage tile of the kernel is written for that); the ring of d = 128 leaves room for two anyway
+    constexpr int OCC = (DH <= 32 || (DH == 64 && DEG2)) ? 3 : 2;
+    auto kern = attention_bwd_dq_kernel<T, DH, MT, DEG2, OCC>;
     allow_big_lds((const void*)kern, smem);
     hipLaunchKernelGGL(kern, grid, dim3(256), smem, st, a, nblocks, npairs);
   }

@@ -109,7 +109,7 @@ template <typename T, int DH, int MAXR, int NTHR, bool WHOLE>
 __global__ __launch_bounds__(NTHR) void decode_step_kernel(DecodeArgs a) {
   typedef typename VecOf<T>::v8 v8;
   constexpr int LPR = DH / 8, FPP = NTHR / LPR;            // lanes per feature row, feature rows per pass
-  constexpr int RPW = 64 / LPR, NW = NTHR / 64;            // feature rows per wave and pass, waves
+  constexpr int NW = NTHR / 64;                            // waves (each holds 64 / LPR feature rows per pass)
   constexpr int D = 128 * (DH / 16) * (DH / 16 + 1);
   __shared__ float qs[MAXR][DH];
   __shared__ float ks[DH];
@@ -191,7 +191,7 @@ __global__ __launch_bounds__(NTHR) void decode_step_kernel(DecodeArgs a) {
     }
   }
 
-  // Sum over the feature rows: first over the RPW rows a wave holds (lanes LPR apart), then over the waves through
+  // Sum over the feature rows: first over the 64 / LPR rows a wave holds (lanes LPR apart), then over the waves through
   // LDS, one query row at a time.
   // (compile-time row index: a run-time index would put the accumulators in scratch memory for the whole kernel)
   const int wave = tid >> 6, lane = tid & 63;

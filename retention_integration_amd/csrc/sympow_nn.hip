@@ -19,7 +19,6 @@
 #include "kernels.h"
 
 namespace pr {
-#define PR_STAMP(k)
 
 constexpr int NN_FR = 64;   // feature rows per stage
 constexpr int NN_NST = 2;   // two stages keep three workgroups (12 waves) resident per CU, which hides more than a deeper ring
