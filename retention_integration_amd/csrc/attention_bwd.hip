@@ -101,7 +101,7 @@ __global__ __launch_bounds__(256, OCC) void attention_bwd_dq_kernel(AttnBwdArgs 
 #pragma unroll
   for (int ii = 0; ii < LOADS / 2; ii++) {
     const int pos = (ii * 4 + wave) * 64 + l, row = pos / CPR;
-    goff[ii] = (uint32_t)(row * (int)kstride + 16 * ((pos % CPR) ^ swz<CPR>(row)));
+    goff[ii] = (uint32_t)(row * (int)kstride + 16 * ((pos % CPR) ^ swz<CPR, SWZ_ROW>(row)));
   }
   // With the chunked epilogue the workgroup's rows of dQs ride through the ring as one more stage after the last
   // key tile (rows 0..63 in the K area, 64..127 in the V area), so that they arrive under the last tiles' work.
@@ -115,7 +115,7 @@ __global__ __launch_bounds__(256, OCC) void attention_bwd_dq_kernel(AttnBwdArgs 
         const int pos = ((ii % (LOADS / 2)) * 4 + wave) * 64 + l, row = pos / CPR;
         const int fr = min(row0 + (ii / (LOADS / 2)) * AB_BN + row, rows - 1), t = fr / a.r;
         const long eo = ((long)t * hq + hh * a.r + (fr - t * a.r)) * DH;
-        async_copy16((const char*)(dQsg + eo) + 16 * ((pos % CPR) ^ swz<CPR>(row)),
+        async_copy16((const char*)(dQsg + eo) + 16 * ((pos % CPR) ^ swz<CPR, SWZ_ROW>(row)),
                      st + (ii / (LOADS / 2)) * TILE + ((ii % (LOADS / 2)) * 4 + wave) * 1024);
       }
       if (Gg && wave == 0) async_copy4(Gg, st + 2 * TILE);   // keeps the count of copies per stage fixed
@@ -131,8 +131,8 @@ __global__ __launch_bounds__(256, OCC) void attention_bwd_dq_kernel(AttnBwdArgs 
 #pragma unroll
       for (int ii = 0; ii < LOADS / 2; ii++) async_copy16_sv(vb_, goff[ii], sa + TILE + ii * 4096);
     } else {   // last, partial tile: rows past the end repeat the last key (they are masked)
-      async_load_tile<CPR, AB_BN>(st, [&](int row) { return Kg + (long)min(j0 + row, a.tk - 1) * kstride; });
-      async_load_tile<CPR, AB_BN>(st + TILE, [&](int row) { return Vg + (long)min(j0 + row, a.tk - 1) * kstride; });
+      async_load_tile<CPR, AB_BN, SWZ_ROW>(st, [&](int row) { return Kg + (long)min(j0 + row, a.tk - 1) * kstride; });
+      async_load_tile<CPR, AB_BN, SWZ_ROW>(st + TILE, [&](int row) { return Vg + (long)min(j0 + row, a.tk - 1) * kstride; });
     }
     if (Gg && wave == 0) async_copy4(Gg + (long)min(j0 + l, a.tk - 1) * a.h, st + 2 * TILE);
   };
@@ -178,13 +178,13 @@ __global__ __launch_bounds__(256, OCC) void attention_bwd_dq_kernel(AttnBwdArgs 
   // per-lane LDS byte offsets inside a tile (the swizzle depends only on the row inside a 16-row group)
   int koff[KS], toff[NT];
 #pragma unroll
-  for (int ks = 0; ks < KS; ks++) koff[ks] = tcol * RB + (((4 * ks + g) ^ swz<CPR>(tcol)) * 16);
+  for (int ks = 0; ks < KS; ks++) koff[ks] = tcol * RB + (((4 * ks + g) ^ swz<CPR, SWZ_ROW>(tcol)) * 16);
   {
     const int vr = 4 * g + (tcol >> 2);
 #pragma unroll
     for (int nt = 0; nt < NT; nt++) {
       const int col = 16 * nt + 4 * (tcol & 3);
-      toff[nt] = vr * RB + (((col / 8) ^ swz<CPR>(vr)) * 16) + (col % 8) * 2;
+      toff[nt] = vr * RB + (((col / 8) ^ swz<CPR, SWZ_ROW>(vr)) * 16) + (col % 8) * 2;
     }
   }
 
@@ -377,13 +377,13 @@ __global__ __launch_bounds__(256, OCC) void attention_bwd_dq_kernel(AttnBwdArgs 
       for (int ks = 0; ks < KS; ks++) {
         float q8[8], d8[8];
         unpack8(Qf[mi][ks], q8);
-        unpack8((v8)(*(const lds_v8*)(rb + tce * RB + (((4 * ks + ge) ^ swz<CPR>(tce)) * 16))), d8);
+        unpack8((v8)(*(const lds_v8*)(rb + tce * RB + (((4 * ks + ge) ^ swz<CPR, SWZ_ROW>(tce)) * 16))), d8);
 #pragma unroll
         for (int i = 0; i < 8; i++) dotq = __builtin_fmaf(q8[i], d8[i], dotq);
       }
 #pragma unroll
       for (int nt = 0; nt < NT; nt++)
-        add4[nt] = *(const lds_v4*)(rb + tce * RB + (((2 * nt + (ge >> 1)) ^ swz<CPR>(tce)) * 16) + (ge & 1) * 8);
+        add4[nt] = *(const lds_v4*)(rb + tce * RB + (((2 * nt + (ge >> 1)) ^ swz<CPR, SWZ_ROW>(tce)) * 16) + (ge & 1) * 8);
       tot += sum_over_rows(dotq) * u / a.deg;
     }
     if (!live_e) continue;
@@ -474,7 +474,7 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
   auto grow = [&](int ii) __attribute__((always_inline)) -> int { return ((ii * 4 + wave) * 64 + l) / CPR; };
   auto gchk = [&](int ii) __attribute__((always_inline)) -> uint32_t {
     const int pos = (ii * 4 + wave) * 64 + l;
-    return 16 * ((pos % CPR) ^ swz<CPR>(pos / CPR));
+    return 16 * ((pos % CPR) ^ swz<CPR, SWZ_ROW>(pos / CPR));
   };
   auto row_elem = [&](int row) __attribute__((always_inline)) -> long {   // element offset of a (clamped) folded row in a [tq, hq] array
     row = min(row, rows - 1);
@@ -592,13 +592,13 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
 
   int qoff_[KS], toff[NT];
 #pragma unroll
-  for (int ks = 0; ks < KS; ks++) qoff_[ks] = kcol * RB + (((4 * ks + g) ^ swz<CPR>(kcol)) * 16);
+  for (int ks = 0; ks < KS; ks++) qoff_[ks] = kcol * RB + (((4 * ks + g) ^ swz<CPR, SWZ_ROW>(kcol)) * 16);
   {
     const int vr = 4 * g + (kcol >> 2);
 #pragma unroll
     for (int nt = 0; nt < NT; nt++) {
       const int col = 16 * nt + 4 * (kcol & 3);
-      toff[nt] = vr * RB + (((col / 8) ^ swz<CPR>(vr)) * 16) + (col % 8) * 2;
+      toff[nt] = vr * RB + (((col / 8) ^ swz<CPR, SWZ_ROW>(vr)) * 16) + (col % 8) * 2;
     }
   }
 
@@ -823,13 +823,13 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
       for (int ks = 0; ks < KS; ks++) {
         float k8[8], d8[8];
         unpack8(Kf[kj][ks], k8);
-        unpack8((v8)(*(const lds_v8*)(epk + ro + kce * RB + (((4 * ks + ge) ^ swz<CPR>(kce)) * 16))), d8);
+        unpack8((v8)(*(const lds_v8*)(epk + ro + kce * RB + (((4 * ks + ge) ^ swz<CPR, SWZ_ROW>(kce)) * 16))), d8);
 #pragma unroll
         for (int i = 0; i < 8; i++) dotk = __builtin_fmaf(k8[i], d8[i], dotk);
       }
 #pragma unroll
       for (int nt = 0; nt < NT; nt++) {
-        const uint32_t co = ro + kce * RB + (((2 * nt + (ge >> 1)) ^ swz<CPR>(kce)) * 16) + (ge & 1) * 8;
+        const uint32_t co = ro + kce * RB + (((2 * nt + (ge >> 1)) ^ swz<CPR, SWZ_ROW>(kce)) * 16) + (ge & 1) * 8;
         addk[nt] = *(const lds_v4*)(epk + co);
         addv[nt] = *(const lds_v4*)(epv + co);
       }

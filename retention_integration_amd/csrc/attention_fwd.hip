@@ -100,7 +100,7 @@ __global__ __launch_bounds__(256, OCC) void attention_fwd_kernel(AttnFwdArgs a, 
 #pragma unroll
   for (int ii = 0; ii < LOADS / 2; ii++) {
     const int pos = (ii * 4 + wave) * 64 + l, row = pos / CPR;
-    goff[ii] = (uint32_t)(row * (int)kstride + 16 * ((pos % CPR) ^ swz<CPR>(row)));
+    goff[ii] = (uint32_t)(row * (int)kstride + 16 * ((pos % CPR) ^ swz<CPR, SWZ_ROW>(row)));
   }
   auto issue = [&](int it) __attribute__((always_inline)) {
     char* st = smem + (it % NST) * STAGE;
@@ -114,8 +114,8 @@ __global__ __launch_bounds__(256, OCC) void attention_fwd_kernel(AttnFwdArgs a, 
 #pragma unroll
       for (int ii = 0; ii < LOADS / 2; ii++) async_copy16_sv(vb_, goff[ii], sa + TILE + ii * 4096);
     } else {   // last, partial tile: rows past the end repeat the last key (they are masked)
-      async_load_tile<CPR, AT_BN>(st, [&](int row) { return Kg + (long)min(j0 + row, a.tk - 1) * kstride; });
-      async_load_tile<CPR, AT_BN>(st + TILE, [&](int row) { return Vg + (long)min(j0 + row, a.tk - 1) * kstride; });
+      async_load_tile<CPR, AT_BN, SWZ_ROW>(st, [&](int row) { return Kg + (long)min(j0 + row, a.tk - 1) * kstride; });
+      async_load_tile<CPR, AT_BN, SWZ_ROW>(st + TILE, [&](int row) { return Vg + (long)min(j0 + row, a.tk - 1) * kstride; });
     }
     if (Gg && wave == 0) async_copy4(Gg + (long)min(j0 + l, a.tk - 1) * a.h, st + 2 * TILE);
   };
@@ -162,13 +162,13 @@ __global__ __launch_bounds__(256, OCC) void attention_fwd_kernel(AttnFwdArgs a, 
   // Per-lane LDS byte offsets; the swizzle depends only on the lane's row inside a 16-row group.
   int koff[KS], voff[NT];
 #pragma unroll
-  for (int ks = 0; ks < KS; ks++) koff[ks] = tcol * RB + (((4 * ks + g) ^ swz<CPR>(tcol)) * 16);
+  for (int ks = 0; ks < KS; ks++) koff[ks] = tcol * RB + (((4 * ks + g) ^ swz<CPR, SWZ_ROW>(tcol)) * 16);
   {
     const int vr = 4 * g + (tcol >> 2);   // V^T operand: row 4g + (s>>2) of a 16-key group, columns 16*nt + 4*(s&3) ..
 #pragma unroll
     for (int nt = 0; nt < NT; nt++) {
       const int col = 16 * nt + 4 * (tcol & 3);
-      voff[nt] = vr * RB + (((col / 8) ^ swz<CPR>(vr)) * 16) + (col % 8) * 2;
+      voff[nt] = vr * RB + (((col / 8) ^ swz<CPR, SWZ_ROW>(vr)) * 16) + (col % 8) * 2;
     }
   }
 

@@ -112,10 +112,18 @@ __device__ __forceinline__ typename VecOf<T>::v8 lds_frag(const T* tile, int ld,
 // instruction (global_load_lds_dwordx4) writes lane i's 16 bytes at wave_base + 16*i, so a wave
 // fills 64 consecutive chunk slots and every lane fetches the global chunk that belongs in its slot.
 // Completion is tracked by vmcnt only: the consumer waits with wait_vmcnt<N>() and then barriers.
-// swz is a bijection of the rows that share a bank phase, bit-rotated so that the four consecutive rows a
-// transposing read touches land in different pairs of chunk slots as well.
-template <int CPR> __device__ __forceinline__ int swz(int row) {
+// Which swizzle is free of bank conflicts depends on how the tile is read (measured on gfx950 with every candidate,
+// wave-wide reads of a tile with 64-, 128- and 256-byte rows):
+//  * SWZ_K8: tiles whose transposing reads take rows 8g + (s >> 2) (contraction index along the rows, eight rows per
+//    lane group: the operand tiles of sympow_tn and sympow_nn) -- a bit rotation of the row index;
+//  * SWZ_ROW: tiles read row-wise as 16-byte operand chunks (row = lane % 16, chunk 4*ks + g) and/or with transposing
+//    reads that take rows 4g + (s >> 2) (the attention tiles, the state tile of sympow_grad) -- the chunk slot advances
+//    by one every 128 bytes of rows.
+// With the other kind's swizzle these reads take 1.8-1.9 times as long.
+enum { SWZ_K8 = 0, SWZ_ROW = 1 };
+template <int CPR, int KIND = SWZ_K8> __device__ __forceinline__ int swz(int row) {
   static_assert(CPR == 4 || CPR == 8 || CPR == 16, "rows of 64, 128 or 256 bytes");
+  if (KIND == SWZ_ROW) return ((row * CPR) >> 3) & (CPR - 1);
   if (CPR == 8) {
     const int k = (row >> 1) & 7;
     return ((k & 1) << 2) | (k >> 1);
@@ -181,13 +189,13 @@ __device__ __forceinline__ void lds_barrier() {
 // Issue the copies of a tile of R rows (R*CPR a multiple of 256) by a 256-thread workgroup: every thread
 // issues exactly R*CPR/256 copies.  row_ptr(row) returns the global address of the row's first byte and
 // must be valid for every row (clamp out-of-range rows; zero them afterwards with zero_tile_rows).
-template <int CPR, int R, typename F> __device__ __forceinline__ void async_load_tile(char* tile, F row_ptr) {
+template <int CPR, int R, int KIND = SWZ_K8, typename F> __device__ __forceinline__ void async_load_tile(char* tile, F row_ptr) {
   static_assert((R * CPR) % 256 == 0, "tile must be a whole number of workgroup-wide copies");
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
 #pragma unroll
   for (int ii = 0; ii < R * CPR / 256; ii++) {
     const int inst = ii * 4 + wave;
-    const int pos = inst * 64 + lane, row = pos / CPR, c = (pos % CPR) ^ swz<CPR>(row);
+    const int pos = inst * 64 + lane, row = pos / CPR, c = (pos % CPR) ^ swz<CPR, KIND>(row);
     async_copy16(row_ptr(row) + 16 * c, tile + inst * 1024);
   }
 }

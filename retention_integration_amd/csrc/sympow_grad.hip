@@ -99,7 +99,7 @@ __global__ __launch_bounds__(256, (MT == 2 && DK <= 64) ? 4 : 2) void sympow_gra
 #pragma unroll
   for (int ii = 0; ii < LOADS; ii++) {
     const int pos = (ii * 4 + wave) * 64 + l, row = pos / CB;
-    boffs[ii] = (uint32_t)(row * (DV * 2) + 16 * ((pos % CB) ^ swz<CB>(row)));
+    boffs[ii] = (uint32_t)(row * (DV * 2) + 16 * ((pos % CB) ^ swz<CB, SWZ_ROW>(row)));
   }
   const uint32_t ring_lds = lds_addr(ring) + wave * 1024;
   auto issue = [&](int step) {
@@ -146,7 +146,7 @@ __global__ __launch_bounds__(256, (MT == 2 && DK <= 64) ? 4 : 2) void sympow_gra
   const uint32_t ring_a = (uint32_t)(uintptr_t)(lds_char*)ring, xt_a = (uint32_t)(uintptr_t)(lds_char*)xt;
   uint32_t aoff[KS];            // B rows as the A operand: row tcol of a 16-row group, chunk 4*ks + g
 #pragma unroll
-  for (int ks = 0; ks < KS; ks++) aoff[ks] = tcol * (CB * 16) + (((4 * ks + g) ^ swz<CB>(tcol)) * 16);
+  for (int ks = 0; ks < KS; ks++) aoff[ks] = tcol * (CB * 16) + (((4 * ks + g) ^ swz<CB, SWZ_ROW>(tcol)) * 16);
   uint32_t xrow_a[MT], xsw[MT];
 #pragma unroll
   for (int mi = 0; mi < MT; mi++) {
