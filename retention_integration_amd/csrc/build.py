@@ -51,9 +51,10 @@ def build(jobs=8, verbose=True):
 
 def build_probe():
     """The stand-alone probes (probe_issue.hip: the VALU / MFMA issue microbenchmark; probe_attention.hip: per-workgroup
-    phase timing of the attention kernels) as executables next to the library; not part of it."""
+    phase timing of the attention kernels; probe_lds.hip: LDS read throughput of the kernels' address patterns under
+    the candidate swizzles) as executables next to the library; not part of it."""
     outs = []
-    for name in ("probe_issue", "probe_attention"):
+    for name in ("probe_issue", "probe_attention", "probe_lds"):
         out = os.path.join(os.path.dirname(HERE), name)
         cmd = [hipcc(), *[f for f in FLAGS if f != "-fPIC"], os.path.join(HERE, name + ".hip"), "-o", out]
         p = subprocess.run(cmd, capture_output=True, text=True)
