@@ -2,9 +2,11 @@
 (b=1, t=65536, h=8, d=64, bf16, deg=2, chunk_size=1024, gated; ref: perf/benchmark.py:58-61,335-343)
 on one MI355X.  Prints ONE JSON line.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-breakdown] [--no-decode]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--settle-ms T] [--no-cpu] [--no-breakdown] [--no-decode]
 
-A step = one forward + one backward over one synthetic batch already resident in HBM.
+A step = one forward + one backward over one synthetic batch already resident in HBM.  After the W warm-up steps the
+step keeps running untimed for T ms (default 60) so that the chip's clock has settled; then K steps are timed back to
+back, and K steps each after a cache flush (their median is the headline).
 """
 import argparse
 import json
@@ -41,12 +43,19 @@ def make_inputs(b, t, h, d, device, seed=42):
     return Q, K, V, lg, dO
 
 
-def event_time_ms(fn, iters, warmup=2):
-    """Average duration of fn() on the current stream, by HIP events on that stream."""
-    for _ in range(warmup):
-        fn()
+def event_time_ms(fn, iters, settle_ms=30.0):
+    """Average duration of fn() on the current stream, by HIP events on that stream, after fn has run untimed for about
+    settle_ms (the clock governor's ramp; the lead-in calls sit in the same queue, directly ahead of the timed ones)."""
     st = torch.cuda.current_stream()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    fn()
+    e0.record(st)
+    fn()
+    e1.record(st)
+    e1.synchronize()
+    lead = int(settle_ms / max(e0.elapsed_time(e1), 1e-3)) + 1
+    for _ in range(lead):
+        fn()
     e0.record(st)
     for _ in range(iters):
         fn()
@@ -121,7 +130,7 @@ def counter_run(pra, Q, K, V, cfg, dev):
 
 
 def attention_scaling(pra, dev, chunk):
-    """For a kernel trace: the three attention kernels alone (operator level, four forward + backward calls) on the
+    """For a kernel trace: the three attention kernels alone (operator level, 64 forward + backward calls) on the
     headline's 65536 x 8 rows cut into chunks of `chunk` keys.  The tile work of a launch is proportional to the chunk
     length while everything per row and per workgroup (loading the block's own rows, storing its results, set-up) is
     not, so two chunk lengths separate the two."""
@@ -131,12 +140,13 @@ def attention_scaling(pra, dev, chunk):
     n = t // chunk
     Qf, Kf, Vf, dOf = (x.view(n, chunk, h, d) for x in (Q, K, V, dO))
     A = lg.view(n, chunk, h).cumsum(1).contiguous()
+    calls = 64   # ~35 ms of lead-in for the clock governor; a summary takes the last few launches
     with torch.no_grad():
-        for _ in range(4):
+        for _ in range(calls):
             Ya, la, rm = ops.attention_fwd(Qf, Kf, Vf, A, 2, d ** -0.5, False)
             ops.attention_bwd(Qf, Kf, Vf, A, rm, dOf, la, None, 2, d ** -0.5)
         torch.cuda.synchronize()
-    print(f"attention scaling run done: 4 x (attention_fwd, attention_bwd) at chunk {chunk}, {n} chunks x {h} heads")
+    print(f"attention scaling run done: {calls} x (attention_fwd, attention_bwd) at chunk {chunk}, {n} chunks x {h} heads")
 
 
 def decode_bench(pra, dev, steps=512):
@@ -305,6 +315,9 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--settle-ms", type=float, default=60.0,
+                    help="after the warm-up steps, keep stepping untimed for this long so that the chip's clock governor "
+                         "reaches its sustained state before anything is timed (0: time straight after the warm-up)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-oracle baseline leg")
     ap.add_argument("--no-breakdown", action="store_true", help="skip the per-operator timings")
     ap.add_argument("--no-decode", action="store_true", help="skip the inference (prefill + decode) leg")
@@ -312,7 +325,7 @@ def main():
                     help="for rocprofv3 --pmc: launch only the dominant kernel (sympow_grad, dK of update_state "
                          "backward) a few times, and a plain device copy of 256 MiB for calibrating byte counters")
     ap.add_argument("--attention-chunk", type=int, default=0,
-                    help="for rocprofv3 --kernel-trace: run only the attention kernels, four times, with the headline's "
+                    help="for rocprofv3 --kernel-trace: run only the attention kernels, 64 times, with the headline's "
                          "rows cut into chunks of this length")
     ap.add_argument("--short-chunks", action="store_true",
                     help="instead of the headline workload: BASELINE configs[4] (fp16, b=4, t=16384, h=16, d=128, "
@@ -346,12 +359,45 @@ def main():
         Y.backward(dO)
 
     from retention_integration_amd import fused
+
+    def timed_steps(k, before=None, lead=0):
+        """k steps, each bracketed by HIP events of its own; `before` is enqueued ahead of every step, outside them.
+        `lead` untimed iterations of the same sequence go first, in the same queue (the host work between two phases
+        idles the GPU long enough for its clock to drop)."""
+        ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(k)]
+        torch.cuda.synchronize()
+        for _ in range(lead):
+            if before is not None:
+                before()
+            step()
+        for e0, e1 in ev:
+            if before is not None:
+                before()
+            e0.record()
+            step()
+            e1.record()
+        torch.cuda.synchronize()
+        return [a.elapsed_time(b_) for a, b_ in ev]
+
+    def median(v):
+        v = sorted(v)
+        return v[len(v) // 2] if len(v) % 2 else 0.5 * (v[len(v) // 2 - 1] + v[len(v) // 2])
+
+    flush = torch.empty(512 * 1024 * 1024, dtype=torch.int8, device=dev)   # (allocated before anything is timed)
     for _ in range(args.warmup):
         step()
-    torch.cuda.synchronize()
+    # The chip's clock governor drops the clock within a fraction of a millisecond of idling (an allocation, a long
+    # device-side pause) and needs ~25 ms of sustained load to bring it back: straight after a few warm-up steps the
+    # first step takes 2.08 ms and the twelfth 1.80.  The figures of a training loop are the settled ones, so the steps
+    # run untimed for `settle_ms` before anything is timed; the unsettled steps are reported as well (first_steps_ms).
+    first = timed_steps(min(args.steps, 5)) if args.settle_ms > 0 else []
+    settle_steps = int(args.settle_ms / median(first)) + 1 if args.settle_ms > 0 else 0
+    for _ in range(settle_steps):
+        step()
     # (a) K steps back to back between two synchronisations.  The two kernels of the roofline blocks are timed where
     # they run: HIP events on the launch stream around each of their launches inside these steps.
     fused.KERNEL_TIMERS = {}
+    torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(args.steps):
         step()
@@ -359,23 +405,13 @@ def main():
     dt_b2b = (time.perf_counter() - t0) / args.steps
     in_step_ms = {k: sum(a.elapsed_time(b_) for a, b_ in v) / len(v) for k, v in fused.KERNEL_TIMERS.items()}
     fused.KERNEL_TIMERS = None
-    # (b) the reference's protocol (ref: perf/_timing.py:77-110): before every step the caches are flushed (a fill of
-    # 512 MB: L2 and the 256 MB memory-side cache), the step is bracketed by HIP events of its own, and the MEDIAN over
-    # the K steps is the headline figure; the fill and a short device-side pause (which lets the host run ahead, so
-    # launch latency is not measured) sit outside the events.
-    flush = torch.empty(512 * 1024 * 1024, dtype=torch.int8, device=dev)
-    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
-    torch.cuda.synchronize()
-    for e0, e1 in ev:
-        flush.zero_()
-        torch.cuda._sleep(200_000)
-        e0.record()
-        step()
-        e1.record()
-    torch.cuda.synchronize()
-    times = sorted(a.elapsed_time(b_) for a, b_ in ev)
+    # (b) the headline, by the reference's protocol (ref: perf/_timing.py:77-110): before every step the caches are
+    # flushed (a fill of 512 MB: L2 and the 256 MB memory-side cache), then a short device-side pause lets the host run
+    # ahead (launch latency is not measured), the step is bracketed by HIP events of its own, and the MEDIAN over the K
+    # steps is reported.  (The reference pauses for 25 ms; here that alone would cost 10 %, see above: 0.1 ms.)
+    times = timed_steps(args.steps, lambda: (flush.zero_(), torch.cuda._sleep(200_000)), lead=settle_steps // 2)
     del flush
-    dt = times[len(times) // 2] * 1e-3 if len(times) % 2 else 0.5e-3 * (times[len(times) // 2 - 1] + times[len(times) // 2])
+    dt = median(times) * 1e-3
 
     D_compact = cfg["d"] * (cfg["d"] + 1) // 2
     f_fwd, f_bwd = flops(cfg["b"], cfg["t"], cfg["h"], cfg["d"], cfg["chunk"], D_compact)
@@ -388,10 +424,15 @@ def main():
         "config": {"workload": "power_retention fwd+bwd b=1 t=65536 h=8 d=64 deg=2 chunk_size=1024 gating=True "
                                "(BASELINE configs[1]+[2])", "D_state": expanded_dim(cfg["d"])},
         "tflops": round(tflops, 2), "pct_bf16_mfma_peak": round(100 * tflops / PEAK_BF16_TFLOPS, 2),
-        "timing": {"protocol": "median over the K steps, each after a 512 MB cache flush, HIP events per step "
-                               "(ref: perf/_timing.py:77-110); back_to_back = wall clock of K consecutive steps / K",
-                   "flushed_ms": {"median": round(dt * 1e3, 4), "min": round(times[0], 4), "max": round(times[-1], 4)},
-                   "back_to_back_ms_per_step": round(dt_b2b * 1e3, 4)},
+        "timing": {"protocol": "W warm-up steps, then untimed steps for settle_ms (the clock governor's ramp); value = "
+                               "median over K steps, each after a 512 MB cache flush and a short device-side pause, HIP "
+                               "events per step (ref: perf/_timing.py:77-110); back_to_back = wall clock of K "
+                               "consecutive steps / K; first_steps = the steps right after the W warm-up steps, "
+                               "before settling",
+                   "flushed_ms": {"median": round(dt * 1e3, 4), "min": round(min(times), 4), "max": round(max(times), 4)},
+                   "back_to_back_ms_per_step": round(dt_b2b * 1e3, 4),
+                   "first_steps_ms": [round(x, 4) for x in first],
+                   "settle_ms": args.settle_ms, "settle_steps": settle_steps},
     }
     n = cfg["t"] // cfg["chunk"]
     bh = cfg["b"] * cfg["h"]
