@@ -422,6 +422,7 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
   constexpr int NV = 6;
   constexpr int STAGE = 2 * TILE + NV * AB_BM * 4;
   constexpr int NST = ab_stages(DH);
+  constexpr bool EARLY_T = DEG2 && DH <= 64;   // the other instances have no registers left for it
   PR_STAMP(8)
   constexpr int LOADS = 2 * AB_BM * CPR / 256;
   extern __shared__ __attribute__((aligned(1024))) char smem[];
@@ -714,6 +715,17 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
             sc[half][kj] = mfma16(qf[half][ks], Kf[kj][ks], sc[half][kj]);
             dp[half][kj] = mfma16(dof[half][ks], Vf[kj][ks], dp[half][kj]);
           }
+      // dO^T and Q^T operands of the same 32 rows.  Where the registers allow it they are requested here, so that they
+      // arrive while the pair terms are formed (they take the registers the plain operands leave); with two waves per
+      // SIMD little else covers the LDS latency (6 us of a step).
+      v8 doT[NT], qT[NT];
+      if constexpr (EARLY_T) {
+#pragma unroll
+        for (int nt = 0; nt < NT; nt++) {
+          doT[nt] = ab_tr8<T>(otb[nt] + qp * 32 * RB, otb[nt] + qp * 32 * RB + 16 * RB);
+          qT[nt] = ab_tr8<T>(qtb[nt] + qp * 32 * RB, qtb[nt] + qp * 32 * RB + 16 * RB);
+        }
+      }
       v8 pf[MK], dsf[MK];
 #pragma unroll
       for (int kj = 0; kj < MK; kj++) {
@@ -752,12 +764,14 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
       // dV^T[e, key] += dO^T[e, row] P[row, key];  dK^T[d, key] += Q^T[d, row] dsr[row, key]
 #pragma unroll
       for (int nt = 0; nt < NT; nt++) {
-        const v8 doT = ab_tr8<T>(otb[nt] + qp * 32 * RB, otb[nt] + qp * 32 * RB + 16 * RB);
-        const v8 qT = ab_tr8<T>(qtb[nt] + qp * 32 * RB, qtb[nt] + qp * 32 * RB + 16 * RB);
+        if constexpr (!EARLY_T) {
+          doT[nt] = ab_tr8<T>(otb[nt] + qp * 32 * RB, otb[nt] + qp * 32 * RB + 16 * RB);
+          qT[nt] = ab_tr8<T>(qtb[nt] + qp * 32 * RB, qtb[nt] + qp * 32 * RB + 16 * RB);
+        }
 #pragma unroll
         for (int kj = 0; kj < MK; kj++) {
-          accV[kj][nt] = mfma16(doT, pf[kj], accV[kj][nt]);
-          accK[kj][nt] = mfma16(qT, dsf[kj], accK[kj][nt]);
+          accV[kj][nt] = mfma16(doT[nt], pf[kj], accV[kj][nt]);
+          accK[kj][nt] = mfma16(qT[nt], dsf[kj], accK[kj][nt]);
         }
       }
     }
