@@ -177,13 +177,14 @@ __global__ __launch_bounds__(256, DK <= 64 ? 3 : 2) void sympow_nn_kernel(NNArgs
     typedef __attribute__((address_space(3))) char lds_char;
     typedef __attribute__((address_space(3))) unsigned short lds_u16;
     const uint32_t ring_a = (uint32_t)(uintptr_t)(lds_char*)ring, xt_a = (uint32_t)(uintptr_t)(lds_char*)xt;
-    uint32_t boff[NT][2];      // B^T operand: rows 8g + (s>>2) (+4), columns 16*nt + 4*(s&3) ..
+    uint32_t boff[NT][2];      // B^T operand (LDS address in slot 0): rows 8g + (s>>2) (+4), columns 16*nt + 4*(s&3) ..
 #pragma unroll
     for (int nt = 0; nt < NT; nt++)
 #pragma unroll
       for (int hf = 0; hf < 2; hf++) {
         const int row = 8 * g + 4 * hf + (tcol >> 2), col = 16 * nt + 4 * (tcol & 3);
-        boff[nt][hf] = row * (CB * 16) + (((col / 8) ^ swz<CB>(row)) * 16) + (col % 8) * 2;
+        boff[nt][hf] = ring_a + row * (CB * 16) + (((col / 8) ^ swz<CB>(row)) * 16) + (col % 8) * 2;
+        asm volatile("" : "+v"(boff[nt][hf]));   // one register each: the ring slot and the stage's halves are immediates
       }
     const int xlane = 2 * (g >> 1), xlane_n = 2 * ((g & 1) + 4 * (g >> 1));   // byte offsets of the lane's x column
     uint32_t xrow_a[MT], xsw[MT];   // start of this lane's row of the X tile, its swizzle
@@ -193,11 +194,16 @@ __global__ __launch_bounds__(256, DK <= 64 ? 3 : 2) void sympow_nn_kernel(NNArgs
       xrow_a[mi] = xt_a + lrow * (DK * 2);
       xsw[mi] = swz<CX>(lrow);
     }
-    while (!cur.done()) {
+    static_assert(NN_NST == 2, "the stage loop is unrolled over two ring slots");
+    // One stage, held in ring slot SL: a compile-time constant, so that every operand address of the stage is a lane
+    // register plus an immediate (with the slot a run-time value the eight address additions per stage cost 7 us of a
+    // training step at the headline shape).
+    auto stage = [&](auto sl_c) __attribute__((always_inline)) {
+      constexpr int SL = decltype(sl_c)::value;
       if (issued > step + 1) wait_vmcnt<LOADS>(); else wait_vmcnt<0>();
       lds_barrier();
       if (!nxt.done()) {
-        issue(nxt.f0(), issued % NN_NST, nxt.narrow());
+        issue(nxt.f0(), 1 - SL, nxt.narrow());
         nxt.next();
         issued++;
       }
@@ -214,13 +220,8 @@ __global__ __launch_bounds__(256, DK <= 64 ? 3 : 2) void sympow_nn_kernel(NNArgs
 #pragma unroll
         for (int mi = 0; mi < MT; mi++) prow[mi].scale(f);
       }
-      uint32_t ba[NT][2], xa[MT];
+      uint32_t xa[MT];
       {
-        const uint32_t sa = ring_a + (step % NN_NST) * STAGE;
-#pragma unroll
-        for (int nt = 0; nt < NT; nt++)
-#pragma unroll
-          for (int hf = 0; hf < 2; hf++) { ba[nt][hf] = sa + boff[nt][hf]; asm volatile("" : "+v"(ba[nt][hf])); }
         // x[row, X0 + 2*ks + g/2] (narrow stage: x[row, X0 + 2*ks + (g & 1) + 4*(g >> 1)]): X0 is a multiple of 4 (8),
         // so the 16-byte chunk is X0/8 and the rest is a lane constant plus an immediate
         const int xc = cur.X0 >> 3, xo = (cur.X0 & 7) * 2 + ((SYM && narrow) ? xlane_n : xlane);
@@ -232,8 +233,8 @@ __global__ __launch_bounds__(256, DK <= 64 ? 3 : 2) void sympow_nn_kernel(NNArgs
         v8 vf[NT];
 #pragma unroll
         for (int nt = 0; nt < NT; nt++) {
-          const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(ba[nt][0] + ks * 32 * (CB * 16)));
-          const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(ba[nt][1] + ks * 32 * (CB * 16)));
+          const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(boff[nt][0] + SL * STAGE + ks * 32 * (CB * 16)));
+          const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(boff[nt][1] + SL * STAGE + ks * 32 * (CB * 16)));
           const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
           vf[nt] = __builtin_bit_cast(v8, both);
         }
@@ -253,6 +254,11 @@ __global__ __launch_bounds__(256, DK <= 64 ? 3 : 2) void sympow_nn_kernel(NNArgs
           for (int nt = 0; nt < NT; nt++) acc[mi][nt] *= 2.f;
       }
       step++;
+    };
+    while (!cur.done()) {
+      stage(IC<0>{});
+      if (cur.done()) break;
+      stage(IC<1>{});
     }
 
     if (EPI == NN_EPI_MERGE) {
@@ -397,16 +403,17 @@ static int nn_launch(const NNArgs& a, int BN, hipStream_t st) {
 }
 
 int sympow_nn(const NNArgs& a, int BN, int d, int mult, int epi, int dtype, hipStream_t st) {
+  // two forms exist: the merge epilogue without the multiplier (query_state forward) and the plain epilogue with it
+  // (update_state's dV)
+  if ((epi == NN_EPI_MERGE) == (mult != 0)) return -1;
 #define PR_NN_D(T, DD)                                                                                                 \
   case DD:                                                                                                             \
     if (a.sym_diag) {                                                                                                  \
       if (epi == NN_EPI_MERGE) return nn_launch<T, DD, DD, false, NN_EPI_MERGE, true>(a, BN, st);                     \
-      return mult ? nn_launch<T, DD, DD, true, NN_EPI_PLAIN, true>(a, BN, st)                                         \
-                  : nn_launch<T, DD, DD, false, NN_EPI_PLAIN, true>(a, BN, st);                                       \
+      return nn_launch<T, DD, DD, true, NN_EPI_PLAIN, true>(a, BN, st);                                               \
     }                                                                                                                  \
     if (epi == NN_EPI_MERGE) return nn_launch<T, DD, DD, false, NN_EPI_MERGE, false>(a, BN, st);                      \
-    return mult ? nn_launch<T, DD, DD, true, NN_EPI_PLAIN, false>(a, BN, st)                                          \
-                : nn_launch<T, DD, DD, false, NN_EPI_PLAIN, false>(a, BN, st);
+    return nn_launch<T, DD, DD, true, NN_EPI_PLAIN, false>(a, BN, st);
 #define PR_NN_T(T)                                                                                                     \
   switch (d) { PR_NN_D(T, 32) PR_NN_D(T, 64) PR_NN_D(T, 128) default: return -2; }
   if (dtype == DT_BF16) { PR_NN_T(bf16_t) }
