@@ -11,7 +11,7 @@
 //                                                  (ref: retention/_update_state/reference.py:55-83)
 //
 // dphi is never stored.  A workgroup = 4 waves owns 64*MT rows (16*MT per wave) and sweeps B in memory order,
-// 64 feature rows (four x columns of one 16-wide strip y) per pipeline stage, through a 3-deep ring of
+// 64 feature rows (four x columns of one 16-wide strip y) per pipeline stage, through a 2-deep ring of
 // asynchronous global->LDS copies.  For an x column X the wave forms the 16x16 tile dphi^T[i, row] on the matrix
 // cores (B rows from LDS as the A operand, G^T from registers as the B operand) and folds it twice:
 //   * into dX[row, 16y+i]: multiply by the per-row scalar X[row, X] and accumulate (VALU);
@@ -28,7 +28,7 @@
 namespace pr {
 
 constexpr int GR_FR = 64;    // feature rows per stage
-constexpr int GR_NST = 3;
+constexpr int GR_NST = 2;   // ring stages; the stage loop is unrolled over them (see there)
 
 template <typename T> struct OnePair;   // two packed 1.0 values
 template <> struct OnePair<bf16_t> { static constexpr uint32_t v = 0x3F803F80u; static constexpr float down = 1.f, up = 1.f; };
@@ -107,7 +107,7 @@ __global__ __launch_bounds__(256, (MT == 2 && DK <= 64) ? 4 : 2) void sympow_gra
 #pragma unroll
     for (int ii = 0; ii < LOADS; ii++) async_copy16_sv(src, boffs[ii], ring_lds + (step % GR_NST) * STAGE + ii * 4096);
   };
-  // X rows of this workgroup (waited for together with stage 0), then the first two stages
+  // X rows of this workgroup (waited for together with stage 0), then the first stage(s)
   async_load_tile<CX, ROWS>(xt, [&](int row) { return (const char*)(Xg + row_off(row0 + row) * DK); });
   issue(0);
   if (GR_NST > 2) issue(1);
@@ -147,6 +147,9 @@ __global__ __launch_bounds__(256, (MT == 2 && DK <= 64) ? 4 : 2) void sympow_gra
   uint32_t aoff[KS];            // B rows as the A operand: row tcol of a 16-row group, chunk 4*ks + g
 #pragma unroll
   for (int ks = 0; ks < KS; ks++) aoff[ks] = tcol * (CB * 16) + (((4 * ks + g) ^ swz<CB, SWZ_ROW>(tcol)) * 16);
+  uint32_t aoffa[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ks++) { aoffa[ks] = ring_a + aoff[ks]; asm volatile("" : "+v"(aoffa[ks])); }
   uint32_t xrow_a[MT], xsw[MT];
 #pragma unroll
   for (int mi = 0; mi < MT; mi++) {
@@ -165,8 +168,12 @@ __global__ __launch_bounds__(256, (MT == 2 && DK <= 64) ? 4 : 2) void sympow_gra
     static_for<y + 1>([&](auto xc) {
       constexpr int xb = decltype(xc)::value;
       constexpr bool diag = xb == y;
-#pragma unroll 1
-      for (int sb = 0; sb < 256 / GR_FR; sb++, step++) {
+      // One stage, held in ring slot SL.  The slot is a compile-time constant (a block has an even number of stages, so
+      // its stages alternate between the two slots starting at 0): every operand address is then a lane register plus
+      // an immediate, which is worth more than a third stage in the ring (16 us of a training step at the headline
+      // shape: the address additions per stage and their pinned registers).
+      auto stage = [&](int sb, auto sl_c) __attribute__((always_inline)) {
+        constexpr int SL = decltype(sl_c)::value;
         if (GR_NST > 2 && step + 1 < NSTEP) wait_vmcnt<LOADS>(); else wait_vmcnt<0>();
         lds_barrier();
         if (step + GR_NST - 1 < NSTEP) issue(step + GR_NST - 1);
@@ -182,9 +189,8 @@ __global__ __launch_bounds__(256, (MT == 2 && DK <= 64) ? 4 : 2) void sympow_gra
         }
         uint32_t ab[KS], xa[MT];
         {
-          const uint32_t sa = ring_a + (step % GR_NST) * STAGE;
 #pragma unroll
-          for (int ks = 0; ks < KS; ks++) { ab[ks] = sa + aoff[ks]; asm volatile("" : "+v"(ab[ks])); }
+          for (int ks = 0; ks < KS; ks++) ab[ks] = aoffa[ks];
           // X[row, 16*xb + (GR_FR/16)*sb + 2*pr2 (+1)]: one 32-bit read per pair of columns
           const int X0 = 16 * xb + (GR_FR / 16) * sb, xc = X0 >> 3, xo = (X0 & 7) * 2;
 #pragma unroll
@@ -196,8 +202,8 @@ __global__ __launch_bounds__(256, (MT == 2 && DK <= 64) ? 4 : 2) void sympow_gra
           v8 af0[KS], af1[KS];
 #pragma unroll
           for (int ks = 0; ks < KS; ks++) {
-            af0[ks] = *(const lds_v8*)(ab[ks] + (32 * pr2) * (CB * 16));
-            af1[ks] = *(const lds_v8*)(ab[ks] + (32 * pr2 + 16) * (CB * 16));
+            af0[ks] = *(const lds_v8*)(ab[ks] + SL * STAGE + (32 * pr2) * (CB * 16));
+            af1[ks] = *(const lds_v8*)(ab[ks] + SL * STAGE + (32 * pr2 + 16) * (CB * 16));
           }
           // selector: accumulator row m0 sums the first 16 contraction slots (column X), row m0+1 the last 16
           const uint32_t s_lo = (tcol == m0) ? OnePair<T>::v : 0u, s_hi = (tcol == m0 + 1) ? OnePair<T>::v : 0u;
@@ -235,6 +241,13 @@ __global__ __launch_bounds__(256, (MT == 2 && DK <= 64) ? 4 : 2) void sympow_gra
             acc[mi][xb] = mfma16(sel, pack8<T>(w8), acc[mi][xb]);   // fold into dX[row, 16*xb + X]
           }
         }
+        step++;
+      };
+      static_assert(GR_NST == 2 && (256 / GR_FR) % 2 == 0, "stages of a block alternate between the two ring slots");
+#pragma unroll 1
+      for (int sb = 0; sb < 256 / GR_FR; sb += 2) {
+        stage(sb, IC<0>{});
+        stage(sb + 1, IC<1>{});
       }
     });
   });
