@@ -244,7 +244,8 @@ __global__ __launch_bounds__(256, OCC) void attention_bwd_dq_kernel(AttnBwdArgs 
     const float* graw = (const float*)(st + 2 * TILE);
     uint32_t kb[KS], tb[NT], eb;
     {
-      const uint32_t sa = (uint32_t)(uintptr_t)(ab_lds_char*)st;
+      uint32_t sa = (uint32_t)(uintptr_t)(ab_lds_char*)st;
+      asm volatile("" : "+s"(sa));   // one scalar: or the slot arithmetic is redone inside every address below
 #pragma unroll
       for (int ks = 0; ks < KS; ks++) {
         kb[ks] = sa + koff[ks];
@@ -657,7 +658,8 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
     constexpr bool FAR = decltype(far_c)::value != 0;
     uint32_t qb[KS], ob[KS], qtb[NT], otb[NT], fb;
     {
-      const uint32_t sa = (uint32_t)(uintptr_t)(ab_lds_char*)st;
+      uint32_t sa = (uint32_t)(uintptr_t)(ab_lds_char*)st;
+      asm volatile("" : "+s"(sa));   // one scalar: or the slot arithmetic is redone inside every address below
 #pragma unroll
       for (int ks = 0; ks < KS; ks++) {
         qb[ks] = sa + qoff_[ks];
