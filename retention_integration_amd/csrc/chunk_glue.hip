@@ -15,9 +15,10 @@ namespace pr {
 
 constexpr int GLUE_MAX_C = 8192;
 
-// In-place inclusive scan of a[0..c) in LDS by 256 threads (reverse = suffix sums).
+// In-place inclusive scan of a[0..c) in LDS by 256 threads (reverse = suffix sums): every thread scans its own run of
+// elements, the run totals are scanned inside each wave with lane shifts and across the four waves through tot[0..4).
 __device__ inline void block_scan(float* a, float* tot, int c, bool reverse) {
-  const int tid = threadIdx.x;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int seg = (c + 255) / 256;
   const int lo = min(tid * seg, c), hi = min(lo + seg, c);
   float run = 0.f;
@@ -26,15 +27,16 @@ __device__ inline void block_scan(float* a, float* tot, int c, bool reverse) {
     run += a[j];
     a[j] = run;
   }
-  tot[tid] = run;
-  __syncthreads();
-  for (int off = 1; off < 256; off <<= 1) {
-    const float add = tid >= off ? tot[tid - off] : 0.f;
-    __syncthreads();
-    tot[tid] += add;
-    __syncthreads();
+  float x = run;
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    const float y = __shfl_up(x, off);
+    if (lane >= off) x += y;
   }
-  const float base = tid > 0 ? tot[tid - 1] : 0.f;
+  if (lane == 63) tot[wave] = x;   // (callers that used tot before have synchronised since)
+  __syncthreads();
+  float base = x - run;
+  for (int w = 0; w < wave; w++) base += tot[w];
   for (int i = lo; i < hi; i++) a[reverse ? c - 1 - i : i] += base;
   __syncthreads();
 }
@@ -103,13 +105,13 @@ __global__ __launch_bounds__(256) void gate_scan_bwd_kernel(float* __restrict__ 
     a[i] = v;
     ks += dotk[base + (long)i * h];
   }
-  tot[tid] = ks;
+#pragma unroll
+  for (int m = 32; m > 0; m >>= 1) ks += __shfl_xor(ks, m);
+  if ((tid & 63) == 0) tot[tid >> 6] = ks;
   __syncthreads();
-  for (int off = 128; off > 0; off >>= 1) {
-    if (tid < off) tot[tid] += tot[tid + off];
-    __syncthreads();
-  }
-  if (tid == 0) a[c - 1] += tot[0] * inv_deg + dlcs_a[(long)bn * h + hh] + (dlcs_b ? dlcs_b[(long)bn * h + hh] : 0.f);
+  if (tid == 0)
+    a[c - 1] += (tot[0] + tot[1] + tot[2] + tot[3]) * inv_deg + dlcs_a[(long)bn * h + hh] +
+                (dlcs_b ? dlcs_b[(long)bn * h + hh] : 0.f);
   __syncthreads();
   block_scan(a, tot, c, true);
   for (int i = tid; i < c; i += 256) dA[base + (long)i * h] = a[i];
