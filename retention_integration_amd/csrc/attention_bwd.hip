@@ -880,6 +880,17 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
 
 template <typename T, int DH, bool DEG2> static int attn_bwd_launch(const AttnBwdArgs& a, int B, hipStream_t st) {
   const int npairs = B * a.h;
+  // dK/dV first: its epilogue reads the state-path gradients that the kernels just before this call wrote (4 us of a
+  // training step at the headline shape against the other order)
+  {
+    constexpr int MK = DH <= 64 ? 2 : 1;
+    constexpr size_t smem = ab_stages(DH) * (2 * AB_BM * DH * 2 + 6 * AB_BM * 4);
+    const int nblocks = (a.tk + 64 * MK - 1) / (64 * MK);
+    dim3 grid((unsigned)((npairs + 31) / 32 * 32 * nblocks));
+    auto kern = attention_bwd_dkv_kernel<T, DH, MK, DEG2>;
+    allow_big_lds((const void*)kern, smem);
+    hipLaunchKernelGGL(kern, grid, dim3(256), smem, st, a, nblocks, npairs);
+  }
   {
     constexpr int MT = DH <= 64 ? 2 : 1;
     constexpr size_t smem = ab_stages(DH) * (2 * AB_BN * DH * 2 + 4 * AB_BN * 4);
@@ -890,15 +901,6 @@ template <typename T, int DH, bool DEG2> static int attn_bwd_launch(const AttnBw
     // stage-by-stage tile of the kernel is written for that); the ring of d = 128 leaves room for two anyway
     constexpr int OCC = (DH <= 32 || (DH == 64 && DEG2)) ? 3 : 2;
     auto kern = attention_bwd_dq_kernel<T, DH, MT, DEG2, OCC>;
-    allow_big_lds((const void*)kern, smem);
-    hipLaunchKernelGGL(kern, grid, dim3(256), smem, st, a, nblocks, npairs);
-  }
-  {
-    constexpr int MK = DH <= 64 ? 2 : 1;
-    constexpr size_t smem = ab_stages(DH) * (2 * AB_BM * DH * 2 + 6 * AB_BM * 4);
-    const int nblocks = (a.tk + 64 * MK - 1) / (64 * MK);
-    dim3 grid((unsigned)((npairs + 31) / 32 * 32 * nblocks));
-    auto kern = attention_bwd_dkv_kernel<T, DH, MK, DEG2>;
     allow_big_lds((const void*)kern, smem);
     hipLaunchKernelGGL(kern, grid, dim3(256), smem, st, a, nblocks, npairs);
   }
