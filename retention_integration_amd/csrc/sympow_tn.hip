@@ -102,8 +102,8 @@ __device__ __forceinline__ void tn_store_diag(const f32x4 (&acc)[TN_NDIAG][DV / 
     for (int j = 0; j < DV / 32; j++) {
       const int q = j * 1024 + l * 16, i = q / (DV * 2), col = q % (DV * 2), i2 = (i - J) & 15;
       const u32x4 v = *(const lds_u32x4*)(tb + i * TP + col);
-      *(u32x4*)((char*)S + (16 * i + i2) * (DV * 2) + col) = v;
-      if (J != 0 && J != 8) *(u32x4*)((char*)S + (16 * i2 + i) * (DV * 2) + col) = v;
+      __builtin_nontemporal_store(v, (u32x4*)((char*)S + (16 * i + i2) * (DV * 2) + col));
+      if (J != 0 && J != 8) __builtin_nontemporal_store(v, (u32x4*)((char*)S + (16 * i2 + i) * (DV * 2) + col));
     }
     asm volatile("" ::: "memory");   // the buffer is rewritten for the next fragment
   });
@@ -138,9 +138,10 @@ __device__ __forceinline__ void tn_store_rows(const f32x4 (&acc)[XPW][DV / 16], 
     asm volatile("" ::: "memory");   // (LDS operations of one wave execute in order)
     char* dst = (char*)(S + 16 * X * DV);
 #pragma unroll
-    for (int j = 0; j < DV / 32; j++) {   // one kilobyte per store instruction
+    for (int j = 0; j < DV / 32; j++) {   // one kilobyte per store instruction; non-temporal: the scan that reads the
+                                          // result streams it once (3 us of a training step at the headline shape)
       const int q = j * 1024 + l * 16;
-      *(u32x4*)(dst + q) = *(const lds_u32x4*)(tb + (q / (DV * 2)) * TP + q % (DV * 2));
+      __builtin_nontemporal_store(*(const lds_u32x4*)(tb + (q / (DV * 2)) * TP + q % (DV * 2)), (u32x4*)(dst + q));
     }
     asm volatile("" ::: "memory");   // the buffer is rewritten for the next x
   });
