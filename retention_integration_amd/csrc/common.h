@@ -162,6 +162,12 @@ __device__ __forceinline__ void async_copy16_sv(const void* uniform_base, uint32
                "s"(uniform_base)
                : "memory", "m0");
 }
+// Non-temporal form, for bytes that no other workgroup reads (a state streamed once).
+__device__ __forceinline__ void async_copy16_sv_nt(const void* uniform_base, uint32_t lane_off, uint32_t lds_wave_base) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt" ::"s"(lds_wave_base), "v"(lane_off),
+               "s"(uniform_base)
+               : "memory", "m0");
+}
 __device__ __forceinline__ void async_copy4_sv(const void* uniform_base, uint32_t lane_off, uint32_t lds_wave_base) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" ::"s"(lds_wave_base), "v"(lane_off),
                "s"(uniform_base)

@@ -50,7 +50,7 @@ template <> __device__ __forceinline__ void unpack2<f16_t>(uint32_t u, float& lo
 // SYM: the caller guarantees B[(a, b)] == B[(b, a)] inside the blocks on the diagonal (true of every state and state
 // gradient this library forms: both orders of a pair are the same sum).  dphi is then symmetric there, the two folds
 // of a diagonal block are equal, and the block takes twice the first fold instead of both.
-template <typename T, int DK, int DV, int MT, bool MULT, bool SYM>
+template <typename T, int DK, int DV, int MT, bool MULT, bool SYM, bool ALONE>
 __global__ __launch_bounds__(256, (MT == 2 && DK <= 64) ? 4 : 2) void sympow_grad_kernel(GradArgs a, int row_blocks, int npairs) {
   typedef typename VecOf<T>::v8 v8;
   typedef typename VecOf<T>::v4 v4;
@@ -102,10 +102,19 @@ __global__ __launch_bounds__(256, (MT == 2 && DK <= 64) ? 4 : 2) void sympow_gra
     boffs[ii] = (uint32_t)(row * (DV * 2) + 16 * ((pos % CB) ^ swz<CB, SWZ_ROW>(row)));
   }
   const uint32_t ring_lds = lds_addr(ring) + wave * 1024;
+  // ALONE: one row block per (chunk, head), so nobody else reads this state and its copies are marked non-temporal
+  // (1.5 % of a training step at chunks of 128 rows; with several row blocks the tiles are shared through L2 and the
+  // mark costs 10 us of a step at the headline shape).  A template parameter: as a run-time flag it cost the other
+  // case 10 us through the registers and the schedule the compiler then chose.
   auto issue = [&](int step) {
     const char* src = Bg + (long)step * GR_FR * DV * 2;
+    if constexpr (ALONE) {
 #pragma unroll
-    for (int ii = 0; ii < LOADS; ii++) async_copy16_sv(src, boffs[ii], ring_lds + (step % GR_NST) * STAGE + ii * 4096);
+      for (int ii = 0; ii < LOADS; ii++) async_copy16_sv_nt(src, boffs[ii], ring_lds + (step % GR_NST) * STAGE + ii * 4096);
+    } else {
+#pragma unroll
+      for (int ii = 0; ii < LOADS; ii++) async_copy16_sv(src, boffs[ii], ring_lds + (step % GR_NST) * STAGE + ii * 4096);
+    }
   };
   // X rows of this workgroup (waited for together with stage 0), then the first stage(s)
   async_load_tile<CX, ROWS>(xt, [&](int row) { return (const char*)(Xg + row_off(row0 + row) * DK); });
@@ -330,13 +339,14 @@ __global__ __launch_bounds__(256, (MT == 2 && DK <= 64) ? 4 : 2) void sympow_gra
 template <typename T, int DK, int DV, bool MULT, bool SYM>
 static int grad_launch(const GradArgs& a, int BN, hipStream_t st) {
   const int rows = a.c * a.r, npairs = BN * a.h;
-  auto go = [&](auto mt) {
+  auto go = [&](auto mt, auto alone_c) {
     constexpr int MT = decltype(mt)::value;
+    constexpr bool ALONE = decltype(alone_c)::value != 0;
     constexpr size_t ring = GR_NST * GR_FR * DV * 2, mtile = (size_t)DK * (DK + 8) * 2;
     constexpr size_t smem = ((ring > mtile ? ring : mtile) + 1023) / 1024 * 1024 + 64 * MT * DK * 2;
     const int row_blocks = (rows + 64 * MT - 1) / (64 * MT);
     dim3 grid((unsigned)(((npairs + 7) / 8) * 8 * row_blocks));
-    auto kern = sympow_grad_kernel<T, DK, DV, MT, MULT, SYM>;
+    auto kern = sympow_grad_kernel<T, DK, DV, MT, MULT, SYM, ALONE>;
     allow_big_lds((const void*)kern, smem);
     hipLaunchKernelGGL(kern, grid, dim3(256), smem, st, a, row_blocks, npairs);
   };
@@ -344,8 +354,9 @@ static int grad_launch(const GradArgs& a, int BN, hipStream_t st) {
   // instructions of the two folds issue at twice the rate of a 256-row tiling at two workgroups (measured 7 %
   // faster at d = 64 although a state tile is reused half as often, equal at d = 32).  At d = 128 a workgroup
   // streams the whole 2.4 MB state from L2, and 128 rows instead of 64 halve that traffic (27 % faster).
-  if (rows > 64) { go(IC<2>{}); return (int)hipGetLastError(); }
-  go(IC<1>{});
+  if (rows > 128) go(IC<2>{}, IC<0>{});
+  else if (rows > 64) go(IC<2>{}, IC<1>{});
+  else go(IC<1>{}, IC<1>{});
   return (int)hipGetLastError();
 }
 

@@ -83,7 +83,7 @@ template <> struct PhiRow<f16_t> {
   __device__ __forceinline__ f16x8 make(f16_t x) const { return row * x; }
 };
 
-template <typename T, int DK, int DV, int MT, bool MULT, int EPI, bool SYM>
+template <typename T, int DK, int DV, int MT, bool MULT, int EPI, bool SYM, bool ALONE>
 __global__ __launch_bounds__(256, DK <= 64 ? 3 : 2) void sympow_nn_kernel(NNArgs a, int row_blocks, int npairs) {
   typedef typename VecOf<T>::v8 v8;
   typedef typename VecOf<T>::v4 v4;
@@ -135,13 +135,16 @@ __global__ __launch_bounds__(256, DK <= 64 ? 3 : 2) void sympow_nn_kernel(NNArgs
     }
   }
   const uint32_t ring_lds = lds_addr(ring) + wave * 1024;
+  // ALONE: one row block per (chunk, head), so nobody else reads this state and its copies are marked non-temporal
+  // (a template parameter: as a run-time flag it changed the registers and the schedule of the other case)
   auto issue = [&](int f0, int ringpos, bool narrow) {
     const char* src = Bg + (long)f0 * DV * 2;
 #pragma unroll
     for (int ii = 0; ii < LOADS; ii++) {
       uint32_t bo = boffs[ii];
       if constexpr (SYM) bo = narrow ? boffs_n[ii] : bo;
-      async_copy16_sv(src, bo, ring_lds + ringpos * STAGE + ii * 4096);
+      if constexpr (ALONE) async_copy16_sv_nt(src, bo, ring_lds + ringpos * STAGE + ii * 4096);
+      else async_copy16_sv(src, bo, ring_lds + ringpos * STAGE + ii * 4096);
     }
   };
 
@@ -384,21 +387,23 @@ __global__ __launch_bounds__(256, DK <= 64 ? 3 : 2) void sympow_nn_kernel(NNArgs
 template <typename T, int DK, int DV, bool MULT, int EPI, bool SYM>
 static int nn_launch(const NNArgs& a, int BN, hipStream_t st) {
   const int rows = a.c * a.r, npairs = BN * a.h;
-  auto go = [&](auto mt) {
+  auto go = [&](auto mt, auto alone_c) {
     constexpr int MT = decltype(mt)::value;
+    constexpr bool ALONE = decltype(alone_c)::value != 0;
     constexpr size_t ring = NN_NST * NN_FR * DV * 2, mtile = (size_t)DK * (DK + 8) * 2;
     constexpr size_t smem = ((ring > mtile ? ring : mtile) + 1023) / 1024 * 1024 + 64 * MT * DK * 2;
     const int row_blocks = (rows + 64 * MT - 1) / (64 * MT);
     dim3 grid((unsigned)(((npairs + 7) / 8) * 8 * row_blocks));
-    auto kern = sympow_nn_kernel<T, DK, DV, MT, MULT, EPI, SYM>;
+    auto kern = sympow_nn_kernel<T, DK, DV, MT, MULT, EPI, SYM, ALONE>;
     allow_big_lds((const void*)kern, smem);
     hipLaunchKernelGGL(kern, grid, dim3(256), smem, st, a, row_blocks, npairs);
   };
   if constexpr (DK <= 64) {
-    if (rows >= 256) { go(IC<4>{}); return (int)hipGetLastError(); }
+    if (rows >= 256) { go(IC<4>{}, IC<0>{}); return (int)hipGetLastError(); }
   }
-  if (rows > 64) go(IC<2>{});
-  else go(IC<1>{});
+  if (rows > 128) go(IC<2>{}, IC<0>{});
+  else if (rows > 64) go(IC<2>{}, IC<1>{});
+  else go(IC<1>{}, IC<1>{});
   return (int)hipGetLastError();
 }
 
