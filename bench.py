@@ -3,6 +3,7 @@
 on one MI355X.  Prints ONE JSON line.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--settle-ms T] [--no-cpu] [--no-breakdown] [--no-decode]
+                    [--no-short-chunks]
 
 A step = one forward + one backward over one synthetic batch already resident in HBM.  After the W warm-up steps the
 step keeps running untimed for T ms (default 60) so that the chip's clock has settled; then K steps are timed back to
@@ -237,6 +238,83 @@ def decode_bench(pra, dev, steps=512):
     return out
 
 
+class KernelTimers:
+    """Times every kernel of the library where it runs: the library's launch hook (pr_set_launch_hook) calls back right
+    before and right after each kernel launch, and a HIP event is recorded on the launch stream at both points.
+    `per_step()` gives, in launch order, the label of every kernel of a step (name#k for the k-th launch of that name in
+    the step) and its average duration in ms over the steps recorded (the first `skip` steps left out)."""
+
+    def __init__(self, _lib):
+        self._lib, self.lib = _lib, _lib.load()
+        self.records, self.steps = [], []
+        self._t0 = None
+
+        def hook(name, phase, stream, user):
+            assert stream == torch.cuda.current_stream().cuda_stream, "kernel launched on another stream than torch's"
+            ev = torch.cuda.Event(enable_timing=True)
+            ev.record()
+            if phase == 0:
+                self._t0 = ev
+            else:
+                self.records.append((name.decode(), self._t0, ev))
+        self._cb = _lib.LAUNCH_HOOK(hook)   # (kept alive for as long as it is registered)
+
+    def __enter__(self):
+        self.lib.pr_set_launch_hook(self._cb, None)
+        return self
+
+    def __exit__(self, *exc):
+        self.lib.pr_set_launch_hook(None, None)
+
+    def end_step(self):
+        self.steps.append(self.records)
+        self.records = []
+
+    def per_step(self, skip=2):
+        torch.cuda.synchronize()
+        steps = self.steps[skip:] or self.steps
+        out = {}
+        for rec in steps:
+            seen = {}
+            for name, e0, e1 in rec:
+                k = seen.get(name, 0)
+                seen[name] = k + 1
+                out.setdefault(f"{name}#{k}", []).append(e0.elapsed_time(e1))
+        return {k: sum(v) / len(v) for k, v in out.items()}
+
+
+def kernel_work(cfg, D_stored):
+    """Algorithmic work per launch of every kernel of the headline step, by kernel name: ("mfma", flops) for the
+    contractions (canonical count: compact D, causal-halved attention products, the n-1 chunks whose state is read),
+    ("hbm", bytes) for the streaming kernels (what the stored layouts make them move).  The five products of the
+    attention backward are split over its two kernels as 3 (dK/dV: its own two results and half of the two
+    recomputed products S and dP that both kernels need) and 2 (dQ)."""
+    b, t, h, d, c = cfg["b"], cfg["t"], cfg["h"], cfg["d"], cfg["chunk"]
+    n, bh = t // c, b * h
+    Dc = d * (d + 1) // 2
+    attn = bh * n * d * c * (c + 1)          # one causal-halved product over all chunks
+    state = 2.0 * bh * (n - 1) * c * Dc * d  # one state contraction
+    R = b * t * h * d * 2                    # one [b, t, h, d] 16-bit tensor
+    St = bh * n * D_stored * (d * 2 + 4)     # one state tensor with its fp32 key sums, all chunks
+    return {
+        "sympow_tn": ("mfma", state), "sympow_nn": ("mfma", state), "sympow_grad": ("mfma", state),
+        "attention_fwd": ("mfma", 2.0 * attn), "attention_bwd_dkv": ("mfma", 3.0 * attn),
+        "attention_bwd_dq": ("mfma", 2.0 * attn),
+        "discumsum_pair_fwd": ("hbm", 2.0 * St * (n - 1) / n), "discumsum_pair_bwd": ("hbm", 3.0 * St * (n - 1) / n),
+        "qs_bwd_prep": ("hbm", 3.0 * R), "gate_apply_fwd": ("hbm", 2.0 * R), "chunk_prep_fwd": ("hbm", 2.0 * R),
+    }
+
+
+def roofline_block(label, ms, work):
+    kind, amount = work
+    if kind == "mfma":
+        ach, peak, unit = amount / ms / 1e9, PEAK_BF16_TFLOPS, "TFLOP/s"
+    else:
+        ach, peak, unit = amount / ms / 1e6, PEAK_HBM_GBS, "GB/s"
+    return {"kernel": label, "bound": kind, "achieved": round(ach, 2), "peak": peak, "unit": unit,
+            "frac": round(ach / peak, 4), "ms_per_launch": round(ms, 4)}
+
+
 def measured_traffic(name):
     """HBM bytes per launch of the roofline kernel as measured with rocprofv3 byte counters: read from the line
     'total HBM traffic <x> MB' of the tracked summary profiles/<name> (which gives the commands and the calibration).
@@ -278,7 +356,9 @@ def cpu_baseline(cfg, seconds_hint=20):
 
 def short_chunks(pra, dev, steps, warmup):
     """BASELINE configs[4]: many short chunks of a wide head -- the state tensors (19.3 GB each) dominate, and the
-    chained state kernels apply."""
+    chained state kernels apply.  Returns the figures of that workload (also printed on its own by --short-chunks):
+    ms per step, tokens/s, canonical TFLOP/s, and the chained state kernel's rate over the state tensor it writes."""
+    from retention_integration_amd import _lib
     b, t, h, d, c = 4, 16384, 16, 128, 128
     g = torch.Generator().manual_seed(42)
     Q, K, V = ((0.5 * torch.randn(b, t, h, d, generator=g)).to(torch.float16).to(dev).requires_grad_(True)
@@ -298,8 +378,14 @@ def short_chunks(pra, dev, steps, warmup):
         step()
     torch.cuda.synchronize()
     dt = (time.perf_counter() - t0) / steps
+    with KernelTimers(_lib) as kt:
+        for _ in range(3):
+            step()
+            kt.end_step()
+        per = kt.per_step(skip=1)
     f_fwd, f_bwd = flops(b, t, h, d, c, d * (d + 1) // 2)
-    print(json.dumps({
+    state_bytes = b * (t // c) * h * pra.expanded_dim(d) * d * 2
+    out = {
         "metric": "fwd+bwd tokens/s at b=4,t=16384,h=16,d=128,deg=2,chunk=128 (no gating, fp16)",
         "value": round(b * t / dt, 1), "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
         "ms_per_step": round(dt * 1e3, 3), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
@@ -307,7 +393,14 @@ def short_chunks(pra, dev, steps, warmup):
         "config": {"workload": "power_retention fwd+bwd b=4 t=16384 h=16 d=128 deg=2 chunk_size=128 gating=False "
                                "(BASELINE configs[4])"},
         "tflops": round((f_fwd + f_bwd) / dt / 1e12, 2),
-        "state_bytes_per_tensor": b * (t // c) * h * 128 * (d // 16) * (d // 16 + 1) * d * 2}))
+        "state_bytes_per_tensor": state_bytes,
+        "kernels_us": {k: round(v * 1e3, 1) for k, v in per.items()}}
+    chain = [v for k, v in per.items() if k.startswith("sympow_tn_chain#")]
+    if chain:
+        out["sympow_tn_chain_hbm"] = [
+            {"ms_per_launch": round(v, 3), "achieved": round(state_bytes / v / 1e6, 1), "peak": PEAK_HBM_GBS,
+             "unit": "GB/s", "frac": round(state_bytes / v / 1e6 / PEAK_HBM_GBS, 4)} for v in chain]
+    return out
 
 
 def main():
@@ -321,9 +414,10 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-oracle baseline leg")
     ap.add_argument("--no-breakdown", action="store_true", help="skip the per-operator timings")
     ap.add_argument("--no-decode", action="store_true", help="skip the inference (prefill + decode) leg")
+    ap.add_argument("--no-short-chunks", action="store_true", help="skip the BASELINE configs[4] leg (short_chunks key)")
     ap.add_argument("--counter-run", action="store_true",
-                    help="for rocprofv3 --pmc: launch only the dominant kernel (sympow_grad, dK of update_state "
-                         "backward) a few times, and a plain device copy of 256 MiB for calibrating byte counters")
+                    help="for rocprofv3 --pmc: launch only sympow_grad (dK of update_state backward) a few times, and a "
+                         "plain device copy of 256 MiB for calibrating byte counters")
     ap.add_argument("--attention-chunk", type=int, default=0,
                     help="for rocprofv3 --kernel-trace: run only the attention kernels, 64 times, with the headline's "
                          "rows cut into chunks of this length")
@@ -340,7 +434,7 @@ def main():
 
     dev = torch.device("cuda:0")
     if args.short_chunks:
-        short_chunks(pra, dev, args.steps, args.warmup)
+        print(json.dumps(short_chunks(pra, dev, args.steps, args.warmup)))
         return
     if args.attention_chunk:
         attention_scaling(pra, dev, args.attention_chunk)
@@ -358,7 +452,7 @@ def main():
         Y = pra.power_retention(*leaves, deg=cfg["deg"], chunk_size=cfg["chunk"])
         Y.backward(dO)
 
-    from retention_integration_amd import fused
+    from retention_integration_amd import _lib
 
     def timed_steps(k, before=None, lead=0):
         """k steps, each bracketed by HIP events of its own; `before` is enqueued ahead of every step, outside them.
@@ -394,17 +488,20 @@ def main():
     settle_steps = int(args.settle_ms / median(first)) + 1 if args.settle_ms > 0 else 0
     for _ in range(settle_steps):
         step()
-    # (a) K steps back to back between two synchronisations.  The two kernels of the roofline blocks are timed where
-    # they run: HIP events on the launch stream around each of their launches inside these steps.
-    fused.KERNEL_TIMERS = {}
+    # (a) K steps back to back between two synchronisations
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(args.steps):
         step()
     torch.cuda.synchronize()
     dt_b2b = (time.perf_counter() - t0) / args.steps
-    in_step_ms = {k: sum(a.elapsed_time(b_) for a, b_ in v) / len(v) for k, v in fused.KERNEL_TIMERS.items()}
-    fused.KERNEL_TIMERS = None
+    # (a') the same steps once more with EVERY kernel timed where it runs: HIP events on the launch stream around each
+    # launch (the library's launch hook); the events make these steps a little longer, so they are not the ones above
+    with KernelTimers(_lib) as kt:
+        for _ in range(args.steps + 2):
+            step()
+            kt.end_step()
+        in_step_ms = kt.per_step(skip=2)
     # (b) the headline, by the reference's protocol (ref: perf/_timing.py:77-110): before every step the caches are
     # flushed (a fill of 512 MB: L2 and the 256 MB memory-side cache), then a short device-side pause lets the host run
     # ahead (launch latency is not measured), the step is bracketed by HIP events of its own, and the MEDIAN over the K
@@ -436,25 +533,29 @@ def main():
     }
     n = cfg["t"] // cfg["chunk"]
     bh = cfg["b"] * cfg["h"]
-    # dominant single kernel (two launches per step, the largest share of the step): the feature-gradient contraction
-    # sympow_grad, here its dK launch of update_state backward.  Algorithmic flops per launch = the d(phi) product
-    # 2*c*D*d per (chunk, head) with the compact D over the n-1 chunks whose state is read (the same convention as
-    # flops() above).  Duration: HIP events around that launch inside the back-to-back steps, which is what the kernel
-    # trace of the same command shows.
-    k_flops = 2.0 * bh * (n - 1) * cfg["chunk"] * D_compact * cfg["d"]
-    k_ms = in_step_ms["sympow_grad(dK)"]
-    traffic, traffic_src = measured_traffic("sympow_grad_t65536_hbm_traffic.txt")
-    esz = 2
-    algo_bytes = bh * (n - 1) * (3 * cfg["chunk"] * cfg["d"] * esz + expanded_dim(cfg["d"]) * (cfg["d"] * esz + 4))
-    out["roofline"] = {"kernel": "sympow_grad_kernel (dK of update_state backward)", "bound": "mfma",
-                       "achieved": round(k_flops / k_ms / 1e9, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                       "frac": round(k_flops / k_ms / 1e9 / PEAK_BF16_TFLOPS, 4), "ms_per_launch": round(k_ms, 4),
-                       "traffic": traffic, "traffic_source": traffic_src, "algorithmic_bytes": algo_bytes}
-    t_ms = in_step_ms["sympow_tn(update_state)"]
-    out["roofline_update_state_fwd"] = {"kernel": "sympow_tn_kernel", "bound": "mfma",
-                                        "achieved": round(k_flops / t_ms / 1e9, 2), "peak": PEAK_BF16_TFLOPS,
-                                        "unit": "TFLOP/s", "frac": round(k_flops / t_ms / 1e9 / PEAK_BF16_TFLOPS, 4),
-                                        "ms_per_launch": round(t_ms, 4)}
+    # Roofline blocks.  `roofline` is the LONGEST single kernel of the step as just measured; its work per launch is the
+    # algorithmic count of kernel_work().  HBM traffic of a launch comes from the tracked rocprofv3 counter summary of
+    # that kernel when profiles/ holds one (parsed at run time, never typed in here).
+    work = kernel_work(cfg, expanded_dim(cfg["d"]))
+    out["kernels_us"] = {k: round(v * 1e3, 1) for k, v in in_step_ms.items()}
+    out["kernels_us_sum"] = round(sum(in_step_ms.values()) * 1e3, 1)
+    longest = max(in_step_ms, key=in_step_ms.get)
+    base = longest.split("#")[0]
+    blk = roofline_block(longest, in_step_ms[longest], work.get(base, ("hbm", 0.0)))
+    traffic, traffic_src = measured_traffic(base + "_t65536_hbm_traffic.txt")
+    blk["traffic"], blk["traffic_source"] = traffic, traffic_src
+    out["roofline"] = blk
+    ab = [k for k in in_step_ms if k.startswith("attention_bwd_")]
+    if ab:
+        ms = sum(in_step_ms[k] for k in ab)
+        out["roofline_attention_bwd"] = roofline_block(" + ".join(ab), ms, ("mfma", 5.0 * bh * n * cfg["d"] * cfg["chunk"] * (cfg["chunk"] + 1)))
+    for key, label in (("roofline_attention_fwd", "attention_fwd#0"), ("roofline_update_state_fwd", "sympow_tn#0"),
+                       ("roofline_query_state_fwd", "sympow_nn#0"), ("roofline_update_state_bwd_dK", "sympow_grad#1"),
+                       ("roofline_state_scan_fwd", "discumsum_pair_fwd#0"), ("roofline_state_scan_bwd", "discumsum_pair_bwd#0")):
+        if label in in_step_ms:
+            out[key] = roofline_block(label, in_step_ms[label], work[label.split("#")[0]])
+    mf = sum(v for k, v in in_step_ms.items() if work.get(k.split("#")[0], ("hbm",))[0] == "mfma")
+    out["kernel_time_split_us"] = {"mfma_bound": round(mf * 1e3, 1), "hbm_bound": round((sum(in_step_ms.values()) - mf) * 1e3, 1)}
     detach = [x.detach() for x in (Q, K, V, lg)]
     if not args.no_breakdown:
         with torch.no_grad():
@@ -466,6 +567,11 @@ def main():
     if not args.no_decode:
         with torch.no_grad():
             out["decode"] = decode_bench(pra, dev)
+    if not args.no_short_chunks:
+        torch.cuda.empty_cache()
+        sc = short_chunks(pra, dev, 5, 2)
+        out["short_chunks"] = {k: sc[k] for k in ("config", "dtype", "ms_per_step", "value", "unit", "tflops",
+                                                  "state_bytes_per_tensor", "kernels_us", "sympow_tn_chain_hbm") if k in sc}
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(cfg)
     print(json.dumps(out))

@@ -39,9 +39,19 @@ enum {
 /* 2: pr_update_state_bwd and pr_query_state_bwd take the symmetric-state promise (dS_symmetric, S_symmetric).
  * 3: pr_decode_step_noalloc.  4: pr_cache_append, pr_cache_attention_fwd; pr_update_state_fwd takes skip_last_of and
  * pr_update_state_bwd zero_last_of; pr_query_state_fwd / _bwd / _scan_bwd take q_log_gate and
- * pr_chunk_attention_bwd dQ_state_plain.  5: pr_query_state_fwd takes S_symmetric. */
+ * pr_chunk_attention_bwd dQ_state_plain.  5: pr_query_state_fwd takes S_symmetric.  6: pr_set_launch_hook;
+ * pr_decode_step takes up to 16 query rows per (batch, kv head). */
 int pr_abi_version(void);
 const char* pr_last_error(void);
+
+/* Per-kernel hook for benchmarks and profilers (no counterpart in the reference, whose harness times whole operators:
+ * perf/_timing.py:77-110).  Once set, the hook is called on the launching host thread right before (phase 0) and right
+ * after (phase 1) EVERY kernel launch of the library, with the kernel's short name (a static string such as
+ * "sympow_grad" or "attention_bwd_dkv") and the stream it is launched on -- record a pair of events there to time a
+ * kernel where it runs, inside a step.  NULL removes it.  Process-wide; set it while no other thread is inside the
+ * library.  The hook must not call back into the library. */
+typedef void (*pr_launch_hook_t)(const char* kernel, int phase, void* stream, void* user);
+void pr_set_launch_hook(pr_launch_hook_t hook, void* user);
 
 /* Size D of the expanded state for head dim d: 256 * T(T+1)/2, T = d/16; -1 if d is not a multiple of 16.
  * Replaces retention/_utils.py:18-19 compute_expanded_dim. */
@@ -212,7 +222,7 @@ int pr_chunk_gate_scan_bwd(float* dlog_G, const float* dGq, const float* dotk, c
 /* Single-token inference step on the state -- query: retention/power_retention_maker.py:358-363 with
  * retention/_query_state/reference.py:36-96 (one query position per sequence); update:
  * retention/power_retention_maker.py:366-382 with retention/_update_state/reference.py:33-52 for ONE new token.
- *   Q [B,tq,h*r,d] with tq*r <= 8, gq [B,h] fp32 or NULL: accumulated log gate at the query position
+ *   Q [B,tq,h*r,d] with tq*r <= 16, gq [B,h] fp32 or NULL: accumulated log gate at the query position
  *   (Q is used as Q * exp(gq/deg), rounded to dtype), S [B,h,D,d], s [B,h,D] fp32,
  *   Y_attn [B,tq,h*r,d], l_attn, rowmax [B,tq,h*r] fp32 or all NULL (attention over the not yet folded cache)
  *   -> out [B,tq,h*r,d] = the merged, normalised output.
@@ -252,6 +262,10 @@ int pr_cache_attention_fwd(const void* Q, const void* K_cache, const void* V_cac
  * holds on every GPU it runs on until the process ends; the call allocates and frees nothing.  A step whose
  * pr_decode_step_workspace() exceeds that size is refused with PR_ERR_ARG (use pr_decode_step).  All calls on one
  * GPU share the array: calls that overlap in time on one GPU (two streams) race; calls on one stream do not.
+ * The array is that of the GPU the stream belongs to, which must be the current device (PR_ERR_ARG otherwise).
+ * Set-up: the array's address is looked up once per GPU (hipGetSymbolAddress, not stream work).
+ * pr_decode_step_noalloc_max_workspace() does that for the current device, so call it once per GPU before a first
+ * pr_decode_step_noalloc that is issued under stream capture; outside capture the first step does it by itself.
  * Same arguments, results and in-place rules as pr_decode_step. */
 size_t pr_decode_step_noalloc_max_workspace(void);
 int pr_decode_step_noalloc(const void* Q, const float* gq, const void* S, const float* s, const void* Y_attn,

@@ -51,7 +51,11 @@ SIGNATURES = {
     "pr_cache_attention_fwd": (c_int, [_P] * 7 + [_I] * 7 + [_F, _I, _I, _I, _P]),
     "pr_decode_step_noalloc_max_workspace": (c_size_t, []),
     "pr_decode_step_noalloc": (c_int, [_P] * 13 + [_I] * 5 + [_F, _I, _I, _I, _P]),
+    "pr_set_launch_hook": (None, [_P, _P]),
 }
+
+# signature of the per-kernel hook: (kernel name, phase 0 / 1, stream, user pointer)
+LAUNCH_HOOK = ctypes.CFUNCTYPE(None, c_char_p, c_int, c_void_p, c_void_p)
 
 _lib = None
 

@@ -29,7 +29,10 @@ class RetentionCache:
         assert dtype in (torch.bfloat16, torch.float16) and head_dim in (32, 64, 128)
         self.b, self.h, self.d, self.capacity = batch, kv_heads, head_dim, capacity
         self.hq = q_heads or kv_heads
-        assert self.hq % kv_heads == 0 and self.hq // kv_heads <= 8, "at most 8 query heads per kv head in a decode step"
+        assert self.hq % kv_heads == 0, "query heads must be a multiple of kv heads"
+        # the single-pass decode kernel takes up to 16 query rows per kv head; wider groups run the state query as the
+        # query_state operator over the same preallocated buffers (a few more launches per token, same results)
+        self._fused_step = self.hq // kv_heads <= 16
         self.dtype, self.device = dtype, torch.device(device)
         D = expanded_dim(head_dim)
         f32 = torch.float32
@@ -48,7 +51,7 @@ class RetentionCache:
         self._gq = torch.empty(batch, kv_heads, dtype=f32, device=device)   # accumulated gate at the newest position
         self._lib = _lib.load()
         self._code = _lib.dtype_code(dtype)
-        ws = self._lib.pr_decode_step_workspace(batch, 1, kv_heads, self.hq // kv_heads, head_dim)
+        ws = self._lib.pr_decode_step_workspace(batch, 1, kv_heads, self.hq // kv_heads, head_dim) if self._fused_step else 0
         self._ws = torch.empty(max(ws, 16), dtype=torch.uint8, device=device)
 
     # ---- the reference layer's interface ---------------------------------------------------------------------
@@ -112,7 +115,7 @@ class RetentionCache:
         scale = float(scale) if scale else 1.0 / self.d ** 0.5
         r = self.hq // self.h
         fold = switch_over_seq_len is not None and self.length + 1 >= switch_over_seq_len
-        if self.has_state and fold and self.length == 0:
+        if self.has_state and fold and self.length == 0 and self._fused_step:
             # one-token cache folded at once (switch_over_seq_len = 1): the recurrent step, one pass over the state
             g = None if log_g is None else log_g.to(torch.float32).reshape(self.b, self.h).contiguous()
             _lib.check(lib.pr_decode_step(p(q.contiguous()), p(g), p(self.state), p(self.sum_of_keys), None, None, None,
@@ -132,6 +135,18 @@ class RetentionCache:
             _lib.check(lib.pr_cache_attention_fwd(p(q.contiguous()), p(self.keys), p(self.values), p(self.gatings),
                                                   p(self._ya), p(self._la), p(self._rm), self.b, 1, n, self.capacity,
                                                   self.h, r, self.d, scale, 2, 0, self._code, stream), "cache_attention_fwd")
+            if not self._fused_step:
+                # more query rows per kv head than the single-pass kernel holds: the state query as the operator
+                # (ref: retention/power_retention_maker.py:358-363), gated by the accumulated gate at the newest position
+                from . import ops
+                qg = q
+                if log_g is not None:
+                    qg = (q * torch.exp(self._gq / 2).repeat_interleave(r, dim=-1)[:, None, :, None]).to(self.dtype)
+                out.copy_(ops.query_state(qg.contiguous(), self.state, self.sum_of_keys, self._ya, self._la, self._rm, 2,
+                                          scale, False))
+                if fold:
+                    self._fold()
+                return out
             # (the query is gated by the accumulated gate at the newest cache position, which the append left in _gq)
             _lib.check(lib.pr_decode_step(p(q.contiguous()), p(self._gq), p(self.state), p(self.sum_of_keys), p(self._ya),
                                           p(self._la), p(self._rm), None, None, None, None, None, p(out),

@@ -58,7 +58,6 @@ __global__ __launch_bounds__(256, OCC) void attention_bwd_dq_kernel(AttnBwdArgs 
   constexpr int KS = DH / 32, NT = DH / 16, KT = AB_BN / 16, ROWS = 64 * MT, CPR = DH / 8, RB = CPR * 16;
   constexpr int TILE = AB_BN * RB;
   constexpr int STAGE = 2 * TILE + 4 * AB_BN * 4;   // K, V, raw gates, two sets of key gate factors
-  PR_STAMP(0)
   constexpr int NST = ab_stages(DH);
   constexpr int LOADS = 2 * AB_BN * CPR / 256;
   extern __shared__ __attribute__((aligned(1024))) char smem[];
@@ -202,12 +201,10 @@ __global__ __launch_bounds__(256, OCC) void attention_bwd_dq_kernel(AttnBwdArgs 
     graw[2 * AB_BN + l] = __expf(fminf(Rs - gv, AB_EXP_CLAMP));
     if (!Gg) graw[l] = 0.f;
   };
-  PR_STAMP(1)
   if (wave == 0) {
     wait_vmcnt<0>();
     gate_factors(0);
   }
-  PR_STAMP(2)
   auto sync_step = [&](int it) __attribute__((always_inline)) -> char* {
     char* st = smem + (it % NST) * STAGE;
     if constexpr (NST == 3) {
@@ -346,7 +343,6 @@ __global__ __launch_bounds__(256, OCC) void attention_bwd_dq_kernel(AttnBwdArgs 
     sync_step(it);
     after_step(it);
   }
-  PR_STAMP(3)
 
   T* dQg = (T*)a.dQ + (long)b * a.tq * hq * DH;
   // Indices of this lane for the epilogue, re-derived from a copy of the lane id that the compiler cannot match with
@@ -400,8 +396,6 @@ __global__ __launch_bounds__(256, OCC) void attention_bwd_dq_kernel(AttnBwdArgs 
     }
     if (ge == 0 && a.dGq) a.dGq[(long)b * a.tq * hq + qoff_e] = tot;
   }
-  PR_STAMP(4)
-  PR_STAMP_VALUE(5, ntiles)
 }
 
 // ------------------------------------------------------------------ dK, dV, dGk
@@ -424,7 +418,6 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
   constexpr int STAGE = 2 * TILE + NV * AB_BM * 4;
   constexpr int NST = ab_stages(DH);
   constexpr bool EARLY_T = DEG2 && DH <= 64;   // the other instances have no registers left for it
-  PR_STAMP(8)
   constexpr int LOADS = 2 * AB_BM * CPR / 256;
   extern __shared__ __attribute__((aligned(1024))) char smem[];
 
@@ -621,12 +614,10 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
     rv[4 * AB_BM + l] = eu * os_;
     rv[5 * AB_BM + l] = eu * dl_;
   };
-  PR_STAMP(9)
   if (wave == 0 && nsteps > 0) {
     wait_vmcnt<0>();
     row_factors(0);
   }
-  PR_STAMP(10)
   auto sync_step = [&](int step) __attribute__((always_inline)) -> char* {
     char* st = smem + (step % NST) * STAGE;
     if constexpr (NST == 3) {
@@ -804,7 +795,6 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
     sync_step(step);
     after_step(step);
   }
-  PR_STAMP(11)
   if (NST == 2 && nsteps + 1 < ntot) {   // the second of the two epilogue stages has no step that would copy it
     lds_barrier();
     issue(nsteps + 1);
@@ -874,8 +864,6 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
       if (a.dotk) a.dotk[go] = dotk;
     }
   }
-  PR_STAMP(12)
-  PR_STAMP_VALUE(13, nsteps)
 }
 
 template <typename T, int DH, bool DEG2> static int attn_bwd_launch(const AttnBwdArgs& a, int B, hipStream_t st) {
@@ -889,7 +877,7 @@ template <typename T, int DH, bool DEG2> static int attn_bwd_launch(const AttnBw
     dim3 grid((unsigned)((npairs + 31) / 32 * 32 * nblocks));
     auto kern = attention_bwd_dkv_kernel<T, DH, MK, DEG2>;
     allow_big_lds((const void*)kern, smem);
-    hipLaunchKernelGGL(kern, grid, dim3(256), smem, st, a, nblocks, npairs);
+    PR_LAUNCH("attention_bwd_dkv", kern, grid, dim3(256), smem, st, a, nblocks, npairs);
   }
   {
     constexpr int MT = DH <= 64 ? 2 : 1;
@@ -902,7 +890,7 @@ template <typename T, int DH, bool DEG2> static int attn_bwd_launch(const AttnBw
     constexpr int OCC = (DH <= 32 || (DH == 64 && DEG2)) ? 3 : 2;
     auto kern = attention_bwd_dq_kernel<T, DH, MT, DEG2, OCC>;
     allow_big_lds((const void*)kern, smem);
-    hipLaunchKernelGGL(kern, grid, dim3(256), smem, st, a, nblocks, npairs);
+    PR_LAUNCH("attention_bwd_dq", kern, grid, dim3(256), smem, st, a, nblocks, npairs);
   }
   return (int)hipGetLastError();
 }

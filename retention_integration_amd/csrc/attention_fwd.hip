@@ -57,7 +57,6 @@ __global__ __launch_bounds__(256, OCC) void attention_fwd_kernel(AttnFwdArgs a, 
   constexpr int NST = at_stages(DH);
   extern __shared__ __attribute__((aligned(1024))) char smem[];
 
-  PR_STAMP(0)
   const int tid = threadIdx.x, l = tid & 63, g = l >> 4, tcol = l & 15;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform, so branches on it are scalar
   // Workgroups are dealt round-robin by their linear index: to the 8 XCDs first, then inside an XCD to its 4
@@ -190,12 +189,10 @@ __global__ __launch_bounds__(256, OCC) void attention_fwd_kernel(AttnFwdArgs a, 
     graw[2 * AT_BN + l] = __expf(fminf(Rs - gv, AT_EXP_CLAMP));
     if (!Gg) graw[l] = 0.f;
   };
-  PR_STAMP(1)
   if (wave == 0) {
     wait_vmcnt<0>();
     gate_factors(0);
   }
-  PR_STAMP(2)
   // Make tile `it` visible to the workgroup, start the copy of tile it+2, and (wave 0) prepare the gate factors of
   // tile it+1 while the others already compute.
   auto sync_step = [&](int it) __attribute__((always_inline)) -> char* {
@@ -378,7 +375,6 @@ __global__ __launch_bounds__(256, OCC) void attention_fwd_kernel(AttnFwdArgs a, 
   } else {
     run_pass(IC<0>{});
   }
-  PR_STAMP(3)
 
   T* Og = (T*)a.O + (long)b * a.tq * hq * DH;
 #pragma unroll
@@ -402,8 +398,6 @@ __global__ __launch_bounds__(256, OCC) void attention_fwd_kernel(AttnFwdArgs a, 
       if (a.rowmax) a.rowmax[o] = __logf(wmax);
     }
   }
-  PR_STAMP(4)
-  PR_STAMP_VALUE(5, ntiles)
 }
 
 template <typename T, int DH, bool DEG2> static int attn_fwd_launch(const AttnFwdArgs& a, int B, hipStream_t st) {
@@ -415,7 +409,7 @@ template <typename T, int DH, bool DEG2> static int attn_fwd_launch(const AttnFw
     dim3 grid((unsigned)(((npairs + 31) / 32) * 32 * row_blocks));
     auto kern = attention_fwd_kernel<T, DH, MT, DEG2, OCC>;
     allow_big_lds((const void*)kern, smem);
-    hipLaunchKernelGGL(kern, grid, dim3(256), smem, st, a, row_blocks, npairs);
+    PR_LAUNCH("attention_fwd", kern, grid, dim3(256), smem, st, a, row_blocks, npairs);
   };
   // 128 rows per workgroup: 123 registers at d = 32 (four workgroups per CU), 166 at d = 64 (three); measured 9 % and
   // 6 % faster than 256 rows at two workgroups -- the kernel is mostly vector work, which issues faster with more

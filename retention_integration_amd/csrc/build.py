@@ -36,6 +36,15 @@ def hipcc():
     raise RuntimeError("hipcc not found")
 
 
+def stale(name):
+    """Whether the object of a source is older than the source or a shared header."""
+    obj = os.path.join(HERE, "build", name + ".o")
+    if not os.path.exists(obj):
+        return True
+    deps = [os.path.join(HERE, name + ".hip"), os.path.join(HERE, "common.h"), os.path.join(HERE, "kernels.h")]
+    return any(os.path.getmtime(d) > os.path.getmtime(obj) for d in deps)
+
+
 def compile_one(name):
     obj = os.path.join(HERE, "build", name + ".o")
     extra = os.environ.get("PR_HIPCC_EXTRA_FLAGS", "").split()
@@ -47,10 +56,15 @@ def compile_one(name):
     return obj
 
 
-def build(jobs=8, verbose=True):
+def build(jobs=8, verbose=True, only_stale=False):
+    """Compiles every source (only_stale: just those whose object is out of date) and links the library."""
     os.makedirs(os.path.join(HERE, "build"), exist_ok=True)
+    todo = [n for n in SOURCES if not only_stale or stale(n)]
+    if verbose and only_stale:
+        print("compiling", todo)
     with cf.ThreadPoolExecutor(max_workers=jobs) as ex:
-        objs = list(ex.map(compile_one, SOURCES))
+        list(ex.map(compile_one, todo))
+    objs = [os.path.join(HERE, "build", n + ".o") for n in SOURCES]
     cmd = [hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", OUT, *objs]
     p = subprocess.run(cmd, capture_output=True, text=True)
     if p.returncode != 0:
@@ -60,28 +74,9 @@ def build(jobs=8, verbose=True):
     return OUT
 
 
-def build_probe():
-    """The stand-alone probes (probe_issue.hip: the VALU / MFMA issue microbenchmark; probe_attention.hip: per-workgroup
-    phase timing of the attention kernels; probe_lds.hip: LDS read throughput of the kernels' address patterns under
-    the candidate swizzles) as executables next to the library; not part of it."""
-    outs = []
-    for name in ("probe_issue", "probe_attention", "probe_lds"):
-        out = os.path.join(os.path.dirname(HERE), name)
-        cmd = [hipcc(), *[f for f in FLAGS if f != "-fPIC"], os.path.join(HERE, name + ".hip"), "-o", out]
-        p = subprocess.run(cmd, capture_output=True, text=True)
-        if p.returncode != 0:
-            raise RuntimeError(f"hipcc failed for {name}.hip:\n" + p.stderr)
-        print("built", out)
-        outs.append(out)
-    return outs
-
-
 if __name__ == "__main__":
     ap = argparse.ArgumentParser()
     ap.add_argument("--jobs", type=int, default=min(8, os.cpu_count() or 1))
-    ap.add_argument("--probe", action="store_true", help="build only the stand-alone probes")
+    ap.add_argument("--changed", action="store_true", help="compile only the sources that changed since their object")
     args = ap.parse_args()
-    if args.probe:
-        build_probe()
-    else:
-        build(args.jobs)
+    build(args.jobs, only_stale=args.changed)

@@ -43,10 +43,10 @@ int cache_append(void* Kc, void* Vc, float* Ac, const void* k, const void* v, co
   const long threads = (long)B * t_new * h * (d / 8) + (long)B * h;
   const dim3 grid((unsigned)((threads + 255) / 256));
   if (dtype == DT_BF16)
-    hipLaunchKernelGGL(cache_append_kernel<bf16_t>, grid, dim3(256), 0, st, (bf16_t*)Kc, (bf16_t*)Vc, Ac, (const bf16_t*)k,
+    PR_LAUNCH("cache_append", cache_append_kernel<bf16_t>, grid, dim3(256), 0, st, (bf16_t*)Kc, (bf16_t*)Vc, Ac, (const bf16_t*)k,
                        (const bf16_t*)v, g, a_last, B, cap, pos, t_new, h, d);
   else if (dtype == DT_F16)
-    hipLaunchKernelGGL(cache_append_kernel<f16_t>, grid, dim3(256), 0, st, (f16_t*)Kc, (f16_t*)Vc, Ac, (const f16_t*)k,
+    PR_LAUNCH("cache_append", cache_append_kernel<f16_t>, grid, dim3(256), 0, st, (f16_t*)Kc, (f16_t*)Vc, Ac, (const f16_t*)k,
                        (const f16_t*)v, g, a_last, B, cap, pos, t_new, h, d);
   else
     return -1;

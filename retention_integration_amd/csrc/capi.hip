@@ -8,6 +8,11 @@
 #include "kernels.h"
 
 
+namespace pr {
+launch_hook_t g_launch_hook = nullptr;
+void* g_launch_hook_user = nullptr;
+}  // namespace pr
+
 namespace {
 thread_local char g_err[256] = "";
 int fail(int code, const char* fmt, ...) {
@@ -38,7 +43,13 @@ size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 
 extern "C" {
 
-int pr_abi_version(void) { return 5; }
+int pr_abi_version(void) { return 6; }
+
+void pr_set_launch_hook(pr_launch_hook_t hook, void* user) {
+  pr::g_launch_hook = nullptr;   // (never a new hook with the old user pointer)
+  pr::g_launch_hook_user = user;
+  pr::g_launch_hook = hook;
+}
 const char* pr_last_error(void) { return g_err; }
 
 int pr_expanded_dim(int d, int deg) {
@@ -368,7 +379,7 @@ int check_decode(const char* what, const void* Q, const void* S, const float* s,
   if (K_new && ((S_out == S) != (s_out == s)))
     return fail(PR_ERR_ARG, "%s: update S and s both in place or both out of place", what);
   if (B <= 0 || tq <= 0 || h <= 0 || r <= 0) return fail(PR_ERR_ARG, "%s: need B,tq,h,r > 0", what);
-  if (tq * r > 8) return fail(PR_ERR_ARG, "%s: at most 8 query rows per (batch, kv head) (got %d)", what, tq * r);
+  if (tq * r > 16) return fail(PR_ERR_ARG, "%s: at most 16 query rows per (batch, kv head) (got %d)", what, tq * r);
   return 0;
 }
 }  // namespace
@@ -387,7 +398,12 @@ int pr_decode_step(const void* Q, const float* gq, const void* S, const float* s
                 "decode_step");
 }
 
-size_t pr_decode_step_noalloc_max_workspace(void) { return (size_t)pr::decode_static_floats() * sizeof(float); }
+size_t pr_decode_step_noalloc_max_workspace(void) {
+  // also the set-up call: the array's address on the current GPU is taken here, so that a first
+  // pr_decode_step_noalloc issued while a stream is being captured has no runtime query left to make
+  (void)pr::decode_static_prepare();
+  return (size_t)pr::decode_static_floats() * sizeof(float);
+}
 
 int pr_decode_step_noalloc(const void* Q, const float* gq, const void* S, const float* s, const void* Y_attn,
                            const float* l_attn, const float* rowmax, const void* K_new, const void* V_new,
@@ -403,6 +419,7 @@ int pr_decode_step_noalloc(const void* Q, const float* gq, const void* S, const 
   const int rc = pr::decode_step_static(Q, gq, S, s, Y_attn, l_attn, rowmax, K_new, V_new, log_decay, S_out, s_out, out,
                                         B, tq, h, r, d, deg, scale_p, dtype, attend_new ? 1 : 0, (hipStream_t)stream);
   if (rc == -6) return fail(PR_ERR_ARG, "decode_step_noalloc: the step needs more partial sums than the library's array holds");
+  if (rc == -7) return fail(PR_ERR_ARG, "decode_step_noalloc: the stream belongs to another GPU than the current one");
   return finish(rc, "decode_step_noalloc");
 }
 

@@ -121,11 +121,11 @@ template <typename T>
 static int prep_launch(const float* logG, const void* K, const void* Q, float* A, float* lcs, void* Kd, void* Qg, int BN,
                        int c, int h, int r, int d, int deg, hipStream_t st) {
   const size_t smem = (size_t)(c + 256) * sizeof(float);
-  hipLaunchKernelGGL(gate_scan_fwd_kernel, dim3((unsigned)(BN * h)), dim3(256), smem, st, logG, A, lcs, c, h);
+  PR_LAUNCH("gate_scan_fwd", gate_scan_fwd_kernel, dim3((unsigned)(BN * h)), dim3(256), smem, st, logG, A, lcs, c, h);
   const long groups = (long)BN * c * h;
 #define PR_CP(DD)                                                                                                      \
   case DD:                                                                                                             \
-    hipLaunchKernelGGL((gate_apply_fwd_kernel<T, DD>), dim3((unsigned)((groups * (DD / 8) + 255) / 256)), dim3(256), 0, \
+    PR_LAUNCH("gate_apply_fwd", (gate_apply_fwd_kernel<T, DD>), dim3((unsigned)((groups * (DD / 8) + 255) / 256)), dim3(256), 0, \
                        st, A, lcs, (const T*)K, (const T*)Q, (T*)Kd, (T*)Qg, groups, c, h, r, 1.f / deg);              \
     break;
   switch (d) { PR_CP(32) PR_CP(64) PR_CP(128) default: return -2; }
@@ -136,7 +136,7 @@ static int prep_launch(const float* logG, const void* K, const void* Q, float* A
 int gate_cumsum(const float* logG, float* A, int B, int t, int h, hipStream_t st) {
   if (t > GLUE_MAX_C) return -5;
   const size_t smem = (size_t)(t + 256) * sizeof(float);
-  hipLaunchKernelGGL(gate_scan_fwd_kernel, dim3((unsigned)(B * h)), dim3(256), smem, st, logG, A, (float*)nullptr, t, h);
+  PR_LAUNCH("gate_scan_fwd", gate_scan_fwd_kernel, dim3((unsigned)(B * h)), dim3(256), smem, st, logG, A, (float*)nullptr, t, h);
   return (int)hipGetLastError();
 }
 
@@ -152,7 +152,7 @@ int chunk_gate_scan_bwd(float* dA, const float* dGq, const float* dotk, const fl
                         int c, int h, int r, int deg, hipStream_t st) {
   if (c > GLUE_MAX_C) return -5;
   const size_t smem = (size_t)(c + 256) * sizeof(float);
-  hipLaunchKernelGGL(gate_scan_bwd_kernel, dim3((unsigned)(BN * h)), dim3(256), smem, st, dA, dGq, dotk, dlcs_a, dlcs_b,
+  PR_LAUNCH("gate_scan_bwd", gate_scan_bwd_kernel, dim3((unsigned)(BN * h)), dim3(256), smem, st, dA, dGq, dotk, dlcs_a, dlcs_b,
                      c, h, r, 1.f / deg);
   return (int)hipGetLastError();
 }

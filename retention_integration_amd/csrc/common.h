@@ -285,12 +285,28 @@ __device__ __forceinline__ float wave_sum(float x) {
   return sum_over_rows(sum_in_row(x));
 }
 
-// Hook points for a stand-alone timing probe (probe_attention.hip defines them to record wall-clock stamps per
-// workgroup); in the library they expand to nothing.
-#ifndef PR_STAMP
-#define PR_STAMP(i)
-#define PR_STAMP_VALUE(i, v)
-#endif
+// Every kernel launch of the library goes through PR_LAUNCH.  A caller may register a hook (pr_set_launch_hook of the
+// C ABI) that is called on the host right before and right after each launch with the kernel's name and stream --
+// a benchmark records a pair of events there and so times every kernel where it runs.  No hook: one load and a branch.
+typedef void (*launch_hook_t)(const char* kernel, int phase, void* stream, void* user);
+extern launch_hook_t g_launch_hook;
+extern void* g_launch_hook_user;
+struct LaunchScope {
+  const char* name;
+  hipStream_t st;
+  launch_hook_t hook;
+  LaunchScope(const char* n, hipStream_t s) : name(n), st(s), hook(g_launch_hook) {
+    if (hook) hook(name, 0, (void*)st, g_launch_hook_user);
+  }
+  ~LaunchScope() {
+    if (hook) hook(name, 1, (void*)st, g_launch_hook_user);
+  }
+};
+#define PR_LAUNCH(name, kern, grid, block, smem, st, ...)                                                              \
+  do {                                                                                                                 \
+    ::pr::LaunchScope pr_launch_scope_(name, st);                                                                      \
+    hipLaunchKernelGGL(kern, grid, block, smem, st, __VA_ARGS__);                                                      \
+  } while (0)
 
 // Kernels that use more than 64 KB of dynamic LDS must opt in once per function.
 static inline void allow_big_lds(const void* kernel, size_t bytes) {

@@ -30,7 +30,7 @@ namespace pr {
 constexpr long DEC_STATIC_FLOATS = 2L << 20;   // 8 MiB
 static __device__ __align__(256) float scratch[DEC_STATIC_FLOATS];
 
-constexpr int DEC_MAXROWS = 8;   // query rows (positions x query heads per kv head) handled per (batch, kv head)
+constexpr int DEC_MAXROWS = 16;   // query rows (positions x query heads per kv head) handled per (batch, kv head)
 
 
 __device__ __forceinline__ void feature_pair(int f, int& x, int& w, float& mult) {
@@ -282,17 +282,18 @@ static int decode_launch(const DecodeArgs& a0, int B, hipStream_t st) {
   if (decode_whole_pair(B, a.h, rows)) {
     a.split = 1;
     const dim3 grid((unsigned)(B * a.h));
-    if (rows <= 1) hipLaunchKernelGGL((decode_step_kernel<T, DH, 1, 1024, true>), grid, dim3(1024), 0, st, a);
-    else hipLaunchKernelGGL((decode_step_kernel<T, DH, 2, 1024, true>), grid, dim3(1024), 0, st, a);
+    if (rows <= 1) PR_LAUNCH("decode_step", (decode_step_kernel<T, DH, 1, 1024, true>), grid, dim3(1024), 0, st, a);
+    else PR_LAUNCH("decode_step", (decode_step_kernel<T, DH, 2, 1024, true>), grid, dim3(1024), 0, st, a);
     return (int)hipGetLastError();
   }
   a.split = decode_split(B, a.h);
   const dim3 grid((unsigned)(B * a.h), (unsigned)a.split);
-  if (rows <= 1) hipLaunchKernelGGL((decode_step_kernel<T, DH, 1, 256, false>), grid, dim3(256), 0, st, a);
-  else if (rows <= 2) hipLaunchKernelGGL((decode_step_kernel<T, DH, 2, 256, false>), grid, dim3(256), 0, st, a);
-  else if (rows <= 4) hipLaunchKernelGGL((decode_step_kernel<T, DH, 4, 256, false>), grid, dim3(256), 0, st, a);
-  else hipLaunchKernelGGL((decode_step_kernel<T, DH, DEC_MAXROWS, 256, false>), grid, dim3(256), 0, st, a);
-  hipLaunchKernelGGL((decode_merge_kernel<T, DH>), dim3((unsigned)(B * a.h), (unsigned)rows), dim3(64), 0, st, a);
+  if (rows <= 1) PR_LAUNCH("decode_step", (decode_step_kernel<T, DH, 1, 256, false>), grid, dim3(256), 0, st, a);
+  else if (rows <= 2) PR_LAUNCH("decode_step", (decode_step_kernel<T, DH, 2, 256, false>), grid, dim3(256), 0, st, a);
+  else if (rows <= 4) PR_LAUNCH("decode_step", (decode_step_kernel<T, DH, 4, 256, false>), grid, dim3(256), 0, st, a);
+  else if (rows <= 8) PR_LAUNCH("decode_step", (decode_step_kernel<T, DH, 8, 256, false>), grid, dim3(256), 0, st, a);
+  else PR_LAUNCH("decode_step", (decode_step_kernel<T, DH, DEC_MAXROWS, 256, false>), grid, dim3(256), 0, st, a);
+  PR_LAUNCH("decode_merge", (decode_merge_kernel<T, DH>), dim3((unsigned)(B * a.h), (unsigned)rows), dim3(64), 0, st, a);
   return (int)hipGetLastError();
 }
 
@@ -318,33 +319,54 @@ int decode_step(const void* Q, const float* gq, const void* S, const float* s, c
 
 long decode_static_floats() { return DEC_STATIC_FLOATS; }
 
+// The address of the library's per-GPU array on the current device, taken once per device with
+// hipGetSymbolAddress (a runtime call that is not stream work: it must not happen for the first time while a stream
+// is being captured, so decode_static_prepare() lets a caller do it ahead of time).  Returns 0 or a hipError_t.
+namespace {
+constexpr int MAX_DEVICES = 64;
+std::mutex static_mu;
+float* static_ptr[MAX_DEVICES] = {};   // the array's address on each GPU (each holds its own copy)
+int static_array(int dev, float** out) {
+  if (dev < 0 || dev >= MAX_DEVICES) return (int)hipErrorInvalidDevice;
+  std::lock_guard<std::mutex> lock(static_mu);
+  if (!static_ptr[dev]) {   // first use on this GPU, which is the current one
+    float* p = nullptr;
+    if (hipError_t e = hipGetSymbolAddress((void**)&p, HIP_SYMBOL(scratch))) return (int)e;
+    if (!p) return (int)hipErrorInvalidSymbol;
+    static_ptr[dev] = p;
+  }
+  *out = static_ptr[dev];
+  return 0;
+}
+}  // namespace
+
+int decode_static_prepare() {
+  int dev = -1;
+  if (hipError_t e = hipGetDevice(&dev)) return (int)e;
+  float* p;
+  return static_array(dev, &p);
+}
+
 // decode_step with the partial sums in the library's own per-GPU array instead of a caller's workspace: nothing is
 // allocated here or below.  Every slice of every (batch, kv head) writes all of its partial sums before the merge
 // kernel reads them, so nothing has to be cleared between calls; two calls in flight on one GPU at the same time
-// would share the array and race.  Returns -6 when the step needs more than the array holds, or a positive
-// hipError_t if the array's address cannot be obtained.
+// would share the array and race.  The array used is that of the GPU the stream belongs to, which must be the
+// current one (-7 otherwise: each GPU has its own copy, and the kernels run where the stream lives).  Returns -6 when
+// the step needs more than the array holds, or a positive hipError_t if the array's address cannot be obtained.
 int decode_step_static(const void* Q, const float* gq, const void* S, const float* s, const void* Y_attn,
                        const float* l_attn, const float* rowmax, const void* Knew, const void* Vnew,
                        const float* decay, void* Sout, float* sout, void* out, int B, int tq, int h, int r, int d,
                        int deg, float scale_p, int dtype, int attend_new, hipStream_t st) {
-  constexpr int MAX_DEVICES = 64;
-  static std::mutex mu;
-  static float* ptr[MAX_DEVICES] = {};   // the array's address on each GPU (each holds its own copy)
   if (decode_workspace_floats(B, h, r, tq, d) > DEC_STATIC_FLOATS) return -6;
   int dev = -1;
   if (hipError_t e = hipGetDevice(&dev)) return (int)e;
-  if (dev < 0 || dev >= MAX_DEVICES) return (int)hipErrorInvalidDevice;
-  float* part;
-  {
-    std::lock_guard<std::mutex> lock(mu);
-    if (!ptr[dev]) {   // first call on this GPU, which is the current one
-      float* p = nullptr;
-      if (hipError_t e = hipGetSymbolAddress((void**)&p, HIP_SYMBOL(scratch))) return (int)e;
-      if (!p) return (int)hipErrorInvalidSymbol;
-      ptr[dev] = p;
-    }
-    part = ptr[dev];
+  if (st != nullptr) {   // (the null stream is the current device's by definition)
+    hipDevice_t sdev = -1;
+    if (hipError_t e = hipStreamGetDevice(st, &sdev)) return (int)e;
+    if ((int)sdev != dev) return -7;
   }
+  float* part;
+  if (int rc = static_array(dev, &part)) return rc;
   return decode_step(Q, gq, S, s, Y_attn, l_attn, rowmax, Knew, Vnew, decay, Sout, sout, out, part, B, tq, h, r, d, deg,
                      scale_p, dtype, attend_new, st);
 }

@@ -220,14 +220,14 @@ static int launch_fwd(const void* X, const float* logG, void* Y, int B, int n, i
   // walk costs one memory round trip instead of n
   if (sizeof(T) == 4 && F * B * H < 256 * 1024) {
     dim3 g1((unsigned)((F + 255) / 256), (unsigned)(B * H));
-    hipLaunchKernelGGL((discumsum_fwd_kernel<T, 64, 4>), g1, dim3(256), 0, st, (const T*)X, logG, (T*)Y, n, n_out, H, F);
+    PR_LAUNCH("discumsum_fwd", (discumsum_fwd_kernel<T, 64, 4>), g1, dim3(256), 0, st, (const T*)X, logG, (T*)Y, n, n_out, H, F);
     return (int)hipGetLastError();
   }
   // few threads in flight (small F): keep many chunks' loads outstanding per thread instead
   if (per_bh * B * H < 256 * 1024)
-    hipLaunchKernelGGL((discumsum_fwd_kernel<T, 16>), grid, dim3(256), 0, st, (const T*)X, logG, (T*)Y, n, n_out, H, F);
+    PR_LAUNCH("discumsum_fwd", (discumsum_fwd_kernel<T, 16>), grid, dim3(256), 0, st, (const T*)X, logG, (T*)Y, n, n_out, H, F);
   else
-    hipLaunchKernelGGL((discumsum_fwd_kernel<T, 4>), grid, dim3(256), 0, st, (const T*)X, logG, (T*)Y, n, n_out, H, F);
+    PR_LAUNCH("discumsum_fwd", (discumsum_fwd_kernel<T, 4>), grid, dim3(256), 0, st, (const T*)X, logG, (T*)Y, n, n_out, H, F);
   return (int)hipGetLastError();
 }
 template <typename T>
@@ -238,9 +238,9 @@ static int launch_bwd(const void* dY, const void* Y, const float* logG, void* dX
   const int tot = B * H * n;
   if (sizeof(T) == 4 && F * B * H < 256 * 1024) {   // see launch_fwd: one element per thread, all chunks in flight
     const unsigned b1 = (unsigned)((F + 255) / 256);
-    hipLaunchKernelGGL((discumsum_bwd_kernel<T, 64, 4>), dim3(b1, (unsigned)(B * H)), dim3(256), 0, st, (const T*)dY,
+    PR_LAUNCH("discumsum_bwd", (discumsum_bwd_kernel<T, 64, 4>), dim3(b1, (unsigned)(B * H)), dim3(256), 0, st, (const T*)dY,
                        (const T*)Y, logG, (T*)dX, partial, n, n_out, H, F, (int)b1 * 4);
-    hipLaunchKernelGGL(discumsum_reduce_kernel, dim3((tot * 64 + 255) / 256), dim3(256), 0, st, partial, dlogG, n, H,
+    PR_LAUNCH("discumsum_reduce", discumsum_reduce_kernel, dim3((tot * 64 + 255) / 256), dim3(256), 0, st, partial, dlogG, n, H,
                        (int)b1 * 4, B * H);
     return (int)hipGetLastError();
   }
@@ -248,12 +248,12 @@ static int launch_bwd(const void* dY, const void* Y, const float* logG, void* dX
   const int waves = blocks * 4;
   dim3 grid(blocks, (unsigned)(B * H));
   if (per_bh * B * H < 256 * 1024)
-    hipLaunchKernelGGL((discumsum_bwd_kernel<T, 8>), grid, dim3(256), 0, st, (const T*)dY, (const T*)Y, logG, (T*)dX,
+    PR_LAUNCH("discumsum_bwd", (discumsum_bwd_kernel<T, 8>), grid, dim3(256), 0, st, (const T*)dY, (const T*)Y, logG, (T*)dX,
                        partial, n, n_out, H, F, waves);
   else
-    hipLaunchKernelGGL((discumsum_bwd_kernel<T, 2>), grid, dim3(256), 0, st, (const T*)dY, (const T*)Y, logG, (T*)dX,
+    PR_LAUNCH("discumsum_bwd", (discumsum_bwd_kernel<T, 2>), grid, dim3(256), 0, st, (const T*)dY, (const T*)Y, logG, (T*)dX,
                        partial, n, n_out, H, F, waves);
-  hipLaunchKernelGGL(discumsum_reduce_kernel, dim3((tot * 64 + 255) / 256), dim3(256), 0, st, partial, dlogG, n, H,
+  PR_LAUNCH("discumsum_reduce", discumsum_reduce_kernel, dim3((tot * 64 + 255) / 256), dim3(256), 0, st, partial, dlogG, n, H,
                      waves, B * H);
   return (int)hipGetLastError();
 }
@@ -264,10 +264,10 @@ static int launch_pair_fwd(const void* X, const float* X2, const float* logG, vo
   const int nblk = (int)((F / Pack16<T>::N + 255) / 256), nblk2 = (int)((F2 + 255) / 256);
   dim3 grid((unsigned)(nblk + nblk2), (unsigned)(B * H));
   if ((F / Pack16<T>::N) * B * H < 256 * 1024)
-    hipLaunchKernelGGL((discumsum_pair_fwd_kernel<T, 16>), grid, dim3(256), 0, st, (const T*)X, X2, logG, (T*)Y, Y2, n,
+    PR_LAUNCH("discumsum_pair_fwd", (discumsum_pair_fwd_kernel<T, 16>), grid, dim3(256), 0, st, (const T*)X, X2, logG, (T*)Y, Y2, n,
                        n_out, H, F, F2, nblk);
   else
-    hipLaunchKernelGGL((discumsum_pair_fwd_kernel<T, 4>), grid, dim3(256), 0, st, (const T*)X, X2, logG, (T*)Y, Y2, n,
+    PR_LAUNCH("discumsum_pair_fwd", (discumsum_pair_fwd_kernel<T, 4>), grid, dim3(256), 0, st, (const T*)X, X2, logG, (T*)Y, Y2, n,
                        n_out, H, F, F2, nblk);
   return (int)hipGetLastError();
 }
@@ -279,12 +279,12 @@ static int launch_pair_bwd(const void* dY, const void* Y, const float* dY2, cons
   const int waves = (nblk + nblk2) * 4, tot = B * H * n;
   dim3 grid((unsigned)(nblk + nblk2), (unsigned)(B * H));
   if ((F / Pack16<T>::N) * B * H < 256 * 1024)
-    hipLaunchKernelGGL((discumsum_pair_bwd_kernel<T, 8>), grid, dim3(256), 0, st, (const T*)dY, (const T*)Y, dY2, Y2,
+    PR_LAUNCH("discumsum_pair_bwd", (discumsum_pair_bwd_kernel<T, 8>), grid, dim3(256), 0, st, (const T*)dY, (const T*)Y, dY2, Y2,
                        logG, (T*)dX, dX2, partial, n, n_out, H, F, F2, nblk, waves);
   else
-    hipLaunchKernelGGL((discumsum_pair_bwd_kernel<T, 2>), grid, dim3(256), 0, st, (const T*)dY, (const T*)Y, dY2, Y2,
+    PR_LAUNCH("discumsum_pair_bwd", (discumsum_pair_bwd_kernel<T, 2>), grid, dim3(256), 0, st, (const T*)dY, (const T*)Y, dY2, Y2,
                        logG, (T*)dX, dX2, partial, n, n_out, H, F, F2, nblk, waves);
-  hipLaunchKernelGGL(discumsum_reduce_kernel, dim3((tot * 64 + 255) / 256), dim3(256), 0, st, partial, dlogG, n, H,
+  PR_LAUNCH("discumsum_reduce", discumsum_reduce_kernel, dim3((tot * 64 + 255) / 256), dim3(256), 0, st, partial, dlogG, n, H,
                      waves, B * H);
   return (int)hipGetLastError();
 }
@@ -357,14 +357,14 @@ int scan_gate_grad(const void* Y, const void* R, const float* Y2, const float* R
   const int waves = (nblk + nblk2) * 4, tot = B * H * n;
   dim3 grid((unsigned)(nblk + nblk2), (unsigned)(B * H), (unsigned)n);
   if (dtype == DT_BF16)
-    hipLaunchKernelGGL(scan_gate_grad_kernel<bf16_t>, grid, dim3(256), 0, st, (const bf16_t*)Y, (const bf16_t*)R, Y2, R2,
+    PR_LAUNCH("scan_gate_grad", scan_gate_grad_kernel<bf16_t>, grid, dim3(256), 0, st, (const bf16_t*)Y, (const bf16_t*)R, Y2, R2,
                        logG, partial, n, H, F, F2, nblk, waves);
   else if (dtype == DT_F16)
-    hipLaunchKernelGGL(scan_gate_grad_kernel<f16_t>, grid, dim3(256), 0, st, (const f16_t*)Y, (const f16_t*)R, Y2, R2,
+    PR_LAUNCH("scan_gate_grad", scan_gate_grad_kernel<f16_t>, grid, dim3(256), 0, st, (const f16_t*)Y, (const f16_t*)R, Y2, R2,
                        logG, partial, n, H, F, F2, nblk, waves);
   else
     return -1;
-  hipLaunchKernelGGL(discumsum_reduce_kernel, dim3((tot * 64 + 255) / 256), dim3(256), 0, st, partial, dlogG, n, H,
+  PR_LAUNCH("discumsum_reduce", discumsum_reduce_kernel, dim3((tot * 64 + 255) / 256), dim3(256), 0, st, partial, dlogG, n, H,
                      waves, B * H);
   return (int)hipGetLastError();
 }

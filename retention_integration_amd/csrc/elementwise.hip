@@ -75,7 +75,7 @@ static int prep_launch(const void* O, const void* dO, const float* den, const fl
   dim3 grid((unsigned)((threads + 255) / 256));
 #define PR_PREP(DD)                                                                                                    \
   case DD:                                                                                                             \
-    hipLaunchKernelGGL((qs_bwd_prep_kernel<T, DD>), grid, dim3(256), 0, st, (const T*)O, (const T*)dO, den, rowmax,    \
+    PR_LAUNCH("qs_bwd_prep", (qs_bwd_prep_kernel<T, DD>), grid, dim3(256), 0, st, (const T*)O, (const T*)dO, den, rowmax,    \
                        qgate, (T*)dOs, cvec, (T*)dYa, dla, dYscale, rows, h, r, scale_p);                              \
     break;
   switch (d) { PR_PREP(32) PR_PREP(64) PR_PREP(128) default: return -2; }

@@ -130,7 +130,7 @@ int chunk_gate_scan_bwd(float* dA, const float* dGq, const float* dotk, const fl
 int cache_append(void* Kc, void* Vc, float* Ac, const void* k, const void* v, const float* g, float* a_last, int B,
                  int cap, int pos, int t_new, int h, int d, int dtype, hipStream_t st);
 
-// decode.hip (return -3: more than 8 query rows per (batch, kv head))
+// decode.hip (return -3: more than 16 query rows per (batch, kv head))
 long decode_workspace_floats(int B, int h, int r, int tq, int d);
 int decode_step(const void* Q, const float* gq, const void* S, const float* s, const void* Y_attn, const float* l_attn,
                 const float* rowmax, const void* Knew, const void* Vnew, const float* decay, void* Sout, float* sout,
@@ -138,8 +138,10 @@ int decode_step(const void* Q, const float* gq, const void* S, const float* s, c
                 int attend_new, hipStream_t st);
 
 // the same step with its partial sums in a per-GPU array of the library (return -6: the step needs more than
-// decode_static_floats() floats of partial sums)
+// decode_static_floats() floats of partial sums; -7: the stream belongs to another GPU than the current one).
+// decode_static_prepare() takes the array's address on the current GPU ahead of the first step (0 or a hipError_t).
 long decode_static_floats();
+int decode_static_prepare();
 int decode_step_static(const void* Q, const float* gq, const void* S, const float* s, const void* Y_attn,
                        const float* l_attn, const float* rowmax, const void* Knew, const void* Vnew,
                        const float* decay, void* Sout, float* sout, void* out, int B, int tq, int h, int r, int d,

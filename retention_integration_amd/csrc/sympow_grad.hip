@@ -348,7 +348,7 @@ static int grad_launch(const GradArgs& a, int BN, hipStream_t st) {
     dim3 grid((unsigned)(((npairs + 7) / 8) * 8 * row_blocks));
     auto kern = sympow_grad_kernel<T, DK, DV, MT, MULT, SYM, ALONE>;
     allow_big_lds((const void*)kern, smem);
-    hipLaunchKernelGGL(kern, grid, dim3(256), smem, st, a, row_blocks, npairs);
+    PR_LAUNCH("sympow_grad", kern, grid, dim3(256), smem, st, a, row_blocks, npairs);
   };
   // 128 rows per workgroup.  Up to d = 64 that is four workgroups (16 waves) per compute unit, and the vector
   // instructions of the two folds issue at twice the rate of a 256-row tiling at two workgroups (measured 7 %

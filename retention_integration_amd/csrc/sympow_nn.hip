@@ -396,7 +396,7 @@ static int nn_launch(const NNArgs& a, int BN, hipStream_t st) {
     dim3 grid((unsigned)(((npairs + 7) / 8) * 8 * row_blocks));
     auto kern = sympow_nn_kernel<T, DK, DV, MT, MULT, EPI, SYM, ALONE>;
     allow_big_lds((const void*)kern, smem);
-    hipLaunchKernelGGL(kern, grid, dim3(256), smem, st, a, row_blocks, npairs);
+    PR_LAUNCH("sympow_nn", kern, grid, dim3(256), smem, st, a, row_blocks, npairs);
   };
   if constexpr (DK <= 64) {
     if (rows >= 256) { go(IC<4>{}, IC<0>{}); return (int)hipGetLastError(); }

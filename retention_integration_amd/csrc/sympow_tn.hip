@@ -670,7 +670,7 @@ static int tn_chain_launch(const void* A, const void* Bm, const float* w, const 
   {                                                                                                                    \
     auto kern = sympow_tn_chain_kernel<T, DK, DV, XPW, NW, KT, W, R>;                                                          \
     allow_big_lds((const void*)kern, smem);                                                                            \
-    hipLaunchKernelGGL(kern, grid, dim3(64 * NW), smem, st, (const T*)A, (const T*)Bm, w, lcs, (T*)S, s, n, c, h * r, \
+    PR_LAUNCH("sympow_tn_chain", kern, grid, dim3(64 * NW), smem, st, (const T*)A, (const T*)Bm, w, lcs, (T*)S, s, n, c, h * r, \
                        r, h, use_mult);                                                                                \
   }
   if (w) {
@@ -724,11 +724,11 @@ static int tn_launch(const void* A, const void* Bm, const float* w, void* S, flo
   if (w) {
     auto kern = sympow_tn_kernel<T, DK, DV, XPW, true>;
     allow_big_lds((const void*)kern, smem);
-    hipLaunchKernelGGL(kern, grid, dim3(256), smem, st, (const T*)A, (const T*)Bm, w, (T*)S, s, c, h * r, r, h, use_mult, skip);
+    PR_LAUNCH("sympow_tn", kern, grid, dim3(256), smem, st, (const T*)A, (const T*)Bm, w, (T*)S, s, c, h * r, r, h, use_mult, skip);
   } else {
     auto kern = sympow_tn_kernel<T, DK, DV, XPW, false>;
     allow_big_lds((const void*)kern, smem);
-    hipLaunchKernelGGL(kern, grid, dim3(256), smem, st, (const T*)A, (const T*)Bm, w, (T*)S, s, c, h * r, r, h, use_mult, skip);
+    PR_LAUNCH("sympow_tn", kern, grid, dim3(256), smem, st, (const T*)A, (const T*)Bm, w, (T*)S, s, c, h * r, r, h, use_mult, skip);
   }
   return (int)hipGetLastError();
 }

@@ -20,24 +20,6 @@ from . import _lib
 from .ops import expanded_dim
 
 
-# Optional in-step timing of the two kernels a benchmark reports on their own: set to a dict and every call appends a
-# pair of events (recorded on the launch stream around that kernel alone) under "sympow_grad(dK)" and
-# "sympow_tn(update_state)".  None (the default) records nothing.
-KERNEL_TIMERS = None
-
-
-def _timed(name, launch):
-    tm = KERNEL_TIMERS
-    if tm is None:
-        return launch()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
-    rc = launch()
-    e1.record()
-    tm.setdefault(name, []).append((e0, e1))
-    return rc
-
-
 # The state kernels chained with the scan over the chunk axis (short chunks, many batch elements x heads).
 # None: where the library says it is the faster form; True: wherever the shape allows it; False: never.
 CHAIN = None
@@ -93,8 +75,7 @@ def chunked_fwd(Q: Tensor, K: Tensor, V: Tensor, log_G: Optional[Tensor], deg: i
                                                 deg, code, st), "update_state_scan_fwd")
     else:
         S, s = torch.empty_like(Sc), torch.empty_like(sc)
-        _lib.check(_timed("sympow_tn(update_state)", lambda: lib.pr_update_state_fwd(
-            p(Kd_), p(V), p(S), p(s), BN, c, h, d, deg, n, code, st)), "update_state_fwd")
+        _lib.check(lib.pr_update_state_fwd(p(Kd_), p(V), p(S), p(s), BN, c, h, d, deg, n, code, st), "update_state_fwd")
         _lib.check(lib.pr_state_scan_fwd(p(S), p(s), p(lcs), p(Sc), p(sc), b, n, n, h, D * d, D, code, st),
                    "state_scan_fwd")
         del S, s
@@ -167,12 +148,9 @@ def chunked_bwd(Q: Tensor, K: Tensor, V: Tensor, A: Tensor, lcs: Tensor, Kd: Ten
                                          D * d, D, code, st), "state_scan_bwd")
         del dSc, dsc
     dKd, dVs = torch.empty_like(K), torch.empty_like(V)
-    # (two calls: the value gradient and the key gradient are separate kernels, and the latter is timed on its own)
-    # (dS comes from the kernels above, so both orders of a pair hold the same sum: the last flag says so)
-    _lib.check(lib.pr_update_state_bwd(p(Kd), p(V), p(dS), p(ds), None, p(dVs), BN, c, h, d, deg, 1, n, code, st),
-               "update_state_bwd(dV)")
-    _lib.check(_timed("sympow_grad(dK)", lambda: lib.pr_update_state_bwd(
-        p(Kd), p(V), p(dS), p(ds), p(dKd), None, BN, c, h, d, deg, 1, n, code, st)), "update_state_bwd(dK)")
+    # (dS comes from the kernels above, so both orders of a pair hold the same sum: the symmetry flag says so)
+    _lib.check(lib.pr_update_state_bwd(p(Kd), p(V), p(dS), p(ds), p(dKd), p(dVs), BN, c, h, d, deg, 1, n, code, st),
+               "update_state_bwd")
 
     # the attention backward adds the state-path gradients in its epilogue and writes the final dQ, dK, dV
     dQa, dKa, dVa = torch.empty_like(Q), torch.empty_like(K), torch.empty_like(V)

@@ -1,6 +1,6 @@
 """``power_retention_inference`` with the single-token step fused (ref: retention/power_retention_maker.py:284-395).
 
-Same signature, results and state layout as the maker-assembled function; calls with a state and at most 8 query
+Same signature, results and state layout as the maker-assembled function; calls with a state and at most 16 query
 rows per (batch, kv head) -- the decode step -- go through one pass over the state (query, and the fold of a
 single new token when ``switch_over_seq_len`` is reached with a one-token cache) instead of the operator chain.
 Everything else is delegated to the composed function.
@@ -30,7 +30,7 @@ def make_fused_inference(composed):
         has_cache = K is not None and V is not None
         fast = (initial_state is not None and sum_of_keys is not None and deg == 2 and Q.dim() == 4
                 and Q.dtype in (torch.bfloat16, torch.float16) and initial_state.dtype == Q.dtype
-                and Q.shape[1] * (Q.shape[2] // initial_state.shape[1]) <= 8
+                and Q.shape[1] * (Q.shape[2] // initial_state.shape[1]) <= 16
                 and Q.shape[3] in (32, 64, 128))
         if has_cache:
             fast = fast and K.shape[1] >= Q.shape[1] and K.dtype == Q.dtype == V.dtype and K.shape[0] == Q.shape[0] \

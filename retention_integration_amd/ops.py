@@ -387,7 +387,7 @@ def _(log_G):
 def decode_step(Q: Tensor, gq: Optional[Tensor], S: Tensor, s: Tensor, Y_attn: Optional[Tensor],
                 l_attn: Optional[Tensor], rowmax: Optional[Tensor], K_new: Optional[Tensor], V_new: Optional[Tensor],
                 log_decay: Optional[Tensor], scale_p: float, attend_new: bool = False) -> Tuple[Tensor, Tensor, Tensor]:
-    """Q [b, tq, hq, d] (tq * hq/h <= 8), gq [b, h] fp32 or None, S [b, h, D, d], s [b, h, D] fp32, attention part or
+    """Q [b, tq, hq, d] (tq * hq/h <= 16), gq [b, h] fp32 or None, S [b, h, D, d], s [b, h, D] fp32, attention part or
     None, and optionally one new token K_new, V_new [b, h, d] with log_decay [b, h] -> (out [b, tq, hq, d],
     S_new, s_new); without a new token S_new, s_new are empty tensors.  attend_new: the attention part is the new
     token attending to itself (tq == 1, no Y_attn)."""

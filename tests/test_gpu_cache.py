@@ -37,6 +37,9 @@ def tokens(b, n, h, r, d, dtype, seed, gated=True):
     (torch.bfloat16, 3, 2, 2, 64, 8, True),      # several switch-overs in 30 steps
     (torch.float16, 2, 2, 1, 128, 5, True),
     (torch.bfloat16, 2, 1, 4, 32, 7, False),     # no gates
+    (torch.bfloat16, 2, 2, 8, 64, 6, True),      # 8 query heads per kv head
+    (torch.bfloat16, 1, 2, 16, 32, 6, True),     # 16: still one pass over the state
+    (torch.bfloat16, 1, 1, 24, 32, 6, True),     # 24: the state query runs as the operator over the same buffers
 ])
 def test_cache_step_follows_the_reference_callers_sequence(dtype, b, h, r, d, sw, gated):
     """30 tokens through RetentionCache.step and through the caller's loop over the maker-assembled function and over

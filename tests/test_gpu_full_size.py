@@ -114,3 +114,47 @@ def test_inference_config_at_size_prefill_then_512_recurrent_steps(pra):
             check(f"step {i} Y", Y[rows], Yo)
     check("final state", S[rows], So)
     check("final sum_of_keys", s[rows], so)
+
+
+@pytest.mark.parametrize("bi,hd", [(2, 5), (1, 11)])
+def test_short_chunk_config_at_full_size_matches_the_oracle_on_a_slice(pra, bi, hd):
+    """BASELINE configs[4] at its full size: fp16, b=4, t=16384, h=16, d=128, deg=2, chunk 128, no gating, inputs
+    N(0,1) * 0.5, dO ~ N(0,1).  The GPU launch holds all 4 x 128 x 16 (batch, chunk, head) pairs (the library picks the
+    chained state kernels there); batch entries and heads are independent, so the fp32 oracle runs on one head of one
+    batch entry per case (0.6 GB of fp32 state, about a minute of host time).  Y, dQ, dK, dV per tensor and per chunk."""
+    b, t, h, d, c = 4, 16384, 16, 128, 128
+    n = t // c
+    heads = [hd]
+    g = torch.Generator().manual_seed(404)
+    Q, K, V = ((0.5 * torch.randn(b, t, h, d, generator=g)).to(torch.float16) for _ in range(3))
+    dO = torch.randn(b, t, h, d, generator=g).to(torch.float16)
+    xs = [x.to(DEV).requires_grad_(True) for x in (Q, K, V)]
+    Y = pra.power_retention(*xs, None, deg=2, chunk_size=c)
+    Y.backward(dO.to(DEV))
+    torch.cuda.synchronize()
+    got = {"Y": Y.detach()[bi][:, heads].cpu(), "dQ": xs[0].grad[bi][:, heads].cpu(), "dK": xs[1].grad[bi][:, heads].cpu(),
+           "dV": xs[2].grad[bi][:, heads].cpu()}
+    for x in [Y] + [x.grad for x in xs]:
+        assert torch.isfinite(x).all()
+    del xs, Y
+    torch.cuda.empty_cache()
+
+    worst = {}
+    for j, hd in enumerate(heads):     # one head per oracle pass
+        xo = [x[bi:bi + 1, :, hd:hd + 1].float().clone().requires_grad_(True) for x in (Q, K, V)]
+        Yo = oracle.power_retention(*xo, None, deg=2, chunk_size=c)
+        Yo.backward(dO[bi:bi + 1, :, hd:hd + 1].float())
+        want = {"Y": Yo.detach()[0, :, 0], "dQ": xo[0].grad[0, :, 0], "dK": xo[1].grad[0, :, 0], "dV": xo[2].grad[0, :, 0]}
+        for nm, w in want.items():
+            gsl = got[nm][:, j]
+            tol = OUT_TOL if nm == "Y" else GRAD_TOL
+            whole = _rel(gsl, w, (0, 1)).item()
+            per = _rel(gsl.reshape(n, c, d), w.reshape(n, c, d), (1, 2))     # [n]
+            k = int(per.argmax())
+            print(f"  batch {bi} head {hd} {nm}: rel-L2 {whole:.3e}, worst chunk {per.max().item():.3e} at chunk {k}",
+                  flush=True)
+            worst[nm] = max(worst.get(nm, 0.0), per.max().item())
+            assert whole <= tol, f"{nm} head {hd}: rel-L2 {whole:.3e} > {tol}"
+            assert per.max().item() <= tol, f"{nm}: chunk {k} of head {hd} is off: rel-L2 {per.max().item():.3e} > {tol}"
+        del xo, Yo, want
+    print("  worst per-(chunk, head) rel-L2:", {k: f"{v:.3e}" for k, v in worst.items()}, flush=True)

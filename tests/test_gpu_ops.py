@@ -150,7 +150,9 @@ def test_update_state_inference_form(pra):
 @pytest.mark.parametrize("dtype,d,c,r,zis,attn", [
     (torch.bfloat16, 64, 128, 1, True, True), (torch.bfloat16, 32, 40, 2, False, True),
     (torch.float16, 128, 64, 1, True, True), (torch.bfloat16, 64, 256, 1, False, False),
-    (torch.bfloat16, 64, 16, 4, False, True)])
+    (torch.bfloat16, 64, 16, 4, False, True),
+    # query-head ratios of the reference's own lists (ref: perf/tests/test_list.py:50-84 ratio 8, :189-218 ratio 16)
+    (torch.bfloat16, 64, 64, 8, True, True), (torch.bfloat16, 32, 24, 16, False, True)])
 def test_query_state(pra, dtype, d, c, r, zis, attn):
     b, n, h = 1, 2, 2
     D = oracle.expanded_dim(d)
@@ -186,13 +188,39 @@ def test_query_state(pra, dtype, d, c, r, zis, attn):
         check(nm, ga, gb, GRAD_TOL)
 
 
+@pytest.mark.parametrize("d,r", [(32, 1), (64, 1), (32, 16), (64, 16)])
+def test_query_state_inference_form_gqa(pra, d, r):
+    """The 4-D (inference) form at the reference's sizes: b = 32, 128 query positions, one or sixteen query heads per
+    kv head, forward only (ref: perf/tests/test_list.py:189-218)."""
+    b, c, h, dtype = 32, 128, 2, torch.bfloat16
+    Q = rnd(b, c, h * r, d, dtype=dtype, seed=40)
+    Ks = rnd(b, 48, h, d, dtype=torch.float32, scale=d ** -0.25, seed=41)
+    Vs = rnd(b, 48, h, d, dtype=torch.float32, seed=42)
+    S, s = oracle.update_state(Ks, Vs, 2)
+    S = S.to(dtype)
+    Ya = rnd(b, c, h * r, d, dtype=dtype, seed=43)
+    la = rnd(b, c, h * r, dtype=torch.float32, seed=44).abs() + c
+    rm = rnd(b, c, h * r, dtype=torch.float32, seed=45).abs() * 3 + 1.0
+    scale = 1.0 / math.sqrt(d)
+    O = pra.query_state(dev(Q), dev(S), dev(s), dev(Ya), dev(la), dev(rm), 2, scale, False)
+    Oo = oracle.query_state(gold(Q), gold(S), gold(s), gold(Ya), gold(la), gold(rm), 2, scale, False)
+    check("O", O, Oo, OUT_TOL)
+    O2 = pra.query_state(dev(Q), dev(S), dev(s), None, None, None, 2, scale, False)
+    Oo2 = oracle.query_state(gold(Q), gold(S), gold(s), None, None, None, 2, scale, False)
+    check("O (state only)", O2, Oo2, OUT_TOL)
+
+
 # ---------------------------------------------------------------- attention
 @pytest.mark.parametrize("dtype,d,tq,tk,r,gated,norm,deg", [
     (torch.bfloat16, 64, 128, 128, 1, True, False, 2), (torch.bfloat16, 64, 200, 200, 1, False, True, 2),
     (torch.float16, 128, 96, 96, 1, True, False, 2), (torch.bfloat16, 32, 1, 130, 2, True, False, 2),
     (torch.bfloat16, 64, 70, 150, 2, True, True, 2), (torch.bfloat16, 64, 384, 384, 1, True, False, 2),
     (torch.bfloat16, 64, 1024, 1024, 1, True, False, 2), (torch.bfloat16, 64, 160, 160, 1, True, False, 4),
-    (torch.bfloat16, 32, 128, 128, 2, False, True, 4)])
+    (torch.bfloat16, 32, 128, 128, 2, False, True, 4),
+    # query-head ratio 8 (ref: perf/tests/test_list.py:50-84, and its single-query "inference" cases) and 16
+    (torch.bfloat16, 64, 128, 128, 8, True, False, 2), (torch.bfloat16, 32, 128, 128, 8, False, True, 4),
+    (torch.bfloat16, 64, 1, 64, 8, True, True, 2), (torch.bfloat16, 64, 1, 64, 8, True, False, 4),
+    (torch.bfloat16, 64, 1, 100, 16, True, False, 2), (torch.bfloat16, 64, 64, 64, 16, True, False, 2)])
 def test_attention(pra, dtype, d, tq, tk, r, gated, norm, deg):
     b, h = 2, 2
     Q, K, V = (rnd(b, tq, h * r, d, dtype=dtype, seed=30), rnd(b, tk, h, d, dtype=dtype, seed=31),

@@ -80,6 +80,9 @@ def run_both(pra, Q, K, V, lg, chunk, dO=None, **kw):
     (torch.bfloat16, 1, 96, 2, 1, 64, None, True),      # quadratic path
     (torch.bfloat16, 1, 384, 2, 3, 64, 128, True),      # GQA ratio that is not a power of two (irregular tile copies)
     (torch.float16, 2, 320, 1, 3, 32, 64, True),        # the same with d = 32, fp16, padding
+    (torch.bfloat16, 1, 512, 1, 8, 64, 128, True),      # GQA ratio 8 (ref: perf/tests/test_list.py:50-84)
+    (torch.bfloat16, 1, 256, 1, 16, 32, 64, True),      # GQA ratio 16 (ref: perf/tests/test_list.py:189-218)
+    (torch.bfloat16, 1, 128, 2, 8, 64, None, True),     # ratio 8 on the quadratic path
 ])
 def test_power_retention_fwd_bwd(pra, dtype, b, t, h, r, d, chunk, gated):
     std = 0.5 if dtype == torch.float16 else 1.0
@@ -89,7 +92,7 @@ def test_power_retention_fwd_bwd(pra, dtype, b, t, h, r, d, chunk, gated):
     run_both(pra, Q, K, V, lg, chunk, dO)
 
 
-@pytest.mark.parametrize("gated,r", [(True, 1), (True, 2), (False, 1)])
+@pytest.mark.parametrize("gated,r", [(True, 1), (True, 2), (False, 1), (True, 8), (True, 16)])
 def test_fused_node_equals_operator_composition(pra, gated, r):
     """power_retention (one fused autograd node) vs the same function assembled from the four operators
     through make_power_retention: same kernels, so agreement is at rounding level."""
@@ -403,7 +406,12 @@ def test_large_shape_invariants(pra):
 
 
 @pytest.mark.parametrize("dtype,d,r,gated", [(torch.bfloat16, 64, 1, True), (torch.bfloat16, 32, 4, True),
-                                             (torch.float16, 128, 2, False), (torch.bfloat16, 64, 8, True)])
+                                             (torch.float16, 128, 2, False), (torch.bfloat16, 64, 8, True),
+                                             # ratios 12 and 16 (ref: perf/tests/test_list.py:270-320, :189-218): one
+                                             # pass over the state up to 16 query rows per kv head
+                                             (torch.bfloat16, 64, 12, True), (torch.bfloat16, 32, 16, True),
+                                             # beyond 16 rows the operator chain takes over (both names, same values)
+                                             (torch.bfloat16, 32, 24, True)])
 def test_fused_decode_step_equals_operator_chain(pra, dtype, d, r, gated):
     """The one-pass decode step (query + fold of one token) against the maker-assembled operator chain and the
     oracle: with a growing cache (no fold), with a one-token cache folded every step, and from the state alone."""

@@ -80,3 +80,61 @@ def test_noalloc_decode_step_refuses_what_does_not_fit():
     rc = lib.pr_decode_step_noalloc(x.data_ptr(), None, x.data_ptr(), x.data_ptr(), None, None, None, None, None, None,
                                     None, None, x.data_ptr(), B, tq, h, r, d, 1.0 / d, 2, 0, 0, _lib.stream())
     assert rc == -3 and b"partial sums" in lib.pr_last_error()
+
+
+def test_noalloc_decode_step_captured_in_a_hip_graph_replays_bit_for_bit():
+    """The entry point is meant for callers under stream capture: after the set-up call (which takes the array's
+    address on this GPU) a recurrent step is captured, and every replay -- with eager work and synchronisations in
+    between -- must give the eager result of the same step bit for bit (state updated in place, so each replay is
+    compared with an eager step from the same starting state)."""
+    from retention_integration_amd import _lib
+    lib = _lib.load()
+    assert lib.pr_decode_step_noalloc_max_workspace() == 8 << 20   # set-up call: resolves the array on this GPU
+    p = _lib.ptr
+    B, h, r, d, dtype = 4, 2, 2, 64, torch.bfloat16
+    code = _lib.dtype_code(dtype)
+    D = lib.pr_expanded_dim(d, 2)
+    g = torch.Generator().manual_seed(11)
+    S0 = (torch.randn(B, h, D, d, generator=g) * 0.3).to(dtype).to(DEV)
+    s0 = (torch.rand(B, h, D, generator=g) + 0.5).to(DEV)
+    Q = torch.randn(B, 1, h * r, d, generator=g).to(dtype).to(DEV)
+    K, V = (torch.randn(B, h, d, generator=g).to(dtype).to(DEV) for _ in range(2))
+    lg = torch.nn.functional.logsigmoid(torch.randn(B, h, generator=g)).to(DEV)
+
+    def step(S, s, out, stream, noalloc):
+        head = (p(Q), p(lg), p(S), p(s), None, None, None, p(K), p(V), p(lg), p(S), p(s), p(out))
+        tail = (B, 1, h, r, d, 1.0 / d, 2, code, 1, stream)
+        if noalloc:
+            _lib.check(lib.pr_decode_step_noalloc(*head, *tail), "decode_step_noalloc")
+        else:
+            ws = torch.empty(lib.pr_decode_step_workspace(B, 1, h, r, d), dtype=torch.uint8, device=DEV)
+            _lib.check(lib.pr_decode_step(*head, p(ws), *tail), "decode_step")
+
+    # eager trajectory of three steps with the workspace form
+    S, s = S0.clone(), s0.clone()
+    want = []
+    for _ in range(3):
+        out = torch.empty_like(Q)
+        step(S, s, out, _lib.stream(), False)
+        torch.cuda.synchronize()
+        want.append((out.clone(), S.clone(), s.clone()))
+
+    Sg, sg, outg = S0.clone(), s0.clone(), torch.empty_like(Q)
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step(Sg, sg, outg, side.cuda_stream, True)   # warm-up on the capture stream
+        torch.cuda.synchronize()
+        Sg.copy_(S0)
+        sg.copy_(s0)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    with torch.cuda.graph(graph):
+        step(Sg, sg, outg, torch.cuda.current_stream().cuda_stream, True)
+    for k in range(3):
+        graph.replay()
+        torch.cuda.synchronize()
+        (torch.ones(1024, device=DEV) * 2).sum().item()   # eager work and a synchronisation between the replays
+        assert torch.equal(outg, want[k][0]), f"replay {k}: out differs"
+        assert torch.equal(Sg, want[k][1]) and torch.equal(sg, want[k][2]), f"replay {k}: state differs"
