@@ -102,8 +102,12 @@ def test_cache_layer_bookkeeping(cpu_cache):
     assert cache.get_seq_length() == 0 and not cache.has_state and float(cache.state.abs().sum()) == 0.0
 
 
-def test_cache_layer_refuses_more_than_eight_query_heads_per_kv_head(monkeypatch):
+def test_cache_layer_takes_wide_query_groups_and_refuses_ragged_ones(monkeypatch):
+    """Up to 16 query heads per kv head use the single-pass decode kernel, wider groups the operator chain (the
+    reference's own lists go to 16: perf/tests/test_list.py:189-218); a head count that is no multiple is refused."""
     from retention_integration_amd import _lib
     monkeypatch.setattr(_lib, "load", lambda: _RecordingLibrary())
+    assert pra.RetentionCache(batch=1, kv_heads=1, head_dim=32, capacity=4, device="cpu", q_heads=16)._fused_step
+    assert not pra.RetentionCache(batch=1, kv_heads=1, head_dim=32, capacity=4, device="cpu", q_heads=24)._fused_step
     with pytest.raises(AssertionError):
-        pra.RetentionCache(batch=1, kv_heads=1, head_dim=32, capacity=4, device="cpu", q_heads=16)
+        pra.RetentionCache(batch=1, kv_heads=2, head_dim=32, capacity=4, device="cpu", q_heads=5)
