@@ -250,7 +250,7 @@ class KernelTimers:
         self._t0 = None
 
         def hook(name, phase, stream, user):
-            assert stream == torch.cuda.current_stream().cuda_stream, "kernel launched on another stream than torch's"
+            assert (stream or 0) == torch.cuda.current_stream().cuda_stream, "kernel launched on another stream than torch's"
             ev = torch.cuda.Event(enable_timing=True)
             ev.record()
             if phase == 0:
@@ -567,6 +567,26 @@ def main():
     if not args.no_decode:
         with torch.no_grad():
             out["decode"] = decode_bench(pra, dev)
+    # chunked prefill: the forward of the same sequence in one call and in two calls that hand the state over
+    # (initial_state / return_final_state), each timed like the breakdown entries (HIP events after a lead-in)
+    with torch.no_grad():
+        half = cfg["t"] // 2
+        dq, dk, dv, dg = detach
+
+        def one_call():
+            return pra.power_retention(dq, dk, dv, dg, deg=cfg["deg"], chunk_size=cfg["chunk"])
+
+        def two_calls():
+            y1, st = pra.power_retention(dq[:, :half], dk[:, :half], dv[:, :half], dg[:, :half], deg=cfg["deg"],
+                                         chunk_size=cfg["chunk"], return_final_state=True)
+            y2 = pra.power_retention(dq[:, half:], dk[:, half:], dv[:, half:], dg[:, half:], deg=cfg["deg"],
+                                     chunk_size=cfg["chunk"], initial_state=st)
+            return y1, y2
+        t1, t2 = event_time_ms(one_call, 10), event_time_ms(two_calls, 10)
+        out["state_across_calls"] = {"forward_one_call_ms": round(t1, 4), "forward_two_calls_ms": round(t2, 4),
+                                     "ratio": round(t2 / t1, 4),
+                                     "workload": "forward only, the headline sequence whole vs as two halves chained "
+                                                 "through (state, sum_of_keys)"}
     if not args.no_short_chunks:
         torch.cuda.empty_cache()
         sc = short_chunks(pra, dev, 5, 2)

@@ -37,9 +37,12 @@ template <typename V> __device__ __forceinline__ void store_streaming(const V& v
   if constexpr (sizeof(V) == 16) __builtin_nontemporal_store(v, p); else *p = v;
 }
 
+// Y0 [B, H, F] or null: the scan starts from it instead of zero (Y[0] = Y0).  Yfin [B, H, F] or null: receives entry n
+// of the scan when the tensor itself keeps only n entries (n_out == n).
 template <typename T, int AHEAD, int BYTES>
 __device__ __forceinline__ void discumsum_fwd_body(const T* __restrict__ X, const float* __restrict__ logG,
-                                                   T* __restrict__ Y, int n, int n_out, int H, long F, int block) {
+                                                   T* __restrict__ Y, int n, int n_out, int H, long F, int block,
+                                                   const T* __restrict__ Y0 = nullptr, T* __restrict__ Yfin = nullptr) {
   constexpr int N = Pack16<T, BYTES>::N;
   typedef typename Pack16<T, BYTES>::type vec;
   const long per_bh = F / N;
@@ -58,9 +61,15 @@ __device__ __forceinline__ void discumsum_fwd_body(const T* __restrict__ X, cons
   vec zero;
 #pragma unroll
   for (int i = 0; i < N; i++) zero[i] = (T)0.f;
+  if (Y0) {
+    zero = *((const vec*)(Y0 + (long)bh * F) + idx);
+#pragma unroll
+    for (int i = 0; i < N; i++) st[i] = to_f32(zero[i]);
+  }
   y[0] = zero;
+  vec* yfin = Yfin ? (vec*)(Yfin + (long)bh * F) + idx : nullptr;
 
-  const int steps = n_out - 1;  // chunks that are consumed
+  const int steps = (Yfin && n_out == n) ? n : n_out - 1;  // chunks that are consumed
   vec buf[AHEAD];
 #pragma unroll
   for (int a = 0; a < AHEAD; a++)
@@ -72,14 +81,15 @@ __device__ __forceinline__ void discumsum_fwd_body(const T* __restrict__ X, cons
       if (k < steps) {
         const vec cur = buf[a];
         if (k + AHEAD < steps) buf[a] = load_streaming(&x[(long)(k + AHEAD) * xs]);
-        const float g = (k == 0) ? 0.f : __expf(lg[(long)k * H]);
+        const float g = (k == 0 && !Y0) ? 0.f : __expf(lg[(long)k * H]);
         vec o;
 #pragma unroll
         for (int i = 0; i < N; i++) {
           st[i] = st[i] * g + to_f32(cur[i]);
           o[i] = (T)st[i];
         }
-        store_streaming(o, &y[(long)(k + 1) * xs]);
+        if (k + 1 < n_out) store_streaming(o, &y[(long)(k + 1) * xs]);
+        else *yfin = o;
       }
     }
   }
@@ -97,20 +107,28 @@ template <typename T, int AHEAD>
 __global__ __launch_bounds__(256) void discumsum_pair_fwd_kernel(const T* __restrict__ X, const float* __restrict__ X2,
                                                                  const float* __restrict__ logG, T* __restrict__ Y,
                                                                  float* __restrict__ Y2, int n, int n_out, int H,
-                                                                 long F, long F2, int nblk) {
-  if ((int)blockIdx.x < nblk) discumsum_fwd_body<T, AHEAD, 16>(X, logG, Y, n, n_out, H, F, blockIdx.x);
-  else discumsum_fwd_body<float, 64, 4>(X2, logG, Y2, n, n_out, H, F2, blockIdx.x - nblk);
+                                                                 long F, long F2, int nblk, const T* __restrict__ Y0,
+                                                                 const float* __restrict__ Y02, T* __restrict__ Yfin,
+                                                                 float* __restrict__ Yfin2) {
+  if ((int)blockIdx.x < nblk) discumsum_fwd_body<T, AHEAD, 16>(X, logG, Y, n, n_out, H, F, blockIdx.x, Y0, Yfin);
+  else discumsum_fwd_body<float, 64, 4>(X2, logG, Y2, n, n_out, H, F2, blockIdx.x - nblk, Y02, Yfin2);
 }
 
 // Reverse scan: r_k = dY[k+1] + exp(log_G[k+1]) * r_{k+1};  dX[k] = r_k;
 // dlog_G[k] = exp(log_G[k]) * sum_F Y[k] * r_k, written as one partial per wave (summed by
 // discumsum_reduce_kernel in a fixed order, so the result is deterministic).
 // partial layout: [BH][n][waves_per_bh]
+// dYfin [B, H, F] or null: the gradient of entry n when the tensors keep only n entries (the forward's Yfin).
+// dY0 [B, H, F] or null: receives the gradient of the scan's starting value, dY[0] + exp(log_G[0]) * r_0.
+// wdim: 0, or the head dim of a compact state tensor whose rows of `relems` elements stand for one or two entries of
+// the full layout (common.h): the gate gradient then counts every row by its weight.
 template <typename T, int AHEAD, int BYTES>
 __device__ __forceinline__ void discumsum_bwd_body(const T* __restrict__ dY, const T* __restrict__ Y,
                                                    const float* __restrict__ logG, T* __restrict__ dX,
                                                    float* __restrict__ partial, int n, int n_out, int H, long F,
-                                                   int waves_per_bh, int block, int wave0) {
+                                                   int waves_per_bh, int block, int wave0,
+                                                   const T* __restrict__ dYfin = nullptr, T* __restrict__ dY0 = nullptr,
+                                                   int wdim = 0, int relems = 1) {
   constexpr int N = Pack16<T, BYTES>::N;
   typedef typename Pack16<T, BYTES>::type vec;
   const long per_bh = F / N;
@@ -133,6 +151,8 @@ __device__ __forceinline__ void discumsum_bwd_body(const T* __restrict__ dY, con
   vec zero;
 #pragma unroll
   for (int i = 0; i < N; i++) zero[i] = (T)0.f;
+  if (dYfin) zero = *((const vec*)(dYfin + (long)bh * F) + safe);   // stands for dY[n] below
+  const float rw = wdim ? (float)compact_row_weight((int)(safe * N / relems), wdim) : 1.f;
   // step j = 0 .. n-1 handles chunk k = n-1-j; dY[k+1] exists when k+1 < n_out
   vec bd[AHEAD], by[AHEAD];
 #pragma unroll
@@ -165,11 +185,18 @@ __device__ __forceinline__ void discumsum_bwd_body(const T* __restrict__ dY, con
           dot += to_f32(yk[i]) * r[i];
         }
         if (live) dx[(long)k * xs] = o;
-        dot = wave_sum_dpp(live ? dot : 0.f);
+        dot = wave_sum_dpp(live ? dot * rw : 0.f);
         if (lane_id() == 0) part[(long)k * waves_per_bh] = dot * gk;
         g_next = gk;
       }
     }
+  }
+  if (dY0 && live) {   // r = r_0, g_next = exp(log_G[0])
+    const vec d0 = dy[0];
+    vec o;
+#pragma unroll
+    for (int i = 0; i < N; i++) o[i] = (T)(to_f32(d0[i]) + g_next * r[i]);
+    *((vec*)(dY0 + (long)bh * F) + safe) = o;
   }
 }
 
@@ -189,12 +216,16 @@ __global__ __launch_bounds__(256) void discumsum_pair_bwd_kernel(const T* __rest
                                                                  const float* __restrict__ logG, T* __restrict__ dX,
                                                                  float* __restrict__ dX2, float* __restrict__ partial,
                                                                  int n, int n_out, int H, long F, long F2, int nblk,
-                                                                 int waves_per_bh) {
+                                                                 int waves_per_bh, const T* __restrict__ dYfin,
+                                                                 const float* __restrict__ dYfin2,
+                                                                 T* __restrict__ dY0, float* __restrict__ dY02,
+                                                                 int wdim) {
   if ((int)blockIdx.x < nblk)
-    discumsum_bwd_body<T, AHEAD, 16>(dY, Y, logG, dX, partial, n, n_out, H, F, waves_per_bh, blockIdx.x, 0);
+    discumsum_bwd_body<T, AHEAD, 16>(dY, Y, logG, dX, partial, n, n_out, H, F, waves_per_bh, blockIdx.x, 0, dYfin, dY0,
+                                     wdim, wdim);
   else
     discumsum_bwd_body<float, 64, 4>(dY2, Y2, logG, dX2, partial, n, n_out, H, F2, waves_per_bh, blockIdx.x - nblk,
-                                     nblk * 4);
+                                     nblk * 4, dYfin2, dY02, wdim, 1);
 }
 
 // one wave per (bh, k): sums the waves_per_bh partials in a fixed order
@@ -260,39 +291,41 @@ static int launch_bwd(const void* dY, const void* Y, const float* logG, void* dX
 
 template <typename T>
 static int launch_pair_fwd(const void* X, const float* X2, const float* logG, void* Y, float* Y2, int B, int n,
-                           int n_out, int H, long F, long F2, hipStream_t st) {
+                           int n_out, int H, long F, long F2, const ScanCarry& cy, hipStream_t st) {
   const int nblk = (int)((F / Pack16<T>::N + 255) / 256), nblk2 = (int)((F2 + 255) / 256);
   dim3 grid((unsigned)(nblk + nblk2), (unsigned)(B * H));
   if ((F / Pack16<T>::N) * B * H < 256 * 1024)
     PR_LAUNCH("discumsum_pair_fwd", (discumsum_pair_fwd_kernel<T, 16>), grid, dim3(256), 0, st, (const T*)X, X2, logG, (T*)Y, Y2, n,
-                       n_out, H, F, F2, nblk);
+              n_out, H, F, F2, nblk, (const T*)cy.in, cy.in2, (T*)cy.out, cy.out2);
   else
     PR_LAUNCH("discumsum_pair_fwd", (discumsum_pair_fwd_kernel<T, 4>), grid, dim3(256), 0, st, (const T*)X, X2, logG, (T*)Y, Y2, n,
-                       n_out, H, F, F2, nblk);
+              n_out, H, F, F2, nblk, (const T*)cy.in, cy.in2, (T*)cy.out, cy.out2);
   return (int)hipGetLastError();
 }
 template <typename T>
 static int launch_pair_bwd(const void* dY, const void* Y, const float* dY2, const float* Y2, const float* logG,
                            void* dX, float* dX2, float* dlogG, float* partial, int B, int n, int n_out, int H, long F,
-                           long F2, hipStream_t st) {
+                           long F2, const ScanCarry& cy, hipStream_t st) {
   const int nblk = (int)((F / Pack16<T>::N + 255) / 256), nblk2 = (int)((F2 + 255) / 256);
   const int waves = (nblk + nblk2) * 4, tot = B * H * n;
   dim3 grid((unsigned)(nblk + nblk2), (unsigned)(B * H));
   if ((F / Pack16<T>::N) * B * H < 256 * 1024)
     PR_LAUNCH("discumsum_pair_bwd", (discumsum_pair_bwd_kernel<T, 8>), grid, dim3(256), 0, st, (const T*)dY, (const T*)Y, dY2, Y2,
-                       logG, (T*)dX, dX2, partial, n, n_out, H, F, F2, nblk, waves);
+              logG, (T*)dX, dX2, partial, n, n_out, H, F, F2, nblk, waves, (const T*)cy.in, cy.in2, (T*)cy.out, cy.out2,
+              cy.compact_d);
   else
     PR_LAUNCH("discumsum_pair_bwd", (discumsum_pair_bwd_kernel<T, 2>), grid, dim3(256), 0, st, (const T*)dY, (const T*)Y, dY2, Y2,
-                       logG, (T*)dX, dX2, partial, n, n_out, H, F, F2, nblk, waves);
+              logG, (T*)dX, dX2, partial, n, n_out, H, F, F2, nblk, waves, (const T*)cy.in, cy.in2, (T*)cy.out, cy.out2,
+              cy.compact_d);
   PR_LAUNCH("discumsum_reduce", discumsum_reduce_kernel, dim3((tot * 64 + 255) / 256), dim3(256), 0, st, partial, dlogG, n, H,
                      waves, B * H);
   return (int)hipGetLastError();
 }
 
 int discumsum_pair_fwd(const void* X, const float* X2, const float* logG, void* Y, float* Y2, int B, int n, int n_out,
-                       int H, long F, long F2, int dtype, hipStream_t st) {
-  if (dtype == DT_BF16) return launch_pair_fwd<bf16_t>(X, X2, logG, Y, Y2, B, n, n_out, H, F, F2, st);
-  if (dtype == DT_F16) return launch_pair_fwd<f16_t>(X, X2, logG, Y, Y2, B, n, n_out, H, F, F2, st);
+                       int H, long F, long F2, const ScanCarry& cy, int dtype, hipStream_t st) {
+  if (dtype == DT_BF16) return launch_pair_fwd<bf16_t>(X, X2, logG, Y, Y2, B, n, n_out, H, F, F2, cy, st);
+  if (dtype == DT_F16) return launch_pair_fwd<f16_t>(X, X2, logG, Y, Y2, B, n, n_out, H, F, F2, cy, st);
   return -1;
 }
 long discumsum_pair_bwd_workspace_floats(int B, int n, int H, long F, long F2) {
@@ -300,11 +333,11 @@ long discumsum_pair_bwd_workspace_floats(int B, int n, int H, long F, long F2) {
 }
 int discumsum_pair_bwd(const void* dY, const void* Y, const float* dY2, const float* Y2, const float* logG, void* dX,
                        float* dX2, float* dlogG, float* partial, int B, int n, int n_out, int H, long F, long F2,
-                       int dtype, hipStream_t st) {
+                       const ScanCarry& cy, int dtype, hipStream_t st) {
   if (dtype == DT_BF16)
-    return launch_pair_bwd<bf16_t>(dY, Y, dY2, Y2, logG, dX, dX2, dlogG, partial, B, n, n_out, H, F, F2, st);
+    return launch_pair_bwd<bf16_t>(dY, Y, dY2, Y2, logG, dX, dX2, dlogG, partial, B, n, n_out, H, F, F2, cy, st);
   if (dtype == DT_F16)
-    return launch_pair_bwd<f16_t>(dY, Y, dY2, Y2, logG, dX, dX2, dlogG, partial, B, n, n_out, H, F, F2, st);
+    return launch_pair_bwd<f16_t>(dY, Y, dY2, Y2, logG, dX, dX2, dlogG, partial, B, n, n_out, H, F, F2, cy, st);
   return -1;
 }
 

@@ -35,10 +35,65 @@ def _empty(shape, dtype, device):
     return torch.empty(shape, dtype=dtype, device=device)
 
 
+def compact_dim(d):
+    """Rows of the compact state layout (the library's pr_compact_dim): the layout of the chunk states INSIDE this node
+    when the head dim is at most 64 and the separate state kernels run -- every pair of a diagonal feature block once
+    instead of twice, 2112 rows for 2560 at d = 64.  States that enter or leave the node use the reference layout."""
+    T = d // 16
+    return 128 * T * (T - 1) + 144 * T
+
+
+_LAYOUT_MAPS = {}
+
+
+def _layout_maps(d, device):
+    """Index maps between the reference layout (ref: retention/_utils.py:18-19; D rows) and the compact one (Dc rows):
+    (a, b, c) with compact[row] = (ref[a[row]] + ref[b[row]]) / 2 -- the two orders of the row's pair, a == b where the
+    layout holds one -- and ref[f] = compact[c[f]]."""
+    key = (d, str(device))
+    if key not in _LAYOUT_MAPS:
+        T = d // 16
+        D, Dc = expanded_dim(d), compact_dim(d)
+        ia, ib, ic = [0] * Dc, [0] * Dc, [0] * D
+        for y in range(T):
+            rbase, cbase = 128 * y * (y + 1), 128 * y * (y - 1) + 144 * y
+            for k in range(256 * y):              # the blocks below the diagonal keep their order
+                ia[cbase + k] = ib[cbase + k] = rbase + k
+                ic[rbase + k] = cbase + k
+            rb, cb = rbase + 256 * y, cbase + 256 * y
+            for J in range(9):
+                for i in range(16):
+                    o = (i - J) % 16
+                    ia[cb + 16 * J + i] = rb + 16 * i + o
+                    ib[cb + 16 * J + i] = rb + 16 * (o if J < 8 else i) + (i if J < 8 else o)
+            for x in range(16):
+                for w in range(16):
+                    J = (x - w) % 16
+                    ic[rb + 16 * x + w] = cb + (16 * J + x if J <= 8 else 16 * (16 - J) + w)
+        _LAYOUT_MAPS[key] = tuple(torch.tensor(v, dtype=torch.long, device=device) for v in (ia, ib, ic))
+    return _LAYOUT_MAPS[key]
+
+
+def _to_compact(x, d, dim):
+    ia, ib, _ = _layout_maps(d, x.device)
+    return ((x.index_select(dim, ia).float() + x.index_select(dim, ib).float()) * 0.5).to(x.dtype)
+
+
+def _to_reference(x, d, dim):
+    return x.index_select(dim, _layout_maps(d, x.device)[2])
+
+
 @torch.library.custom_op("pr::chunked_fwd", mutates_args=(), device_types="cuda")
-def chunked_fwd(Q: Tensor, K: Tensor, V: Tensor, log_G: Optional[Tensor], deg: int, scale: float,
-                c: int) -> Tuple[Tensor, Tensor, Tensor, Tensor, Tensor, Tensor, Tensor, Tensor]:
-    """-> O, and what the backward needs: A, lcs, Kd (empty when ungated), Sc, sc, rowmax, den.
+def chunked_fwd(Q: Tensor, K: Tensor, V: Tensor, log_G: Optional[Tensor], deg: int, scale: float, c: int,
+                S0: Optional[Tensor] = None, s0: Optional[Tensor] = None, want_final: bool = False
+                ) -> Tuple[Tensor, Tensor, Tensor, Tensor, Tensor, Tensor, Tensor, Tensor, Tensor, Tensor]:
+    """-> O, what the backward needs: A, lcs, Kd (empty when ungated), Sc, sc, rowmax, den, and the state after the
+    last token (Sf [b,h,D,d], sf [b,h,D]; empty unless want_final).
+
+    S0 [b,h,D,d], s0 [b,h,D] fp32: the state the sequence starts from (the pair a previous call returned), in the
+    reference layout; chunk k then sees it decayed by the gates of chunks 0..k-1 like any chunk state, and the final
+    state is the scan's entry n (ref: retention/power_retention_maker.py:131-140,158-172 carries a state of the same
+    shape but returns the one at the START of the last chunk and leaves the carried one undecayed).
 
     The gated queries Q * exp(A / deg) (ref: retention/power_retention_maker.py:183-186) are never formed: the state part
     is homogeneous of degree deg in the query, so the gate is a per-row factor exp(A) on it, applied where the state
@@ -50,12 +105,16 @@ def chunked_fwd(Q: Tensor, K: Tensor, V: Tensor, log_G: Optional[Tensor], deg: i
     r = hq // h
     n = t // c
     BN = b * n
-    D = expanded_dim(d)
     dev, dt = Q.device, Q.dtype
     code = _lib.dtype_code(dt)
     f32 = torch.float32
     gated = log_G is not None
+    carried = S0 is not None
     p = _lib.ptr
+    chained = _chained(lib, b, n, c, h, 1, d) and not carried and not want_final
+    compact = d <= 64 and not chained
+    D = compact_dim(d) if compact else expanded_dim(d)
+    sym = 2 if compact else 1
 
     if gated:
         A, lcs = _empty((BN, c, h), f32, dev), _empty((BN, h), f32, dev)
@@ -69,15 +128,26 @@ def chunked_fwd(Q: Tensor, K: Tensor, V: Tensor, log_G: Optional[Tensor], deg: i
         lcs = torch.zeros((BN, h), dtype=f32, device=dev)
 
     Sc, sc = _empty((BN, h, D, d), dt, dev), _empty((BN, h, D), f32, dev)
-    if _chained(lib, b, n, c, h, 1, d):
+    Sf, sf = _empty((0,), dt, dev), _empty((0,), f32, dev)
+    if chained:
         # short chunks: the chunk states are scanned as they are formed and never written on their own
         _lib.check(lib.pr_update_state_scan_fwd(p(Kd_), p(V), p(lcs) if gated else None, p(Sc), p(sc), b, n, c, h, d,
                                                 deg, code, st), "update_state_scan_fwd")
     else:
         S, s = torch.empty_like(Sc), torch.empty_like(sc)
-        _lib.check(lib.pr_update_state_fwd(p(Kd_), p(V), p(S), p(s), BN, c, h, d, deg, n, code, st), "update_state_fwd")
-        _lib.check(lib.pr_state_scan_fwd(p(S), p(s), p(lcs), p(Sc), p(sc), b, n, n, h, D * d, D, code, st),
-                   "state_scan_fwd")
+        # (the last chunk's own state is only needed for the state after the last token)
+        _lib.check(lib.pr_update_state_fwd(p(Kd_), p(V), p(S), p(s), BN, c, h, d, deg, 0 if want_final else n,
+                                           1 if compact else 0, code, st), "update_state_fwd")
+        S0c = s0c = Sfc = sfc = None
+        if carried:
+            S0c = (_to_compact(S0, d, 2) if compact else S0).contiguous()
+            s0c = (_to_compact(s0.to(f32), d, 2) if compact else s0.to(f32)).contiguous()
+        if want_final:
+            Sfc, sfc = _empty((b, h, D, d), dt, dev), _empty((b, h, D), f32, dev)
+        _lib.check(lib.pr_state_scan_fwd(p(S), p(s), p(lcs), p(Sc), p(sc), p(S0c), p(s0c), p(Sfc), p(sfc), b, n, n, h,
+                                         D * d, D, code, st), "state_scan_fwd")
+        if want_final:
+            Sf, sf = (_to_reference(Sfc, d, 2), _to_reference(sfc, d, 2)) if compact else (Sfc, sfc)
         del S, s
 
     Ya = torch.empty_like(Q)
@@ -86,29 +156,41 @@ def chunked_fwd(Q: Tensor, K: Tensor, V: Tensor, log_G: Optional[Tensor], deg: i
                                     scale, deg, 0, code, st), "attention_fwd")
     O, den = torch.empty_like(Q), _empty((BN, c, hq), f32, dev)
     _lib.check(lib.pr_query_state_fwd(p(Q), p(Sc), p(sc), p(Ya), p(la), p(rm), p(A) if gated else None, p(O), p(den),
-                                      BN, n, c, h, r, d, scale ** deg, deg, 1, 1, code, st), "query_state_fwd")
-    return O, A, lcs, Kd, Sc, sc, rm, den
+                                      BN, n, c, h, r, d, scale ** deg, deg, 0 if carried else 1, sym, code, st),
+               "query_state_fwd")
+    return O, A, lcs, Kd, Sc, sc, rm, den, Sf, sf
 
 
 @chunked_fwd.register_fake
-def _(Q, K, V, log_G, deg, scale, c):
+def _(Q, K, V, log_G, deg, scale, c, S0=None, s0=None, want_final=False):
     b, t, hq, d = Q.shape
     h = K.shape[2]
-    BN, D = b * (t // c), expanded_dim(d)
+    BN = b * (t // c)
+    D = _state_rows(b, t // c, c, h, d, S0 is not None, want_final)
+    Dr = expanded_dim(d)
     f32 = torch.float32
     gated = log_G is not None
     A = Q.new_empty((BN, c, h) if gated else (0,), dtype=f32)
     return (torch.empty_like(Q), A, Q.new_empty((BN, h), dtype=f32),
             torch.empty_like(K) if gated else K.new_empty((0,)),
             Q.new_empty((BN, h, D, d)), Q.new_empty((BN, h, D), dtype=f32), Q.new_empty((BN, c, hq), dtype=f32),
-            Q.new_empty((BN, c, hq), dtype=f32))
+            Q.new_empty((BN, c, hq), dtype=f32),
+            Q.new_empty((b, h, Dr, d) if want_final else (0,)), Q.new_empty((b, h, Dr) if want_final else (0,), dtype=f32))
+
+
+def _state_rows(b, n, c, h, d, carried, want_final):
+    """Rows of the chunk-state tensors as the node stores them (shape inference without launching anything)."""
+    chained = _chained(_lib.load(), b, n, c, h, 1, d) and not carried and not want_final
+    return compact_dim(d) if (d <= 64 and not chained) else expanded_dim(d)
 
 
 @torch.library.custom_op("pr::chunked_bwd", mutates_args=(), device_types="cuda")
 def chunked_bwd(Q: Tensor, K: Tensor, V: Tensor, A: Tensor, lcs: Tensor, Kd: Tensor, Sc: Tensor,
                 sc: Tensor, rm: Tensor, O: Tensor, den: Tensor, dO: Tensor, deg: int, scale: float, c: int,
-                gated: bool) -> Tuple[Tensor, Tensor, Tensor, Tensor]:
-    """-> dQ, dK, dV, dlog_G (empty when ungated)."""
+                gated: bool, carried: bool = False, dSf: Optional[Tensor] = None, dsf: Optional[Tensor] = None
+                ) -> Tuple[Tensor, Tensor, Tensor, Tensor, Tensor, Tensor]:
+    """-> dQ, dK, dV, dlog_G (empty when ungated), and the gradient of the state the sequence started from
+    (dS0 [b,h,D,d], ds0 [b,h,D]; empty unless carried).  dSf, dsf: gradient of the returned final state, or None."""
     if not gated:
         Kd = K
     qgate = _lib.ptr(A) if gated else None
@@ -119,7 +201,9 @@ def chunked_bwd(Q: Tensor, K: Tensor, V: Tensor, A: Tensor, lcs: Tensor, Kd: Ten
     r = hq // h
     n = t // c
     BN = b * n
-    D = expanded_dim(d)
+    D = Sc.shape[2]
+    compact = D != expanded_dim(d)
+    sym = 2 if compact else 1
     dev, dt = Q.device, Q.dtype
     code = _lib.dtype_code(dt)
     f32, u8 = torch.float32, torch.uint8
@@ -130,7 +214,9 @@ def chunked_bwd(Q: Tensor, K: Tensor, V: Tensor, A: Tensor, lcs: Tensor, Kd: Ten
     dla, dys = torch.empty_like(den), torch.empty_like(den)
     dS, ds = torch.empty_like(Sc), torch.empty_like(sc)
     dlcs = torch.empty_like(lcs)   # gate gradient of both scans
-    if _chained(lib, b, n, c, h, r, d):
+    dS0, ds0 = _empty((0,), dt, dev), _empty((0,), f32, dev)
+    has_dfin = dSf is not None or dsf is not None
+    if not carried and not has_dfin and _chained(lib, b, n, c, h, r, d) and not compact:
         ws = _empty((lib.pr_query_state_scan_bwd_workspace(b, n, c, h, r, d, code),), u8, dev)
         _lib.check(lib.pr_query_state_scan_bwd(p(Q), p(Sc), p(sc), p(rm), qgate, p(O), p(den), p(dO),
                                                p(lcs) if gated else None, p(dQg), p(dS), p(ds), None, p(dla), p(dys),
@@ -139,18 +225,31 @@ def chunked_bwd(Q: Tensor, K: Tensor, V: Tensor, A: Tensor, lcs: Tensor, Kd: Ten
     else:
         dSc, dsc = torch.empty_like(Sc), torch.empty_like(sc)
         ws = _empty((lib.pr_query_state_bwd_workspace(BN, c, h, r, d, code),), u8, dev)
+        # (zero_initial_state: 2 = chunk 0 sees no state and nobody wants its gradient; 0 = it sees the carried one)
         _lib.check(lib.pr_query_state_bwd(p(Q), p(Sc), p(sc), p(rm), qgate, p(O), p(den), p(dO), p(dQg), p(dSc), p(dsc),
-                                          None, p(dla), p(dys), p(ws), BN, n, c, h, r, d, scale ** deg, deg, 2, 1, code,
-                                          st),
+                                          None, p(dla), p(dys), p(ws), BN, n, c, h, r, d, scale ** deg, deg,
+                                          0 if carried else 2, sym, code, st),
                    "query_state_bwd")
+        dSfc = dsfc = dS0c = ds0c = None
+        if has_dfin:
+            dSf_ = dSf if dSf is not None else torch.zeros((b, h, expanded_dim(d), d), dtype=dt, device=dev)
+            dsf_ = dsf.to(f32) if dsf is not None else torch.zeros((b, h, expanded_dim(d)), dtype=f32, device=dev)
+            dSfc = (_to_compact(dSf_, d, 2) if compact else dSf_).contiguous()
+            dsfc = (_to_compact(dsf_, d, 2) if compact else dsf_).contiguous()
+        if carried:
+            dS0c, ds0c = _empty((b, h, D, d), dt, dev), _empty((b, h, D), f32, dev)
         ws = _empty((lib.pr_state_scan_bwd_workspace(b, n, h, D * d, D),), u8, dev)
-        _lib.check(lib.pr_state_scan_bwd(p(dSc), p(Sc), p(dsc), p(sc), p(lcs), p(dS), p(ds), p(dlcs), p(ws), b, n, n, h,
-                                         D * d, D, code, st), "state_scan_bwd")
+        _lib.check(lib.pr_state_scan_bwd(p(dSc), p(Sc), p(dsc), p(sc), p(lcs), p(dS), p(ds), p(dlcs), p(ws), p(dSfc),
+                                         p(dsfc), p(dS0c), p(ds0c), d if compact else 0, b, n, n, h, D * d, D, code, st),
+                   "state_scan_bwd")
+        if carried:
+            dS0, ds0 = (_to_reference(dS0c, d, 2), _to_reference(ds0c, d, 2)) if compact else (dS0c, ds0c)
         del dSc, dsc
     dKd, dVs = torch.empty_like(K), torch.empty_like(V)
-    # (dS comes from the kernels above, so both orders of a pair hold the same sum: the symmetry flag says so)
-    _lib.check(lib.pr_update_state_bwd(p(Kd), p(V), p(dS), p(ds), p(dKd), p(dVs), BN, c, h, d, deg, 1, n, code, st),
-               "update_state_bwd")
+    # (dS comes from the kernels above, so both orders of a pair hold the same sum: the symmetry flag says so; the last
+    # chunk's dS is zero unless a gradient arrived through the final state)
+    _lib.check(lib.pr_update_state_bwd(p(Kd), p(V), p(dS), p(ds), p(dKd), p(dVs), BN, c, h, d, deg, sym,
+                                       0 if has_dfin else n, code, st), "update_state_bwd")
 
     # the attention backward adds the state-path gradients in its epilogue and writes the final dQ, dK, dV
     dQa, dKa, dVa = torch.empty_like(Q), torch.empty_like(K), torch.empty_like(V)
@@ -165,40 +264,54 @@ def chunked_bwd(Q: Tensor, K: Tensor, V: Tensor, A: Tensor, lcs: Tensor, Kd: Ten
         dlg = dGk
         _lib.check(lib.pr_chunk_gate_scan_bwd(p(dlg), p(dGq), p(dotk), p(dlcs), None, BN, c, h, r, deg, st),
                    "chunk_gate_scan_bwd")
-    return dQa, dKa, dVa, dlg
+    return dQa, dKa, dVa, dlg, dS0, ds0
 
 
 @chunked_bwd.register_fake
-def _(Q, K, V, A, lcs, Kd, Sc, sc, rm, O, den, dO, deg, scale, c, gated):
-    b, t, _, _ = Q.shape
+def _(Q, K, V, A, lcs, Kd, Sc, sc, rm, O, den, dO, deg, scale, c, gated, carried=False, dSf=None, dsf=None):
+    b, t, _, d = Q.shape
     h = K.shape[2]
+    Dr = expanded_dim(d)
     return (torch.empty_like(Q), torch.empty_like(K), torch.empty_like(V),
-            Q.new_empty((b, t, h) if gated else (0,), dtype=torch.float32))
+            Q.new_empty((b, t, h) if gated else (0,), dtype=torch.float32),
+            Q.new_empty((b, h, Dr, d) if carried else (0,)),
+            Q.new_empty((b, h, Dr) if carried else (0,), dtype=torch.float32))
 
 
 def _chunked_setup(ctx, inputs, output):
-    Q, K, V, log_G, deg, scale, c = inputs
-    O, A, lcs, Kd, Sc, sc, rm, den = output
+    Q, K, V, log_G, deg, scale, c, S0, s0, want_final = inputs
+    O, A, lcs, Kd, Sc, sc, rm, den, Sf, sf = output
     ctx.save_for_backward(Q, K, V, A, lcs, Kd, Sc, sc, rm, O, den)
-    ctx.meta = (deg, scale, c, log_G is not None)
+    ctx.meta = (deg, scale, c, log_G is not None, S0 is not None, None if s0 is None else s0.dtype, bool(want_final))
     ctx.set_materialize_grads(False)
 
 
-def _chunked_backward(ctx, dO, *unused):
+def _chunked_backward(ctx, dO, dA, dlcs, dKd, dSc, dsc, drm, dden, dSf, dsf):
     Q, K, V, A, lcs, Kd, Sc, sc, rm, O, den = ctx.saved_tensors
-    deg, scale, c, gated = ctx.meta
+    deg, scale, c, gated, carried, s0_dtype, want_final = ctx.meta
+    if not want_final:   # (the placeholders returned in place of a final state carry no gradient)
+        dSf = dsf = None
+    if dO is None and dSf is None and dsf is None:
+        return (None,) * 10
     if dO is None:
-        return None, None, None, None, None, None, None
-    dQ, dK, dV, dlg = chunked_bwd(Q, K, V, A, lcs, Kd, Sc, sc, rm, O, den, dO, deg, scale, c, gated)
-    return dQ, dK, dV, (dlg if gated else None), None, None, None
+        dO = torch.zeros_like(O)
+    dQ, dK, dV, dlg, dS0, ds0 = chunked_bwd(Q, K, V, A, lcs, Kd, Sc, sc, rm, O, den, dO, deg, scale, c, gated, carried,
+                                            dSf, dsf)
+    return (dQ, dK, dV, (dlg if gated else None), None, None, None, dS0 if carried else None,
+            ds0.to(s0_dtype) if carried else None, None)
 
 
 torch.library.register_autograd("pr::chunked_fwd", _chunked_backward, setup_context=_chunked_setup)
 
 
-def chunked_power_retention(Q, K, V, log_G, deg, scale, chunk_size):
-    """Q [b,t,hq,d], K, V [b,t,h,d] contiguous, t a multiple of chunk_size, log_G [b,t,h] fp32 or None.
-    Only deg = 2 has a state (ref: retention/_update_state/triton.py:310-311 raises the same way)."""
+def chunked_power_retention(Q, K, V, log_G, deg, scale, chunk_size, initial_state=None, return_final_state=False):
+    """Q [b,t,hq,d], K, V [b,t,h,d] contiguous, t a multiple of chunk_size, log_G [b,t,h] fp32 or None;
+    initial_state = (state [b,h,D,d], sum_of_keys [b,h,D]) or None -> out, or (out, (state, sum_of_keys)) with
+    return_final_state.  Only deg = 2 has a state (ref: retention/_update_state/triton.py:310-311 raises the same way)."""
     if deg != 2:
         raise NotImplementedError(f"the chunked algorithm needs the degree-2 state layout (got deg={deg})")
-    return chunked_fwd(Q, K, V, log_G, int(deg), float(scale), int(chunk_size))[0]
+    S0, s0 = (None, None) if initial_state is None else (initial_state[0].contiguous(), initial_state[1].contiguous())
+    out = chunked_fwd(Q, K, V, log_G, int(deg), float(scale), int(chunk_size), S0, s0, bool(return_final_state))
+    if return_final_state:
+        return out[0], (out[8], out[9])
+    return out[0]

@@ -94,9 +94,14 @@ def make_power_retention(update_state_impl, query_state_impl, discumsum_impl, at
         if deg != 2:
             raise NotImplementedError(f"the chunked algorithm needs the degree-2 state layout (got deg={deg})")
 
-        if chunked_impl is not None and not with_state:
-            return chunked_impl(Q.contiguous(), K.contiguous(), V.contiguous(),
-                                log_G.contiguous() if gated else None, deg, scale, c)
+        if chunked_impl is not None:
+            # one autograd node; a carried state enters the scan as its starting value and the state after the last
+            # token leaves it as the scan's last entry (no copy of the chunk states, no second path)
+            if not with_state:
+                return chunked_impl(Q.contiguous(), K.contiguous(), V.contiguous(),
+                                    log_G.contiguous() if gated else None, deg, scale, c)
+            return chunked_impl(Q.contiguous(), K.contiguous(), V.contiguous(), log_G.contiguous() if gated else None,
+                                deg, scale, c, initial_state, return_final_state)
 
         Qc, Kc, Vc = Q.view(b, n, c, hq, d), K.view(b, n, c, h, d), V.view(b, n, c, h, d)
         if gated:

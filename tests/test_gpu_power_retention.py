@@ -525,16 +525,25 @@ def test_decode_step_large_batch_equals_small_batches(pra, dtype, d, r, mode):
         check("oracle sum_of_keys", s2[sl], so, OUT_TOL)
 
 
-def _short_d128_case(pra, seed, chain):
-    """bf16, b=1, t=256, h=2, r=2, d=128, chunk 64, gated: errors of the HIP path and of the oracle run in bf16, both
-    against the fp32 oracle on the same inputs."""
-    from retention_integration_amd import fused
-    dtype, b, t, h, r, d, chunk = torch.bfloat16, 1, 256, 2, 2, 128, 64
+def _short_d128_inputs(seed):
+    dtype, b, t, h, r, d = torch.bfloat16, 1, 256, 2, 2, 128
     g = torch.Generator().manual_seed(seed)
     Q = torch.randn(b, t, h * r, d, generator=g).to(dtype)
     K, V = (torch.randn(b, t, h, d, generator=g).to(dtype) for _ in range(2))
     lg = torch.nn.functional.logsigmoid(torch.randn(b, t, h, generator=g))
     dO = torch.randn(b, t, h * r, d, generator=g).to(dtype)
+    return Q, K, V, lg, dO
+
+
+def _short_d128_case(pra, seed, chain, dO_mask=None):
+    """bf16, b=1, t=256, h=2, r=2, d=128, chunk 64, gated: errors of the HIP path and of the oracle run in bf16, both
+    against the fp32 oracle on the same inputs; also returns the three sets of tensors.  dO_mask [b, t, hq] zeroes the
+    output gradient of some rows in all three runs."""
+    from retention_integration_amd import fused
+    chunk = 64
+    Q, K, V, lg, dO = _short_d128_inputs(seed)
+    if dO_mask is not None:
+        dO = dO * dO_mask.unsqueeze(-1).to(dO.dtype)
     xo = [x.float().clone().requires_grad_(True) for x in (Q, K, V, lg)]
     Yo = oracle.power_retention(*xo, deg=2, chunk_size=chunk)
     Yo.backward(dO.float())
@@ -542,7 +551,8 @@ def _short_d128_case(pra, seed, chain):
     Yr = oracle.power_retention(*xr, deg=2, chunk_size=chunk)
     Yr.backward(dO)
     want = [Yo] + [x.grad for x in xo]
-    e16 = [rel_l2(a, w) for a, w in zip([Yr] + [x.grad for x in xr], want)]
+    ref16 = [Yr] + [x.grad for x in xr]
+    e16 = [rel_l2(a, w) for a, w in zip(ref16, want)]
     fused.CHAIN = chain
     try:
         xs = [x.to(DEV).requires_grad_(True) for x in (Q, K, V, lg)]
@@ -552,33 +562,64 @@ def _short_d128_case(pra, seed, chain):
         fused.CHAIN = None
     got = [Y] + [x.grad for x in xs]
     assert all(torch.isfinite(x.float()).all() for x in got)
-    return [rel_l2(a, w) for a, w in zip(got, want)], e16
+    return [rel_l2(a, w) for a, w in zip(got, want)], e16, (got, ref16, want)
+
+
+def _row_weight_totals(Q, K, lg, r):
+    """L[b, hq, i] = sum_{j <= i} (q_i . k_j / sqrt(d))^2 exp(sum of the log gates after j up to i) in fp64: the
+    normaliser of row i over its whole history (ref: retention/_attention/reference.py:42-55 without the chunking)."""
+    d = Q.shape[-1]
+    A = lg.double().cumsum(1).repeat_interleave(r, 2).permute(0, 2, 1)
+    s = torch.einsum("bihd,bjhd->bhij", Q.double(), K.double().repeat_interleave(r, 2)) / d ** 0.5
+    return torch.tril(s ** 2 * torch.exp(A[..., :, None] - A[..., None, :])).sum(-1)
 
 
 def test_short_d128_chunks_against_the_16_bit_oracle(pra):
-    """Four short chunks of a wide head, with the chained and the separate state kernels.  Every chunk's first row sees
-    one key of its own chunk, so its output is almost entirely the state part: a ratio of two cancelling sums over
-    16-bit state entries, where any 16-bit evaluation is a few per cent off and which one is off by how much is luck.
-    Averaged over seeds the HIP path must stay inside the fixed bars and be no worse than the oracle run in bf16
-    (the reference's own kind of bar, ref: perf/_checks.py:272-320); for the one seed where such a row dominates
-    (1001: the bf16 oracle itself is at 1.4-1.7e-2 on dQ, dK, dlog_G; two evaluation orders of this library land at 1.2x
-    and 2.1x of that) the bar is three times the bf16 oracle's error."""
+    """Four short chunks of a wide head, with the chained and the separate state kernels.  Averaged over seeds the HIP
+    path must stay inside the fixed bars and be no worse than the oracle run in bf16 (the reference's own kind of bar,
+    ref: perf/_checks.py:272-320).
+
+    Seed 1001 holds an ill-conditioned row: position 192 of query head 1 is the first row of its chunk, its own key
+    weighs (q.k)^2 ~ 7e-9, and the total weight of its whole history is 0.015 of the median row's -- its output is a
+    ratio of two small sums over state entries that were rounded to 16 bits once per chunk, and 1/total multiplies
+    that rounding in dQ of the row and, through the state, in dK and dlog_G of the keys it sees (the last keys of the
+    chunk before).  Measured: that one row carries 2.9e-2 of dQ's 2.95e-2 (the oracle run in bf16: 1.5e-2 of 1.6e-2)
+    and everything else is at 4e-3; the chained and the separate kernels agree to 1e-5 on it.  So the seed is checked
+    in two parts at the FIXED bars: with the output gradient of the ill-conditioned rows (total weight below 2 % of
+    the median; two of 1024 rows) zeroed in every run, all tensors; and dQ on all other rows with the full dO.  The
+    ill-conditioned rows themselves are held to three times the bf16 oracle's error on the same rows."""
     names = ["Y", "dQ", "dK", "dV", "dlog_G"]
     fixed = [OUT_TOL] + [GRAD_TOL] * 4
     for chain in (True, False):
         seeds = [2000, 2001, 2002, 2003, 2004, 2005]
         mine, ref16 = [0.0] * 5, [0.0] * 5
         for seed in seeds:
-            e, e16 = _short_d128_case(pra, seed, chain)
+            e, e16, _ = _short_d128_case(pra, seed, chain)
             mine = [a + x / len(seeds) for a, x in zip(mine, e)]
             ref16 = [a + x / len(seeds) for a, x in zip(ref16, e16)]
         for nm, a, r16, tol in zip(names, mine, ref16, fixed):
             print(f"  chain={chain} mean over seeds {nm}: {a:.3e} (bf16 oracle {r16:.3e})", flush=True)
             assert a <= tol and a <= 1.1 * r16, (nm, a, r16)
-        e, e16 = _short_d128_case(pra, 1001, chain)
-        for nm, a, r16, tol in zip(names, e, e16, fixed):
-            print(f"  chain={chain} seed 1001 {nm}: {a:.3e} (bf16 oracle {r16:.3e})", flush=True)
-            assert a <= max(tol, 3.0 * r16), (nm, a, r16)
+
+        Q, K, V, lg, _ = _short_d128_inputs(1001)
+        L = _row_weight_totals(Q, K, lg, 2)                      # [b, hq, t]
+        bad = (L < 0.02 * L.median()).permute(0, 2, 1)           # [b, t, hq]
+        assert 1 <= int(bad.sum()) <= 4, int(bad.sum())
+        e, e16, (got, r16, want) = _short_d128_case(pra, 1001, chain)
+        for nm, a, b16 in zip(names, e, e16):
+            print(f"  chain={chain} seed 1001, all rows {nm}: {a:.3e} (bf16 oracle {b16:.3e})", flush=True)
+        keep = (~bad).unsqueeze(-1).float()
+        dq, dq16, dqw = got[1].float().cpu(), r16[1].float(), want[1]
+        a = rel_l2(dq * keep, dqw * keep)
+        print(f"  chain={chain} seed 1001, dQ without the {int(bad.sum())} ill-conditioned rows: {a:.3e}", flush=True)
+        assert a <= GRAD_TOL, a
+        a, b16 = rel_l2(dq * (1 - keep), dqw * (1 - keep)), rel_l2(dq16 * (1 - keep), dqw * (1 - keep))
+        print(f"  chain={chain} seed 1001, dQ on the ill-conditioned rows: {a:.3e} (bf16 oracle {b16:.3e})", flush=True)
+        assert a <= max(GRAD_TOL, 3.0 * b16), (a, b16)
+        e, e16, _ = _short_d128_case(pra, 1001, chain, dO_mask=~bad)
+        for nm, a, b16, tol in zip(names, e, e16, fixed):
+            print(f"  chain={chain} seed 1001, dO of those rows zeroed {nm}: {a:.3e} (bf16 oracle {b16:.3e})", flush=True)
+            assert a <= tol, (nm, a, tol)
 
 
 @pytest.mark.parametrize("chunk", [32, 96])
@@ -635,6 +676,19 @@ def test_state_carried_across_calls(pra, dtype, b, t, h, r, d, chunk, gated, cut
     for nm, a, o in zip(["dQ", "dK", "dV", "dlog_G"], xs, xo):
         if a is not None:
             check(nm, a.grad, o.grad, GRAD_TOL)
+    # the same two calls through the operator composition (the carried state as one more entry in front of the chunk
+    # states, ref: retention/power_retention_maker.py:158-172): same kernels, agreement at rounding level
+    xc = [x.to(DEV).requires_grad_(True) if x is not None else None for x in (Q, K, V, lg)]
+    c1, sc1 = pra.power_retention_composed(*(sl(x, 0, cut) for x in xc), return_final_state=True, deg=2, chunk_size=chunk)
+    c2, sc2 = pra.power_retention_composed(*(sl(x, cut, t) for x in xc), initial_state=sc1, return_final_state=True,
+                                           deg=2, chunk_size=chunk)
+    torch.cat([c1, c2], 1).backward(dO.to(DEV))
+    check("fused vs composed Y", Y, torch.cat([c1, c2], 1), 6e-3)
+    check("fused vs composed final state", st2[0], sc2[0], 6e-3)
+    check("fused vs composed final sum_of_keys", st2[1], sc2[1], 6e-3)
+    for nm, a, o in zip(["dQ", "dK", "dV", "dlog_G"], xs, xc):
+        if a is not None:
+            check(f"fused vs composed {nm}", a.grad, o.grad, 8e-3)
     # and the inference function continues from the same pair
     q1 = torch.randn(b, 1, h * r, d, generator=torch.Generator().manual_seed(63)).to(dtype)
     Yi, _, _ = pra.power_retention_inference(q1.to(DEV), None, None, None, st2[0].detach(), st2[1].detach(), deg=2)
