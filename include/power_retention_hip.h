@@ -40,9 +40,8 @@ enum {
  * 3: pr_decode_step_noalloc.  4: pr_cache_append, pr_cache_attention_fwd; pr_update_state_fwd takes skip_last_of and
  * pr_update_state_bwd zero_last_of; pr_query_state_fwd / _bwd / _scan_bwd take q_log_gate and
  * pr_chunk_attention_bwd dQ_state_plain.  5: pr_query_state_fwd takes S_symmetric.  6: pr_set_launch_hook;
- * pr_decode_step takes up to 16 query rows per (batch, kv head); the compact state layout (pr_update_state_fwd
- * compact, the value 2 of S_symmetric / dS_symmetric, pr_compact_dim); pr_state_scan_fwd / _bwd connect a scan to the
- * calls before and after it (S_init, S_final and their gradients). */
+ * pr_decode_step takes up to 16 query rows per (batch, kv head); pr_state_scan_fwd / _bwd connect a scan to the calls
+ * before and after it (S_init, S_final and their gradients). */
 int pr_abi_version(void);
 const char* pr_last_error(void);
 
@@ -59,18 +58,6 @@ void pr_set_launch_hook(pr_launch_hook_t hook, void* user);
  * Replaces retention/_utils.py:18-19 compute_expanded_dim. */
 int pr_expanded_dim(int d, int deg);
 
-/* Rows of the COMPACT state layout: 128 T (T - 1) + 144 T, T = d/16 (544 / 2112 for d = 32 / 64); -1 unless d is 16, 32,
- * 48 or 64.  No counterpart in the reference.  The reference layout (retention/_utils.py:18-19) stores every product of
- * a block on the diagonal twice, (a, b) and (b, a); the compact layout keeps the blocks below the diagonal where they
- * would be if every diagonal block took 144 rows, and stores a diagonal block of strip y (first row
- * 128 y (y - 1) + 144 y + 256 y) along its cyclic diagonals: row 16 J + i, J = 0..8, holds the pair
- * (16 y + i, 16 y + (i - J) mod 16).  A compact tensor stands for the SYMMETRIC tensor of the reference layout (each row
- * is the value of both orders of its pair), which every state and state gradient of the chunked algorithm is.  It is
- * an internal format of the chunked path: pr_update_state_fwd writes it on request, the scans move it, and
- * pr_query_state_fwd / _bwd and pr_update_state_bwd read it (S_symmetric / dS_symmetric = 2); 17.5 % fewer bytes at
- * d = 64.  States that cross the API (power_retention_inference, initial / final states) use the reference layout. */
-int pr_compact_dim(int d);
-
 /* attention(Q, K, V, log_G_accum, deg, scale, norm) -- retention/_attention/reference.py:10-69,
  * Triton twin retention/_attention/triton.py:606-721 (_attn_fwd).
  *   Q [B,tq,h*r,d], K,V [B,tk,h,d], G [B,tk,h] fp32 accumulated log gate or NULL
@@ -86,7 +73,9 @@ int pr_attention_fwd(const void* Q, const void* K, const void* V, const float* G
  *   form passes dY with dO_scale = 1/l and dl = -sum(dY*Y)/l, which keeps the cancellation of rows that see
  *   a single key exact)
  *   -> dQ [B,tq,h*r,d], dK, dV [B,tk,h,d]; when G != NULL also dGq [B,tq,h*r] (sum_j dz_ij) and
- *   dGk [B,tk,h] (-sum_i dz_ij), whose sum over the aligned positions is d log_G_accum. */
+ *   dGk [B,tk,h] (-sum_i dz_ij), whose sum over the aligned positions is d log_G_accum.
+ *   The query side (dQ, dGq) and the key side (dK, dV, dGk) are separate kernels: with dQ == NULL, or with dK == dV ==
+ *   NULL, only the other side runs (two calls may then be issued on two streams). */
 int pr_attention_bwd(const void* Q, const void* K, const void* V, const float* G, const float* rowmax,
                      const void* dO, const float* dl, const float* dO_scale, void* dQ, void* dK, void* dV,
                      float* dGq, float* dGk, int B, int tq, int tk, int h, int r, int d, float scale, int deg,
@@ -96,10 +85,9 @@ int pr_attention_bwd(const void* Q, const void* K, const void* V, const float* G
  * Triton twin retention/_update_state/triton.py:61-133,280-320.
  *   K, V [BN,c,h,d] (BN = b*n chunks) -> S [BN,h,D,d], s [BN,h,D] fp32.
  *   skip_last_of = n > 0: the last of every n chunks is not computed and its S, s are left unwritten (the composed
- *   function never reads the last chunk's state, retention/power_retention_maker.py:168-170); 0 computes every chunk.
- *   compact != 0 (d <= 64): S [BN,h,Dc,d], s [BN,h,Dc] are written in the compact layout, Dc = pr_compact_dim(d). */
+ *   function never reads the last chunk's state, retention/power_retention_maker.py:168-170); 0 computes every chunk. */
 int pr_update_state_fwd(const void* K, const void* V, void* S, float* s, int BN, int c, int h, int d, int deg,
-                        int skip_last_of, int compact, int dtype, void* stream);
+                        int skip_last_of, int dtype, void* stream);
 
 /* Backward -- retention/_update_state/reference.py:55-83, Triton twin retention/_update_state/triton.py:148-260.
  *   dS [BN,h,D,d], ds [BN,h,D] fp32 -> dK, dV [BN,c,h,d]; one of dK, dV may be NULL (that gradient is skipped).
@@ -136,15 +124,14 @@ int pr_discumsum_bwd(const void* dY, const void* Y, const float* log_G, void* dX
  *   S_init [B,H,F], s_init [B,H,F2] or both NULL: the scans start from them (entry 0 = S_init) instead of zero;
  *   S_final, s_final or both NULL (n_out == n only): receive entry n, exp(log_G[n-1]) * entry n-1 + S[n-1].
  *   Backward: dS_final / ds_final (NULL = zero) is the gradient of that entry n, dS_init / ds_init (NULL = not wanted)
- *   receive the gradient of the starting value.  compact_d: 0, or the head dim d when the tensors are in the compact
- *   layout (F2 = pr_compact_dim(d), F = F2 * d): rows that stand for two entries count twice in the gate gradient. */
+ *   receive the gradient of the starting value. */
 int pr_state_scan_fwd(const void* S, const float* s, const float* log_G, void* S_out, float* s_out,
                       const void* S_init, const float* s_init, void* S_final, float* s_final, int B, int n,
                       int n_out, int H, int64_t F, int64_t F2, int dtype, void* stream);
 size_t pr_state_scan_bwd_workspace(int B, int n, int H, int64_t F, int64_t F2);
 int pr_state_scan_bwd(const void* dS_out, const void* S_out, const float* ds_out, const float* s_out,
                       const float* log_G, void* dS, float* ds, float* dlog_G, void* workspace, const void* dS_final,
-                      const float* ds_final, void* dS_init, float* ds_init, int compact_d, int B, int n, int n_out,
+                      const float* ds_final, void* dS_init, float* ds_init, int B, int n, int n_out,
                       int H, int64_t F, int64_t F2, int dtype, void* stream);
 
 /* Short chunks: update_state followed by the scan that keeps its first n entries
@@ -182,8 +169,7 @@ int pr_query_state_scan_bwd(const void* Q, const void* S, const float* s, const 
  *   is that of Q * exp(q_log_gate / deg): the state part is homogeneous of degree deg in the query, so the gate is a
  *   factor exp(q_log_gate) on that part of each row and is applied in the merge (exact; the reference rounds the gated
  *   copy to 16 bits first).
- *   S_symmetric = 2 (d <= 64): S [BN,h,Dc,d], s [BN,h,Dc] are in the compact layout (pr_compact_dim).
- *   S_symmetric = 1: the caller's promise that S[(a,b)] == S[(b,a)] in the blocks on the diagonal (true of every
+ *   S_symmetric != 0: the caller's promise that S[(a,b)] == S[(b,a)] in the blocks on the diagonal (true of every
  *   state made by pr_update_state_fwd and the scans): the mirrored quarter of each such block is then not read
  *   (a tenth of the state less to contract). */
 int pr_query_state_fwd(const void* Q, const void* S, const float* s, const void* Y_attn, const float* l_attn,
@@ -203,9 +189,8 @@ int pr_query_state_fwd(const void* Q, const void* S, const float* s, const void*
  *   workspace: pr_query_state_bwd_workspace() bytes (scaled dO and two fp32 row vectors).
  *   q_log_gate as in the forward: Q is then the ungated query and dQ the gradient w.r.t. it through the state part
  *   (the gate's own gradient is (Q . dQ) / deg per row, which pr_chunk_attention_bwd forms with dQ_state_plain).
- *   S_symmetric = 1: the caller's promise that S[(a,b)] == S[(b,a)] in the blocks on the diagonal (true of every
- *   state made by pr_update_state_fwd and the scans); the query gradient then takes a shorter path through them.
- *   S_symmetric = 2 (d <= 64): S, s are in the compact layout (pr_compact_dim) and dS, ds are written in it. */
+ *   S_symmetric != 0: the caller's promise that S[(a,b)] == S[(b,a)] in the blocks on the diagonal (true of every
+ *   state made by pr_update_state_fwd and the scans); the query gradient then takes a shorter path through them. */
 size_t pr_query_state_bwd_workspace(int BN, int c, int h, int r, int d, int dtype);
 int pr_query_state_bwd(const void* Q, const void* S, const float* s, const float* rowmax, const float* q_log_gate,
                        const void* O, const float* den, const void* dO, void* dQ, void* dS, float* ds, void* dY_attn,

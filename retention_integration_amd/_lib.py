@@ -26,8 +26,7 @@ SIGNATURES = {
     "pr_expanded_dim": (c_int, [_I, _I]),
     "pr_attention_fwd": (c_int, [_P] * 7 + [_I] * 6 + [_F, _I, _I, _I, _P]),
     "pr_attention_bwd": (c_int, [_P] * 13 + [_I] * 6 + [_F, _I, _I, _P]),
-    "pr_compact_dim": (c_int, [_I]),
-    "pr_update_state_fwd": (c_int, [_P] * 4 + [_I] * 8 + [_P]),
+    "pr_update_state_fwd": (c_int, [_P] * 4 + [_I] * 7 + [_P]),
     "pr_update_state_bwd": (c_int, [_P] * 6 + [_I] * 8 + [_P]),
     "pr_discumsum_fwd": (c_int, [_P] * 3 + [_I] * 4 + [c_int64, _I, _P]),
     "pr_discumsum_bwd_workspace": (c_size_t, [_I, _I, _I, c_int64, _I]),
@@ -43,7 +42,7 @@ SIGNATURES = {
     "pr_query_state_scan_bwd_workspace": (c_size_t, [_I] * 7),
     "pr_query_state_scan_bwd": (c_int, [_P] * 17 + [_I] * 6 + [_F, _I, _I, _P]),
     "pr_state_scan_bwd_workspace": (c_size_t, [_I] * 3 + [c_int64, c_int64]),
-    "pr_state_scan_bwd": (c_int, [_P] * 13 + [_I] * 5 + [c_int64, c_int64, _I, _P]),
+    "pr_state_scan_bwd": (c_int, [_P] * 13 + [_I] * 4 + [c_int64, c_int64, _I, _P]),
     "pr_chunk_attention_bwd": (c_int, [_P] * 17 + [_I] * 5 + [_F, _I, _I, _I, _P]),
     "pr_chunk_gate_scan_bwd": (c_int, [_P] * 5 + [_I] * 5 + [_P]),
     "pr_decode_step_workspace": (c_size_t, [_I] * 5),

@@ -869,8 +869,8 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
 template <typename T, int DH, bool DEG2> static int attn_bwd_launch(const AttnBwdArgs& a, int B, hipStream_t st) {
   const int npairs = B * a.h;
   // dK/dV first: its epilogue reads the state-path gradients that the kernels just before this call wrote (4 us of a
-  // training step at the headline shape against the other order)
-  {
+  // training step at the headline shape against the other order).  Either half is skipped when its outputs are null.
+  if (a.dK) {
     constexpr int MK = DH <= 64 ? 2 : 1;
     constexpr size_t smem = ab_stages(DH) * (2 * AB_BM * DH * 2 + 6 * AB_BM * 4);
     const int nblocks = (a.tk + 64 * MK - 1) / (64 * MK);
@@ -879,7 +879,7 @@ template <typename T, int DH, bool DEG2> static int attn_bwd_launch(const AttnBw
     allow_big_lds((const void*)kern, smem);
     PR_LAUNCH("attention_bwd_dkv", kern, grid, dim3(256), smem, st, a, nblocks, npairs);
   }
-  {
+  if (a.dQ) {
     constexpr int MT = DH <= 64 ? 2 : 1;
     constexpr size_t smem = ab_stages(DH) * (2 * AB_BN * DH * 2 + 4 * AB_BN * 4);
     const int rows = a.tq * a.r;

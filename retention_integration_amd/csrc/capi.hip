@@ -57,11 +57,6 @@ int pr_expanded_dim(int d, int deg) {
   return pr::expanded_dim(d);
 }
 
-int pr_compact_dim(int d) {
-  if (d != 16 && d != 32 && d != 48 && d != 64) return -1;
-  return pr::compact_dim(d);
-}
-
 int pr_attention_fwd(const void* Q, const void* K, const void* V, const float* G, void* O, float* l, float* rowmax,
                      int B, int tq, int tk, int h, int r, int d, float scale, int deg, int norm, int dtype,
                      void* stream) {
@@ -80,10 +75,13 @@ int pr_attention_bwd(const void* Q, const void* K, const void* V, const float* G
                      float* dGq, float* dGk, int B, int tq, int tk, int h, int r, int d, float scale, int deg,
                      int dtype, void* stream) {
   if (int rc = check_common("attention_bwd", d, deg, dtype, false)) return rc;
-  if (bad_ptr(Q) || bad_ptr(K) || bad_ptr(V) || bad_ptr(rowmax) || bad_ptr(dO) || bad_ptr(dQ) || bad_ptr(dK) ||
-      bad_ptr(dV) || bad_opt(G) || bad_opt(dl) || bad_opt(dGq) || bad_opt(dGk))
+  if (bad_ptr(Q) || bad_ptr(K) || bad_ptr(V) || bad_ptr(rowmax) || bad_ptr(dO) || bad_opt(dQ) || bad_opt(dK) ||
+      bad_opt(dV) || bad_opt(G) || bad_opt(dl) || bad_opt(dGq) || bad_opt(dGk))
     return fail(PR_ERR_ARG, "attention_bwd: null or misaligned pointer");
-  if (G && (!dGq || !dGk)) return fail(PR_ERR_ARG, "attention_bwd: dGq and dGk are required when G is given");
+  if ((dK == nullptr) != (dV == nullptr) || (!dQ && !dK))
+    return fail(PR_ERR_ARG, "attention_bwd: ask for dQ, for dK and dV, or for all three");
+  if (G && ((dQ && !dGq) || (dK && !dGk)))
+    return fail(PR_ERR_ARG, "attention_bwd: dGq (with dQ) and dGk (with dK, dV) are required when G is given");
   if (B <= 0 || tq <= 0 || tk <= 0 || h <= 0 || r <= 0 || tq > tk)
     return fail(PR_ERR_ARG, "attention_bwd: need B,tq,tk,h,r > 0 and tq <= tk");
   pr::AttnBwdArgs a{Q, K, V, G, rowmax, dO, dl, dO_scale, dQ, dK, dV, G ? dGq : nullptr, G ? dGk : nullptr,
@@ -97,12 +95,16 @@ int pr_chunk_attention_bwd(const void* Q, const void* K, const void* V, const fl
                            float* dGk, float* dotk, int BN, int c, int h, int r, int d, float scale, int deg,
                            int dQ_state_plain, int dtype, void* stream) {
   if (int rc = check_common("chunk_attention_bwd", d, deg, dtype, false)) return rc;
-  if (bad_ptr(Q) || bad_ptr(K) || bad_ptr(V) || bad_ptr(rowmax) || bad_ptr(dO) || bad_ptr(dQ) || bad_ptr(dK) ||
-      bad_ptr(dV) || bad_ptr(dQ_state) || bad_ptr(dK_state) || bad_ptr(dV_state) || bad_opt(A) || bad_opt(dl) ||
+  if (bad_ptr(Q) || bad_ptr(K) || bad_ptr(V) || bad_ptr(rowmax) || bad_ptr(dO) || bad_opt(dQ) || bad_opt(dK) ||
+      bad_opt(dV) || bad_opt(dQ_state) || bad_opt(dK_state) || bad_opt(dV_state) || bad_opt(A) || bad_opt(dl) ||
       bad_opt(dO_scale) || bad_opt(dGq) || bad_opt(dGk) || bad_opt(dotk))
     return fail(PR_ERR_ARG, "chunk_attention_bwd: null or misaligned pointer");
-  if (A && (!dGq || !dGk || !dotk))
-    return fail(PR_ERR_ARG, "chunk_attention_bwd: dGq, dGk and dotk are required when A is given");
+  if ((dK == nullptr) != (dV == nullptr) || (!dQ && !dK))
+    return fail(PR_ERR_ARG, "chunk_attention_bwd: ask for dQ, for dK and dV, or for all three");
+  if ((dQ && !dQ_state) || (dK && (!dK_state || !dV_state)))
+    return fail(PR_ERR_ARG, "chunk_attention_bwd: the state-path gradients of the requested outputs are required");
+  if (A && ((dQ && !dGq) || (dK && (!dGk || !dotk))))
+    return fail(PR_ERR_ARG, "chunk_attention_bwd: dGq (with dQ), dGk and dotk (with dK, dV) are required when A is given");
   if (BN <= 0 || c <= 0 || h <= 0 || r <= 0) return fail(PR_ERR_ARG, "chunk_attention_bwd: need BN,c,h,r > 0");
   pr::AttnBwdArgs a{Q, K, V, A, rowmax, dO, dl, dO_scale, dQ, dK, dV, A ? dGq : nullptr, A ? dGk : nullptr,
                     c, c, h, r, scale, (float)deg, dQ_state, dK_state, dV_state, A ? dotk : nullptr, dQ_state_plain ? 1 : 0};
@@ -110,15 +112,14 @@ int pr_chunk_attention_bwd(const void* Q, const void* K, const void* V, const fl
 }
 
 int pr_update_state_fwd(const void* K, const void* V, void* S, float* s, int BN, int c, int h, int d, int deg,
-                        int skip_last_of, int compact, int dtype, void* stream) {
+                        int skip_last_of, int dtype, void* stream) {
   if (int rc = check_common("update_state_fwd", d, deg, dtype, true)) return rc;
   if (bad_ptr(K) || bad_ptr(V) || bad_ptr(S) || bad_ptr(s)) return fail(PR_ERR_ARG, "update_state_fwd: null or misaligned pointer");
   if (BN <= 0 || c <= 0 || h <= 0) return fail(PR_ERR_ARG, "update_state_fwd: need BN,c,h > 0");
   if (skip_last_of < 0 || (skip_last_of > 0 && BN % skip_last_of != 0))
     return fail(PR_ERR_ARG, "update_state_fwd: skip_last_of must be 0 or a divisor of BN (got %d, BN %d)", skip_last_of, BN);
-  if (compact && d > 64) return fail(PR_ERR_ARG, "update_state_fwd: the compact layout exists for head dims up to 64");
-  return finish(pr::sympow_tn(K, V, nullptr, S, s, BN, c, h, 1, d, 1, skip_last_of, compact ? 1 : 0, dtype,
-                              (hipStream_t)stream), "update_state_fwd");
+  return finish(pr::sympow_tn(K, V, nullptr, S, s, BN, c, h, 1, d, 1, skip_last_of, dtype, (hipStream_t)stream),
+                "update_state_fwd");
 }
 
 int pr_update_state_bwd(const void* K, const void* V, const void* dS, const float* ds, void* dK, void* dV, int BN,
@@ -129,15 +130,13 @@ int pr_update_state_bwd(const void* K, const void* V, const void* dS, const floa
   if (BN <= 0 || c <= 0 || h <= 0) return fail(PR_ERR_ARG, "update_state_bwd: need BN,c,h > 0");
   if (zero_last_of < 0 || (zero_last_of > 0 && BN % zero_last_of != 0))
     return fail(PR_ERR_ARG, "update_state_bwd: zero_last_of must be 0 or a divisor of BN (got %d, BN %d)", zero_last_of, BN);
-  if (dS_symmetric < 0 || dS_symmetric > 2 || (dS_symmetric == 2 && d > 64))
-    return fail(PR_ERR_ARG, "update_state_bwd: dS_symmetric must be 0, 1 or (head dims up to 64) 2");
   const int nn_ = zero_last_of > 0 ? zero_last_of : 1, skl = zero_last_of > 0 ? 1 : 0;
   if (dV) {
-    pr::NNArgs nn{K, dS, nullptr, dV, nullptr, nullptr, nullptr, nullptr, 1.f, c, h, 1, nn_, 0, skl, dS_symmetric, nullptr};
+    pr::NNArgs nn{K, dS, nullptr, dV, nullptr, nullptr, nullptr, nullptr, 1.f, c, h, 1, nn_, 0, skl, dS_symmetric ? 1 : 0, nullptr};
     if (int rc = finish(pr::sympow_nn(nn, BN, d, 1, 0, dtype, (hipStream_t)stream), "update_state_bwd(dV)")) return rc;
   }
   if (!dK) return 0;
-  pr::GradArgs g{K, V, nullptr, dS, ds, dK, c, h, 1, nn_, skl ? 2 : 0, dS_symmetric};
+  pr::GradArgs g{K, V, nullptr, dS, ds, dK, c, h, 1, nn_, skl ? 2 : 0, dS_symmetric ? 1 : 0};
   return finish(pr::sympow_grad(g, BN, d, 1, dtype, (hipStream_t)stream), "update_state_bwd(dK)");
 }
 
@@ -191,7 +190,7 @@ size_t pr_state_scan_bwd_workspace(int B, int n, int H, int64_t F, int64_t F2) {
 
 int pr_state_scan_bwd(const void* dS_out, const void* S_out, const float* ds_out, const float* s_out,
                       const float* log_G, void* dS, float* ds, float* dlog_G, void* workspace, const void* dS_final,
-                      const float* ds_final, void* dS_init, float* ds_init, int compact_d, int B, int n, int n_out,
+                      const float* ds_final, void* dS_init, float* ds_init, int B, int n, int n_out,
                       int H, int64_t F, int64_t F2, int dtype, void* stream) {
   if (dtype != PR_BF16 && dtype != PR_F16) return fail(PR_ERR_DTYPE, "state_scan_bwd: unsupported dtype");
   if (bad_ptr(dS_out) || bad_ptr(S_out) || bad_ptr(ds_out) || bad_ptr(s_out) || log_G == nullptr || bad_ptr(dS) ||
@@ -203,10 +202,8 @@ int pr_state_scan_bwd(const void* dS_out, const void* S_out, const float* ds_out
       bad_opt(dS_final) || bad_opt(dS_init))
     return fail(PR_ERR_ARG, "state_scan_bwd: dS_final / ds_final and dS_init / ds_init come in pairs, 16-byte aligned");
   if (dS_final && n_out != n) return fail(PR_ERR_ARG, "state_scan_bwd: dS_final belongs to a scan that keeps n entries");
-  if (compact_d && (compact_d % 16 != 0 || F2 != pr::compact_dim(compact_d) || F != F2 * compact_d))
-    return fail(PR_ERR_ARG, "state_scan_bwd: compact_d = %d does not fit F = %ld, F2 = %ld", compact_d, (long)F, (long)F2);
   pr::ScanCarry cy;
-  cy.in = dS_final, cy.in2 = ds_final, cy.out = dS_init, cy.out2 = ds_init, cy.compact_d = compact_d;
+  cy.in = dS_final, cy.in2 = ds_final, cy.out = dS_init, cy.out2 = ds_init;
   return finish(pr::discumsum_pair_bwd(dS_out, S_out, ds_out, s_out, log_G, dS, ds, dlog_G, (float*)workspace, B, n,
                                        n_out, H, (long)F, (long)F2, cy, dtype, (hipStream_t)stream), "state_scan_bwd");
 }
@@ -224,10 +221,8 @@ int pr_query_state_fwd(const void* Q, const void* S, const float* s, const void*
   if (q_log_gate && !Y_attn) return fail(PR_ERR_ARG, "query_state_fwd: q_log_gate needs the attention part (it enters the merge)");
   if (BN <= 0 || n <= 0 || c <= 0 || h <= 0 || r <= 0 || BN % n != 0)
     return fail(PR_ERR_ARG, "query_state_fwd: need BN,n,c,h,r > 0 and BN a multiple of n");
-  if (S_symmetric < 0 || S_symmetric > 2 || (S_symmetric == 2 && d > 64))
-    return fail(PR_ERR_ARG, "query_state_fwd: S_symmetric must be 0, 1 or (head dims up to 64) 2");
   pr::NNArgs a{Q, S, s, O, den, Y_attn, l_attn, rowmax, scale_p, c, h, r, n, zero_initial_state ? 1 : 0, 0,
-               S_symmetric, q_log_gate};
+               S_symmetric ? 1 : 0, q_log_gate};
   return finish(pr::sympow_nn(a, BN, d, 0, 1, dtype, (hipStream_t)stream), "query_state_fwd");
 }
 
@@ -250,8 +245,7 @@ int pr_query_state_bwd(const void* Q, const void* S, const float* s, const float
   if (q_log_gate && !rowmax) return fail(PR_ERR_ARG, "query_state_bwd: q_log_gate needs the attention part");
   if (BN <= 0 || n <= 0 || c <= 0 || h <= 0 || r <= 0 || BN % n != 0)
     return fail(PR_ERR_ARG, "query_state_bwd: need BN,n,c,h,r > 0 and BN a multiple of n");
-  if (S_symmetric < 0 || S_symmetric > 2 || (S_symmetric == 2 && d > 64))
-    return fail(PR_ERR_ARG, "query_state_bwd: S_symmetric must be 0, 1 or (head dims up to 64) 2");
+
   const size_t rows = (size_t)BN * c * h * r;
   void* dOs = workspace;
   float* cvec = (float*)((char*)workspace + align256(rows * d * 2));
@@ -262,11 +256,10 @@ int pr_query_state_bwd(const void* Q, const void* S, const float* s, const float
                       "query_state_bwd(prep)"))
     return rc;
   // (zero_initial_state == 2: the caller does not want the gradient of the first chunk's (zero) state either)
-  if (int rc = finish(pr::sympow_tn(Q, dOs, cvec, dS, ds, BN, c, h, r, d, 0, zero_initial_state == 2 ? -n : 0,
-                                    S_symmetric == 2 ? 1 : 0, dtype, st),
+  if (int rc = finish(pr::sympow_tn(Q, dOs, cvec, dS, ds, BN, c, h, r, d, 0, zero_initial_state == 2 ? -n : 0, dtype, st),
                       "query_state_bwd(dS)"))
     return rc;
-  pr::GradArgs g{Q, dOs, cvec, S, s, dQ, c, h, r, n, zero_initial_state ? 1 : 0, S_symmetric};
+  pr::GradArgs g{Q, dOs, cvec, S, s, dQ, c, h, r, n, zero_initial_state ? 1 : 0, S_symmetric ? 1 : 0};
   return finish(pr::sympow_grad(g, BN, d, 0, dtype, st), "query_state_bwd(dQ)");
 }
 

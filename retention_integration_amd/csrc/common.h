@@ -344,34 +344,8 @@ __device__ __forceinline__ void deal_causal_blocks(int u, int nblocks, int ppg, 
 // Features are grouped in blocks of 256 = 16 x 16: block (y, xb), xb <= y, holds the products
 // k[16*xb + X] * k[16*y + i] at feature 128*y*(y+1) + 256*xb + 16*X + i.  Blocks are numbered
 // in memory order: blk = y*(y+1)/2 + xb.
-__host__ __device__ __forceinline__ int expanded_dim(int d) { return 128 * (d / 16) * (d / 16 + 1); }
+__host__ __device__ constexpr int expanded_dim(int d) { return 128 * (d / 16) * (d / 16 + 1); }
 
-// ---- compact state layout (internal to the chunked path; never seen through the operator interface) --------------
-// The layout above stores every product of a diagonal block (xb == y) twice, (a, b) and (b, a): 256 rows for 136
-// distinct pairs.  The compact layout keeps the blocks below the diagonal as they are and stores a diagonal block
-// along its cyclic diagonals, the order in which sympow_tn computes it: row 16*J + i, J = 0..8, is the pair
-// (i, (i - J) mod 16) -- 144 rows (J = 8 holds its eight pairs in both orders).  Strip y then starts at
-// 128*y*(y-1) + 144*y and D = 128*T*(T-1) + 144*T (544 / 2112 at d = 32 / 64).  A compact tensor stands for the
-// symmetric tensor of the full layout: row (J, i) is the value of BOTH entries (i, i-J) and (i-J, i), so a kernel
-// that contracts or sums over a compact tensor counts the rows with 1 <= J <= 7 twice.
-__host__ __device__ __forceinline__ int compact_dim(int d) { return 128 * (d / 16) * (d / 16 - 1) + 144 * (d / 16); }
-__host__ __device__ __forceinline__ int strip_base(int y, bool compact) {
-  return compact ? 128 * y * (y - 1) + 144 * y : 128 * y * (y + 1);
-}
-// row, inside a compact diagonal block, of the pair (x, i) (either order)
-__host__ __device__ __forceinline__ int compact_diag_row(int x, int i) {
-  const int J = (x - i) & 15;
-  return J <= 8 ? 16 * J + x : 16 * (16 - J) + i;
-}
-// how many entries of the full layout a row of the compact layout stands for (d = head dim)
-__host__ __device__ __forceinline__ int compact_row_weight(int row, int d) {
-  const int T = d / 16;
-  for (int y = 0; y < T; y++) {
-    const int r0 = strip_base(y, true) + 256 * y, r = row - r0;
-    if (r >= 0 && r < 144) return (r >= 16 && r < 128) ? 2 : 1;
-  }
-  return 1;
-}
 __device__ __forceinline__ void block_to_yx(int blk, int& y, int& xb) {
   y = 0;
   while ((y + 1) * (y + 2) / 2 <= blk) y++;

@@ -39,10 +39,23 @@ template <typename V> __device__ __forceinline__ void store_streaming(const V& v
 
 // Y0 [B, H, F] or null: the scan starts from it instead of zero (Y[0] = Y0).  Yfin [B, H, F] or null: receives entry n
 // of the scan when the tensor itself keeps only n entries (n_out == n).
+// The gate factors exp(log_G[k]) of the block's (batch, head) for all chunks, staged in LDS once per block, so that
+// the walk has no global load of its own besides the streams (and no exponential per step).
+constexpr int SCAN_MAXN = 2048;   // chunks whose gates fit the LDS table (longer scans read the gates as they go)
+__device__ __forceinline__ const float* stage_gates(float* gsh, const float* __restrict__ logG, int n, int H) {
+  if (n > SCAN_MAXN) return nullptr;
+  const int bh = blockIdx.y, b = bh / H, hh = bh % H;
+  const float* lg = logG + (long)b * n * H + hh;
+  for (int k = threadIdx.x; k < n; k += blockDim.x) gsh[k] = __expf(lg[(long)k * H]);
+  __syncthreads();
+  return gsh;
+}
+
 template <typename T, int AHEAD, int BYTES>
 __device__ __forceinline__ void discumsum_fwd_body(const T* __restrict__ X, const float* __restrict__ logG,
                                                    T* __restrict__ Y, int n, int n_out, int H, long F, int block,
-                                                   const T* __restrict__ Y0 = nullptr, T* __restrict__ Yfin = nullptr) {
+                                                   const float* gsh, const T* __restrict__ Y0 = nullptr,
+                                                   T* __restrict__ Yfin = nullptr) {
   constexpr int N = Pack16<T, BYTES>::N;
   typedef typename Pack16<T, BYTES>::type vec;
   const long per_bh = F / N;
@@ -70,35 +83,54 @@ __device__ __forceinline__ void discumsum_fwd_body(const T* __restrict__ X, cons
   vec* yfin = Yfin ? (vec*)(Yfin + (long)bh * F) + idx : nullptr;
 
   const int steps = (Yfin && n_out == n) ? n : n_out - 1;  // chunks that are consumed
+  if (steps <= 0) return;
+  // One step of the walk.  No branches inside: the loads of later chunks stay in flight across the steps only while
+  // the compiler can count them -- with a conditional load or store in the loop it waited for ALL of them at every step
+  // (vmcnt(0)); counted, the forward walk is 8 % faster at the headline shape.  (The backward walk, two input streams,
+  // measured 10 % SLOWER that way and keeps the simple loop.)
+  auto walk = [&](int k, const vec& cur) __attribute__((always_inline)) {
+    const float gk = gsh ? gsh[k] : __expf(lg[(long)k * H]);
+    const float g = (k == 0 && !Y0) ? 0.f : gk;
+    vec o;
+#pragma unroll
+    for (int i = 0; i < N; i++) {
+      st[i] = st[i] * g + to_f32(cur[i]);
+      o[i] = (T)st[i];
+    }
+    vec* dst = (k + 1 < n_out) ? &y[(long)(k + 1) * xs] : yfin;
+    store_streaming(o, dst);
+  };
   vec buf[AHEAD];
 #pragma unroll
-  for (int a = 0; a < AHEAD; a++)
-    if (a < steps) buf[a] = load_streaming(&x[(long)a * xs]);
-  for (int k0 = 0; k0 < steps; k0 += AHEAD) {
+  for (int a = 0; a < AHEAD; a++) buf[a] = load_streaming(&x[(long)min(a, steps - 1) * xs]);
+  int k0 = 0;
+  for (; k0 + 2 * AHEAD <= steps; k0 += AHEAD) {   // whole batches whose successors exist
 #pragma unroll
     for (int a = 0; a < AHEAD; a++) {
-      const int k = k0 + a;
-      if (k < steps) {
-        const vec cur = buf[a];
-        if (k + AHEAD < steps) buf[a] = load_streaming(&x[(long)(k + AHEAD) * xs]);
-        const float g = (k == 0 && !Y0) ? 0.f : __expf(lg[(long)k * H]);
-        vec o;
-#pragma unroll
-        for (int i = 0; i < N; i++) {
-          st[i] = st[i] * g + to_f32(cur[i]);
-          o[i] = (T)st[i];
-        }
-        if (k + 1 < n_out) store_streaming(o, &y[(long)(k + 1) * xs]);
-        else *yfin = o;
-      }
+      const vec cur = buf[a];
+      buf[a] = load_streaming(&x[(long)(k0 + a + AHEAD) * xs]);
+      walk(k0 + a, cur);
     }
   }
+  if (k0 + AHEAD <= steps) {   // a whole batch followed by a partial one (loads past the end repeat the last chunk)
+#pragma unroll
+    for (int a = 0; a < AHEAD; a++) {
+      const vec cur = buf[a];
+      buf[a] = load_streaming(&x[(long)min(k0 + a + AHEAD, steps - 1) * xs]);
+      walk(k0 + a, cur);
+    }
+    k0 += AHEAD;
+  }
+#pragma unroll
+  for (int a = 0; a < AHEAD; a++)
+    if (k0 + a < steps) walk(k0 + a, buf[a]);
 }
 
 template <typename T, int AHEAD, int BYTES = 16>
 __global__ __launch_bounds__(256) void discumsum_fwd_kernel(const T* __restrict__ X, const float* __restrict__ logG,
                                                             T* __restrict__ Y, int n, int n_out, int H, long F) {
-  discumsum_fwd_body<T, AHEAD, BYTES>(X, logG, Y, n, n_out, H, F, blockIdx.x);
+  __shared__ float gsh[SCAN_MAXN];
+  discumsum_fwd_body<T, AHEAD, BYTES>(X, logG, Y, n, n_out, H, F, blockIdx.x, stage_gates(gsh, logG, n, H));
 }
 // Two tensors that share their gates in one launch: a 16-bit one (16 bytes per lane) in the first nblk blocks of a
 // row of the grid, a small fp32 one (one element per lane, every chunk in flight) in the rest.  The small scan is
@@ -110,8 +142,10 @@ __global__ __launch_bounds__(256) void discumsum_pair_fwd_kernel(const T* __rest
                                                                  long F, long F2, int nblk, const T* __restrict__ Y0,
                                                                  const float* __restrict__ Y02, T* __restrict__ Yfin,
                                                                  float* __restrict__ Yfin2) {
-  if ((int)blockIdx.x < nblk) discumsum_fwd_body<T, AHEAD, 16>(X, logG, Y, n, n_out, H, F, blockIdx.x, Y0, Yfin);
-  else discumsum_fwd_body<float, 64, 4>(X2, logG, Y2, n, n_out, H, F2, blockIdx.x - nblk, Y02, Yfin2);
+  __shared__ float gsh[SCAN_MAXN];
+  const float* gs = stage_gates(gsh, logG, n, H);
+  if ((int)blockIdx.x < nblk) discumsum_fwd_body<T, AHEAD, 16>(X, logG, Y, n, n_out, H, F, blockIdx.x, gs, Y0, Yfin);
+  else discumsum_fwd_body<float, 64, 4>(X2, logG, Y2, n, n_out, H, F2, blockIdx.x - nblk, gs, Y02, Yfin2);
 }
 
 // Reverse scan: r_k = dY[k+1] + exp(log_G[k+1]) * r_{k+1};  dX[k] = r_k;
@@ -120,15 +154,12 @@ __global__ __launch_bounds__(256) void discumsum_pair_fwd_kernel(const T* __rest
 // partial layout: [BH][n][waves_per_bh]
 // dYfin [B, H, F] or null: the gradient of entry n when the tensors keep only n entries (the forward's Yfin).
 // dY0 [B, H, F] or null: receives the gradient of the scan's starting value, dY[0] + exp(log_G[0]) * r_0.
-// wdim: 0, or the head dim of a compact state tensor whose rows of `relems` elements stand for one or two entries of
-// the full layout (common.h): the gate gradient then counts every row by its weight.
 template <typename T, int AHEAD, int BYTES>
 __device__ __forceinline__ void discumsum_bwd_body(const T* __restrict__ dY, const T* __restrict__ Y,
                                                    const float* __restrict__ logG, T* __restrict__ dX,
                                                    float* __restrict__ partial, int n, int n_out, int H, long F,
-                                                   int waves_per_bh, int block, int wave0,
-                                                   const T* __restrict__ dYfin = nullptr, T* __restrict__ dY0 = nullptr,
-                                                   int wdim = 0, int relems = 1) {
+                                                   int waves_per_bh, int block, int wave0, const float* gsh,
+                                                   const T* __restrict__ dYfin = nullptr, T* __restrict__ dY0 = nullptr) {
   constexpr int N = Pack16<T, BYTES>::N;
   typedef typename Pack16<T, BYTES>::type vec;
   const long per_bh = F / N;
@@ -152,7 +183,6 @@ __device__ __forceinline__ void discumsum_bwd_body(const T* __restrict__ dY, con
 #pragma unroll
   for (int i = 0; i < N; i++) zero[i] = (T)0.f;
   if (dYfin) zero = *((const vec*)(dYfin + (long)bh * F) + safe);   // stands for dY[n] below
-  const float rw = wdim ? (float)compact_row_weight((int)(safe * N / relems), wdim) : 1.f;
   // step j = 0 .. n-1 handles chunk k = n-1-j; dY[k+1] exists when k+1 < n_out
   vec bd[AHEAD], by[AHEAD];
 #pragma unroll
@@ -175,7 +205,7 @@ __device__ __forceinline__ void discumsum_bwd_body(const T* __restrict__ dY, con
           bd[a] = load_streaming(&dy[(long)(kn + 1) * xs]);   // kn + 1 <= n - AHEAD < n_out
           by[a] = load_streaming(&y[(long)kn * xs]);
         }
-        const float gk = __expf(lg[(long)k * H]);
+        const float gk = gsh ? gsh[k] : __expf(lg[(long)k * H]);
         float dot = 0.f;
         vec o;
 #pragma unroll
@@ -185,7 +215,7 @@ __device__ __forceinline__ void discumsum_bwd_body(const T* __restrict__ dY, con
           dot += to_f32(yk[i]) * r[i];
         }
         if (live) dx[(long)k * xs] = o;
-        dot = wave_sum_dpp(live ? dot * rw : 0.f);
+        dot = wave_sum_dpp(live ? dot : 0.f);
         if (lane_id() == 0) part[(long)k * waves_per_bh] = dot * gk;
         g_next = gk;
       }
@@ -205,7 +235,9 @@ __global__ __launch_bounds__(256) void discumsum_bwd_kernel(const T* __restrict_
                                                             const float* __restrict__ logG, T* __restrict__ dX,
                                                             float* __restrict__ partial, int n, int n_out, int H,
                                                             long F, int waves_per_bh) {
-  discumsum_bwd_body<T, AHEAD, BYTES>(dY, Y, logG, dX, partial, n, n_out, H, F, waves_per_bh, blockIdx.x, 0);
+  __shared__ float gsh[SCAN_MAXN];
+  discumsum_bwd_body<T, AHEAD, BYTES>(dY, Y, logG, dX, partial, n, n_out, H, F, waves_per_bh, blockIdx.x, 0,
+                                      stage_gates(gsh, logG, n, H));
 }
 // The pair of tensors of discumsum_pair_fwd_kernel; their gate gradients land in one set of partials, so dlog_G is
 // the sum of both.
@@ -218,14 +250,15 @@ __global__ __launch_bounds__(256) void discumsum_pair_bwd_kernel(const T* __rest
                                                                  int n, int n_out, int H, long F, long F2, int nblk,
                                                                  int waves_per_bh, const T* __restrict__ dYfin,
                                                                  const float* __restrict__ dYfin2,
-                                                                 T* __restrict__ dY0, float* __restrict__ dY02,
-                                                                 int wdim) {
+                                                                 T* __restrict__ dY0, float* __restrict__ dY02) {
+  __shared__ float gsh[SCAN_MAXN];
+  const float* gs = stage_gates(gsh, logG, n, H);
   if ((int)blockIdx.x < nblk)
-    discumsum_bwd_body<T, AHEAD, 16>(dY, Y, logG, dX, partial, n, n_out, H, F, waves_per_bh, blockIdx.x, 0, dYfin, dY0,
-                                     wdim, wdim);
+    discumsum_bwd_body<T, AHEAD, 16>(dY, Y, logG, dX, partial, n, n_out, H, F, waves_per_bh, blockIdx.x, 0, gs, dYfin,
+                                     dY0);
   else
     discumsum_bwd_body<float, 64, 4>(dY2, Y2, logG, dX2, partial, n, n_out, H, F2, waves_per_bh, blockIdx.x - nblk,
-                                     nblk * 4, dYfin2, dY02, wdim, 1);
+                                     nblk * 4, gs, dYfin2, dY02);
 }
 
 // one wave per (bh, k): sums the waves_per_bh partials in a fixed order
@@ -311,12 +344,10 @@ static int launch_pair_bwd(const void* dY, const void* Y, const float* dY2, cons
   dim3 grid((unsigned)(nblk + nblk2), (unsigned)(B * H));
   if ((F / Pack16<T>::N) * B * H < 256 * 1024)
     PR_LAUNCH("discumsum_pair_bwd", (discumsum_pair_bwd_kernel<T, 8>), grid, dim3(256), 0, st, (const T*)dY, (const T*)Y, dY2, Y2,
-              logG, (T*)dX, dX2, partial, n, n_out, H, F, F2, nblk, waves, (const T*)cy.in, cy.in2, (T*)cy.out, cy.out2,
-              cy.compact_d);
+              logG, (T*)dX, dX2, partial, n, n_out, H, F, F2, nblk, waves, (const T*)cy.in, cy.in2, (T*)cy.out, cy.out2);
   else
     PR_LAUNCH("discumsum_pair_bwd", (discumsum_pair_bwd_kernel<T, 2>), grid, dim3(256), 0, st, (const T*)dY, (const T*)Y, dY2, Y2,
-              logG, (T*)dX, dX2, partial, n, n_out, H, F, F2, nblk, waves, (const T*)cy.in, cy.in2, (T*)cy.out, cy.out2,
-              cy.compact_d);
+              logG, (T*)dX, dX2, partial, n, n_out, H, F, F2, nblk, waves, (const T*)cy.in, cy.in2, (T*)cy.out, cy.out2);
   PR_LAUNCH("discumsum_reduce", discumsum_reduce_kernel, dim3((tot * 64 + 255) / 256), dim3(256), 0, st, partial, dlogG, n, H,
                      waves, B * H);
   return (int)hipGetLastError();

@@ -13,15 +13,12 @@ int discumsum_bwd(const void* dY, const void* Y, const float* logG, void* dX, fl
 // ScanCarry (all optional) connects a scan to the calls before and after it:
 //   forward:  in / in2 [B, H, F / F2]: the value the scan starts from (Y[0] = in instead of 0);
 //             out / out2: receive entry n of the scan when the tensors keep n entries (n_out == n);
-//   backward: in / in2: the gradient of that entry n;  out / out2: receive the gradient of the starting value;
-//             compact_d: head dim when the tensors are in the compact layout (rows that stand for two entries of the
-//             full layout count twice in the gate gradient), else 0.
+//   backward: in / in2: the gradient of that entry n;  out / out2: receive the gradient of the starting value.
 struct ScanCarry {
   const void* in = nullptr;
   const float* in2 = nullptr;
   void* out = nullptr;
   float* out2 = nullptr;
-  int compact_d = 0;
 };
 int discumsum_pair_fwd(const void* X, const float* X2, const float* logG, void* Y, float* Y2, int B, int n, int n_out,
                        int H, long F, long F2, const ScanCarry& cy, int dtype, hipStream_t st);
@@ -38,9 +35,8 @@ int scan_gate_grad(const void* Y, const void* R, const float* Y2, const float* R
 // sympow_tn.hip: A [BN,c,h*r,d], Bm [BN,c,h*r,d], w [BN,c,h*r] or null -> S [BN,h,D,d], s [BN,h,D]
 // skip: 0 = every chunk; +n = the last chunk of every n is not computed and its S, s are left unwritten (nobody reads
 // them); -n = the first chunk of every n is not computed and its S, s are written as zeros.
-// compact: S, s are written in the compact layout of common.h (head dims up to 64; -3 otherwise).
 int sympow_tn(const void* A, const void* Bm, const float* w, void* S, float* s, int BN, int c, int h, int r, int d,
-              int use_mult, int skip, int compact, int dtype, hipStream_t st);
+              int use_mult, int skip, int dtype, hipStream_t st);
 // The same contraction chained with the gated scan over the n chunks of a batch element (A, Bm [B,n*c,h*r,d],
 // lcs [B,n,h] or null): entry k of S, s [B*n,h,D,*] is the scan's k-th value (forward) or the scan's input gradient
 // (reverse).  sympow_tn_chain_ok: 0 = shape not supported, 1 = supported, 2 = and enough independent work to pay.
@@ -63,9 +59,8 @@ struct NNArgs {
   int c, h, r, n;       // n: chunks per batch entry
   int skip_first;       // chunk 0 of every batch entry has a zero state
   int skip_last;        // chunk n-1 of every batch entry has a zero B: the output there is zero (nothing is read)
-  int sym_diag;         // 1: B[(a, b)] == B[(b, a)] in the blocks on the diagonal (the caller's promise): the mirrored
-                        // quarter of every such block is not read;  2: B and sB are in the compact layout (common.h),
-                        // which holds such a tensor with every pair of a diagonal block once (head dims up to 64)
+  int sym_diag;         // B[(a, b)] == B[(b, a)] in the blocks on the diagonal (the caller's promise): the mirrored
+                        // quarter of every such block is not read
   const float* qgate;   // [BN, c, h] or null (merge only): log of a factor on the state part of every row of a kv head
                         // at a position -- out and den are those of X * exp(qgate / 2) without forming that product
 };
@@ -82,8 +77,7 @@ struct GradArgs {
   int c, h, r, n;
   int skip_first;     // bit 0: chunk 0 of every batch entry has a zero state, bit 1: chunk n-1 has a zero B: dX = 0
                       // there and nothing is read
-  int sym_diag;       // 1: B[(a, b)] == B[(b, a)] in the blocks on the diagonal (the caller's promise);
-                      // 2: B and sB are in the compact layout (common.h; head dims up to 64)
+  int sym_diag;       // B[(a, b)] == B[(b, a)] in the blocks on the diagonal (the caller's promise)
 };
 int sympow_grad(const GradArgs& a, int BN, int d, int mult, int dtype, hipStream_t st);
 

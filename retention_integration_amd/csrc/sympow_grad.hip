@@ -74,12 +74,10 @@ __global__ __launch_bounds__(256, (MT == 2 && DK <= 64) ? 4 : 2) void sympow_gra
   const int tid = threadIdx.x, l = tid & 63, g = l >> 4, tcol = l & 15;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int hA = a.h * a.r, rows = a.c * a.r;
-  const bool compact = SYM && a.sym_diag == 2;
-  const int Dst = compact ? compact_dim(DK) : D;   // rows of B per (chunk, head) as stored
   const T* Xg = (const T*)a.X + (long)bn * a.c * hA * DK;
   const T* Gg = (const T*)a.G + (long)bn * a.c * hA * DV;
-  const char* Bg = (const char*)((const T*)a.B + ((long)bn * a.h + hh) * Dst * DV);
-  const float* sBg = a.sB + ((long)bn * a.h + hh) * Dst;
+  const char* Bg = (const char*)((const T*)a.B + ((long)bn * a.h + hh) * D * DV);
+  const float* sBg = a.sB + ((long)bn * a.h + hh) * D;
   T* dXg = (T*)a.dX + (long)bn * a.c * hA * DK;
   auto row_off = [&](int row) -> long {
     row = min(row, rows - 1);
@@ -108,38 +106,14 @@ __global__ __launch_bounds__(256, (MT == 2 && DK <= 64) ? 4 : 2) void sympow_gra
   // (1.5 % of a training step at chunks of 128 rows; with several row blocks the tiles are shared through L2 and the
   // mark costs 10 us of a step at the headline shape).  A template parameter: as a run-time flag it cost the other
   // case 10 us through the registers and the schedule the compiler then chose.
-  // Compact layout: the blocks below the diagonal sit at other offsets, and the 64 rows of a diagonal block's stage
-  // (x columns 4 sb .. 4 sb + 3, all 16 i) are gathered from the block's 144 rows -- the row of the full layout that
-  // a lane would copy is the pair (x, i) = (row / 16, row % 16) of the block, stored at compact_diag_row.
   auto issue = [&](int step) {
     const char* src = Bg + (long)step * GR_FR * DV * 2;
-    uint32_t bo[LOADS];
-#pragma unroll
-    for (int ii = 0; ii < LOADS; ii++) bo[ii] = boffs[ii];
-    if constexpr (SYM) {
-      if (compact) {
-        constexpr int SPB = 256 / GR_FR;   // stages per block
-        int yb, xbb;
-        block_to_yx(step / SPB, yb, xbb);
-        const int sbb = step % SPB;
-        if (xbb == yb) {
-          src = Bg + (long)(strip_base(yb, true) + 256 * yb) * DV * 2;
-#pragma unroll
-          for (int ii = 0; ii < LOADS; ii++) {
-            const int rho = GR_FR * sbb + (int)(bo[ii] / (DV * 2));
-            bo[ii] = (uint32_t)(compact_diag_row(rho >> 4, rho & 15) * (DV * 2)) + bo[ii] % (DV * 2);
-          }
-        } else {
-          src = Bg + (long)(strip_base(yb, true) + 256 * xbb + GR_FR * sbb) * DV * 2;
-        }
-      }
-    }
     if constexpr (ALONE) {
 #pragma unroll
-      for (int ii = 0; ii < LOADS; ii++) async_copy16_sv_nt(src, bo[ii], ring_lds + (step % GR_NST) * STAGE + ii * 4096);
+      for (int ii = 0; ii < LOADS; ii++) async_copy16_sv_nt(src, boffs[ii], ring_lds + (step % GR_NST) * STAGE + ii * 4096);
     } else {
 #pragma unroll
-      for (int ii = 0; ii < LOADS; ii++) async_copy16_sv(src, bo[ii], ring_lds + (step % GR_NST) * STAGE + ii * 4096);
+      for (int ii = 0; ii < LOADS; ii++) async_copy16_sv(src, boffs[ii], ring_lds + (step % GR_NST) * STAGE + ii * 4096);
     }
   };
   // X rows of this workgroup (waited for together with stage 0), then the first stage(s)
@@ -308,13 +282,9 @@ __global__ __launch_bounds__(256, (MT == 2 && DK <= 64) ? 4 : 2) void sympow_gra
     for (int idx = tid; idx < DK * TT; idx += 256) {
       const int aa = idx % DK, yb = idx / DK;
       float v16[16];
-      if (SYM && compact && aa >= 16 * yb && aa < 16 * (yb + 1)) {   // a diagonal block of the compact layout
-        const float* src = sBg + strip_base(yb, true) + 256 * yb;
-#pragma unroll
-        for (int q = 0; q < 16; q++) v16[q] = src[compact_diag_row(aa - 16 * yb, q)] * OnePair<T>::down;
-      } else if (aa < 16 * (yb + 1)) {
+      if (aa < 16 * (yb + 1)) {
         const float m = ((MULT && aa < 16 * yb) ? 2.f : 1.f) * OnePair<T>::down;
-        const f32x4* src = (const f32x4*)(sBg + strip_base(yb, compact) + 16 * aa);
+        const f32x4* src = (const f32x4*)(sBg + 128 * yb * (yb + 1) + 16 * aa);
 #pragma unroll
         for (int q = 0; q < 4; q++) {
           const f32x4 t4 = src[q];

@@ -33,19 +33,14 @@ constexpr int NN_NST = 2;   // two stages keep three workgroups (12 waves) resid
 // upper half ("narrow" stage).
 template <bool MULT, bool SYM> struct FeatIter {
   int y, X0, phase, T;
-  bool compact = false;   // B is in the compact layout (SYM only): strips start elsewhere, diagonal stages are gathered
   __device__ bool narrow() const { return SYM && X0 == 16 * y + 8; }
   __device__ bool enters_diag() const { return SYM && X0 == 16 * y; }
-  __device__ bool diag() const { return X0 >= 16 * y; }
-  // first row of the stage's block when it is a diagonal one, and the stage's first row relative to it (full layout)
-  __device__ int diag_base() const { return strip_base(y, compact) + 256 * y; }
-  __device__ int diag_rel() const { return 16 * (X0 - 16 * y); }
   __device__ void init(int T_) {
     T = T_;
     if (MULT && T > 1) { phase = 0; y = 1; X0 = 0; } else { phase = MULT ? 1 : 2; y = 0; X0 = 0; }
   }
   __device__ bool done() const { return y >= T; }
-  __device__ int f0() const { return strip_base(y, compact) + 16 * X0; }
+  __device__ int f0() const { return 128 * y * (y + 1) + 16 * X0; }
   // returns true when the stage just consumed was the last one below the diagonal
   __device__ bool next() {
     X0 += narrow() ? 8 : 4;
@@ -109,11 +104,9 @@ __global__ __launch_bounds__(256, DK <= 64 ? 3 : 2) void sympow_nn_kernel(NNArgs
   const int tid = threadIdx.x, l = tid & 63, g = l >> 4, tcol = l & 15;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int hA = a.h * a.r, rows = a.c * a.r;
-  const bool compact = SYM && a.sym_diag == 2;
-  const int Dst = compact ? compact_dim(DK) : D;   // rows of B per (chunk, head) as stored
   const T* Xg = (const T*)a.X + (long)bn * a.c * hA * DK;
-  const char* Bg = (const char*)((const T*)a.B + ((long)bn * a.h + hh) * Dst * DV);
-  const float* sBg = a.sB ? a.sB + ((long)bn * a.h + hh) * Dst : nullptr;
+  const char* Bg = (const char*)((const T*)a.B + ((long)bn * a.h + hh) * D * DV);
+  const float* sBg = a.sB ? a.sB + ((long)bn * a.h + hh) * D : nullptr;
   auto row_off = [&](int row) -> long {  // element offset of a (clamped) folded row, per unit of the last dim
     row = min(row, rows - 1);
     const int t = row / a.r, rr = row - t * a.r;
@@ -144,22 +137,12 @@ __global__ __launch_bounds__(256, DK <= 64 ? 3 : 2) void sympow_nn_kernel(NNArgs
   const uint32_t ring_lds = lds_addr(ring) + wave * 1024;
   // ALONE: one row block per (chunk, head), so nobody else reads this state and its copies are marked non-temporal
   // (a template parameter: as a run-time flag it changed the registers and the schedule of the other case)
-  // (compact layout: the rows of a diagonal stage are gathered -- the row of the full layout that a lane would copy,
-  // rel + offset / row bytes inside the block, is the pair (x, i) = (row / 16, row % 16), stored at compact_diag_row)
-  auto issue = [&](const FeatIter<MULT, SYM>& it, int ringpos) {
-    const bool narrow = it.narrow(), gather = SYM && compact && it.diag();
-    const char* src = Bg + (long)(gather ? it.diag_base() : it.f0()) * DV * 2;
-    const int rel = it.diag_rel();
+  auto issue = [&](int f0, int ringpos, bool narrow) {
+    const char* src = Bg + (long)f0 * DV * 2;
 #pragma unroll
     for (int ii = 0; ii < LOADS; ii++) {
       uint32_t bo = boffs[ii];
-      if constexpr (SYM) {
-        bo = narrow ? boffs_n[ii] : bo;
-        if (gather) {
-          const int rho = rel + (int)(bo / (DV * 2));
-          bo = (uint32_t)(compact_diag_row(rho >> 4, rho & 15) * (DV * 2)) + bo % (DV * 2);
-        }
-      }
+      if constexpr (SYM) bo = narrow ? boffs_n[ii] : bo;
       if constexpr (ALONE) async_copy16_sv_nt(src, bo, ring_lds + ringpos * STAGE + ii * 4096);
       else async_copy16_sv(src, bo, ring_lds + ringpos * STAGE + ii * 4096);
     }
@@ -183,10 +166,9 @@ __global__ __launch_bounds__(256, DK <= 64 ? 3 : 2) void sympow_nn_kernel(NNArgs
     FeatIter<MULT, SYM> cur, nxt;
     cur.init(TT);
     nxt.init(TT);
-    cur.compact = nxt.compact = compact;
     int issued = 0;
     for (; issued < NN_NST - 1 && !nxt.done(); issued++) {
-      issue(nxt, issued % NN_NST);
+      issue(nxt.f0(), issued % NN_NST, nxt.narrow());
       nxt.next();
     }
     PhiRow<T> prow[MT];
@@ -224,7 +206,7 @@ __global__ __launch_bounds__(256, DK <= 64 ? 3 : 2) void sympow_nn_kernel(NNArgs
       if (issued > step + 1) wait_vmcnt<LOADS>(); else wait_vmcnt<0>();
       lds_barrier();
       if (!nxt.done()) {
-        issue(nxt, 1 - SL);
+        issue(nxt.f0(), 1 - SL, nxt.narrow());
         nxt.next();
         issued++;
       }
@@ -292,12 +274,8 @@ __global__ __launch_bounds__(256, DK <= 64 ? 3 : 2) void sympow_nn_kernel(NNArgs
         for (int idx = tid; idx < DK * TT; idx += 256) {
           const int aa = idx % DK, yb = idx / DK;
           float v16[16];
-          if (SYM && compact && aa >= 16 * yb && aa < 16 * (yb + 1)) {   // a diagonal block of the compact layout
-            const float* src = sBg + strip_base(yb, true) + 256 * yb;
-#pragma unroll
-            for (int q = 0; q < 16; q++) v16[q] = src[compact_diag_row(aa - 16 * yb, q)] * ScaleS<T>::down;
-          } else if (aa < 16 * (yb + 1)) {
-            const f32x4* src = (const f32x4*)(sBg + strip_base(yb, compact) + 16 * aa);
+          if (aa < 16 * (yb + 1)) {
+            const f32x4* src = (const f32x4*)(sBg + 128 * yb * (yb + 1) + 16 * aa);
 #pragma unroll
             for (int q = 0; q < 4; q++) {
               const f32x4 t4 = src[q];

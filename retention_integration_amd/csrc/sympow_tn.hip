@@ -76,8 +76,7 @@ constexpr int TN_NDIAG = 9;   // fragments of a diagonal block
 
 // The diagonal block's counterpart of tn_store_rows below: fragment J's row i is feature (i, i') with
 // i' = (i - J) mod 16, stored at 16 i + i' and at 16 i' + i.  S, s point at the block's first feature.
-// COMPACT: the block is stored along the cyclic diagonals themselves, row 16 J + i, every sum once (common.h).
-template <typename T, int DV, bool COMPACT>
+template <typename T, int DV>
 __device__ __forceinline__ void tn_store_diag(const f32x4 (&acc)[TN_NDIAG][DV / 16], const f32x4& sacc, uint32_t tb,
                                               T* __restrict__ S, float* __restrict__ s) {
   typedef __attribute__((address_space(3))) unsigned short lds_u16;
@@ -103,26 +102,12 @@ __device__ __forceinline__ void tn_store_diag(const f32x4 (&acc)[TN_NDIAG][DV / 
     for (int j = 0; j < DV / 32; j++) {
       const int q = j * 1024 + l * 16, i = q / (DV * 2), col = q % (DV * 2), i2 = (i - J) & 15;
       const u32x4 v = *(const lds_u32x4*)(tb + i * TP + col);
-      if constexpr (COMPACT) {
-        __builtin_nontemporal_store(v, (u32x4*)((char*)S + (16 * J + i) * (DV * 2) + col));
-      } else {
-        __builtin_nontemporal_store(v, (u32x4*)((char*)S + (16 * i + i2) * (DV * 2) + col));
-        if (J != 0 && J != 8) __builtin_nontemporal_store(v, (u32x4*)((char*)S + (16 * i2 + i) * (DV * 2) + col));
-      }
+      __builtin_nontemporal_store(v, (u32x4*)((char*)S + (16 * i + i2) * (DV * 2) + col));
+      if (J != 0 && J != 8) __builtin_nontemporal_store(v, (u32x4*)((char*)S + (16 * i2 + i) * (DV * 2) + col));
     }
     asm volatile("" ::: "memory");   // the buffer is rewritten for the next fragment
   });
-  if constexpr (COMPACT) {
-    // sacc[v] is the key sum of the pair (x = sl, i = 4g + v) -- the accumulator row is the first operand's (the
-    // strip's column i), the accumulator column the second's (column x): row (J, i), J = (i - x) mod 16, when J <= 8
-#pragma unroll
-    for (int v = 0; v < 4; v++) {
-      const int i = 4 * g + v, J = (i - sl) & 15;
-      if (J <= 8) s[16 * J + i] = sacc[v];
-    }
-  } else {
-    *(f32x4*)(s + 16 * sl + 4 * g) = sacc;
-  }
+  *(f32x4*)(s + 16 * sl + 4 * g) = sacc;
 }
 
 // Writes a wave's accumulators -- for each of its XPW x values the 16 feature rows (4g+v) x DV value columns
@@ -166,8 +151,7 @@ __device__ __forceinline__ void tn_store_rows(const f32x4 (&acc)[XPW][DV / 16], 
 template <typename T, int DK, int DV, int XPW, int PART, bool HAS_W, bool DIAG = false>
 __device__ __forceinline__ void tn_body(const T* __restrict__ A, const T* __restrict__ Bm, const float* __restrict__ w,
                                         T* __restrict__ S, float* __restrict__ s, int c, int hA, int r, int hh,
-                                        int bn, int h, int y, int xb, bool active, bool use_mult, bool compact,
-                                        char* smem) {
+                                        int bn, int h, int y, int xb, bool active, bool use_mult, char* smem) {
   typedef typename VecOf<T>::v8 v8;
   typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
   typedef __attribute__((address_space(3))) f32x4 lds_f32x4;
@@ -371,14 +355,10 @@ __device__ __forceinline__ void tn_body(const T* __restrict__ A, const T* __rest
   lds_barrier();   // every wave is done with the ring: its memory stages the stores
   if (!active) return;
   const float mul = (use_mult && xb < y) ? 2.f : 1.f;
-  const int D = compact ? compact_dim(DK) : expanded_dim(DK);
-  const long so = ((long)bn * h + hh) * D + strip_base(y, compact) + 256 * xb;
-  if constexpr (DIAG) {
-    if (compact) tn_store_diag<T, DV, true>(acc, sacc, smem_a + wave * (16 * (DV * 2 + 16)), S + so * DV, s + so);
-    else tn_store_diag<T, DV, false>(acc, sacc, smem_a + wave * (16 * (DV * 2 + 16)), S + so * DV, s + so);
-  } else {
-    tn_store_rows<T, DV, XPW, PART>(acc, sacc, mul, smem_a + wave * (16 * (DV * 2 + 16)), S + so * DV, s + so);
-  }
+  constexpr int D = 128 * (DK / 16) * (DK / 16 + 1);
+  const long so = ((long)bn * h + hh) * D + 128 * y * (y + 1) + 256 * xb;
+  if constexpr (DIAG) tn_store_diag<T, DV>(acc, sacc, smem_a + wave * (16 * (DV * 2 + 16)), S + so * DV, s + so);
+  else tn_store_rows<T, DV, XPW, PART>(acc, sacc, mul, smem_a + wave * (16 * (DV * 2 + 16)), S + so * DV, s + so);
 }
 
 // Wave tasks of a (chunk, head).  With eight x columns per wave (XPW == 8) the blocks below the block diagonal give
@@ -393,10 +373,9 @@ template <typename T, int DK, int DV, int XPW, bool HAS_W>
 __global__ __launch_bounds__(256, 2) void sympow_tn_kernel(const T* __restrict__ A, const T* __restrict__ Bm,
                                                            const float* __restrict__ w, T* __restrict__ S,
                                                            float* __restrict__ s, int c, int hA, int r, int h,
-                                                           int use_mult, int skip, int compact_i) {
+                                                           int use_mult, int skip) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   constexpr int PARTS = 16 / XPW;
-  const bool compact = XPW == 8 && compact_i != 0;   // (the compact layout exists where the cyclic-diagonal form does)
   constexpr int NB = (DK / 16) * (DK / 16 + 1) / 2;
   // Workgroups are handed to the 8 XCDs (each with its own L2) round-robin by linear id.  The workgroups of a
   // (chunk, head) read the same rows, so ids are permuted to put them on one XCD: XCD x takes the x-th eighth.
@@ -418,12 +397,12 @@ __global__ __launch_bounds__(256, 2) void sympow_tn_kernel(const T* __restrict__
   if (skip > 0 && bn % skip == skip - 1) return;
   if (skip < 0 && bn % (-skip) == 0) {
     if (!active) return;
-    const int D = compact ? compact_dim(DK) : expanded_dim(DK);
+    constexpr int D = 128 * (DK / 16) * (DK / 16 + 1);
     int f0, nf;   // the feature rows this wave owns
     if (XPW == 8 && t2 >= (DK / 16) * (DK / 16 - 1)) {
       y = t2 - (DK / 16) * (DK / 16 - 1);
-      f0 = strip_base(y, compact) + 256 * y;
-      nf = compact ? 144 : 256;
+      f0 = 128 * y * (y + 1) + 256 * y;
+      nf = 256;
     } else {
       if (XPW == 8) {
         y = 1;
@@ -432,7 +411,7 @@ __global__ __launch_bounds__(256, 2) void sympow_tn_kernel(const T* __restrict__
       } else {
         block_to_yx(t2 / PARTS, y, xb);
       }
-      f0 = strip_base(y, compact) + 256 * xb + 16 * XPW * part;
+      f0 = 128 * y * (y + 1) + 256 * xb + 16 * XPW * part;
       nf = 16 * XPW;
     }
     const long so = ((long)bn * h + hh) * D + f0;
@@ -445,8 +424,7 @@ __global__ __launch_bounds__(256, 2) void sympow_tn_kernel(const T* __restrict__
     constexpr int NOFF = (DK / 16) * (DK / 16 - 1);   // tasks below the block diagonal
     if (t2 >= NOFF) {
       y = xb = t2 - NOFF;
-      tn_body<T, DK, DV, XPW, 0, HAS_W, true>(A, Bm, w, S, s, c, hA, r, hh, bn, h, y, xb, active, use_mult != 0, compact,
-                                              smem);
+      tn_body<T, DK, DV, XPW, 0, HAS_W, true>(A, Bm, w, S, s, c, hA, r, hh, bn, h, y, xb, active, use_mult != 0, smem);
       return;
     }
     y = 1;
@@ -459,7 +437,7 @@ __global__ __launch_bounds__(256, 2) void sympow_tn_kernel(const T* __restrict__
   case P:                                                                                                              \
     if (P < PARTS)                                                                                                     \
       tn_body<T, DK, DV, XPW, (P < PARTS ? P : 0), HAS_W>(A, Bm, w, S, s, c, hA, r, hh, bn, h, y, xb, active,         \
-                                                          use_mult != 0, compact, smem);                               \
+                                                          use_mult != 0, smem);                                        \
     break;
   switch (part) {
     PR_TN_CASE(0)
@@ -736,7 +714,7 @@ int sympow_tn_chain(const void* A, const void* Bm, const float* w, const float* 
 
 template <typename T, int DK, int DV>
 static int tn_launch(const void* A, const void* Bm, const float* w, void* S, float* s, int BN, int c, int h, int r,
-                     int use_mult, int skip, int compact, hipStream_t st) {
+                     int use_mult, int skip, hipStream_t st) {
   constexpr int XPW = DV <= 64 ? 8 : 4;
   constexpr int NB = (DK / 16) * (DK / 16 + 1) / 2;
   constexpr int TASKS = tn_tasks<DK, XPW>();
@@ -746,28 +724,24 @@ static int tn_launch(const void* A, const void* Bm, const float* w, void* S, flo
   if (w) {
     auto kern = sympow_tn_kernel<T, DK, DV, XPW, true>;
     allow_big_lds((const void*)kern, smem);
-    PR_LAUNCH("sympow_tn", kern, grid, dim3(256), smem, st, (const T*)A, (const T*)Bm, w, (T*)S, s, c, h * r, r, h, use_mult, skip,
-              compact);
+    PR_LAUNCH("sympow_tn", kern, grid, dim3(256), smem, st, (const T*)A, (const T*)Bm, w, (T*)S, s, c, h * r, r, h, use_mult, skip);
   } else {
     auto kern = sympow_tn_kernel<T, DK, DV, XPW, false>;
     allow_big_lds((const void*)kern, smem);
-    PR_LAUNCH("sympow_tn", kern, grid, dim3(256), smem, st, (const T*)A, (const T*)Bm, w, (T*)S, s, c, h * r, r, h, use_mult, skip,
-              compact);
+    PR_LAUNCH("sympow_tn", kern, grid, dim3(256), smem, st, (const T*)A, (const T*)Bm, w, (T*)S, s, c, h * r, r, h, use_mult, skip);
   }
   return (int)hipGetLastError();
 }
 
 // A: [BN, c, h*r, d], Bm: [BN, c, h*r, d], w: [BN, c, h*r] or null -> S: [BN, h, D, d], s: [BN, h, D]
 // skip: 0, or +n / -n to skip the last / first chunk of every n (see the kernel)
-// compact: S, s in the compact layout (D = compact_dim(d); d <= 64 only: -3 otherwise)
 int sympow_tn(const void* A, const void* Bm, const float* w, void* S, float* s, int BN, int c, int h, int r, int d,
-              int use_mult, int skip, int compact, int dtype, hipStream_t st) {
-  if (compact && d > 64) return -3;
+              int use_mult, int skip, int dtype, hipStream_t st) {
 #define PR_TN_DISPATCH(T)                                                                                              \
   switch (d) {                                                                                                         \
-    case 32: return tn_launch<T, 32, 32>(A, Bm, w, S, s, BN, c, h, r, use_mult, skip, compact, st);                          \
-    case 64: return tn_launch<T, 64, 64>(A, Bm, w, S, s, BN, c, h, r, use_mult, skip, compact, st);                          \
-    case 128: return tn_launch<T, 128, 128>(A, Bm, w, S, s, BN, c, h, r, use_mult, skip, compact, st);                       \
+    case 32: return tn_launch<T, 32, 32>(A, Bm, w, S, s, BN, c, h, r, use_mult, skip, st);                                   \
+    case 64: return tn_launch<T, 64, 64>(A, Bm, w, S, s, BN, c, h, r, use_mult, skip, st);                                   \
+    case 128: return tn_launch<T, 128, 128>(A, Bm, w, S, s, BN, c, h, r, use_mult, skip, st);                                \
     default: return -2;                                                                                                \
   }
   if (dtype == DT_BF16) { PR_TN_DISPATCH(bf16_t) }

@@ -31,56 +31,22 @@ def _chained(lib, b, n, c, h, r, d):
     return lib.pr_state_chain_supported(b, n, c, h, r, d) >= (1 if CHAIN else 2)
 
 
+# The two kernels of the attention backward (key side, query side) read the same Q, K, V, dO of every (chunk, head) and
+# deal their workgroups to the XCDs pair by pair in the same order: launched side by side on two streams of the same
+# priority they share those rows in L2 instead of fetching them twice (12 us of a training step at the headline shape).
+ATTN_BWD_TWO_STREAMS = True
+_SIDE = {}
+
+
+def _side_stream(device):
+    key = str(device)
+    if key not in _SIDE:
+        _SIDE[key] = torch.cuda.Stream(device=device)
+    return _SIDE[key]
+
+
 def _empty(shape, dtype, device):
     return torch.empty(shape, dtype=dtype, device=device)
-
-
-def compact_dim(d):
-    """Rows of the compact state layout (the library's pr_compact_dim): the layout of the chunk states INSIDE this node
-    when the head dim is at most 64 and the separate state kernels run -- every pair of a diagonal feature block once
-    instead of twice, 2112 rows for 2560 at d = 64.  States that enter or leave the node use the reference layout."""
-    T = d // 16
-    return 128 * T * (T - 1) + 144 * T
-
-
-_LAYOUT_MAPS = {}
-
-
-def _layout_maps(d, device):
-    """Index maps between the reference layout (ref: retention/_utils.py:18-19; D rows) and the compact one (Dc rows):
-    (a, b, c) with compact[row] = (ref[a[row]] + ref[b[row]]) / 2 -- the two orders of the row's pair, a == b where the
-    layout holds one -- and ref[f] = compact[c[f]]."""
-    key = (d, str(device))
-    if key not in _LAYOUT_MAPS:
-        T = d // 16
-        D, Dc = expanded_dim(d), compact_dim(d)
-        ia, ib, ic = [0] * Dc, [0] * Dc, [0] * D
-        for y in range(T):
-            rbase, cbase = 128 * y * (y + 1), 128 * y * (y - 1) + 144 * y
-            for k in range(256 * y):              # the blocks below the diagonal keep their order
-                ia[cbase + k] = ib[cbase + k] = rbase + k
-                ic[rbase + k] = cbase + k
-            rb, cb = rbase + 256 * y, cbase + 256 * y
-            for J in range(9):
-                for i in range(16):
-                    o = (i - J) % 16
-                    ia[cb + 16 * J + i] = rb + 16 * i + o
-                    ib[cb + 16 * J + i] = rb + 16 * (o if J < 8 else i) + (i if J < 8 else o)
-            for x in range(16):
-                for w in range(16):
-                    J = (x - w) % 16
-                    ic[rb + 16 * x + w] = cb + (16 * J + x if J <= 8 else 16 * (16 - J) + w)
-        _LAYOUT_MAPS[key] = tuple(torch.tensor(v, dtype=torch.long, device=device) for v in (ia, ib, ic))
-    return _LAYOUT_MAPS[key]
-
-
-def _to_compact(x, d, dim):
-    ia, ib, _ = _layout_maps(d, x.device)
-    return ((x.index_select(dim, ia).float() + x.index_select(dim, ib).float()) * 0.5).to(x.dtype)
-
-
-def _to_reference(x, d, dim):
-    return x.index_select(dim, _layout_maps(d, x.device)[2])
 
 
 @torch.library.custom_op("pr::chunked_fwd", mutates_args=(), device_types="cuda")
@@ -112,9 +78,7 @@ def chunked_fwd(Q: Tensor, K: Tensor, V: Tensor, log_G: Optional[Tensor], deg: i
     carried = S0 is not None
     p = _lib.ptr
     chained = _chained(lib, b, n, c, h, 1, d) and not carried and not want_final
-    compact = d <= 64 and not chained
-    D = compact_dim(d) if compact else expanded_dim(d)
-    sym = 2 if compact else 1
+    D = expanded_dim(d)
 
     if gated:
         A, lcs = _empty((BN, c, h), f32, dev), _empty((BN, h), f32, dev)
@@ -136,18 +100,15 @@ def chunked_fwd(Q: Tensor, K: Tensor, V: Tensor, log_G: Optional[Tensor], deg: i
     else:
         S, s = torch.empty_like(Sc), torch.empty_like(sc)
         # (the last chunk's own state is only needed for the state after the last token)
-        _lib.check(lib.pr_update_state_fwd(p(Kd_), p(V), p(S), p(s), BN, c, h, d, deg, 0 if want_final else n,
-                                           1 if compact else 0, code, st), "update_state_fwd")
-        S0c = s0c = Sfc = sfc = None
-        if carried:
-            S0c = (_to_compact(S0, d, 2) if compact else S0).contiguous()
-            s0c = (_to_compact(s0.to(f32), d, 2) if compact else s0.to(f32)).contiguous()
+        _lib.check(lib.pr_update_state_fwd(p(Kd_), p(V), p(S), p(s), BN, c, h, d, deg, 0 if want_final else n, code, st),
+                   "update_state_fwd")
+        s0f = s0.to(f32).contiguous() if carried else None
         if want_final:
-            Sfc, sfc = _empty((b, h, D, d), dt, dev), _empty((b, h, D), f32, dev)
-        _lib.check(lib.pr_state_scan_fwd(p(S), p(s), p(lcs), p(Sc), p(sc), p(S0c), p(s0c), p(Sfc), p(sfc), b, n, n, h,
+            Sf, sf = _empty((b, h, D, d), dt, dev), _empty((b, h, D), f32, dev)
+        # the carried state is the scan's starting value, the state after the last token its entry n
+        _lib.check(lib.pr_state_scan_fwd(p(S), p(s), p(lcs), p(Sc), p(sc), p(S0) if carried else None, p(s0f),
+                                         p(Sf) if want_final else None, p(sf) if want_final else None, b, n, n, h,
                                          D * d, D, code, st), "state_scan_fwd")
-        if want_final:
-            Sf, sf = (_to_reference(Sfc, d, 2), _to_reference(sfc, d, 2)) if compact else (Sfc, sfc)
         del S, s
 
     Ya = torch.empty_like(Q)
@@ -156,7 +117,7 @@ def chunked_fwd(Q: Tensor, K: Tensor, V: Tensor, log_G: Optional[Tensor], deg: i
                                     scale, deg, 0, code, st), "attention_fwd")
     O, den = torch.empty_like(Q), _empty((BN, c, hq), f32, dev)
     _lib.check(lib.pr_query_state_fwd(p(Q), p(Sc), p(sc), p(Ya), p(la), p(rm), p(A) if gated else None, p(O), p(den),
-                                      BN, n, c, h, r, d, scale ** deg, deg, 0 if carried else 1, sym, code, st),
+                                      BN, n, c, h, r, d, scale ** deg, deg, 0 if carried else 1, 1, code, st),
                "query_state_fwd")
     return O, A, lcs, Kd, Sc, sc, rm, den, Sf, sf
 
@@ -166,8 +127,7 @@ def _(Q, K, V, log_G, deg, scale, c, S0=None, s0=None, want_final=False):
     b, t, hq, d = Q.shape
     h = K.shape[2]
     BN = b * (t // c)
-    D = _state_rows(b, t // c, c, h, d, S0 is not None, want_final)
-    Dr = expanded_dim(d)
+    D = Dr = expanded_dim(d)
     f32 = torch.float32
     gated = log_G is not None
     A = Q.new_empty((BN, c, h) if gated else (0,), dtype=f32)
@@ -176,12 +136,6 @@ def _(Q, K, V, log_G, deg, scale, c, S0=None, s0=None, want_final=False):
             Q.new_empty((BN, h, D, d)), Q.new_empty((BN, h, D), dtype=f32), Q.new_empty((BN, c, hq), dtype=f32),
             Q.new_empty((BN, c, hq), dtype=f32),
             Q.new_empty((b, h, Dr, d) if want_final else (0,)), Q.new_empty((b, h, Dr) if want_final else (0,), dtype=f32))
-
-
-def _state_rows(b, n, c, h, d, carried, want_final):
-    """Rows of the chunk-state tensors as the node stores them (shape inference without launching anything)."""
-    chained = _chained(_lib.load(), b, n, c, h, 1, d) and not carried and not want_final
-    return compact_dim(d) if (d <= 64 and not chained) else expanded_dim(d)
 
 
 @torch.library.custom_op("pr::chunked_bwd", mutates_args=(), device_types="cuda")
@@ -201,9 +155,7 @@ def chunked_bwd(Q: Tensor, K: Tensor, V: Tensor, A: Tensor, lcs: Tensor, Kd: Ten
     r = hq // h
     n = t // c
     BN = b * n
-    D = Sc.shape[2]
-    compact = D != expanded_dim(d)
-    sym = 2 if compact else 1
+    D = expanded_dim(d)
     dev, dt = Q.device, Q.dtype
     code = _lib.dtype_code(dt)
     f32, u8 = torch.float32, torch.uint8
@@ -216,7 +168,7 @@ def chunked_bwd(Q: Tensor, K: Tensor, V: Tensor, A: Tensor, lcs: Tensor, Kd: Ten
     dlcs = torch.empty_like(lcs)   # gate gradient of both scans
     dS0, ds0 = _empty((0,), dt, dev), _empty((0,), f32, dev)
     has_dfin = dSf is not None or dsf is not None
-    if not carried and not has_dfin and _chained(lib, b, n, c, h, r, d) and not compact:
+    if not carried and not has_dfin and _chained(lib, b, n, c, h, r, d):
         ws = _empty((lib.pr_query_state_scan_bwd_workspace(b, n, c, h, r, d, code),), u8, dev)
         _lib.check(lib.pr_query_state_scan_bwd(p(Q), p(Sc), p(sc), p(rm), qgate, p(O), p(den), p(dO),
                                                p(lcs) if gated else None, p(dQg), p(dS), p(ds), None, p(dla), p(dys),
@@ -228,27 +180,23 @@ def chunked_bwd(Q: Tensor, K: Tensor, V: Tensor, A: Tensor, lcs: Tensor, Kd: Ten
         # (zero_initial_state: 2 = chunk 0 sees no state and nobody wants its gradient; 0 = it sees the carried one)
         _lib.check(lib.pr_query_state_bwd(p(Q), p(Sc), p(sc), p(rm), qgate, p(O), p(den), p(dO), p(dQg), p(dSc), p(dsc),
                                           None, p(dla), p(dys), p(ws), BN, n, c, h, r, d, scale ** deg, deg,
-                                          0 if carried else 2, sym, code, st),
+                                          0 if carried else 2, 1, code, st),
                    "query_state_bwd")
-        dSfc = dsfc = dS0c = ds0c = None
-        if has_dfin:
-            dSf_ = dSf if dSf is not None else torch.zeros((b, h, expanded_dim(d), d), dtype=dt, device=dev)
-            dsf_ = dsf.to(f32) if dsf is not None else torch.zeros((b, h, expanded_dim(d)), dtype=f32, device=dev)
-            dSfc = (_to_compact(dSf_, d, 2) if compact else dSf_).contiguous()
-            dsfc = (_to_compact(dsf_, d, 2) if compact else dsf_).contiguous()
+        dSf_ = dsf_ = None
+        if has_dfin:   # the gradient that arrived through the returned final state enters the reverse scan as entry n
+            dSf_ = (dSf if dSf is not None else torch.zeros((b, h, D, d), dtype=dt, device=dev)).contiguous()
+            dsf_ = (dsf.to(f32) if dsf is not None else torch.zeros((b, h, D), dtype=f32, device=dev)).contiguous()
         if carried:
-            dS0c, ds0c = _empty((b, h, D, d), dt, dev), _empty((b, h, D), f32, dev)
+            dS0, ds0 = _empty((b, h, D, d), dt, dev), _empty((b, h, D), f32, dev)
         ws = _empty((lib.pr_state_scan_bwd_workspace(b, n, h, D * d, D),), u8, dev)
-        _lib.check(lib.pr_state_scan_bwd(p(dSc), p(Sc), p(dsc), p(sc), p(lcs), p(dS), p(ds), p(dlcs), p(ws), p(dSfc),
-                                         p(dsfc), p(dS0c), p(ds0c), d if compact else 0, b, n, n, h, D * d, D, code, st),
-                   "state_scan_bwd")
-        if carried:
-            dS0, ds0 = (_to_reference(dS0c, d, 2), _to_reference(ds0c, d, 2)) if compact else (dS0c, ds0c)
+        _lib.check(lib.pr_state_scan_bwd(p(dSc), p(Sc), p(dsc), p(sc), p(lcs), p(dS), p(ds), p(dlcs), p(ws), p(dSf_),
+                                         p(dsf_), p(dS0) if carried else None, p(ds0) if carried else None, b, n, n, h,
+                                         D * d, D, code, st), "state_scan_bwd")
         del dSc, dsc
     dKd, dVs = torch.empty_like(K), torch.empty_like(V)
     # (dS comes from the kernels above, so both orders of a pair hold the same sum: the symmetry flag says so; the last
     # chunk's dS is zero unless a gradient arrived through the final state)
-    _lib.check(lib.pr_update_state_bwd(p(Kd), p(V), p(dS), p(ds), p(dKd), p(dVs), BN, c, h, d, deg, sym,
+    _lib.check(lib.pr_update_state_bwd(p(Kd), p(V), p(dS), p(ds), p(dKd), p(dVs), BN, c, h, d, deg, 1,
                                        0 if has_dfin else n, code, st), "update_state_bwd")
 
     # the attention backward adds the state-path gradients in its epilogue and writes the final dQ, dK, dV
@@ -256,9 +204,22 @@ def chunked_bwd(Q: Tensor, K: Tensor, V: Tensor, A: Tensor, lcs: Tensor, Kd: Ten
     dGq = _empty((BN, c, hq), f32, dev) if gated else None
     dGk = _empty((b, t, h), f32, dev) if gated else None
     dotk = _empty((BN, c, h), f32, dev) if gated else None
-    _lib.check(lib.pr_chunk_attention_bwd(p(Q), p(K), p(V), p(A) if gated else None, p(rm), p(dO), p(dla), p(dys), p(dQg), p(dKd),
-                                          p(dVs), p(dQa), p(dKa), p(dVa), p(dGq), p(dGk), p(dotk), BN, c, h, r, d,
-                                          scale, deg, 1, code, st), "chunk_attention_bwd")
+    Ag = p(A) if gated else None
+    if ATTN_BWD_TWO_STREAMS:
+        # the key side on the launch stream, the query side next to it on a second stream of the same priority
+        main, side = torch.cuda.current_stream(), _side_stream(dev)
+        side.wait_stream(main)
+        _lib.check(lib.pr_chunk_attention_bwd(p(Q), p(K), p(V), Ag, p(rm), p(dO), p(dla), p(dys), None, p(dKd), p(dVs),
+                                              None, p(dKa), p(dVa), None, p(dGk), p(dotk), BN, c, h, r, d, scale, deg, 1,
+                                              code, st), "chunk_attention_bwd(dK, dV)")
+        _lib.check(lib.pr_chunk_attention_bwd(p(Q), p(K), p(V), Ag, p(rm), p(dO), p(dla), p(dys), p(dQg), None, None,
+                                              p(dQa), None, None, p(dGq), None, None, BN, c, h, r, d, scale, deg, 1,
+                                              code, side.cuda_stream), "chunk_attention_bwd(dQ)")
+        main.wait_stream(side)
+    else:
+        _lib.check(lib.pr_chunk_attention_bwd(p(Q), p(K), p(V), Ag, p(rm), p(dO), p(dla), p(dys), p(dQg), p(dKd),
+                                              p(dVs), p(dQa), p(dKa), p(dVa), p(dGq), p(dGk), p(dotk), BN, c, h, r, d,
+                                              scale, deg, 1, code, st), "chunk_attention_bwd")
     dlg = _empty((0,), f32, dev)
     if gated:
         dlg = dGk

@@ -143,7 +143,7 @@ def update_state_fwd(K: Tensor, V: Tensor) -> Tuple[Tensor, Tensor]:
     S = torch.empty((b, n, h, D, d), dtype=K.dtype, device=K.device)
     s = torch.empty((b, n, h, D), dtype=torch.float32, device=K.device)
     lib = _lib.load()
-    _lib.check(lib.pr_update_state_fwd(_lib.ptr(K), _lib.ptr(V), _lib.ptr(S), _lib.ptr(s), b * n, c, h, d, 2, 0, 0,
+    _lib.check(lib.pr_update_state_fwd(_lib.ptr(K), _lib.ptr(V), _lib.ptr(S), _lib.ptr(s), b * n, c, h, d, 2, 0,
                                        _lib.dtype_code(K.dtype), _lib.stream()), "update_state_fwd")
     return S, s
 

@@ -109,7 +109,7 @@ def test_state_scan_pair_equals_separate_scans(pra, dtype, F, n_out_extra):
     dS, ds, dlg = torch.empty_like(S), torch.empty_like(s), torch.empty_like(lg)
     ws = torch.empty(lib.pr_state_scan_bwd_workspace(b, n, h, F, F2), dtype=u8, device=DEV)
     _lib.check(lib.pr_state_scan_bwd(p(dSc), p(Sc), p(dsc), p(sc), p(lg), p(dS), p(ds), p(dlg), p(ws), None, None, None,
-                                     None, 0, b, n, n_out, h, F, F2, code, st), "pair bwd")
+                                     None, b, n, n_out, h, F, F2, code, st), "pair bwd")
     dS1, ds1, dl1, dl2 = torch.empty_like(S), torch.empty_like(s), torch.empty_like(lg), torch.empty_like(lg)
     ws1 = torch.empty(max(lib.pr_discumsum_bwd_workspace(b, n, h, F, code),
                           lib.pr_discumsum_bwd_workspace(b, n, h, F2, _lib.PR_F32)), dtype=u8, device=DEV)
@@ -363,101 +363,52 @@ def test_golden_update_state_d64_forward_and_backward():
     assert rel(dK, dKo) <= 2e-2 and rel(dV, dVo) <= 2e-2
 
 
-# ---------------------------------------------------------------- compact state layout (internal to the fused node)
-@pytest.mark.parametrize("dtype,d,c,r", [(torch.bfloat16, 64, 192, 1), (torch.float16, 32, 80, 2), (torch.bfloat16, 64, 64, 4)])
-def test_compact_state_layout_through_the_c_abi(pra, dtype, d, c, r):
-    """The compact layout holds every pair of a diagonal feature block once.  Written by pr_update_state_fwd and by the
-    dS half of pr_query_state_bwd, it must equal the reference-layout result row for row (both orders of a pair are
-    the same sum there); read by pr_query_state_fwd / _bwd and pr_update_state_bwd it must give the bits the
-    reference-layout tensors give (the kernels expand it while staging, the arithmetic is the same); and the scans'
-    gate gradient over compact tensors must equal the one over the expanded tensors."""
+# ---------------------------------------------------------------- state handed across scans
+@pytest.mark.parametrize("dtype,d", [(torch.bfloat16, 64), (torch.float16, 32)])
+def test_state_scan_with_a_starting_value_and_a_final_entry(pra, dtype, d):
+    """pr_state_scan_fwd / _bwd connected to the calls before and after (ref: retention/power_retention_maker.py:131-140,
+    158-172): the scans start from (S_init, s_init) instead of zero and hand out entry n; the backward takes the
+    gradient of that entry and hands out the gradient of the starting value.  Against the recurrence written out in
+    fp32 with autograd."""
     from retention_integration_amd import _lib
-    from retention_integration_amd.fused import _to_compact, _to_reference, compact_dim
     lib, st, p = _lib.load(), _lib.stream(), _lib.ptr
     code = _lib.dtype_code(dtype)
-    b, n, h = 2, 3, 2
-    BN, hq = b * n, h * r
-    D, Dc = oracle.expanded_dim(d), compact_dim(d)
-    assert lib.pr_compact_dim(d) == Dc
-    std = 0.5 if dtype == torch.float16 else 1.0
-    K, V = dev(rnd(BN, c, h, d, dtype=dtype, scale=std, seed=50)), dev(rnd(BN, c, h, d, dtype=dtype, scale=std, seed=51))
-    Q = dev(rnd(BN, c, hq, d, dtype=dtype, scale=std, seed=52))
+    b, n, h = 2, 5, 3
+    D = oracle.expanded_dim(d)
     f32 = torch.float32
+    S, s = rnd(b, n, h, D, d, dtype=dtype, seed=70), rnd(b, n, h, D, dtype=f32, seed=71)
+    S0, s0 = rnd(b, h, D, d, dtype=dtype, seed=72), rnd(b, h, D, dtype=f32, seed=73)
+    lg = gates(b, n, h, seed=74)
+    dY, dy = rnd(b, n, h, D, d, dtype=dtype, seed=75), rnd(b, n, h, D, dtype=f32, seed=76)
+    dYf, dyf = rnd(b, h, D, d, dtype=dtype, seed=77), rnd(b, h, D, dtype=f32, seed=78)
     E = lambda *shape, dt=dtype: torch.empty(*shape, dtype=dt, device=DEV)  # noqa: E731
+    Y, y, Yf, yf = E(b, n, h, D, d), E(b, n, h, D, dt=f32), E(b, h, D, d), E(b, h, D, dt=f32)
+    g = [dev(x) for x in (S, s, lg, S0, s0, dY, dy, dYf, dyf)]
+    _lib.check(lib.pr_state_scan_fwd(p(g[0]), p(g[1]), p(g[2]), p(Y), p(y), p(g[3]), p(g[4]), p(Yf), p(yf), b, n, n, h,
+                                     D * d, D, code, st), "scan fwd")
+    dX, dx, dlg, dY0, dy0 = E(b, n, h, D, d), E(b, n, h, D, dt=f32), E(b, n, h, dt=f32), E(b, h, D, d), E(b, h, D, dt=f32)
+    ws = torch.empty(lib.pr_state_scan_bwd_workspace(b, n, h, D * d, D), dtype=torch.uint8, device=DEV)
+    _lib.check(lib.pr_state_scan_bwd(p(g[5]), p(Y), p(g[6]), p(y), p(g[2]), p(dX), p(dx), p(dlg), p(ws), p(g[7]), p(g[8]),
+                                     p(dY0), p(dy0), b, n, n, h, D * d, D, code, st), "scan bwd")
 
-    # update_state forward
-    S, s, Sk, sk = E(BN, h, D, d), E(BN, h, D, dt=f32), E(BN, h, Dc, d), E(BN, h, Dc, dt=f32)
-    _lib.check(lib.pr_update_state_fwd(p(K), p(V), p(S), p(s), BN, c, h, d, 2, 0, 0, code, st), "fwd ref")
-    _lib.check(lib.pr_update_state_fwd(p(K), p(V), p(Sk), p(sk), BN, c, h, d, 2, 0, 1, code, st), "fwd compact")
-    assert torch.equal(Sk, _to_compact(S, d, 2)) and torch.equal(_to_reference(Sk, d, 2), S)
-    assert torch.equal(sk, _to_compact(s, d, 2)) and torch.equal(_to_reference(sk, d, 2), s)
+    # the recurrence, in fp32 with autograd (the kernel rounds the running state only when it stores an entry)
+    o = [gold(x, True) for x in (S, s, lg, S0, s0)]
 
-    # query_state forward and backward on the same state in both layouts
-    Ya = dev(rnd(BN, c, hq, d, dtype=dtype, seed=53))
-    la = dev(rnd(BN, c, hq, dtype=f32, seed=54).abs() + c)
-    rm = dev(rnd(BN, c, hq, dtype=f32, seed=55).abs() + 1.0)
-    dO = dev(rnd(BN, c, hq, d, dtype=dtype, seed=56))
-    scale_p = 1.0 / d
-    outs = []
-    for sym, S_, s_, D_ in ((1, S, s, D), (2, Sk, sk, Dc)):
-        O, den = E(BN, c, hq, d), E(BN, c, hq, dt=f32)
-        _lib.check(lib.pr_query_state_fwd(p(Q), p(S_), p(s_), p(Ya), p(la), p(rm), None, p(O), p(den), BN, n, c, h, r, d,
-                                          scale_p, 2, 0, sym, code, st), "qs fwd")
-        dQ, dS, ds = E(BN, c, hq, d), E(BN, h, D_, d), E(BN, h, D_, dt=f32)
-        dla, dys = E(BN, c, hq, dt=f32), E(BN, c, hq, dt=f32)
-        ws = torch.empty(lib.pr_query_state_bwd_workspace(BN, c, h, r, d, code), dtype=torch.uint8, device=DEV)
-        _lib.check(lib.pr_query_state_bwd(p(Q), p(S_), p(s_), p(rm), None, p(O), p(den), p(dO), p(dQ), p(dS), p(ds), None,
-                                          p(dla), p(dys), p(ws), BN, n, c, h, r, d, scale_p, 2, 0, sym, code, st), "qs bwd")
-        outs.append((O, den, dQ, dS, ds, dla, dys))
-    for nm, a, k in zip(("O", "den", "dQ", "dS", "ds", "dl_attn", "dY_scale"), *outs):
-        if nm == "ds":
-            # (the weighted key sums round one factor of a pair before the product, so the two orders of a pair differ
-            # in the last bit in the reference layout; the compact layout keeps one of them)
-            check("ds", k, _to_compact(a, d, 2), 1e-2)
-        elif nm == "dS":
-            assert torch.equal(k, _to_compact(a, d, 2)), nm
-        else:
-            assert torch.equal(a, k), nm
-
-    # update_state backward reading a symmetric gradient in both layouts
-    dS, dSk, dsk = outs[0][3], outs[1][3], outs[1][4]
-    ds = _to_reference(dsk, d, 2)                                    # (the same key sums for both orders of a pair)
-    Kq, Vq = Q[:, :, ::r].contiguous(), dO[:, :, ::r].contiguous()   # any [BN, c, h, d] operands
-    res = []
-    for sym, dS_, ds_ in ((1, dS, ds), (2, dSk, dsk)):
-        dK, dV = E(BN, c, h, d), E(BN, c, h, d)
-        _lib.check(lib.pr_update_state_bwd(p(Kq), p(Vq), p(dS_), p(ds_), p(dK), p(dV), BN, c, h, d, 2, sym, 0, code, st), "us bwd")
-        res.append((dK, dV))
-    assert torch.equal(res[0][0], res[1][0]) and torch.equal(res[0][1], res[1][1])
-
-    # the scans: values row for row, the gate gradient with the rows of a pair counted twice, state handed over
-    lg = dev(gates(b, n, h, seed=57))
-    S0, s0 = dev(rnd(b, h, D, d, dtype=dtype, seed=58)), dev(rnd(b, h, D, dtype=f32, seed=59))
-    S0 = _to_reference(_to_compact(S0, d, 2), d, 2)      # a symmetric starting value
-    s0 = _to_reference(_to_compact(s0, d, 2), d, 2)
-    dSf, dsf = dev(rnd(b, h, D, d, dtype=dtype, seed=60)), dev(rnd(b, h, D, dtype=f32, seed=61))
-    dSf, dsf = _to_reference(_to_compact(dSf, d, 2), d, 2), _to_reference(_to_compact(dsf, d, 2), d, 2)
-    got = []
-    for comp, D_, conv in ((0, D, lambda x: x.contiguous()), (d, Dc, lambda x: _to_compact(x, d, 2).contiguous())):
-        X, x = conv(S), conv(s)
-        Y, y, Yf, yf = E(BN, h, D_, d), E(BN, h, D_, dt=f32), E(b, h, D_, d), E(b, h, D_, dt=f32)
-        a0, b0 = conv(S0), conv(s0)
-        _lib.check(lib.pr_state_scan_fwd(p(X), p(x), p(lg), p(Y), p(y), p(a0), p(b0), p(Yf), p(yf), b, n, n, h, D_ * d, D_,
-                                         code, st), "scan fwd")
-        dY, dy = conv(outs[0][3]), conv(ds)   # (symmetric gradients, as every gradient the node forms is)
-        dX, dx, dlg = E(BN, h, D_, d), E(BN, h, D_, dt=f32), E(b, n, h, dt=f32)
-        dY0, dy0 = E(b, h, D_, d), E(b, h, D_, dt=f32)
-        c0, c1 = conv(dSf), conv(dsf)
-        ws = torch.empty(lib.pr_state_scan_bwd_workspace(b, n, h, D_ * d, D_), dtype=torch.uint8, device=DEV)
-        _lib.check(lib.pr_state_scan_bwd(p(dY), p(Y), p(dy), p(y), p(lg), p(dX), p(dx), p(dlg), p(ws), p(c0), p(c1),
-                                         p(dY0), p(dy0), comp, b, n, n, h, D_ * d, D_, code, st), "scan bwd")
-        got.append((Y, y, Yf, yf, dX, dx, dY0, dy0, dlg))
-    for nm, a, k in zip(("Y", "y", "Y_final", "y_final", "dX", "dx", "dY_init", "dy_init"), *got):
-        assert torch.equal(k, _to_compact(a, d, 2)), nm
-    check("dlog_G (compact vs expanded)", got[1][8], got[0][8], 1e-5)
-    # and the handed-over state against the closed form of the recurrence, in fp32
-    g = torch.exp(lg)                                          # [b, n, h]
-    Sv, ref = S.view(b, n, h, D, d).float(), S0.float()
-    for k_ in range(n):
-        ref = ref * g[:, k_, :, None, None] + Sv[:, k_]
-    check("final state vs recurrence", got[0][2], ref, 1e-2)
+    def scan(X, init, gates_):
+        cur, out = init, []
+        for k in range(n):
+            out.append(cur)
+            cur = cur * torch.exp(gates_[:, k]).reshape(b, h, *([1] * (X.dim() - 3))) + X[:, k]
+        return torch.stack(out, 1), cur
+    Yo, Yfo = scan(o[0], o[3], o[2])
+    yo, yfo = scan(o[1], o[4], o[2])
+    check("Y", Y, Yo, OUT_TOL)
+    check("y", y, yo, 1e-5)
+    check("Y_final", Yf, Yfo, OUT_TOL)
+    check("y_final", yf, yfo, 1e-5)
+    torch.autograd.backward([Yo, yo, Yfo, yfo], [gold(dY), gold(dy), gold(dYf), gold(dyf)])
+    check("dX", dX, o[0].grad, GRAD_TOL)
+    check("dx", dx, o[1].grad, 1e-5)
+    check("dS_init", dY0, o[3].grad, GRAD_TOL)
+    check("ds_init", dy0, o[4].grad, 1e-5)
+    check("dlog_G", dlg, o[2].grad, GRAD_TOL)

@@ -111,41 +111,3 @@ def test_cache_layer_takes_wide_query_groups_and_refuses_ragged_ones(monkeypatch
     assert not pra.RetentionCache(batch=1, kv_heads=1, head_dim=32, capacity=4, device="cpu", q_heads=24)._fused_step
     with pytest.raises(AssertionError):
         pra.RetentionCache(batch=1, kv_heads=2, head_dim=32, capacity=4, device="cpu", q_heads=5)
-
-
-@pytest.mark.parametrize("d", [32, 64])
-def test_compact_layout_maps_against_the_oracles_feature_table(d):
-    """The index maps between the reference state layout and the compact one the fused node keeps its chunk states in:
-    every compact row is one unordered pair of coordinates, found at both of its places in the reference layout
-    (the oracle's feature table, ref: retention/_update_state/reference.py:22-28), every pair appears, and a symmetric
-    tensor survives the round trip."""
-    import oracle
-    from retention_integration_amd.fused import _layout_maps, _to_compact, _to_reference, compact_dim
-    from retention_integration_amd.ops import expanded_dim
-    D, Dc = expanded_dim(d), compact_dim(d)
-    assert Dc == {32: 544, 64: 2112}[d]
-    ia, ib, ic = (m.tolist() for m in _layout_maps(d, torch.device("cpu")))
-    xi, wi, _ = oracle.state_feature_table(d)
-    pairs = [tuple(sorted((int(a), int(b)))) for a, b in zip(xi.tolist(), wi.tolist())]
-    assert len(ia) == Dc and len(ic) == D
-    for row in range(Dc):
-        assert pairs[ia[row]] == pairs[ib[row]]
-    assert set(pairs[ia[row]] for row in range(Dc)) == set(pairs)
-    for f in range(D):
-        assert pairs[ia[ic[f]]] == pairs[f]
-    # a symmetric tensor (both orders of a pair equal) is reproduced exactly; of any other tensor the symmetric part is
-    # (all that a query of the state sees: phi(q) is symmetric)
-    g = torch.Generator().manual_seed(d)
-    x = torch.randn(2, D, 3, generator=g)
-    first = {}
-    for f, pr_ in enumerate(pairs):
-        first.setdefault(pr_, []).append(f)
-
-    def symmetric_part(t):
-        out = torch.zeros_like(t)
-        for fs in first.values():
-            out[:, fs] = t[:, fs].mean(1, keepdim=True)
-        return out
-    sym = symmetric_part(x)
-    assert torch.allclose(_to_reference(_to_compact(sym, d, 1), d, 1), sym, atol=1e-6)
-    assert torch.allclose(symmetric_part(_to_reference(_to_compact(x, d, 1), d, 1)), sym, atol=1e-6)
