@@ -190,12 +190,17 @@ int pr_query_state_fwd(const void* Q, const void* S, const float* s, const void*
  *   q_log_gate as in the forward: Q is then the ungated query and dQ the gradient w.r.t. it through the state part
  *   (the gate's own gradient is (Q . dQ) / deg per row, which pr_chunk_attention_bwd forms with dQ_state_plain).
  *   S_symmetric != 0: the caller's promise that S[(a,b)] == S[(b,a)] in the blocks on the diagonal (true of every
- *   state made by pr_update_state_fwd and the scans); the query gradient then takes a shorter path through them. */
+ *   state made by pr_update_state_fwd and the scans); the query gradient then takes a shorter path through them.
+ *   The call is three kernels: the row-wise preparation (fills the workspace, dY_attn / dY_scale, dl_attn), dS / ds, and
+ *   dQ.  With dS == ds == NULL or dQ == NULL that kernel is skipped; prepared != 0 says that an earlier call with the
+ *   same inputs has filled this workspace and skips the preparation -- so the two contractions, which do not depend
+ *   on each other, can be issued as two calls on two streams. */
 size_t pr_query_state_bwd_workspace(int BN, int c, int h, int r, int d, int dtype);
 int pr_query_state_bwd(const void* Q, const void* S, const float* s, const float* rowmax, const float* q_log_gate,
                        const void* O, const float* den, const void* dO, void* dQ, void* dS, float* ds, void* dY_attn,
                        float* dl_attn, float* dY_scale, void* workspace, int BN, int n, int c, int h, int r, int d,
-                       float scale_p, int deg, int zero_initial_state, int S_symmetric, int dtype, void* stream);
+                       float scale_p, int deg, int zero_initial_state, int S_symmetric, int prepared, int dtype,
+                       void* stream);
 
 /* Accumulated gates of the quadratic / inference paths -- log_G.cumsum(1), retention/power_retention_maker.py:129,
  * 348-349.  log_G, A [B,t,h] fp32, t <= 8192. */

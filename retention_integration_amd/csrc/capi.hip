@@ -235,11 +235,13 @@ size_t pr_query_state_bwd_workspace(int BN, int c, int h, int r, int d, int dtyp
 int pr_query_state_bwd(const void* Q, const void* S, const float* s, const float* rowmax, const float* q_log_gate,
                        const void* O, const float* den, const void* dO, void* dQ, void* dS, float* ds, void* dY_attn,
                        float* dl_attn, float* dY_scale, void* workspace, int BN, int n, int c, int h, int r, int d,
-                       float scale_p, int deg, int zero_initial_state, int S_symmetric, int dtype, void* stream) {
+                       float scale_p, int deg, int zero_initial_state, int S_symmetric, int prepared, int dtype,
+                       void* stream) {
   if (int rc = check_common("query_state_bwd", d, deg, dtype, true)) return rc;
-  if (bad_ptr(Q) || bad_ptr(S) || bad_ptr(s) || bad_ptr(O) || bad_ptr(den) || bad_ptr(dO) || bad_ptr(dQ) ||
-      bad_ptr(dS) || bad_ptr(ds) || bad_ptr(workspace) || bad_opt(rowmax) || bad_opt(dY_attn) || bad_opt(dl_attn))
+  if (bad_ptr(Q) || bad_ptr(S) || bad_ptr(s) || bad_ptr(O) || bad_ptr(den) || bad_ptr(dO) || bad_opt(dQ) ||
+      bad_opt(dS) || bad_ptr(workspace) || bad_opt(rowmax) || bad_opt(dY_attn) || bad_opt(dl_attn))
     return fail(PR_ERR_ARG, "query_state_bwd: null or misaligned pointer");
+  if ((dS == nullptr) != (ds == nullptr)) return fail(PR_ERR_ARG, "query_state_bwd: dS and ds come together");
   if (rowmax && ((!dY_attn && !dY_scale) || !dl_attn))
     return fail(PR_ERR_ARG, "query_state_bwd: dl_attn and one of dY_attn, dY_scale are required when rowmax is given");
   if (q_log_gate && !rowmax) return fail(PR_ERR_ARG, "query_state_bwd: q_log_gate needs the attention part");
@@ -250,15 +252,18 @@ int pr_query_state_bwd(const void* Q, const void* S, const float* s, const float
   void* dOs = workspace;
   float* cvec = (float*)((char*)workspace + align256(rows * d * 2));
   hipStream_t st = (hipStream_t)stream;
-  if (int rc = finish(pr::qs_bwd_prep(O, dO, den, rowmax, q_log_gate, dOs, cvec, rowmax ? dY_attn : nullptr,
-                                      rowmax ? dl_attn : nullptr, rowmax ? dY_scale : nullptr, (long)rows, h, r, d,
-                                      scale_p, dtype, st),
-                      "query_state_bwd(prep)"))
-    return rc;
+  if (!prepared)
+    if (int rc = finish(pr::qs_bwd_prep(O, dO, den, rowmax, q_log_gate, dOs, cvec, rowmax ? dY_attn : nullptr,
+                                        rowmax ? dl_attn : nullptr, rowmax ? dY_scale : nullptr, (long)rows, h, r, d,
+                                        scale_p, dtype, st),
+                        "query_state_bwd(prep)"))
+      return rc;
   // (zero_initial_state == 2: the caller does not want the gradient of the first chunk's (zero) state either)
-  if (int rc = finish(pr::sympow_tn(Q, dOs, cvec, dS, ds, BN, c, h, r, d, 0, zero_initial_state == 2 ? -n : 0, dtype, st),
-                      "query_state_bwd(dS)"))
-    return rc;
+  if (dS)
+    if (int rc = finish(pr::sympow_tn(Q, dOs, cvec, dS, ds, BN, c, h, r, d, 0, zero_initial_state == 2 ? -n : 0, dtype, st),
+                        "query_state_bwd(dS)"))
+      return rc;
+  if (!dQ) return 0;
   pr::GradArgs g{Q, dOs, cvec, S, s, dQ, c, h, r, n, zero_initial_state ? 1 : 0, S_symmetric ? 1 : 0};
   return finish(pr::sympow_grad(g, BN, d, 0, dtype, st), "query_state_bwd(dQ)");
 }

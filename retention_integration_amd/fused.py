@@ -35,6 +35,13 @@ def _chained(lib, b, n, c, h, r, d):
 # deal their workgroups to the XCDs pair by pair in the same order: launched side by side on two streams of the same
 # priority they share those rows in L2 instead of fetching them twice (12 us of a training step at the headline shape).
 ATTN_BWD_TWO_STREAMS = True
+# Forward: the attention kernel needs only the gate sums, so it runs next to  key discount -> chunk states -> scan.
+FWD_TWO_STREAMS = True
+# The same for the whole query side of the backward: the query gradient through the state depends only on the
+# row-wise preparation, so it can run next to the chain  dS -> reverse scan -> dK, dV  instead of in front of it.
+BWD_TWO_STREAMS = True
+# Forward: the attention kernel needs only the gate sums, so it runs next to  key discount -> chunk states -> scan.
+FWD_TWO_STREAMS = True
 _SIDE = {}
 
 
@@ -91,6 +98,17 @@ def chunked_fwd(Q: Tensor, K: Tensor, V: Tensor, log_G: Optional[Tensor], deg: i
         Kd_ = K
         lcs = torch.zeros((BN, h), dtype=f32, device=dev)
 
+    Ya = torch.empty_like(Q)
+    la, rm = _empty((BN, c, hq), f32, dev), _empty((BN, c, hq), f32, dev)
+
+    def attention(stream):
+        _lib.check(lib.pr_attention_fwd(p(Q), p(K), p(V), p(A) if gated else None, p(Ya), p(la), p(rm), BN, c, c, h, r,
+                                        d, scale, deg, 0, code, stream), "attention_fwd")
+    if FWD_TWO_STREAMS:
+        main, side = torch.cuda.current_stream(), _side_stream(dev)
+        side.wait_stream(main)
+        attention(side.cuda_stream)
+
     Sc, sc = _empty((BN, h, D, d), dt, dev), _empty((BN, h, D), f32, dev)
     Sf, sf = _empty((0,), dt, dev), _empty((0,), f32, dev)
     if chained:
@@ -111,10 +129,10 @@ def chunked_fwd(Q: Tensor, K: Tensor, V: Tensor, log_G: Optional[Tensor], deg: i
                                          D * d, D, code, st), "state_scan_fwd")
         del S, s
 
-    Ya = torch.empty_like(Q)
-    la, rm = _empty((BN, c, hq), f32, dev), _empty((BN, c, hq), f32, dev)
-    _lib.check(lib.pr_attention_fwd(p(Q), p(K), p(V), p(A) if gated else None, p(Ya), p(la), p(rm), BN, c, c, h, r, d,
-                                    scale, deg, 0, code, st), "attention_fwd")
+    if FWD_TWO_STREAMS:
+        main.wait_stream(side)
+    else:
+        attention(st)
     O, den = torch.empty_like(Q), _empty((BN, c, hq), f32, dev)
     _lib.check(lib.pr_query_state_fwd(p(Q), p(Sc), p(sc), p(Ya), p(la), p(rm), p(A) if gated else None, p(O), p(den),
                                       BN, n, c, h, r, d, scale ** deg, deg, 0 if carried else 1, 1, code, st),
@@ -168,6 +186,7 @@ def chunked_bwd(Q: Tensor, K: Tensor, V: Tensor, A: Tensor, lcs: Tensor, Kd: Ten
     dlcs = torch.empty_like(lcs)   # gate gradient of both scans
     dS0, ds0 = _empty((0,), dt, dev), _empty((0,), f32, dev)
     has_dfin = dSf is not None or dsf is not None
+    two_streams = False
     if not carried and not has_dfin and _chained(lib, b, n, c, h, r, d):
         ws = _empty((lib.pr_query_state_scan_bwd_workspace(b, n, c, h, r, d, code),), u8, dev)
         _lib.check(lib.pr_query_state_scan_bwd(p(Q), p(Sc), p(sc), p(rm), qgate, p(O), p(den), p(dO),
@@ -176,23 +195,34 @@ def chunked_bwd(Q: Tensor, K: Tensor, V: Tensor, A: Tensor, lcs: Tensor, Kd: Ten
                                                code, st), "query_state_scan_bwd")
     else:
         dSc, dsc = torch.empty_like(Sc), torch.empty_like(sc)
-        ws = _empty((lib.pr_query_state_bwd_workspace(BN, c, h, r, d, code),), u8, dev)
-        # (zero_initial_state: 2 = chunk 0 sees no state and nobody wants its gradient; 0 = it sees the carried one)
-        _lib.check(lib.pr_query_state_bwd(p(Q), p(Sc), p(sc), p(rm), qgate, p(O), p(den), p(dO), p(dQg), p(dSc), p(dsc),
-                                          None, p(dla), p(dys), p(ws), BN, n, c, h, r, d, scale ** deg, deg,
-                                          0 if carried else 2, 1, code, st),
-                   "query_state_bwd")
+        qws = _empty((lib.pr_query_state_bwd_workspace(BN, c, h, r, d, code),), u8, dev)
+        zis = 0 if carried else 2   # (2 = chunk 0 sees no state and nobody wants its gradient; 0 = it sees the carried one)
+
+        def qs_bwd(dQ_, dS_, ds_, prepared, stream):
+            _lib.check(lib.pr_query_state_bwd(p(Q), p(Sc), p(sc), p(rm), qgate, p(O), p(den), p(dO), dQ_, dS_, ds_, None,
+                                              p(dla), p(dys), p(qws), BN, n, c, h, r, d, scale ** deg, deg, zis, 1,
+                                              prepared, code, stream), "query_state_bwd")
+        if BWD_TWO_STREAMS:
+            # The query gradient through the state (and, after it, the query side of the attention backward) depends
+            # only on the row-wise preparation: it runs on a second stream next to the chain dS -> scan -> dK, dV.
+            main, side = torch.cuda.current_stream(), _side_stream(dev)
+            qs_bwd(None, None, None, 0, st)              # preparation only
+            side.wait_stream(main)
+            qs_bwd(p(dQg), None, None, 1, side.cuda_stream)
+            qs_bwd(None, p(dSc), p(dsc), 1, st)
+        else:
+            qs_bwd(p(dQg), p(dSc), p(dsc), 0, st)
         dSf_ = dsf_ = None
         if has_dfin:   # the gradient that arrived through the returned final state enters the reverse scan as entry n
             dSf_ = (dSf if dSf is not None else torch.zeros((b, h, D, d), dtype=dt, device=dev)).contiguous()
             dsf_ = (dsf.to(f32) if dsf is not None else torch.zeros((b, h, D), dtype=f32, device=dev)).contiguous()
         if carried:
             dS0, ds0 = _empty((b, h, D, d), dt, dev), _empty((b, h, D), f32, dev)
-        ws = _empty((lib.pr_state_scan_bwd_workspace(b, n, h, D * d, D),), u8, dev)
-        _lib.check(lib.pr_state_scan_bwd(p(dSc), p(Sc), p(dsc), p(sc), p(lcs), p(dS), p(ds), p(dlcs), p(ws), p(dSf_),
+        sws = _empty((lib.pr_state_scan_bwd_workspace(b, n, h, D * d, D),), u8, dev)
+        _lib.check(lib.pr_state_scan_bwd(p(dSc), p(Sc), p(dsc), p(sc), p(lcs), p(dS), p(ds), p(dlcs), p(sws), p(dSf_),
                                          p(dsf_), p(dS0) if carried else None, p(ds0) if carried else None, b, n, n, h,
                                          D * d, D, code, st), "state_scan_bwd")
-        del dSc, dsc
+        two_streams = BWD_TWO_STREAMS
     dKd, dVs = torch.empty_like(K), torch.empty_like(V)
     # (dS comes from the kernels above, so both orders of a pair hold the same sum: the symmetry flag says so; the last
     # chunk's dS is zero unless a gradient arrived through the final state)
@@ -205,16 +235,18 @@ def chunked_bwd(Q: Tensor, K: Tensor, V: Tensor, A: Tensor, lcs: Tensor, Kd: Ten
     dGk = _empty((b, t, h), f32, dev) if gated else None
     dotk = _empty((BN, c, h), f32, dev) if gated else None
     Ag = p(A) if gated else None
-    if ATTN_BWD_TWO_STREAMS:
-        # the key side on the launch stream, the query side next to it on a second stream of the same priority
+    if two_streams or ATTN_BWD_TWO_STREAMS:
+        # the key side on the launch stream, the query side next to it on the second stream (which, with
+        # BWD_TWO_STREAMS, already holds the state part of the query gradient)
         main, side = torch.cuda.current_stream(), _side_stream(dev)
-        side.wait_stream(main)
-        _lib.check(lib.pr_chunk_attention_bwd(p(Q), p(K), p(V), Ag, p(rm), p(dO), p(dla), p(dys), None, p(dKd), p(dVs),
-                                              None, p(dKa), p(dVa), None, p(dGk), p(dotk), BN, c, h, r, d, scale, deg, 1,
-                                              code, st), "chunk_attention_bwd(dK, dV)")
+        if not two_streams:
+            side.wait_stream(main)
         _lib.check(lib.pr_chunk_attention_bwd(p(Q), p(K), p(V), Ag, p(rm), p(dO), p(dla), p(dys), p(dQg), None, None,
                                               p(dQa), None, None, p(dGq), None, None, BN, c, h, r, d, scale, deg, 1,
                                               code, side.cuda_stream), "chunk_attention_bwd(dQ)")
+        _lib.check(lib.pr_chunk_attention_bwd(p(Q), p(K), p(V), Ag, p(rm), p(dO), p(dla), p(dys), None, p(dKd), p(dVs),
+                                              None, p(dKa), p(dVa), None, p(dGk), p(dotk), BN, c, h, r, d, scale, deg, 1,
+                                              code, st), "chunk_attention_bwd(dK, dV)")
         main.wait_stream(side)
     else:
         _lib.check(lib.pr_chunk_attention_bwd(p(Q), p(K), p(V), Ag, p(rm), p(dO), p(dla), p(dys), p(dQg), p(dKd),

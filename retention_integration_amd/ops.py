@@ -311,7 +311,7 @@ def query_state_bwd(Q: Tensor, S: Tensor, s: Tensor, rowmax: Optional[Tensor], O
     _lib.check(lib.pr_query_state_bwd(_lib.ptr(Q), _lib.ptr(S), _lib.ptr(s), _lib.ptr(rowmax), None, _lib.ptr(O),
                                       _lib.ptr(den), _lib.ptr(dO), _lib.ptr(dQ), _lib.ptr(dS), _lib.ptr(ds),
                                       _lib.ptr(dYa), _lib.ptr(dla), None, _lib.ptr(ws), b * n, n, c, h, r, d,
-                                      float(scale_p), 2, int(zero_initial_state), 0, code, _lib.stream()),
+                                      float(scale_p), 2, int(zero_initial_state), 0, 0, code, _lib.stream()),
                "query_state_bwd")
     if not has_attn:
         dYa = torch.empty((0,), dtype=Q.dtype, device=Q.device)

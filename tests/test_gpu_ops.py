@@ -306,7 +306,7 @@ def test_symmetric_state_flag_changes_nothing_for_a_symmetric_state(pra, dtype, 
         dQ, dS, ds = torch.empty_like(Q), torch.empty_like(S), torch.empty_like(s)
         ws = torch.empty(lib.pr_query_state_bwd_workspace(b * n, c, h, 1, d, code), dtype=torch.uint8, device=DEV)
         _lib.check(lib.pr_query_state_bwd(p(Q), p(S), p(s), None, None, p(O), p(den), p(dO), p(dQ), p(dS), p(ds), None, None,
-                                          None, p(ws), b * n, n, c, h, 1, d, 1.0 / d, 2, 0, flag, code, st),
+                                          None, p(ws), b * n, n, c, h, 1, d, 1.0 / d, 2, 0, flag, 0, code, st),
                    "query_state_bwd")
         res.append((dK, dV, dQ, dS, ds, O, den))
     for nm, a, b_ in zip(["dK", "dV", "dQ", "dS", "ds", "O", "den"], res[1], res[0]):
