@@ -249,10 +249,15 @@ class KernelTimers:
         self.records, self.steps = [], []
         self._t0 = None
 
+        self._streams = {}
+
         def hook(name, phase, stream, user):
-            assert (stream or 0) == torch.cuda.current_stream().cuda_stream, "kernel launched on another stream than torch's"
+            sp = stream or 0
+            if sp not in self._streams:
+                self._streams[sp] = torch.cuda.current_stream() if sp == torch.cuda.current_stream().cuda_stream \
+                    else torch.cuda.ExternalStream(sp)
             ev = torch.cuda.Event(enable_timing=True)
-            ev.record()
+            ev.record(self._streams[sp])
             if phase == 0:
                 self._t0 = ev
             else:
@@ -496,12 +501,26 @@ def main():
     torch.cuda.synchronize()
     dt_b2b = (time.perf_counter() - t0) / args.steps
     # (a') the same steps once more with EVERY kernel timed where it runs: HIP events on the launch stream around each
-    # launch (the library's launch hook); the events make these steps a little longer, so they are not the ones above
-    with KernelTimers(_lib) as kt:
-        for _ in range(args.steps + 2):
+    # launch (the library's launch hook).  For these steps the kernels run one after the other: in the steps above,
+    # independent kernels of a step share the GPU on two streams, and a kernel timed while another one runs beside it
+    # says nothing about either.  (So the sum of these times exceeds a headline step.)
+    from retention_integration_amd import fused
+    overlap = (fused.FWD_TWO_STREAMS, fused.BWD_TWO_STREAMS, fused.ATTN_BWD_TWO_STREAMS)
+    fused.FWD_TWO_STREAMS = fused.BWD_TWO_STREAMS = fused.ATTN_BWD_TWO_STREAMS = False
+    try:
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
             step()
-            kt.end_step()
-        in_step_ms = kt.per_step(skip=2)
+        torch.cuda.synchronize()
+        dt_seq = (time.perf_counter() - t0) / args.steps
+        with KernelTimers(_lib) as kt:
+            for _ in range(args.steps + 2):
+                step()
+                kt.end_step()
+            in_step_ms = kt.per_step(skip=2)
+    finally:
+        fused.FWD_TWO_STREAMS, fused.BWD_TWO_STREAMS, fused.ATTN_BWD_TWO_STREAMS = overlap
     # (b) the headline, by the reference's protocol (ref: perf/_timing.py:77-110): before every step the caches are
     # flushed (a fill of 512 MB: L2 and the 256 MB memory-side cache), then a short device-side pause lets the host run
     # ahead (launch latency is not measured), the step is bracketed by HIP events of its own, and the MEDIAN over the K
@@ -528,6 +547,7 @@ def main():
                                "before settling",
                    "flushed_ms": {"median": round(dt * 1e3, 4), "min": round(min(times), 4), "max": round(max(times), 4)},
                    "back_to_back_ms_per_step": round(dt_b2b * 1e3, 4),
+                   "back_to_back_one_stream_ms_per_step": round(dt_seq * 1e3, 4),
                    "first_steps_ms": [round(x, 4) for x in first],
                    "settle_ms": args.settle_ms, "settle_steps": settle_steps},
     }

@@ -209,7 +209,9 @@ int pr_gate_cumsum(const float* log_G, float* A, int B, int t, int h, void* stre
 /* Gate arithmetic of the chunked algorithm, forward -- retention/power_retention_maker.py:146-153,163-164,183-186.
  *   log_G [BN,c,h] fp32 (BN = b*n chunks of length c <= 8192), K [BN,c,h,d], Q [BN,c,h*r,d]
  *   -> A [BN,c,h] = cumsum over the chunk, lcs [BN,h] = A[c-1],
- *      Kd = K * exp((A[c-1] - A)/deg), Qg = Q * exp(A/deg) (Qg may be NULL: not formed). */
+ *      Kd = K * exp((A[c-1] - A)/deg), Qg = Q * exp(A/deg) (Qg may be NULL: not formed).
+ *   Two kernels (the sums, then the row-wise products): with Kd == NULL only A and lcs are written; with
+ *   log_G == NULL, A and lcs are inputs and only the products are formed. */
 int pr_chunk_prep_fwd(const float* log_G, const void* K, const void* Q, float* A, float* lcs, void* Kd, void* Qg, int BN,
                       int c, int h, int r, int d, int deg, int dtype, void* stream);
 

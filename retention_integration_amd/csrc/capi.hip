@@ -341,7 +341,7 @@ int pr_gate_cumsum(const float* log_G, float* A, int B, int t, int h, void* stre
 int pr_chunk_prep_fwd(const float* log_G, const void* K, const void* Q, float* A, float* lcs, void* Kd, void* Qg, int BN,
                       int c, int h, int r, int d, int deg, int dtype, void* stream) {
   if (int rc = check_common("chunk_prep_fwd", d, deg, dtype, false)) return rc;
-  if (log_G == nullptr || bad_ptr(K) || bad_ptr(Q) || A == nullptr || lcs == nullptr || bad_ptr(Kd) || bad_opt(Qg))
+  if (bad_ptr(K) || bad_ptr(Q) || A == nullptr || lcs == nullptr || bad_opt(Kd) || bad_opt(Qg) || (!log_G && !Kd))
     return fail(PR_ERR_ARG, "chunk_prep_fwd: null or misaligned pointer");
   if (BN <= 0 || c <= 0 || h <= 0 || r <= 0) return fail(PR_ERR_ARG, "chunk_prep_fwd: need BN,c,h,r > 0");
   return finish(pr::chunk_prep_fwd(log_G, K, Q, A, lcs, Kd, Qg, BN, c, h, r, d, deg, dtype, (hipStream_t)stream),

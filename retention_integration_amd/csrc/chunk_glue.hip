@@ -121,7 +121,9 @@ template <typename T>
 static int prep_launch(const float* logG, const void* K, const void* Q, float* A, float* lcs, void* Kd, void* Qg, int BN,
                        int c, int h, int r, int d, int deg, hipStream_t st) {
   const size_t smem = (size_t)(c + 256) * sizeof(float);
-  PR_LAUNCH("gate_scan_fwd", gate_scan_fwd_kernel, dim3((unsigned)(BN * h)), dim3(256), smem, st, logG, A, lcs, c, h);
+  // (either half on its own: no log_G = A and lcs are already there; no Kd = only the sums are wanted)
+  if (logG) PR_LAUNCH("gate_scan_fwd", gate_scan_fwd_kernel, dim3((unsigned)(BN * h)), dim3(256), smem, st, logG, A, lcs, c, h);
+  if (!Kd) return (int)hipGetLastError();
   const long groups = (long)BN * c * h;
 #define PR_CP(DD)                                                                                                      \
   case DD:                                                                                                             \

@@ -90,8 +90,9 @@ def chunked_fwd(Q: Tensor, K: Tensor, V: Tensor, log_G: Optional[Tensor], deg: i
     if gated:
         A, lcs = _empty((BN, c, h), f32, dev), _empty((BN, h), f32, dev)
         Kd = torch.empty_like(K)
-        _lib.check(lib.pr_chunk_prep_fwd(p(log_G), p(K), p(Q), p(A), p(lcs), p(Kd), None, BN, c, h, r, d, deg, code,
-                                         st), "chunk_prep_fwd")
+        # (the sums first: the attention kernel needs nothing else; the discounted keys follow below)
+        _lib.check(lib.pr_chunk_prep_fwd(p(log_G), p(K), p(Q), p(A), p(lcs), None, None, BN, c, h, r, d, deg, code,
+                                         st), "chunk_prep_fwd(sums)")
         Kd_ = Kd
     else:
         A, Kd = _empty((0,), f32, dev), _empty((0,), dt, dev)
@@ -109,6 +110,9 @@ def chunked_fwd(Q: Tensor, K: Tensor, V: Tensor, log_G: Optional[Tensor], deg: i
         side.wait_stream(main)
         attention(side.cuda_stream)
 
+    if gated:
+        _lib.check(lib.pr_chunk_prep_fwd(None, p(K), p(Q), p(A), p(lcs), p(Kd), None, BN, c, h, r, d, deg, code, st),
+                   "chunk_prep_fwd(keys)")
     Sc, sc = _empty((BN, h, D, d), dt, dev), _empty((BN, h, D), f32, dev)
     Sf, sf = _empty((0,), dt, dev), _empty((0,), f32, dev)
     if chained:
