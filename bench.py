@@ -303,7 +303,8 @@ def kernel_work(cfg, D_stored):
     St = bh * n * D_stored * (d * 2 + 4)     # one state tensor with its fp32 key sums, all chunks
     return {
         "sympow_tn": ("mfma", state), "sympow_nn": ("mfma", state), "sympow_grad": ("mfma", state),
-        "attention_fwd": ("mfma", 2.0 * attn), "attention_bwd_dkv": ("mfma", 3.0 * attn),
+        "attention_fwd": ("mfma", 2.0 * attn), "chunk_fwd": ("mfma", 2.0 * attn + state),
+        "attention_bwd_dkv": ("mfma", 3.0 * attn),
         "attention_bwd_dq": ("mfma", 2.0 * attn),
         "discumsum_pair_fwd": ("hbm", 2.0 * St * (n - 1) / n), "discumsum_pair_bwd": ("hbm", 3.0 * St * (n - 1) / n),
         "qs_bwd_prep": ("hbm", 3.0 * R), "gate_apply_fwd": ("hbm", 2.0 * R), "chunk_prep_fwd": ("hbm", 2.0 * R),
@@ -569,8 +570,13 @@ def main():
     if ab:
         ms = sum(in_step_ms[k] for k in ab)
         out["roofline_attention_bwd"] = roofline_block(" + ".join(ab), ms, ("mfma", 5.0 * bh * n * cfg["d"] * cfg["chunk"] * (cfg["chunk"] + 1)))
-    for key, label in (("roofline_attention_fwd", "attention_fwd#0"), ("roofline_update_state_fwd", "sympow_tn#0"),
-                       ("roofline_query_state_fwd", "sympow_nn#0"), ("roofline_update_state_bwd_dK", "sympow_grad#1"),
+    # (forward: one kernel for the attention inside the chunks, the state query and their merge where the library has it,
+    # else attention_fwd and sympow_nn#0; sympow_nn's other launch is update_state's dV)
+    one_kernel = "chunk_fwd#0" in in_step_ms
+    for key, label in (("roofline_chunk_fwd", "chunk_fwd#0"), ("roofline_attention_fwd", "attention_fwd#0"),
+                       ("roofline_update_state_fwd", "sympow_tn#0"),
+                       ("roofline_update_state_bwd_dV" if one_kernel else "roofline_query_state_fwd", "sympow_nn#0"),
+                       ("roofline_update_state_bwd_dK", "sympow_grad#1"),
                        ("roofline_state_scan_fwd", "discumsum_pair_fwd#0"), ("roofline_state_scan_bwd", "discumsum_pair_bwd#0")):
         if label in in_step_ms:
             out[key] = roofline_block(label, in_step_ms[label], work[label.split("#")[0]])

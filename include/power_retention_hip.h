@@ -41,7 +41,7 @@ enum {
  * pr_update_state_bwd zero_last_of; pr_query_state_fwd / _bwd / _scan_bwd take q_log_gate and
  * pr_chunk_attention_bwd dQ_state_plain.  5: pr_query_state_fwd takes S_symmetric.  6: pr_set_launch_hook;
  * pr_decode_step takes up to 16 query rows per (batch, kv head); pr_state_scan_fwd / _bwd connect a scan to the calls
- * before and after it (S_init, S_final and their gradients). */
+ * before and after it (S_init, S_final and their gradients).  7: pr_chunk_fwd, pr_chunk_fwd_supported. */
 int pr_abi_version(void);
 const char* pr_last_error(void);
 
@@ -201,6 +201,22 @@ int pr_query_state_bwd(const void* Q, const void* S, const float* s, const float
                        float* dl_attn, float* dY_scale, void* workspace, int BN, int n, int c, int h, int r, int d,
                        float scale_p, int deg, int zero_initial_state, int S_symmetric, int prepared, int dtype,
                        void* stream);
+
+/* Forward of every chunk in one kernel: the attention inside the chunk (retention/_attention/reference.py:10-69), the
+ * query of the state the chunk starts from and the merge of the two (retention/_query_state/reference.py:36-96, with
+ * the query gating of retention/power_retention_maker.py:183-186 as a row factor) -- what pr_chunk_attention_fwd
+ * followed by pr_query_state_fwd(q_log_gate = A, S_symmetric = 1) compute, without the attention part going to memory
+ * and back.  bf16, d in {32, 64}, deg 2: pr_chunk_fwd_supported() says whether the case exists; the others take the
+ * two calls.
+ *   Q [BN,c,h*r,d] (ungated), K, V [BN,c,h,d], A [BN,c,h] fp32 accumulated log gates of the chunk or NULL,
+ *   S [BN,h,D,d] / s [BN,h,D] fp32: the scanned states, symmetric in the diagonal feature blocks
+ *   -> O [BN,c,h*r,d], rowmax [BN,c,h*r] (log of the row's largest attention weight) and den [BN,c,h*r], both fp32 and
+ *      in the units pr_query_state_bwd and pr_chunk_attention_bwd expect.
+ *   scale multiplies q.k before the power; n, zero_initial_state as in pr_query_state_fwd. */
+int pr_chunk_fwd_supported(int d, int deg, int dtype);
+int pr_chunk_fwd(const void* Q, const void* K, const void* V, const float* A, const void* S, const float* s, void* O,
+                 float* rowmax, float* den, int BN, int n, int c, int h, int r, int d, float scale, int deg,
+                 int zero_initial_state, int dtype, void* stream);
 
 /* Accumulated gates of the quadratic / inference paths -- log_G.cumsum(1), retention/power_retention_maker.py:129,
  * 348-349.  log_G, A [B,t,h] fp32, t <= 8192. */

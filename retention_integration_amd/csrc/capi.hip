@@ -43,7 +43,7 @@ size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 
 extern "C" {
 
-int pr_abi_version(void) { return 6; }
+int pr_abi_version(void) { return 7; }
 
 void pr_set_launch_hook(pr_launch_hook_t hook, void* user) {
   pr::g_launch_hook = nullptr;   // (never a new hook with the old user pointer)
@@ -224,6 +224,24 @@ int pr_query_state_fwd(const void* Q, const void* S, const float* s, const void*
   pr::NNArgs a{Q, S, s, O, den, Y_attn, l_attn, rowmax, scale_p, c, h, r, n, zero_initial_state ? 1 : 0, 0,
                S_symmetric ? 1 : 0, q_log_gate};
   return finish(pr::sympow_nn(a, BN, d, 0, 1, dtype, (hipStream_t)stream), "query_state_fwd");
+}
+
+int pr_chunk_fwd_supported(int d, int deg, int dtype) { return deg == 2 && pr::chunk_fwd_supported(d, dtype); }
+
+int pr_chunk_fwd(const void* Q, const void* K, const void* V, const float* A, const void* S, const float* s, void* O,
+                 float* rowmax, float* den, int BN, int n, int c, int h, int r, int d, float scale, int deg,
+                 int zero_initial_state, int dtype, void* stream) {
+  if (int rc = check_common("chunk_fwd", d, deg, dtype, true)) return rc;
+  if (!pr_chunk_fwd_supported(d, deg, dtype))
+    return fail(PR_ERR_DTYPE, "chunk_fwd: bf16, head dim 32 or 64, degree 2 (ask pr_chunk_fwd_supported); other cases "
+                              "take pr_chunk_attention_fwd and pr_query_state_fwd");
+  if (bad_ptr(Q) || bad_ptr(K) || bad_ptr(V) || bad_opt(A) || bad_ptr(S) || bad_ptr(s) || bad_ptr(O) ||
+      bad_ptr(rowmax) || bad_ptr(den))
+    return fail(PR_ERR_ARG, "chunk_fwd: null or misaligned pointer");
+  if (BN <= 0 || n <= 0 || c <= 0 || h <= 0 || r <= 0 || BN % n != 0)
+    return fail(PR_ERR_ARG, "chunk_fwd: need BN,n,c,h,r > 0 and BN a multiple of n");
+  pr::ChunkFwdArgs a{Q, K, V, A, S, s, O, rowmax, den, c, h, r, n, scale, zero_initial_state ? 1 : 0};
+  return finish(pr::chunk_fwd(a, BN, d, dtype, (hipStream_t)stream), "chunk_fwd");
 }
 
 size_t pr_query_state_bwd_workspace(int BN, int c, int h, int r, int d, int dtype) {

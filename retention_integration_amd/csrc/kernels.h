@@ -66,6 +66,24 @@ struct NNArgs {
 };
 int sympow_nn(const NNArgs& a, int BN, int d, int mult, int epi, int dtype, hipStream_t st);
 
+// chunk_fwd.hip: attention inside every chunk, the query of the chunk's starting state and their merge, in one kernel
+struct ChunkFwdArgs {
+  const void* Q;     // [BN, c, h*r, d]  (ungated)
+  const void* K;     // [BN, c, h, d]
+  const void* V;     // [BN, c, h, d]
+  const float* G;    // [BN, c, h] accumulated log gates inside the chunk, or null
+  const void* S;     // [BN, h, D, d]   state at the start of each chunk, symmetric in the diagonal blocks
+  const float* s;    // [BN, h, D]
+  void* O;           // [BN, c, h*r, d]
+  float* rowmax;     // [BN, c, h*r]  log of the largest attention weight of the row
+  float* den;        // [BN, c, h*r]  normaliser, in the units sympow_nn's merge writes
+  int c, h, r, n;    // n: chunks per batch entry
+  float scale;
+  int skip_first;    // chunk 0 of every batch entry has a zero state (not read)
+};
+int chunk_fwd_supported(int d, int dtype);
+int chunk_fwd(const ChunkFwdArgs& a, int BN, int d, int dtype, hipStream_t st);
+
 // sympow_grad.hip
 struct GradArgs {
   const void* X;      // [BN, c, h*r, d]

@@ -40,8 +40,9 @@ FWD_TWO_STREAMS = True
 # The same for the whole query side of the backward: the query gradient through the state depends only on the
 # row-wise preparation, so it can run next to the chain  dS -> reverse scan -> dK, dV  instead of in front of it.
 BWD_TWO_STREAMS = True
-# Forward: the attention kernel needs only the gate sums, so it runs next to  key discount -> chunk states -> scan.
-FWD_TWO_STREAMS = True
+# Forward: attention inside the chunks, the query of the scanned states and their merge as one kernel where the library
+# has it (pr_chunk_fwd_supported); False runs the attention kernel and the state query with its merge epilogue.
+ONE_KERNEL_FWD = True
 _SIDE = {}
 
 
@@ -99,13 +100,16 @@ def chunked_fwd(Q: Tensor, K: Tensor, V: Tensor, log_G: Optional[Tensor], deg: i
         Kd_ = K
         lcs = torch.zeros((BN, h), dtype=f32, device=dev)
 
-    Ya = torch.empty_like(Q)
-    la, rm = _empty((BN, c, hq), f32, dev), _empty((BN, c, hq), f32, dev)
+    one_kernel = ONE_KERNEL_FWD and bool(lib.pr_chunk_fwd_supported(d, deg, code))
+    rm = _empty((BN, c, hq), f32, dev)
+    if not one_kernel:
+        Ya, la = torch.empty_like(Q), _empty((BN, c, hq), f32, dev)
 
     def attention(stream):
         _lib.check(lib.pr_attention_fwd(p(Q), p(K), p(V), p(A) if gated else None, p(Ya), p(la), p(rm), BN, c, c, h, r,
                                         d, scale, deg, 0, code, stream), "attention_fwd")
-    if FWD_TWO_STREAMS:
+    two_streams = FWD_TWO_STREAMS and not one_kernel
+    if two_streams:
         main, side = torch.cuda.current_stream(), _side_stream(dev)
         side.wait_stream(main)
         attention(side.cuda_stream)
@@ -133,11 +137,15 @@ def chunked_fwd(Q: Tensor, K: Tensor, V: Tensor, log_G: Optional[Tensor], deg: i
                                          D * d, D, code, st), "state_scan_fwd")
         del S, s
 
-    if FWD_TWO_STREAMS:
+    O, den = torch.empty_like(Q), _empty((BN, c, hq), f32, dev)
+    if one_kernel:
+        _lib.check(lib.pr_chunk_fwd(p(Q), p(K), p(V), p(A) if gated else None, p(Sc), p(sc), p(O), p(rm), p(den), BN, n,
+                                    c, h, r, d, scale, deg, 0 if carried else 1, code, st), "chunk_fwd")
+        return O, A, lcs, Kd, Sc, sc, rm, den, Sf, sf
+    if two_streams:
         main.wait_stream(side)
     else:
         attention(st)
-    O, den = torch.empty_like(Q), _empty((BN, c, hq), f32, dev)
     _lib.check(lib.pr_query_state_fwd(p(Q), p(Sc), p(sc), p(Ya), p(la), p(rm), p(A) if gated else None, p(O), p(den),
                                       BN, n, c, h, r, d, scale ** deg, deg, 0 if carried else 1, 1, code, st),
                "query_state_fwd")

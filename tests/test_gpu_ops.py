@@ -412,3 +412,72 @@ def test_state_scan_with_a_starting_value_and_a_final_entry(pra, dtype, d):
     check("dS_init", dY0, o[3].grad, GRAD_TOL)
     check("ds_init", dy0, o[4].grad, 1e-5)
     check("dlog_G", dlg, o[2].grad, GRAD_TOL)
+
+
+# ---------------------------------------------------------------- one-kernel forward of the chunks
+@pytest.mark.parametrize("d,c,r,gated,zis", [
+    (64, 128, 1, True, True),      # one full row block per (chunk, head)
+    (64, 256, 1, True, False),     # two row blocks, a state in every chunk
+    (64, 40, 3, True, True),       # 120 folded rows: a ragged row block, keys short of one tile
+    (32, 96, 2, True, False),      # d = 32; 192 folded rows (one full and one half row block), 1.5 key tiles
+    (64, 192, 1, False, True),     # no gates
+    (32, 16, 16, False, False),    # 16 query heads per kv head on a quarter of a key tile
+    (64, 1024, 1, True, True),     # the benchmark's chunk
+])
+def test_chunk_fwd_in_one_kernel(pra, d, c, r, gated, zis):
+    """pr_chunk_fwd against (a) the oracle's attention and query_state composed as the chunked algorithm composes them
+    (ref: retention/power_retention_maker.py:176-190: attention without normalisation inside the chunk, the gated
+    queries against the chunk's starting state, merged) and (b) the two library calls it replaces, whose rowmax and
+    normaliser it must reproduce because the backward kernels take them as they are."""
+    from retention_integration_amd import _lib
+    lib, st, p = _lib.load(), _lib.stream(), _lib.ptr
+    dtype = torch.bfloat16
+    code = _lib.dtype_code(dtype)
+    assert lib.pr_chunk_fwd_supported(d, 2, code) == 1
+    assert lib.pr_chunk_fwd_supported(128, 2, code) == 0 and lib.pr_chunk_fwd_supported(d, 2, _lib.dtype_code(torch.float16)) == 0
+    b, n, h = 2, 3, 2
+    BN, hq = b * n, h * r
+    D = oracle.expanded_dim(d)
+    f32 = torch.float32
+    scale = 1.0 / math.sqrt(d)
+    Q, K, V = (rnd(BN, c, hq, d, dtype=dtype, seed=80), rnd(BN, c, h, d, dtype=dtype, seed=81),
+               rnd(BN, c, h, d, dtype=dtype, seed=82))
+    A = gates(BN, c, h, seed=83).cumsum(1) if gated else None
+    # states that real keys produced (positive normaliser); chunk 0 of every batch entry zero when declared so
+    Ks, Vs = rnd(BN, 64, h, d, dtype=f32, scale=1.0, seed=84), rnd(BN, 64, h, d, dtype=f32, seed=85)
+    S, s = oracle.update_state(Ks, Vs, 2)
+    S = S.to(dtype)
+    if zis:
+        S.view(b, n, h, D, d)[:, 0] = 0
+        s.view(b, n, h, D)[:, 0] = 0
+
+    E = lambda *shape, dt=dtype: torch.empty(*shape, dtype=dt, device=DEV)  # noqa: E731
+    g = {k: dev(v) for k, v in dict(Q=Q, K=K, V=V, A=A, S=S, s=s).items()}
+    pa = p(g["A"]) if gated else None
+    O, rm, den = E(BN, c, hq, d), E(BN, c, hq, dt=f32), E(BN, c, hq, dt=f32)
+    _lib.check(lib.pr_chunk_fwd(p(g["Q"]), p(g["K"]), p(g["V"]), pa, p(g["S"]), p(g["s"]), p(O), p(rm), p(den), BN, n, c,
+                                h, r, d, scale, 2, 1 if zis else 0, code, st), "chunk_fwd")
+    # (b) the two calls
+    Ya, la, rm2, O2, den2 = E(BN, c, hq, d), E(BN, c, hq, dt=f32), E(BN, c, hq, dt=f32), E(BN, c, hq, d), E(BN, c, hq, dt=f32)
+    _lib.check(lib.pr_attention_fwd(p(g["Q"]), p(g["K"]), p(g["V"]), pa, p(Ya), p(la), p(rm2), BN, c, c, h, r, d, scale,
+                                    2, 0, code, st), "attention_fwd")
+    _lib.check(lib.pr_query_state_fwd(p(g["Q"]), p(g["S"]), p(g["s"]), p(Ya), p(la), p(rm2), pa, p(O2), p(den2), BN, n, c,
+                                      h, r, d, scale ** 2, 2, 1 if zis else 0, 1, code, st), "query_state_fwd")
+    torch.cuda.synchronize()
+    check("rowmax vs two calls", rm, rm2, 1e-6)
+    check("den vs two calls", den, den2, 2e-3)      # (the two calls take the attention sums through one more rounding)
+    check("O vs two calls", O, O2, 5e-3)
+
+    # (a) the oracle's composition, in fp32 on the same inputs; the query gate exp(A / 2) as the reference applies it
+    Qo = gold(Q).view(b, n, c, hq, d)
+    Ao = gold(A).view(b, n, c, h) if gated else None
+    Ya_o, la_o, rm_o = oracle.attention(gold(Q), gold(K), gold(V), gold(A), 2, scale=scale, norm=False)
+    if gated:
+        Qo = Qo * torch.exp(Ao / 2).repeat_interleave(r, dim=3)[..., None]
+    Oo = oracle.query_state(Qo, gold(S).view(b, n, h, D, d), gold(s).view(b, n, h, D), Ya_o.view(b, n, c, hq, d),
+                            la_o.view(b, n, c, hq), rm_o.view(b, n, c, hq), 2, scale, zis)
+    check("rowmax vs oracle", rm, rm_o, 1e-3)
+    check("O vs oracle", O.view(b, n, c, hq, d), Oo, OUT_TOL)
+    per_chunk = ((O.view(b, n, c, hq, d).float().cpu() - Oo).pow(2).sum((2, 4)).sqrt() / Oo.pow(2).sum((2, 4)).sqrt())
+    print(f"  worst (batch, chunk, head): {per_chunk.max().item():.3e}", flush=True)
+    assert per_chunk.max().item() <= OUT_TOL

@@ -13,6 +13,11 @@ import oracle
 pytestmark = pytest.mark.gpu
 
 OUT_TOL, GRAD_TOL = 1e-2, 2e-2
+# The fused node against the operator composition, rel-L2.  Both are checked against the oracle at the bars above; the
+# one-kernel forward keeps the attention part of a row in fp32 until the merge where the composition rounds it (and its
+# gradient) to 16 bits, which puts the two at 5.0e-3 to 6.1e-3 of each other on gradients, the fused node being the one
+# closer to the oracle.
+FUSED_VS_COMPOSED = 8e-3
 DEV = "cuda"
 G = os.path.join(os.path.dirname(__file__), "golden")
 
@@ -105,9 +110,9 @@ def test_fused_node_equals_operator_composition(pra, gated, r):
         Y.backward(dO)
         outs.append([Y] + [x.grad for x in xs if x is not None])
     for nm, a, b_ in zip(["Y", "dQ", "dK", "dV", "dlog_G"], *outs):
-        # (one bf16 rounding apart: the composed path rounds the attention part's output gradient to 16 bits, the
-        # fused path scales dO on the fly)
-        check(f"fused vs composed {nm}", a, b_, 6e-3)
+        # (two bf16 roundings apart: the composed path writes the attention part of the output and its gradient in 16
+        # bits, the fused path keeps the first in its accumulators and scales dO on the fly)
+        check(f"fused vs composed {nm}", a, b_, FUSED_VS_COMPOSED)
 
 
 def test_shape_sweep_fused_vs_composed_vs_oracle(pra):
@@ -133,7 +138,7 @@ def test_shape_sweep_fused_vs_composed_vs_oracle(pra):
             Y.backward(dO.to(DEV))
             outs.append([Y] + [x.grad for x in xs if x is not None])
         for nm, a, b_ in zip(["Y", "dQ", "dK", "dV", "dlog_G"], *outs):
-            check(f"fused vs composed {nm}", a, b_, 6e-3)
+            check(f"fused vs composed {nm}", a, b_, FUSED_VS_COMPOSED)
         xo = [x.float().clone().requires_grad_(True) if x is not None else None for x in (Q, K, V, lg)]
         Yo = oracle.power_retention(*xo, deg=2, chunk_size=chunk)
         Yo.backward(dO.float())
