@@ -109,25 +109,45 @@ def op_breakdown(pra, Q, K, V, lg, dO, cfg, iters=5):
     return {k: round(v, 4) for k, v in res.items()}
 
 
-def counter_run(pra, Q, K, V, cfg, dev):
-    """Three launches of sympow_grad alone and three plain copies of 256 MiB (read 256 MiB + write 256 MiB)."""
+def counter_run(pra, Q, K, V, lg, cfg, dev, kernel):
+    """For the byte counters (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE): three launches of one kernel alone, each followed
+    by a plain copy of 256 MiB (read 256 MiB + write 256 MiB) that calibrates the counter.  kernel: "sympow_grad" (the dK
+    half of update_state's backward) or "chunk_fwd" (the forward of all chunks in one kernel)."""
     from retention_integration_amd import _lib, ops
     b, t, h, d, c = cfg["b"], cfg["t"], cfg["h"], cfg["d"], cfg["chunk"]
     n = t // c
+    p, st = _lib.ptr, _lib.stream()
     with torch.no_grad():
         Kc, Vc = K.view(b, n, c, h, d), V.view(b, n, c, h, d)
         S, s = ops.update_state_fwd(Kc, Vc)
-        dK = torch.empty_like(Kc)
         lib = _lib.load()
+        code = _lib.dtype_code(Kc.dtype)
         src = torch.empty(256 * 1024 * 1024, dtype=torch.uint8, device=dev)
         dst = torch.empty_like(src)
+        if kernel == "sympow_grad":
+            dK = torch.empty_like(Kc)
+
+            def launch():
+                _lib.check(lib.pr_update_state_bwd(p(Kc), p(Vc), p(S), p(s), p(dK), None, b * n, c, h, d, 2, 1, 0, code, st),
+                           "update_state_bwd(dK)")
+        elif kernel == "chunk_fwd":
+            A = lg.view(b * n, c, h).cumsum(1).contiguous()
+            lcs = A[:, -1].contiguous().view(b, n, h)
+            Sc, sc = ops.discumsum_fwd(S, lcs, n), ops.discumsum_fwd(s, lcs, n)
+            O = torch.empty_like(Q)
+            rm, den = (torch.empty(b * n, c, h, dtype=torch.float32, device=dev) for _ in range(2))
+
+            def launch():
+                _lib.check(lib.pr_chunk_fwd(p(Q), p(K), p(V), p(A), p(Sc), p(sc), p(O), p(rm), p(den), b * n, n, c, h, 1, d,
+                                            d ** -0.5, 2, 1, code, st), "chunk_fwd")
+        else:
+            sys.exit(f"--counter-run: unknown kernel {kernel!r} (sympow_grad, chunk_fwd)")
         torch.cuda.synchronize()
         for _ in range(3):
-            _lib.check(lib.pr_update_state_bwd(_lib.ptr(Kc), _lib.ptr(Vc), _lib.ptr(S), _lib.ptr(s), _lib.ptr(dK), None,
-                                               b * n, c, h, d, 2, 1, 0, _lib.dtype_code(Kc.dtype), _lib.stream()), "grad")
+            launch()
             dst.copy_(src)
         torch.cuda.synchronize()
-    print("counter run done: 3 x sympow_grad, 3 x 256 MiB device copy")
+    print(f"counter run done: 3 x {kernel}, 3 x 256 MiB device copy")
 
 
 def attention_scaling(pra, dev, chunk):
@@ -421,9 +441,10 @@ def main():
     ap.add_argument("--no-breakdown", action="store_true", help="skip the per-operator timings")
     ap.add_argument("--no-decode", action="store_true", help="skip the inference (prefill + decode) leg")
     ap.add_argument("--no-short-chunks", action="store_true", help="skip the BASELINE configs[4] leg (short_chunks key)")
-    ap.add_argument("--counter-run", action="store_true",
-                    help="for rocprofv3 --pmc: launch only sympow_grad (dK of update_state backward) a few times, and a "
-                         "plain device copy of 256 MiB for calibrating byte counters")
+    ap.add_argument("--counter-run", nargs="?", const="sympow_grad", default=None, metavar="KERNEL",
+                    help="for rocprofv3 --pmc: launch only one kernel a few times -- sympow_grad (dK of update_state "
+                         "backward, the default) or chunk_fwd -- and a plain device copy of 256 MiB for calibrating "
+                         "byte counters")
     ap.add_argument("--attention-chunk", type=int, default=0,
                     help="for rocprofv3 --kernel-trace: run only the attention kernels, 64 times, with the headline's "
                          "rows cut into chunks of this length")
@@ -448,7 +469,7 @@ def main():
     cfg = CFG
     Q, K, V, lg, dO = make_inputs(cfg["b"], cfg["t"], cfg["h"], cfg["d"], dev)
     if args.counter_run:
-        counter_run(pra, Q, K, V, cfg, dev)
+        counter_run(pra, Q.detach(), K.detach(), V.detach(), lg.detach(), cfg, dev, args.counter_run)
         return
     leaves = [x.requires_grad_(True) for x in (Q, K, V, lg)]
 
