@@ -41,7 +41,7 @@ enum {
  * pr_update_state_bwd zero_last_of; pr_query_state_fwd / _bwd / _scan_bwd take q_log_gate and
  * pr_chunk_attention_bwd dQ_state_plain.  5: pr_query_state_fwd takes S_symmetric.  6: pr_set_launch_hook;
  * pr_decode_step takes up to 16 query rows per (batch, kv head); pr_state_scan_fwd / _bwd connect a scan to the calls
- * before and after it (S_init, S_final and their gradients).  7: pr_chunk_fwd, pr_chunk_fwd_supported. */
+ * before and after it (S_init, S_final and their gradients).  7: pr_chunk_fwd, pr_chunk_bwd_dq and their _supported queries. */
 int pr_abi_version(void);
 const char* pr_last_error(void);
 
@@ -217,6 +217,24 @@ int pr_chunk_fwd_supported(int d, int deg, int dtype);
 int pr_chunk_fwd(const void* Q, const void* K, const void* V, const float* A, const void* S, const float* s, void* O,
                  float* rowmax, float* den, int BN, int n, int c, int h, int r, int d, float scale, int deg,
                  int zero_initial_state, int dtype, void* stream);
+
+/* Query side of the chunked backward in one kernel: dQ and dGq of the attention inside every chunk
+ * (retention/_attention/triton.py:248-387) plus the query gradient through the chunk's starting state
+ * (retention/_query_state/triton.py:546-553) and its share of the gate gradient, (q . dQ_state) / deg -- what
+ * pr_query_state_bwd (its dQ kernel, q_log_gate = A, S_symmetric = 1) followed by pr_chunk_attention_bwd
+ * (dK == dV == NULL, dQ_state_plain = 1) compute, without the state-path gradient going to memory and back.
+ * bf16, d in {32, 64}, deg 2: pr_chunk_bwd_dq_supported() says whether the case exists; the others take the two calls.
+ *   Q, K, V, A, S, s as for pr_chunk_fwd; rowmax, den [BN,c,h*r] from it; dO [BN,c,h*r,d];
+ *   dl_attn, dY_scale [BN,c,h*r] and cvec [BN,c,h*r] fp32: the row vectors an earlier pr_query_state_bwd call on the
+ *   same inputs has written (its dl_attn and dY_scale outputs; cvec is the second part of its workspace, behind the
+ *   scaled dO: byte offset rows * d * 2 rounded up to 256, rows = BN*c*h*r) -- call it with dQ == dS == NULL for the
+ *   preparation alone
+ *   -> dQ [BN,c,h*r,d] (final), dGq [BN,c,h*r] fp32 (required when A is given). */
+int pr_chunk_bwd_dq_supported(int d, int deg, int dtype);
+int pr_chunk_bwd_dq(const void* Q, const void* K, const void* V, const float* A, const float* rowmax, const float* den,
+                    const void* dO, const float* dl_attn, const float* dY_scale, const float* cvec, const void* S,
+                    const float* s, void* dQ, float* dGq, int BN, int n, int c, int h, int r, int d, float scale,
+                    int deg, int zero_initial_state, int dtype, void* stream);
 
 /* Accumulated gates of the quadratic / inference paths -- log_G.cumsum(1), retention/power_retention_maker.py:129,
  * 348-349.  log_G, A [B,t,h] fp32, t <= 8192. */

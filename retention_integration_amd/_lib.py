@@ -37,6 +37,8 @@ SIGNATURES = {
     "pr_chunk_prep_fwd": (c_int, [_P] * 7 + [_I] * 7 + [_P]),
     "pr_chunk_fwd_supported": (c_int, [_I] * 3),
     "pr_chunk_fwd": (c_int, [_P] * 9 + [_I] * 6 + [_F, _I, _I, _I, _P]),
+    "pr_chunk_bwd_dq_supported": (c_int, [_I] * 3),
+    "pr_chunk_bwd_dq": (c_int, [_P] * 14 + [_I] * 6 + [_F, _I, _I, _I, _P]),
     "pr_gate_cumsum": (c_int, [_P] * 2 + [_I] * 3 + [_P]),
     "pr_state_scan_fwd": (c_int, [_P] * 9 + [_I] * 4 + [c_int64, c_int64, _I, _P]),
     "pr_state_chain_supported": (c_int, [_I] * 6),

@@ -13,7 +13,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 OUT = os.path.join(os.path.dirname(HERE), "libpower_retention_hip.so")
 SOURCES = ["capi", "discumsum", "sympow_tn", "sympow_nn", "sympow_grad", "attention_fwd", "attention_bwd", "elementwise",
-           "chunk_glue", "chunk_fwd", "decode", "cache"]
+           "chunk_glue", "chunk_fwd", "chunk_bwd_dq", "decode", "cache"]
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Xclang", "-target-feature", "-Xclang",
          "-packed-fp32-ops", "-Wno-unused-command-line-argument"]
 

@@ -244,6 +244,27 @@ int pr_chunk_fwd(const void* Q, const void* K, const void* V, const float* A, co
   return finish(pr::chunk_fwd(a, BN, d, dtype, (hipStream_t)stream), "chunk_fwd");
 }
 
+int pr_chunk_bwd_dq_supported(int d, int deg, int dtype) { return deg == 2 && pr::chunk_bwd_dq_supported(d, dtype); }
+
+int pr_chunk_bwd_dq(const void* Q, const void* K, const void* V, const float* A, const float* rowmax, const float* den,
+                    const void* dO, const float* dl_attn, const float* dY_scale, const float* cvec, const void* S,
+                    const float* s, void* dQ, float* dGq, int BN, int n, int c, int h, int r, int d, float scale,
+                    int deg, int zero_initial_state, int dtype, void* stream) {
+  if (int rc = check_common("chunk_bwd_dq", d, deg, dtype, true)) return rc;
+  if (!pr_chunk_bwd_dq_supported(d, deg, dtype))
+    return fail(PR_ERR_DTYPE, "chunk_bwd_dq: bf16, head dim 32 or 64, degree 2 (ask pr_chunk_bwd_dq_supported); other "
+                              "cases take pr_query_state_bwd and pr_chunk_attention_bwd");
+  if (bad_ptr(Q) || bad_ptr(K) || bad_ptr(V) || bad_opt(A) || bad_ptr(rowmax) || bad_ptr(den) || bad_ptr(dO) ||
+      bad_ptr(dl_attn) || bad_ptr(dY_scale) || bad_ptr(cvec) || bad_ptr(S) || bad_ptr(s) || bad_ptr(dQ) || bad_opt(dGq))
+    return fail(PR_ERR_ARG, "chunk_bwd_dq: null or misaligned pointer");
+  if (A && !dGq) return fail(PR_ERR_ARG, "chunk_bwd_dq: dGq is required when A is given");
+  if (BN <= 0 || n <= 0 || c <= 0 || h <= 0 || r <= 0 || BN % n != 0)
+    return fail(PR_ERR_ARG, "chunk_bwd_dq: need BN,n,c,h,r > 0 and BN a multiple of n");
+  pr::ChunkBwdDqArgs a{Q, K, V, A, rowmax, den, dO, dl_attn, dY_scale, cvec, S, s, dQ, A ? dGq : nullptr,
+                       c, h, r, n, scale, zero_initial_state ? 1 : 0};
+  return finish(pr::chunk_bwd_dq(a, BN, d, dtype, (hipStream_t)stream), "chunk_bwd_dq");
+}
+
 size_t pr_query_state_bwd_workspace(int BN, int c, int h, int r, int d, int dtype) {
   (void)dtype;
   const size_t rows = (size_t)BN * c * h * r;

@@ -84,6 +84,29 @@ struct ChunkFwdArgs {
 int chunk_fwd_supported(int d, int dtype);
 int chunk_fwd(const ChunkFwdArgs& a, int BN, int d, int dtype, hipStream_t st);
 
+// chunk_bwd_dq.hip: the query side of the chunked backward in one kernel (attention dQ/dGq + the state path's dQ)
+struct ChunkBwdDqArgs {
+  const void* Q;          // [BN, c, h*r, d] (ungated)
+  const void* K;          // [BN, c, h, d]
+  const void* V;          // [BN, c, h, d]
+  const float* G;         // [BN, c, h] accumulated log gates inside the chunk, or null
+  const float* rowmax;    // [BN, c, h*r]   from the forward
+  const float* den;       // [BN, c, h*r]   from the forward
+  const void* dO;         // [BN, c, h*r, d]
+  const float* dl;        // [BN, c, h*r]   gradient of the attention part's row sum (row-wise preparation)
+  const float* dO_scale;  // [BN, c, h*r]   factor on dO for the attention part (row-wise preparation)
+  const float* cvec;      // [BN, c, h*r]   factor of the key-sum term of the state part (row-wise preparation)
+  const void* S;          // [BN, h, D, d]  states at the start of each chunk, symmetric in the diagonal blocks
+  const float* s;         // [BN, h, D]
+  void* dQ;               // [BN, c, h*r, d]
+  float* dGq;             // [BN, c, h*r] or null
+  int c, h, r, n;         // n: chunks per batch entry
+  float scale;
+  int skip_first;         // chunk 0 of every batch entry has a zero state (not read)
+};
+int chunk_bwd_dq_supported(int d, int dtype);
+int chunk_bwd_dq(const ChunkBwdDqArgs& a, int BN, int d, int dtype, hipStream_t st);
+
 // sympow_grad.hip
 struct GradArgs {
   const void* X;      // [BN, c, h*r, d]

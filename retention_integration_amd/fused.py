@@ -43,6 +43,10 @@ BWD_TWO_STREAMS = True
 # Forward: attention inside the chunks, the query of the scanned states and their merge as one kernel where the library
 # has it (pr_chunk_fwd_supported); False runs the attention kernel and the state query with its merge epilogue.
 ONE_KERNEL_FWD = True
+# Backward, query side: the query gradient through the state and the query side of the attention backward as one kernel
+# where the library has it (pr_chunk_bwd_dq_supported); False runs sympow_grad and then the attention kernel, which adds
+# the former's result in its epilogue.
+ONE_KERNEL_BWD_DQ = True
 _SIDE = {}
 
 
@@ -198,7 +202,7 @@ def chunked_bwd(Q: Tensor, K: Tensor, V: Tensor, A: Tensor, lcs: Tensor, Kd: Ten
     dlcs = torch.empty_like(lcs)   # gate gradient of both scans
     dS0, ds0 = _empty((0,), dt, dev), _empty((0,), f32, dev)
     has_dfin = dSf is not None or dsf is not None
-    two_streams = False
+    two_streams = dq_one_kernel = False
     if not carried and not has_dfin and _chained(lib, b, n, c, h, r, d):
         ws = _empty((lib.pr_query_state_scan_bwd_workspace(b, n, c, h, r, d, code),), u8, dev)
         _lib.check(lib.pr_query_state_scan_bwd(p(Q), p(Sc), p(sc), p(rm), qgate, p(O), p(den), p(dO),
@@ -214,7 +218,21 @@ def chunked_bwd(Q: Tensor, K: Tensor, V: Tensor, A: Tensor, lcs: Tensor, Kd: Ten
             _lib.check(lib.pr_query_state_bwd(p(Q), p(Sc), p(sc), p(rm), qgate, p(O), p(den), p(dO), dQ_, dS_, ds_, None,
                                               p(dla), p(dys), p(qws), BN, n, c, h, r, d, scale ** deg, deg, zis, 1,
                                               prepared, code, stream), "query_state_bwd")
-        if BWD_TWO_STREAMS:
+        dq_one_kernel = ONE_KERNEL_BWD_DQ and bool(lib.pr_chunk_bwd_dq_supported(d, deg, code))
+        dQa = torch.empty_like(Q)
+        dGq = _empty((BN, c, hq), f32, dev) if gated else None
+
+        def query_side(stream):
+            # (the workspace of pr_query_state_bwd: the scaled dO, then the row vector of the key-sum term)
+            cvec = qws.data_ptr() + (BN * c * hq * d * 2 + 255) // 256 * 256
+            _lib.check(lib.pr_chunk_bwd_dq(p(Q), p(K), p(V), qgate, p(rm), p(den), p(dO), p(dla), p(dys), cvec, p(Sc),
+                                           p(sc), p(dQa), p(dGq), BN, n, c, h, r, d, scale, deg, 0 if carried else 1,
+                                           code, stream), "chunk_bwd_dq")
+        if dq_one_kernel:
+            qs_bwd(None, p(dSc), p(dsc), 0, st)          # preparation and dS; the query side follows further down
+            if not BWD_TWO_STREAMS:
+                query_side(st)
+        elif BWD_TWO_STREAMS:
             # The query gradient through the state (and, after it, the query side of the attention backward) depends
             # only on the row-wise preparation: it runs on a second stream next to the chain dS -> scan -> dK, dV.
             main, side = torch.cuda.current_stream(), _side_stream(dev)
@@ -238,16 +256,38 @@ def chunked_bwd(Q: Tensor, K: Tensor, V: Tensor, A: Tensor, lcs: Tensor, Kd: Ten
     dKd, dVs = torch.empty_like(K), torch.empty_like(V)
     # (dS comes from the kernels above, so both orders of a pair hold the same sum: the symmetry flag says so; the last
     # chunk's dS is zero unless a gradient arrived through the final state)
-    _lib.check(lib.pr_update_state_bwd(p(Kd), p(V), p(dS), p(ds), p(dKd), p(dVs), BN, c, h, d, deg, 1,
-                                       0 if has_dfin else n, code, st), "update_state_bwd")
+    if two_streams and dq_one_kernel:
+        # The one-kernel query side needs only the row-wise preparation, so where it runs is a matter of what it runs
+        # beside: started after dV, next to dK and the key side of the attention backward, the step is 15-25 us shorter
+        # than with it next to dS and the reverse scan (measured at every point of the chain).
+        def usb(dk_, dv_):
+            _lib.check(lib.pr_update_state_bwd(p(Kd), p(V), p(dS), p(ds), dk_, dv_, BN, c, h, d, deg, 1,
+                                               0 if has_dfin else n, code, st), "update_state_bwd")
+        main, side = torch.cuda.current_stream(), _side_stream(dev)
+        usb(None, p(dVs))
+        side.wait_stream(main)
+        query_side(side.cuda_stream)
+        usb(p(dKd), None)
+    else:
+        _lib.check(lib.pr_update_state_bwd(p(Kd), p(V), p(dS), p(ds), p(dKd), p(dVs), BN, c, h, d, deg, 1,
+                                           0 if has_dfin else n, code, st), "update_state_bwd")
 
     # the attention backward adds the state-path gradients in its epilogue and writes the final dQ, dK, dV
-    dQa, dKa, dVa = torch.empty_like(Q), torch.empty_like(K), torch.empty_like(V)
-    dGq = _empty((BN, c, hq), f32, dev) if gated else None
+    dKa, dVa = torch.empty_like(K), torch.empty_like(V)
+    if not dq_one_kernel:
+        dQa = torch.empty_like(Q)
+        dGq = _empty((BN, c, hq), f32, dev) if gated else None
     dGk = _empty((b, t, h), f32, dev) if gated else None
     dotk = _empty((BN, c, h), f32, dev) if gated else None
     Ag = p(A) if gated else None
-    if two_streams or ATTN_BWD_TWO_STREAMS:
+    if dq_one_kernel:
+        # the query side is done (or running on the second stream): the key side alone
+        _lib.check(lib.pr_chunk_attention_bwd(p(Q), p(K), p(V), Ag, p(rm), p(dO), p(dla), p(dys), None, p(dKd), p(dVs),
+                                              None, p(dKa), p(dVa), None, p(dGk), p(dotk), BN, c, h, r, d, scale, deg, 1,
+                                              code, st), "chunk_attention_bwd(dK, dV)")
+        if two_streams:
+            torch.cuda.current_stream().wait_stream(_side_stream(dev))
+    elif two_streams or ATTN_BWD_TWO_STREAMS:
         # the key side on the launch stream, the query side next to it on the second stream (which, with
         # BWD_TWO_STREAMS, already holds the state part of the query gradient)
         main, side = torch.cuda.current_stream(), _side_stream(dev)

@@ -701,3 +701,49 @@ def test_state_carried_across_calls(pra, dtype, b, t, h, r, d, chunk, gated, cut
     # (one random query against the state alone: numerator and denominator are cancelling sums over 16-bit state
     # entries, so the 16-bit state's own rounding -- a few 1e-3 -- shows amplified; the bar only has to catch a wrong pair)
     check("inference from the returned state", Yi, Yio, 5e-2)
+
+
+@pytest.mark.parametrize("b,t,h,r,d,chunk,gated,carried", [
+    (2, 512, 2, 1, 64, 128, True, False),     # one full row block per (chunk, head)
+    (1, 1024, 2, 1, 64, 256, True, True),     # two row blocks per chunk, a state in chunk 0 as well
+    (1, 495, 1, 3, 64, 40, True, False),      # padded length, ragged row blocks, keys short of one tile
+    (2, 384, 2, 2, 32, 96, False, False),     # d = 32, no gates, 1.5 key tiles
+    (1, 128, 1, 16, 32, 16, True, True),      # 16 query heads per kv head on a quarter of a key tile
+    (1, 4096, 2, 1, 64, 1024, True, False),   # the benchmark's chunk
+])
+def test_one_kernel_query_side_of_the_backward(pra, b, t, h, r, d, chunk, gated, carried):
+    """The query side of the backward as one kernel (pr_chunk_bwd_dq) against the two kernels it replaces -- the query
+    gradient through the state (sympow_grad) added in the attention kernel's epilogue -- and against the oracle: dQ and,
+    through the row sums that feed the gate scan, dlog_G; dK, dV do not depend on the choice and must not move."""
+    from retention_integration_amd import fused
+    Q, K, V, lg = make_inputs(b, t, h, r, d, torch.bfloat16, gated, seed=77)
+    dO = torch.randn(b, t, h * r, d, generator=torch.Generator().manual_seed(78)).to(torch.bfloat16)
+    st0 = None
+    if carried:
+        Kp, Vp, lgp = (x[:, :2 * chunk] if x is not None else None for x in (K, V, lg))
+        st0 = pra.power_retention(Q[:, :2 * chunk].to(DEV), Kp.to(DEV), Vp.to(DEV), None if lgp is None else lgp.to(DEV),
+                                  deg=2, chunk_size=chunk, return_final_state=True)[1]
+    outs = []
+    try:
+        for one in (True, False):
+            fused.ONE_KERNEL_BWD_DQ = one
+            xs = [x.to(DEV).requires_grad_(True) if x is not None else None for x in (Q, K, V, lg)]
+            Y = pra.power_retention(*xs, deg=2, chunk_size=chunk, initial_state=st0)
+            Y.backward(dO.to(DEV))
+            outs.append([Y] + [x.grad for x in xs if x is not None])
+    finally:
+        fused.ONE_KERNEL_BWD_DQ = True
+    names = ["Y", "dQ", "dK", "dV", "dlog_G"]
+    for nm, a, b_ in zip(names, *outs):
+        if nm in ("Y", "dK", "dV"):
+            assert torch.equal(a, b_), f"{nm} depends on the query side's kernels"
+        else:
+            check(f"one kernel vs two {nm}", a, b_, 5e-3)   # (the state part of dQ is not rounded to 16 bits on the way)
+    So = None
+    if carried:
+        So = tuple(x.float().cpu() for x in st0)
+    xo = [x.float().clone().requires_grad_(True) if x is not None else None for x in (Q, K, V, lg)]
+    Yo = oracle.power_retention(*xo, deg=2, chunk_size=chunk, initial_state=So)
+    Yo.backward(dO.float())
+    for nm, a, b_ in zip(names, outs[0], [Yo] + [x.grad for x in xo if x is not None]):
+        check(f"one kernel vs oracle {nm}", a, b_, OUT_TOL if nm == "Y" else GRAD_TOL)
