@@ -112,7 +112,8 @@ def op_breakdown(pra, Q, K, V, lg, dO, cfg, iters=5):
 def counter_run(pra, Q, K, V, lg, cfg, dev, kernel):
     """For the byte counters (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE): three launches of one kernel alone, each followed
     by a plain copy of 256 MiB (read 256 MiB + write 256 MiB) that calibrates the counter.  kernel: "sympow_grad" (the dK
-    half of update_state's backward) or "chunk_fwd" (the forward of all chunks in one kernel)."""
+    half of update_state's backward), "chunk_fwd" (the forward of all chunks in one kernel) or "chunk_bwd_dq" (the query
+    side of the backward in one kernel)."""
     from retention_integration_amd import _lib, ops
     b, t, h, d, c = cfg["b"], cfg["t"], cfg["h"], cfg["d"], cfg["chunk"]
     n = t // c
@@ -140,8 +141,26 @@ def counter_run(pra, Q, K, V, lg, cfg, dev, kernel):
             def launch():
                 _lib.check(lib.pr_chunk_fwd(p(Q), p(K), p(V), p(A), p(Sc), p(sc), p(O), p(rm), p(den), b * n, n, c, h, 1, d,
                                             d ** -0.5, 2, 1, code, st), "chunk_fwd")
+        elif kernel == "chunk_bwd_dq":
+            from retention_integration_amd import fused
+            O, A, _, _, Sc, sc, rm, den, _, _ = fused.chunked_fwd(Q, K, V, lg, 2, d ** -0.5, c)
+            dO = torch.randn_like(Q)
+            rows = b * t * h
+            qws = torch.empty(lib.pr_query_state_bwd_workspace(b * n, c, h, 1, d, code), dtype=torch.uint8, device=dev)
+            dla, dys = torch.empty_like(den), torch.empty_like(den)
+            # the row-wise preparation alone (no dQ, no dS): fills the workspace and the two row vectors
+            _lib.check(lib.pr_query_state_bwd(p(Q), p(Sc), p(sc), p(rm), p(A), p(O), p(den), p(dO), None, None, None, None,
+                                              p(dla), p(dys), p(qws), b * n, n, c, h, 1, d, 1.0 / d, 2, 2, 1, 0, code, st),
+                       "query_state_bwd(prep)")
+            cvec = qws.data_ptr() + (rows * d * 2 + 255) // 256 * 256
+            dQ, dGq = torch.empty_like(Q), torch.empty_like(den)
+
+            def launch():
+                _lib.check(lib.pr_chunk_bwd_dq(p(Q), p(K), p(V), p(A), p(rm), p(den), p(dO), p(dla), p(dys), cvec, p(Sc),
+                                               p(sc), p(dQ), p(dGq), b * n, n, c, h, 1, d, d ** -0.5, 2, 1, code, st),
+                           "chunk_bwd_dq")
         else:
-            sys.exit(f"--counter-run: unknown kernel {kernel!r} (sympow_grad, chunk_fwd)")
+            sys.exit(f"--counter-run: unknown kernel {kernel!r} (sympow_grad, chunk_fwd, chunk_bwd_dq)")
         torch.cuda.synchronize()
         for _ in range(3):
             launch()
@@ -285,11 +304,18 @@ class KernelTimers:
         self._cb = _lib.LAUNCH_HOOK(hook)   # (kept alive for as long as it is registered)
 
     def __enter__(self):
+        # One stream while the kernels are timed: a kernel timed while another one runs beside it says nothing about
+        # either (so the sum of these times exceeds a step of the node as it normally runs).
+        from retention_integration_amd import fused
+        self._flags = (fused.FWD_TWO_STREAMS, fused.BWD_TWO_STREAMS, fused.ATTN_BWD_TWO_STREAMS)
+        fused.FWD_TWO_STREAMS = fused.BWD_TWO_STREAMS = fused.ATTN_BWD_TWO_STREAMS = False
         self.lib.pr_set_launch_hook(self._cb, None)
         return self
 
     def __exit__(self, *exc):
+        from retention_integration_amd import fused
         self.lib.pr_set_launch_hook(None, None)
+        fused.FWD_TWO_STREAMS, fused.BWD_TWO_STREAMS, fused.ATTN_BWD_TWO_STREAMS = self._flags
 
     def end_step(self):
         self.steps.append(self.records)
@@ -324,7 +350,7 @@ def kernel_work(cfg, D_stored):
     return {
         "sympow_tn": ("mfma", state), "sympow_nn": ("mfma", state), "sympow_grad": ("mfma", state),
         "attention_fwd": ("mfma", 2.0 * attn), "chunk_fwd": ("mfma", 2.0 * attn + state),
-        "attention_bwd_dkv": ("mfma", 3.0 * attn),
+        "attention_bwd_dkv": ("mfma", 3.0 * attn), "chunk_bwd_dq": ("mfma", 2.0 * attn + state),
         "attention_bwd_dq": ("mfma", 2.0 * attn),
         "discumsum_pair_fwd": ("hbm", 2.0 * St * (n - 1) / n), "discumsum_pair_bwd": ("hbm", 3.0 * St * (n - 1) / n),
         "qs_bwd_prep": ("hbm", 3.0 * R), "gate_apply_fwd": ("hbm", 2.0 * R), "chunk_prep_fwd": ("hbm", 2.0 * R),
@@ -443,7 +469,7 @@ def main():
     ap.add_argument("--no-short-chunks", action="store_true", help="skip the BASELINE configs[4] leg (short_chunks key)")
     ap.add_argument("--counter-run", nargs="?", const="sympow_grad", default=None, metavar="KERNEL",
                     help="for rocprofv3 --pmc: launch only one kernel a few times -- sympow_grad (dK of update_state "
-                         "backward, the default) or chunk_fwd -- and a plain device copy of 256 MiB for calibrating "
+                         "backward, the default), chunk_fwd or chunk_bwd_dq -- and a plain device copy of 256 MiB for calibrating "
                          "byte counters")
     ap.add_argument("--attention-chunk", type=int, default=0,
                     help="for rocprofv3 --kernel-trace: run only the attention kernels, 64 times, with the headline's "
@@ -587,17 +613,22 @@ def main():
     traffic, traffic_src = measured_traffic(base + "_t65536_hbm_traffic.txt")
     blk["traffic"], blk["traffic_source"] = traffic, traffic_src
     out["roofline"] = blk
+    # The attention backward: its two kernels together (canonical 5 products) where both run; where the query side is
+    # one kernel with the query gradient through the state (chunk_bwd_dq), that kernel and the key side on their own.
     ab = [k for k in in_step_ms if k.startswith("attention_bwd_")]
-    if ab:
+    if len(ab) == 2:
         ms = sum(in_step_ms[k] for k in ab)
         out["roofline_attention_bwd"] = roofline_block(" + ".join(ab), ms, ("mfma", 5.0 * bh * n * cfg["d"] * cfg["chunk"] * (cfg["chunk"] + 1)))
+    for key, label in (("roofline_attention_bwd_dkv", "attention_bwd_dkv#0"), ("roofline_chunk_bwd_dq", "chunk_bwd_dq#0")):
+        if label in in_step_ms and len(ab) != 2:
+            out[key] = roofline_block(label, in_step_ms[label], work[label.split("#")[0]])
     # (forward: one kernel for the attention inside the chunks, the state query and their merge where the library has it,
     # else attention_fwd and sympow_nn#0; sympow_nn's other launch is update_state's dV)
     one_kernel = "chunk_fwd#0" in in_step_ms
     for key, label in (("roofline_chunk_fwd", "chunk_fwd#0"), ("roofline_attention_fwd", "attention_fwd#0"),
                        ("roofline_update_state_fwd", "sympow_tn#0"),
                        ("roofline_update_state_bwd_dV" if one_kernel else "roofline_query_state_fwd", "sympow_nn#0"),
-                       ("roofline_update_state_bwd_dK", "sympow_grad#1"),
+                       ("roofline_update_state_bwd_dK", "sympow_grad#0" if "chunk_bwd_dq#0" in in_step_ms else "sympow_grad#1"),
                        ("roofline_state_scan_fwd", "discumsum_pair_fwd#0"), ("roofline_state_scan_bwd", "discumsum_pair_bwd#0")):
         if label in in_step_ms:
             out[key] = roofline_block(label, in_step_ms[label], work[label.split("#")[0]])

@@ -24,6 +24,7 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Xclang", "-tar
 # under max-ilp and max-memory-clause).
 FILE_FLAGS = {
     "attention_bwd": ["-mllvm", "-amdgpu-sched-strategy=max-memory-clause"],
+    "chunk_bwd_dq": ["-mllvm", "-amdgpu-sched-strategy=max-memory-clause"],
     "sympow_grad": ["-mllvm", "-amdgpu-sched-strategy=max-memory-clause"],
     "sympow_tn": ["-mllvm", "-amdgpu-use-amdgpu-trackers=1"],
 }
