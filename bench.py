@@ -467,6 +467,7 @@ def main():
     ap.add_argument("--no-breakdown", action="store_true", help="skip the per-operator timings")
     ap.add_argument("--no-decode", action="store_true", help="skip the inference (prefill + decode) leg")
     ap.add_argument("--no-short-chunks", action="store_true", help="skip the BASELINE configs[4] leg (short_chunks key)")
+    ap.add_argument("--no-chained-calls", action="store_true", help="skip the state_across_calls leg")
     ap.add_argument("--counter-run", nargs="?", const="sympow_grad", default=None, metavar="KERNEL",
                     help="for rocprofv3 --pmc: launch only one kernel a few times -- sympow_grad (dK of update_state "
                          "backward, the default), chunk_fwd or chunk_bwd_dq -- and a plain device copy of 256 MiB for calibrating "
@@ -647,24 +648,25 @@ def main():
             out["decode"] = decode_bench(pra, dev)
     # chunked prefill: the forward of the same sequence in one call and in two calls that hand the state over
     # (initial_state / return_final_state), each timed like the breakdown entries (HIP events after a lead-in)
-    with torch.no_grad():
-        half = cfg["t"] // 2
-        dq, dk, dv, dg = detach
+    if not args.no_chained_calls:
+        with torch.no_grad():
+            half = cfg["t"] // 2
+            dq, dk, dv, dg = detach
 
-        def one_call():
-            return pra.power_retention(dq, dk, dv, dg, deg=cfg["deg"], chunk_size=cfg["chunk"])
+            def one_call():
+                return pra.power_retention(dq, dk, dv, dg, deg=cfg["deg"], chunk_size=cfg["chunk"])
 
-        def two_calls():
-            y1, st = pra.power_retention(dq[:, :half], dk[:, :half], dv[:, :half], dg[:, :half], deg=cfg["deg"],
-                                         chunk_size=cfg["chunk"], return_final_state=True)
-            y2 = pra.power_retention(dq[:, half:], dk[:, half:], dv[:, half:], dg[:, half:], deg=cfg["deg"],
-                                     chunk_size=cfg["chunk"], initial_state=st)
-            return y1, y2
-        t1, t2 = event_time_ms(one_call, 10), event_time_ms(two_calls, 10)
-        out["state_across_calls"] = {"forward_one_call_ms": round(t1, 4), "forward_two_calls_ms": round(t2, 4),
-                                     "ratio": round(t2 / t1, 4),
-                                     "workload": "forward only, the headline sequence whole vs as two halves chained "
-                                                 "through (state, sum_of_keys)"}
+            def two_calls():
+                y1, st = pra.power_retention(dq[:, :half], dk[:, :half], dv[:, :half], dg[:, :half], deg=cfg["deg"],
+                                             chunk_size=cfg["chunk"], return_final_state=True)
+                y2 = pra.power_retention(dq[:, half:], dk[:, half:], dv[:, half:], dg[:, half:], deg=cfg["deg"],
+                                         chunk_size=cfg["chunk"], initial_state=st)
+                return y1, y2
+            t1, t2 = event_time_ms(one_call, 10), event_time_ms(two_calls, 10)
+            out["state_across_calls"] = {"forward_one_call_ms": round(t1, 4), "forward_two_calls_ms": round(t2, 4),
+                                         "ratio": round(t2 / t1, 4),
+                                         "workload": "forward only, the headline sequence whole vs as two halves chained "
+                                                     "through (state, sum_of_keys)"}
     if not args.no_short_chunks:
         torch.cuda.empty_cache()
         sc = short_chunks(pra, dev, 5, 2)
