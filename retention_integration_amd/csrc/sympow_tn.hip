@@ -74,6 +74,27 @@ template <int J> struct PhiDiag<f16_t, J> {
 };
 constexpr int TN_NDIAG = 9;   // fragments of a diagonal block
 
+// Writes a wave's 16 x 16 accumulator tile (lane: feature rows 4g+v of value column c0 + lane%16, already rounded:
+// pk = {row 4g | row 4g+1 << 16, row 4g+2 | row 4g+3 << 16}) into a row-major LDS buffer of pitch TP bytes.  Neighbouring
+// lanes hold neighbouring columns, so a lane pair first trades halves (one DPP move): the even lane then owns rows 4g,
+// 4g+1 of both columns and the odd lane rows 4g+2, 4g+3 -- two 4-byte writes per lane instead of four 2-byte ones
+// (the 2-byte form cost the chained kernel a quarter of its time in LDS instructions).
+// wbase: tb + (4g + 2 (lane & 1)) * TP + 2 (lane%16 & ~1), + 2 * column offset; sel_a / sel_b: byte selectors of the
+// lane's parity (tn_pair_selectors).
+__device__ __forceinline__ void tn_pair_selectors(uint32_t& sel_a, uint32_t& sel_b) {
+  const bool odd = lane_id() & 1;
+  sel_a = odd ? 0x01000504u : 0x05040100u;
+  sel_b = odd ? 0x03020706u : 0x07060302u;
+}
+__device__ __forceinline__ void tn_write_pair(u32x2 pk, uint32_t addr, int TP, uint32_t sel_a, uint32_t sel_b) {
+  typedef __attribute__((address_space(3))) uint32_t lds_u32;
+  const bool odd = lane_id() & 1;
+  const uint32_t send = odd ? pk[0] : pk[1], keep = odd ? pk[1] : pk[0];
+  const uint32_t recv = (uint32_t)__builtin_amdgcn_mov_dpp((int)send, 0xB1, 0xf, 0xf, true);   // quad_perm [1,0,3,2]
+  *(lds_u32*)addr = __builtin_amdgcn_perm(recv, keep, sel_a);
+  *(lds_u32*)(addr + TP) = __builtin_amdgcn_perm(recv, keep, sel_b);
+}
+
 // The diagonal block's counterpart of tn_store_rows below: fragment J's row i is feature (i, i') with
 // i' = (i - J) mod 16, stored at 16 i + i' and at 16 i' + i.  S, s point at the block's first feature.
 template <typename T, int DV>
@@ -83,7 +104,9 @@ __device__ __forceinline__ void tn_store_diag(const f32x4 (&acc)[TN_NDIAG][DV / 
   typedef __attribute__((address_space(3))) u32x4 lds_u32x4;
   constexpr int NT = DV / 16, TP = DV * 2 + 16;
   const int l = lane_id(), g = l >> 4, sl = l & 15;
-  const uint32_t tb_w = tb + 4 * g * TP + sl * 2;
+  const uint32_t tb_w = tb + (4 * g + 2 * (sl & 1)) * TP + (sl & ~1) * 2;
+  uint32_t sel_a, sel_b;
+  tn_pair_selectors(sel_a, sel_b);
   static_for<TN_NDIAG>([&](auto ji) {
     constexpr int J = decltype(ji)::value;
 #pragma unroll
@@ -91,11 +114,7 @@ __device__ __forceinline__ void tn_store_diag(const f32x4 (&acc)[TN_NDIAG][DV / 
       float o[4];
 #pragma unroll
       for (int v = 0; v < 4; v++) o[v] = acc[J][nt][v];
-      const u32x2 pk = __builtin_bit_cast(u32x2, pack4<T>(o));
-      *(lds_u16*)(tb_w + 32 * nt) = (unsigned short)pk[0];
-      *(lds_u16*)(tb_w + 32 * nt + TP) = (unsigned short)(pk[0] >> 16);
-      *(lds_u16*)(tb_w + 32 * nt + 2 * TP) = (unsigned short)pk[1];
-      *(lds_u16*)(tb_w + 32 * nt + 3 * TP) = (unsigned short)(pk[1] >> 16);
+      tn_write_pair(__builtin_bit_cast(u32x2, pack4<T>(o)), tb_w + 32 * nt, TP, sel_a, sel_b);
     }
     asm volatile("" ::: "memory");   // (LDS operations of one wave execute in order)
 #pragma unroll
@@ -121,7 +140,9 @@ __device__ __forceinline__ void tn_store_rows(const f32x4 (&acc)[XPW][DV / 16], 
   typedef __attribute__((address_space(3))) u32x4 lds_u32x4;
   constexpr int NT = DV / 16, TP = DV * 2 + 16;
   const int l = lane_id(), g = l >> 4, sl = l & 15;
-  const uint32_t tb_w = tb + 4 * g * TP + sl * 2;   // + 32*nt (+ v*TP): rows 4g+v of column 16nt+sl
+  const uint32_t tb_w = tb + (4 * g + 2 * (sl & 1)) * TP + (sl & ~1) * 2;   // + 32*nt (+ TP): see tn_write_pair
+  uint32_t sel_a, sel_b;
+  tn_pair_selectors(sel_a, sel_b);
   static_for<XPW>([&](auto xi) {
     constexpr int X = PART * XPW + decltype(xi)::value;
 #pragma unroll
@@ -129,11 +150,7 @@ __device__ __forceinline__ void tn_store_rows(const f32x4 (&acc)[XPW][DV / 16], 
       float o[4];
 #pragma unroll
       for (int v = 0; v < 4; v++) o[v] = acc[xi.value][nt][v] * mul;
-      const u32x2 pk = __builtin_bit_cast(u32x2, pack4<T>(o));
-      *(lds_u16*)(tb_w + 32 * nt) = (unsigned short)pk[0];
-      *(lds_u16*)(tb_w + 32 * nt + TP) = (unsigned short)(pk[0] >> 16);
-      *(lds_u16*)(tb_w + 32 * nt + 2 * TP) = (unsigned short)pk[1];
-      *(lds_u16*)(tb_w + 32 * nt + 3 * TP) = (unsigned short)(pk[1] >> 16);
+      tn_write_pair(__builtin_bit_cast(u32x2, pack4<T>(o)), tb_w + 32 * nt, TP, sel_a, sel_b);
     }
     asm volatile("" ::: "memory");   // (LDS operations of one wave execute in order)
     char* dst = (char*)(S + 16 * X * DV);
