@@ -103,7 +103,7 @@ def op_breakdown(pra, Q, K, V, lg, dO, cfg, iters=5):
     lib = _lib.load()
     dK = torch.empty_like(Kc)
     grad_only = lambda: _lib.check(lib.pr_update_state_bwd(  # noqa: E731
-        _lib.ptr(Kc), _lib.ptr(Vc), _lib.ptr(S), _lib.ptr(s), _lib.ptr(dK), None, b * n, c, h, d, 2, 1, 0,
+        _lib.ptr(Kc), _lib.ptr(Vc), _lib.ptr(S), _lib.ptr(s), None, None, None, None, _lib.ptr(dK), None, b * n, c, h, d, 2, 1, 0,
         _lib.dtype_code(Kc.dtype), _lib.stream()), "update_state_bwd(dK)")
     res["sympow_grad(dK)"] = event_time_ms(grad_only, iters)
     return {k: round(v, 4) for k, v in res.items()}
@@ -129,7 +129,8 @@ def counter_run(pra, Q, K, V, lg, cfg, dev, kernel):
             dK = torch.empty_like(Kc)
 
             def launch():
-                _lib.check(lib.pr_update_state_bwd(p(Kc), p(Vc), p(S), p(s), p(dK), None, b * n, c, h, d, 2, 1, 0, code, st),
+                _lib.check(lib.pr_update_state_bwd(p(Kc), p(Vc), p(S), p(s), None, None, None, None, p(dK), None, b * n, c, h, d,
+                                                   2, 1, 0, code, st),
                            "update_state_bwd(dK)")
         elif kernel == "chunk_fwd":
             A = lg.view(b * n, c, h).cumsum(1).contiguous()
@@ -139,25 +140,28 @@ def counter_run(pra, Q, K, V, lg, cfg, dev, kernel):
             rm, den = (torch.empty(b * n, c, h, dtype=torch.float32, device=dev) for _ in range(2))
 
             def launch():
-                _lib.check(lib.pr_chunk_fwd(p(Q), p(K), p(V), p(A), p(Sc), p(sc), p(O), p(rm), p(den), b * n, n, c, h, 1, d,
+                _lib.check(lib.pr_chunk_fwd(p(Q), p(K), p(V), p(A), p(Sc), p(sc), None, None, None, p(O), p(rm), p(den), b * n, n,
+                                            c, h, 1, d,
                                             d ** -0.5, 2, 1, code, st), "chunk_fwd")
         elif kernel == "chunk_bwd_dq":
             from retention_integration_amd import fused
-            O, A, _, _, Sc, sc, rm, den, _, _ = fused.chunked_fwd(Q, K, V, lg, 2, d ** -0.5, c)
+            O, A, _, _, Sc, sc, rm, den = fused.chunked_fwd(Q, K, V, lg, 2, d ** -0.5, c)[:8]
             dO = torch.randn_like(Q)
             rows = b * t * h
             qws = torch.empty(lib.pr_query_state_bwd_workspace(b * n, c, h, 1, d, code), dtype=torch.uint8, device=dev)
             dla, dys = torch.empty_like(den), torch.empty_like(den)
             # the row-wise preparation alone (no dQ, no dS): fills the workspace and the two row vectors
             _lib.check(lib.pr_query_state_bwd(p(Q), p(Sc), p(sc), p(rm), p(A), p(O), p(den), p(dO), None, None, None, None,
-                                              p(dla), p(dys), p(qws), b * n, n, c, h, 1, d, 1.0 / d, 2, 2, 1, 0, code, st),
+                                              p(dla), p(dys), p(qws), None, b * n, n, c, h, 1, d, 1.0 / d, 2, 2, 1, 0, code,
+                                              st),
                        "query_state_bwd(prep)")
             cvec = qws.data_ptr() + (rows * d * 2 + 255) // 256 * 256
             dQ, dGq = torch.empty_like(Q), torch.empty_like(den)
 
             def launch():
                 _lib.check(lib.pr_chunk_bwd_dq(p(Q), p(K), p(V), p(A), p(rm), p(den), p(dO), p(dla), p(dys), cvec, p(Sc),
-                                               p(sc), p(dQ), p(dGq), b * n, n, c, h, 1, d, d ** -0.5, 2, 1, code, st),
+                                               p(sc), None, None, None, p(dQ), p(dGq), b * n, n, c, h, 1, d, d ** -0.5, 2, 1,
+                                               code, st),
                            "chunk_bwd_dq")
         else:
             sys.exit(f"--counter-run: unknown kernel {kernel!r} (sympow_grad, chunk_fwd, chunk_bwd_dq)")

@@ -41,7 +41,10 @@ enum {
  * pr_update_state_bwd zero_last_of; pr_query_state_fwd / _bwd / _scan_bwd take q_log_gate and
  * pr_chunk_attention_bwd dQ_state_plain.  5: pr_query_state_fwd takes S_symmetric.  6: pr_set_launch_hook;
  * pr_decode_step takes up to 16 query rows per (batch, kv head); pr_state_scan_fwd / _bwd connect a scan to the calls
- * before and after it (S_init, S_final and their gradients).  7: pr_chunk_fwd, pr_chunk_bwd_dq and their _supported queries. */
+ * before and after it (S_init, S_final and their gradients).  7: pr_chunk_fwd, pr_chunk_bwd_dq and their _supported queries.
+ * 8: pr_set_gate_skipping / pr_get_gate_skipping; live_rows of pr_chunk_prep_fwd, pr_update_state_fwd / _bwd and
+ * pr_query_state_bwd; consumers_follow_gates of pr_state_scan_fwd / _bwd and the *_scan_in arguments of pr_chunk_fwd,
+ * pr_chunk_bwd_dq and pr_update_state_bwd. */
 int pr_abi_version(void);
 const char* pr_last_error(void);
 
@@ -53,6 +56,18 @@ const char* pr_last_error(void);
  * library.  The hook must not call back into the library. */
 typedef void (*pr_launch_hook_t)(const char* kernel, int phase, void* stream, void* user);
 void pr_set_launch_hook(pr_launch_hook_t hook, void* user);
+
+/* Gate skipping (no counterpart in the reference, whose kernels visit every tile below the diagonal:
+ * retention/_attention/impl_triton.py, retention/_query_state/impl_triton.py).  Accumulated log gates only fall along a
+ * chunk, and a weight exp(A_i - A_j) of a query i on a key j that underflows fp32 IS zero in the reference's arithmetic
+ * too (so is the factor exp(A_i) on the state part of a row, and the factor exp((A_last - A_j) / deg) on a key's
+ * contribution to the next state).  With skipping on (the default) the kernels leave out the key tiles, state sweeps and
+ * row blocks whose every term is such an exact zero, instead of multiplying through them; results are the same bit for
+ * bit wherever a kernel decides per tile, and gates that do not decay that far (|A| below about 87 inside a chunk)
+ * change nothing at all.  Off: every tile is visited, whatever the gates -- the data-independent cost.  Process-wide;
+ * set it while no other thread is inside the library. */
+void pr_set_gate_skipping(int on);
+int pr_get_gate_skipping(void);
 
 /* Size D of the expanded state for head dim d: 256 * T(T+1)/2, T = d/16; -1 if d is not a multiple of 16.
  * Replaces retention/_utils.py:18-19 compute_expanded_dim. */
@@ -85,9 +100,11 @@ int pr_attention_bwd(const void* Q, const void* K, const void* V, const float* G
  * Triton twin retention/_update_state/triton.py:61-133,280-320.
  *   K, V [BN,c,h,d] (BN = b*n chunks) -> S [BN,h,D,d], s [BN,h,D] fp32.
  *   skip_last_of = n > 0: the last of every n chunks is not computed and its S, s are left unwritten (the composed
- *   function never reads the last chunk's state, retention/power_retention_maker.py:168-170); 0 computes every chunk. */
-int pr_update_state_fwd(const void* K, const void* V, void* S, float* s, int BN, int c, int h, int d, int deg,
-                        int skip_last_of, int dtype, void* stream);
+ *   function never reads the last chunk's state, retention/power_retention_maker.py:168-170); 0 computes every chunk.
+ *   live_rows (NULL, or the [BN,h,2] int32 array that pr_chunk_prep_fwd wrote for the gates that discounted K): the
+ *   time steps before live_rows[bn,h,0] hold keys that the discount turned into exact zeros and are not read. */
+int pr_update_state_fwd(const void* K, const void* V, void* S, float* s, const int* live_rows, int BN, int c, int h,
+                        int d, int deg, int skip_last_of, int dtype, void* stream);
 
 /* Backward -- retention/_update_state/reference.py:55-83, Triton twin retention/_update_state/triton.py:148-260.
  *   dS [BN,h,D,d], ds [BN,h,D] fp32 -> dK, dV [BN,c,h,d]; one of dK, dV may be NULL (that gradient is skipped).
@@ -96,8 +113,15 @@ int pr_update_state_fwd(const void* K, const void* V, void* S, float* s, int BN,
  *   an arbitrary tensor.  The key gradient then takes a shorter path through those blocks; with 0 every feature is
  *   used as given, as the reference does.
  *   zero_last_of = n > 0 is the promise that dS, ds of the last of every n chunks are zero (that chunk's state feeds
- *   nothing): they are not read and dK, dV are written as zeros there; 0 makes no such promise. */
-int pr_update_state_bwd(const void* K, const void* V, const void* dS, const float* ds, void* dK, void* dV, int BN,
+ *   nothing): they are not read and dK, dV are written as zeros there; 0 makes no such promise.
+ *   live_rows (NULL, or what pr_chunk_prep_fwd wrote for the gates that discounted K): the time steps before
+ *   live_rows[bn,h,0] hold keys that are exact zeros; dK, dV are written as zeros there and not computed.
+ *   dS_scan_in, ds_scan_in, scan_log_G (all NULL, or all given together with zero_last_of = n): dS, ds are the output of
+ *   pr_state_scan_bwd and these its inputs dS_out, ds_out, log_G.  Entry k of that scan equals its input entry k + 1
+ *   bit for bit when exp(scan_log_G[k + 1]) == 0; the kernels then read the input entry (see consumers_follow_gates
+ *   of pr_state_scan_bwd). */
+int pr_update_state_bwd(const void* K, const void* V, const void* dS, const float* ds, const void* dS_scan_in,
+                        const float* ds_scan_in, const float* scan_log_G, const int* live_rows, void* dK, void* dV, int BN,
                         int c, int h, int d, int deg, int dS_symmetric, int zero_last_of, int dtype, void* stream);
 
 /* discumsum(X, log_G) -- retention/_discumsum/reference.py:3-15, Triton twin retention/_discumsum/triton.py:34-94.
@@ -124,15 +148,23 @@ int pr_discumsum_bwd(const void* dY, const void* Y, const float* log_G, void* dX
  *   S_init [B,H,F], s_init [B,H,F2] or both NULL: the scans start from them (entry 0 = S_init) instead of zero;
  *   S_final, s_final or both NULL (n_out == n only): receive entry n, exp(log_G[n-1]) * entry n-1 + S[n-1].
  *   Backward: dS_final / ds_final (NULL = zero) is the gradient of that entry n, dS_init / ds_init (NULL = not wanted)
- *   receive the gradient of the starting value. */
+ *   receive the gradient of the starting value.
+ * consumers_follow_gates != 0 (honoured only without S_init / S_final resp. dS_final / dS_init, with n_out == n, and
+ * while gate skipping is on) is the caller's promise that every reader of the scan's output takes the scan's INPUT
+ * wherever the two are equal bit for bit because the carry into the entry is an exact zero -- forward: entry k is input
+ * k - 1 when exp(log_G[k-1]) == 0 or k == 1, and entry 0 (zero) is not read; backward: entry k is input k + 1 when
+ * exp(log_G[k+1]) == 0, and entry n - 1 (zero) is not read.  pr_chunk_fwd, pr_chunk_bwd_dq (S_scan_in ...) and
+ * pr_update_state_bwd (dS_scan_in ...) are such readers.  A (batch, head) whose every factor exp(log_G[k]), k >= 1, is
+ * zero is then not scanned: nothing of it is read, its output entries are left unwritten and, backward, its gate
+ * gradient is written as zero. */
 int pr_state_scan_fwd(const void* S, const float* s, const float* log_G, void* S_out, float* s_out,
                       const void* S_init, const float* s_init, void* S_final, float* s_final, int B, int n,
-                      int n_out, int H, int64_t F, int64_t F2, int dtype, void* stream);
+                      int n_out, int H, int64_t F, int64_t F2, int consumers_follow_gates, int dtype, void* stream);
 size_t pr_state_scan_bwd_workspace(int B, int n, int H, int64_t F, int64_t F2);
 int pr_state_scan_bwd(const void* dS_out, const void* S_out, const float* ds_out, const float* s_out,
                       const float* log_G, void* dS, float* ds, float* dlog_G, void* workspace, const void* dS_final,
                       const float* ds_final, void* dS_init, float* ds_init, int B, int n, int n_out,
-                      int H, int64_t F, int64_t F2, int dtype, void* stream);
+                      int H, int64_t F, int64_t F2, int consumers_follow_gates, int dtype, void* stream);
 
 /* Short chunks: update_state followed by the scan that keeps its first n entries
  * (retention/power_retention_maker.py:156,167-170) as ONE pass that never writes the per-chunk states:
@@ -194,13 +226,16 @@ int pr_query_state_fwd(const void* Q, const void* S, const float* s, const void*
  *   The call is three kernels: the row-wise preparation (fills the workspace, dY_attn / dY_scale, dl_attn), dS / ds, and
  *   dQ.  With dS == ds == NULL or dQ == NULL that kernel is skipped; prepared != 0 says that an earlier call with the
  *   same inputs has filled this workspace and skips the preparation -- so the two contractions, which do not depend
- *   on each other, can be issued as two calls on two streams. */
+ *   on each other, can be issued as two calls on two streams.
+ *   live_rows (NULL, or the [BN,h,2] int32 array that pr_chunk_prep_fwd wrote for the gates in q_log_gate): from time
+ *   step live_rows[bn,h,1] on, the factor exp(q_log_gate) has underflowed to zero, the state part of those rows has a
+ *   zero gradient, and the dS / ds contraction does not read them. */
 size_t pr_query_state_bwd_workspace(int BN, int c, int h, int r, int d, int dtype);
 int pr_query_state_bwd(const void* Q, const void* S, const float* s, const float* rowmax, const float* q_log_gate,
                        const void* O, const float* den, const void* dO, void* dQ, void* dS, float* ds, void* dY_attn,
-                       float* dl_attn, float* dY_scale, void* workspace, int BN, int n, int c, int h, int r, int d,
-                       float scale_p, int deg, int zero_initial_state, int S_symmetric, int prepared, int dtype,
-                       void* stream);
+                       float* dl_attn, float* dY_scale, void* workspace, const int* live_rows, int BN, int n, int c,
+                       int h, int r, int d, float scale_p, int deg, int zero_initial_state, int S_symmetric,
+                       int prepared, int dtype, void* stream);
 
 /* Forward of every chunk in one kernel: the attention inside the chunk (retention/_attention/reference.py:10-69), the
  * query of the state the chunk starts from and the merge of the two (retention/_query_state/reference.py:36-96, with
@@ -212,11 +247,15 @@ int pr_query_state_bwd(const void* Q, const void* S, const float* s, const float
  *   S [BN,h,D,d] / s [BN,h,D] fp32: the scanned states, symmetric in the diagonal feature blocks
  *   -> O [BN,c,h*r,d], rowmax [BN,c,h*r] (log of the row's largest attention weight) and den [BN,c,h*r], both fp32 and
  *      in the units pr_query_state_bwd and pr_chunk_attention_bwd expect.
- *   scale multiplies q.k before the power; n, zero_initial_state as in pr_query_state_fwd. */
+ *   scale multiplies q.k before the power; n, zero_initial_state as in pr_query_state_fwd.
+ *   S_scan_in, s_scan_in, scan_log_G (all NULL, or all given): S, s are the output of pr_state_scan_fwd and these its
+ *   inputs S, s, log_G.  Entry k of that scan equals its input entry k - 1 bit for bit when exp(scan_log_G[k-1]) == 0
+ *   (and, with zero_initial_state, for k == 1): the kernel then reads the input entry (see consumers_follow_gates). */
 int pr_chunk_fwd_supported(int d, int deg, int dtype);
-int pr_chunk_fwd(const void* Q, const void* K, const void* V, const float* A, const void* S, const float* s, void* O,
-                 float* rowmax, float* den, int BN, int n, int c, int h, int r, int d, float scale, int deg,
-                 int zero_initial_state, int dtype, void* stream);
+int pr_chunk_fwd(const void* Q, const void* K, const void* V, const float* A, const void* S, const float* s,
+                 const void* S_scan_in, const float* s_scan_in, const float* scan_log_G, void* O, float* rowmax,
+                 float* den, int BN, int n, int c, int h, int r, int d, float scale, int deg, int zero_initial_state,
+                 int dtype, void* stream);
 
 /* Query side of the chunked backward in one kernel: dQ and dGq of the attention inside every chunk
  * (retention/_attention/triton.py:248-387) plus the query gradient through the chunk's starting state
@@ -229,12 +268,14 @@ int pr_chunk_fwd(const void* Q, const void* K, const void* V, const float* A, co
  *   same inputs has written (its dl_attn and dY_scale outputs; cvec is the second part of its workspace, behind the
  *   scaled dO: byte offset rows * d * 2 rounded up to 256, rows = BN*c*h*r) -- call it with dQ == dS == NULL for the
  *   preparation alone
+ *   S_scan_in, s_scan_in, scan_log_G: as for pr_chunk_fwd
  *   -> dQ [BN,c,h*r,d] (final), dGq [BN,c,h*r] fp32 (required when A is given). */
 int pr_chunk_bwd_dq_supported(int d, int deg, int dtype);
 int pr_chunk_bwd_dq(const void* Q, const void* K, const void* V, const float* A, const float* rowmax, const float* den,
                     const void* dO, const float* dl_attn, const float* dY_scale, const float* cvec, const void* S,
-                    const float* s, void* dQ, float* dGq, int BN, int n, int c, int h, int r, int d, float scale,
-                    int deg, int zero_initial_state, int dtype, void* stream);
+                    const float* s, const void* S_scan_in, const float* s_scan_in, const float* scan_log_G, void* dQ,
+                    float* dGq, int BN, int n, int c, int h, int r, int d, float scale, int deg,
+                    int zero_initial_state, int dtype, void* stream);
 
 /* Accumulated gates of the quadratic / inference paths -- log_G.cumsum(1), retention/power_retention_maker.py:129,
  * 348-349.  log_G, A [B,t,h] fp32, t <= 8192. */
@@ -245,9 +286,13 @@ int pr_gate_cumsum(const float* log_G, float* A, int B, int t, int h, void* stre
  *   -> A [BN,c,h] = cumsum over the chunk, lcs [BN,h] = A[c-1],
  *      Kd = K * exp((A[c-1] - A)/deg), Qg = Q * exp(A/deg) (Qg may be NULL: not formed).
  *   Two kernels (the sums, then the row-wise products): with Kd == NULL only A and lcs are written; with
- *   log_G == NULL, A and lcs are inputs and only the products are formed. */
-int pr_chunk_prep_fwd(const float* log_G, const void* K, const void* Q, float* A, float* lcs, void* Kd, void* Qg, int BN,
-                      int c, int h, int r, int d, int deg, int dtype, void* stream);
+ *   log_G == NULL, A and lcs are inputs and only the products are formed.
+ *   live_rows (NULL or [BN,h,2] int32, written with the sums): per (chunk, kv head), [0] the first time step whose
+ *   factor exp((A[c-1] - A)/deg) has not underflowed to zero -- the rows of Kd before it are exact zeros -- and [1] one
+ *   past the last time step with exp(A) != 0 -- from there on the state part of a query row is an exact zero.  Hand it
+ *   to pr_update_state_fwd and pr_query_state_bwd, which then leave those rows out (see pr_set_gate_skipping). */
+int pr_chunk_prep_fwd(const float* log_G, const void* K, const void* Q, float* A, float* lcs, void* Kd, void* Qg,
+                      int* live_rows, int BN, int c, int h, int r, int d, int deg, int dtype, void* stream);
 
 /* Backward of the same glue plus the final gradient sums (autograd of retention/power_retention_maker.py:143-193).
  * The row-wise part rides in the attention backward's epilogue (no extra pass over the gradients):

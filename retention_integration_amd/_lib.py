@@ -22,31 +22,33 @@ _P, _I, _F = c_void_p, c_int, c_float
 # name -> (restype, argtypes); mirrors include/power_retention_hip.h declaration by declaration
 SIGNATURES = {
     "pr_abi_version": (c_int, []),
+    "pr_set_gate_skipping": (None, [_I]),
+    "pr_get_gate_skipping": (c_int, []),
     "pr_last_error": (c_char_p, []),
     "pr_expanded_dim": (c_int, [_I, _I]),
     "pr_attention_fwd": (c_int, [_P] * 7 + [_I] * 6 + [_F, _I, _I, _I, _P]),
     "pr_attention_bwd": (c_int, [_P] * 13 + [_I] * 6 + [_F, _I, _I, _P]),
-    "pr_update_state_fwd": (c_int, [_P] * 4 + [_I] * 7 + [_P]),
-    "pr_update_state_bwd": (c_int, [_P] * 6 + [_I] * 8 + [_P]),
+    "pr_update_state_fwd": (c_int, [_P] * 5 + [_I] * 7 + [_P]),
+    "pr_update_state_bwd": (c_int, [_P] * 10 + [_I] * 8 + [_P]),
     "pr_discumsum_fwd": (c_int, [_P] * 3 + [_I] * 4 + [c_int64, _I, _P]),
     "pr_discumsum_bwd_workspace": (c_size_t, [_I, _I, _I, c_int64, _I]),
     "pr_discumsum_bwd": (c_int, [_P] * 6 + [_I] * 4 + [c_int64, _I, _P]),
     "pr_query_state_fwd": (c_int, [_P] * 9 + [_I] * 6 + [_F, _I, _I, _I, _I, _P]),
     "pr_query_state_bwd_workspace": (c_size_t, [_I] * 6),
-    "pr_query_state_bwd": (c_int, [_P] * 15 + [_I] * 6 + [_F, _I, _I, _I, _I, _I, _P]),
-    "pr_chunk_prep_fwd": (c_int, [_P] * 7 + [_I] * 7 + [_P]),
+    "pr_query_state_bwd": (c_int, [_P] * 16 + [_I] * 6 + [_F, _I, _I, _I, _I, _I, _P]),
+    "pr_chunk_prep_fwd": (c_int, [_P] * 8 + [_I] * 7 + [_P]),
     "pr_chunk_fwd_supported": (c_int, [_I] * 3),
-    "pr_chunk_fwd": (c_int, [_P] * 9 + [_I] * 6 + [_F, _I, _I, _I, _P]),
+    "pr_chunk_fwd": (c_int, [_P] * 12 + [_I] * 6 + [_F, _I, _I, _I, _P]),
     "pr_chunk_bwd_dq_supported": (c_int, [_I] * 3),
-    "pr_chunk_bwd_dq": (c_int, [_P] * 14 + [_I] * 6 + [_F, _I, _I, _I, _P]),
+    "pr_chunk_bwd_dq": (c_int, [_P] * 17 + [_I] * 6 + [_F, _I, _I, _I, _P]),
     "pr_gate_cumsum": (c_int, [_P] * 2 + [_I] * 3 + [_P]),
-    "pr_state_scan_fwd": (c_int, [_P] * 9 + [_I] * 4 + [c_int64, c_int64, _I, _P]),
+    "pr_state_scan_fwd": (c_int, [_P] * 9 + [_I] * 4 + [c_int64, c_int64, _I, _I, _P]),
     "pr_state_chain_supported": (c_int, [_I] * 6),
     "pr_update_state_scan_fwd": (c_int, [_P] * 5 + [_I] * 7 + [_P]),
     "pr_query_state_scan_bwd_workspace": (c_size_t, [_I] * 7),
     "pr_query_state_scan_bwd": (c_int, [_P] * 17 + [_I] * 6 + [_F, _I, _I, _P]),
     "pr_state_scan_bwd_workspace": (c_size_t, [_I] * 3 + [c_int64, c_int64]),
-    "pr_state_scan_bwd": (c_int, [_P] * 13 + [_I] * 4 + [c_int64, c_int64, _I, _P]),
+    "pr_state_scan_bwd": (c_int, [_P] * 13 + [_I] * 4 + [c_int64, c_int64, _I, _I, _P]),
     "pr_chunk_attention_bwd": (c_int, [_P] * 17 + [_I] * 5 + [_F, _I, _I, _I, _P]),
     "pr_chunk_gate_scan_bwd": (c_int, [_P] * 5 + [_I] * 5 + [_P]),
     "pr_decode_step_workspace": (c_size_t, [_I] * 5),

@@ -405,7 +405,7 @@ __global__ __launch_bounds__(256, OCC) void attention_bwd_dq_kernel(AttnBwdArgs 
 // times dl) are prepared once per tile in LDS, and the key factor exp(R - G_k) <= 1 is applied to the accumulators
 // once after the far tiles; the tiles near the diagonal then add absolute terms (reference: last key of each 16).
 template <typename T, int DH, int MK, bool DEG2>
-__global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a, int nblocks, int npairs) {
+__global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a, int nblocks, int npairs, int gate_skip) {
   typedef typename VecOf<T>::v8 v8;
   typedef typename VecOf<T>::v4 v4;
   typedef __attribute__((address_space(3))) v8 lds_v8;
@@ -549,9 +549,7 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
       async_copy4(osg ? osg + ro : rmg + ro, rv + 3 * AB_BM);
     }
   };
-  if (ntot > 0) issue(0);
-  if (NST == 3 && ntot > 1) issue(1);
-
+  // (the keys and values of the workgroup first: their loads are in flight while the far tiles are tested)
   v8 Kf[MK][KS], Vf[MK][KS];
   int key[MK];
   bool live[MK];
@@ -576,6 +574,46 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
     evg[kj] = __expf(fminf(Rk[kj] - Gk[kj], AB_EXP_CLAMP));   // key factor inside its group of 16, <= 1
     dgk[kj] = 0.f;
   }
+  // ---- far tiles that the gates have already forgotten -------------------------------------------------------------
+  // Every term of a far tile carries its row's factor scale^deg exp(G_q - m - R) (row_factors below).  The walk starts
+  // at the last tile, the one the gates have decayed most: while that factor has underflowed to zero for every row of
+  // a tile, the tile adds exact zeros to dK, dV and the gate sums, and is neither copied nor visited (step0 = the first
+  // tile that is).  Each wave tests every fourth tile, a row per lane, eight tiles at a time so that the latencies of
+  // their loads overlap.
+  // (Tested only when the gates fall by more than 40 from the workgroup's keys to the last row: short of that no factor
+  // can have underflowed unless a row's largest weight exceeds e^47, and such a tile is merely visited.)
+  int step0 = 0;
+  if (gate_skip && Gg && n_far > 0 && Gg[(long)((rows - 1) / a.r + shift) * a.h] - Rblk < -40.f) {
+    int* first = (int*)smem;
+    for (int base = 0; base < n_far; base += 32) {
+      float bsv[8];
+#pragma unroll
+      for (int i = 0; i < 8; i++) {
+        const int s = base + 4 * i + wave;
+        const int row = (ntile_total - 1 - s) * AB_BM + l;
+        const bool real = s < n_far && row < rows;
+        const int rc = min(max(row, 0), rows - 1);
+        bsv[i] = real ? Gg[(long)(rc / a.r + shift) * a.h] - rmg[row_elem(rc)] : -INFINITY;
+      }
+      int fa = n_far;   // this wave's first tile of the round with a row that still counts (tiles past the far ones do)
+#pragma unroll
+      for (int i = 7; i >= 0; i--) {
+        const int s = base + 4 * i + wave;
+        const bool alive = s >= n_far || __expf(fminf(bsv[i] - Rblk, AB_EXP_CLAMP)) != 0.f;
+        if (__ballot(alive) != 0) fa = min(s, n_far);
+      }
+      __syncthreads();   // (the previous round's values have been read)
+      if (l == 0) first[wave] = fa;
+      __syncthreads();
+      step0 = min(min(first[0], first[1]), min(first[2], first[3]));
+      if (step0 < base + 32) break;
+    }
+    step0 = __builtin_amdgcn_readfirstlane(min(step0, n_far));
+    __syncthreads();   // the first stage's copies land where the four values were
+  }
+  if (ntot > step0) issue(step0);
+  if (NST == 3 && ntot > step0 + 1) issue(step0 + 1);
+
   f32x4 accK[MK][NT], accV[MK][NT];
 #pragma unroll
   for (int kj = 0; kj < MK; kj++)
@@ -614,9 +652,9 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
     rv[4 * AB_BM + l] = eu * os_;
     rv[5 * AB_BM + l] = eu * dl_;
   };
-  if (wave == 0 && nsteps > 0) {
+  if (wave == 0 && nsteps > step0) {
     wait_vmcnt<0>();
-    row_factors(0);
+    row_factors(step0);
   }
   auto sync_step = [&](int step) __attribute__((always_inline)) -> char* {
     char* st = smem + (step % NST) * STAGE;
@@ -770,7 +808,7 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
     }
   };
 
-  int step = 0;
+  int step = step0;
   for (; step < n_far; step++) {
     tile(sync_step(step), (ntile_total - 1 - step) * AB_BM, IC<1>{});
     after_step(step);
@@ -877,7 +915,7 @@ template <typename T, int DH, bool DEG2> static int attn_bwd_launch(const AttnBw
     dim3 grid((unsigned)((npairs + 31) / 32 * 32 * nblocks));
     auto kern = attention_bwd_dkv_kernel<T, DH, MK, DEG2>;
     allow_big_lds((const void*)kern, smem);
-    PR_LAUNCH("attention_bwd_dkv", kern, grid, dim3(256), smem, st, a, nblocks, npairs);
+    PR_LAUNCH("attention_bwd_dkv", kern, grid, dim3(256), smem, st, a, nblocks, npairs, g_gate_skip);
   }
   if (a.dQ) {
     constexpr int MT = DH <= 64 ? 2 : 1;

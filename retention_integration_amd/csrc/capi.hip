@@ -11,6 +11,7 @@
 namespace pr {
 launch_hook_t g_launch_hook = nullptr;
 void* g_launch_hook_user = nullptr;
+int g_gate_skip = 1;
 }  // namespace pr
 
 namespace {
@@ -43,13 +44,15 @@ size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 
 extern "C" {
 
-int pr_abi_version(void) { return 7; }
+int pr_abi_version(void) { return 8; }
 
 void pr_set_launch_hook(pr_launch_hook_t hook, void* user) {
   pr::g_launch_hook = nullptr;   // (never a new hook with the old user pointer)
   pr::g_launch_hook_user = user;
   pr::g_launch_hook = hook;
 }
+void pr_set_gate_skipping(int on) { pr::g_gate_skip = on ? 1 : 0; }
+int pr_get_gate_skipping(void) { return pr::g_gate_skip; }
 const char* pr_last_error(void) { return g_err; }
 
 int pr_expanded_dim(int d, int deg) {
@@ -111,32 +114,48 @@ int pr_chunk_attention_bwd(const void* Q, const void* K, const void* V, const fl
   return finish(pr::attention_bwd(a, BN, d, dtype, (hipStream_t)stream), "chunk_attention_bwd");
 }
 
-int pr_update_state_fwd(const void* K, const void* V, void* S, float* s, int BN, int c, int h, int d, int deg,
-                        int skip_last_of, int dtype, void* stream) {
+int pr_update_state_fwd(const void* K, const void* V, void* S, float* s, const int* live_rows, int BN, int c, int h,
+                        int d, int deg, int skip_last_of, int dtype, void* stream) {
   if (int rc = check_common("update_state_fwd", d, deg, dtype, true)) return rc;
   if (bad_ptr(K) || bad_ptr(V) || bad_ptr(S) || bad_ptr(s)) return fail(PR_ERR_ARG, "update_state_fwd: null or misaligned pointer");
   if (BN <= 0 || c <= 0 || h <= 0) return fail(PR_ERR_ARG, "update_state_fwd: need BN,c,h > 0");
   if (skip_last_of < 0 || (skip_last_of > 0 && BN % skip_last_of != 0))
     return fail(PR_ERR_ARG, "update_state_fwd: skip_last_of must be 0 or a divisor of BN (got %d, BN %d)", skip_last_of, BN);
-  return finish(pr::sympow_tn(K, V, nullptr, S, s, BN, c, h, 1, d, 1, skip_last_of, dtype, (hipStream_t)stream),
+  return finish(pr::sympow_tn(K, V, nullptr, S, s, BN, c, h, 1, d, 1, skip_last_of, live_rows, 0, dtype, (hipStream_t)stream),
                 "update_state_fwd");
 }
 
-int pr_update_state_bwd(const void* K, const void* V, const void* dS, const float* ds, void* dK, void* dV, int BN,
-                        int c, int h, int d, int deg, int dS_symmetric, int zero_last_of, int dtype, void* stream) {
+int pr_update_state_bwd(const void* K, const void* V, const void* dS, const float* ds, const void* dS_scan_in,
+                        const float* ds_scan_in, const float* scan_log_G, const int* live_rows, void* dK, void* dV,
+                        int BN, int c, int h, int d, int deg, int dS_symmetric, int zero_last_of, int dtype,
+                        void* stream) {
   if (int rc = check_common("update_state_bwd", d, deg, dtype, true)) return rc;
-  if (bad_ptr(K) || bad_ptr(V) || bad_ptr(dS) || bad_ptr(ds) || bad_opt(dK) || bad_opt(dV) || (!dK && !dV))
+  if (bad_ptr(K) || bad_ptr(V) || bad_ptr(dS) || bad_ptr(ds) || bad_opt(dK) || bad_opt(dV) || (!dK && !dV) ||
+      bad_opt(dS_scan_in))
     return fail(PR_ERR_ARG, "update_state_bwd: null or misaligned pointer");
+  if ((dS_scan_in != nullptr) != (ds_scan_in != nullptr) || (dS_scan_in != nullptr) != (scan_log_G != nullptr))
+    return fail(PR_ERR_ARG, "update_state_bwd: dS_scan_in, ds_scan_in and scan_log_G come together");
+  if (dS_scan_in && zero_last_of <= 0)
+    return fail(PR_ERR_ARG, "update_state_bwd: dS_scan_in needs zero_last_of (the chunks per scanned sequence)");
   if (BN <= 0 || c <= 0 || h <= 0) return fail(PR_ERR_ARG, "update_state_bwd: need BN,c,h > 0");
   if (zero_last_of < 0 || (zero_last_of > 0 && BN % zero_last_of != 0))
     return fail(PR_ERR_ARG, "update_state_bwd: zero_last_of must be 0 or a divisor of BN (got %d, BN %d)", zero_last_of, BN);
   const int nn_ = zero_last_of > 0 ? zero_last_of : 1, skl = zero_last_of > 0 ? 1 : 0;
   if (dV) {
     pr::NNArgs nn{K, dS, nullptr, dV, nullptr, nullptr, nullptr, nullptr, 1.f, c, h, 1, nn_, 0, skl, dS_symmetric ? 1 : 0, nullptr};
+    nn.live_rows = live_rows;
+    nn.B_alt = dS_scan_in;
+    nn.carry = scan_log_G;
     if (int rc = finish(pr::sympow_nn(nn, BN, d, 1, 0, dtype, (hipStream_t)stream), "update_state_bwd(dV)")) return rc;
   }
   if (!dK) return 0;
   pr::GradArgs g{K, V, nullptr, dS, ds, dK, c, h, 1, nn_, skl ? 2 : 0, dS_symmetric ? 1 : 0};
+  g.live_rows = live_rows;
+  g.live_side = 0;
+  g.B_alt = dS_scan_in;
+  g.sB_alt = ds_scan_in;
+  g.carry = scan_log_G;
+  g.alt_shift = 1;
   return finish(pr::sympow_grad(g, BN, d, 1, dtype, (hipStream_t)stream), "update_state_bwd(dK)");
 }
 
@@ -168,7 +187,7 @@ int pr_discumsum_bwd(const void* dY, const void* Y, const float* log_G, void* dX
 
 int pr_state_scan_fwd(const void* S, const float* s, const float* log_G, void* S_out, float* s_out,
                       const void* S_init, const float* s_init, void* S_final, float* s_final, int B, int n,
-                      int n_out, int H, int64_t F, int64_t F2, int dtype, void* stream) {
+                      int n_out, int H, int64_t F, int64_t F2, int consumers_follow_gates, int dtype, void* stream) {
   if (dtype != PR_BF16 && dtype != PR_F16) return fail(PR_ERR_DTYPE, "state_scan_fwd: unsupported dtype");
   if (bad_ptr(S) || bad_ptr(s) || log_G == nullptr || bad_ptr(S_out) || bad_ptr(s_out))
     return fail(PR_ERR_ARG, "state_scan_fwd: null or misaligned pointer");
@@ -180,8 +199,8 @@ int pr_state_scan_fwd(const void* S, const float* s, const float* log_G, void* S
   if (S_final && n_out != n) return fail(PR_ERR_ARG, "state_scan_fwd: S_final is entry n of a scan that keeps n entries");
   pr::ScanCarry cy;
   cy.in = S_init, cy.in2 = s_init, cy.out = S_final, cy.out2 = s_final;
-  return finish(pr::discumsum_pair_fwd(S, s, log_G, S_out, s_out, B, n, n_out, H, (long)F, (long)F2, cy, dtype,
-                                       (hipStream_t)stream), "state_scan_fwd");
+  return finish(pr::discumsum_pair_fwd(S, s, log_G, S_out, s_out, B, n, n_out, H, (long)F, (long)F2, cy,
+                                       consumers_follow_gates, dtype, (hipStream_t)stream), "state_scan_fwd");
 }
 
 size_t pr_state_scan_bwd_workspace(int B, int n, int H, int64_t F, int64_t F2) {
@@ -191,7 +210,7 @@ size_t pr_state_scan_bwd_workspace(int B, int n, int H, int64_t F, int64_t F2) {
 int pr_state_scan_bwd(const void* dS_out, const void* S_out, const float* ds_out, const float* s_out,
                       const float* log_G, void* dS, float* ds, float* dlog_G, void* workspace, const void* dS_final,
                       const float* ds_final, void* dS_init, float* ds_init, int B, int n, int n_out,
-                      int H, int64_t F, int64_t F2, int dtype, void* stream) {
+                      int H, int64_t F, int64_t F2, int consumers_follow_gates, int dtype, void* stream) {
   if (dtype != PR_BF16 && dtype != PR_F16) return fail(PR_ERR_DTYPE, "state_scan_bwd: unsupported dtype");
   if (bad_ptr(dS_out) || bad_ptr(S_out) || bad_ptr(ds_out) || bad_ptr(s_out) || log_G == nullptr || bad_ptr(dS) ||
       bad_ptr(ds) || dlog_G == nullptr || bad_ptr(workspace))
@@ -205,7 +224,8 @@ int pr_state_scan_bwd(const void* dS_out, const void* S_out, const float* ds_out
   pr::ScanCarry cy;
   cy.in = dS_final, cy.in2 = ds_final, cy.out = dS_init, cy.out2 = ds_init;
   return finish(pr::discumsum_pair_bwd(dS_out, S_out, ds_out, s_out, log_G, dS, ds, dlog_G, (float*)workspace, B, n,
-                                       n_out, H, (long)F, (long)F2, cy, dtype, (hipStream_t)stream), "state_scan_bwd");
+                                       n_out, H, (long)F, (long)F2, cy, consumers_follow_gates, dtype,
+                                       (hipStream_t)stream), "state_scan_bwd");
 }
 
 int pr_query_state_fwd(const void* Q, const void* S, const float* s, const void* Y_attn, const float* l_attn,
@@ -228,9 +248,10 @@ int pr_query_state_fwd(const void* Q, const void* S, const float* s, const void*
 
 int pr_chunk_fwd_supported(int d, int deg, int dtype) { return deg == 2 && pr::chunk_fwd_supported(d, dtype); }
 
-int pr_chunk_fwd(const void* Q, const void* K, const void* V, const float* A, const void* S, const float* s, void* O,
-                 float* rowmax, float* den, int BN, int n, int c, int h, int r, int d, float scale, int deg,
-                 int zero_initial_state, int dtype, void* stream) {
+int pr_chunk_fwd(const void* Q, const void* K, const void* V, const float* A, const void* S, const float* s,
+                 const void* S_scan_in, const float* s_scan_in, const float* scan_log_G, void* O, float* rowmax,
+                 float* den, int BN, int n, int c, int h, int r, int d, float scale, int deg, int zero_initial_state,
+                 int dtype, void* stream) {
   if (int rc = check_common("chunk_fwd", d, deg, dtype, true)) return rc;
   if (!pr_chunk_fwd_supported(d, deg, dtype))
     return fail(PR_ERR_DTYPE, "chunk_fwd: bf16, head dim 32 or 64, degree 2 (ask pr_chunk_fwd_supported); other cases "
@@ -240,7 +261,11 @@ int pr_chunk_fwd(const void* Q, const void* K, const void* V, const float* A, co
     return fail(PR_ERR_ARG, "chunk_fwd: null or misaligned pointer");
   if (BN <= 0 || n <= 0 || c <= 0 || h <= 0 || r <= 0 || BN % n != 0)
     return fail(PR_ERR_ARG, "chunk_fwd: need BN,n,c,h,r > 0 and BN a multiple of n");
-  pr::ChunkFwdArgs a{Q, K, V, A, S, s, O, rowmax, den, c, h, r, n, scale, zero_initial_state ? 1 : 0};
+  if ((S_scan_in != nullptr) != (s_scan_in != nullptr) || (S_scan_in != nullptr) != (scan_log_G != nullptr) ||
+      bad_opt(S_scan_in))
+    return fail(PR_ERR_ARG, "chunk_fwd: S_scan_in, s_scan_in and scan_log_G come together, 16-byte aligned");
+  pr::ChunkFwdArgs a{Q, K, V, A, S, s, O, rowmax, den, c, h, r, n, scale, zero_initial_state ? 1 : 0, pr::g_gate_skip};
+  if (pr::g_gate_skip) a.S_alt = S_scan_in, a.s_alt = s_scan_in, a.carry = scan_log_G;
   return finish(pr::chunk_fwd(a, BN, d, dtype, (hipStream_t)stream), "chunk_fwd");
 }
 
@@ -248,8 +273,9 @@ int pr_chunk_bwd_dq_supported(int d, int deg, int dtype) { return deg == 2 && pr
 
 int pr_chunk_bwd_dq(const void* Q, const void* K, const void* V, const float* A, const float* rowmax, const float* den,
                     const void* dO, const float* dl_attn, const float* dY_scale, const float* cvec, const void* S,
-                    const float* s, void* dQ, float* dGq, int BN, int n, int c, int h, int r, int d, float scale,
-                    int deg, int zero_initial_state, int dtype, void* stream) {
+                    const float* s, const void* S_scan_in, const float* s_scan_in, const float* scan_log_G, void* dQ,
+                    float* dGq, int BN, int n, int c, int h, int r, int d, float scale, int deg,
+                    int zero_initial_state, int dtype, void* stream) {
   if (int rc = check_common("chunk_bwd_dq", d, deg, dtype, true)) return rc;
   if (!pr_chunk_bwd_dq_supported(d, deg, dtype))
     return fail(PR_ERR_DTYPE, "chunk_bwd_dq: bf16, head dim 32 or 64, degree 2 (ask pr_chunk_bwd_dq_supported); other "
@@ -261,7 +287,11 @@ int pr_chunk_bwd_dq(const void* Q, const void* K, const void* V, const float* A,
   if (BN <= 0 || n <= 0 || c <= 0 || h <= 0 || r <= 0 || BN % n != 0)
     return fail(PR_ERR_ARG, "chunk_bwd_dq: need BN,n,c,h,r > 0 and BN a multiple of n");
   pr::ChunkBwdDqArgs a{Q, K, V, A, rowmax, den, dO, dl_attn, dY_scale, cvec, S, s, dQ, A ? dGq : nullptr,
-                       c, h, r, n, scale, zero_initial_state ? 1 : 0};
+                       c, h, r, n, scale, zero_initial_state ? 1 : 0, pr::g_gate_skip};
+  if ((S_scan_in != nullptr) != (s_scan_in != nullptr) || (S_scan_in != nullptr) != (scan_log_G != nullptr) ||
+      bad_opt(S_scan_in))
+    return fail(PR_ERR_ARG, "chunk_bwd_dq: S_scan_in, s_scan_in and scan_log_G come together, 16-byte aligned");
+  if (pr::g_gate_skip) a.S_alt = S_scan_in, a.s_alt = s_scan_in, a.carry = scan_log_G;
   return finish(pr::chunk_bwd_dq(a, BN, d, dtype, (hipStream_t)stream), "chunk_bwd_dq");
 }
 
@@ -273,10 +303,11 @@ size_t pr_query_state_bwd_workspace(int BN, int c, int h, int r, int d, int dtyp
 
 int pr_query_state_bwd(const void* Q, const void* S, const float* s, const float* rowmax, const float* q_log_gate,
                        const void* O, const float* den, const void* dO, void* dQ, void* dS, float* ds, void* dY_attn,
-                       float* dl_attn, float* dY_scale, void* workspace, int BN, int n, int c, int h, int r, int d,
-                       float scale_p, int deg, int zero_initial_state, int S_symmetric, int prepared, int dtype,
-                       void* stream) {
+                       float* dl_attn, float* dY_scale, void* workspace, const int* live_rows, int BN, int n, int c,
+                       int h, int r, int d, float scale_p, int deg, int zero_initial_state, int S_symmetric,
+                       int prepared, int dtype, void* stream) {
   if (int rc = check_common("query_state_bwd", d, deg, dtype, true)) return rc;
+  if (live_rows && !q_log_gate) return fail(PR_ERR_ARG, "query_state_bwd: live_rows describes q_log_gate");
   if (bad_ptr(Q) || bad_ptr(S) || bad_ptr(s) || bad_ptr(O) || bad_ptr(den) || bad_ptr(dO) || bad_opt(dQ) ||
       bad_opt(dS) || bad_ptr(workspace) || bad_opt(rowmax) || bad_opt(dY_attn) || bad_opt(dl_attn))
     return fail(PR_ERR_ARG, "query_state_bwd: null or misaligned pointer");
@@ -299,11 +330,14 @@ int pr_query_state_bwd(const void* Q, const void* S, const float* s, const float
       return rc;
   // (zero_initial_state == 2: the caller does not want the gradient of the first chunk's (zero) state either)
   if (dS)
-    if (int rc = finish(pr::sympow_tn(Q, dOs, cvec, dS, ds, BN, c, h, r, d, 0, zero_initial_state == 2 ? -n : 0, dtype, st),
+    if (int rc = finish(pr::sympow_tn(Q, dOs, cvec, dS, ds, BN, c, h, r, d, 0, zero_initial_state == 2 ? -n : 0, live_rows, 1,
+                                      dtype, st),
                         "query_state_bwd(dS)"))
       return rc;
   if (!dQ) return 0;
   pr::GradArgs g{Q, dOs, cvec, S, s, dQ, c, h, r, n, zero_initial_state ? 1 : 0, S_symmetric ? 1 : 0};
+  g.live_rows = live_rows;
+  g.live_side = 1;
   return finish(pr::sympow_grad(g, BN, d, 0, dtype, st), "query_state_bwd(dQ)");
 }
 
@@ -377,13 +411,14 @@ int pr_gate_cumsum(const float* log_G, float* A, int B, int t, int h, void* stre
   return finish(pr::gate_cumsum(log_G, A, B, t, h, (hipStream_t)stream), "gate_cumsum");
 }
 
-int pr_chunk_prep_fwd(const float* log_G, const void* K, const void* Q, float* A, float* lcs, void* Kd, void* Qg, int BN,
+int pr_chunk_prep_fwd(const float* log_G, const void* K, const void* Q, float* A, float* lcs, void* Kd, void* Qg,
+                      int* live_rows, int BN,
                       int c, int h, int r, int d, int deg, int dtype, void* stream) {
   if (int rc = check_common("chunk_prep_fwd", d, deg, dtype, false)) return rc;
   if (bad_ptr(K) || bad_ptr(Q) || A == nullptr || lcs == nullptr || bad_opt(Kd) || bad_opt(Qg) || (!log_G && !Kd))
     return fail(PR_ERR_ARG, "chunk_prep_fwd: null or misaligned pointer");
   if (BN <= 0 || c <= 0 || h <= 0 || r <= 0) return fail(PR_ERR_ARG, "chunk_prep_fwd: need BN,c,h,r > 0");
-  return finish(pr::chunk_prep_fwd(log_G, K, Q, A, lcs, Kd, Qg, BN, c, h, r, d, deg, dtype, (hipStream_t)stream),
+  return finish(pr::chunk_prep_fwd(log_G, K, Q, A, lcs, Kd, Qg, live_rows, BN, c, h, r, d, deg, dtype, (hipStream_t)stream),
                 "chunk_prep_fwd");
 }
 

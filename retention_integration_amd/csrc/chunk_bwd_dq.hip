@@ -73,10 +73,17 @@ __global__ __launch_bounds__(256, 3) void chunk_bwd_dq_kernel(ChunkBwdDqArgs a, 
   const float* Gg = a.G ? a.G + (long)b * a.c * a.h + hh : nullptr;
   const char* Sg = (const char*)((const T*)a.S + ((long)b * a.h + hh) * D * DH);
   const float* sg = a.s + ((long)b * a.h + hh) * D;
+  // (S, s are a gated scan's output: with a zero carry into it -- and, whatever the gate, at the second chunk of a
+  // sequence that starts from nothing -- an entry is the scan's input entry before it, bit for bit)
+  if (a.S_alt && b % a.n != 0 &&
+      ((a.skip_first && (b - 1) % a.n == 0) || __expf(a.carry[(long)(b - 1) * a.h + hh]) == 0.f)) {
+    Sg = (const char*)((const T*)a.S_alt + ((long)(b - 1) * a.h + hh) * D * DH);
+    sg = a.s_alt + ((long)(b - 1) * a.h + hh) * D;
+  }
   const long kstride = (long)a.h * DH * 2;
   const float eps_s = CB_LOG_EPS / a.scale, eps2 = eps_s * eps_s;
   const float scale_p = a.scale * a.scale;
-  const bool has_state = !(a.skip_first && (b % a.n == 0));
+  bool has_state = !(a.skip_first && (b % a.n == 0));
 
   const int last_row = min(row0 + ROWS, rows) - 1;
   const int kmax = min(a.c, last_row / a.r + 1);
@@ -96,6 +103,26 @@ __global__ __launch_bounds__(256, 3) void chunk_bwd_dq_kernel(ChunkBwdDqArgs a, 
   for (int ii = 0; ii < LOADS / 2; ii++) {
     const int pos = (ii * 4 + wave) * 64 + l, row = pos / CPR;
     goff[ii] = (uint32_t)(row * (int)kstride + 16 * ((pos % CPR) ^ swz<CPR, SWZ_ROW>(row)));
+  }
+  // What the gates have already forgotten (see chunk_fwd.hip): key tiles whose factor exp(R - A_last) has underflowed to
+  // zero for the workgroup's first row contribute exact zeros to every row of the workgroup -- dQ, dGq -- and are
+  // neither copied nor visited; a state part whose factor exp(A_row) has underflowed at the first row has a zero
+  // gradient for every row (the row-wise preparation wrote zeros for its scaled dO and its key-sum factor), so the
+  // sweep is left out.
+  int it0 = 0;
+  if (Gg && a.gate_skip) {
+    const float a_first = Gg[(long)(min(row0, rows - 1) / a.r) * a.h];
+    if (__expf(a_first) == 0.f) has_state = false;
+    for (int base = 0; base < ntiles; base += 64) {
+      const int tl = min(base + l, ntiles - 1);
+      const float a_last = Gg[(long)min(CB_BN * tl + CB_BN - 1, a.c - 1) * a.h];
+      const unsigned long long dead = __ballot(__expf(fminf(a_first - a_last, CB_EXP_CLAMP)) == 0.f);
+      const int lanes = min(64, ntiles - base);
+      const int nd = __builtin_popcountll(lanes == 64 ? dead : (dead & ((1ull << lanes) - 1)));
+      it0 += nd;
+      if (nd < lanes) break;
+    }
+    it0 = __builtin_amdgcn_readfirstlane(min(it0, ntiles - 1));
   }
   // Stage ntiles of the ring: the block's rows of Q (the sweep's row values; chunk slots rotated per row as the state
   // kernels read them).  Stage ntiles + 1: the first two stages of the state.
@@ -134,8 +161,8 @@ __global__ __launch_bounds__(256, 3) void chunk_bwd_dq_kernel(ChunkBwdDqArgs a, 
     }
     if (Gg && wave == 0) async_copy4(Gg + (long)min(j0 + l, a.c - 1) * a.h, st + 2 * TILE);
   };
-  issue(0);
-  if (ntot > 1) issue(1);
+  issue(it0);
+  if (ntot > it0 + 1) issue(it0 + 1);
 
   v8 Qf[MT][KS], dOf[MT][KS];
   int ti[MT];
@@ -205,7 +232,7 @@ __global__ __launch_bounds__(256, 3) void chunk_bwd_dq_kernel(ChunkBwdDqArgs a, 
   };
   if (wave == 0) {
     wait_vmcnt<0>();
-    gate_factors(0);
+    gate_factors(it0);
   }
   auto sync_step = [&](int it) __attribute__((always_inline)) -> char* {
     char* st = smem + (it % CB_NST) * STAGE;
@@ -242,6 +269,8 @@ __global__ __launch_bounds__(256, 3) void chunk_bwd_dq_kernel(ChunkBwdDqArgs a, 
 #pragma unroll
     for (int mi = 0; mi < MT; mi++) lim[mi] = DIAG ? min(ti[mi], a.c - 1) - j0 - 4 * g : 0;
     const float cw = DIAG ? 1.f : __expf(fminf(Rw - graw[CB_BN - 1], CB_EXP_CLAMP));
+    // (forgotten by this wave's rows, though not by the workgroup's first: every term of the tile is an exact zero)
+    if (!DIAG && a.gate_skip && __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, cw)) == 0) return;
 #pragma unroll
     for (int kp = 0; kp < KT / 2; kp++) {
       if (DIAG && j0 + 32 * kp > w_last_ti) continue;   // these 32 keys come after every row of the wave
@@ -303,7 +332,7 @@ __global__ __launch_bounds__(256, 3) void chunk_bwd_dq_kernel(ChunkBwdDqArgs a, 
     }
   };
 
-  int it = 0;
+  int it = it0;
   for (; it < n_past; it++) tile(it, sync_step(it), IC<0>{});
   // the past tiles were accumulated without the row factor scale^2 * exp(G_q - m - Rw); apply it once
 #pragma unroll

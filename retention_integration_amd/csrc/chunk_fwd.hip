@@ -93,10 +93,17 @@ __global__ __launch_bounds__(256, 3) void chunk_fwd_kernel(ChunkFwdArgs a, int r
   const float* Gg = a.G ? a.G + (long)b * a.c * a.h + hh : nullptr;
   const char* Sg = (const char*)((const T*)a.S + ((long)b * a.h + hh) * D * DH);
   const float* sg = a.s + ((long)b * a.h + hh) * D;
+  // (S, s are a gated scan's output: with a zero carry into it -- and, whatever the gate, at the second chunk of a
+  // sequence that starts from nothing -- an entry is the scan's input entry before it, bit for bit)
+  if (a.S_alt && b % a.n != 0 &&
+      ((a.skip_first && (b - 1) % a.n == 0) || __expf(a.carry[(long)(b - 1) * a.h + hh]) == 0.f)) {
+    Sg = (const char*)((const T*)a.S_alt + ((long)(b - 1) * a.h + hh) * D * DH);
+    sg = a.s_alt + ((long)(b - 1) * a.h + hh) * D;
+  }
   const long kstride = (long)a.h * DH * 2;
   const float eps_s = CF_LOG_EPS / a.scale, eps2 = eps_s * eps_s;
   const float scale_p = a.scale * a.scale;
-  const bool no_state = a.skip_first && (b % a.n == 0);
+  bool no_state = a.skip_first && (b % a.n == 0);
 
   const int last_row = min(row0 + ROWS, rows) - 1;
   const int kmax = min(a.c, last_row / a.r + 1);   // keys any row of the workgroup can see
@@ -113,8 +120,10 @@ __global__ __launch_bounds__(256, 3) void chunk_fwd_kernel(ChunkFwdArgs a, int r
     const int pos = (ii * 4 + wave) * 64 + l, row = pos / CPR;
     goff[ii] = (uint32_t)(row * (int)kstride + 16 * ((pos % CPR) ^ swz<CPR, SWZ_ROW>(row)));
   }
+  int it0 = 0;   // first key tile that is visited (set below); ring slots count from it: its slot is the one apart from
+                 // the state phase's memory
   auto issue = [&](int it) __attribute__((always_inline)) {
-    char* st = smem + (it % CF_NST) * STAGE;
+    char* st = smem + ((it - it0) % CF_NST) * STAGE;
     const int j0 = it * CF_BN;
     if (j0 + CF_BN <= a.c) {
       const char* kb_ = Kg + (long)j0 * kstride;
@@ -130,8 +139,6 @@ __global__ __launch_bounds__(256, 3) void chunk_fwd_kernel(ChunkFwdArgs a, int r
     }
     if (Gg && wave == 0) async_copy4(Gg + (long)min(j0 + l, a.c - 1) * a.h, st + 2 * TILE);
   };
-  issue(0);   // older than every copy of the state phase, so it has landed whenever one of those has
-
   // ---- the workgroup's query rows, into LDS (operands of both parts) ---------------------------------------------
   auto row_off = [&](int row) -> long {   // element offset of a (clamped) folded row, per unit of the last dim
     row = min(row, rows - 1);
@@ -142,6 +149,29 @@ __global__ __launch_bounds__(256, 3) void chunk_fwd_kernel(ChunkFwdArgs a, int r
     return xt + lrow * (DH * 2) + (((col / 8) ^ swz<CPR>(lrow)) * 16) + (col % 8) * 2;
   };
   async_load_tile<CPR, ROWS>(xt, [&](int row) { return (const char*)(Qg + row_off(row0 + row) * DH); });
+
+  // ---- what the gates have already forgotten -------------------------------------------------------------------
+  // A key tile entirely in a wave's past enters with the factor exp(R - A_last), R the gate sum at the wave's first row
+  // and A_last the one at the tile's last key.  Gate sums only fall along the chunk, so once that factor has underflowed
+  // to zero for the workgroup's FIRST row it is zero for every row of the workgroup and for every older tile: those
+  // tiles contribute exact zeros and are neither copied nor visited (it0 = the first tile that is).  Likewise the
+  // state part of a row carries exp(A_row): with it underflowed at the first row, the sweep over the state adds exact
+  // zeros to every row of the workgroup and is left out.  (Nothing changes for gates that do not decay that far.)
+  if (Gg && a.gate_skip) {
+    const float a_first = Gg[(long)(min(row0, rows - 1) / a.r) * a.h];
+    if (__expf(a_first) == 0.f) no_state = true;
+    for (int base = 0; base < ntiles; base += 64) {
+      const int tl = min(base + l, ntiles - 1);
+      const float a_last = Gg[(long)min(CF_BN * tl + CF_BN - 1, a.c - 1) * a.h];
+      const unsigned long long dead = __ballot(__expf(fminf(a_first - a_last, CF_EXP_CLAMP)) == 0.f);
+      const int lanes = min(64, ntiles - base);
+      const int nd = __builtin_popcountll(lanes == 64 ? dead : (dead & ((1ull << lanes) - 1)));
+      it0 += nd;
+      if (nd < lanes) break;
+    }
+    it0 = __builtin_amdgcn_readfirstlane(min(it0, ntiles - 1));
+  }
+  issue(it0);   // older than every copy of the state phase but the rows', so it has landed whenever one of those has
 
   int ti[MT], lrow[MT];
   long qoff[MT];
@@ -320,7 +350,7 @@ __global__ __launch_bounds__(256, 3) void chunk_fwd_kernel(ChunkFwdArgs a, int r
       }
     }
     // hand over to the attention part: exp(R) times the state part, which the row factor of the past tiles completes
-    const float eR = __expf(fmaxf(Rw, -CF_EXP_CLAMP));
+    const float eR = __expf(Rw);   // (may underflow: the state part of these rows is then zero, as its definition has it)
 #pragma unroll
     for (int mi = 0; mi < MT; mi++) {
       lq[mi] = sum_over_rows(aux[mi]) * eR;
@@ -340,7 +370,7 @@ __global__ __launch_bounds__(256, 3) void chunk_fwd_kernel(ChunkFwdArgs a, int r
       Qf[mi][ks] = __builtin_bit_cast(v8, z);
     }
   lds_barrier();   // every wave is done with the state ring and the query rows: attention stages 1, 2 may land there
-  if (ntiles > 1) issue(1);
+  if (ntiles > it0 + 1) issue(it0 + 1);
 
   // ---- attention part (attention_fwd.hip, bf16 path) -----------------------------------------------------------
   const uint32_t one2 = 0x3F803F80u;
@@ -360,7 +390,7 @@ __global__ __launch_bounds__(256, 3) void chunk_fwd_kernel(ChunkFwdArgs a, int r
   const int n_past = min(ntiles, min(w_first_ti + 1, a.c) / CF_BN);   // tiles with every pair visible
   const int n_seen = min(ntiles, w_last_ti / CF_BN + 1);              // tiles with at least one visible pair
   auto gate_factors = [&](int it) __attribute__((always_inline)) {
-    float* graw = (float*)(smem + (it % CF_NST) * STAGE + 2 * TILE);
+    float* graw = (float*)(smem + ((it - it0) % CF_NST) * STAGE + 2 * TILE);
     const int rpos = min(CF_BN - 1, a.c - 1 - it * CF_BN);
     const float gv = Gg ? graw[l] : 0.f;
     const float R_ = Gg ? graw[rpos] : 0.f, Rs = Gg ? graw[l & ~15] : 0.f;
@@ -369,11 +399,11 @@ __global__ __launch_bounds__(256, 3) void chunk_fwd_kernel(ChunkFwdArgs a, int r
     if (!Gg) graw[l] = 0.f;
   };
   if (wave == 0) {
-    if (ntiles > 1) wait_vmcnt<LOADS + 1>(); else wait_vmcnt<0>();   // all but the stage just issued
-    gate_factors(0);
+    if (ntiles > it0 + 1) wait_vmcnt<LOADS + 1>(); else wait_vmcnt<0>();   // all but the stage just issued
+    gate_factors(it0);
   }
   auto sync_step = [&](int it) __attribute__((always_inline)) -> char* {
-    char* st = smem + (it % CF_NST) * STAGE;
+    char* st = smem + ((it - it0) % CF_NST) * STAGE;
     if (it + 1 < ntiles) wait_vmcnt<LOADS>(); else wait_vmcnt<0>();
     lds_barrier();
     if (it + 2 < ntiles) issue(it + 2);
@@ -401,6 +431,8 @@ __global__ __launch_bounds__(256, 3) void chunk_fwd_kernel(ChunkFwdArgs a, int r
 #pragma unroll
     for (int mi = 0; mi < MT; mi++) lim[mi] = min(ti[mi], a.c - 1) - j0 - 4 * g;
     const float cw = DIAG ? 1.f : __expf(fminf(Rw - graw[CF_BN - 1], CF_EXP_CLAMP));
+    // (forgotten by this wave's rows, though not by the workgroup's first: every weight of the tile is an exact zero)
+    if (!DIAG && a.gate_skip && __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, cw)) == 0) return;
 #pragma unroll
     for (int kp = 0; kp < KT / 2; kp++) {
       if (DIAG && j0 + 32 * kp > w_last_ti) continue;   // these 32 keys come after every row of the wave
@@ -461,7 +493,7 @@ __global__ __launch_bounds__(256, 3) void chunk_fwd_kernel(ChunkFwdArgs a, int r
     }
   };
 
-  int it = 0;
+  int it = it0;
   for (; it < n_past; it++) tile(it, sync_step(it), IC<0>{});
   // the past tiles and the state part were accumulated without the row factor exp(A_i - R) * scale^2; apply it once
 #pragma unroll

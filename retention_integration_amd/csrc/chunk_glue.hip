@@ -42,8 +42,13 @@ __device__ inline void block_scan(float* a, float* tot, int c, bool reverse) {
 }
 
 // A[bn, :, hh] = cumsum(log_G[bn, :, hh]);  lcs[bn, hh] = A[bn, c-1, hh]
+// live[bn, hh] = {first t whose key factor exp((A[c-1] - A[t]) / deg) is not zero (the expression of gate_apply_fwd),
+//                 one past the last t with exp(A[t]) != 0}: outside them the discounted keys, resp. everything that
+// carries the factor exp(A[t]) of a query's state part, are exact zeros, and the kernels that contract over the chunk's
+// rows leave those rows out.
 __global__ __launch_bounds__(256) void gate_scan_fwd_kernel(const float* __restrict__ logG, float* __restrict__ A,
-                                                            float* __restrict__ lcs, int c, int h) {
+                                                            float* __restrict__ lcs, int* __restrict__ live, int c, int h,
+                                                            float inv_deg) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   float* a = (float*)smem;
   float* tot = a + c;
@@ -54,6 +59,29 @@ __global__ __launch_bounds__(256) void gate_scan_fwd_kernel(const float* __restr
   block_scan(a, tot, c, false);
   for (int i = tid; i < c; i += 256) A[base + (long)i * h] = a[i];
   if (tid == 0 && lcs) lcs[(long)bn * h + hh] = a[c - 1];
+  if (live) {
+    const float al = a[c - 1];
+    int lo = c, hi = 0;
+    for (int i = tid; i < c; i += 256) {
+      if (__expf((al - a[i]) * inv_deg) != 0.f) lo = min(lo, i);
+      if (__expf(a[i]) != 0.f) hi = max(hi, i + 1);
+    }
+#pragma unroll
+    for (int m = 32; m > 0; m >>= 1) {
+      lo = min(lo, __shfl_xor(lo, m));
+      hi = max(hi, __shfl_xor(hi, m));
+    }
+    int* red = (int*)(tot + 8);   // (tot[0..4) may still be read by a slower wave of the scan)
+    if ((tid & 63) == 0) {
+      red[2 * (tid >> 6)] = lo;
+      red[2 * (tid >> 6) + 1] = hi;
+    }
+    __syncthreads();
+    if (tid == 0) {
+      live[((long)bn * h + hh) * 2] = min(min(red[0], red[2]), min(red[4], red[6]));
+      live[((long)bn * h + hh) * 2 + 1] = max(max(red[1], red[3]), max(red[5], red[7]));
+    }
+  }
 }
 
 // one group of DH/8 lanes per (chunk, position, kv head)
@@ -118,11 +146,11 @@ __global__ __launch_bounds__(256) void gate_scan_bwd_kernel(float* __restrict__ 
 }
 
 template <typename T>
-static int prep_launch(const float* logG, const void* K, const void* Q, float* A, float* lcs, void* Kd, void* Qg, int BN,
-                       int c, int h, int r, int d, int deg, hipStream_t st) {
+static int prep_launch(const float* logG, const void* K, const void* Q, float* A, float* lcs, void* Kd, void* Qg, int* live,
+                       int BN, int c, int h, int r, int d, int deg, hipStream_t st) {
   const size_t smem = (size_t)(c + 256) * sizeof(float);
   // (either half on its own: no log_G = A and lcs are already there; no Kd = only the sums are wanted)
-  if (logG) PR_LAUNCH("gate_scan_fwd", gate_scan_fwd_kernel, dim3((unsigned)(BN * h)), dim3(256), smem, st, logG, A, lcs, c, h);
+  if (logG) PR_LAUNCH("gate_scan_fwd", gate_scan_fwd_kernel, dim3((unsigned)(BN * h)), dim3(256), smem, st, logG, A, lcs, live, c, h, 1.f / deg);
   if (!Kd) return (int)hipGetLastError();
   const long groups = (long)BN * c * h;
 #define PR_CP(DD)                                                                                                      \
@@ -138,15 +166,15 @@ static int prep_launch(const float* logG, const void* K, const void* Q, float* A
 int gate_cumsum(const float* logG, float* A, int B, int t, int h, hipStream_t st) {
   if (t > GLUE_MAX_C) return -5;
   const size_t smem = (size_t)(t + 256) * sizeof(float);
-  PR_LAUNCH("gate_scan_fwd", gate_scan_fwd_kernel, dim3((unsigned)(B * h)), dim3(256), smem, st, logG, A, (float*)nullptr, t, h);
+  PR_LAUNCH("gate_scan_fwd", gate_scan_fwd_kernel, dim3((unsigned)(B * h)), dim3(256), smem, st, logG, A, (float*)nullptr, (int*)nullptr, t, h, 1.f);
   return (int)hipGetLastError();
 }
 
-int chunk_prep_fwd(const float* logG, const void* K, const void* Q, float* A, float* lcs, void* Kd, void* Qg, int BN,
-                   int c, int h, int r, int d, int deg, int dtype, hipStream_t st) {
+int chunk_prep_fwd(const float* logG, const void* K, const void* Q, float* A, float* lcs, void* Kd, void* Qg, int* live,
+                   int BN, int c, int h, int r, int d, int deg, int dtype, hipStream_t st) {
   if (c > GLUE_MAX_C) return -5;
-  if (dtype == DT_BF16) return prep_launch<bf16_t>(logG, K, Q, A, lcs, Kd, Qg, BN, c, h, r, d, deg, st);
-  if (dtype == DT_F16) return prep_launch<f16_t>(logG, K, Q, A, lcs, Kd, Qg, BN, c, h, r, d, deg, st);
+  if (dtype == DT_BF16) return prep_launch<bf16_t>(logG, K, Q, A, lcs, Kd, Qg, live, BN, c, h, r, d, deg, st);
+  if (dtype == DT_F16) return prep_launch<f16_t>(logG, K, Q, A, lcs, Kd, Qg, live, BN, c, h, r, d, deg, st);
   return -1;
 }
 

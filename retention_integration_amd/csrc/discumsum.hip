@@ -51,6 +51,14 @@ __device__ __forceinline__ const float* stage_gates(float* gsh, const float* __r
   return gsh;
 }
 
+// True for the whole block when every factor exp(log_G[k]), k >= 1, of the block's (batch, head) is an exact zero: each
+// entry of the scan is then a copy of the input entry next to it (gsh: the staged factors).
+__device__ __forceinline__ bool all_carries_zero(const float* gsh, int n) {
+  bool nz = false;
+  for (int k = 1 + (int)threadIdx.x; k < n; k += blockDim.x) nz |= gsh[k] != 0.f;
+  return __syncthreads_or(nz ? 1 : 0) == 0;
+}
+
 template <typename T, int AHEAD, int BYTES>
 __device__ __forceinline__ void discumsum_fwd_body(const T* __restrict__ X, const float* __restrict__ logG,
                                                    T* __restrict__ Y, int n, int n_out, int H, long F, int block,
@@ -141,9 +149,11 @@ __global__ __launch_bounds__(256) void discumsum_pair_fwd_kernel(const T* __rest
                                                                  float* __restrict__ Y2, int n, int n_out, int H,
                                                                  long F, long F2, int nblk, const T* __restrict__ Y0,
                                                                  const float* __restrict__ Y02, T* __restrict__ Yfin,
-                                                                 float* __restrict__ Yfin2) {
+                                                                 float* __restrict__ Yfin2, int follow) {
   __shared__ float gsh[SCAN_MAXN];
   const float* gs = stage_gates(gsh, logG, n, H);
+  // (the readers take the input wherever an entry equals it: nothing of this (batch, head) is read or written)
+  if (follow && gs && all_carries_zero(gs, n)) return;
   if ((int)blockIdx.x < nblk) discumsum_fwd_body<T, AHEAD, 16>(X, logG, Y, n, n_out, H, F, blockIdx.x, gs, Y0, Yfin);
   else discumsum_fwd_body<float, 64, 4>(X2, logG, Y2, n, n_out, H, F2, blockIdx.x - nblk, gs, Y02, Yfin2);
 }
@@ -250,9 +260,19 @@ __global__ __launch_bounds__(256) void discumsum_pair_bwd_kernel(const T* __rest
                                                                  int n, int n_out, int H, long F, long F2, int nblk,
                                                                  int waves_per_bh, const T* __restrict__ dYfin,
                                                                  const float* __restrict__ dYfin2,
-                                                                 T* __restrict__ dY0, float* __restrict__ dY02) {
+                                                                 T* __restrict__ dY0, float* __restrict__ dY02,
+                                                                 int follow) {
   __shared__ float gsh[SCAN_MAXN];
   const float* gs = stage_gates(gsh, logG, n, H);
+  if (follow && gs && all_carries_zero(gs, n)) {
+    // the readers take dY[k + 1] for dX[k]; the gate gradient exp(log_G[k]) * (Y[k] . dX[k]) is zero for k >= 1 by the
+    // factor and for k = 0 by Y[0] = 0: this block's partial sums are written as zeros and nothing else is touched
+    const int wave = (int)((blockIdx.x * blockDim.x + threadIdx.x) >> 6);   // (as the bodies number their waves)
+    float* part = partial + (long)blockIdx.y * n * waves_per_bh + wave;
+    if (lane_id() == 0)
+      for (int k = 0; k < n; k++) part[(long)k * waves_per_bh] = 0.f;
+    return;
+  }
   if ((int)blockIdx.x < nblk)
     discumsum_bwd_body<T, AHEAD, 16>(dY, Y, logG, dX, partial, n, n_out, H, F, waves_per_bh, blockIdx.x, 0, gs, dYfin,
                                      dY0);
@@ -324,39 +344,46 @@ static int launch_bwd(const void* dY, const void* Y, const float* logG, void* dX
 
 template <typename T>
 static int launch_pair_fwd(const void* X, const float* X2, const float* logG, void* Y, float* Y2, int B, int n,
-                           int n_out, int H, long F, long F2, const ScanCarry& cy, hipStream_t st) {
+                           int n_out, int H, long F, long F2, const ScanCarry& cy, int follow, hipStream_t st) {
   const int nblk = (int)((F / Pack16<T>::N + 255) / 256), nblk2 = (int)((F2 + 255) / 256);
   dim3 grid((unsigned)(nblk + nblk2), (unsigned)(B * H));
   if ((F / Pack16<T>::N) * B * H < 256 * 1024)
     PR_LAUNCH("discumsum_pair_fwd", (discumsum_pair_fwd_kernel<T, 16>), grid, dim3(256), 0, st, (const T*)X, X2, logG, (T*)Y, Y2, n,
-              n_out, H, F, F2, nblk, (const T*)cy.in, cy.in2, (T*)cy.out, cy.out2);
+              n_out, H, F, F2, nblk, (const T*)cy.in, cy.in2, (T*)cy.out, cy.out2, follow);
   else
     PR_LAUNCH("discumsum_pair_fwd", (discumsum_pair_fwd_kernel<T, 4>), grid, dim3(256), 0, st, (const T*)X, X2, logG, (T*)Y, Y2, n,
-              n_out, H, F, F2, nblk, (const T*)cy.in, cy.in2, (T*)cy.out, cy.out2);
+              n_out, H, F, F2, nblk, (const T*)cy.in, cy.in2, (T*)cy.out, cy.out2, follow);
   return (int)hipGetLastError();
 }
 template <typename T>
 static int launch_pair_bwd(const void* dY, const void* Y, const float* dY2, const float* Y2, const float* logG,
                            void* dX, float* dX2, float* dlogG, float* partial, int B, int n, int n_out, int H, long F,
-                           long F2, const ScanCarry& cy, hipStream_t st) {
+                           long F2, const ScanCarry& cy, int follow, hipStream_t st) {
   const int nblk = (int)((F / Pack16<T>::N + 255) / 256), nblk2 = (int)((F2 + 255) / 256);
   const int waves = (nblk + nblk2) * 4, tot = B * H * n;
   dim3 grid((unsigned)(nblk + nblk2), (unsigned)(B * H));
   if ((F / Pack16<T>::N) * B * H < 256 * 1024)
     PR_LAUNCH("discumsum_pair_bwd", (discumsum_pair_bwd_kernel<T, 8>), grid, dim3(256), 0, st, (const T*)dY, (const T*)Y, dY2, Y2,
-              logG, (T*)dX, dX2, partial, n, n_out, H, F, F2, nblk, waves, (const T*)cy.in, cy.in2, (T*)cy.out, cy.out2);
+              logG, (T*)dX, dX2, partial, n, n_out, H, F, F2, nblk, waves, (const T*)cy.in, cy.in2, (T*)cy.out, cy.out2, follow);
   else
     PR_LAUNCH("discumsum_pair_bwd", (discumsum_pair_bwd_kernel<T, 2>), grid, dim3(256), 0, st, (const T*)dY, (const T*)Y, dY2, Y2,
-              logG, (T*)dX, dX2, partial, n, n_out, H, F, F2, nblk, waves, (const T*)cy.in, cy.in2, (T*)cy.out, cy.out2);
+              logG, (T*)dX, dX2, partial, n, n_out, H, F, F2, nblk, waves, (const T*)cy.in, cy.in2, (T*)cy.out, cy.out2, follow);
   PR_LAUNCH("discumsum_reduce", discumsum_reduce_kernel, dim3((tot * 64 + 255) / 256), dim3(256), 0, st, partial, dlogG, n, H,
                      waves, B * H);
   return (int)hipGetLastError();
 }
 
+// (the promise is used only where the scan has no value to start from or to hand on, keeps n entries, and its factors fit
+// the staged table)
+static int follow_ok(int follow, const ScanCarry& cy, int n, int n_out) {
+  return follow && g_gate_skip && !cy.in && !cy.out && n_out == n && n <= SCAN_MAXN;
+}
 int discumsum_pair_fwd(const void* X, const float* X2, const float* logG, void* Y, float* Y2, int B, int n, int n_out,
-                       int H, long F, long F2, const ScanCarry& cy, int dtype, hipStream_t st) {
-  if (dtype == DT_BF16) return launch_pair_fwd<bf16_t>(X, X2, logG, Y, Y2, B, n, n_out, H, F, F2, cy, st);
-  if (dtype == DT_F16) return launch_pair_fwd<f16_t>(X, X2, logG, Y, Y2, B, n, n_out, H, F, F2, cy, st);
+                       int H, long F, long F2, const ScanCarry& cy, int consumers_follow_gates, int dtype,
+                       hipStream_t st) {
+  const int fl = follow_ok(consumers_follow_gates, cy, n, n_out);
+  if (dtype == DT_BF16) return launch_pair_fwd<bf16_t>(X, X2, logG, Y, Y2, B, n, n_out, H, F, F2, cy, fl, st);
+  if (dtype == DT_F16) return launch_pair_fwd<f16_t>(X, X2, logG, Y, Y2, B, n, n_out, H, F, F2, cy, fl, st);
   return -1;
 }
 long discumsum_pair_bwd_workspace_floats(int B, int n, int H, long F, long F2) {
@@ -364,11 +391,12 @@ long discumsum_pair_bwd_workspace_floats(int B, int n, int H, long F, long F2) {
 }
 int discumsum_pair_bwd(const void* dY, const void* Y, const float* dY2, const float* Y2, const float* logG, void* dX,
                        float* dX2, float* dlogG, float* partial, int B, int n, int n_out, int H, long F, long F2,
-                       const ScanCarry& cy, int dtype, hipStream_t st) {
+                       const ScanCarry& cy, int consumers_follow_gates, int dtype, hipStream_t st) {
+  const int fl = follow_ok(consumers_follow_gates, cy, n, n_out);
   if (dtype == DT_BF16)
-    return launch_pair_bwd<bf16_t>(dY, Y, dY2, Y2, logG, dX, dX2, dlogG, partial, B, n, n_out, H, F, F2, cy, st);
+    return launch_pair_bwd<bf16_t>(dY, Y, dY2, Y2, logG, dX, dX2, dlogG, partial, B, n, n_out, H, F, F2, cy, fl, st);
   if (dtype == DT_F16)
-    return launch_pair_bwd<f16_t>(dY, Y, dY2, Y2, logG, dX, dX2, dlogG, partial, B, n, n_out, H, F, F2, cy, st);
+    return launch_pair_bwd<f16_t>(dY, Y, dY2, Y2, logG, dX, dX2, dlogG, partial, B, n, n_out, H, F, F2, cy, fl, st);
   return -1;
 }
 

@@ -4,6 +4,9 @@
 
 namespace pr {
 
+// 1 (default): kernels leave out work whose every term the gates have decayed to an exact zero (pr_set_gate_skipping)
+extern int g_gate_skip;
+
 // discumsum.hip
 int discumsum_fwd(const void* X, const float* logG, void* Y, int B, int n, int n_out, int H, long F, int dtype,
                   hipStream_t st);
@@ -20,12 +23,18 @@ struct ScanCarry {
   void* out = nullptr;
   float* out2 = nullptr;
 };
+// consumers_follow_gates != 0 (both directions; only without a ScanCarry and with n_out == n): the caller promises that
+// whoever reads entry k of the scan's output reads the scan's input instead wherever the two are equal because the
+// carry into it is an exact zero (forward: Y[k] = X[k-1] when exp(logG[k-1]) == 0 or k == 1; backward: dX[k] = dY[k+1]
+// when exp(logG[k+1]) == 0).  A (batch, head) whose every factor exp(logG[k]), k >= 1, is zero is then not scanned at
+// all: nothing of it is read or written (backward: its gate gradient is written as zero).
 int discumsum_pair_fwd(const void* X, const float* X2, const float* logG, void* Y, float* Y2, int B, int n, int n_out,
-                       int H, long F, long F2, const ScanCarry& cy, int dtype, hipStream_t st);
+                       int H, long F, long F2, const ScanCarry& cy, int consumers_follow_gates, int dtype,
+                       hipStream_t st);
 long discumsum_pair_bwd_workspace_floats(int B, int n, int H, long F, long F2);
 int discumsum_pair_bwd(const void* dY, const void* Y, const float* dY2, const float* Y2, const float* logG, void* dX,
                        float* dX2, float* dlogG, float* partial, int B, int n, int n_out, int H, long F, long F2,
-                       const ScanCarry& cy, int dtype, hipStream_t st);
+                       const ScanCarry& cy, int consumers_follow_gates, int dtype, hipStream_t st);
 long discumsum_bwd_workspace_floats(int B, int n, int H, long F, int dtype);
 // gate gradient of the pair of scans from the scans Y, Y2 and the already formed input gradients R, R2 ([B,n,H,*])
 long scan_gate_grad_workspace_floats(int B, int n, int H, long F, long F2);
@@ -35,8 +44,11 @@ int scan_gate_grad(const void* Y, const void* R, const float* Y2, const float* R
 // sympow_tn.hip: A [BN,c,h*r,d], Bm [BN,c,h*r,d], w [BN,c,h*r] or null -> S [BN,h,D,d], s [BN,h,D]
 // skip: 0 = every chunk; +n = the last chunk of every n is not computed and its S, s are left unwritten (nobody reads
 // them); -n = the first chunk of every n is not computed and its S, s are written as zeros.
+// live [BN, h, 2] or null: per (chunk, kv head) {first time step whose A rows are not all zero, end of the time steps
+// whose Bm rows are not all zero} (chunk_prep_fwd writes them from the gates); live_side 0 / 1 says which of the two
+// holds for this call's operands: the stages of rows outside it are not read.
 int sympow_tn(const void* A, const void* Bm, const float* w, void* S, float* s, int BN, int c, int h, int r, int d,
-              int use_mult, int skip, int dtype, hipStream_t st);
+              int use_mult, int skip, const int* live, int live_side, int dtype, hipStream_t st);
 // The same contraction chained with the gated scan over the n chunks of a batch element (A, Bm [B,n*c,h*r,d],
 // lcs [B,n,h] or null): entry k of S, s [B*n,h,D,*] is the scan's k-th value (forward) or the scan's input gradient
 // (reverse).  sympow_tn_chain_ok: 0 = shape not supported, 1 = supported, 2 = and enough independent work to pay.
@@ -63,6 +75,13 @@ struct NNArgs {
                         // quarter of every such block is not read
   const float* qgate;   // [BN, c, h] or null (merge only): log of a factor on the state part of every row of a kv head
                         // at a position -- out and den are those of X * exp(qgate / 2) without forming that product
+  const int* live_rows = nullptr;   // [BN, h, 2] or null (plain only): X rows before time step live_rows[bn, hh, 0] are
+                                    // exact zeros (chunk_prep_fwd writes it); their output is zero and is not computed
+  // Optional stand-in for B (plain only; all null otherwise).  B is the output of the reverse gated scan over the
+  // chunks, whose entry bn equals the scan's INPUT entry bn + 1 exactly when the carry exp(carry[bn + 1, hh]) is zero:
+  // the kernel then reads B_alt[bn + 1] (and the scan need not have written B[bn]; see discumsum_pair_bwd).
+  const void* B_alt = nullptr;      // [BN, h, D, d]
+  const float* carry = nullptr;     // [BN, h] log of the scan's factors
 };
 int sympow_nn(const NNArgs& a, int BN, int d, int mult, int epi, int dtype, hipStream_t st);
 
@@ -80,6 +99,13 @@ struct ChunkFwdArgs {
   int c, h, r, n;    // n: chunks per batch entry
   float scale;
   int skip_first;    // chunk 0 of every batch entry has a zero state (not read)
+  int gate_skip;     // leave out what the gates have decayed to exact zeros (key tiles, the state sweep of a row block)
+  // Optional stand-ins for S, s (null otherwise): the per-chunk sums that the forward scan turned into S, s.  Entry bn of
+  // the scan equals entry bn - 1 of its input exactly when the carry exp(carry[bn - 1, hh]) is zero (or, with
+  // skip_first, bn - 1 is the first chunk of its batch entry): the kernel then reads S_alt[bn - 1], s_alt[bn - 1].
+  const void* S_alt = nullptr;
+  const float* s_alt = nullptr;
+  const float* carry = nullptr;   // [BN, h]
 };
 int chunk_fwd_supported(int d, int dtype);
 int chunk_fwd(const ChunkFwdArgs& a, int BN, int d, int dtype, hipStream_t st);
@@ -103,6 +129,10 @@ struct ChunkBwdDqArgs {
   int c, h, r, n;         // n: chunks per batch entry
   float scale;
   int skip_first;         // chunk 0 of every batch entry has a zero state (not read)
+  int gate_skip;          // leave out what the gates have decayed to exact zeros (key tiles, the state sweep of a row block)
+  const void* S_alt = nullptr;    // stand-ins for S, s as in ChunkFwdArgs
+  const float* s_alt = nullptr;
+  const float* carry = nullptr;
 };
 int chunk_bwd_dq_supported(int d, int dtype);
 int chunk_bwd_dq(const ChunkBwdDqArgs& a, int BN, int d, int dtype, hipStream_t st);
@@ -119,6 +149,17 @@ struct GradArgs {
   int skip_first;     // bit 0: chunk 0 of every batch entry has a zero state, bit 1: chunk n-1 has a zero B: dX = 0
                       // there and nothing is read
   int sym_diag;       // B[(a, b)] == B[(b, a)] in the blocks on the diagonal (the caller's promise)
+  // [BN, h, 2] or null (chunk_prep_fwd writes it): live_side 0 -- X rows before time step live_rows[bn, hh, 0] are exact
+  // zeros; live_side 1 -- G rows and cvec from time step live_rows[bn, hh, 1] on are.  dX is zero there, not computed.
+  const int* live_rows = nullptr;
+  int live_side = 0;
+  // Optional stand-ins for B, sB as in NNArgs (alt_shift = +1: B is a reverse scan's output and B_alt its input; -1: B
+  // is a forward scan's output, whose entry bn equals the input entry bn - 1 when exp(carry[bn - 1, hh]) is zero or,
+  // with bit 0 of skip_first, bn - 1 is the first chunk of its batch entry).
+  const void* B_alt = nullptr;
+  const float* sB_alt = nullptr;
+  const float* carry = nullptr;
+  int alt_shift = 0;
 };
 int sympow_grad(const GradArgs& a, int BN, int d, int mult, int dtype, hipStream_t st);
 
@@ -172,8 +213,11 @@ int qs_bwd_prep(const void* O, const void* dO, const float* den, const float* ro
 // chunk_glue.hip (return -5: chunk longer than the LDS-resident gate vector allows)
 int gate_cumsum(const float* logG, float* A, int B, int t, int h, hipStream_t st);
 // (Qg may be null: the gated queries are then not formed)
-int chunk_prep_fwd(const float* logG, const void* K, const void* Q, float* A, float* lcs, void* Kd, void* Qg, int BN,
-                   int c, int h, int r, int d, int deg, int dtype, hipStream_t st);
+// live [BN, h, 2] or null: receives, per (chunk, kv head), the first time step whose discounted key is not zeroed by
+// its factor exp((A_last - A_t) / deg), and one past the last time step whose factor exp(A_t) on the state part of a
+// query is not zero (written with the sums, i.e. when logG is given)
+int chunk_prep_fwd(const float* logG, const void* K, const void* Q, float* A, float* lcs, void* Kd, void* Qg, int* live,
+                   int BN, int c, int h, int r, int d, int deg, int dtype, hipStream_t st);
 int chunk_gate_scan_bwd(float* dA, const float* dGq, const float* dotk, const float* dlcs_a, const float* dlcs_b, int BN,
                         int c, int h, int r, int deg, hipStream_t st);
 

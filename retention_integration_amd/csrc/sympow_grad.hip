@@ -68,7 +68,10 @@ __global__ __launch_bounds__(256, (MT == 2 && DK <= 64) ? 4 : 2) void sympow_gra
   const int xcd = blockIdx.x % 8, slot = blockIdx.x / 8;
   const int pair = (slot / row_blocks) * 8 + xcd;
   if (pair >= npairs) return;
-  const int row0 = (slot % row_blocks) * ROWS;
+  // (the row blocks of a pair stay neighbours in launch order, but which of them comes first rotates from pair to pair:
+  // when the blocks of one position finish at once -- zero rows, see below -- the ones that do work would otherwise sit
+  // at a fixed stride of the launch order, and with it on a fixed subset of the compute units)
+  const int row0 = ((slot + slot / row_blocks) % row_blocks) * ROWS;
   const int bn = pair / a.h, hh = pair % a.h;
 
   const int tid = threadIdx.x, l = tid & 63, g = l >> 4, tcol = l & 15;
@@ -78,6 +81,16 @@ __global__ __launch_bounds__(256, (MT == 2 && DK <= 64) ? 4 : 2) void sympow_gra
   const T* Gg = (const T*)a.G + (long)bn * a.c * hA * DV;
   const char* Bg = (const char*)((const T*)a.B + ((long)bn * a.h + hh) * D * DV);
   const float* sBg = a.sB + ((long)bn * a.h + hh) * D;
+  // (B, sB are a gated scan's output: with a zero carry into it, an entry is the scan's input entry next to it, bit for
+  // bit -- bn + 1 for the reverse scan, bn - 1 for the forward one, whose entry 1 is its input entry 0 whatever the gate)
+  if (a.B_alt && (a.alt_shift > 0 ? bn % a.n != a.n - 1 : bn % a.n != 0)) {
+    const int nb = bn + a.alt_shift;
+    const bool first = a.alt_shift < 0 && (a.skip_first & 1) && nb % a.n == 0;
+    if (first || __expf(a.carry[(long)nb * a.h + hh]) == 0.f) {
+      Bg = (const char*)((const T*)a.B_alt + ((long)nb * a.h + hh) * D * DV);
+      sBg = a.sB_alt + ((long)nb * a.h + hh) * D;
+    }
+  }
   T* dXg = (T*)a.dX + (long)bn * a.c * hA * DK;
   auto row_off = [&](int row) -> long {
     row = min(row, rows - 1);
@@ -86,11 +99,14 @@ __global__ __launch_bounds__(256, (MT == 2 && DK <= 64) ? 4 : 2) void sympow_gra
   };
 
   // (skip_first: bit 0 = the first, bit 1 = the last chunk of every n contributes nothing and is written as zeros)
-  if (a.skip_first && (((a.skip_first & 1) && bn % a.n == 0) || ((a.skip_first & 2) && bn % a.n == a.n - 1))) {
+  auto write_zeros = [&]() {
     for (int i = tid; i < ROWS * DK / 8; i += 256) {
       const int rl = i / (DK / 8), col = (i % (DK / 8)) * 8;
       if (row0 + rl < rows) *(u32x4*)(dXg + row_off(row0 + rl) * DK + col) = (u32x4){0, 0, 0, 0};
     }
+  };
+  if (a.skip_first && (((a.skip_first & 1) && bn % a.n == 0) || ((a.skip_first & 2) && bn % a.n == a.n - 1))) {
+    write_zeros();
     return;
   }
 
@@ -120,6 +136,19 @@ __global__ __launch_bounds__(256, (MT == 2 && DK <= 64) ? 4 : 2) void sympow_gra
   async_load_tile<CX, ROWS>(xt, [&](int row) { return (const char*)(Xg + row_off(row0 + row) * DK); });
   issue(0);
   if (GR_NST > 2) issue(1);
+  // dX is linear in the row's x (every feature is a product of two of its entries) and in the pair (g, cvec) of the
+  // row.  live_rows (per (chunk, head): {first time step whose x row -- a discounted key -- is not an exact zero, end of
+  // the time steps whose (g, cvec) -- a query row's scaled dO and key-sum factor -- are not}; live_side says which of the
+  // two applies to this call) bounds the rows that can have a gradient: a block outside them is written as zeros
+  // without the sweep.
+  if (a.live_rows) {
+    const int v = a.live_rows[((long)bn * a.h + hh) * 2 + a.live_side];
+    if (a.live_side == 0 ? row0 + ROWS <= v * a.r : row0 >= v * a.r) {
+      wait_vmcnt<0>();
+      write_zeros();
+      return;
+    }
+  }
 
   // per-lane row data (row = this lane's column of the dphi^T tiles)
   v8 Gf[MT][KS];
@@ -337,7 +366,12 @@ __global__ __launch_bounds__(256, (MT == 2 && DK <= 64) ? 4 : 2) void sympow_gra
 }
 
 template <typename T, int DK, int DV, bool MULT, bool SYM>
-static int grad_launch(const GradArgs& a, int BN, hipStream_t st) {
+static int grad_launch(const GradArgs& a_, int BN, hipStream_t st) {
+  GradArgs a = a_;
+  if (!g_gate_skip) {   // every row block is swept and the scan's own output is read
+    a.live_rows = nullptr;
+    a.B_alt = nullptr;
+  }
   const int rows = a.c * a.r, npairs = BN * a.h;
   auto go = [&](auto mt, auto alone_c) {
     constexpr int MT = decltype(mt)::value;

@@ -98,7 +98,10 @@ __global__ __launch_bounds__(256, DK <= 64 ? 3 : 2) void sympow_nn_kernel(NNArgs
   const int xcd = blockIdx.x % 8, slot = blockIdx.x / 8;
   const int pair = (slot / row_blocks) * 8 + xcd;
   if (pair >= npairs) return;
-  const int row0 = (slot % row_blocks) * ROWS;
+  // (the row blocks of a pair stay neighbours in launch order, but which of them comes first rotates from pair to pair:
+  // when the blocks of one position finish at once -- zero rows, see below -- the ones that do work would otherwise sit
+  // at a fixed stride of the launch order, and with it on a fixed subset of the compute units)
+  const int row0 = ((slot + slot / row_blocks) % row_blocks) * ROWS;
   const int bn = pair / a.h, hh = pair % a.h;
 
   const int tid = threadIdx.x, l = tid & 63, g = l >> 4, tcol = l & 15;
@@ -106,6 +109,9 @@ __global__ __launch_bounds__(256, DK <= 64 ? 3 : 2) void sympow_nn_kernel(NNArgs
   const int hA = a.h * a.r, rows = a.c * a.r;
   const T* Xg = (const T*)a.X + (long)bn * a.c * hA * DK;
   const char* Bg = (const char*)((const T*)a.B + ((long)bn * a.h + hh) * D * DV);
+  // (B is a reverse scan's output: with a zero carry into it, entry bn is the scan's input entry bn + 1, bit for bit)
+  if (a.B_alt && bn % a.n != a.n - 1 && __expf(a.carry[(long)(bn + 1) * a.h + hh]) == 0.f)
+    Bg = (const char*)((const T*)a.B_alt + ((long)(bn + 1) * a.h + hh) * D * DV);
   const float* sBg = a.sB ? a.sB + ((long)bn * a.h + hh) * D : nullptr;
   auto row_off = [&](int row) -> long {  // element offset of a (clamped) folded row, per unit of the last dim
     row = min(row, rows - 1);
@@ -170,6 +176,16 @@ __global__ __launch_bounds__(256, DK <= 64 ? 3 : 2) void sympow_nn_kernel(NNArgs
     for (; issued < NN_NST - 1 && !nxt.done(); issued++) {
       issue(nxt.f0(), issued % NN_NST, nxt.narrow());
       nxt.next();
+    }
+    // X rows before time step live_rows[bn, hh, 0] are exact zeros (keys that their discount has turned into zeros), and
+    // so are their features: a block of such rows is written as zeros without the sweep.
+    bool x_zero = false;
+    if (EPI == NN_EPI_PLAIN && a.live_rows) {
+      x_zero = row0 + ROWS <= a.live_rows[((long)bn * a.h + hh) * 2] * a.r;
+      if (x_zero) {
+        wait_vmcnt<0>();
+        lds_barrier();
+      }
     }
     PhiRow<T> prow[MT];
     int y_loaded = -1, step = 0;
@@ -258,7 +274,7 @@ __global__ __launch_bounds__(256, DK <= 64 ? 3 : 2) void sympow_nn_kernel(NNArgs
       }
       step++;
     };
-    while (!cur.done()) {
+    while (!x_zero && !cur.done()) {
       stage(IC<0>{});
       if (cur.done()) break;
       stage(IC<1>{});
@@ -385,7 +401,12 @@ __global__ __launch_bounds__(256, DK <= 64 ? 3 : 2) void sympow_nn_kernel(NNArgs
 }
 
 template <typename T, int DK, int DV, bool MULT, int EPI, bool SYM>
-static int nn_launch(const NNArgs& a, int BN, hipStream_t st) {
+static int nn_launch(const NNArgs& a_, int BN, hipStream_t st) {
+  NNArgs a = a_;
+  if (!g_gate_skip) {   // every row block is swept and the scan's own output is read
+    a.live_rows = nullptr;
+    a.B_alt = nullptr;
+  }
   const int rows = a.c * a.r, npairs = BN * a.h;
   auto go = [&](auto mt, auto alone_c) {
     constexpr int MT = decltype(mt)::value;

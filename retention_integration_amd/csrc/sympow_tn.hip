@@ -168,7 +168,8 @@ __device__ __forceinline__ void tn_store_rows(const f32x4 (&acc)[XPW][DV / 16], 
 template <typename T, int DK, int DV, int XPW, int PART, bool HAS_W, bool DIAG = false>
 __device__ __forceinline__ void tn_body(const T* __restrict__ A, const T* __restrict__ Bm, const float* __restrict__ w,
                                         T* __restrict__ S, float* __restrict__ s, int c, int hA, int r, int hh,
-                                        int bn, int h, int y, int xb, bool active, bool use_mult, char* smem) {
+                                        int bn, int h, int y, int xb, bool active, bool use_mult, char* smem,
+                                        int k0, int k1) {
   typedef typename VecOf<T>::v8 v8;
   typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
   typedef __attribute__((address_space(3))) f32x4 lds_f32x4;
@@ -181,12 +182,14 @@ __device__ __forceinline__ void tn_body(const T* __restrict__ A, const T* __rest
   static_assert(CA == CB && TN_NST == 3 && (KT == 64 || DV > 64), "the loops below are written for these shapes");
   const int tid = threadIdx.x, l = tid & 63, g = l >> 4;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int rows = c * r;
+  // Stages k0 .. k1-1 of the chunk's rows are walked (the others are known to hold zero rows of A or of Bm): below,
+  // rows and stages count from stage k0.
+  const int roff = k0 * KT, rows = c * r - roff;
   const char* a_base = (const char*)(A + (long)bn * c * hA * DK);
   const char* b_base = (const char*)(Bm + (long)bn * c * hA * DV);
   const float* w_base = w + (long)bn * c * hA;
   auto row_index = [&](int row) -> long {   // element offset of a (clamped) folded row, per unit of the last dim
-    row = min(row, rows - 1);
+    row = min(row, rows - 1) + roff;
     const int t = row / r, rr = row - t * r;
     return (long)t * hA + hh * r + rr;
   };
@@ -307,8 +310,10 @@ __device__ __forceinline__ void tn_body(const T* __restrict__ A, const T* __rest
     }
   };
 
-  const int steps = (rows + KT - 1) / KT;
-  if constexpr (PREFETCH) {
+  const int steps = k1 - k0;
+  if (steps <= 0) {
+    // nothing to add up: the zero accumulators are stored
+  } else if constexpr (PREFETCH) {
     issue(0);
     if (steps > 1) issue(1);
     if (steps > 2) issue(2);
@@ -390,7 +395,8 @@ template <typename T, int DK, int DV, int XPW, bool HAS_W>
 __global__ __launch_bounds__(256, 2) void sympow_tn_kernel(const T* __restrict__ A, const T* __restrict__ Bm,
                                                            const float* __restrict__ w, T* __restrict__ S,
                                                            float* __restrict__ s, int c, int hA, int r, int h,
-                                                           int use_mult, int skip) {
+                                                           int use_mult, int skip, const int* __restrict__ live,
+                                                           int live_side) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   constexpr int PARTS = 16 / XPW;
   constexpr int NB = (DK / 16) * (DK / 16 + 1) / 2;
@@ -437,11 +443,21 @@ __global__ __launch_bounds__(256, 2) void sympow_tn_kernel(const T* __restrict__
     for (int q = l; q < nf; q += 64) s[so + q] = 0.f;
     return;
   }
+  // Stages of the chunk's rows that can hold anything but zero rows (live: per (chunk, head) the first time step whose
+  // row of A is not zero and the end of the time steps whose rows of Bm are not; live_side picks which one applies).
+  constexpr int KT_ = tn_stage_rows(DV);
+  int k0 = 0, k1 = (c * r + KT_ - 1) / KT_;
+  if (live) {
+    const int v = live[((long)bn * h + hh) * 2 + live_side];
+    if (live_side == 0) k0 = min(max(v, 0) * r / KT_, k1);
+    else k1 = min((max(v, 0) * r + KT_ - 1) / KT_, k1);
+  }
   if constexpr (XPW == 8) {
     constexpr int NOFF = (DK / 16) * (DK / 16 - 1);   // tasks below the block diagonal
     if (t2 >= NOFF) {
       y = xb = t2 - NOFF;
-      tn_body<T, DK, DV, XPW, 0, HAS_W, true>(A, Bm, w, S, s, c, hA, r, hh, bn, h, y, xb, active, use_mult != 0, smem);
+      tn_body<T, DK, DV, XPW, 0, HAS_W, true>(A, Bm, w, S, s, c, hA, r, hh, bn, h, y, xb, active, use_mult != 0, smem,
+                                              k0, k1);
       return;
     }
     y = 1;
@@ -454,7 +470,7 @@ __global__ __launch_bounds__(256, 2) void sympow_tn_kernel(const T* __restrict__
   case P:                                                                                                              \
     if (P < PARTS)                                                                                                     \
       tn_body<T, DK, DV, XPW, (P < PARTS ? P : 0), HAS_W>(A, Bm, w, S, s, c, hA, r, hh, bn, h, y, xb, active,         \
-                                                          use_mult != 0, smem);                                        \
+                                                          use_mult != 0, smem, k0, k1);                                \
     break;
   switch (part) {
     PR_TN_CASE(0)
@@ -731,7 +747,7 @@ int sympow_tn_chain(const void* A, const void* Bm, const float* w, const float* 
 
 template <typename T, int DK, int DV>
 static int tn_launch(const void* A, const void* Bm, const float* w, void* S, float* s, int BN, int c, int h, int r,
-                     int use_mult, int skip, hipStream_t st) {
+                     int use_mult, int skip, const int* live, int live_side, hipStream_t st) {
   constexpr int XPW = DV <= 64 ? 8 : 4;
   constexpr int NB = (DK / 16) * (DK / 16 + 1) / 2;
   constexpr int TASKS = tn_tasks<DK, XPW>();
@@ -741,24 +757,28 @@ static int tn_launch(const void* A, const void* Bm, const float* w, void* S, flo
   if (w) {
     auto kern = sympow_tn_kernel<T, DK, DV, XPW, true>;
     allow_big_lds((const void*)kern, smem);
-    PR_LAUNCH("sympow_tn", kern, grid, dim3(256), smem, st, (const T*)A, (const T*)Bm, w, (T*)S, s, c, h * r, r, h, use_mult, skip);
+    PR_LAUNCH("sympow_tn", kern, grid, dim3(256), smem, st, (const T*)A, (const T*)Bm, w, (T*)S, s, c, h * r, r, h, use_mult, skip,
+              live, live_side);
   } else {
     auto kern = sympow_tn_kernel<T, DK, DV, XPW, false>;
     allow_big_lds((const void*)kern, smem);
-    PR_LAUNCH("sympow_tn", kern, grid, dim3(256), smem, st, (const T*)A, (const T*)Bm, w, (T*)S, s, c, h * r, r, h, use_mult, skip);
+    PR_LAUNCH("sympow_tn", kern, grid, dim3(256), smem, st, (const T*)A, (const T*)Bm, w, (T*)S, s, c, h * r, r, h, use_mult, skip,
+              live, live_side);
   }
   return (int)hipGetLastError();
 }
 
 // A: [BN, c, h*r, d], Bm: [BN, c, h*r, d], w: [BN, c, h*r] or null -> S: [BN, h, D, d], s: [BN, h, D]
 // skip: 0, or +n / -n to skip the last / first chunk of every n (see the kernel)
+// live ([BN, h, 2] or null), live_side: see the kernel; ignored while gate skipping is switched off
 int sympow_tn(const void* A, const void* Bm, const float* w, void* S, float* s, int BN, int c, int h, int r, int d,
-              int use_mult, int skip, int dtype, hipStream_t st) {
+              int use_mult, int skip, const int* live, int live_side, int dtype, hipStream_t st) {
+  if (!g_gate_skip) live = nullptr;
 #define PR_TN_DISPATCH(T)                                                                                              \
   switch (d) {                                                                                                         \
-    case 32: return tn_launch<T, 32, 32>(A, Bm, w, S, s, BN, c, h, r, use_mult, skip, st);                                   \
-    case 64: return tn_launch<T, 64, 64>(A, Bm, w, S, s, BN, c, h, r, use_mult, skip, st);                                   \
-    case 128: return tn_launch<T, 128, 128>(A, Bm, w, S, s, BN, c, h, r, use_mult, skip, st);                                \
+    case 32: return tn_launch<T, 32, 32>(A, Bm, w, S, s, BN, c, h, r, use_mult, skip, live, live_side, st);                                   \
+    case 64: return tn_launch<T, 64, 64>(A, Bm, w, S, s, BN, c, h, r, use_mult, skip, live, live_side, st);                                   \
+    case 128: return tn_launch<T, 128, 128>(A, Bm, w, S, s, BN, c, h, r, use_mult, skip, live, live_side, st);                                \
     default: return -2;                                                                                                \
   }
   if (dtype == DT_BF16) { PR_TN_DISPATCH(bf16_t) }

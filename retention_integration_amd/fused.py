@@ -57,6 +57,13 @@ def _side_stream(device):
     return _SIDE[key]
 
 
+def _follows_gates(lib, d, deg, code):
+    """True when both readers of the scanned chunk states are the one-kernel ones, which take a chunk's own sum in
+    place of the scan's entry wherever the gates make the two equal (and gate skipping is on)."""
+    return bool(ONE_KERNEL_FWD and ONE_KERNEL_BWD_DQ and lib.pr_get_gate_skipping()
+                and lib.pr_chunk_fwd_supported(d, deg, code) and lib.pr_chunk_bwd_dq_supported(d, deg, code))
+
+
 def _empty(shape, dtype, device):
     return torch.empty(shape, dtype=dtype, device=device)
 
@@ -64,9 +71,12 @@ def _empty(shape, dtype, device):
 @torch.library.custom_op("pr::chunked_fwd", mutates_args=(), device_types="cuda")
 def chunked_fwd(Q: Tensor, K: Tensor, V: Tensor, log_G: Optional[Tensor], deg: int, scale: float, c: int,
                 S0: Optional[Tensor] = None, s0: Optional[Tensor] = None, want_final: bool = False
-                ) -> Tuple[Tensor, Tensor, Tensor, Tensor, Tensor, Tensor, Tensor, Tensor, Tensor, Tensor]:
-    """-> O, what the backward needs: A, lcs, Kd (empty when ungated), Sc, sc, rowmax, den, and the state after the
-    last token (Sf [b,h,D,d], sf [b,h,D]; empty unless want_final).
+                ) -> Tuple[Tensor, Tensor, Tensor, Tensor, Tensor, Tensor, Tensor, Tensor, Tensor, Tensor, Tensor, Tensor,
+                           Tensor]:
+    """-> O, what the backward needs: A, lcs, Kd (empty when ungated), Sc, sc, rowmax, den, the state after the
+    last token (Sf [b,h,D,d], sf [b,h,D]; empty unless want_final), and for the backward again the rows of every chunk
+    that the gates have not decayed to exact zeros (live [BN,h,2] int32; empty when ungated) and the per-chunk sums S, s
+    that the scan turned into Sc, sc (empty unless the readers of Sc, sc follow the gates, see below).
 
     S0 [b,h,D,d], s0 [b,h,D] fp32: the state the sequence starts from (the pair a previous call returned), in the
     reference layout; chunk k then sees it decayed by the gates of chunks 0..k-1 like any chunk state, and the final
@@ -95,12 +105,14 @@ def chunked_fwd(Q: Tensor, K: Tensor, V: Tensor, log_G: Optional[Tensor], deg: i
     if gated:
         A, lcs = _empty((BN, c, h), f32, dev), _empty((BN, h), f32, dev)
         Kd = torch.empty_like(K)
+        live = _empty((BN, h, 2), torch.int32, dev)
         # (the sums first: the attention kernel needs nothing else; the discounted keys follow below)
-        _lib.check(lib.pr_chunk_prep_fwd(p(log_G), p(K), p(Q), p(A), p(lcs), None, None, BN, c, h, r, d, deg, code,
-                                         st), "chunk_prep_fwd(sums)")
+        _lib.check(lib.pr_chunk_prep_fwd(p(log_G), p(K), p(Q), p(A), p(lcs), None, None, p(live), BN, c, h, r, d, deg,
+                                         code, st), "chunk_prep_fwd(sums)")
         Kd_ = Kd
     else:
         A, Kd = _empty((0,), f32, dev), _empty((0,), dt, dev)
+        live = _empty((0,), torch.int32, dev)
         Kd_ = K
         lcs = torch.zeros((BN, h), dtype=f32, device=dev)
 
@@ -119,33 +131,43 @@ def chunked_fwd(Q: Tensor, K: Tensor, V: Tensor, log_G: Optional[Tensor], deg: i
         attention(side.cuda_stream)
 
     if gated:
-        _lib.check(lib.pr_chunk_prep_fwd(None, p(K), p(Q), p(A), p(lcs), p(Kd), None, BN, c, h, r, d, deg, code, st),
-                   "chunk_prep_fwd(keys)")
+        _lib.check(lib.pr_chunk_prep_fwd(None, p(K), p(Q), p(A), p(lcs), p(Kd), None, None, BN, c, h, r, d, deg, code,
+                                         st), "chunk_prep_fwd(keys)")
     Sc, sc = _empty((BN, h, D, d), dt, dev), _empty((BN, h, D), f32, dev)
     Sf, sf = _empty((0,), dt, dev), _empty((0,), f32, dev)
+    S, s = _empty((0,), dt, dev), _empty((0,), f32, dev)
+    follow = False
     if chained:
         # short chunks: the chunk states are scanned as they are formed and never written on their own
         _lib.check(lib.pr_update_state_scan_fwd(p(Kd_), p(V), p(lcs) if gated else None, p(Sc), p(sc), b, n, c, h, d,
                                                 deg, code, st), "update_state_scan_fwd")
     else:
         S, s = torch.empty_like(Sc), torch.empty_like(sc)
+        # Where the gates let nothing through from one chunk to the next (exp(lcs) == 0), the scan's entry k IS the sum
+        # of chunk k-1: the kernels that read a chunk's state then take that sum directly (they are handed both), and a
+        # sequence of a head whose every carry is zero is not scanned at all.  Only with the one-kernel readers, which
+        # know the rule, on both sides of the step.
+        follow = bool(gated and not carried and not want_final and _follows_gates(lib, d, deg, code))
         # (the last chunk's own state is only needed for the state after the last token)
-        _lib.check(lib.pr_update_state_fwd(p(Kd_), p(V), p(S), p(s), BN, c, h, d, deg, 0 if want_final else n, code, st),
-                   "update_state_fwd")
+        # (... or when the sums themselves are handed to the backward: an output of the node holds no unwritten memory)
+        _lib.check(lib.pr_update_state_fwd(p(Kd_), p(V), p(S), p(s), p(live) if gated else None, BN, c, h, d, deg,
+                                           0 if want_final or follow else n, code, st), "update_state_fwd")
         s0f = s0.to(f32).contiguous() if carried else None
         if want_final:
             Sf, sf = _empty((b, h, D, d), dt, dev), _empty((b, h, D), f32, dev)
         # the carried state is the scan's starting value, the state after the last token its entry n
         _lib.check(lib.pr_state_scan_fwd(p(S), p(s), p(lcs), p(Sc), p(sc), p(S0) if carried else None, p(s0f),
                                          p(Sf) if want_final else None, p(sf) if want_final else None, b, n, n, h,
-                                         D * d, D, code, st), "state_scan_fwd")
-        del S, s
+                                         D * d, D, 1 if follow else 0, code, st), "state_scan_fwd")
+        if not follow:
+            S, s = _empty((0,), dt, dev), _empty((0,), f32, dev)
 
     O, den = torch.empty_like(Q), _empty((BN, c, hq), f32, dev)
     if one_kernel:
-        _lib.check(lib.pr_chunk_fwd(p(Q), p(K), p(V), p(A) if gated else None, p(Sc), p(sc), p(O), p(rm), p(den), BN, n,
+        _lib.check(lib.pr_chunk_fwd(p(Q), p(K), p(V), p(A) if gated else None, p(Sc), p(sc), p(S) if follow else None,
+                                    p(s) if follow else None, p(lcs) if follow else None, p(O), p(rm), p(den), BN, n,
                                     c, h, r, d, scale, deg, 0 if carried else 1, code, st), "chunk_fwd")
-        return O, A, lcs, Kd, Sc, sc, rm, den, Sf, sf
+        return O, A, lcs, Kd, Sc, sc, rm, den, Sf, sf, live, S, s
     if two_streams:
         main.wait_stream(side)
     else:
@@ -153,7 +175,7 @@ def chunked_fwd(Q: Tensor, K: Tensor, V: Tensor, log_G: Optional[Tensor], deg: i
     _lib.check(lib.pr_query_state_fwd(p(Q), p(Sc), p(sc), p(Ya), p(la), p(rm), p(A) if gated else None, p(O), p(den),
                                       BN, n, c, h, r, d, scale ** deg, deg, 0 if carried else 1, 1, code, st),
                "query_state_fwd")
-    return O, A, lcs, Kd, Sc, sc, rm, den, Sf, sf
+    return O, A, lcs, Kd, Sc, sc, rm, den, Sf, sf, live, S, s
 
 
 @chunked_fwd.register_fake
@@ -164,24 +186,34 @@ def _(Q, K, V, log_G, deg, scale, c, S0=None, s0=None, want_final=False):
     D = Dr = expanded_dim(d)
     f32 = torch.float32
     gated = log_G is not None
+    lib = _lib.load()
+    follow = bool(gated and S0 is None and not want_final and not _chained(lib, b, t // c, c, h, 1, d)
+                  and _follows_gates(lib, d, deg, _lib.dtype_code(Q.dtype)))
     A = Q.new_empty((BN, c, h) if gated else (0,), dtype=f32)
     return (torch.empty_like(Q), A, Q.new_empty((BN, h), dtype=f32),
             torch.empty_like(K) if gated else K.new_empty((0,)),
             Q.new_empty((BN, h, D, d)), Q.new_empty((BN, h, D), dtype=f32), Q.new_empty((BN, c, hq), dtype=f32),
             Q.new_empty((BN, c, hq), dtype=f32),
-            Q.new_empty((b, h, Dr, d) if want_final else (0,)), Q.new_empty((b, h, Dr) if want_final else (0,), dtype=f32))
+            Q.new_empty((b, h, Dr, d) if want_final else (0,)), Q.new_empty((b, h, Dr) if want_final else (0,), dtype=f32),
+            Q.new_empty((BN, h, 2) if gated else (0,), dtype=torch.int32),
+            Q.new_empty((BN, h, D, d) if follow else (0,)), Q.new_empty((BN, h, D) if follow else (0,), dtype=f32))
 
 
 @torch.library.custom_op("pr::chunked_bwd", mutates_args=(), device_types="cuda")
 def chunked_bwd(Q: Tensor, K: Tensor, V: Tensor, A: Tensor, lcs: Tensor, Kd: Tensor, Sc: Tensor,
                 sc: Tensor, rm: Tensor, O: Tensor, den: Tensor, dO: Tensor, deg: int, scale: float, c: int,
-                gated: bool, carried: bool = False, dSf: Optional[Tensor] = None, dsf: Optional[Tensor] = None
+                gated: bool, carried: bool = False, dSf: Optional[Tensor] = None, dsf: Optional[Tensor] = None,
+                live: Optional[Tensor] = None, S: Optional[Tensor] = None, s: Optional[Tensor] = None
                 ) -> Tuple[Tensor, Tensor, Tensor, Tensor, Tensor, Tensor]:
     """-> dQ, dK, dV, dlog_G (empty when ungated), and the gradient of the state the sequence started from
-    (dS0 [b,h,D,d], ds0 [b,h,D]; empty unless carried).  dSf, dsf: gradient of the returned final state, or None."""
+    (dS0 [b,h,D,d], ds0 [b,h,D]; empty unless carried).  dSf, dsf: gradient of the returned final state, or None.
+    live: the forward's array of the rows that the gates left alive, or None.  S, s: the per-chunk sums, given when the
+    forward's scan counted on readers that follow the gates (the backward then does the same, and must)."""
     if not gated:
         Kd = K
     qgate = _lib.ptr(A) if gated else None
+    live_p = _lib.ptr(live) if gated and live is not None and live.numel() else None
+    follow = S is not None and S.numel() > 0
     lib = _lib.load()
     st = _lib.stream()
     b, t, hq, d = Q.shape
@@ -216,9 +248,12 @@ def chunked_bwd(Q: Tensor, K: Tensor, V: Tensor, A: Tensor, lcs: Tensor, Kd: Ten
 
         def qs_bwd(dQ_, dS_, ds_, prepared, stream):
             _lib.check(lib.pr_query_state_bwd(p(Q), p(Sc), p(sc), p(rm), qgate, p(O), p(den), p(dO), dQ_, dS_, ds_, None,
-                                              p(dla), p(dys), p(qws), BN, n, c, h, r, d, scale ** deg, deg, zis, 1,
-                                              prepared, code, stream), "query_state_bwd")
+                                              p(dla), p(dys), p(qws), live_p, BN, n, c, h, r, d, scale ** deg, deg, zis,
+                                              1, prepared, code, stream), "query_state_bwd")
         dq_one_kernel = ONE_KERNEL_BWD_DQ and bool(lib.pr_chunk_bwd_dq_supported(d, deg, code))
+        if follow and not (dq_one_kernel and lib.pr_get_gate_skipping()):
+            raise RuntimeError("the forward left out scans that this backward would read: keep ONE_KERNEL_BWD_DQ and "
+                               "gate skipping as they were for the forward")
         dQa = torch.empty_like(Q)
         dGq = _empty((BN, c, hq), f32, dev) if gated else None
 
@@ -226,8 +261,9 @@ def chunked_bwd(Q: Tensor, K: Tensor, V: Tensor, A: Tensor, lcs: Tensor, Kd: Ten
             # (the workspace of pr_query_state_bwd: the scaled dO, then the row vector of the key-sum term)
             cvec = qws.data_ptr() + (BN * c * hq * d * 2 + 255) // 256 * 256
             _lib.check(lib.pr_chunk_bwd_dq(p(Q), p(K), p(V), qgate, p(rm), p(den), p(dO), p(dla), p(dys), cvec, p(Sc),
-                                           p(sc), p(dQa), p(dGq), BN, n, c, h, r, d, scale, deg, 0 if carried else 1,
-                                           code, stream), "chunk_bwd_dq")
+                                           p(sc), p(S) if follow else None, p(s) if follow else None,
+                                           p(lcs) if follow else None, p(dQa), p(dGq), BN, n, c, h, r, d, scale, deg,
+                                           0 if carried else 1, code, stream), "chunk_bwd_dq")
         if dq_one_kernel:
             qs_bwd(None, p(dSc), p(dsc), 0, st)          # preparation and dS; the query side follows further down
             if not BWD_TWO_STREAMS:
@@ -251,9 +287,11 @@ def chunked_bwd(Q: Tensor, K: Tensor, V: Tensor, A: Tensor, lcs: Tensor, Kd: Ten
         sws = _empty((lib.pr_state_scan_bwd_workspace(b, n, h, D * d, D),), u8, dev)
         _lib.check(lib.pr_state_scan_bwd(p(dSc), p(Sc), p(dsc), p(sc), p(lcs), p(dS), p(ds), p(dlcs), p(sws), p(dSf_),
                                          p(dsf_), p(dS0) if carried else None, p(ds0) if carried else None, b, n, n, h,
-                                         D * d, D, code, st), "state_scan_bwd")
+                                         D * d, D, 1 if follow else 0, code, st), "state_scan_bwd")
         two_streams = BWD_TWO_STREAMS
     dKd, dVs = torch.empty_like(K), torch.empty_like(V)
+    # (where the reverse scan lets nothing through, its entry k IS its input entry k + 1: the kernels are handed both)
+    scan_in = (p(dSc), p(dsc), p(lcs)) if follow else (None, None, None)
     # (dS comes from the kernels above, so both orders of a pair hold the same sum: the symmetry flag says so; the last
     # chunk's dS is zero unless a gradient arrived through the final state)
     if two_streams and dq_one_kernel:
@@ -261,7 +299,7 @@ def chunked_bwd(Q: Tensor, K: Tensor, V: Tensor, A: Tensor, lcs: Tensor, Kd: Ten
         # beside: started after dV, next to dK and the key side of the attention backward, the step is 15-25 us shorter
         # than with it next to dS and the reverse scan (measured at every point of the chain).
         def usb(dk_, dv_):
-            _lib.check(lib.pr_update_state_bwd(p(Kd), p(V), p(dS), p(ds), dk_, dv_, BN, c, h, d, deg, 1,
+            _lib.check(lib.pr_update_state_bwd(p(Kd), p(V), p(dS), p(ds), *scan_in, live_p, dk_, dv_, BN, c, h, d, deg, 1,
                                                0 if has_dfin else n, code, st), "update_state_bwd")
         main, side = torch.cuda.current_stream(), _side_stream(dev)
         usb(None, p(dVs))
@@ -269,8 +307,8 @@ def chunked_bwd(Q: Tensor, K: Tensor, V: Tensor, A: Tensor, lcs: Tensor, Kd: Ten
         query_side(side.cuda_stream)
         usb(p(dKd), None)
     else:
-        _lib.check(lib.pr_update_state_bwd(p(Kd), p(V), p(dS), p(ds), p(dKd), p(dVs), BN, c, h, d, deg, 1,
-                                           0 if has_dfin else n, code, st), "update_state_bwd")
+        _lib.check(lib.pr_update_state_bwd(p(Kd), p(V), p(dS), p(ds), *scan_in, live_p, p(dKd), p(dVs), BN, c, h, d, deg,
+                                           1, 0 if has_dfin else n, code, st), "update_state_bwd")
 
     # the attention backward adds the state-path gradients in its epilogue and writes the final dQ, dK, dV
     dKa, dVa = torch.empty_like(K), torch.empty_like(V)
@@ -313,7 +351,8 @@ def chunked_bwd(Q: Tensor, K: Tensor, V: Tensor, A: Tensor, lcs: Tensor, Kd: Ten
 
 
 @chunked_bwd.register_fake
-def _(Q, K, V, A, lcs, Kd, Sc, sc, rm, O, den, dO, deg, scale, c, gated, carried=False, dSf=None, dsf=None):
+def _(Q, K, V, A, lcs, Kd, Sc, sc, rm, O, den, dO, deg, scale, c, gated, carried=False, dSf=None, dsf=None, live=None,
+      S=None, s=None):
     b, t, _, d = Q.shape
     h = K.shape[2]
     Dr = expanded_dim(d)
@@ -325,14 +364,14 @@ def _(Q, K, V, A, lcs, Kd, Sc, sc, rm, O, den, dO, deg, scale, c, gated, carried
 
 def _chunked_setup(ctx, inputs, output):
     Q, K, V, log_G, deg, scale, c, S0, s0, want_final = inputs
-    O, A, lcs, Kd, Sc, sc, rm, den, Sf, sf = output
-    ctx.save_for_backward(Q, K, V, A, lcs, Kd, Sc, sc, rm, O, den)
+    O, A, lcs, Kd, Sc, sc, rm, den, Sf, sf, live, S, s = output
+    ctx.save_for_backward(Q, K, V, A, lcs, Kd, Sc, sc, rm, O, den, live, S, s)
     ctx.meta = (deg, scale, c, log_G is not None, S0 is not None, None if s0 is None else s0.dtype, bool(want_final))
     ctx.set_materialize_grads(False)
 
 
-def _chunked_backward(ctx, dO, dA, dlcs, dKd, dSc, dsc, drm, dden, dSf, dsf):
-    Q, K, V, A, lcs, Kd, Sc, sc, rm, O, den = ctx.saved_tensors
+def _chunked_backward(ctx, dO, dA, dlcs, dKd, dSc, dsc, drm, dden, dSf, dsf, dlive, dS_, ds_):
+    Q, K, V, A, lcs, Kd, Sc, sc, rm, O, den, live, S, s = ctx.saved_tensors
     deg, scale, c, gated, carried, s0_dtype, want_final = ctx.meta
     if not want_final:   # (the placeholders returned in place of a final state carry no gradient)
         dSf = dsf = None
@@ -341,7 +380,7 @@ def _chunked_backward(ctx, dO, dA, dlcs, dKd, dSc, dsc, drm, dden, dSf, dsf):
     if dO is None:
         dO = torch.zeros_like(O)
     dQ, dK, dV, dlg, dS0, ds0 = chunked_bwd(Q, K, V, A, lcs, Kd, Sc, sc, rm, O, den, dO, deg, scale, c, gated, carried,
-                                            dSf, dsf)
+                                            dSf, dsf, live, S, s)
     return (dQ, dK, dV, (dlg if gated else None), None, None, None, dS0 if carried else None,
             ds0.to(s0_dtype) if carried else None, None)
 

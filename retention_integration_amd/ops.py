@@ -143,7 +143,7 @@ def update_state_fwd(K: Tensor, V: Tensor) -> Tuple[Tensor, Tensor]:
     S = torch.empty((b, n, h, D, d), dtype=K.dtype, device=K.device)
     s = torch.empty((b, n, h, D), dtype=torch.float32, device=K.device)
     lib = _lib.load()
-    _lib.check(lib.pr_update_state_fwd(_lib.ptr(K), _lib.ptr(V), _lib.ptr(S), _lib.ptr(s), b * n, c, h, d, 2, 0,
+    _lib.check(lib.pr_update_state_fwd(_lib.ptr(K), _lib.ptr(V), _lib.ptr(S), _lib.ptr(s), None, b * n, c, h, d, 2, 0,
                                        _lib.dtype_code(K.dtype), _lib.stream()), "update_state_fwd")
     return S, s
 
@@ -160,7 +160,8 @@ def update_state_bwd(K: Tensor, V: Tensor, dS: Tensor, ds: Tensor) -> Tuple[Tens
     b, n, c, h, d = K.shape
     dK, dV = torch.empty_like(K), torch.empty_like(V)
     lib = _lib.load()
-    _lib.check(lib.pr_update_state_bwd(_lib.ptr(K), _lib.ptr(V), _lib.ptr(dS), _lib.ptr(ds), _lib.ptr(dK),
+    _lib.check(lib.pr_update_state_bwd(_lib.ptr(K), _lib.ptr(V), _lib.ptr(dS), _lib.ptr(ds), None, None, None, None,
+                                       _lib.ptr(dK),
                                        _lib.ptr(dV), b * n, c, h, d, 2, 0, 0, _lib.dtype_code(K.dtype), _lib.stream()),
                "update_state_bwd")
     return dK, dV
@@ -310,7 +311,7 @@ def query_state_bwd(Q: Tensor, S: Tensor, s: Tensor, rowmax: Optional[Tensor], O
     ws = torch.empty((lib.pr_query_state_bwd_workspace(b * n, c, h, r, d, code),), dtype=torch.uint8, device=Q.device)
     _lib.check(lib.pr_query_state_bwd(_lib.ptr(Q), _lib.ptr(S), _lib.ptr(s), _lib.ptr(rowmax), None, _lib.ptr(O),
                                       _lib.ptr(den), _lib.ptr(dO), _lib.ptr(dQ), _lib.ptr(dS), _lib.ptr(ds),
-                                      _lib.ptr(dYa), _lib.ptr(dla), None, _lib.ptr(ws), b * n, n, c, h, r, d,
+                                      _lib.ptr(dYa), _lib.ptr(dla), None, _lib.ptr(ws), None, b * n, n, c, h, r, d,
                                       float(scale_p), 2, int(zero_initial_state), 0, 0, code, _lib.stream()),
                "query_state_bwd")
     if not has_attn:

@@ -42,7 +42,7 @@ def test_library_exports_every_declared_symbol():
     assert [lib.pr_expanded_dim(d, 2) for d in (32, 64, 128)] == [768, 2560, 9216]
     # argument checks run before any launch: a bad head dimension is refused with a message
     lib.pr_update_state_fwd.restype = ctypes.c_int
-    lib.pr_update_state_fwd.argtypes = [ctypes.c_void_p] * 4 + [ctypes.c_int] * 7 + [ctypes.c_void_p]
-    rc = lib.pr_update_state_fwd(16, 16, 16, 16, 1, 16, 1, 48, 2, 0, 0, None)
+    lib.pr_update_state_fwd.argtypes = [ctypes.c_void_p] * 5 + [ctypes.c_int] * 7 + [ctypes.c_void_p]
+    rc = lib.pr_update_state_fwd(16, 16, 16, 16, None, 1, 16, 1, 48, 2, 0, 0, None)
     lib.pr_last_error.restype = ctypes.c_char_p
     assert rc != 0 and b"head dim" in lib.pr_last_error()

@@ -98,7 +98,7 @@ def test_state_scan_pair_equals_separate_scans(pra, dtype, F, n_out_extra):
     code = _lib.dtype_code(dtype)
     Sc, sc = torch.empty(b, n_out, h, F, dtype=dtype, device=DEV), torch.empty(b, n_out, h, F2, device=DEV)
     Sc1, sc1 = torch.empty_like(Sc), torch.empty_like(sc)
-    _lib.check(lib.pr_state_scan_fwd(p(S), p(s), p(lg), p(Sc), p(sc), None, None, None, None, b, n, n_out, h, F, F2, code,
+    _lib.check(lib.pr_state_scan_fwd(p(S), p(s), p(lg), p(Sc), p(sc), None, None, None, None, b, n, n_out, h, F, F2, 0, code,
                                      st), "pair fwd")
     _lib.check(lib.pr_discumsum_fwd(p(S), p(lg), p(Sc1), b, n, n_out, h, F, code, st), "fwd")
     _lib.check(lib.pr_discumsum_fwd(p(s), p(lg), p(sc1), b, n, n_out, h, F2, _lib.PR_F32, st), "fwd")
@@ -109,7 +109,7 @@ def test_state_scan_pair_equals_separate_scans(pra, dtype, F, n_out_extra):
     dS, ds, dlg = torch.empty_like(S), torch.empty_like(s), torch.empty_like(lg)
     ws = torch.empty(lib.pr_state_scan_bwd_workspace(b, n, h, F, F2), dtype=u8, device=DEV)
     _lib.check(lib.pr_state_scan_bwd(p(dSc), p(Sc), p(dsc), p(sc), p(lg), p(dS), p(ds), p(dlg), p(ws), None, None, None,
-                                     None, b, n, n_out, h, F, F2, code, st), "pair bwd")
+                                     None, b, n, n_out, h, F, F2, 0, code, st), "pair bwd")
     dS1, ds1, dl1, dl2 = torch.empty_like(S), torch.empty_like(s), torch.empty_like(lg), torch.empty_like(lg)
     ws1 = torch.empty(max(lib.pr_discumsum_bwd_workspace(b, n, h, F, code),
                           lib.pr_discumsum_bwd_workspace(b, n, h, F2, _lib.PR_F32)), dtype=u8, device=DEV)
@@ -298,7 +298,8 @@ def test_symmetric_state_flag_changes_nothing_for_a_symmetric_state(pra, dtype, 
     res = []
     for flag in (0, 1):
         dK, dV = torch.empty_like(K), torch.empty_like(V)
-        _lib.check(lib.pr_update_state_bwd(p(K), p(V), p(S), p(s), p(dK), p(dV), b * n, c, h, d, 2, flag, 0, code, st),
+        _lib.check(lib.pr_update_state_bwd(p(K), p(V), p(S), p(s), None, None, None, None, p(dK), p(dV), b * n, c, h, d, 2,
+                                           flag, 0, code, st),
                    "update_state_bwd")
         O, den = torch.empty_like(Q), torch.empty(b, n, c, h, dtype=torch.float32, device=DEV)
         _lib.check(lib.pr_query_state_fwd(p(Q), p(S), p(s), None, None, None, None, p(O), p(den), b * n, n, c, h, 1, d,
@@ -306,7 +307,7 @@ def test_symmetric_state_flag_changes_nothing_for_a_symmetric_state(pra, dtype, 
         dQ, dS, ds = torch.empty_like(Q), torch.empty_like(S), torch.empty_like(s)
         ws = torch.empty(lib.pr_query_state_bwd_workspace(b * n, c, h, 1, d, code), dtype=torch.uint8, device=DEV)
         _lib.check(lib.pr_query_state_bwd(p(Q), p(S), p(s), None, None, p(O), p(den), p(dO), p(dQ), p(dS), p(ds), None, None,
-                                          None, p(ws), b * n, n, c, h, 1, d, 1.0 / d, 2, 0, flag, 0, code, st),
+                                          None, p(ws), None, b * n, n, c, h, 1, d, 1.0 / d, 2, 0, flag, 0, code, st),
                    "query_state_bwd")
         res.append((dK, dV, dQ, dS, ds, O, den))
     for nm, a, b_ in zip(["dK", "dV", "dQ", "dS", "ds", "O", "den"], res[1], res[0]):
@@ -385,11 +386,11 @@ def test_state_scan_with_a_starting_value_and_a_final_entry(pra, dtype, d):
     Y, y, Yf, yf = E(b, n, h, D, d), E(b, n, h, D, dt=f32), E(b, h, D, d), E(b, h, D, dt=f32)
     g = [dev(x) for x in (S, s, lg, S0, s0, dY, dy, dYf, dyf)]
     _lib.check(lib.pr_state_scan_fwd(p(g[0]), p(g[1]), p(g[2]), p(Y), p(y), p(g[3]), p(g[4]), p(Yf), p(yf), b, n, n, h,
-                                     D * d, D, code, st), "scan fwd")
+                                     D * d, D, 0, code, st), "scan fwd")
     dX, dx, dlg, dY0, dy0 = E(b, n, h, D, d), E(b, n, h, D, dt=f32), E(b, n, h, dt=f32), E(b, h, D, d), E(b, h, D, dt=f32)
     ws = torch.empty(lib.pr_state_scan_bwd_workspace(b, n, h, D * d, D), dtype=torch.uint8, device=DEV)
     _lib.check(lib.pr_state_scan_bwd(p(g[5]), p(Y), p(g[6]), p(y), p(g[2]), p(dX), p(dx), p(dlg), p(ws), p(g[7]), p(g[8]),
-                                     p(dY0), p(dy0), b, n, n, h, D * d, D, code, st), "scan bwd")
+                                     p(dY0), p(dy0), b, n, n, h, D * d, D, 0, code, st), "scan bwd")
 
     # the recurrence, in fp32 with autograd (the kernel rounds the running state only when it stores an entry)
     o = [gold(x, True) for x in (S, s, lg, S0, s0)]
@@ -455,7 +456,8 @@ def test_chunk_fwd_in_one_kernel(pra, d, c, r, gated, zis):
     g = {k: dev(v) for k, v in dict(Q=Q, K=K, V=V, A=A, S=S, s=s).items()}
     pa = p(g["A"]) if gated else None
     O, rm, den = E(BN, c, hq, d), E(BN, c, hq, dt=f32), E(BN, c, hq, dt=f32)
-    _lib.check(lib.pr_chunk_fwd(p(g["Q"]), p(g["K"]), p(g["V"]), pa, p(g["S"]), p(g["s"]), p(O), p(rm), p(den), BN, n, c,
+    _lib.check(lib.pr_chunk_fwd(p(g["Q"]), p(g["K"]), p(g["V"]), pa, p(g["S"]), p(g["s"]), None, None, None, p(O), p(rm),
+                                p(den), BN, n, c,
                                 h, r, d, scale, 2, 1 if zis else 0, code, st), "chunk_fwd")
     # (b) the two calls
     Ya, la, rm2, O2, den2 = E(BN, c, hq, d), E(BN, c, hq, dt=f32), E(BN, c, hq, dt=f32), E(BN, c, hq, d), E(BN, c, hq, dt=f32)
