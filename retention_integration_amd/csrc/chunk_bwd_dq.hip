@@ -104,14 +104,17 @@ __global__ __launch_bounds__(256, 3) void chunk_bwd_dq_kernel(ChunkBwdDqArgs a, 
     const int pos = (ii * 4 + wave) * 64 + l, row = pos / CPR;
     goff[ii] = (uint32_t)(row * (int)kstride + 16 * ((pos % CPR) ^ swz<CPR, SWZ_ROW>(row)));
   }
-  // What the gates have already forgotten (see chunk_fwd.hip): key tiles whose factor exp(R - A_last) has underflowed to
-  // zero for the workgroup's first row contribute exact zeros to every row of the workgroup -- dQ, dGq -- and are
-  // neither copied nor visited; a state part whose factor exp(A_row) has underflowed at the first row has a zero
-  // gradient for every row (the row-wise preparation wrote zeros for its scaled dO and its key-sum factor), so the
-  // sweep is left out.
+  // What the gates have already forgotten (see chunk_fwd.hip): the oldest key tiles whose factor exp(R - A_last) has
+  // underflowed to zero for the largest gate sum among the workgroup's rows contribute exact zeros to every row -- dQ,
+  // dGq -- and are neither copied nor visited; a state part whose factor exp(A_row) has underflowed for that largest sum
+  // has a zero gradient for every row (its scaled dO and its key-sum factor are zeros), so the sweep is left out.
   int it0 = 0;
   if (Gg && a.gate_skip) {
-    const float a_first = Gg[(long)(min(row0, rows - 1) / a.r) * a.h];
+    // (the largest gate sum among the workgroup's rows: the first row's, unless the caller's log gates are positive)
+    float a_first = -INFINITY;
+    for (int i = l; i < ROWS; i += 64) a_first = fmaxf(a_first, Gg[(long)(min(row0 + i, rows - 1) / a.r) * a.h]);
+#pragma unroll
+    for (int m = 32; m > 0; m >>= 1) a_first = fmaxf(a_first, __shfl_xor(a_first, m));
     if (__expf(a_first) == 0.f) has_state = false;
     for (int base = 0; base < ntiles; base += 64) {
       const int tl = min(base + l, ntiles - 1);
@@ -122,7 +125,7 @@ __global__ __launch_bounds__(256, 3) void chunk_bwd_dq_kernel(ChunkBwdDqArgs a, 
       it0 += nd;
       if (nd < lanes) break;
     }
-    it0 = __builtin_amdgcn_readfirstlane(min(it0, ntiles - 1));
+    it0 = __builtin_amdgcn_readfirstlane(min(min(it0, ntiles - 1), min(row0 / a.r + 1, a.c) / CB_BN));
   }
   // Stage ntiles of the ring: the block's rows of Q (the sweep's row values; chunk slots rotated per row as the state
   // kernels read them).  Stage ntiles + 1: the first two stages of the state.

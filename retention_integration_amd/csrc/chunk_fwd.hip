@@ -152,13 +152,18 @@ __global__ __launch_bounds__(256, 3) void chunk_fwd_kernel(ChunkFwdArgs a, int r
 
   // ---- what the gates have already forgotten -------------------------------------------------------------------
   // A key tile entirely in a wave's past enters with the factor exp(R - A_last), R the gate sum at the wave's first row
-  // and A_last the one at the tile's last key.  Gate sums only fall along the chunk, so once that factor has underflowed
-  // to zero for the workgroup's FIRST row it is zero for every row of the workgroup and for every older tile: those
-  // tiles contribute exact zeros and are neither copied nor visited (it0 = the first tile that is).  Likewise the
-  // state part of a row carries exp(A_row): with it underflowed at the first row, the sweep over the state adds exact
-  // zeros to every row of the workgroup and is left out.  (Nothing changes for gates that do not decay that far.)
+  // and A_last the one at the tile's last key.  Once that factor has underflowed to zero for the LARGEST gate sum among
+  // the workgroup's rows (its first row's: gate sums only fall along a chunk, unless the caller's log gates are
+  // positive) it is zero for every wave: the oldest tiles for which it has, as far as they lie before the workgroup's
+  // first row, contribute exact zeros and are neither copied nor visited (it0 = the first tile that is).  Likewise the
+  // state part of a wave's rows carries exp(R): with exp of that largest sum underflowed, the sweep over the state adds
+  // exact zeros to every row of the workgroup and is left out.  (Nothing changes for gates that do not decay that far.)
   if (Gg && a.gate_skip) {
-    const float a_first = Gg[(long)(min(row0, rows - 1) / a.r) * a.h];
+    // (the largest gate sum among the workgroup's rows: the first row's, unless the caller's log gates are positive)
+    float a_first = -INFINITY;
+    for (int i = l; i < ROWS; i += 64) a_first = fmaxf(a_first, Gg[(long)(min(row0 + i, rows - 1) / a.r) * a.h]);
+#pragma unroll
+    for (int m = 32; m > 0; m >>= 1) a_first = fmaxf(a_first, __shfl_xor(a_first, m));
     if (__expf(a_first) == 0.f) no_state = true;
     for (int base = 0; base < ntiles; base += 64) {
       const int tl = min(base + l, ntiles - 1);
@@ -169,7 +174,7 @@ __global__ __launch_bounds__(256, 3) void chunk_fwd_kernel(ChunkFwdArgs a, int r
       it0 += nd;
       if (nd < lanes) break;
     }
-    it0 = __builtin_amdgcn_readfirstlane(min(it0, ntiles - 1));
+    it0 = __builtin_amdgcn_readfirstlane(min(min(it0, ntiles - 1), min(row0 / a.r + 1, a.c) / CF_BN));
   }
   issue(it0);   // older than every copy of the state phase but the rows', so it has landed whenever one of those has
 
