@@ -122,6 +122,7 @@ def counter_run(pra, Q, K, V, lg, cfg, dev, kernel):
         Kc, Vc = K.view(b, n, c, h, d), V.view(b, n, c, h, d)
         S, s = ops.update_state_fwd(Kc, Vc)
         lib = _lib.load()
+        lib.pr_set_gate_skipping(0)   # (every tile visited: the traffic of the whole algorithmic work)
         code = _lib.dtype_code(Kc.dtype)
         src = torch.empty(256 * 1024 * 1024, dtype=torch.uint8, device=dev)
         dst = torch.empty_like(src)
@@ -502,97 +503,142 @@ def main():
     if args.counter_run:
         counter_run(pra, Q.detach(), K.detach(), V.detach(), lg.detach(), cfg, dev, args.counter_run)
         return
-    leaves = [x.requires_grad_(True) for x in (Q, K, V, lg)]
-
-    def step():
-        for x in leaves:
-            x.grad = None
-        Y = pra.power_retention(*leaves, deg=cfg["deg"], chunk_size=cfg["chunk"])
-        Y.backward(dO)
-
-    from retention_integration_amd import _lib
-
-    def timed_steps(k, before=None, lead=0):
-        """k steps, each bracketed by HIP events of its own; `before` is enqueued ahead of every step, outside them.
-        `lead` untimed iterations of the same sequence go first, in the same queue (the host work between two phases
-        idles the GPU long enough for its clock to drop)."""
-        ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(k)]
-        torch.cuda.synchronize()
-        for _ in range(lead):
-            if before is not None:
-                before()
-            step()
-        for e0, e1 in ev:
-            if before is not None:
-                before()
-            e0.record()
-            step()
-            e1.record()
-        torch.cuda.synchronize()
-        return [a.elapsed_time(b_) for a, b_ in ev]
+    from retention_integration_amd import _lib, fused
+    lib = _lib.load()
+    # gates that forget nothing inside a chunk (the distribution of the reference's own inference inputs,
+    # ref: retention/create_inputs.py:39): the same step with nothing for gate skipping to leave out
+    g2 = torch.Generator().manual_seed(43)
+    lg_dense = torch.nn.functional.logsigmoid(6.906768 + torch.randn(cfg["b"], cfg["t"], cfg["h"], generator=g2)).to(dev)
 
     def median(v):
         v = sorted(v)
         return v[len(v) // 2] if len(v) % 2 else 0.5 * (v[len(v) // 2 - 1] + v[len(v) // 2])
 
     flush = torch.empty(512 * 1024 * 1024, dtype=torch.int8, device=dev)   # (allocated before anything is timed)
-    for _ in range(args.warmup):
-        step()
-    # The chip's clock governor drops the clock within a fraction of a millisecond of idling (an allocation, a long
-    # device-side pause) and needs ~25 ms of sustained load to bring it back: straight after a few warm-up steps the
-    # first step takes 2.08 ms and the twelfth 1.80.  The figures of a training loop are the settled ones, so the steps
-    # run untimed for `settle_ms` before anything is timed; the unsettled steps are reported as well (first_steps_ms).
-    first = timed_steps(min(args.steps, 5)) if args.settle_ms > 0 else []
-    settle_steps = int(args.settle_ms / median(first)) + 1 if args.settle_ms > 0 else 0
-    for _ in range(settle_steps):
-        step()
-    # (a) K steps back to back between two synchronisations
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    dt_b2b = (time.perf_counter() - t0) / args.steps
-    # (a') the same steps once more with EVERY kernel timed where it runs: HIP events on the launch stream around each
-    # launch (the library's launch hook).  For these steps the kernels run one after the other: in the steps above,
-    # independent kernels of a step share the GPU on two streams, and a kernel timed while another one runs beside it
-    # says nothing about either.  (So the sum of these times exceeds a headline step.)
-    from retention_integration_amd import fused
-    overlap = (fused.FWD_TWO_STREAMS, fused.BWD_TWO_STREAMS, fused.ATTN_BWD_TWO_STREAMS)
-    fused.FWD_TWO_STREAMS = fused.BWD_TWO_STREAMS = fused.ATTN_BWD_TWO_STREAMS = False
-    try:
+
+    def measure(gates, skipping):
+        """The whole protocol for one choice of gates and of the library's gate skipping switch: -> dict with the median
+        of the flushed steps (ms), the back-to-back figures, the first steps, and every kernel's time inside a step."""
+        lib.pr_set_gate_skipping(1 if skipping else 0)
+        leaves = [x.detach().clone().requires_grad_(True) for x in (Q, K, V, gates)]
+
+        def step():
+            for x in leaves:
+                x.grad = None
+            Y = pra.power_retention(*leaves, deg=cfg["deg"], chunk_size=cfg["chunk"])
+            Y.backward(dO)
+
+        def timed_steps(k, before=None, lead=0):
+            """k steps, each bracketed by HIP events of its own; `before` is enqueued ahead of every step, outside them.
+            `lead` untimed iterations of the same sequence go first, in the same queue (the host work between two
+            phases idles the GPU long enough for its clock to drop)."""
+            ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(k)]
+            torch.cuda.synchronize()
+            for _ in range(lead):
+                if before is not None:
+                    before()
+                step()
+            for e0, e1 in ev:
+                if before is not None:
+                    before()
+                e0.record()
+                step()
+                e1.record()
+            torch.cuda.synchronize()
+            return [a.elapsed_time(b_) for a, b_ in ev]
+
+        for _ in range(args.warmup):
+            step()
+        # The chip's clock governor drops the clock within a fraction of a millisecond of idling (an allocation, a long
+        # device-side pause) and needs ~25 ms of sustained load to bring it back: straight after a few warm-up steps the
+        # first step takes 2.08 ms and the twelfth 1.80.  The figures of a training loop are the settled ones, so the
+        # steps run untimed for `settle_ms` before anything is timed; the unsettled steps are reported as well.
+        first = timed_steps(min(args.steps, 5)) if args.settle_ms > 0 else []
+        settle_steps = int(args.settle_ms / median(first)) + 1 if args.settle_ms > 0 else 0
+        for _ in range(settle_steps):
+            step()
+        # (a) K steps back to back between two synchronisations
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         for _ in range(args.steps):
             step()
         torch.cuda.synchronize()
-        dt_seq = (time.perf_counter() - t0) / args.steps
-        with KernelTimers(_lib) as kt:
-            for _ in range(args.steps + 2):
+        dt_b2b = (time.perf_counter() - t0) / args.steps
+        # (a') the same steps once more with EVERY kernel timed where it runs: HIP events on the launch stream around
+        # each launch (the library's launch hook).  For these steps the kernels run one after the other: in the steps
+        # above, independent kernels of a step share the GPU on two streams, and a kernel timed while another one runs
+        # beside it says nothing about either.  (So the sum of these times exceeds a headline step.)
+        overlap = (fused.FWD_TWO_STREAMS, fused.BWD_TWO_STREAMS, fused.ATTN_BWD_TWO_STREAMS)
+        fused.FWD_TWO_STREAMS = fused.BWD_TWO_STREAMS = fused.ATTN_BWD_TWO_STREAMS = False
+        try:
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(args.steps):
                 step()
-                kt.end_step()
-            in_step_ms = kt.per_step(skip=2)
-    finally:
-        fused.FWD_TWO_STREAMS, fused.BWD_TWO_STREAMS, fused.ATTN_BWD_TWO_STREAMS = overlap
-    # (b) the headline, by the reference's protocol (ref: perf/_timing.py:77-110): before every step the caches are
-    # flushed (a fill of 512 MB: L2 and the 256 MB memory-side cache), then a short device-side pause lets the host run
-    # ahead (launch latency is not measured), the step is bracketed by HIP events of its own, and the MEDIAN over the K
-    # steps is reported.  (The reference pauses for 25 ms; here that alone would cost 10 %, see above: 0.1 ms.)
-    times = timed_steps(args.steps, lambda: (flush.zero_(), torch.cuda._sleep(200_000)), lead=settle_steps // 2)
+            torch.cuda.synchronize()
+            dt_seq = (time.perf_counter() - t0) / args.steps
+            with KernelTimers(_lib) as kt:
+                for _ in range(args.steps + 2):
+                    step()
+                    kt.end_step()
+                in_step = kt.per_step(skip=2)
+        finally:
+            fused.FWD_TWO_STREAMS, fused.BWD_TWO_STREAMS, fused.ATTN_BWD_TWO_STREAMS = overlap
+        # (b) the headline, by the reference's protocol (ref: perf/_timing.py:77-110): before every step the caches are
+        # flushed (a fill of 512 MB: L2 and the 256 MB memory-side cache), then a short device-side pause lets the host
+        # run ahead (launch latency is not measured), the step is bracketed by HIP events of its own, and the MEDIAN over
+        # the K steps is reported.  (The reference pauses for 25 ms; here that alone would cost 10 %, see above: 0.1 ms.)
+        times = timed_steps(args.steps, lambda: (flush.zero_(), torch.cuda._sleep(200_000)), lead=settle_steps // 2)
+        lib.pr_set_gate_skipping(1)
+        return {"dt": median(times) * 1e-3, "times": times, "b2b": dt_b2b, "seq": dt_seq, "first": first,
+                "settle_steps": settle_steps, "in_step_ms": in_step}
+
+    # The headline: the gates the benchmark contract names, the library as it ships (gate skipping on).  Beside it the
+    # same step with skipping switched off -- every tile visited whatever the gates: the figures that say how good the
+    # kernels are (rooflines, matrix-core share) come from THAT run -- and with gates that forget nothing.
+    head = measure(lg, True)
+    every = measure(lg, False)
+    dense = measure(lg_dense, True)
     del flush
-    dt = median(times) * 1e-3
+    dt, times, dt_b2b, dt_seq, first, settle_steps = (head[k] for k in ("dt", "times", "b2b", "seq", "first", "settle_steps"))
+    in_step_ms = every["in_step_ms"]
 
     D_compact = cfg["d"] * (cfg["d"] + 1) // 2
     f_fwd, f_bwd = flops(cfg["b"], cfg["t"], cfg["h"], cfg["d"], cfg["chunk"], D_compact)
-    tflops = (f_fwd + f_bwd) / dt / 1e12
+    canon = f_fwd + f_bwd
+    tflops = canon / every["dt"] / 1e12   # (every product of the canonical count executed: skipping off)
+
+    def summary(m):
+        return {"ms_per_step": round(m["dt"] * 1e3, 4), "tokens_per_s": round(cfg["b"] * cfg["t"] / m["dt"], 1),
+                "flushed_ms": {"median": round(m["dt"] * 1e3, 4), "min": round(min(m["times"]), 4),
+                               "max": round(max(m["times"]), 4)},
+                "back_to_back_ms_per_step": round(m["b2b"] * 1e3, 4),
+                "back_to_back_one_stream_ms_per_step": round(m["seq"] * 1e3, 4),
+                "kernels_us": {k: round(v * 1e3, 1) for k, v in m["in_step_ms"].items()},
+                "kernels_us_sum": round(sum(m["in_step_ms"].values()) * 1e3, 1)}
     out = {
         "metric": "fwd+bwd tokens/s at t=65536,h=8,d=64,deg=2,chunk=1024 (gated, bf16)",
         "value": round(cfg["b"] * cfg["t"] / dt, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(dt * 1e3, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": "power_retention fwd+bwd b=1 t=65536 h=8 d=64 deg=2 chunk_size=1024 gating=True "
-                               "(BASELINE configs[1]+[2])", "D_state": expanded_dim(cfg["d"])},
+        "config": {"workload": "power_retention fwd+bwd b=1 t=65536 h=8 d=64 deg=2 chunk_size=1024 gating=True, "
+                               "log_G = logsigmoid(N(0,1)) (BASELINE configs[1]+[2])", "D_state": expanded_dim(cfg["d"])},
+        # value: the library as it ships -- gate skipping on -- on the gates the benchmark contract names.  Those gates
+        # fall by 0.8 per step, so inside a chunk of 1024 most weights are exact zeros in fp32 and the kernels leave them
+        # out (outputs and gradients identical bit for bit: tests/test_gpu_gate_skipping.py).  What a step costs when
+        # nothing can be left out is reported beside it, and every kernel-quality figure (tflops, pct_bf16_mfma_peak,
+        # the roofline blocks, kernels_us) is from the run with skipping OFF, in which every product is executed.
+        "gate_skipping": {
+            "value_measured_with": "on (library default)",
+            "identical_results": "bit for bit, skipping on vs off: tests/test_gpu_gate_skipping.py",
+            "on": summary(head),
+            "off_every_tile_visited": summary(every),
+            "gates_that_forget_nothing": dict(summary(dense), gates="log_G = logsigmoid(6.906768 + N(0,1)), skipping on"),
+            "canonical_tflops_at_value": round(canon / dt / 1e12, 2),
+            "note": "canonical_tflops_at_value counts products the kernels did not execute: a rate of useful work, not a "
+                    "matrix-core utilisation"},
         "tflops": round(tflops, 2), "pct_bf16_mfma_peak": round(100 * tflops / PEAK_BF16_TFLOPS, 2),
+        "tflops_measured_with": "gate skipping off (every product of the canonical count executed)",
         "timing": {"protocol": "W warm-up steps, then untimed steps for settle_ms (the clock governor's ramp); value = "
                                "median over K steps, each after a 512 MB cache flush and a short device-side pause, HIP "
                                "events per step (ref: perf/_timing.py:77-110); back_to_back = wall clock of K "
@@ -606,12 +652,14 @@ def main():
     }
     n = cfg["t"] // cfg["chunk"]
     bh = cfg["b"] * cfg["h"]
-    # Roofline blocks.  `roofline` is the LONGEST single kernel of the step as just measured; its work per launch is the
-    # algorithmic count of kernel_work().  HBM traffic of a launch comes from the tracked rocprofv3 counter summary of
+    # Roofline blocks, from the run with gate skipping off (in_step_ms = its kernel times): every product of the
+    # algorithmic count is executed there.  `roofline` is the LONGEST single kernel of that step; its work per launch is
+    # the algorithmic count of kernel_work().  HBM traffic of a launch comes from the tracked rocprofv3 counter summary of
     # that kernel when profiles/ holds one (parsed at run time, never typed in here).
     work = kernel_work(cfg, expanded_dim(cfg["d"]))
     out["kernels_us"] = {k: round(v * 1e3, 1) for k, v in in_step_ms.items()}
     out["kernels_us_sum"] = round(sum(in_step_ms.values()) * 1e3, 1)
+    out["kernels_us_measured_with"] = "gate skipping off; gate_skipping.on.kernels_us has the kernels of the headline step"
     longest = max(in_step_ms, key=in_step_ms.get)
     base = longest.split("#")[0]
     blk = roofline_block(longest, in_step_ms[longest], work.get(base, ("hbm", 0.0)))
@@ -640,6 +688,7 @@ def main():
     mf = sum(v for k, v in in_step_ms.items() if work.get(k.split("#")[0], ("hbm",))[0] == "mfma")
     out["kernel_time_split_us"] = {"mfma_bound": round(mf * 1e3, 1), "hbm_bound": round((sum(in_step_ms.values()) - mf) * 1e3, 1)}
     detach = [x.detach() for x in (Q, K, V, lg)]
+    lib.pr_set_gate_skipping(0)   # the legs below time operators and chained calls as such: every tile visited
     if not args.no_breakdown:
         with torch.no_grad():
             bd = op_breakdown(pra, *detach, dO, cfg)
@@ -670,7 +719,8 @@ def main():
             out["state_across_calls"] = {"forward_one_call_ms": round(t1, 4), "forward_two_calls_ms": round(t2, 4),
                                          "ratio": round(t2 / t1, 4),
                                          "workload": "forward only, the headline sequence whole vs as two halves chained "
-                                                     "through (state, sum_of_keys)"}
+                                                     "through (state, sum_of_keys); gate skipping off"}
+    lib.pr_set_gate_skipping(1)
     if not args.no_short_chunks:
         torch.cuda.empty_cache()
         sc = short_chunks(pra, dev, 5, 2)
