@@ -290,7 +290,10 @@ int pr_gate_cumsum(const float* log_G, float* A, int B, int t, int h, void* stre
  *   live_rows (NULL or [BN,h,2] int32, written with the sums): per (chunk, kv head), [0] the first time step whose
  *   factor exp((A[c-1] - A)/deg) has not underflowed to zero -- the rows of Kd before it are exact zeros -- and [1] one
  *   past the last time step with exp(A) != 0 -- from there on the state part of a query row is an exact zero.  Hand it
- *   to pr_update_state_fwd and pr_query_state_bwd, which then leave those rows out (see pr_set_gate_skipping). */
+ *   to pr_update_state_fwd / _bwd and pr_query_state_bwd, which then leave those rows out (see pr_set_gate_skipping).
+ *   In a call with log_G == NULL (products only) live_rows is an INPUT and a promise: every reader of Kd is handed the
+ *   same array; the rows of Kd before the block of 256 steps that holds live_rows[bn,h,0] -- exact zeros -- are then
+ *   left unwritten. */
 int pr_chunk_prep_fwd(const float* log_G, const void* K, const void* Q, float* A, float* lcs, void* Kd, void* Qg,
                       int* live_rows, int BN, int c, int h, int r, int d, int deg, int dtype, void* stream);
 

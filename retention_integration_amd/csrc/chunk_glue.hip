@@ -89,7 +89,8 @@ template <typename T, int DH>
 __global__ __launch_bounds__(256) void gate_apply_fwd_kernel(const float* __restrict__ A, const float* __restrict__ lcs,
                                                              const T* __restrict__ K, const T* __restrict__ Q,
                                                              T* __restrict__ Kd, T* __restrict__ Qg, long groups,
-                                                             int c, int h, int r, float inv_deg) {
+                                                             int c, int h, int r, float inv_deg,
+                                                             const int* __restrict__ live) {
   typedef typename VecOf<T>::v8 v8;
   constexpr int LPR = DH / 8;
   const long gid = ((long)blockIdx.x * 256 + threadIdx.x) / LPR;
@@ -100,10 +101,15 @@ __global__ __launch_bounds__(256) void gate_apply_fwd_kernel(const float* __rest
   const float at = A[gid], al = lcs[bn * h + hh];
   const float w = __expf((al - at) * inv_deg), u = __expf(at * inv_deg);
   float f[8];
-  unpack8(*(const v8*)(K + gid * DH + col), f);
+  // (live: the readers of Kd leave out the time steps before live[bn, hh, 0], whose factor w is zero, in whole row
+  // blocks of theirs -- 64, 128 or 256 rows: the rows before the block of 256 that holds the first live one are neither
+  // read nor written here)
+  if (!live || (int)((gid / h) % c) >= (live[(bn * h + hh) * 2] & ~255)) {
+    unpack8(*(const v8*)(K + gid * DH + col), f);
 #pragma unroll
-  for (int i = 0; i < 8; i++) f[i] *= w;
-  *(v8*)(Kd + gid * DH + col) = pack8<T>(f);
+    for (int i = 0; i < 8; i++) f[i] *= w;
+    *(v8*)(Kd + gid * DH + col) = pack8<T>(f);
+  }
   for (int rr = 0; Qg && rr < r; rr++) {
     const long o = (gid * r + rr) * DH + col;
     unpack8(*(const v8*)(Q + o), f);
@@ -156,7 +162,8 @@ static int prep_launch(const float* logG, const void* K, const void* Q, float* A
 #define PR_CP(DD)                                                                                                      \
   case DD:                                                                                                             \
     PR_LAUNCH("gate_apply_fwd", (gate_apply_fwd_kernel<T, DD>), dim3((unsigned)((groups * (DD / 8) + 255) / 256)), dim3(256), 0, \
-                       st, A, lcs, (const T*)K, (const T*)Q, (T*)Kd, (T*)Qg, groups, c, h, r, 1.f / deg);              \
+                       st, A, lcs, (const T*)K, (const T*)Q, (T*)Kd, (T*)Qg, groups, c, h, r, 1.f / deg,               \
+                       (!logG && g_gate_skip) ? live : nullptr);                                                      \
     break;
   switch (d) { PR_CP(32) PR_CP(64) PR_CP(128) default: return -2; }
 #undef PR_CP

@@ -215,7 +215,10 @@ int gate_cumsum(const float* logG, float* A, int B, int t, int h, hipStream_t st
 // (Qg may be null: the gated queries are then not formed)
 // live [BN, h, 2] or null: receives, per (chunk, kv head), the first time step whose discounted key is not zeroed by
 // its factor exp((A_last - A_t) / deg), and one past the last time step whose factor exp(A_t) on the state part of a
-// query is not zero (written with the sums, i.e. when logG is given)
+// query is not zero (written with the sums, i.e. when logG is given).  Given WITHOUT logG it is an input: the caller's
+// promise that every reader of Kd leaves out the time steps before live[bn, hh, 0] (as sympow_tn, sympow_nn and
+// sympow_grad do when handed the same array); those rows of Kd, exact zeros, are then not written
+// (up to the block of 256 rows that holds the first live one).
 int chunk_prep_fwd(const float* logG, const void* K, const void* Q, float* A, float* lcs, void* Kd, void* Qg, int* live,
                    int BN, int c, int h, int r, int d, int deg, int dtype, hipStream_t st);
 int chunk_gate_scan_bwd(float* dA, const float* dGq, const float* dotk, const float* dlcs_a, const float* dlcs_b, int BN,

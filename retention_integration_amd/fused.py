@@ -131,8 +131,9 @@ def chunked_fwd(Q: Tensor, K: Tensor, V: Tensor, log_G: Optional[Tensor], deg: i
         attention(side.cuda_stream)
 
     if gated:
-        _lib.check(lib.pr_chunk_prep_fwd(None, p(K), p(Q), p(A), p(lcs), p(Kd), None, None, BN, c, h, r, d, deg, code,
-                                         st), "chunk_prep_fwd(keys)")
+        # (every reader of Kd below and in the backward is handed `live`: its dead rows need not be written)
+        _lib.check(lib.pr_chunk_prep_fwd(None, p(K), p(Q), p(A), p(lcs), p(Kd), None, None if chained else p(live), BN, c,
+                                         h, r, d, deg, code, st), "chunk_prep_fwd(keys)")
     Sc, sc = _empty((BN, h, D, d), dt, dev), _empty((BN, h, D), f32, dev)
     Sf, sf = _empty((0,), dt, dev), _empty((0,), f32, dev)
     S, s = _empty((0,), dt, dev), _empty((0,), f32, dev)
