@@ -473,6 +473,10 @@ def main():
     ap.add_argument("--no-decode", action="store_true", help="skip the inference (prefill + decode) leg")
     ap.add_argument("--no-short-chunks", action="store_true", help="skip the BASELINE configs[4] leg (short_chunks key)")
     ap.add_argument("--no-chained-calls", action="store_true", help="skip the state_across_calls leg")
+    ap.add_argument("--gate-runs", default="on,off,dense",
+                    help="which of the three measurements of the headline step to make: on (gate skipping on: the value), "
+                         "off (every tile visited: the kernel-quality figures), dense (gates that forget nothing); a "
+                         "profiler run picks one so that its trace holds one kind of step")
     ap.add_argument("--counter-run", nargs="?", const="sympow_grad", default=None, metavar="KERNEL",
                     help="for rocprofv3 --pmc: launch only one kernel a few times -- sympow_grad (dK of update_state "
                          "backward, the default), chunk_fwd or chunk_bwd_dq -- and a plain device copy of 256 MiB for calibrating "
@@ -596,9 +600,13 @@ def main():
     # The headline: the gates the benchmark contract names, the library as it ships (gate skipping on).  Beside it the
     # same step with skipping switched off -- every tile visited whatever the gates: the figures that say how good the
     # kernels are (rooflines, matrix-core share) come from THAT run -- and with gates that forget nothing.
-    head = measure(lg, True)
-    every = measure(lg, False)
-    dense = measure(lg_dense, True)
+    runs = [r for r in args.gate_runs.split(",") if r]
+    assert runs and all(r in ("on", "off", "dense") for r in runs), "--gate-runs takes on, off, dense"
+    head = measure(lg, True) if "on" in runs else None
+    every = measure(lg, False) if "off" in runs else None
+    dense = measure(lg_dense, True) if "dense" in runs else None
+    head = head or every or dense      # (a run that leaves measurements out reports what it has in their place)
+    every = every or head
     del flush
     dt, times, dt_b2b, dt_seq, first, settle_steps = (head[k] for k in ("dt", "times", "b2b", "seq", "first", "settle_steps"))
     in_step_ms = every["in_step_ms"]
@@ -633,7 +641,9 @@ def main():
             "identical_results": "bit for bit, skipping on vs off: tests/test_gpu_gate_skipping.py",
             "on": summary(head),
             "off_every_tile_visited": summary(every),
-            "gates_that_forget_nothing": dict(summary(dense), gates="log_G = logsigmoid(6.906768 + N(0,1)), skipping on"),
+            "gates_that_forget_nothing": dict(summary(dense or every),
+                                              gates="log_G = logsigmoid(6.906768 + N(0,1)), skipping on"),
+            "measured": runs,
             "canonical_tflops_at_value": round(canon / dt / 1e12, 2),
             "note": "canonical_tflops_at_value counts products the kernels did not execute: a rate of useful work, not a "
                     "matrix-core utilisation"},
