@@ -17,13 +17,13 @@ from .cache import RetentionCache
 from .fused import chunked_power_retention
 from .inference import make_fused_inference
 from .maker import make_power_retention, make_power_retention_inference
-from .ops import attention, discumsum, expanded_dim, query_state, update_state
+from .ops import attention, discumsum, expanded_dim, gate_cumsum_or_none, query_state, update_state
 
 power_retention_composed = make_power_retention(update_state, query_state, partial(discumsum, keep_last=False),
                                                 attention, scan_keeps_last=False, full_scan_impl=discumsum)
 power_retention = make_power_retention(update_state, query_state, partial(discumsum, keep_last=False), attention,
                                        scan_keeps_last=False, chunked_impl=chunked_power_retention,
-                                       full_scan_impl=discumsum)
+                                       full_scan_impl=discumsum, gate_cumsum_impl=gate_cumsum_or_none)
 power_retention_inference_composed = make_power_retention_inference(update_state, query_state, attention,
                                                                     fused_normalizer=False)
 power_retention_inference = make_fused_inference(power_retention_inference_composed)

@@ -50,7 +50,7 @@ template <typename T> __device__ __forceinline__ typename VecOf<T>::v8 ab_tr8(ui
 
 // ------------------------------------------------------------------ dQ, dGq
 template <typename T, int DH, int MT, bool DEG2, int OCC>
-__global__ __launch_bounds__(256, OCC) void attention_bwd_dq_kernel(AttnBwdArgs a, int nblocks, int npairs) {
+__global__ __launch_bounds__(256, OCC) void attention_bwd_dq_kernel(AttnBwdArgs a, int nblocks, int npairs, int gate_skip) {
   typedef typename VecOf<T>::v8 v8;
   typedef typename VecOf<T>::v4 v4;
   typedef __attribute__((address_space(3))) v8 lds_v8;
@@ -135,8 +135,30 @@ __global__ __launch_bounds__(256, OCC) void attention_bwd_dq_kernel(AttnBwdArgs 
     }
     if (Gg && wave == 0) async_copy4(Gg + (long)min(j0 + l, a.tk - 1) * a.h, st + 2 * TILE);
   };
-  issue(0);
-  if (NST == 3 && ntot > 1) issue(1);
+  // What the gates have already forgotten (as in attention_fwd.hip): the oldest key tiles whose factor exp(R - A_last)
+  // has underflowed to zero for the largest gate sum among the workgroup's rows, as far as they lie before its first row,
+  // contribute exact zeros to dQ and dGq and are neither copied nor visited; a wave also returns from a past tile whose
+  // factor is zero for its own rows.
+  int it0 = 0;
+  if (Gg && gate_skip) {
+    float a_max = -INFINITY;
+    for (int i = l; i < ROWS; i += 64) a_max = fmaxf(a_max, Gg[(long)(min(row0 + i, rows - 1) / a.r + shift) * a.h]);
+    const float a_last0 = Gg[(long)min(AB_BN * min(l, ntiles - 1) + AB_BN - 1, a.tk - 1) * a.h];
+#pragma unroll
+    for (int m = 32; m > 0; m >>= 1) a_max = fmaxf(a_max, __shfl_xor(a_max, m));
+    for (int base_t = 0; base_t < ntiles; base_t += 64) {
+      const int tl = min(base_t + l, ntiles - 1);
+      const float a_last = base_t == 0 ? a_last0 : Gg[(long)min(AB_BN * tl + AB_BN - 1, a.tk - 1) * a.h];
+      const unsigned long long dead = __ballot(__expf(fminf(a_max - a_last, AB_EXP_CLAMP)) == 0.f);
+      const int lanes = min(64, ntiles - base_t);
+      const int nd = __builtin_popcountll(lanes == 64 ? dead : (dead & ((1ull << lanes) - 1)));
+      it0 += nd;
+      if (nd < lanes) break;
+    }
+    it0 = __builtin_amdgcn_readfirstlane(min(min(it0, ntiles - 1), min(row0 / a.r + shift + 1, a.tk) / AB_BN));
+  }
+  issue(it0);
+  if (NST == 3 && ntot > it0 + 1) issue(it0 + 1);
 
   v8 Qf[MT][KS], dOf[MT][KS];
   int ti[MT];
@@ -203,7 +225,7 @@ __global__ __launch_bounds__(256, OCC) void attention_bwd_dq_kernel(AttnBwdArgs 
   };
   if (wave == 0) {
     wait_vmcnt<0>();
-    gate_factors(0);
+    gate_factors(it0);
   }
   auto sync_step = [&](int it) __attribute__((always_inline)) -> char* {
     char* st = smem + (it % NST) * STAGE;
@@ -257,6 +279,8 @@ __global__ __launch_bounds__(256, OCC) void attention_bwd_dq_kernel(AttnBwdArgs 
 #pragma unroll
     for (int mi = 0; mi < MT; mi++) lim[mi] = DIAG ? min(ti[mi], a.tk - 1) - j0 - 4 * g : 0;
     const float cw = DIAG ? 1.f : __expf(fminf(Rw - graw[AB_BN - 1], AB_EXP_CLAMP));
+    // (forgotten by this wave's rows, though not by the workgroup's first: every term of the tile is an exact zero)
+    if (!DIAG && gate_skip && __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, cw)) == 0) return;
 #pragma unroll
     for (int kp = 0; kp < KT / 2; kp++) {
       if (DIAG && j0 + 32 * kp > w_last_ti) continue;   // these 32 keys come after every row of the wave
@@ -322,7 +346,7 @@ __global__ __launch_bounds__(256, OCC) void attention_bwd_dq_kernel(AttnBwdArgs 
     }
   };
 
-  int it = 0;
+  int it = it0;
   for (; it < n_past; it++) {
     tile(it, sync_step(it), IC<0>{});
     after_step(it);
@@ -928,7 +952,7 @@ template <typename T, int DH, bool DEG2> static int attn_bwd_launch(const AttnBw
     constexpr int OCC = (DH <= 32 || (DH == 64 && DEG2)) ? 3 : 2;
     auto kern = attention_bwd_dq_kernel<T, DH, MT, DEG2, OCC>;
     allow_big_lds((const void*)kern, smem);
-    PR_LAUNCH("attention_bwd_dq", kern, grid, dim3(256), smem, st, a, nblocks, npairs);
+    PR_LAUNCH("attention_bwd_dq", kern, grid, dim3(256), smem, st, a, nblocks, npairs, g_gate_skip);
   }
   return (int)hipGetLastError();
 }

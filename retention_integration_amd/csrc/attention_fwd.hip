@@ -43,7 +43,7 @@ template <bool DEG2> __device__ __forceinline__ float pow_even(float sv, float e
 }
 
 template <typename T, int DH, int MT, bool DEG2, int OCC>
-__global__ __launch_bounds__(256, OCC) void attention_fwd_kernel(AttnFwdArgs a, int row_blocks, int npairs) {
+__global__ __launch_bounds__(256, OCC) void attention_fwd_kernel(AttnFwdArgs a, int row_blocks, int npairs, int gate_skip) {
   typedef typename VecOf<T>::v8 v8;
   typedef typename VecOf<T>::v4 v4;
   typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
@@ -118,8 +118,32 @@ __global__ __launch_bounds__(256, OCC) void attention_fwd_kernel(AttnFwdArgs a, 
     }
     if (Gg && wave == 0) async_copy4(Gg + (long)min(j0 + l, a.tk - 1) * a.h, st + 2 * TILE);
   };
-  issue(0);
-  if (NST == 3 && ntiles > 1) issue(1);
+  // What the gates have already forgotten.  A key tile entirely in a wave's past enters with the wave-uniform factor
+  // exp(R - A_last) (R: gate sum at the wave's first row, A_last: at the tile's last key; see the tile code).  Once that
+  // factor has underflowed to zero for the LARGEST gate sum among the workgroup's rows (its first row's: gate sums only
+  // fall along a sequence, unless the caller's log gates are positive) it is zero for every wave: the oldest tiles for
+  // which it has, as far as they lie before the workgroup's first row, contribute exact zeros and are neither copied nor
+  // visited (it0 = the first tile that is); a wave also returns from a past tile whose factor is zero for its own rows.
+  int it0 = 0;
+  if (Gg && gate_skip) {
+    float a_max = -INFINITY;
+    for (int i = l; i < ROWS; i += 64) a_max = fmaxf(a_max, Gg[(long)(min(row0 + i, rows - 1) / a.r + shift) * a.h]);
+    const float a_last0 = Gg[(long)min(AT_BN * min(l, ntiles - 1) + AT_BN - 1, a.tk - 1) * a.h];
+#pragma unroll
+    for (int m = 32; m > 0; m >>= 1) a_max = fmaxf(a_max, __shfl_xor(a_max, m));
+    for (int base = 0; base < ntiles; base += 64) {
+      const int tl = min(base + l, ntiles - 1);
+      const float a_last = base == 0 ? a_last0 : Gg[(long)min(AT_BN * tl + AT_BN - 1, a.tk - 1) * a.h];
+      const unsigned long long dead = __ballot(__expf(fminf(a_max - a_last, AT_EXP_CLAMP)) == 0.f);
+      const int lanes = min(64, ntiles - base);
+      const int nd = __builtin_popcountll(lanes == 64 ? dead : (dead & ((1ull << lanes) - 1)));
+      it0 += nd;
+      if (nd < lanes) break;
+    }
+    it0 = __builtin_amdgcn_readfirstlane(min(min(it0, ntiles - 1), min(row0 / a.r + shift + 1, a.tk) / AT_BN));
+  }
+  issue(it0);
+  if (NST == 3 && ntiles > it0 + 1) issue(it0 + 1);
 
   v8 Qf[MT][KS];
   int ti[MT];
@@ -191,7 +215,7 @@ __global__ __launch_bounds__(256, OCC) void attention_fwd_kernel(AttnFwdArgs a, 
   };
   if (wave == 0) {
     wait_vmcnt<0>();
-    gate_factors(0);
+    gate_factors(it0);
   }
   // Make tile `it` visible to the workgroup, start the copy of tile it+2, and (wave 0) prepare the gate factors of
   // tile it+1 while the others already compute.
@@ -255,6 +279,8 @@ __global__ __launch_bounds__(256, OCC) void attention_fwd_kernel(AttnFwdArgs a, 
     }
     // past tiles: key factors relative to the gate at the wave's first row (<= 1 for every past key)
     const float cw = DIAG ? 1.f : __expf(fminf(Rw - graw[AT_BN - 1], AT_EXP_CLAMP));
+    // (forgotten by this wave's rows, though not by the workgroup's first: every weight of the tile is an exact zero)
+    if (!DIAG && gate_skip && __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, cw)) == 0) return;
 #pragma unroll
     for (int kp = 0; kp < KT / 2; kp++) {
       if (DIAG && j0 + 32 * kp > w_last_ti) continue;   // these 32 keys come after every row of the wave
@@ -329,7 +355,7 @@ __global__ __launch_bounds__(256, OCC) void attention_fwd_kernel(AttnFwdArgs a, 
 
   auto run_pass = [&](auto mode_c) __attribute__((always_inline)) {
     constexpr int MODE = decltype(mode_c)::value;
-    int it = 0;
+    int it = it0;
     for (; it < n_past; it++) {
       tile(it, sync_step(it), IC<0>{}, mode_c);
       after_step(it);
@@ -365,11 +391,11 @@ __global__ __launch_bounds__(256, OCC) void attention_fwd_kernel(AttnFwdArgs a, 
       prow[mi] = scale_p * __expf(fminf(Gq[mi] - Rw, AT_EXP_CLAMP)) * pn[mi];
     }
     lds_barrier();   // every wave is done with the ring: start the copies over
-    issue(0);
-    if (NST == 3 && ntiles > 1) issue(1);
+    issue(it0);
+    if (NST == 3 && ntiles > it0 + 1) issue(it0 + 1);
     if (wave == 0) {
       wait_vmcnt<0>();
-      gate_factors(0);
+      gate_factors(it0);
     }
     run_pass(IC<2>{});
   } else {
@@ -409,7 +435,7 @@ template <typename T, int DH, bool DEG2> static int attn_fwd_launch(const AttnFw
     dim3 grid((unsigned)(((npairs + 31) / 32) * 32 * row_blocks));
     auto kern = attention_fwd_kernel<T, DH, MT, DEG2, OCC>;
     allow_big_lds((const void*)kern, smem);
-    PR_LAUNCH("attention_fwd", kern, grid, dim3(256), smem, st, a, row_blocks, npairs);
+    PR_LAUNCH("attention_fwd", kern, grid, dim3(256), smem, st, a, row_blocks, npairs, g_gate_skip);
   };
   // 128 rows per workgroup: 123 registers at d = 32 (four workgroups per CU), 166 at d = 64 (three); measured 9 % and
   // 6 % faster than 256 rows at two workgroups -- the kernel is mostly vector work, which issues faster with more

@@ -17,7 +17,7 @@ def _pad_time(x, pad, dims_after):
 
 
 def make_power_retention(update_state_impl, query_state_impl, discumsum_impl, attention_impl, *,
-                         scan_keeps_last=True, chunked_impl=None, full_scan_impl=None):
+                         scan_keeps_last=True, chunked_impl=None, full_scan_impl=None, gate_cumsum_impl=None):
     """Build ``power_retention`` from operator implementations.
 
     ``scan_keeps_last=False`` declares that ``discumsum_impl(X, log_G)`` already returns only the first n
@@ -25,6 +25,8 @@ def make_power_retention(update_state_impl, query_state_impl, discumsum_impl, at
     scale, chunk_size)``, when given, replaces the composition of the four operators on the chunked branch
     (same result; used for the fused single-node path).  ``full_scan_impl(X, log_G)`` must return all n + 1
     entries; it is needed for ``return_final_state`` when ``discumsum_impl`` drops the last one.
+    ``gate_cumsum_impl(log_G)``, when given, stands in for ``log_G.cumsum(1)`` on the quadratic branch (fp32
+    ``[b, t, h]``; it may return None for shapes it does not take).
 
     State across calls.  ``initial_state`` is a pair ``(state [b,h,D,d], sum_of_keys [b,h,D])`` -- what
     ``power_retention_inference`` takes and returns -- and ``return_final_state=True`` returns
@@ -86,7 +88,11 @@ def make_power_retention(update_state_impl, query_state_impl, discumsum_impl, at
             assert S0.dtype == dtype, f"initial_state dtype {S0.dtype} must match the inputs' {dtype}"
 
         if (switch_over_seq_len is None or t <= switch_over_seq_len) and not with_state:   # quadratic form (:128-140)
-            A = log_G.cumsum(1) if gated else None
+            A = None
+            if gated:   # (ref: retention/power_retention_maker.py:129)
+                A = gate_cumsum_impl(log_G) if gate_cumsum_impl is not None else None
+                if A is None:
+                    A = log_G.cumsum(1)
             return attention_impl(Q, K, V, A, deg, scale=scale, norm=True)
 
         # Everything below goes through the state, which exists for degree 2 only: refuse here, before anything is

@@ -56,6 +56,14 @@ def test_opcheck_operators(pra):
     Sc = ops.discumsum_fwd(S, lcs.detach(), n).requires_grad_(True)
     sc = ops.discumsum_fwd(s, lcs.detach(), n).requires_grad_(True)
     torch.library.opcheck(ops.query_state_fwd, (Q5, Sc, sc, Ya5, la5, rm5, 0.0625, True), test_utils=OPCHECKS)
+    # the accumulated gates of the quadratic branch (ref: log_G.cumsum(1), retention/power_retention_maker.py:129)
+    lg3 = lg.detach().clone().requires_grad_(True)
+    torch.library.opcheck(ops.gate_cumsum, (lg3,), test_utils=OPCHECKS)
+    dA = torch.randn_like(lg3)
+    (g_lib,) = torch.autograd.grad(ops.gate_cumsum(lg3), lg3, dA)
+    (g_ref,) = torch.autograd.grad(lg3.cumsum(1), lg3, dA)
+    assert torch.allclose(ops.gate_cumsum(lg3), lg3.cumsum(1), rtol=1e-5, atol=1e-5)
+    assert torch.allclose(g_lib, g_ref, rtol=1e-5, atol=1e-5)
 
 
 @pytest.mark.parametrize("chunk", [64, None])
