@@ -75,6 +75,37 @@ def test_headline_shape_fwd_bwd_matches_the_oracle_per_chunk(pra):
     print("  worst per-(chunk, head) rel-L2:", {k: f"{v:.3e}" for k, v in worst.items()}, flush=True)
 
 
+def test_headline_shape_is_the_same_bit_for_bit_with_and_without_gate_skipping(pra):
+    """The same step as above (which runs with the library's default, gate skipping on) once more with skipping off:
+    every tile visited, every state swept, every chunk scanned.  All five tensors must agree bit for bit -- what is
+    left out are products with exact zeros -- with all 512 (chunk, head) pairs in every launch."""
+    from retention_integration_amd import _lib
+    lib = _lib.load()
+    b, t, h, d, c = 1, 65536, 8, 64, 1024
+    g = torch.Generator().manual_seed(2024)
+    Q, K, V = (torch.randn(b, t, h, d, generator=g).to(torch.bfloat16).to(DEV) for _ in range(3))
+    lg = torch.nn.functional.logsigmoid(torch.randn(b, t, h, generator=g)).to(DEV)
+    dO = torch.randn(b, t, h, d, generator=g).to(torch.bfloat16).to(DEV)
+
+    def step():
+        xs = [x.detach().clone().requires_grad_(True) for x in (Q, K, V, lg)]
+        Y = pra.power_retention(*xs, deg=2, chunk_size=c)
+        Y.backward(dO)
+        torch.cuda.synchronize()
+        return [Y.detach()] + [x.grad for x in xs]
+    try:
+        lib.pr_set_gate_skipping(1)
+        on = step()
+        lib.pr_set_gate_skipping(0)
+        off = step()
+    finally:
+        lib.pr_set_gate_skipping(1)
+    for nm, x, y in zip(["Y", "dQ", "dK", "dV", "dlog_G"], on, off):
+        assert torch.isfinite(x.float()).all(), nm
+        assert torch.equal(x, y), f"{nm}: {int((x != y).sum())} values differ, by up to " \
+                                  f"{float((x.float() - y.float()).abs().max()):.3e}"
+
+
 def test_inference_config_at_size_prefill_then_512_recurrent_steps(pra):
     """bf16, b=32, h=8, d=64: prefill with 2048 keys and switch_over_seq_len=1024 (state [32,8,2560,64], key sums
     [32,8,2560]), then 512 single-token steps that fold every token into the state in place of the previous one
