@@ -367,13 +367,19 @@ def _chunked_setup(ctx, inputs, output):
     Q, K, V, log_G, deg, scale, c, S0, s0, want_final = inputs
     O, A, lcs, Kd, Sc, sc, rm, den, Sf, sf, live, S, s = output
     ctx.save_for_backward(Q, K, V, A, lcs, Kd, Sc, sc, rm, O, den, live, S, s)
-    ctx.meta = (deg, scale, c, log_G is not None, S0 is not None, None if s0 is None else s0.dtype, bool(want_final))
+    ctx.meta = (deg, scale, c, log_G is not None, S0 is not None, None if s0 is None else s0.dtype, bool(want_final),
+                int(_lib.load().pr_get_gate_skipping()))
     ctx.set_materialize_grads(False)
 
 
 def _chunked_backward(ctx, dO, dA, dlcs, dKd, dSc, dsc, drm, dden, dSf, dsf, dlive, dS_, ds_):
     Q, K, V, A, lcs, Kd, Sc, sc, rm, O, den, live, S, s = ctx.saved_tensors
-    deg, scale, c, gated, carried, s0_dtype, want_final = ctx.meta
+    deg, scale, c, gated, carried, s0_dtype, want_final, skipping = ctx.meta
+    if gated and skipping != int(_lib.load().pr_get_gate_skipping()):
+        # (with skipping on, the forward leaves unwritten what its own readers leave out -- dead rows of the discounted
+        # keys, scans that nothing survives -- and a backward with skipping off would read them)
+        raise RuntimeError("gate skipping was switched between this forward and its backward (pr_set_gate_skipping): "
+                           "keep the setting for the whole step")
     if not want_final:   # (the placeholders returned in place of a final state carry no gradient)
         dSf = dsf = None
     if dO is None and dSf is None and dsf is None:

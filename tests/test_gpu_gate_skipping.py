@@ -247,3 +247,20 @@ def test_scans_that_the_readers_make_unnecessary(lib):
     lib.pr_set_gate_skipping(0)
     Y2, y2 = fwd(1)
     assert torch.equal(Y2, Y0) and torch.equal(y2, y0)
+
+
+def test_switching_between_forward_and_backward_is_refused(pra, lib):
+    """With skipping on, the forward leaves unwritten what its own readers leave out (dead rows of the discounted keys,
+    scans that nothing survives); a backward that runs with the other setting would read them, so the node refuses."""
+    g = torch.Generator().manual_seed(3)
+    b, t, h, d, c = 1, 2048, 2, 64, 1024
+    Q, K, V = (torch.randn(b, t, h, d, generator=g).bfloat16().to(DEV).requires_grad_(True) for _ in range(3))
+    lg = gates("strong", b, t, h, c, g).to(DEV).requires_grad_(True)
+    lib.pr_set_gate_skipping(1)
+    Y = pra.power_retention(Q, K, V, lg, deg=2, chunk_size=c)
+    lib.pr_set_gate_skipping(0)
+    with pytest.raises(RuntimeError, match="gate skipping was switched"):
+        Y.sum().backward()
+    lib.pr_set_gate_skipping(1)
+    Y.sum().backward()          # (the same graph, with the forward's setting restored)
+    assert torch.isfinite(Q.grad.float()).all()
