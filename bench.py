@@ -647,6 +647,8 @@ def main():
             "canonical_tflops_at_value": round(canon / dt / 1e12, 2),
             "note": "canonical_tflops_at_value counts products the kernels did not execute: a rate of useful work, not a "
                     "matrix-core utilisation"},
+        "value_every_tile_visited": round(cfg["b"] * cfg["t"] / every["dt"], 1),
+        "ms_per_step_every_tile_visited": round(every["dt"] * 1e3, 4),
         "tflops": round(tflops, 2), "pct_bf16_mfma_peak": round(100 * tflops / PEAK_BF16_TFLOPS, 2),
         "tflops_measured_with": "gate skipping off (every product of the canonical count executed)",
         "timing": {"protocol": "W warm-up steps, then untimed steps for settle_ms (the clock governor's ramp); value = "
