@@ -12,7 +12,8 @@ import sys
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 OUT = os.path.join(os.path.dirname(HERE), "libpower_retention_hip.so")
-SOURCES = ["capi", "discumsum", "sympow_tn", "sympow_nn", "sympow_grad", "attention_fwd", "attention_bwd", "elementwise",
+SOURCES = ["capi", "discumsum", "sympow_tn", "sympow_nn", "sympow_grad", "sympow_dvdk", "attention_fwd", "attention_bwd",
+           "elementwise",
            "chunk_glue", "chunk_fwd", "chunk_bwd_dq", "decode", "cache"]
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Xclang", "-target-feature", "-Xclang",
          "-packed-fp32-ops", "-Wno-unused-command-line-argument"]
@@ -26,7 +27,16 @@ FILE_FLAGS = {
     "attention_bwd": ["-mllvm", "-amdgpu-sched-strategy=max-memory-clause"],
     "chunk_bwd_dq": ["-mllvm", "-amdgpu-sched-strategy=max-memory-clause"],
     "sympow_grad": ["-mllvm", "-amdgpu-sched-strategy=max-memory-clause"],
+    "sympow_dvdk": ["-mllvm", "-amdgpu-sched-strategy=max-memory-clause"],
     "sympow_tn": ["-mllvm", "-amdgpu-use-amdgpu-trackers=1"],
+}
+
+
+# headers beyond common.h and kernels.h that a source includes
+FILE_HEADERS = {
+    "sympow_nn": ["sympow_nn_dev.h"],
+    "sympow_grad": ["sympow_grad_dev.h"],
+    "sympow_dvdk": ["sympow_nn_dev.h", "sympow_grad_dev.h"],
 }
 
 
@@ -43,6 +53,7 @@ def stale(name):
     if not os.path.exists(obj):
         return True
     deps = [os.path.join(HERE, name + ".hip"), os.path.join(HERE, "common.h"), os.path.join(HERE, "kernels.h")]
+    deps += [os.path.join(HERE, h) for h in FILE_HEADERS.get(name, [])]
     return any(os.path.getmtime(d) > os.path.getmtime(obj) for d in deps)
 
 

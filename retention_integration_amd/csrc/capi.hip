@@ -141,14 +141,10 @@ int pr_update_state_bwd(const void* K, const void* V, const void* dS, const floa
   if (zero_last_of < 0 || (zero_last_of > 0 && BN % zero_last_of != 0))
     return fail(PR_ERR_ARG, "update_state_bwd: zero_last_of must be 0 or a divisor of BN (got %d, BN %d)", zero_last_of, BN);
   const int nn_ = zero_last_of > 0 ? zero_last_of : 1, skl = zero_last_of > 0 ? 1 : 0;
-  if (dV) {
-    pr::NNArgs nn{K, dS, nullptr, dV, nullptr, nullptr, nullptr, nullptr, 1.f, c, h, 1, nn_, 0, skl, dS_symmetric ? 1 : 0, nullptr};
-    nn.live_rows = live_rows;
-    nn.B_alt = dS_scan_in;
-    nn.carry = scan_log_G;
-    if (int rc = finish(pr::sympow_nn(nn, BN, d, 1, 0, dtype, (hipStream_t)stream), "update_state_bwd(dV)")) return rc;
-  }
-  if (!dK) return 0;
+  pr::NNArgs nn{K, dS, nullptr, dV, nullptr, nullptr, nullptr, nullptr, 1.f, c, h, 1, nn_, 0, skl, dS_symmetric ? 1 : 0, nullptr};
+  nn.live_rows = live_rows;
+  nn.B_alt = dS_scan_in;
+  nn.carry = scan_log_G;
   pr::GradArgs g{K, V, nullptr, dS, ds, dK, c, h, 1, nn_, skl ? 2 : 0, dS_symmetric ? 1 : 0};
   g.live_rows = live_rows;
   g.live_side = 0;
@@ -156,6 +152,12 @@ int pr_update_state_bwd(const void* K, const void* V, const void* dS, const floa
   g.sB_alt = ds_scan_in;
   g.carry = scan_log_G;
   g.alt_shift = 1;
+  // short chunks, both gradients: one launch whose two readers of every chunk's dS share it through L2
+  if (dV && dK && pr::sympow_dvdk_ok(c, 1))
+    return finish(pr::sympow_dvdk(nn, g, BN, d, dtype, (hipStream_t)stream), "update_state_bwd(dV, dK)");
+  if (dV)
+    if (int rc = finish(pr::sympow_nn(nn, BN, d, 1, 0, dtype, (hipStream_t)stream), "update_state_bwd(dV)")) return rc;
+  if (!dK) return 0;
   return finish(pr::sympow_grad(g, BN, d, 1, dtype, (hipStream_t)stream), "update_state_bwd(dK)");
 }
 

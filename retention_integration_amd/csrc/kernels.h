@@ -163,6 +163,12 @@ struct GradArgs {
 };
 int sympow_grad(const GradArgs& a, int BN, int d, int mult, int dtype, hipStream_t st);
 
+// sympow_dvdk.hip: sympow_nn's plain form (dV) and sympow_grad (dK), both with the key multiplier, of the same K and dS
+// in one launch, for chunks that are one row block of either (sympow_dvdk_ok): their workgroups are dealt pair by pair
+// to one XCD, so that the state both stream comes from HBM once.  Results are those of the two launches, bit for bit.
+int sympow_dvdk_ok(int c, int r);
+int sympow_dvdk(const NNArgs& na, const GradArgs& ga, int BN, int d, int dtype, hipStream_t st);
+
 // attention_fwd.hip / attention_bwd.hip
 struct AttnFwdArgs {
   const void* Q;    // [B, tq, h*r, d]
