@@ -44,7 +44,8 @@ enum {
  * before and after it (S_init, S_final and their gradients).  7: pr_chunk_fwd, pr_chunk_bwd_dq and their _supported queries.
  * 8: pr_set_gate_skipping / pr_get_gate_skipping; live_rows of pr_chunk_prep_fwd, pr_update_state_fwd / _bwd and
  * pr_query_state_bwd; consumers_follow_gates of pr_state_scan_fwd / _bwd and the *_scan_in arguments of pr_chunk_fwd,
- * pr_chunk_bwd_dq and pr_update_state_bwd. */
+ * pr_chunk_bwd_dq and pr_update_state_bwd.  9: live_rows of pr_chunk_attention_bwd; with live_rows,
+ * pr_update_state_bwd leaves whole blocks of 256 dead rows of dK, dV unwritten. */
 int pr_abi_version(void);
 const char* pr_last_error(void);
 
@@ -115,7 +116,9 @@ int pr_update_state_fwd(const void* K, const void* V, void* S, float* s, const i
  *   zero_last_of = n > 0 is the promise that dS, ds of the last of every n chunks are zero (that chunk's state feeds
  *   nothing): they are not read and dK, dV are written as zeros there; 0 makes no such promise.
  *   live_rows (NULL, or what pr_chunk_prep_fwd wrote for the gates that discounted K): the time steps before
- *   live_rows[bn,h,0] hold keys that are exact zeros; dK, dV are written as zeros there and not computed.
+ *   live_rows[bn,h,0] hold keys that are exact zeros; dK, dV are zero there and not computed -- and up to the last
+ *   multiple of 256 steps below live_rows[bn,h,0] they are NOT WRITTEN: hand dK, dV to pr_chunk_attention_bwd with the
+ *   same live_rows (which does not read them there), or treat those rows as zeros.
  *   dS_scan_in, ds_scan_in, scan_log_G (all NULL, or all given together with zero_last_of = n): dS, ds are the output of
  *   pr_state_scan_bwd and these its inputs dS_out, ds_out, log_G.  Entry k of that scan equals its input entry k + 1
  *   bit for bit when exp(scan_log_G[k + 1]) == 0; the kernels then read the input entry (see consumers_follow_gates
@@ -308,14 +311,17 @@ int pr_chunk_prep_fwd(const float* log_G, const void* K, const void* Q, float* A
  *   (update_state backward).  With A = NULL the factors are 1 and dGq, dGk, dotk are not written.
  *   dQ_state_plain != 0: dQ_state is already the gradient w.r.t. Q itself (pr_query_state_bwd with q_log_gate):
  *   dQ = dQ_attn + dQ_state and dGq gets (Q.dQ_state)/deg.
+ *   live_rows (NULL, or the array that pr_chunk_prep_fwd wrote for A; needs A, dK and dV): the factor
+ *   exp((A[c-1] - A)/deg) is an exact zero at the keys before live_rows[bn,h,0]; dK_state and dV_state are not read
+ *   there (they are zeros, or were left unwritten by a pr_update_state_bwd that was given the same live_rows).
  * pr_chunk_gate_scan_bwd finishes the gate gradient: dlog_G holds dGk on entry; the r query heads' dGq [BN,c,h*r]
  *   are added (dGq may be NULL), dlog_G[c-1] += (sum_t dotk)/deg + dlcs_a + dlcs_b (dlcs_b may be NULL), then the
  *   reverse cumulative sum over the chunk, in place. */
 int pr_chunk_attention_bwd(const void* Q, const void* K, const void* V, const float* A, const float* rowmax,
                            const void* dO, const float* dl, const float* dO_scale, const void* dQ_state,
-                           const void* dK_state, const void* dV_state, void* dQ, void* dK, void* dV, float* dGq,
-                           float* dGk, float* dotk, int BN, int c, int h, int r, int d, float scale, int deg,
-                           int dQ_state_plain, int dtype, void* stream);
+                           const void* dK_state, const void* dV_state, const int* live_rows, void* dQ, void* dK,
+                           void* dV, float* dGq, float* dGk, float* dotk, int BN, int c, int h, int r, int d, float scale,
+                           int deg, int dQ_state_plain, int dtype, void* stream);
 int pr_chunk_gate_scan_bwd(float* dlog_G, const float* dGq, const float* dotk, const float* dlcs_a, const float* dlcs_b,
                            int BN, int c, int h, int r, int deg, void* stream);
 

@@ -49,7 +49,7 @@ SIGNATURES = {
     "pr_query_state_scan_bwd": (c_int, [_P] * 17 + [_I] * 6 + [_F, _I, _I, _P]),
     "pr_state_scan_bwd_workspace": (c_size_t, [_I] * 3 + [c_int64, c_int64]),
     "pr_state_scan_bwd": (c_int, [_P] * 13 + [_I] * 4 + [c_int64, c_int64, _I, _I, _P]),
-    "pr_chunk_attention_bwd": (c_int, [_P] * 17 + [_I] * 5 + [_F, _I, _I, _I, _P]),
+    "pr_chunk_attention_bwd": (c_int, [_P] * 18 + [_I] * 5 + [_F, _I, _I, _I, _P]),
     "pr_chunk_gate_scan_bwd": (c_int, [_P] * 5 + [_I] * 5 + [_P]),
     "pr_decode_step_workspace": (c_size_t, [_I] * 5),
     "pr_decode_step": (c_int, [_P] * 14 + [_I] * 5 + [_F, _I, _I, _I, _P]),

@@ -502,8 +502,10 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
   };
   // With the chunked epilogue the workgroup's rows of dKs and dVs ride through the ring as two more stages after
   // the last row tile (keys 0..63 in the Q area, 64..127 in the dO area): they arrive under the last tiles' work.
-  const T* dKsg = a.dKs ? (const T*)a.dKs + (long)b * a.tk * a.h * DH + hh * DH : nullptr;
-  const T* dVsg = a.dVs ? (const T*)a.dVs + (long)b * a.tk * a.h * DH + hh * DH : nullptr;
+  // (not for a block of keys whose discount is an exact zero: their rows of dKs and dVs are zeros, or not written at all)
+  const bool dead_keys = gate_skip && a.live_rows && a.dKs && key0 + KEYS <= a.live_rows[((long)b * a.h + hh) * 2];
+  const T* dKsg = a.dKs && !dead_keys ? (const T*)a.dKs + (long)b * a.tk * a.h * DH + hh * DH : nullptr;
+  const T* dVsg = a.dVs && !dead_keys ? (const T*)a.dVs + (long)b * a.tk * a.h * DH + hh * DH : nullptr;
   const int ntot = nsteps + (dKsg ? 2 : 0);
   // lane offsets of the copies of a regular tile (r a power of two): folded row j of a tile is time step j / r, head
   // hh * r + j % r, whatever the tile

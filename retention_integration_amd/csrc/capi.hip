@@ -44,7 +44,7 @@ size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 
 extern "C" {
 
-int pr_abi_version(void) { return 8; }
+int pr_abi_version(void) { return 9; }
 
 void pr_set_launch_hook(pr_launch_hook_t hook, void* user) {
   pr::g_launch_hook = nullptr;   // (never a new hook with the old user pointer)
@@ -94,8 +94,8 @@ int pr_attention_bwd(const void* Q, const void* K, const void* V, const float* G
 
 int pr_chunk_attention_bwd(const void* Q, const void* K, const void* V, const float* A, const float* rowmax,
                            const void* dO, const float* dl, const float* dO_scale, const void* dQ_state,
-                           const void* dK_state, const void* dV_state, void* dQ, void* dK, void* dV, float* dGq,
-                           float* dGk, float* dotk, int BN, int c, int h, int r, int d, float scale, int deg,
+                           const void* dK_state, const void* dV_state, const int* live_rows, void* dQ, void* dK, void* dV,
+                           float* dGq, float* dGk, float* dotk, int BN, int c, int h, int r, int d, float scale, int deg,
                            int dQ_state_plain, int dtype, void* stream) {
   if (int rc = check_common("chunk_attention_bwd", d, deg, dtype, false)) return rc;
   if (bad_ptr(Q) || bad_ptr(K) || bad_ptr(V) || bad_ptr(rowmax) || bad_ptr(dO) || bad_opt(dQ) || bad_opt(dK) ||
@@ -111,6 +111,8 @@ int pr_chunk_attention_bwd(const void* Q, const void* K, const void* V, const fl
   if (BN <= 0 || c <= 0 || h <= 0 || r <= 0) return fail(PR_ERR_ARG, "chunk_attention_bwd: need BN,c,h,r > 0");
   pr::AttnBwdArgs a{Q, K, V, A, rowmax, dO, dl, dO_scale, dQ, dK, dV, A ? dGq : nullptr, A ? dGk : nullptr,
                     c, c, h, r, scale, (float)deg, dQ_state, dK_state, dV_state, A ? dotk : nullptr, dQ_state_plain ? 1 : 0};
+  if (live_rows && (!A || !dK)) return fail(PR_ERR_ARG, "chunk_attention_bwd: live_rows describes the gates' effect on dK_state and dV_state");
+  a.live_rows = live_rows;
   return finish(pr::attention_bwd(a, BN, d, dtype, (hipStream_t)stream), "chunk_attention_bwd");
 }
 

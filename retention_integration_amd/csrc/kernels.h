@@ -207,6 +207,9 @@ struct AttnBwdArgs {
   const void* dVs;      // [B, tk, h, d]:   dV = dV_attn + dVs
   float* dotk;          // [B, tk, h]:      (K.dKs) w
   int dQs_plain;        // dQs is already the gradient w.r.t. Q itself: dQ = dQ_attn + dQs, dGq += (Q.dQs) / deg
+  // [B, h, 2] or null (chunk_prep_fwd writes it): dKs and dVs are zero at the keys before time step live_rows[b, hh, 0]
+  // and need not have been written before the last multiple of 256 below it -- a key block of such keys reads neither
+  const int* live_rows = nullptr;
 };
 int attention_bwd(const AttnBwdArgs& a, int B, int d, int dtype, hipStream_t st);
 

@@ -111,6 +111,9 @@ __device__ __forceinline__ void sympow_grad_body(const GradArgs& a, int row_bloc
       for (int ii = 0; ii < LOADS; ii++) async_copy16_sv(src, boffs[ii], ring_lds + (step % GR_NST) * STAGE + ii * 4096);
     }
   };
+  // (live_rows, side 0: up to the last multiple of 256 rows before the first live time step, dX -- a zero -- is not even
+  // written: its reader, attention_bwd's epilogue, is given the same live_rows and does not read it)
+  if (a.live_rows && a.live_side == 0 && row0 + ROWS <= ((a.live_rows[((long)bn * a.h + hh) * 2] * a.r) & ~255)) return;
   // X rows of this workgroup (waited for together with stage 0), then the first stage(s)
   async_load_tile<CX, ROWS>(xt, [&](int row) { return (const char*)(Xg + row_off(row0 + row) * DK); });
   issue(0);

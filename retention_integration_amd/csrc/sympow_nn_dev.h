@@ -150,6 +150,13 @@ __device__ __forceinline__ void sympow_nn_body(const NNArgs& a, int row_blocks, 
 #pragma unroll
   for (int mi = 0; mi < MT; mi++) aux[mi] = 0.f;
 
+  // X rows before time step live_rows[bn, hh, 0] are exact zeros (keys that their discount has turned into zeros), and
+  // so are their features and their rows of the output.  Up to the last multiple of 256 rows before that step the
+  // output is not even written: its reader (attention_bwd's epilogue, given the same live_rows) does not read it.
+  if (EPI == NN_EPI_PLAIN && a.live_rows) {
+    const int lv = a.live_rows[((long)bn * a.h + hh) * 2] * a.r;
+    if (row0 + ROWS <= (lv & ~255)) return;
+  }
   async_load_tile<CX, ROWS>(xt, [&](int row) { return (const char*)(Xg + row_off(row0 + row) * DK); });
   if (skip) {
     wait_vmcnt<0>();
@@ -163,8 +170,7 @@ __device__ __forceinline__ void sympow_nn_body(const NNArgs& a, int row_blocks, 
       issue(nxt.f0(), issued % NN_NST, nxt.narrow());
       nxt.next();
     }
-    // X rows before time step live_rows[bn, hh, 0] are exact zeros (keys that their discount has turned into zeros), and
-    // so are their features: a block of such rows is written as zeros without the sweep.
+    // a block of zero rows past that multiple of 256 is written as zeros without the sweep
     bool x_zero = false;
     if (EPI == NN_EPI_PLAIN && a.live_rows) {
       x_zero = row0 + ROWS <= a.live_rows[((long)bn * a.h + hh) * 2] * a.r;

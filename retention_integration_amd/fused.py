@@ -322,7 +322,7 @@ def chunked_bwd(Q: Tensor, K: Tensor, V: Tensor, A: Tensor, lcs: Tensor, Kd: Ten
     if dq_one_kernel:
         # the query side is done (or running on the second stream): the key side alone
         _lib.check(lib.pr_chunk_attention_bwd(p(Q), p(K), p(V), Ag, p(rm), p(dO), p(dla), p(dys), None, p(dKd), p(dVs),
-                                              None, p(dKa), p(dVa), None, p(dGk), p(dotk), BN, c, h, r, d, scale, deg, 1,
+                                              live_p, None, p(dKa), p(dVa), None, p(dGk), p(dotk), BN, c, h, r, d, scale, deg, 1,
                                               code, st), "chunk_attention_bwd(dK, dV)")
         if two_streams:
             torch.cuda.current_stream().wait_stream(_side_stream(dev))
@@ -333,15 +333,15 @@ def chunked_bwd(Q: Tensor, K: Tensor, V: Tensor, A: Tensor, lcs: Tensor, Kd: Ten
         if not two_streams:
             side.wait_stream(main)
         _lib.check(lib.pr_chunk_attention_bwd(p(Q), p(K), p(V), Ag, p(rm), p(dO), p(dla), p(dys), p(dQg), None, None,
-                                              p(dQa), None, None, p(dGq), None, None, BN, c, h, r, d, scale, deg, 1,
+                                              None, p(dQa), None, None, p(dGq), None, None, BN, c, h, r, d, scale, deg, 1,
                                               code, side.cuda_stream), "chunk_attention_bwd(dQ)")
         _lib.check(lib.pr_chunk_attention_bwd(p(Q), p(K), p(V), Ag, p(rm), p(dO), p(dla), p(dys), None, p(dKd), p(dVs),
-                                              None, p(dKa), p(dVa), None, p(dGk), p(dotk), BN, c, h, r, d, scale, deg, 1,
+                                              live_p, None, p(dKa), p(dVa), None, p(dGk), p(dotk), BN, c, h, r, d, scale, deg, 1,
                                               code, st), "chunk_attention_bwd(dK, dV)")
         main.wait_stream(side)
     else:
         _lib.check(lib.pr_chunk_attention_bwd(p(Q), p(K), p(V), Ag, p(rm), p(dO), p(dla), p(dys), p(dQg), p(dKd),
-                                              p(dVs), p(dQa), p(dKa), p(dVa), p(dGq), p(dGk), p(dotk), BN, c, h, r, d,
+                                              p(dVs), live_p, p(dQa), p(dKa), p(dVa), p(dGq), p(dGk), p(dotk), BN, c, h, r, d,
                                               scale, deg, 1, code, st), "chunk_attention_bwd")
     dlg = _empty((0,), f32, dev)
     if gated:
