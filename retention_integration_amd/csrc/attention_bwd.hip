@@ -28,6 +28,7 @@ constexpr int AB_BM = 64;    // query rows per stage in the dK/dV kernel
 // stages in the ring: three up to d = 64; two at d = 128, where three would leave room for one workgroup per CU
 constexpr int ab_stages(int d) { return d <= 64 ? 3 : 2; }
 constexpr float AB_LOG_EPS = 1e-7f, AB_EXP_CLAMP = 80.f;
+constexpr float AB_LOG2E = 1.4426950408889634f, AB_EXP2_CLAMP = AB_EXP_CLAMP * AB_LOG2E;
 
 // a2^(half_deg - 1)
 template <bool DEG2> __device__ __forceinline__ float pow_hm1(float a2, int half_deg) {
@@ -86,7 +87,7 @@ __global__ __launch_bounds__(256, OCC) void attention_bwd_dq_kernel(AttnBwdArgs 
   const long kstride = (long)a.h * DH * 2;
   const int half_deg = (int)a.deg / 2;
   const float eps_s = AB_LOG_EPS / a.scale, eps2 = eps_s * eps_s;
-  const float scale_p = __expf(a.deg * __logf(a.scale));
+  const float l2sp = a.deg * __log2f(a.scale);
 
   const int last_row = min(row0 + ROWS, rows) - 1;
   const int kmax = min(a.tk, last_row / a.r + shift + 1);
@@ -164,7 +165,7 @@ __global__ __launch_bounds__(256, OCC) void attention_bwd_dq_kernel(AttnBwdArgs 
   int ti[MT];
   long qoff[MT];
   bool live[MT];
-  float base[MT], dlr[MT], dgq[MT], osc[MT];   // base = G_q - m
+  float base2[MT], dlr[MT], dgq[MT], osc[MT];   // base2 = log2(scale^deg exp(G_q - m))
 #pragma unroll
   for (int mi = 0; mi < MT; mi++) {
     const int row = wrow0 + 16 * mi + tcol;
@@ -184,7 +185,7 @@ __global__ __launch_bounds__(256, OCC) void attention_bwd_dq_kernel(AttnBwdArgs 
       dOf[mi][ks] = __builtin_bit_cast(v8, z2);
     }
     const long so = (long)b * a.tq * hq + qoff[mi];
-    base[mi] = (Gg ? Gg[(long)ti[mi] * a.h] : 0.f) - a.rowmax[so];
+    base2[mi] = __builtin_fmaf((Gg ? Gg[(long)ti[mi] * a.h] : 0.f) - a.rowmax[so], AB_LOG2E, l2sp);
     dlr[mi] = a.dl ? a.dl[so] : 0.f;
     osc[mi] = a.dO_scale ? a.dO_scale[so] : 1.f;
     dgq[mi] = 0.f;
@@ -218,9 +219,9 @@ __global__ __launch_bounds__(256, OCC) void attention_bwd_dq_kernel(AttnBwdArgs 
     float* graw = (float*)(smem + (it % NST) * STAGE + 2 * TILE);
     const int rpos = min(AB_BN - 1, a.tk - 1 - it * AB_BN);
     const float gv = Gg ? graw[l] : 0.f;
-    const float R_ = Gg ? graw[rpos] : 0.f, Rs = Gg ? graw[l & ~15] : 0.f;
+    const float R_ = Gg ? graw[rpos] : 0.f;
     graw[AB_BN + l] = __expf(fminf(R_ - gv, AB_EXP_CLAMP));
-    graw[2 * AB_BN + l] = __expf(fminf(Rs - gv, AB_EXP_CLAMP));
+    graw[2 * AB_BN + l] = gv * AB_LOG2E;   // the gate itself, in powers of two, for the diagonal tiles
     if (!Gg) graw[l] = 0.f;
   };
   if (wave == 0) {
@@ -256,7 +257,7 @@ __global__ __launch_bounds__(256, OCC) void attention_bwd_dq_kernel(AttnBwdArgs 
   };
 
   // One 64-key tile.  Past tiles: key factors relative to the gate at the wave's first row (<= 1), the row factor
-  // is applied to the accumulators after the past tiles.  Diagonal tiles: per-group reference, per-pair mask.
+  // is applied to the accumulators after the past tiles.  Diagonal tiles: per-pair exponent, per-pair mask.
   auto tile = [&](int it, const char* st, auto diag_c) __attribute__((always_inline)) {
     constexpr bool DIAG = decltype(diag_c)::value != 0;
     const int j0 = it * AB_BN;
@@ -311,18 +312,20 @@ __global__ __launch_bounds__(256, OCC) void attention_bwd_dq_kernel(AttnBwdArgs 
 #pragma unroll
         for (int mi = 0; mi < MT; mi++) {
           float d4[4];
-          float e = 1.f;
-          if (DIAG) e = scale_p * __expf(fminf(base[mi] - graw[16 * (2 * kp + half)], AB_EXP_CLAMP));
 #pragma unroll
           for (int v = 0; v < 4; v++) {
             const float s = sc[mi][v];
             const float dpl = __builtin_fmaf(dp[mi][v], osc[mi], dlr[mi]);
-            float q = ev[v] * dpl;                       // E * dP without the row factor
-            if (!DEG2) q *= pow_hm1<DEG2>(__builtin_fmaf(s, s, eps2), half_deg);
+            float q;                                     // E * dP (past tiles: without the row factor)
             if (DIAG) {
-              q *= e;
+              // the pair's own exponent: no reference gate shared by a group of keys, whose two factors could leave
+              // the fp32 range against each other where the gates fall steeply
+              q = __builtin_amdgcn_exp2f(fminf(base2[mi] - ev[v], AB_EXP2_CLAMP)) * dpl;
               q = (32 * kp + 16 * half + v <= lim[mi]) ? q : 0.f;
+            } else {
+              q = ev[v] * dpl;
             }
+            if (!DEG2) q *= pow_hm1<DEG2>(__builtin_fmaf(s, s, eps2), half_deg);
             // dz = (s^2 + eps^2) q: the eps^2 part is all there is for a key with q.k = 0 (an all-zero key)
             dgq[mi] = __builtin_fmaf(__builtin_fmaf(s, s, eps2), q, dgq[mi]);
             d4[v] = s * q;
@@ -354,7 +357,7 @@ __global__ __launch_bounds__(256, OCC) void attention_bwd_dq_kernel(AttnBwdArgs 
   // the past tiles were accumulated without the row factor scale^deg * exp(G_q - m - Rw); apply it once
 #pragma unroll
   for (int mi = 0; mi < MT; mi++) {
-    const float f = scale_p * __expf(fminf(base[mi] - Rw, AB_EXP_CLAMP));
+    const float f = __builtin_amdgcn_exp2f(fminf(base2[mi] - Rw * AB_LOG2E, AB_EXP2_CLAMP));
 #pragma unroll
     for (int nt = 0; nt < NT; nt++) acc[mi][nt] *= f;
     dgq[mi] *= f;
@@ -579,7 +582,7 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
   v8 Kf[MK][KS], Vf[MK][KS];
   int key[MK];
   bool live[MK];
-  float Gk[MK], Rk[MK], evg[MK], dgk[MK], keyf[MK];
+  float Gk[MK], Rk[MK], dk[MK], dgk[MK], keyf[MK];
 #pragma unroll
   for (int kj = 0; kj < MK; kj++) {
     key[kj] = wkey0 + 16 * kj + kcol;
@@ -596,8 +599,12 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
       Vf[kj][ks] = __builtin_bit_cast(v8, z2);
     }
     Gk[kj] = Gg ? Gg[(long)min(key[kj], a.tk - 1) * a.h] : 0.f;
-    Rk[kj] = Gg ? Gg[(long)min(wkey0 + 16 * kj + 15, a.tk - 1) * a.h] : 0.f;   // gate at the group's last key
-    evg[kj] = __expf(fminf(Rk[kj] - Gk[kj], AB_EXP_CLAMP));   // key factor inside its group of 16, <= 1
+    // Near the diagonal the exponent of a pair is G_q - m - G_k itself: a key factor and a row factor relative to a
+    // shared reference gate leave the fp32 range against each other once the gates of a group of keys differ by more
+    // than 87.  It is formed as (G_q - m - Rk) - (G_k - Rk) with Rk the gate at the group's last key, which is the
+    // same for the whole wave and stays in a scalar register.
+    Rk[kj] = Gg ? Gg[(long)min(wkey0 + 16 * kj + 15, a.tk - 1) * a.h] : 0.f;
+    dk[kj] = Gk[kj] - Rk[kj];
     dgk[kj] = 0.f;
   }
   // ---- far tiles that the gates have already forgotten -------------------------------------------------------------
@@ -804,7 +811,7 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(AttnBwdArgs a
               }
             } else {
               const bool vis = (keyf[kj] <= fc[half][v]) && live[kj];
-              float E = scale_p * __expf(fminf(fa[half][v] - Rk[kj], AB_EXP_CLAMP)) * evg[kj] * pow_hm1<DEG2>(a2, half_deg);
+              float E = scale_p * __expf(fminf((fa[half][v] - Rk[kj]) - dk[kj], AB_EXP_CLAMP)) * pow_hm1<DEG2>(a2, half_deg);
               E = vis ? E : 0.f;
               q = E * __builtin_fmaf(dp[half][kj][v], fe[half][v], fd[half][v]);
               pw = a2 * E * fe[half][v];

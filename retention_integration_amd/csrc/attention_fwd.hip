@@ -27,6 +27,7 @@ constexpr int AT_BN = 64;
 // stages in the ring: three up to d = 64; two at d = 128, where three would leave room for one workgroup per CU
 constexpr int at_stages(int d) { return d <= 64 ? 3 : 2; }
 constexpr float AT_LOG_EPS = 1e-7f, AT_SUM_EPS = 1e-6f, AT_EXP_CLAMP = 80.f;
+constexpr float AT_LOG2E = 1.4426950408889634f, AT_EXP2_CLAMP = AT_EXP_CLAMP * AT_LOG2E;
 
 template <typename T> struct OnesBits;
 template <> struct OnesBits<bf16_t> { static constexpr uint32_t v = 0x3F803F80u; };
@@ -83,7 +84,7 @@ __global__ __launch_bounds__(256, OCC) void attention_fwd_kernel(AttnFwdArgs a, 
   const long kstride = (long)a.h * DH * 2;
   const int half_deg = (int)a.deg / 2;
   const float eps_s = AT_LOG_EPS / a.scale;          // |scale*x| + eps = scale * (|x| + eps/scale)
-  const float scale_p = __expf(a.deg * __logf(a.scale));
+  const float l2sp = a.deg * __log2f(a.scale);
 
   const int last_row = min(row0 + ROWS, rows) - 1;
   const int kmax = min(a.tk, last_row / a.r + shift + 1);   // keys any row of the workgroup can see
@@ -149,7 +150,7 @@ __global__ __launch_bounds__(256, OCC) void attention_fwd_kernel(AttnFwdArgs a, 
   int ti[MT];
   long qoff[MT];
   bool live[MT];
-  float Gq[MT], mx[MT];
+  float Gq2[MT], mx[MT];   // Gq2 = log2(scale^deg exp(G_q))
   constexpr bool TWO_PASS = sizeof(T) == 2 && !__is_same(T, bf16_t);   // fp16
   float pn[MT], prow[MT];   // (second pass) 1 / row maximum, and that times the past tiles' row factor
 #pragma unroll
@@ -166,7 +167,7 @@ __global__ __launch_bounds__(256, OCC) void attention_fwd_kernel(AttnFwdArgs a, 
       if (live[mi]) z = *(const u32x4*)(Qg + qoff[mi] * DH + 32 * ks + 8 * g);
       Qf[mi][ks] = __builtin_bit_cast(v8, z);
     }
-    Gq[mi] = Gg ? Gg[(long)ti[mi] * a.h] : 0.f;
+    Gq2[mi] = __builtin_fmaf(Gg ? Gg[(long)ti[mi] * a.h] : 0.f, AT_LOG2E, l2sp);
     mx[mi] = 0.f;
   }
   f32x4 acc[MT][NT], accl[MT];
@@ -208,9 +209,9 @@ __global__ __launch_bounds__(256, OCC) void attention_fwd_kernel(AttnFwdArgs a, 
     float* graw = (float*)(smem + (it % NST) * STAGE + 2 * TILE);
     const int rpos = min(AT_BN - 1, a.tk - 1 - it * AT_BN);
     const float gv = Gg ? graw[l] : 0.f;
-    const float R_ = Gg ? graw[rpos] : 0.f, Rs = Gg ? graw[l & ~15] : 0.f;
+    const float R_ = Gg ? graw[rpos] : 0.f;
     graw[AT_BN + l] = __expf(fminf(R_ - gv, AT_EXP_CLAMP));
-    graw[2 * AT_BN + l] = __expf(fminf(Rs - gv, AT_EXP_CLAMP));
+    graw[2 * AT_BN + l] = gv * AT_LOG2E;   // the gate itself, in powers of two, for the diagonal tiles
     if (!Gg) graw[l] = 0.f;
   };
   if (wave == 0) {
@@ -321,14 +322,19 @@ __global__ __launch_bounds__(256, OCC) void attention_fwd_kernel(AttnFwdArgs a, 
         float p[8];
 #pragma unroll
         for (int half = 0; half < 2; half++) {
-          float e = eu[mi];
-          if (DIAG) e = scale_p * __expf(fminf(Gq[mi] - graw[16 * (2 * kp + half)], AT_EXP_CLAMP));
-          if (DIAG && MODE == 2) e *= pn[mi];
 #pragma unroll
           for (int v = 0; v < 4; v++) {
-            float w = pow_even<DEG2>(sc[half][mi][v], eps2, half_deg) * ev[half][v];
-            if (DIAG || MODE == 2) w *= e;
-            if (DIAG) w = (32 * kp + 16 * half + v <= lim[mi]) ? w : 0.f;
+            float w = pow_even<DEG2>(sc[half][mi][v], eps2, half_deg);
+            if (DIAG) {
+              // the pair's own exponent: no reference gate shared by a group of keys, whose two factors could leave
+              // the fp32 range against each other where the gates fall steeply
+              w *= __builtin_amdgcn_exp2f(fminf(Gq2[mi] - ev[half][v], AT_EXP2_CLAMP));
+              if (MODE == 2) w *= pn[mi];
+              w = (32 * kp + 16 * half + v <= lim[mi]) ? w : 0.f;
+            } else {
+              w *= ev[half][v];
+              if (MODE == 2) w *= eu[mi];
+            }
             p[4 * half + v] = w;
           }
         }
@@ -364,7 +370,7 @@ __global__ __launch_bounds__(256, OCC) void attention_fwd_kernel(AttnFwdArgs a, 
     if constexpr (MODE != 2) {
 #pragma unroll
       for (int mi = 0; mi < MT; mi++) {
-        const float f = scale_p * __expf(fminf(Gq[mi] - Rw, AT_EXP_CLAMP));
+        const float f = __builtin_amdgcn_exp2f(fminf(Gq2[mi] - Rw * AT_LOG2E, AT_EXP2_CLAMP));
         if (MODE == 0) {
 #pragma unroll
           for (int nt = 0; nt < NT; nt++) acc[mi][nt] *= f;
@@ -388,7 +394,7 @@ __global__ __launch_bounds__(256, OCC) void attention_fwd_kernel(AttnFwdArgs a, 
     for (int mi = 0; mi < MT; mi++) {
       mx[mi] = max_over_rows(mx[mi]);
       pn[mi] = mx[mi] > 0.f ? 1.f / mx[mi] : 0.f;
-      prow[mi] = scale_p * __expf(fminf(Gq[mi] - Rw, AT_EXP_CLAMP)) * pn[mi];
+      prow[mi] = __builtin_amdgcn_exp2f(fminf(Gq2[mi] - Rw * AT_LOG2E, AT_EXP2_CLAMP)) * pn[mi];
     }
     lds_barrier();   // every wave is done with the ring: start the copies over
     issue(it0);

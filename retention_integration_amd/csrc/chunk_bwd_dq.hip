@@ -27,6 +27,7 @@ constexpr int CB_BN = 64;    // keys per attention stage
 constexpr int CB_FR = 64;    // feature rows per state stage
 constexpr int CB_NST = 3;    // attention ring
 constexpr float CB_LOG_EPS = 1e-7f, CB_EXP_CLAMP = 80.f;
+constexpr float CB_LOG2E = 1.4426950408889634f, CB_EXP2_CLAMP = CB_EXP_CLAMP * CB_LOG2E;
 
 typedef __attribute__((address_space(3))) s16x4 cb_lds_s16x4;
 typedef __attribute__((address_space(3))) f32x4 cb_lds_f32x4;
@@ -83,6 +84,7 @@ __global__ __launch_bounds__(256, 3) void chunk_bwd_dq_kernel(ChunkBwdDqArgs a, 
   const long kstride = (long)a.h * DH * 2;
   const float eps_s = CB_LOG_EPS / a.scale, eps2 = eps_s * eps_s;
   const float scale_p = a.scale * a.scale;
+  const float l2sp = __log2f(scale_p);
   bool has_state = !(a.skip_first && (b % a.n == 0));
 
   const int last_row = min(row0 + ROWS, rows) - 1;
@@ -170,7 +172,7 @@ __global__ __launch_bounds__(256, 3) void chunk_bwd_dq_kernel(ChunkBwdDqArgs a, 
   v8 Qf[MT][KS], dOf[MT][KS];
   int ti[MT];
   bool live[MT];
-  float base[MT], dlr[MT], dgq[MT], osc[MT];   // base = G_q - m
+  float base2[MT], dlr[MT], dgq[MT], osc[MT];   // base2 = log2(scale^2 exp(G_q - m))
   // the state part's factor on dO, one per row: parked in LDS until the sweep (a register pair through the tile loops
   // would be a spilled one)
   float* cq_lds = (float*)(smem + CB_NST * STAGE);
@@ -194,7 +196,7 @@ __global__ __launch_bounds__(256, 3) void chunk_bwd_dq_kernel(ChunkBwdDqArgs a, 
     }
     const long so = (long)b * a.c * hq + qoff;
     const float gq = Gg ? Gg[(long)t * a.h] : 0.f, m = a.rowmax[so];
-    base[mi] = gq - m;
+    base2[mi] = __builtin_fmaf(gq - m, CB_LOG2E, l2sp);
     dlr[mi] = a.dl[so];
     osc[mi] = a.dO_scale[so];
     // (the expressions of the row-wise preparation kernel, so that the scaled dO below has its bits)
@@ -228,9 +230,9 @@ __global__ __launch_bounds__(256, 3) void chunk_bwd_dq_kernel(ChunkBwdDqArgs a, 
     float* graw = (float*)(smem + (it % CB_NST) * STAGE + 2 * TILE);
     const int rpos = min(CB_BN - 1, a.c - 1 - it * CB_BN);
     const float gv = Gg ? graw[l] : 0.f;
-    const float R_ = Gg ? graw[rpos] : 0.f, Rs = Gg ? graw[l & ~15] : 0.f;
+    const float R_ = Gg ? graw[rpos] : 0.f;
     graw[CB_BN + l] = __expf(fminf(R_ - gv, CB_EXP_CLAMP));
-    graw[2 * CB_BN + l] = __expf(fminf(Rs - gv, CB_EXP_CLAMP));
+    graw[2 * CB_BN + l] = gv * CB_LOG2E;   // the gate itself, in powers of two, for the diagonal tiles
     if (!Gg) graw[l] = 0.f;
   };
   if (wave == 0) {
@@ -304,16 +306,16 @@ __global__ __launch_bounds__(256, 3) void chunk_bwd_dq_kernel(ChunkBwdDqArgs a, 
 #pragma unroll
         for (int mi = 0; mi < MT; mi++) {
           float d4[4];
-          float e = 1.f;
-          if (DIAG) e = scale_p * __expf(fminf(base[mi] - graw[16 * (2 * kp + half)], CB_EXP_CLAMP));
 #pragma unroll
           for (int v = 0; v < 4; v++) {
             const float s = sc[mi][v];
             const float dpl = __builtin_fmaf(dp[mi][v], osc[mi], dlr[mi]);
-            float q = ev[v] * dpl;                       // E * dP without the row factor
+            float q;                                     // E * dP (past tiles: without the row factor)
             if (DIAG) {
-              q *= e;
+              q = __builtin_amdgcn_exp2f(fminf(base2[mi] - ev[v], CB_EXP2_CLAMP)) * dpl;
               q = (32 * kp + 16 * half + v <= lim[mi]) ? q : 0.f;
+            } else {
+              q = ev[v] * dpl;
             }
             dgq[mi] = __builtin_fmaf(__builtin_fmaf(s, s, eps2), q, dgq[mi]);
             d4[v] = s * q;
@@ -340,7 +342,7 @@ __global__ __launch_bounds__(256, 3) void chunk_bwd_dq_kernel(ChunkBwdDqArgs a, 
   // the past tiles were accumulated without the row factor scale^2 * exp(G_q - m - Rw); apply it once
 #pragma unroll
   for (int mi = 0; mi < MT; mi++) {
-    const float f = scale_p * __expf(fminf(base[mi] - Rw, CB_EXP_CLAMP));
+    const float f = __builtin_amdgcn_exp2f(fminf(base2[mi] - Rw * CB_LOG2E, CB_EXP2_CLAMP));
 #pragma unroll
     for (int nt = 0; nt < NT; nt++) acc[mi][nt] *= f;
     dgq[mi] *= f;

@@ -33,6 +33,7 @@ constexpr int CF_BN = 64;   // keys per attention stage
 constexpr int CF_FR = 64;   // feature rows per state stage
 constexpr int CF_NST = 3;   // attention ring
 constexpr float CF_LOG_EPS = 1e-7f, CF_SUM_EPS = 1e-6f, CF_EXP_CLAMP = 80.f;
+constexpr float CF_LOG2E = 1.4426950408889634f, CF_EXP2_CLAMP = CF_EXP_CLAMP * CF_LOG2E;
 
 // Stage order of the state sweep over (strip y, first x column X0): blocks below the diagonal four x columns at a time,
 // then the diagonal block as quarters -- x columns 0-3 and 4-7 with the upper eight w counted twice (they stand for
@@ -103,6 +104,7 @@ __global__ __launch_bounds__(256, 3) void chunk_fwd_kernel(ChunkFwdArgs a, int r
   const long kstride = (long)a.h * DH * 2;
   const float eps_s = CF_LOG_EPS / a.scale, eps2 = eps_s * eps_s;
   const float scale_p = a.scale * a.scale;
+  const float l2sp = __log2f(scale_p);
   bool no_state = a.skip_first && (b % a.n == 0);
 
   const int last_row = min(row0 + ROWS, rows) - 1;
@@ -181,7 +183,7 @@ __global__ __launch_bounds__(256, 3) void chunk_fwd_kernel(ChunkFwdArgs a, int r
   int ti[MT], lrow[MT];
   long qoff[MT];
   bool live[MT];
-  float Gq[MT], mx[MT], lq[MT];
+  float Gq2[MT], mx[MT], lq[MT];   // Gq2 = log2(scale^2 exp(A_i))
 #pragma unroll
   for (int mi = 0; mi < MT; mi++) {
     lrow[mi] = wslice * 16 * MT + 16 * mi + tcol;
@@ -190,7 +192,7 @@ __global__ __launch_bounds__(256, 3) void chunk_fwd_kernel(ChunkFwdArgs a, int r
     const int rr = live[mi] ? row : 0;
     ti[mi] = rr / a.r;
     qoff[mi] = (long)ti[mi] * hq + hh * a.r + (rr - ti[mi] * a.r);
-    Gq[mi] = Gg ? Gg[(long)ti[mi] * a.h] : 0.f;
+    Gq2[mi] = __builtin_fmaf(Gg ? Gg[(long)ti[mi] * a.h] : 0.f, CF_LOG2E, l2sp);
     mx[mi] = 0.f;
     lq[mi] = 0.f;
   }
@@ -398,9 +400,9 @@ __global__ __launch_bounds__(256, 3) void chunk_fwd_kernel(ChunkFwdArgs a, int r
     float* graw = (float*)(smem + ((it - it0) % CF_NST) * STAGE + 2 * TILE);
     const int rpos = min(CF_BN - 1, a.c - 1 - it * CF_BN);
     const float gv = Gg ? graw[l] : 0.f;
-    const float R_ = Gg ? graw[rpos] : 0.f, Rs = Gg ? graw[l & ~15] : 0.f;
+    const float R_ = Gg ? graw[rpos] : 0.f;
     graw[CF_BN + l] = __expf(fminf(R_ - gv, CF_EXP_CLAMP));
-    graw[2 * CF_BN + l] = __expf(fminf(Rs - gv, CF_EXP_CLAMP));
+    graw[2 * CF_BN + l] = gv * CF_LOG2E;   // the gate itself, in powers of two, for the diagonal tiles
     if (!Gg) graw[l] = 0.f;
   };
   if (wave == 0) {
@@ -475,13 +477,15 @@ __global__ __launch_bounds__(256, 3) void chunk_fwd_kernel(ChunkFwdArgs a, int r
         float p[8];
 #pragma unroll
         for (int half = 0; half < 2; half++) {
-          float e = 1.f;
-          if (DIAG) e = scale_p * __expf(fminf(Gq[mi] - graw[16 * (2 * kp + half)], CF_EXP_CLAMP));
 #pragma unroll
           for (int v = 0; v < 4; v++) {
-            float w = __builtin_fmaf(sc[half][mi][v], sc[half][mi][v], eps2) * ev[half][v];
-            if (DIAG) w *= e;
-            if (DIAG) w = (32 * kp + 16 * half + v <= lim[mi]) ? w : 0.f;
+            float w = __builtin_fmaf(sc[half][mi][v], sc[half][mi][v], eps2);
+            if (DIAG) {
+              w *= __builtin_amdgcn_exp2f(fminf(Gq2[mi] - ev[half][v], CF_EXP2_CLAMP));
+              w = (32 * kp + 16 * half + v <= lim[mi]) ? w : 0.f;
+            } else {
+              w *= ev[half][v];
+            }
             p[4 * half + v] = w;
           }
         }
@@ -503,7 +507,7 @@ __global__ __launch_bounds__(256, 3) void chunk_fwd_kernel(ChunkFwdArgs a, int r
   // the past tiles and the state part were accumulated without the row factor exp(A_i - R) * scale^2; apply it once
 #pragma unroll
   for (int mi = 0; mi < MT; mi++) {
-    const float f = scale_p * __expf(fminf(Gq[mi] - Rw, CF_EXP_CLAMP));
+    const float f = __builtin_amdgcn_exp2f(fminf(Gq2[mi] - Rw * CF_LOG2E, CF_EXP2_CLAMP));
 #pragma unroll
     for (int nt = 0; nt < NT; nt++) acc[mi][nt] *= f;
     accl[mi] *= f;

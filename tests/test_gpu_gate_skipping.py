@@ -59,6 +59,14 @@ def gates(kind, b, t, h, c, g):
         lg = ls(torch.randn(b, t, h, generator=g))
         lg.view(b, t // c, c, h)[:, :, 0] = -200.0
         return lg
+    if kind == "burst":       # hardly any forgetting, except that one step in a hundred forgets everything: falls of
+        lg = 0.01 * ls(1.0 + torch.randn(b, t, h, generator=g))   # 150 between two neighbouring keys of a tile
+        lg[torch.rand(b, t, h, generator=g) < 0.01] = -150.0
+        return lg
+    if kind == "steep_head":  # head 0 forgets by e^-6 a step (96 over sixteen keys), the others hardly at all
+        lg = ls(6.9 + torch.randn(b, t, h, generator=g))
+        lg[:, :, 0] = ls(-6.0 + torch.randn(b, t, generator=g))
+        return lg
     raise ValueError(kind)
 
 
@@ -84,6 +92,8 @@ CASES = [
     (torch.float16, 1, 1024, 2, 2, 64, 256, "strong"),        # ... and fp16
     (torch.bfloat16, 1, 1000, 2, 1, 64, 512, "strong"),       # padded last chunk
     (torch.bfloat16, 1, 1024, 2, 1, 64, None, "strong"),      # quadratic path: the attention kernels over the whole length
+    (torch.bfloat16, 1, 2048, 2, 1, 64, 1024, "burst"),
+    (torch.bfloat16, 1, 2048, 2, 2, 64, 512, "steep_head"),
 ]
 
 
@@ -130,6 +140,46 @@ def test_skipping_against_the_oracle(pra, lib):
         err = rel_l2(x, y)
         print(f"  {name}: rel-L2 {err:.3e}", flush=True)
         assert err <= tol, f"{name}: rel-L2 {err:.3e} > {tol}"
+
+
+STEEP_CASES = [
+    # dtype, b, t, h, r, d, chunk, gates
+    (torch.bfloat16, 1, 2048, 2, 1, 64, 1024, "burst"),       # the one-kernel readers
+    (torch.bfloat16, 2, 256, 3, 1, 32, 128, "burst"),
+    (torch.bfloat16, 1, 960, 2, 4, 64, 192, "steep_head"),
+    (torch.float16, 1, 768, 2, 2, 64, 256, "steep_head"),     # the operator-by-operator path: fp16 ...
+    (torch.bfloat16, 1, 512, 2, 1, 128, 128, "burst"),        # ... and d = 128
+    (torch.bfloat16, 1, 700, 2, 2, 64, None, "burst"),        # quadratic path
+]
+
+
+@pytest.mark.parametrize("dtype,b,t,h,r,d,chunk,kind", STEEP_CASES)
+def test_steep_gates_against_the_oracle(pra, lib, dtype, b, t, h, r, d, chunk, kind):
+    """Gate sums that fall by more than the fp32 exponent range (87) inside one group of sixteen keys: the weight of a
+    pair near the diagonal has to come from its own exponent G_q - G_k, as in the reference
+    (retention/_attention/reference.py:38-44), not from a row factor and a key factor relative to a gate that a group
+    shares -- those overflow and flush against each other and leave NaN or zeros where the weight is close to one."""
+    g = torch.Generator().manual_seed(4242 + t + d)
+    std = d ** -0.25 if dtype == torch.float16 else 1.0
+    Q = (torch.randn(b, t, h * r, d, generator=g) * std).to(dtype)
+    K = (torch.randn(b, t, h, d, generator=g) * std).to(dtype)
+    V = (torch.randn(b, t, h, d, generator=g) * std).to(dtype)
+    c_eff = chunk or t
+    tg = (t + c_eff - 1) // c_eff * c_eff
+    lg = gates(kind, b, tg, h, c_eff, g)[:, :t].contiguous()
+    dO = torch.randn(b, t, h * r, d, generator=g).to(dtype)
+    oi = [x.float().clone().requires_grad_(True) for x in (Q, K, V, lg)]
+    Yo = oracle.power_retention(*oi, deg=2, chunk_size=chunk)
+    Yo.backward(dO.float())
+    want = [Yo] + [x.grad for x in oi]
+    for skip in (1, 0):
+        lib.pr_set_gate_skipping(skip)
+        got = step(pra, *(x.to(DEV) for x in (Q, K, V, lg, dO)), chunk)
+        for name, x, y, tol in zip(["Y", "dQ", "dK", "dV", "dlog_G"], got, want, [OUT_TOL] + [GRAD_TOL] * 4):
+            assert torch.isfinite(x.float()).all(), f"{name} (skipping {skip}): non-finite values"
+            err = rel_l2(x, y)
+            print(f"  skipping {skip} {name}: rel-L2 {err:.3e}", flush=True)
+            assert err <= tol, f"{name} (skipping {skip}): rel-L2 {err:.3e} > {tol}"
 
 
 def test_live_rows_keep_their_promise(lib):
