@@ -329,7 +329,7 @@ int pr_query_state_bwd(const void* Q, const void* S, const float* s, const float
   if (!prepared)
     if (int rc = finish(pr::qs_bwd_prep(O, dO, den, rowmax, q_log_gate, dOs, cvec, rowmax ? dY_attn : nullptr,
                                         rowmax ? dl_attn : nullptr, rowmax ? dY_scale : nullptr, (long)rows, h, r, d,
-                                        scale_p, dtype, st),
+                                        scale_p, (dS && !dQ) ? live_rows : nullptr, c, dtype, st),
                         "query_state_bwd(prep)"))
       return rc;
   // (zero_initial_state == 2: the caller does not want the gradient of the first chunk's (zero) state either)
@@ -394,7 +394,7 @@ int pr_query_state_scan_bwd(const void* Q, const void* S, const float* s, const 
   if (q_log_gate && !rowmax) return fail(PR_ERR_ARG, "query_state_scan_bwd: q_log_gate needs the attention part");
   if (int rc = finish(pr::qs_bwd_prep(O, dO, den, rowmax, q_log_gate, dOs, cvec, rowmax ? dY_attn : nullptr,
                                       rowmax ? dl_attn : nullptr, rowmax ? dY_scale : nullptr, (long)rows, h, r, d,
-                                      scale_p, dtype, st),
+                                      scale_p, nullptr, 0, dtype, st),
                       "query_state_scan_bwd(prep)"))
     return rc;
   if (int rc = finish(pr::sympow_tn_chain(Q, dOs, cvec, log_G, dS_in, ds_in, B, n, c, h, r, d, 0, 1, dtype, st),

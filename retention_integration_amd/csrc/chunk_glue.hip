@@ -15,6 +15,13 @@ namespace pr {
 
 constexpr int GLUE_MAX_C = 8192;
 
+// Workgroups go to the 8 XCDs (each with its own L2) round-robin by linear id.  The h workgroups of a chunk read
+// interleaved elements of the same cache lines ([.., position, head] arrays), so ids are permuted to put them on one
+// XCD: XCD x takes the x-th eighth of the (chunk, head) pairs.  Otherwise every line is fetched by up to 8 L2s.
+__device__ __forceinline__ int xcd_contiguous(int id, int total) {
+  return total % 8 == 0 ? (id % 8) * (total / 8) + id / 8 : id;
+}
+
 // In-place inclusive scan of a[0..c) in LDS by 256 threads (reverse = suffix sums): every thread scans its own run of
 // elements, the run totals are scanned inside each wave with lane shifts and across the four waves through tot[0..4).
 __device__ inline void block_scan(float* a, float* tot, int c, bool reverse) {
@@ -52,7 +59,7 @@ __global__ __launch_bounds__(256) void gate_scan_fwd_kernel(const float* __restr
   extern __shared__ __attribute__((aligned(16))) char smem[];
   float* a = (float*)smem;
   float* tot = a + c;
-  const int tid = threadIdx.x, bn = blockIdx.x / h, hh = blockIdx.x % h;
+  const int tid = threadIdx.x, wg = xcd_contiguous(blockIdx.x, gridDim.x), bn = wg / h, hh = wg % h;
   const long base = (long)bn * c * h + hh;
   for (int i = tid; i < c; i += 256) a[i] = logG[base + (long)i * h];
   __syncthreads();
@@ -129,7 +136,7 @@ __global__ __launch_bounds__(256) void gate_scan_bwd_kernel(float* __restrict__ 
   extern __shared__ __attribute__((aligned(16))) char smem[];
   float* a = (float*)smem;
   float* tot = a + c;
-  const int tid = threadIdx.x, bn = blockIdx.x / h, hh = blockIdx.x % h;
+  const int tid = threadIdx.x, wg = xcd_contiguous(blockIdx.x, gridDim.x), bn = wg / h, hh = wg % h;
   const long base = (long)bn * c * h + hh;
   float ks = 0.f;
   for (int i = tid; i < c; i += 256) {

@@ -215,9 +215,12 @@ int attention_bwd(const AttnBwdArgs& a, int B, int d, int dtype, hipStream_t st)
 
 // elementwise.hip
 // qgate [rows / (h*r), h] or null: the forward's log factor on the state part (see NNArgs); rows are (.., position, h*r)
+// live_rows [rows / (c*h*r), h, 2] or null (with chunks of c positions; chunk_prep_fwd writes it): the rows of dOs from
+// the first multiple of 256 positions at or after live_rows[.., 1] on are left unwritten -- only for a reader that
+// stops there (sympow_tn with live_side 1); ignored while gate skipping is switched off
 int qs_bwd_prep(const void* O, const void* dO, const float* den, const float* rowmax, const float* qgate, void* dOs,
                 float* cvec, void* dY_attn, float* dl_attn, float* dY_scale, long rows, int h, int r, int d, float scale_p,
-                int dtype, hipStream_t st);
+                const int* live_rows, int c, int dtype, hipStream_t st);
 
 // chunk_glue.hip (return -5: chunk longer than the LDS-resident gate vector allows)
 int gate_cumsum(const float* logG, float* A, int B, int t, int h, hipStream_t st);
