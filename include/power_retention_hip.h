@@ -232,7 +232,10 @@ int pr_query_state_fwd(const void* Q, const void* S, const float* s, const void*
  *   on each other, can be issued as two calls on two streams.
  *   live_rows (NULL, or the [BN,h,2] int32 array that pr_chunk_prep_fwd wrote for the gates in q_log_gate): from time
  *   step live_rows[bn,h,1] on, the factor exp(q_log_gate) has underflowed to zero, the state part of those rows has a
- *   zero gradient, and the dS / ds contraction does not read them. */
+ *   zero gradient, and the dS / ds contraction does not read them.  A call that prepares and forms dS / ds but not dQ
+ *   (prepared == 0, dQ == NULL) also leaves the scaled dO of the workspace unwritten from the first multiple of 256
+ *   time steps at or after live_rows[bn,h,1] on: a later prepared != 0 call for dQ has to pass the same live_rows (its
+ *   kernel then does not read those rows), as pr_chunk_bwd_dq, which takes dO itself, need not. */
 size_t pr_query_state_bwd_workspace(int BN, int c, int h, int r, int d, int dtype);
 int pr_query_state_bwd(const void* Q, const void* S, const float* s, const float* rowmax, const float* q_log_gate,
                        const void* O, const float* den, const void* dO, void* dQ, void* dS, float* ds, void* dY_attn,
