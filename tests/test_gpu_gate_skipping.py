@@ -237,6 +237,62 @@ def test_live_rows_keep_their_promise(lib):
         assert (cvec.abs().amax(-1)[dead_q] == 0).all(), f"{kind}: key-sum factor past live_rows[1] is not zero"
 
 
+def test_dS_only_call_leaves_the_dead_rows_of_the_workspace_unwritten_and_nobody_reads_them(lib):
+    """pr_query_state_bwd with live_rows, as two calls: preparation + dS / ds, then dQ from the prepared workspace.  The
+    first call does not store the scaled dO past the last live stage (the workspace is filled with NaN beforehand and
+    keeps them there), the second, given the same live_rows, does not read those rows: dQ, dS, ds equal the one-call
+    result without live_rows bit for bit."""
+    from retention_integration_amd import _lib
+    p, st = _lib.ptr, _lib.stream()
+    BN, c, h, r, d = 4, 1024, 2, 2, 64
+    D = oracle.expanded_dim(d)
+    dt, f32 = torch.bfloat16, torch.float32
+    code = _lib.dtype_code(dt)
+    g = torch.Generator().manual_seed(15)
+    K = torch.randn(BN, c, h, d, generator=g).to(dt).to(DEV)
+    Q = torch.randn(BN, c, h * r, d, generator=g).to(dt).to(DEV)
+    lg = gates("strong", BN, c, h, c, g).to(DEV)
+    A, lcs = torch.empty(BN, c, h, device=DEV), torch.empty(BN, h, device=DEV)
+    Kd = torch.empty_like(K)
+    live = torch.empty((BN, h, 2), dtype=torch.int32, device=DEV)
+    _lib.check(lib.pr_chunk_prep_fwd(p(lg), p(K), p(Q), p(A), p(lcs), p(Kd), None, p(live), BN, c, h, r, d, 2, code, st),
+               "chunk_prep_fwd")
+    S = (torch.randn(BN, h, D, d, generator=g) * 0.1).to(dt).to(DEV)
+    s = torch.rand(BN, h, D, generator=g).to(DEV) + 0.5
+    O = torch.randn(BN, c, h * r, d, generator=g).to(dt).to(DEV)
+    dO = torch.randn(BN, c, h * r, d, generator=g).to(dt).to(DEV)
+    den = torch.rand(BN, c, h * r, generator=g).to(DEV) + 0.5
+    rm = torch.randn(BN, c, h * r, generator=g).to(DEV)
+    rows = BN * c * h * r
+    nbytes = lib.pr_query_state_bwd_workspace(BN, c, h, r, d, code)
+
+    def call(ws, dQ, dS, ds, live_p, prepared):
+        dla, dys = torch.empty_like(den), torch.empty_like(den)
+        _lib.check(lib.pr_query_state_bwd(p(Q), p(S), p(s), p(rm), p(A), p(O), p(den), p(dO), dQ, dS, ds, None, p(dla),
+                                          p(dys), p(ws), live_p, BN, 1, c, h, r, d, 1.0 / d, 2, 0, 0, prepared, code, st),
+                   "query_state_bwd")
+
+    lib.pr_set_gate_skipping(1)
+    ws0 = torch.empty(nbytes, dtype=torch.uint8, device=DEV)
+    dQ0, dS0, ds0 = torch.empty_like(Q), torch.empty_like(S), torch.empty_like(s)
+    call(ws0, p(dQ0), p(dS0), p(ds0), None, 0)
+    ws1 = torch.full((nbytes,), 0xFF, dtype=torch.uint8, device=DEV)   # 0xFFFF is a NaN in both 16-bit types
+    dQ1, dS1, ds1 = torch.empty_like(Q), torch.empty_like(S), torch.empty_like(s)
+    call(ws1, None, p(dS1), p(ds1), p(live), 0)
+    call(ws1, p(dQ1), None, None, p(live), 1)
+    torch.cuda.synchronize()
+    assert torch.equal(dS1, dS0) and torch.equal(ds1, ds0) and torch.equal(dQ1, dQ0)
+    hi = live[..., 1].long()
+    assert (hi < c // 2).all()
+    bound = (hi + 255) // 256 * 256
+    t_idx = torch.arange(c, device=DEV).view(1, c, 1)
+    unwritten = (t_idx >= bound.view(BN, 1, h)).view(BN, c, h, 1, 1).expand(BN, c, h, r, d)
+    dOs0 = ws0[:rows * d * 2].view(dt).view(BN, c, h, r, d)
+    dOs1 = ws1[:rows * d * 2].view(dt).view(BN, c, h, r, d)
+    assert torch.isnan(dOs1.float()[unwritten]).all(), "a row of the scaled dO past the last live stage was written"
+    assert torch.equal(dOs1[~unwritten], dOs0[~unwritten])
+
+
 def test_scans_that_the_readers_make_unnecessary(lib):
     """pr_state_scan_fwd / _bwd with consumers_follow_gates: a (batch, head) whose every carry exp(log_G[k]), k >= 1, is
     zero is neither read nor written (its gate gradient is written as zero), every other one is scanned as without the
