@@ -26,6 +26,7 @@ namespace pr {
 constexpr int CB_BN = 64;    // keys per attention stage
 constexpr int CB_FR = 64;    // feature rows per state stage
 constexpr int CB_NST = 3;    // attention ring
+constexpr int CB_LEAD_BLOCKS = 2;   // row blocks of a chunk that are started before the longest ones (see the kernel)
 constexpr float CB_LOG_EPS = 1e-7f, CB_EXP_CLAMP = 80.f;
 constexpr float CB_LOG2E = 1.4426950408889634f, CB_EXP2_CLAMP = CB_EXP_CLAMP * CB_LOG2E;
 
@@ -56,7 +57,7 @@ __global__ __launch_bounds__(256, 3) void chunk_bwd_dq_kernel(ChunkBwdDqArgs a, 
   static_assert(DH * LDM * 2 <= 2 * SSTAGE, "the key-sum matrix fits the state ring");
   extern __shared__ __attribute__((aligned(1024))) char smem[];
 
-  // placement: see attention_bwd.hip (whole (chunk, head) pairs per (XCD, shader engine) group, longest block first)
+  // placement: see attention_bwd.hip (whole (chunk, head) pairs per (XCD, shader engine) group)
   const int grp = blockIdx.x % 32, u = blockIdx.x / 32, ppg = (npairs + 31) / 32;
   int pig, blk;
   deal_causal_blocks(u, nblocks, ppg, pig, blk);
@@ -66,7 +67,12 @@ __global__ __launch_bounds__(256, 3) void chunk_bwd_dq_kernel(ChunkBwdDqArgs a, 
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int b = __builtin_amdgcn_readfirstlane(pair / a.h), hh = pair - b * a.h;
   const int hq = a.h * a.r, rows = a.c * a.r;
-  const int row0 = (nblocks - 1 - blk) * ROWS;   // late rows see the most keys
+  // Order of a pair's row blocks: the first two of the chunk, then the others from the last (late rows see the most
+  // keys) backwards.  Under gates that forget within a hundred steps or so only those first blocks sweep the state and
+  // are the long ones of the pair by far (156 for 172 us when they are started first); where every block sweeps it they
+  // are the shortest, and two short blocks at the front cost nothing.
+  const int lead = nblocks > CB_LEAD_BLOCKS ? CB_LEAD_BLOCKS : 0;
+  const int row0 = (blk < lead ? blk : nblocks - 1 - (blk - lead)) * ROWS;
   const T* Qg = (const T*)a.Q + (long)b * a.c * hq * DH;
   const T* dOg = (const T*)a.dO + (long)b * a.c * hq * DH;
   const char* Kg = (const char*)((const T*)a.K + (long)b * a.c * a.h * DH + hh * DH);

@@ -32,6 +32,7 @@ namespace pr {
 constexpr int CF_BN = 64;   // keys per attention stage
 constexpr int CF_FR = 64;   // feature rows per state stage
 constexpr int CF_NST = 3;   // attention ring
+constexpr int CF_LEAD_BLOCKS = 2;   // row blocks of a chunk that are started before the longest ones (see the kernel)
 constexpr float CF_LOG_EPS = 1e-7f, CF_SUM_EPS = 1e-6f, CF_EXP_CLAMP = 80.f;
 constexpr float CF_LOG2E = 1.4426950408889634f, CF_EXP2_CLAMP = CF_EXP_CLAMP * CF_LOG2E;
 
@@ -78,12 +79,17 @@ __global__ __launch_bounds__(256, 3) void chunk_fwd_kernel(ChunkFwdArgs a, int r
 
   const int tid = threadIdx.x, l = tid & 63, g = l >> 4, tcol = l & 15;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  // (XCD, shader engine) groups take whole (chunk, head) pairs, longest row block first: see attention_fwd.hip
+  // (XCD, shader engine) groups take whole (chunk, head) pairs: see attention_fwd.hip
   const int grp = blockIdx.x % 32, u = blockIdx.x / 32, ppg = (npairs + 31) / 32;
   int pig, blk;
   deal_causal_blocks(u, row_blocks, ppg, pig, blk);
   const int pair = pig * 32 + grp;
-  const int rblk = row_blocks - 1 - blk;
+  // Order of a pair's row blocks: the first two of the chunk, then the others from the last (which sees the most keys)
+  // backwards.  Under gates that forget within a hundred steps or so only those first blocks sweep the state, which
+  // then makes them the long ones of the pair by far (123 for 134 us when they are started first); where every block
+  // sweeps it they are the shortest, and two short blocks at the front cost nothing.
+  const int lead = row_blocks > CF_LEAD_BLOCKS ? CF_LEAD_BLOCKS : 0;
+  const int rblk = blk < lead ? blk : row_blocks - 1 - (blk - lead);
   if (pair >= npairs) return;
   const int b = __builtin_amdgcn_readfirstlane(pair / a.h), hh = pair - b * a.h;
   const int hq = a.h * a.r, rows = a.c * a.r;
